@@ -1,0 +1,121 @@
+/*
+ * libTsHipOps — C ABI of the MI355X (gfx950) GGUF quantized-matmul backend.
+ *
+ * Every entry point mirrors, argument for argument, the export of the reference's
+ * native bridge (libGgmlOps, `TSGgml_*`) that a `TensorSharp.Backends.HIP` P/Invoke
+ * class would bind instead.  Conventions are the bridge's own:
+ *   - cdecl, descriptor structs passed BY VALUE, strides in ELEMENTS;
+ *   - int return 1 = ok / 0 = failure, message through TSHip_GetLastError()
+ *     (thread-local, valid until the next call on that thread) — except
+ *     TSHip_DequantizeToF32*, which keeps the bridge's 0 / -1 / -2 codes;
+ *   - nothing throws across the boundary; the caller owns every buffer.
+ * Supported weight types: Q8_0 (8), Q4_K (12), MXFP4 (39)
+ * (ids: TensorSharp.Runtime/GgufReader.cs:26-37).
+ *
+ * Two families:
+ *   host-pointer entry points   drop-in for the bridge (activations/results in host
+ *                               memory, weights device-resident after preload);
+ *   *Device entry points        same contracts with every pointer in device memory;
+ *                               pure kernel launches on the stream set by TSHip_SetStream.
+ */
+#ifndef TSHIP_OPS_H
+#define TSHIP_OPS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TSHIP_EXPORT __attribute__((visibility("default")))
+
+/* Backend ids. 1..3 are the bridge's (TensorSharp.Backends.GGML/GgmlNative.cs:20-25); 4 is new. */
+enum { TSHIP_BACKEND_METAL = 1, TSHIP_BACKEND_CPU = 2, TSHIP_BACKEND_CUDA = 3, TSHIP_BACKEND_HIP = 4 };
+
+enum { TSHIP_TYPE_F32 = 0, TSHIP_TYPE_Q8_0 = 8, TSHIP_TYPE_Q4_K = 12, TSHIP_TYPE_MXFP4 = 39 };
+
+/* TensorSharp.GGML.Native/ggml_ops_internal.h:69-77 == GgmlNative.cs:27-45 (GgmlTensorView2D). */
+typedef struct TSHipTensorView2D {
+    void* data;
+    int dim0;
+    int dim1;
+    int stride0;
+    int stride1;
+    int64_t raw_bytes;
+} TSHipTensorView2D;
+
+/* ggml_ops_internal.h:104-109 == GgmlNative.cs:100-113 (GgmlContiguousTensor). element_type: 0 = F32, 3 = I32. */
+typedef struct TSHipContiguousTensor {
+    void* data;
+    int64_t element_count;
+    int element_type;
+} TSHipContiguousTensor;
+
+/* ---- utilities -------------------------------------------------------------------- */
+
+/* replaces TSGgml_GetLastError (ggml_ops_core.cpp:1117-1120; GgmlNative.cs:211-212) */
+TSHIP_EXPORT const char* TSHip_GetLastError(void);
+
+/* replaces TSGgml_CanInitializeBackend (ggml_ops_core.cpp:1128-1132): 1 iff backendType == HIP and a gfx950
+ * device answers; does not initialise anything. */
+TSHIP_EXPORT int TSHip_CanInitializeBackend(int backendType);
+
+/* replaces TSGgml_IsBackendAvailable (ggml_ops_core.cpp:1134-1138): initialises the process-wide backend. */
+TSHIP_EXPORT int TSHip_IsBackendAvailable(int backendType);
+
+/* replaces TSGgml_RowSize (ggml_ops_core.cpp:1320-1329): bytes of one row, 0 on any error. */
+TSHIP_EXPORT size_t TSHip_RowSize(int ggml_type, int64_t ne);
+
+/* replace TSGgml_AlignedAlloc / TSGgml_AlignedFree (ggml_ops_core.cpp:1140-1164): 16384-byte aligned host memory. */
+TSHIP_EXPORT void* TSHip_AlignedAlloc(size_t size);
+TSHIP_EXPORT void TSHip_AlignedFree(void* ptr);
+
+/* ---- host-pointer entry points (drop-in) ------------------------------------------- */
+
+/* replaces TSGgml_DequantizeToF32 (ggml_ops_core.cpp:1331-1354; GgmlNative.cs:1493-1536).
+ * 0 ok, -1 bad arguments, -2 unsupported type.  Bit-exact with ManagedQuantizedOps.cs:411-427/447-479/579-598. */
+TSHIP_EXPORT int TSHip_DequantizeToF32(int ggml_type, const void* src, int64_t num_elements, float* dst);
+
+/* replaces TSGgml_AddmmQuantF32 (ggml_ops_matmul.cpp:1308-1337, impl :293-516; GgmlNative.cs:231-240).
+ * result[M x N] = m1[M x K] * W[N x K]^T (overwrites).  m2_data is a readable host pointer to the raw GGUF
+ * blocks or a key previously passed to TSHip_PreloadQuantizedWeight. */
+TSHIP_EXPORT int TSHip_AddmmQuantF32(TSHipTensorView2D result, TSHipTensorView2D m1, void* m2_data,
+                                     int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes);
+
+/* replaces TSGgml_AddmmQuantBatchF32 (ggml_ops_matmul.cpp:1370-1401, impl :672-729): row b of m1 times the
+ * sub-weight at byte offset weight_offsets[b] with weight_ne1[b] rows -> row b of result. */
+TSHIP_EXPORT int TSHip_AddmmQuantBatchF32(TSHipTensorView2D result, TSHipTensorView2D m1, void* m2_data,
+                                          int m2_ggml_type, int64_t m2_ne0, int64_t m2_raw_bytes,
+                                          int batch_count, int64_t* weight_offsets, int64_t* weight_ne1_arr);
+
+/* replaces TSGgml_PreloadQuantizedWeight (ggml_ops_core.cpp:1199-1318): upload once, keep the device copy
+ * under cache_key; the host bytes may be released afterwards. */
+TSHIP_EXPORT int TSHip_PreloadQuantizedWeight(void* cache_key, void* host_data, int ggml_type, int64_t ne0,
+                                              int64_t ne1, int64_t raw_bytes);
+
+/* replace TSGgml_InvalidateHostBuffer / TSGgml_ClearHostBufferCache / TSGgml_SyncHostBuffer
+ * (ggml_ops_core.cpp:1166-1197). */
+TSHIP_EXPORT void TSHip_InvalidateHostBuffer(void* ptr);
+TSHIP_EXPORT void TSHip_ClearHostBufferCache(void);
+TSHIP_EXPORT int TSHip_SyncHostBuffer(void* ptr, size_t size);
+
+/* ---- device-pointer entry points ---------------------------------------------------- */
+
+/* No counterpart in the bridge (its tensors are host memory): selects the HIP stream the *Device entry
+ * points launch on (NULL = default stream).  Process-wide. */
+TSHIP_EXPORT int TSHip_SetStream(void* hip_stream);
+
+/* Device form of TSGgml_DequantizeToF32 (same codes). */
+TSHIP_EXPORT int TSHip_DequantizeToF32Device(int ggml_type, const void* src, int64_t num_elements, float* dst);
+
+/* Device form of TSGgml_AddmmQuantF32: result.data, m1.data and m2_data are device pointers; both views
+ * need stride1 == 1.  Asynchronous on the current stream. */
+TSHIP_EXPORT int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D m1, const void* m2_data,
+                                           int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1,
+                                           int64_t m2_raw_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TSHIP_OPS_H */

@@ -1,0 +1,245 @@
+"""TEST INFRASTRUCTURE: ctypes loader for the CPU oracle (liboracle.so) and, where it
+was built, the reference's own ggml CPU code (oracle/_ref/libggml_ref.so).
+
+Only tests, the smoke check and the benchmark's cpu_baseline leg may import this
+module.  The shipped HIP library never depends on it.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+F32, Q8_0, Q4_K, MXFP4 = 0, 8, 12, 39
+TYPES = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
+BLOCK = {F32: (1, 4), Q8_0: (32, 34), Q4_K: (256, 144), MXFP4: (32, 17)}
+
+_f32p = C.POINTER(C.c_float)
+_f64p = C.POINTER(C.c_double)
+_i32p = C.POINTER(C.c_int32)
+
+
+def build(fast=True):
+    """Compile the oracle libraries (gcc only)."""
+    targets = ["liboracle.so"] + (["liboracle_fast.so"] if fast else [])
+    subprocess.run(["make", "-s", "-C", HERE] + targets, check=True)
+
+
+def build_ref(reference="/root/reference"):
+    """Compile the reference's ggml CPU sources in place (only where the checkout exists)."""
+    if not os.path.isdir(reference):
+        return False
+    subprocess.run(["make", "-s", "-j8", "-C", HERE, "ref", f"REF={reference}"], check=True)
+    return True
+
+
+def _ptr(a, ty):
+    return a.ctypes.data_as(ty)
+
+
+def _vp(a):
+    return C.c_void_p(a.ctypes.data)
+
+
+class Oracle:
+    def __init__(self, fast=False):
+        name = "liboracle_fast.so" if fast else "liboracle.so"
+        path = os.path.join(HERE, name)
+        if not os.path.exists(path):
+            build(fast=fast)
+        self.lib = L = C.CDLL(path)
+        L.tso_fp16_to_fp32.restype = C.c_float
+        L.tso_fp16_to_fp32.argtypes = [C.c_uint16]
+        L.tso_fp32_to_fp16.restype = C.c_uint16
+        L.tso_fp32_to_fp16.argtypes = [C.c_float]
+        L.tso_e8m0_to_fp32_half.restype = C.c_float
+        L.tso_e8m0_to_fp32_half.argtypes = [C.c_uint8]
+        for f in (L.tso_block_size, L.tso_type_size):
+            f.restype = C.c_int64
+            f.argtypes = [C.c_int]
+        L.tso_row_size.restype = C.c_int64
+        L.tso_row_size.argtypes = [C.c_int, C.c_int64]
+        L.tso_quantize.restype = C.c_int
+        L.tso_quantize.argtypes = [C.c_int, _f32p, C.c_void_p, C.c_int64]
+        L.tso_quantize_q8_K.restype = None
+        L.tso_quantize_q8_K.argtypes = [_f32p, C.c_void_p, C.c_int64]
+        L.tso_dequantize.restype = C.c_int
+        L.tso_dequantize.argtypes = [C.c_int, C.c_void_p, C.c_int64, _f32p]
+        L.tso_matmul_f64.restype = C.c_int
+        L.tso_matmul_f64.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int64, _f32p, C.c_int64,
+                                     C.c_int64, _f64p]
+        L.tso_matmul_managed.restype = C.c_int
+        L.tso_matmul_managed.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int64, _f32p, C.c_int64,
+                                         C.c_int64, _f32p, C.c_int, C.c_int]
+        L.tso_matmul_ggml.restype = C.c_int
+        L.tso_matmul_ggml.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int64, _f32p, C.c_int64,
+                                      C.c_int64, _f32p, C.c_int]
+        L.tso_moe_route.restype = None
+        L.tso_moe_route.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, _i32p, _f32p]
+        L.tso_moe_group.restype = None
+        L.tso_moe_group.argtypes = [_i32p, _f32p, C.c_int, C.c_int, C.c_int, _i32p, _i32p, _f32p]
+        L.tso_swiglu_oai.restype = None
+        L.tso_swiglu_oai.argtypes = [_f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
+        L.tso_moe_forward.restype = C.c_int
+        L.tso_moe_forward.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_int, C.c_int, C.c_int, _f32p, C.c_int, C.c_int, _i32p,
+                                      _f32p, _f32p]
+        L.tso_max_threads.restype = C.c_int
+
+    # -- helpers ---------------------------------------------------------
+    def row_size(self, t, ne):
+        return int(self.lib.tso_row_size(t, ne))
+
+    def quantize(self, t, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        bs, bb = BLOCK[t]
+        assert x.size % bs == 0
+        out = np.empty(x.size // bs * bb, dtype=np.uint8)
+        rc = self.lib.tso_quantize(t, _ptr(x, _f32p), _vp(out), x.size)
+        assert rc == 0, rc
+        return out
+
+    def quantize_q8_K(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty(x.size // 256 * 292, dtype=np.uint8)
+        self.lib.tso_quantize_q8_K(_ptr(x, _f32p), _vp(out), x.size)
+        return out
+
+    def dequantize(self, t, raw, n=None):
+        raw = np.ascontiguousarray(raw, dtype=np.uint8)
+        bs, bb = BLOCK[t]
+        if n is None:
+            n = raw.size // bb * bs
+        out = np.empty(n, dtype=np.float32)
+        rc = self.lib.tso_dequantize(t, _vp(raw), n, _ptr(out, _f32p))
+        assert rc == 0, rc
+        return out
+
+    def matmul_f64(self, t, w, N, K, x):
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)
+        M = x.shape[0]
+        out = np.empty((M, N), dtype=np.float64)
+        rc = self.lib.tso_matmul_f64(t, _vp(w), N, K, _ptr(x, _f32p), M, K, _ptr(out, _f64p))
+        assert rc == 0, rc
+        return out
+
+    def matmul_managed(self, t, w, N, K, x, vec_width=8, threads=1):
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)
+        M = x.shape[0]
+        out = np.empty((M, N), dtype=np.float32)
+        rc = self.lib.tso_matmul_managed(t, _vp(w), N, K, _ptr(x, _f32p), M, K, _ptr(out, _f32p),
+                                         vec_width, threads)
+        assert rc == 0, rc
+        return out
+
+    def matmul_ggml(self, t, w, N, K, x, threads=1):
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)
+        M = x.shape[0]
+        out = np.empty((M, N), dtype=np.float32)
+        rc = self.lib.tso_matmul_ggml(t, _vp(w), N, K, _ptr(x, _f32p), M, K, _ptr(out, _f32p), threads)
+        assert rc == 0, rc
+        return out
+
+    def moe_route(self, logits, k):
+        logits = np.ascontiguousarray(logits, dtype=np.float32)
+        T, E = logits.shape
+        ids = np.empty((T, k), dtype=np.int32)
+        wts = np.empty((T, k), dtype=np.float32)
+        self.lib.tso_moe_route(_ptr(logits, _f32p), T, E, k, _ptr(ids, _i32p), _ptr(wts, _f32p))
+        return ids, wts
+
+    def moe_group(self, ids, wts, E):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        wts = np.ascontiguousarray(wts, dtype=np.float32)
+        T, k = ids.shape
+        offs = np.empty(E + 1, dtype=np.int32)
+        tmap = np.empty(T * k, dtype=np.int32)
+        wmap = np.empty(T * k, dtype=np.float32)
+        self.lib.tso_moe_group(_ptr(ids, _i32p), _ptr(wts, _f32p), T, E, k, _ptr(offs, _i32p),
+                               _ptr(tmap, _i32p), _ptr(wmap, _f32p))
+        return offs, tmap, wmap
+
+    def swiglu_oai(self, gate_up, alpha=1.702, limit=7.0):
+        gu = np.ascontiguousarray(gate_up, dtype=np.float32)
+        rows, two_f = gu.shape
+        out = np.empty((rows, two_f // 2), dtype=np.float32)
+        self.lib.tso_swiglu_oai(_ptr(gu, _f32p), rows, two_f // 2, alpha, limit, _ptr(out, _f32p))
+        return out
+
+    def moe_forward(self, t, gu_w, gu_b, dn_w, dn_b, E, H, F, hidden, ids, wts):
+        hidden = np.ascontiguousarray(hidden, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        wts = np.ascontiguousarray(wts, dtype=np.float32)
+        T, k = ids.shape
+        out = np.empty((T, H), dtype=np.float32)
+        rc = self.lib.tso_moe_forward(
+            t, _vp(gu_w), None if gu_b is None else _vp(gu_b), _vp(dn_w),
+            None if dn_b is None else _vp(dn_b), E, H, F, _ptr(hidden, _f32p), T, k,
+            _ptr(ids, _i32p), _ptr(wts, _f32p), _ptr(out, _f32p))
+        assert rc == 0, rc
+        return out
+
+
+class Reference:
+    """The reference's own ggml code, compiled from its sources by `make ref`.
+    Exists only where the reference checkout was available at build time."""
+
+    PATH = os.path.join(HERE, "_ref", "libggml_ref.so")
+
+    @classmethod
+    def available(cls):
+        return os.path.exists(cls.PATH)
+
+    def __init__(self):
+        self.lib = L = C.CDLL(self.PATH)
+        L.ref_quantize.restype = C.c_size_t
+        L.ref_quantize.argtypes = [C.c_int, _f32p, C.c_void_p, C.c_int64, C.c_int64]
+        L.ref_dequantize.restype = C.c_int
+        L.ref_dequantize.argtypes = [C.c_int, C.c_void_p, C.c_int64, _f32p]
+        L.ref_row_size.restype = C.c_size_t
+        L.ref_row_size.argtypes = [C.c_int, C.c_int64]
+        L.ref_fp16_to_fp32.restype = C.c_float
+        L.ref_fp16_to_fp32.argtypes = [C.c_uint16]
+        L.ref_fp32_to_fp16.restype = C.c_uint16
+        L.ref_fp32_to_fp16.argtypes = [C.c_float]
+        L.ref_mul_mat.restype = C.c_int
+        L.ref_mul_mat.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int64, _f32p, C.c_int64, _f32p,
+                                  C.c_int]
+        L.quantize_row_q8_K_ref.restype = None
+        L.quantize_row_q8_K_ref.argtypes = [_f32p, C.c_void_p, C.c_int64]
+
+    def quantize(self, t, x, n_per_row=None):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        bs, bb = BLOCK[t]
+        if n_per_row is None:
+            n_per_row = x.size
+        out = np.empty(x.size // bs * bb, dtype=np.uint8)
+        got = self.lib.ref_quantize(t, _ptr(x, _f32p), _vp(out), x.size // n_per_row, n_per_row)
+        assert got == out.size, (got, out.size)
+        return out
+
+    def quantize_q8_K(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        # zero-filled: the reference leaves bsums of an all-zero block unwritten
+        out = np.zeros(x.size // 256 * 292, dtype=np.uint8)
+        self.lib.quantize_row_q8_K_ref(_ptr(x, _f32p), _vp(out), x.size)
+        return out
+
+    def dequantize(self, t, raw, n=None):
+        raw = np.ascontiguousarray(raw, dtype=np.uint8)
+        bs, bb = BLOCK[t]
+        if n is None:
+            n = raw.size // bb * bs
+        out = np.empty(n, dtype=np.float32)
+        assert self.lib.ref_dequantize(t, _vp(raw), n, _ptr(out, _f32p)) == 0
+        return out
+
+    def mul_mat(self, t, w, N, K, x, threads=4):
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)
+        M = x.shape[0]
+        out = np.empty((M, N), dtype=np.float32)
+        rc = self.lib.ref_mul_mat(t, _vp(w), N, K, _ptr(x, _f32p), M, _ptr(out, _f32p), threads)
+        assert rc == 0, rc
+        return out

@@ -1,0 +1,74 @@
+/*
+ * TEST INFRASTRUCTURE — not part of the shipped library.
+ *
+ * CPU restatement of the reference arithmetic for the GGUF quantized-matmul
+ * path (Q8_0 / Q4_K / MXFP4).  Only tests, the smoke check and the
+ * cpu_baseline leg of the benchmark may load this library; the HIP library
+ * never links or calls it.
+ *
+ * Every function cites the reference file:line it restates
+ * (paths relative to the reference checkout).
+ */
+#ifndef TS_ORACLE_H
+#define TS_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGUF tensor type ids: TensorSharp.Runtime/GgufReader.cs:26-37 */
+enum { TSO_TYPE_F32 = 0, TSO_TYPE_Q8_0 = 8, TSO_TYPE_Q4_K = 12, TSO_TYPE_MXFP4 = 39 };
+
+/* scalar helpers */
+float    tso_fp16_to_fp32(uint16_t h);
+uint16_t tso_fp32_to_fp16(float f);
+float    tso_e8m0_to_fp32_half(uint8_t e);
+
+/* type tables */
+int64_t tso_block_size(int type);              /* elements per block, 0 if unsupported */
+int64_t tso_type_size(int type);               /* bytes per block, 0 if unsupported    */
+int64_t tso_row_size(int type, int64_t ne);    /* bytes per row, 0 on error            */
+
+/* weight quantizers (fp32 -> raw GGUF blocks); n must be a block multiple */
+void tso_quantize_q8_0(const float* x, void* dst, int64_t n);
+void tso_quantize_q4_K(const float* x, void* dst, int64_t n);
+void tso_quantize_mxfp4(const float* x, void* dst, int64_t n);
+int  tso_quantize(int type, const float* x, void* dst, int64_t n);
+
+/* dequantizers (raw blocks -> fp32); returns 0 ok, -1 bad args, -2 unsupported */
+int tso_dequantize(int type, const void* src, int64_t n, float* dst);
+
+/* activation quantizers of the ggml CPU path */
+void tso_quantize_q8_K(const float* x, void* dst, int64_t n);
+
+/* matmuls: result[M x N] = x[M x K] * W[N x K]^T ; W raw blocks, row-major */
+int tso_matmul_f64(int type, const void* w, int64_t N, int64_t K,
+                   const float* x, int64_t M, int64_t x_stride, double* out);
+int tso_matmul_managed(int type, const void* w, int64_t N, int64_t K,
+                       const float* x, int64_t M, int64_t x_stride,
+                       float* out, int vec_width, int n_threads);
+int tso_matmul_ggml(int type, const void* w, int64_t N, int64_t K,
+                    const float* x, int64_t M, int64_t x_stride,
+                    float* out, int n_threads);
+
+/* MoE (GPT-OSS) */
+void tso_moe_route(const float* logits, int T, int E, int k, int32_t* ids, float* weights);
+void tso_moe_group(const int32_t* ids, const float* weights, int T, int E, int k,
+                   int32_t* expert_offsets /* E+1 */, int32_t* token_map /* T*k */,
+                   float* weight_map /* T*k */);
+void tso_swiglu_oai(float* gate_up, int rows, int half_dim, float alpha, float limit,
+                    float* out /* rows x half_dim */);
+int tso_moe_forward(int type, const void* gate_up_w, const float* gate_up_b,
+                    const void* down_w, const float* down_b,
+                    int E, int H, int F, const float* hidden, int T, int k,
+                    const int32_t* ids, const float* weights, float* out);
+
+int tso_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

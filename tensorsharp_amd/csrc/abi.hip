@@ -1,0 +1,548 @@
+// C-ABI shim of libTsHipOps: argument validation, error convention, device weight cache and
+// host<->device staging around the gfx950 kernels.  Entry points and their contracts mirror
+// the reference bridge (TensorSharp.GGML.Native/ggml_ops_core.cpp, ggml_ops_matmul.cpp);
+// see include/tship_ops.h for the export-by-export mapping.
+#include "../../include/tship_ops.h"
+#include "tship_internal.h"
+
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace tship {
+
+// ---- error convention: thread-local message, like ggml_ops_core.cpp:89-97 -------------------
+static thread_local std::string g_last_error;
+
+void set_last_error(const std::string& msg) { g_last_error = msg; }
+void clear_last_error() { g_last_error.clear(); }
+
+bool hip_ok(hipError_t e, const char* what)
+{
+    if (e == hipSuccess) return true;
+    set_last_error(std::string(what) + ": " + hipGetErrorString(e));
+    return false;
+}
+
+// ---- backend state ----------------------------------------------------------------------------
+namespace {
+
+std::once_flag g_init_once;
+bool g_backend_ready = false;
+std::string g_init_error;
+DeviceInfo g_device_info{256, 64 * 1024};
+std::atomic<hipStream_t> g_stream{nullptr};
+
+bool probe_device(std::string& err, DeviceInfo* info)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        err = "No HIP device is available.";
+        return false;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        err = "hipGetDeviceProperties failed.";
+        return false;
+    }
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        err = std::string("libTsHipOps is built for gfx950 only; device 0 is ") + prop.gcnArchName + ".";
+        return false;
+    }
+    if (info) {
+        info->num_cus = prop.multiProcessorCount;
+        info->lds_per_block_optin = prop.sharedMemPerBlockOptin ? prop.sharedMemPerBlockOptin : prop.sharedMemPerBlock;
+    }
+    return true;
+}
+
+// One backend per process, initialised once (ggml_ops_core.cpp:169-195).
+bool ensure_backend()
+{
+    std::call_once(g_init_once, [] {
+        g_backend_ready = probe_device(g_init_error, &g_device_info);
+        if (g_backend_ready && hipSetDevice(0) != hipSuccess) {
+            g_backend_ready = false;
+            g_init_error = "hipSetDevice(0) failed.";
+        }
+    });
+    if (!g_backend_ready) set_last_error(g_init_error);
+    return g_backend_ready;
+}
+
+// ---- device copies of weights ---------------------------------------------------------------
+// Keyed by the pointer the caller passes as m2_data: either the key given to
+// TSHip_PreloadQuantizedWeight or the host address of the raw blocks (cached on first use,
+// like the bridge's host-buffer cache, ggml_ops_core.cpp:580-663).
+struct CachedWeight {
+    void* dev = nullptr;
+    size_t bytes = 0;
+    bool preloaded = false;
+};
+std::mutex g_cache_mutex;
+std::unordered_map<const void*, CachedWeight> g_weight_cache;
+
+// Serialises the host-pointer entry points: they share one staging workspace.
+std::mutex g_host_call_mutex;
+
+struct Workspace {
+    void* dev = nullptr;
+    size_t dev_bytes = 0;
+    void* pinned = nullptr;
+    size_t pinned_bytes = 0;
+};
+Workspace g_ws;
+
+bool ws_reserve(size_t dev_bytes, size_t pinned_bytes)
+{
+    if (dev_bytes > g_ws.dev_bytes) {
+        if (g_ws.dev) (void)hipFree(g_ws.dev);
+        g_ws.dev = nullptr;
+        g_ws.dev_bytes = 0;
+        const size_t want = dev_bytes + dev_bytes / 4;
+        if (!hip_ok(hipMalloc(&g_ws.dev, want), "hipMalloc(workspace)")) return false;
+        g_ws.dev_bytes = want;
+    }
+    if (pinned_bytes > g_ws.pinned_bytes) {
+        if (g_ws.pinned) (void)hipHostFree(g_ws.pinned);
+        g_ws.pinned = nullptr;
+        g_ws.pinned_bytes = 0;
+        const size_t want = pinned_bytes + pinned_bytes / 4;
+        if (!hip_ok(hipHostMalloc(&g_ws.pinned, want, hipHostMallocDefault), "hipHostMalloc(workspace)")) return false;
+        g_ws.pinned_bytes = want;
+    }
+    return true;
+}
+
+// ---- descriptor checks (ggml_ops_core.cpp:222-229 required_raw_bytes, :302-330 validate_desc) ----
+size_t required_raw_bytes(const TSHipTensorView2D& d)
+{
+    const int64_t max_off = ((int64_t)d.dim0 - 1) * d.stride0 + ((int64_t)d.dim1 - 1) * d.stride1;
+    return (size_t)((max_off + 1) * (int64_t)sizeof(float));
+}
+
+bool validate_desc(const TSHipTensorView2D& d, const char* name)
+{
+    if (d.data == nullptr) {
+        set_last_error(std::string("Null pointer passed for ") + name + '.');
+        return false;
+    }
+    if (d.dim0 <= 0 || d.dim1 <= 0) {
+        set_last_error(std::string("Invalid tensor shape passed for ") + name + '.');
+        return false;
+    }
+    if (d.stride0 < 0 || d.stride1 < 0) {
+        set_last_error(std::string("Negative tensor strides are not supported for ") + name + '.');
+        return false;
+    }
+    if (d.raw_bytes <= 0 || (d.raw_bytes % (int64_t)sizeof(float)) != 0) {
+        set_last_error(std::string("Invalid raw byte size passed for ") + name + '.');
+        return false;
+    }
+    if ((size_t)d.raw_bytes < required_raw_bytes(d)) {
+        set_last_error(std::string("Raw byte span is too small for ") + name + '.');
+        return false;
+    }
+    return true;
+}
+
+// stride1 == 1 and rows do not overlap (ggml_ops_core.cpp:441-445 can_map_standard_view)
+bool is_standard_view(const TSHipTensorView2D& d)
+{
+    return d.stride1 == 1 && (d.dim0 == 1 || d.stride0 >= d.dim1);
+}
+
+size_t row_size(int type, int64_t ne)
+{
+    const int64_t bs = block_elems(type);
+    if (bs <= 0 || ne <= 0 || ne % bs != 0) return 0;
+    return (size_t)(ne / bs * block_bytes(type));
+}
+
+// shape agreement + weight descriptor, messages as in ggml_ops_matmul.cpp:303-329
+bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* m2_data, int type,
+                          int64_t ne0, int64_t ne1, int64_t raw_bytes)
+{
+    if (!validate_desc(result, "result") || !validate_desc(m1, "m1")) return false;
+    if (m2_data == nullptr || ne0 <= 0 || ne1 <= 0 || raw_bytes <= 0) {
+        set_last_error("Invalid quantized weight descriptor.");
+        return false;
+    }
+    if (m1.dim0 != result.dim0) {
+        set_last_error("Size mismatch: m1.dim0 != result.dim0 in addmm_quant.");
+        return false;
+    }
+    if (ne0 != m1.dim1 || ne1 != result.dim1) {
+        set_last_error("Size mismatch: quantized weight dims don't match in addmm_quant.");
+        return false;
+    }
+    if (!is_quant_type(type)) {
+        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, MXFP4).");
+        return false;
+    }
+    const size_t rs = row_size(type, ne0);
+    if (rs == 0) {
+        set_last_error("Quantized weight row length is not a multiple of the block size.");
+        return false;
+    }
+    if ((size_t)raw_bytes < rs * (size_t)ne1) {
+        set_last_error("Quantized weight byte span is too small for its dimensions.");
+        return false;
+    }
+    return true;
+}
+
+// result/m1/w are device pointers here.
+bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
+                       int64_t N, hipStream_t stream)
+{
+    const size_t w_bytes = row_size(type, K) * (size_t)N;
+    const uintptr_t wa = reinterpret_cast<uintptr_t>(w);
+    const uintptr_t need_align = type == kTypeQ4_K ? 16 : type == kTypeQ8_0 ? 2 : 1;
+    if (wa % need_align != 0) {
+        set_last_error("Quantized weight pointer is not aligned for its block type.");
+        return false;
+    }
+    if ((reinterpret_cast<uintptr_t>(m1.data) & 15) != 0 || (m1.dim0 > 1 && (m1.stride0 & 3) != 0)) {
+        set_last_error("Activation rows must be 16-byte aligned on the device.");
+        return false;
+    }
+    const int M = m1.dim0;
+    if (K <= gemv_max_k(type)) {
+        // decode / small batch: one GEMV per activation row
+        // TODO(prefill): M > 1 goes to the MFMA GEMM once it lands
+        for (int m = 0; m < M; ++m) {
+            const float* x = static_cast<const float*>(m1.data) + (int64_t)m * m1.stride0;
+            float* y = static_cast<float*>(result.data) + (int64_t)m * result.stride0;
+            if (!launch_gemv(type, w, (int64_t)w_bytes, x, y, (int)N, (int)K, stream)) return false;
+        }
+        return true;
+    }
+    set_last_error("addmm_quant: K is too large for this build.");
+    return false;
+}
+
+// device pointer for m2_data: preloaded key, cached host pointer, or upload now
+const void* resolve_weight(void* m2_data, size_t bytes)
+{
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_weight_cache.find(m2_data);
+    if (it != g_weight_cache.end()) {
+        if (it->second.bytes >= bytes) return it->second.dev;
+        if (it->second.preloaded) {
+            set_last_error("Preloaded quantized weight is smaller than the requested view.");
+            return nullptr;
+        }
+        (void)hipFree(it->second.dev);
+        g_weight_cache.erase(it);
+    }
+    CachedWeight cw;
+    if (!hip_ok(hipMalloc(&cw.dev, bytes + 16), "hipMalloc(weight)")) return nullptr;
+    if (!hip_ok(hipMemcpy(cw.dev, m2_data, bytes, hipMemcpyHostToDevice), "hipMemcpy(weight)")) {
+        (void)hipFree(cw.dev);
+        return nullptr;
+    }
+    cw.bytes = bytes;
+    g_weight_cache[m2_data] = cw;
+    return cw.dev;
+}
+
+int addmm_quant_host(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, void* m2_data, int type, int64_t ne0,
+                     int64_t ne1, int64_t raw_bytes)
+{
+    if (!ensure_backend()) return 0;
+    if (!validate_addmm_quant(result, m1, m2_data, type, ne0, ne1, raw_bytes)) return 0;
+    if (!is_standard_view(result)) {
+        set_last_error("result must be a standard (stride1 == 1, non-overlapping) view in addmm_quant.");
+        return 0;
+    }
+    const int M = m1.dim0;
+    const int64_t K = ne0, N = ne1;
+    const size_t w_bytes = row_size(type, K) * (size_t)N;
+    const void* w_dev = resolve_weight(m2_data, w_bytes);
+    if (!w_dev) return 0;
+
+    std::lock_guard<std::mutex> lock(g_host_call_mutex);
+    const size_t x_bytes = (size_t)M * K * sizeof(float);
+    const size_t y_bytes = (size_t)M * N * sizeof(float);
+    const size_t x_off = 0, y_off = (x_bytes + 255) & ~(size_t)255;
+    if (!ws_reserve(y_off + y_bytes, std::max(x_bytes, y_bytes))) return 0;
+    float* x_dev = reinterpret_cast<float*>(static_cast<char*>(g_ws.dev) + x_off);
+    float* y_dev = reinterpret_cast<float*>(static_cast<char*>(g_ws.dev) + y_off);
+
+    // pack the (possibly strided) activation view into pinned memory, then one H2D copy
+    float* stage = static_cast<float*>(g_ws.pinned);
+    const float* src = static_cast<const float*>(m1.data);
+    if (m1.stride1 == 1) {
+        for (int m = 0; m < M; ++m) std::memcpy(stage + (size_t)m * K, src + (size_t)m * m1.stride0, (size_t)K * sizeof(float));
+    } else {
+        for (int m = 0; m < M; ++m)
+            for (int64_t k = 0; k < K; ++k) stage[(size_t)m * K + k] = src[(size_t)m * m1.stride0 + (size_t)k * m1.stride1];
+    }
+    hipStream_t stream = nullptr;
+    if (!hip_ok(hipMemcpyAsync(x_dev, stage, x_bytes, hipMemcpyHostToDevice, stream), "hipMemcpy(activations)")) return 0;
+
+    TSHipTensorView2D r_dev{y_dev, M, (int)N, (int)N, 1, (int64_t)y_bytes};
+    TSHipTensorView2D x_desc{x_dev, M, (int)K, (int)K, 1, (int64_t)x_bytes};
+    if (!run_matmul_device(r_dev, x_desc, w_dev, type, K, N, stream)) return 0;
+
+    if (!hip_ok(hipMemcpyAsync(stage, y_dev, y_bytes, hipMemcpyDeviceToHost, stream), "hipMemcpy(result)")) return 0;
+    if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+    float* dst = static_cast<float*>(result.data);
+    for (int m = 0; m < M; ++m) std::memcpy(dst + (size_t)m * result.stride0, stage + (size_t)m * N, (size_t)N * sizeof(float));
+    clear_last_error();
+    return 1;
+}
+
+}  // namespace
+
+const DeviceInfo& device_info() { return g_device_info; }
+
+}  // namespace tship
+
+using namespace tship;
+
+// Nothing unwinds across the ABI (ggml_ops_matmul.cpp:1317-1336 pattern).
+template <typename F>
+static int guarded(int fallback, const char* what, F&& body)
+{
+    try {
+        return body();
+    } catch (const std::exception& ex) {
+        set_last_error(ex.what());
+        return fallback;
+    } catch (...) {
+        set_last_error(std::string("Unknown HIP ") + what + " failure.");
+        return fallback;
+    }
+}
+
+extern "C" {
+
+const char* TSHip_GetLastError(void) { return g_last_error.c_str(); }
+
+int TSHip_CanInitializeBackend(int backendType)
+{
+    clear_last_error();
+    if (backendType != TSHIP_BACKEND_HIP) return 0;
+    std::string err;
+    if (probe_device(err, nullptr)) return 1;
+    set_last_error(err);
+    return 0;
+}
+
+int TSHip_IsBackendAvailable(int backendType)
+{
+    clear_last_error();
+    if (backendType != TSHIP_BACKEND_HIP) {
+        set_last_error("libTsHipOps provides the HIP backend only.");
+        return 0;
+    }
+    return ensure_backend() ? 1 : 0;
+}
+
+size_t TSHip_RowSize(int ggml_type, int64_t ne) { return row_size(ggml_type, ne); }
+
+void* TSHip_AlignedAlloc(size_t size)
+{
+    if (size == 0) return nullptr;
+    void* p = nullptr;
+    if (posix_memalign(&p, 16384, size) != 0) return nullptr;
+    return p;
+}
+
+void TSHip_AlignedFree(void* ptr)
+{
+    if (ptr) free(ptr);
+}
+
+int TSHip_SetStream(void* hip_stream)
+{
+    g_stream.store(static_cast<hipStream_t>(hip_stream));
+    clear_last_error();
+    return 1;
+}
+
+int TSHip_DequantizeToF32Device(int ggml_type, const void* src, int64_t num_elements, float* dst)
+{
+    return guarded(-1, "dequantize", [&]() -> int {
+        if (src == nullptr || dst == nullptr || num_elements < 0) return -1;
+        if (num_elements == 0) return 0;
+        if (ggml_type != kTypeF32 && !is_quant_type(ggml_type)) return -2;
+        if (!ensure_backend()) return -1;
+        if (ggml_type == kTypeF32)
+            return hip_ok(hipMemcpyAsync(dst, src, (size_t)num_elements * 4, hipMemcpyDeviceToDevice, g_stream.load()),
+                          "hipMemcpy")
+                       ? 0
+                       : -1;
+        if (num_elements % block_elems(ggml_type) != 0) return -1;
+        return launch_dequant(ggml_type, src, num_elements, dst, g_stream.load()) ? 0 : -1;
+    });
+}
+
+int TSHip_DequantizeToF32(int ggml_type, const void* src, int64_t num_elements, float* dst)
+{
+    return guarded(-1, "dequantize", [&]() -> int {
+        if (src == nullptr || dst == nullptr || num_elements < 0) return -1;
+        if (num_elements == 0) return 0;
+        if (ggml_type == kTypeF32) {
+            std::memcpy(dst, src, (size_t)num_elements * sizeof(float));
+            return 0;
+        }
+        if (!is_quant_type(ggml_type)) return -2;
+        if (num_elements % block_elems(ggml_type) != 0) return -1;
+        if (!ensure_backend()) return -1;
+        const size_t in_bytes = row_size(ggml_type, num_elements);
+        const size_t out_bytes = (size_t)num_elements * sizeof(float);
+        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        const size_t out_off = (in_bytes + 255) & ~(size_t)255;
+        if (!ws_reserve(out_off + out_bytes, 0)) return -1;
+        char* base = static_cast<char*>(g_ws.dev);
+        if (!hip_ok(hipMemcpy(base, src, in_bytes, hipMemcpyHostToDevice), "hipMemcpy(src)")) return -1;
+        if (!launch_dequant(ggml_type, base, num_elements, reinterpret_cast<float*>(base + out_off), nullptr)) return -1;
+        if (!hip_ok(hipMemcpy(dst, base + out_off, out_bytes, hipMemcpyDeviceToHost), "hipMemcpy(dst)")) return -1;
+        return 0;
+    });
+}
+
+int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D m1, const void* m2_data, int m2_ggml_type,
+                              int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "addmm_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_addmm_quant(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes)) return 0;
+        if (!is_standard_view(result) || m1.stride1 != 1) {
+            set_last_error("Device addmm_quant needs stride1 == 1 views.");
+            return 0;
+        }
+        if (!run_matmul_device(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load())) return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_AddmmQuantF32(TSHipTensorView2D result, TSHipTensorView2D m1, void* m2_data, int m2_ggml_type, int64_t m2_ne0,
+                        int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "addmm_quant", [&]() -> int {
+        return addmm_quant_host(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes);
+    });
+}
+
+int TSHip_AddmmQuantBatchF32(TSHipTensorView2D result, TSHipTensorView2D m1, void* m2_data, int m2_ggml_type,
+                             int64_t m2_ne0, int64_t m2_raw_bytes, int batch_count, int64_t* weight_offsets,
+                             int64_t* weight_ne1_arr)
+{
+    return guarded(0, "addmm_quant_batch", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_desc(result, "result") || !validate_desc(m1, "m1")) return 0;
+        if (m2_data == nullptr || batch_count <= 0 || weight_offsets == nullptr || weight_ne1_arr == nullptr) {
+            set_last_error("Invalid arguments for addmm_quant_batch.");
+            return 0;
+        }
+        const size_t rs = row_size(m2_ggml_type, m2_ne0);
+        if (!is_quant_type(m2_ggml_type) || rs == 0) {
+            set_last_error("Unsupported quantized weight type or row length for addmm_quant_batch.");
+            return 0;
+        }
+        if (batch_count > result.dim0 || batch_count > m1.dim0) {
+            set_last_error("addmm_quant_batch: batch_count exceeds the number of rows.");
+            return 0;
+        }
+        // row b of m1 times the sub-weight at weight_offsets[b] -> row b of result (ggml_ops_matmul.cpp:672-729)
+        for (int b = 0; b < batch_count; ++b) {
+            const int64_t ne1 = weight_ne1_arr[b], off = weight_offsets[b];
+            if (off < 0 || ne1 <= 0 || (size_t)off + (size_t)ne1 * rs > (size_t)m2_raw_bytes) {
+                set_last_error("addmm_quant_batch: sub-weight lies outside the weight bytes.");
+                return 0;
+            }
+            TSHipTensorView2D r = result;
+            r.dim0 = 1;
+            r.data = static_cast<char*>(result.data) + (size_t)b * result.stride0 * sizeof(float);
+            r.raw_bytes = (int64_t)r.dim1 * (int64_t)sizeof(float);
+            TSHipTensorView2D x = m1;
+            x.dim0 = 1;
+            x.data = static_cast<char*>(m1.data) + (size_t)b * m1.stride0 * sizeof(float);
+            x.raw_bytes = (int64_t)required_raw_bytes(x);
+            void* sub = static_cast<char*>(m2_data) + off;
+            if (!addmm_quant_host(r, x, sub, m2_ggml_type, m2_ne0, ne1, (int64_t)((size_t)ne1 * rs))) return 0;
+        }
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_PreloadQuantizedWeight(void* cache_key, void* host_data, int ggml_type, int64_t ne0, int64_t ne1,
+                                 int64_t raw_bytes)
+{
+    return guarded(0, "preload", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (cache_key == nullptr || host_data == nullptr || ne0 <= 0 || ne1 <= 0 || raw_bytes <= 0) {
+            set_last_error("Invalid arguments for quantized weight preload.");
+            return 0;
+        }
+        const size_t rs = row_size(ggml_type, ne0);
+        if (!is_quant_type(ggml_type) || rs == 0 || (size_t)raw_bytes < rs * (size_t)ne1) {
+            set_last_error("Unsupported type or inconsistent size for quantized weight preload.");
+            return 0;
+        }
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        auto it = g_weight_cache.find(cache_key);
+        if (it != g_weight_cache.end()) {
+            if (it->second.preloaded && it->second.bytes == (size_t)raw_bytes) {
+                clear_last_error();
+                return 1;  // idempotent
+            }
+            (void)hipFree(it->second.dev);
+            g_weight_cache.erase(it);
+        }
+        CachedWeight cw;
+        if (!hip_ok(hipMalloc(&cw.dev, (size_t)raw_bytes + 16), "hipMalloc(preload)")) return 0;
+        if (!hip_ok(hipMemcpy(cw.dev, host_data, (size_t)raw_bytes, hipMemcpyHostToDevice), "hipMemcpy(preload)")) {
+            (void)hipFree(cw.dev);
+            return 0;
+        }
+        cw.bytes = (size_t)raw_bytes;
+        cw.preloaded = true;
+        g_weight_cache[cache_key] = cw;
+        clear_last_error();
+        return 1;
+    });
+}
+
+void TSHip_InvalidateHostBuffer(void* ptr)
+{
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_weight_cache.find(ptr);
+    if (it == g_weight_cache.end()) return;
+    (void)hipFree(it->second.dev);
+    g_weight_cache.erase(it);
+}
+
+void TSHip_ClearHostBufferCache(void)
+{
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for (auto& kv : g_weight_cache) (void)hipFree(kv.second.dev);
+    g_weight_cache.clear();
+}
+
+int TSHip_SyncHostBuffer(void* ptr, size_t size)
+{
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_weight_cache.find(ptr);
+    if (it == g_weight_cache.end() || it->second.preloaded || ptr == nullptr || size > it->second.bytes) {
+        set_last_error("Failed to synchronize cached HIP device buffer back to host memory.");
+        return 0;
+    }
+    if (!hip_ok(hipMemcpy(ptr, it->second.dev, size, hipMemcpyDeviceToHost), "hipMemcpy(sync)")) return 0;
+    clear_last_error();
+    return 1;
+}
+
+}  // extern "C"

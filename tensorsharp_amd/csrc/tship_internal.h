@@ -1,0 +1,64 @@
+// Internal declarations shared by the C-ABI shim and the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+namespace tship {
+
+constexpr int kTypeF32 = 0;
+constexpr int kTypeQ8_0 = 8;
+constexpr int kTypeQ4_K = 12;
+constexpr int kTypeMXFP4 = 39;
+
+// elements per block / bytes per block; 0 for unsupported types
+// (sizes: TensorSharp.Runtime/GgufReader.cs:303-369)
+inline int64_t block_elems(int type)
+{
+    switch (type) {
+    case kTypeF32: return 1;
+    case kTypeQ8_0: return 32;
+    case kTypeQ4_K: return 256;
+    case kTypeMXFP4: return 32;
+    default: return 0;
+    }
+}
+
+inline int64_t block_bytes(int type)
+{
+    switch (type) {
+    case kTypeF32: return 4;
+    case kTypeQ8_0: return 34;
+    case kTypeQ4_K: return 144;
+    case kTypeMXFP4: return 17;
+    default: return 0;
+    }
+}
+
+inline bool is_quant_type(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4; }
+
+void set_last_error(const std::string& msg);
+void clear_last_error();
+bool hip_ok(hipError_t e, const char* what);   // sets last error on failure
+
+struct DeviceInfo {
+    int num_cus;
+    size_t lds_per_block_optin;
+};
+const DeviceInfo& device_info();
+
+// ---- kernel launchers (all asynchronous on `stream`; return false + last error on bad launch) ----
+
+// dst[n] fp32 = dequant(src); bit-exact with the managed dequantizers.
+bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_t stream);
+
+// y[N] = W[N x K] * x[K]; W raw GGUF blocks, row-major; w_bytes = N * row_size.
+bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K,
+                 hipStream_t stream);
+// largest K the GEMV kernel stages in LDS for this type
+int gemv_max_k(int type);
+
+}  // namespace tship

@@ -1,0 +1,177 @@
+"""Host-side operator facade of the HIP backend — the Python twin of a `HipBasicOps` class.
+
+Names, argument meaning and error behaviour follow the quantized entry points of
+TensorSharp.Backends.GGML/GgmlBasicOps.cs (:313-329 AddmmQuant, :689-704 AddmmQuantBatch,
+:706-709 PreloadQuantizedWeight) and GgmlGgufTensorDequant.cs (:9-33 row size, :36-86 dequant).
+ArgumentException -> ValueError, NotSupportedException -> NotImplementedError,
+InvalidOperationException (native failure) -> RuntimeError.
+
+Host tensors are numpy float32 arrays (the reference's tensors are host memory); device
+tensors are torch CUDA tensors, which only supply memory and the stream.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import hip_native as N
+
+
+class QuantizedWeight:
+    """Raw GGUF blocks of one 2-D weight: the fields of ModelBase.QuantizedWeight
+    (TensorSharp.Models/ModelBase.cs:24-202) that the matmul boundary consumes."""
+
+    def __init__(self, data, ggml_type, ne0, ne1):
+        self.ggml_type = int(ggml_type)
+        self.ne0 = int(ne0)   # K, in features
+        self.ne1 = int(ne1)   # N, out features
+        self.data = data      # numpy uint8 (host) or torch uint8 CUDA tensor (device)
+        self.raw_bytes = int(data.numel() if hasattr(data, "numel") else data.size)
+        expect = HipBasicOps.GetRowSizeBytes(self.ggml_type, self.ne0) * self.ne1
+        if self.raw_bytes < expect:
+            raise ValueError(f"weight bytes {self.raw_bytes} < {expect} for {ne1}x{ne0} type {ggml_type}")
+
+    @property
+    def is_device(self):
+        return hasattr(self.data, "data_ptr")
+
+    @property
+    def ptr(self):
+        return self.data.data_ptr() if self.is_device else self.data.ctypes.data
+
+
+def _host_view(a, standard):
+    if not isinstance(a, np.ndarray) or a.ndim != 2:
+        raise ValueError("AddmmQuant requires 2D tensors for result and m1.")
+    if a.dtype != np.float32:
+        raise ValueError("AddmmQuant requires Float32 tensors for result and m1.")
+    s0, s1 = a.strides[0] // 4, a.strides[1] // 4
+    if a.strides[0] % 4 or a.strides[1] % 4 or s0 < 0 or s1 < 0 or (standard and s1 != 1):
+        raise NotImplementedError("HIP AddmmQuant requires tensors with supported row-contiguous layouts.")
+    span = ((a.shape[0] - 1) * s0 + (a.shape[1] - 1) * s1 + 1) * 4
+    return N.TensorView2D(a.ctypes.data, a.shape[0], a.shape[1], s0, s1, span)
+
+
+def _device_view(t):
+    import torch
+    if not isinstance(t, torch.Tensor) or t.dim() != 2:
+        raise ValueError("AddmmQuant requires 2D tensors for result and m1.")
+    if t.dtype != torch.float32:
+        raise ValueError("AddmmQuant requires Float32 tensors for result and m1.")
+    if not t.is_cuda:
+        raise ValueError("device AddmmQuant requires tensors in GPU memory.")
+    s0, s1 = t.stride()
+    if s1 != 1 and t.shape[1] > 1:
+        raise NotImplementedError("HIP AddmmQuant requires tensors with supported row-contiguous layouts.")
+    span = ((t.shape[0] - 1) * s0 + (t.shape[1] - 1) + 1) * 4
+    return N.TensorView2D(t.data_ptr(), t.shape[0], t.shape[1], s0, 1, span)
+
+
+class HipBasicOps:
+    """Static quantized-matmul entry points of the HIP backend."""
+
+    @staticmethod
+    def IsAvailable():
+        return N.lib().TSHip_IsBackendAvailable(N.BACKEND_HIP) == 1
+
+    @staticmethod
+    def GetRowSizeBytes(ggml_type, ne0):
+        rb = N.lib().TSHip_RowSize(int(ggml_type), int(ne0))
+        if rb <= 0:
+            raise NotImplementedError(
+                f"GGML tensor type {ggml_type} is not supported, or ne[0]={ne0} is not aligned to the type block size.")
+        return int(rb)
+
+    # -- dequantization -------------------------------------------------------------------
+    @staticmethod
+    def DequantizeToFloat32(ggml_type, src, num_elements):
+        """Host bytes -> host fp32 (computed on the GPU).  Codes as GgmlNative.cs:1493-1503."""
+        if not isinstance(src, np.ndarray) or src.dtype != np.uint8:
+            raise ValueError("Source must be a uint8 array.")
+        if num_elements < 0:
+            raise ValueError("numElements out of range.")
+        dst = np.empty(int(num_elements), dtype=np.float32)
+        rc = N.lib().TSHip_DequantizeToF32(int(ggml_type), src.ctypes.data, int(num_elements), dst.ctypes.data)
+        if rc == -2:
+            raise NotImplementedError(f"HIP backend cannot dequantize GGUF tensor type {ggml_type}.")
+        if rc != 0:
+            raise RuntimeError(f"Native HIP dequantization failed (code {rc}): {N.get_last_error()}")
+        return dst
+
+    @staticmethod
+    def DequantizeToFloat32Device(ggml_type, src, num_elements, dst=None):
+        import torch
+        if dst is None:
+            dst = torch.empty(int(num_elements), dtype=torch.float32, device=src.device)
+        HipBasicOps.UseCurrentStream()
+        rc = N.lib().TSHip_DequantizeToF32Device(int(ggml_type), src.data_ptr(), int(num_elements), dst.data_ptr())
+        if rc == -2:
+            raise NotImplementedError(f"HIP backend cannot dequantize GGUF tensor type {ggml_type}.")
+        if rc != 0:
+            raise RuntimeError(f"Native HIP dequantization failed (code {rc}): {N.get_last_error()}")
+        return dst
+
+    # -- matmul ---------------------------------------------------------------------------
+    @staticmethod
+    def AddmmQuant(result, m1, weight_data, ggml_type, ne0, ne1, raw_bytes):
+        """result = m1 * W^T with host tensors (GgmlBasicOps.cs:313-329). weight_data: address (int)."""
+        rv = _host_view(result, standard=True)
+        mv = _host_view(m1, standard=False)
+        ok = N.lib().TSHip_AddmmQuantF32(rv, mv, C.c_void_p(weight_data), int(ggml_type), int(ne0), int(ne1),
+                                         int(raw_bytes))
+        N.check_result(ok, "addmm_quant")
+
+    @staticmethod
+    def AddmmQuantDevice(result, m1, weight_data, ggml_type, ne0, ne1, raw_bytes):
+        """Same contract with every pointer in device memory; asynchronous on the current stream."""
+        rv = _device_view(result)
+        mv = _device_view(m1)
+        ok = N.lib().TSHip_AddmmQuantF32Device(rv, mv, C.c_void_p(weight_data), int(ggml_type), int(ne0), int(ne1),
+                                               int(raw_bytes))
+        N.check_result(ok, "addmm_quant")
+
+    @staticmethod
+    def AddmmQuantBatch(result, m1, weight_data, ggml_type, ne0, raw_bytes, weight_offsets, weight_ne1):
+        """Row b of m1 times the sub-weight at weight_offsets[b] (GgmlBasicOps.cs:689-704)."""
+        rv = _host_view(result, standard=True)
+        mv = _host_view(m1, standard=False)
+        n = len(weight_offsets)
+        if n != len(weight_ne1):
+            raise ValueError("weight_offsets and weight_ne1 must have the same length.")
+        offs = (C.c_int64 * n)(*[int(v) for v in weight_offsets])
+        ne1s = (C.c_int64 * n)(*[int(v) for v in weight_ne1])
+        ok = N.lib().TSHip_AddmmQuantBatchF32(rv, mv, C.c_void_p(weight_data), int(ggml_type), int(ne0),
+                                              int(raw_bytes), n, offs, ne1s)
+        N.check_result(ok, "addmm_quant_batch")
+
+    @staticmethod
+    def PreloadQuantizedWeight(cache_key, host_data, ggml_type, ne0, ne1, raw_bytes):
+        ok = N.lib().TSHip_PreloadQuantizedWeight(C.c_void_p(cache_key), C.c_void_p(host_data), int(ggml_type),
+                                                  int(ne0), int(ne1), int(raw_bytes))
+        N.check_result(ok, "preload_quantized_weight")
+
+    @staticmethod
+    def InvalidateHostBuffer(ptr):
+        N.lib().TSHip_InvalidateHostBuffer(C.c_void_p(ptr))
+
+    @staticmethod
+    def ClearHostBufferCache():
+        N.lib().TSHip_ClearHostBufferCache()
+
+    # -- LinearForward twin (ModelBase.cs:875-905): allocate result, route by residency -----
+    @staticmethod
+    def LinearForward(m1, qw: QuantizedWeight):
+        if qw.is_device:
+            import torch
+            result = torch.empty((m1.shape[0], qw.ne1), dtype=torch.float32, device=m1.device)
+            HipBasicOps.UseCurrentStream()
+            HipBasicOps.AddmmQuantDevice(result, m1, qw.ptr, qw.ggml_type, qw.ne0, qw.ne1, qw.raw_bytes)
+            return result
+        result = np.empty((m1.shape[0], qw.ne1), dtype=np.float32)
+        HipBasicOps.AddmmQuant(result, m1, qw.ptr, qw.ggml_type, qw.ne0, qw.ne1, qw.raw_bytes)
+        return result
+
+    @staticmethod
+    def UseCurrentStream():
+        """Launch the *Device entry points on torch's current stream."""
+        import torch
+        N.lib().TSHip_SetStream(C.c_void_p(torch.cuda.current_stream().cuda_stream))

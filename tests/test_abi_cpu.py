@@ -1,0 +1,100 @@
+"""C-ABI surface checks that need no GPU: the library loads, exports every symbol the header
+declares, keeps the bridge's struct layout, and fails loudly (never silently) without a device."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from tensorsharp_amd import hip_native as N
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_exports():
+    text = open(os.path.join(ROOT, "include", "tship_ops.h")).read()
+    return sorted(set(re.findall(r"TSHIP_EXPORT[^;]*?\b(TSHip_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = declared_exports()
+    assert len(names) >= 16
+    lib = N.lib()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in tship_ops.h but not exported"
+        assert n in N.SIGNATURES, f"{n} has no ctypes signature in hip_native.py"
+    assert sorted(N.SIGNATURES) == names
+
+
+def test_struct_layout_matches_bridge():
+    # TensorView2DDesc is 32 bytes, ContiguousTensorDesc 24 (ggml_ops_internal.h:69-109)
+    assert C.sizeof(N.TensorView2D) == 32
+    assert N.TensorView2D.raw_bytes.offset == 24
+    assert C.sizeof(N.ContiguousTensor) == 24
+
+
+def test_row_size_contract():
+    f = N.lib().TSHip_RowSize
+    assert f(N.TYPE_Q8_0, 2560) == 80 * 34
+    assert f(N.TYPE_Q4_K, 4096) == 16 * 144
+    assert f(N.TYPE_MXFP4, 2880) == 90 * 17
+    assert f(N.TYPE_F32, 7) == 28
+    # 0 on unknown type, non-positive ne, ne not a block multiple (ggml_ops_core.cpp:1320-1329)
+    assert f(N.TYPE_Q4_K, 4000) == 0
+    assert f(N.TYPE_Q8_0, 0) == 0
+    assert f(N.TYPE_Q8_0, -32) == 0
+    assert f(1234, 256) == 0
+
+
+def test_aligned_alloc():
+    lib = N.lib()
+    p = lib.TSHip_AlignedAlloc(1000)
+    assert p and p % 16384 == 0
+    lib.TSHip_AlignedFree(p)
+    assert lib.TSHip_AlignedAlloc(0) is None
+    lib.TSHip_AlignedFree(None)
+
+
+def test_backend_ids():
+    lib = N.lib()
+    for other in (1, 2, 3, 0, 99):
+        assert lib.TSHip_CanInitializeBackend(other) == 0
+        assert lib.TSHip_IsBackendAvailable(other) == 0
+
+
+def _no_gpu():
+    import torch
+    return not torch.cuda.is_available()
+
+
+@pytest.mark.skipif(not _no_gpu(), reason="checks the no-device behaviour")
+def test_compute_calls_fail_loudly_without_a_device():
+    from tensorsharp_amd import HipBasicOps
+    lib = N.lib()
+    assert lib.TSHip_IsBackendAvailable(N.BACKEND_HIP) == 0
+    assert "HIP device" in N.get_last_error()
+    w = np.zeros(34 * 4, dtype=np.uint8)
+    x = np.zeros((1, 64), dtype=np.float32)
+    y = np.zeros((1, 2), dtype=np.float32)
+    with pytest.raises(RuntimeError, match="addmm_quant failed"):
+        HipBasicOps.AddmmQuant(y, x, w.ctypes.data, N.TYPE_Q8_0, 64, 2, w.size)
+    with pytest.raises(RuntimeError):
+        HipBasicOps.DequantizeToFloat32(N.TYPE_Q8_0, w, 128)
+    # argument errors that are decided before the device is touched keep the bridge's codes
+    assert lib.TSHip_DequantizeToF32(N.TYPE_Q8_0, None, 32, y.ctypes.data) == -1
+    assert lib.TSHip_DequantizeToF32(77, w.ctypes.data, 32, y.ctypes.data) == -2
+    assert lib.TSHip_DequantizeToF32(N.TYPE_Q8_0, w.ctypes.data, 0, y.ctypes.data) == 0
+
+
+def test_facade_argument_errors_mirror_the_reference():
+    from tensorsharp_amd import HipBasicOps
+    w = np.zeros(34 * 4, dtype=np.uint8)
+    with pytest.raises(ValueError, match="2D"):
+        HipBasicOps.AddmmQuant(np.zeros(4, np.float32), np.zeros((1, 64), np.float32), w.ctypes.data, 8, 64, 2, w.size)
+    with pytest.raises(ValueError, match="Float32"):
+        HipBasicOps.AddmmQuant(np.zeros((1, 2), np.float64), np.zeros((1, 64), np.float32), w.ctypes.data, 8, 64, 2, w.size)
+    with pytest.raises(NotImplementedError):      # result must be row-contiguous (TryCreateStandardView)
+        HipBasicOps.AddmmQuant(np.zeros((1, 4), np.float32)[:, ::2], np.zeros((1, 64), np.float32), w.ctypes.data, 8, 64, 2, w.size)
+    with pytest.raises(NotImplementedError, match="block size"):
+        HipBasicOps.GetRowSizeBytes(N.TYPE_Q4_K, 100)

@@ -1,0 +1,81 @@
+"""GPU parity: dequantization through the C ABI is bit-exact with the oracle."""
+import numpy as np
+import pytest
+
+import inputs
+from oracle.oracle import Q8_0, Q4_K, MXFP4
+
+pytestmark = pytest.mark.gpu
+T = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
+BB = {"q8_0": 34, "q4_k": 144, "mxfp4": 17}
+
+
+def bits_equal(a, b):
+    a = np.asarray(a, dtype=np.float32).view(np.uint32)
+    b = np.asarray(b, dtype=np.float32).view(np.uint32)
+    nan = (b & 0x7FFFFFFF) > 0x7F800000
+    return np.array_equal(a[~nan], b[~nan]) and np.all(((a[nan] & 0x7FFFFFFF) > 0x7F800000))
+
+
+def test_reference_unit_test_vectors(hip, golden):
+    for name in ("q8_0", "q4_k"):
+        y = hip.DequantizeToFloat32(T[name], golden[f"ref_tests_{name}_raw"], 32 if name == "q8_0" else 256)
+        np.testing.assert_array_equal(y[golden[f"ref_tests_{name}_expect_idx"]], golden[f"ref_tests_{name}_expect_val"])
+
+
+def test_golden_blocks(hip, golden):
+    for name, t in T.items():
+        q = golden[f"blocks_{name}_q"]
+        want = golden[f"blocks_{name}_deq"]
+        assert bits_equal(hip.DequantizeToFloat32(t, q, want.size), want), name
+
+
+def test_all_fp16_scales_q8_0(hip, oracle):
+    codes = np.arange(65536, dtype=np.uint16)
+    raw = np.zeros((65536, 34), dtype=np.uint8)
+    raw[:, 0], raw[:, 1] = codes & 0xFF, codes >> 8
+    raw[:, 2:] = ((np.arange(32)[None, :] * 37 + codes[:, None] * 11) % 256).astype(np.uint8)
+    raw = raw.reshape(-1)
+    assert bits_equal(hip.DequantizeToFloat32(Q8_0, raw, 65536 * 32), oracle.dequantize(Q8_0, raw))
+
+
+def test_all_e8m0_codes_mxfp4(hip, oracle):
+    raw = np.zeros((256, 16, 17), dtype=np.uint8)
+    raw[:, :, 0] = np.arange(256, dtype=np.uint8)[:, None]
+    raw[:, :, 1:] = np.arange(256, dtype=np.uint8).reshape(16, 16)[None]
+    raw = raw.reshape(-1)
+    assert bits_equal(hip.DequantizeToFloat32(MXFP4, raw, 256 * 16 * 32), oracle.dequantize(MXFP4, raw))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+def test_random_bytes_host_and_device_entry(hip, oracle, name):
+    import torch
+    rng = np.random.default_rng(21)
+    raw = rng.integers(0, 256, size=BB[name] * 20000, dtype=np.uint8)
+    want = oracle.dequantize(T[name], raw)
+    assert bits_equal(hip.DequantizeToFloat32(T[name], raw, want.size), want)
+    dev = torch.from_numpy(raw).cuda()
+    out = hip.DequantizeToFloat32Device(T[name], dev, want.size)
+    torch.cuda.synchronize()
+    assert bits_equal(out.cpu().numpy(), want)
+
+
+def test_full_size_weight(hip, oracle):
+    # cfg 2 gate projection, 58.7 M weights, reference-quantized
+    fmt, N, K = inputs.CFG2["gate"]
+    q = oracle.quantize(T[fmt], inputs.weights("cfg2.gate", N * K))
+    assert bits_equal(hip.DequantizeToFloat32(T[fmt], q, N * K), oracle.dequantize(T[fmt], q))
+
+
+def test_codes(hip):
+    from tensorsharp_amd import hip_native as N
+    lib = N.lib()
+    buf = np.zeros(144, dtype=np.uint8)
+    out = np.zeros(256, dtype=np.float32)
+    assert lib.TSHip_DequantizeToF32(Q4_K, None, 256, out.ctypes.data) == -1
+    assert lib.TSHip_DequantizeToF32(Q4_K, buf.ctypes.data, 255, out.ctypes.data) == -1
+    assert lib.TSHip_DequantizeToF32(14, buf.ctypes.data, 256, out.ctypes.data) == -2     # Q6_K: not on this path
+    assert lib.TSHip_DequantizeToF32(Q4_K, buf.ctypes.data, 0, out.ctypes.data) == 0
+    src = np.arange(8, dtype=np.float32)
+    dst = np.zeros(8, dtype=np.float32)
+    assert lib.TSHip_DequantizeToF32(0, src.ctypes.data, 8, dst.ctypes.data) == 0 and np.array_equal(src, dst)

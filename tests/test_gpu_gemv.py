@@ -1,0 +1,166 @@
+"""GPU parity: decode GEMV through the C ABI against the oracle.
+
+Bar: max_j |y[m,j] - ref[m,j]| / ||ref[m,:]||_2 <= 1e-3 per output row, ref = fp64 product of the
+bit-exact dequantised weights with the fp32 activations.  The stricter max|delta|/rms(ref row)
+is asserted too, at 1e-4 for the fp32 Q8_0 path and 5e-3 for the fp16-activation 4-bit paths.
+"""
+import numpy as np
+import pytest
+
+import inputs
+from oracle.oracle import Q8_0, Q4_K, MXFP4
+
+pytestmark = pytest.mark.gpu
+T = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
+RMS_TOL = {"q8_0": 1e-4, "q4_k": 5e-3, "mxfp4": 5e-3}
+
+
+def check(name, y, ref):
+    e1, e2 = inputs.row_l2_err(y, ref), inputs.rms_err(y, ref)
+    assert e1 <= 1e-3, (name, e1)
+    assert e2 <= RMS_TOL[name], (name, e2)
+    return e1, e2
+
+
+def run_device(hip, t, wq, N, K, x):
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    qw = QuantizedWeight(torch.from_numpy(wq).cuda(), t, K, N)
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), qw)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("cfg,tname", [("CFG1", "ffn_up"), ("CFG2", "wq"), ("CFG2", "wk"), ("CFG2", "gate"),
+                                        ("CFG2", "down"), ("CFG4", "gate_up"), ("CFG4", "down")])
+def test_baseline_shapes(hip, oracle, cfg, tname):
+    fmt, N, K = getattr(inputs, cfg)[tname]
+    tag = f"{cfg.lower()}.{tname}"
+    wq = oracle.quantize(T[fmt], inputs.weights(tag, N * K))
+    x = inputs.activations(tag, 1, K)
+    ref = oracle.matmul_f64(T[fmt], wq, N, K, x)
+    y = run_device(hip, T[fmt], wq, N, K, x)
+    e = check(fmt, y, ref)
+    print(tag, "row-L2 err %.2e rms err %.2e" % e)
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+@pytest.mark.parametrize("N,K", [(1, 256), (3, 512), (5, 768), (7, 1024), (130, 2560), (257, 4096), (1001, 2816)])
+def test_ragged_shapes(hip, oracle, name, N, K):
+    if name == "q4_k" and K % 256:
+        pytest.skip("K must be a multiple of 256 for Q4_K")
+    rng = np.random.default_rng(N * 7919 + K)
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    check(name, run_device(hip, T[name], wq, N, K, x), oracle.matmul_f64(T[name], wq, N, K, x))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+def test_activation_ranges_and_linearity(hip, oracle, name):
+    rng = np.random.default_rng(31)
+    N, K = 300, 2048
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    base = run_device(hip, T[name], wq, N, K, x)
+    for s in (1e-20, 1e-6, 3e4, 1e12):       # outside fp16 range both ways: handled by the power-of-two pre-scale
+        xs = (x * np.float32(s)).astype(np.float32)
+        y = run_device(hip, T[name], wq, N, K, xs)
+        check(name, y, oracle.matmul_f64(T[name], wq, N, K, xs))
+    two = run_device(hip, T[name], wq, N, K, (2 * x).astype(np.float32))
+    assert np.array_equal(two, 2 * base)      # scaling by a power of two is exact
+    zero = run_device(hip, T[name], wq, N, K, np.zeros((1, K), np.float32))
+    assert np.all(zero == 0)
+    # sparse activations with one large outlier
+    xo = np.zeros((1, K), np.float32)
+    xo[0, 17], xo[0, K - 1] = 1000.0, -0.001
+    check(name, run_device(hip, T[name], wq, N, K, xo), oracle.matmul_f64(T[name], wq, N, K, xo))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "mxfp4"])
+def test_unaligned_sub_weight_views(hip, oracle, name):
+    """Expert-style views: a weight that starts at an arbitrary block offset inside a bigger
+    allocation (17-byte and 34-byte blocks land on every byte / 2-byte alignment)."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(33)
+    N, K = 64, 1120                              # 35 blocks per row: odd row stride
+    rows_before = (1, 2, 3)
+    total = max(rows_before) + N
+    wq = oracle.quantize(T[name], (rng.standard_normal(total * K) * 0.02).astype(np.float32))
+    dev = torch.from_numpy(wq).cuda()
+    rs = oracle.row_size(T[name], K)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    for rb in rows_before:
+        view = dev[rb * rs: (rb + N) * rs]
+        y = hip.LinearForward(xd, QuantizedWeight(view, T[name], K, N))
+        torch.cuda.synchronize()
+        ref = oracle.matmul_f64(T[name], wq[rb * rs:(rb + N) * rs], N, K, x)
+        check(name, y.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+def test_host_entry_points(hip, oracle, name):
+    """Drop-in path: host pointers, strided activation view, preload key, batch form."""
+    rng = np.random.default_rng(35)
+    N, K, M = 96, 1024, 3
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    big = rng.standard_normal((M, K + 40)).astype(np.float32)
+    x = big[:, 8:8 + K]                               # row stride K+40, stride1 == 1
+    ref = oracle.matmul_f64(T[name], wq, N, K, np.ascontiguousarray(x))
+    out = np.full((M, N + 5), np.nan, dtype=np.float32)
+    res = out[:, :N]                                  # strided result view
+    hip.AddmmQuant(res, x, wq.ctypes.data, T[name], K, N, wq.size)
+    check(name, res, ref)
+    assert np.all(np.isnan(out[:, N:]))               # nothing outside the view was written
+    # column-strided activations are packed by the shim
+    xt = np.asfortranarray(np.ascontiguousarray(x))
+    res2 = np.empty((M, N), dtype=np.float32)
+    hip.AddmmQuant(res2, xt, wq.ctypes.data, T[name], K, N, wq.size)
+    assert np.array_equal(res2, res)
+    # preload under an opaque key, then drop the host bytes
+    key = 0x7000_0000_1234
+    scratch = wq.copy()
+    hip.PreloadQuantizedWeight(key, scratch.ctypes.data, T[name], K, N, scratch.size)
+    scratch[:] = 0
+    res3 = np.empty((M, N), dtype=np.float32)
+    hip.AddmmQuant(res3, np.ascontiguousarray(x), key, T[name], K, N, wq.size)
+    assert np.array_equal(res3, res)
+    hip.InvalidateHostBuffer(key)
+    # batch form == per-row single calls on sub-weights
+    rs = oracle.row_size(T[name], K)
+    n_sub = N // 3
+    offs = [0, n_sub * rs, 2 * n_sub * rs]
+    resb = np.empty((M, n_sub), dtype=np.float32)
+    hip.AddmmQuantBatch(resb, np.ascontiguousarray(x), wq.ctypes.data, T[name], K, wq.size, offs, [n_sub] * 3)
+    for b in range(3):
+        assert np.array_equal(resb[b], res[b, b * n_sub:(b + 1) * n_sub])
+    hip.ClearHostBufferCache()
+
+
+def test_error_paths(hip, oracle):
+    """The failures the bridge reports (ggml_ops_matmul.cpp:303-329) come back as 0 + message."""
+    from tensorsharp_amd import hip_native as N
+    rng = np.random.default_rng(37)
+    Nn, K = 8, 256
+    wq = oracle.quantize(Q4_K, (rng.standard_normal(Nn * K) * 0.02).astype(np.float32))
+    x = np.zeros((2, K), np.float32)
+    y = np.zeros((2, Nn), np.float32)
+
+    def call(result, m1, w, t, ne0, ne1, rb):
+        with pytest.raises(RuntimeError) as ei:
+            hip.AddmmQuant(result, m1, w, t, ne0, ne1, rb)
+        return str(ei.value)
+
+    assert "Invalid quantized weight descriptor" in call(y, x, 0, Q4_K, K, Nn, wq.size)
+    assert "m1.dim0 != result.dim0" in call(y[:1], x, wq.ctypes.data, Q4_K, K, Nn, wq.size)
+    assert "quantized weight dims don't match" in call(y, x, wq.ctypes.data, Q4_K, K, Nn + 1, wq.size)
+    assert "quantized weight dims don't match" in call(y, x[:, :128], wq.ctypes.data, Q4_K, K, Nn, wq.size)
+    assert "Unsupported quantized weight type" in call(y, x, wq.ctypes.data, 14, K, Nn, wq.size)
+    assert "too small" in call(y, x, wq.ctypes.data, Q4_K, K, Nn, wq.size - 144)
+    x32 = np.zeros((2, 32), np.float32)
+    assert "multiple of the block size" in call(y, x32, wq.ctypes.data, Q4_K, 32, Nn, wq.size)
+    # a failed call leaves the message readable until the next call on this thread, success clears it
+    hip.AddmmQuant(y, x, wq.ctypes.data, Q4_K, K, Nn, wq.size)
+    assert N.get_last_error() == ""
+    hip.ClearHostBufferCache()

@@ -1,0 +1,118 @@
+"""Dequantizers of the oracle (restating ManagedQuantizedOps.cs:411-427, :447-479, :579-598)."""
+import numpy as np
+
+from oracle.oracle import Q8_0, Q4_K, MXFP4
+
+T = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
+MXFP4_TABLE = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], dtype=np.float32)
+
+
+def test_reference_unit_test_vectors(oracle, golden):
+    # InferenceWeb.Tests/ManagedQuantizedOpsTests.cs:29-45 and :47-68
+    for name in ("q8_0", "q4_k"):
+        y = oracle.dequantize(T[name], golden[f"ref_tests_{name}_raw"])
+        idx = golden[f"ref_tests_{name}_expect_idx"]
+        np.testing.assert_array_equal(y[idx], golden[f"ref_tests_{name}_expect_val"])
+        rest = np.ones(y.size, bool)
+        rest[idx] = False
+        if name == "q8_0":
+            assert np.all(y[rest] == 0)
+
+
+def test_golden_blocks_bit_exact(oracle, golden):
+    for name, t in T.items():
+        y = oracle.dequantize(t, golden[f"blocks_{name}_q"])
+        want = golden[f"blocks_{name}_deq"]
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), name
+
+
+def test_q8_0_closed_form_all_scales(oracle):
+    # every fp16 scale code x a sweep of int8 values: y = q * float(d), one exact fp32 product
+    codes = np.arange(65536, dtype=np.uint16)
+    raw = np.zeros((65536, 34), dtype=np.uint8)
+    raw[:, 0] = codes & 0xFF
+    raw[:, 1] = codes >> 8
+    q = ((np.arange(32)[None, :] * 37 + codes[:, None] * 11) % 256).astype(np.uint8)
+    raw[:, 2:] = q
+    y = oracle.dequantize(Q8_0, raw.reshape(-1)).reshape(65536, 32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = q.view(np.int8).astype(np.float32) * codes.view(np.float16).astype(np.float32)[:, None]
+    ok = ~np.isnan(want)
+    assert np.array_equal(y.view(np.uint32)[ok], want.view(np.uint32)[ok])
+
+
+def _scale_min(j, p):
+    if j < 4:
+        return p[:, j] & 63, p[:, j + 4] & 63
+    return (p[:, j + 4] & 0x0F) | ((p[:, j - 4] >> 6) << 4), (p[:, j + 4] >> 4) | ((p[:, j] >> 6) << 4)
+
+
+def test_q4_k_closed_form_random_bytes(oracle):
+    # independent numpy restatement: y = (d*sc)*q - (dmin*m), separately rounded fp32 ops
+    rng = np.random.default_rng(3)
+    nb = 4096
+    raw = rng.integers(0, 256, size=(nb, 144), dtype=np.uint8)
+    # keep d/dmin finite
+    raw[:, 1] &= 0x7B
+    raw[:, 3] &= 0x7B
+    y = oracle.dequantize(Q4_K, raw.reshape(-1)).reshape(nb, 256)
+    d = raw[:, 0:2].copy().view(np.float16).astype(np.float32)[:, 0]
+    dmin = raw[:, 2:4].copy().view(np.float16).astype(np.float32)[:, 0]
+    p = raw[:, 4:16].astype(np.uint32)
+    qs = raw[:, 16:]
+    want = np.empty((nb, 256), dtype=np.float32)
+    for g in range(4):
+        sc1, m1 = _scale_min(2 * g, p)
+        sc2, m2 = _scale_min(2 * g + 1, p)
+        d1 = (d * sc1.astype(np.float32)).astype(np.float32)[:, None]
+        d2 = (d * sc2.astype(np.float32)).astype(np.float32)[:, None]
+        o1 = (dmin * m1.astype(np.float32)).astype(np.float32)[:, None]
+        o2 = (dmin * m2.astype(np.float32)).astype(np.float32)[:, None]
+        lo = (qs[:, 32 * g:32 * g + 32] & 0x0F).astype(np.float32)
+        hi = (qs[:, 32 * g:32 * g + 32] >> 4).astype(np.float32)
+        want[:, 64 * g:64 * g + 32] = (d1 * lo).astype(np.float32) - o1
+        want[:, 64 * g + 32:64 * g + 64] = (d2 * hi).astype(np.float32) - o2
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+
+
+def test_mxfp4_closed_form_all_codes(oracle):
+    # all 256 exponent codes x all 256 quant bytes: value = table[nibble] * 2^(e-128)
+    raw = np.zeros((256, 16, 17), dtype=np.uint8)
+    raw[:, :, 0] = np.arange(256, dtype=np.uint8)[:, None]
+    raw[:, :, 1:] = np.arange(256, dtype=np.uint8).reshape(16, 16)[None]
+    y = oracle.dequantize(MXFP4, raw.reshape(-1)).reshape(256, 16, 32)
+    e = np.arange(256)
+    bits = np.where(e < 2, 0x00200000 << np.minimum(e, 1), (np.maximum(e, 1) - 1) << 23).astype(np.uint32)
+    d = bits.view(np.float32)[:, None, None]
+    q = raw[:, :, 1:]
+    want = np.concatenate([d * MXFP4_TABLE[q & 0x0F], d * MXFP4_TABLE[q >> 4]], axis=2).astype(np.float32)
+    ok = ~np.isnan(want)
+    assert np.array_equal(y.view(np.uint32)[ok], want.view(np.uint32)[ok])
+    # spot value: e=127 -> d=0.5, nibble 7 -> 12*0.5
+    blk = np.zeros(17, dtype=np.uint8)
+    blk[0] = 127
+    blk[1] = 0x97   # low nibble 7 -> +12, high nibble 9 -> -1
+    v = oracle.dequantize(MXFP4, blk)
+    assert v[0] == 6.0 and v[16] == -0.5
+
+
+def test_matches_reference_build_on_random_bytes(oracle, reference):
+    rng = np.random.default_rng(4)
+    for name, t in T.items():
+        bb = {"q8_0": 34, "q4_k": 144, "mxfp4": 17}[name]
+        raw = rng.integers(0, 256, size=bb * 3000, dtype=np.uint8)
+        a = oracle.dequantize(t, raw)
+        b = reference.dequantize(t, raw)
+        ok = ~np.isnan(b)
+        assert np.array_equal(a.view(np.uint32)[ok], b.view(np.uint32)[ok]), name
+
+
+def test_error_codes(oracle):
+    import ctypes as C
+    buf = np.zeros(64, dtype=np.uint8)
+    out = np.zeros(64, dtype=np.float32)
+    f32p = C.POINTER(C.c_float)
+    assert oracle.lib.tso_dequantize(8, None, 32, out.ctypes.data_as(f32p)) == -1
+    assert oracle.lib.tso_dequantize(77, C.c_void_p(buf.ctypes.data), 32, out.ctypes.data_as(f32p)) == -2
+    assert oracle.lib.tso_dequantize(8, C.c_void_p(buf.ctypes.data), 33, out.ctypes.data_as(f32p)) == -1
+    assert oracle.lib.tso_dequantize(8, C.c_void_p(buf.ctypes.data), 0, out.ctypes.data_as(f32p)) == 0
