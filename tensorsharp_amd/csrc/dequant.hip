@@ -40,10 +40,12 @@ __device__ __forceinline__ float e8m0_half_scale(uint32_t e)
 
 __device__ __forceinline__ float mxfp4_value(uint32_t nib)
 {
-    // doubled E2M1 magnitudes 0,1,2,3,4,6,8,12 packed one per nibble-indexed byte
-    const uint64_t mags = 0x0c08060403020100ull;
-    const float m = (float)(uint32_t)((mags >> ((nib & 7u) * 8)) & 0xffu);
-    return (nib & 8u) ? -m : m;
+    // doubled E2M1 table {0,1,2,3,4,6,8,12, 0,-1,-2,-3,-4,-6,-8,-12} as signed bytes
+    // (ggml-common.h:1094-1096); the integer route keeps code 8 at +0 like the reference.
+    const uint64_t pos = 0x0c08060403020100ull;
+    const uint64_t neg = 0xf4f8fafcfdfeff00ull;
+    const uint64_t tab = (nib & 8u) ? neg : pos;
+    return (float)(int)(int8_t)((tab >> ((nib & 7u) * 8)) & 0xffu);
 }
 
 // one thread -> 4 consecutive outputs

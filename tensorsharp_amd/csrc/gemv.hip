@@ -11,7 +11,7 @@
 //     128-bit loads.  Unaligned units (34 B / 17 B) are fetched as aligned dwords and
 //     re-aligned in registers with v_alignbyte;
 //   * dequantization happens in registers: Q8_0 int8 -> fp32 (sign-extending byte select),
-//     Q4_K nibbles -> fp16 via the 0x6400 exponent trick feeding v_dot2_f32_f16,
+//     Q4_K nibbles masked in place are fp16 subnormals (q * 2^-24) feeding v_dot2_f32_f16,
 //     MXFP4 E2M1 pairs -> fp16 with v_cvt_scalef32_pk_f16_fp4 feeding v_dot2_f32_f16;
 //     block scales (fp16 d, 6-bit K-quant scales/mins, E8M0) are applied once per unit in fp32;
 //   * R row sums per lane are reduced with DPP inside each row of 16 lanes and four
@@ -197,16 +197,17 @@ __global__ void __launch_bounds__(kThreads) gemv_q4k_kernel(const uint8_t* __res
                 const uint4 xv = xu[j];
                 const uint32_t w = qw[j];
                 const uint32_t w8 = w >> 8;
-                lo = dot2((w & 0x000f000fu) | 0x64006400u, xv.x, lo);
-                lo = dot2((w8 & 0x000f000fu) | 0x64006400u, xv.y, lo);
-                hi = dot2((w & 0x00f000f0u) | 0x64006400u, xv.z, hi);
-                hi = dot2((w8 & 0x00f000f0u) | 0x64006400u, xv.w, hi);
+                // a nibble left in place is an fp16 subnormal: q * 2^-24 (low) or 16q * 2^-24 (high);
+                // v_dot2_f32_f16 honours fp16 denormals, so the integer values enter the dot exactly
+                lo = dot2(w & 0x000f000fu, xv.x, lo);
+                lo = dot2(w8 & 0x000f000fu, xv.y, lo);
+                hi = dot2(w & 0x00f000f0u, xv.z, hi);
+                hi = dot2(w8 & 0x00f000f0u, xv.w, hi);
             }
             const uint4 tail = xu[8];
             const float s1 = __uint_as_float(tail.x), s2 = __uint_as_float(tail.y);
-            // the fp16 operands were 1024+q (low) and 1024+16q (high): remove the offsets
-            const float dl = lo - 1024.f * s1;
-            const float dh = (hi - 1024.f * s2) * 0.0625f;
+            const float dl = lo * 16777216.f;   // 2^24
+            const float dh = hi * 1048576.f;    // 2^24 / 16
 
             // 6-bit scales / mins of sub-blocks 2*g4 and 2*g4+1 (ggml-quants.c:703-710)
             const int sh = (g4 & 1) * 16;
