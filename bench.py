@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized-matmul hot path on one MI355X.
+
+Headline (BASELINE.json configs[1]): Q4_K decode GEMV, batch 1, over the seven projections of
+one transformer layer (hidden 4096 / FFN 14336 / 32 q-heads / 8 kv-heads).  One step = one
+layer = seven GEMVs, issued through the C ABI as one grouped launch
+(TSHip_AddmmQuantGroupF32Device).  Several distinct layer copies are cycled so that the
+256 MB Infinity Cache cannot serve the weights.  `value` is algorithmic GB/s
+(weights + activations + outputs) over the timed region, inputs resident in HBM.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+Q8_0, Q4_K, MXFP4 = 8, 12, 39
+HBM_PEAK_GBS = 8000.0
+
+LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
+    ("wq", 4096, 4096), ("wk", 1024, 4096), ("wv", 1024, 4096), ("wo", 4096, 4096),
+    ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336),
+]
+
+
+def row_bytes(t, k):
+    return {Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), MXFP4: 17 * (k // 32)}[t]
+
+
+def algorithmic_bytes(t, n, k, m=1):
+    return n * row_bytes(t, k) + m * k * 4 + m * n * 4
+
+
+def cpu_baseline(layer_host, xs_host, n_threads):
+    """Oracle port of the reference's managed loop nest (ModelBase.cs:924-991), all host threads,
+    on the same seven matrices; best of 3 passes over one layer."""
+    from oracle.oracle import Oracle
+    try:
+        orc = Oracle(fast=True)
+        orc.lib.tso_max_threads()
+    except OSError:
+        orc = Oracle(fast=False)
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for (name, n, k), w, x in zip(LAYER, layer_host, xs_host):
+            orc.matmul_managed(Q4_K, w, n, k, x, vec_width=8, threads=n_threads)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    total = sum(algorithmic_bytes(Q4_K, n, k) for _, n, k in LAYER)
+    return {"value": round(total / best / 1e9, 3), "unit": "GB/s", "cores": n_threads, "kind": "port",
+            "sample": "one full layer (7 Q4_K GEMVs, 123.0 MB), best of 3 passes, OpenMP over output rows",
+            "seconds_per_layer": round(best, 4)}
+
+
+def time_region(fn, steps, torch):
+    """fn(i) launches step i on the current stream. Returns (event_ms, wall_ms)."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1), wall
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--copies", type=int, default=6, help="distinct layer copies cycled (6 x 123 MB > Infinity Cache)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU kernel path only: this build has no multi-GPU code; run with --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from tensorsharp_amd import HipBasicOps, QuantizedWeight, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback exists for the HIP path).", file=sys.stderr)
+        sys.exit(3)
+    if not HipBasicOps.IsAvailable():
+        from tensorsharp_amd import hip_native
+        print("HIP backend unavailable: " + hip_native.get_last_error(), file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    HipBasicOps.UseCurrentStream()
+
+    # ---- workload: `copies` layers of seven Q4_K matrices, device resident -------------------
+    layers = []
+    for c in range(args.copies):
+        ws = [QuantizedWeight(synth.random_weight(Q4_K, n, k, dev, seed=1000 * c + i), Q4_K, k, n)
+              for i, (_, n, k) in enumerate(LAYER)]
+        layers.append(ws)
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    xs = [torch.randn((1, k), generator=g, device=dev, dtype=torch.float32) for _, _, k in LAYER]
+    ys = [torch.empty((1, n), device=dev, dtype=torch.float32) for _, n, _ in LAYER]
+    packs = [HipBasicOps.PrepareGroup(ys, xs, ws) for ws in layers]
+    step_bytes = sum(algorithmic_bytes(Q4_K, n, k) for _, n, k in LAYER)
+
+    def step(i):
+        HipBasicOps.AddmmQuantGroupDevice(packs[i % len(packs)])
+
+    for i in range(args.warmup):
+        step(i)
+    ev_ms, wall_ms = time_region(step, args.steps, torch)
+    assert all(bool(torch.isfinite(y).all()) for y in ys)
+    ms_per_step = wall_ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    kern_us = ev_ms * 1e3 / args.steps          # one launch per step: HIP-event time per launch
+    achieved = step_bytes / (kern_us * 1e-6) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("q4k_layer_group_gemv")
+        except (OSError, ValueError):
+            traffic = None
+
+    out = {
+        "metric": "Q4_K/Q8_0/MXFP4 matmul: decode GB/s (% HBM peak), prefill TFLOP/s (% MFMA)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "q4_k weights x f32 activations (fp16 operands, f32 accumulate)",
+        "data": "synthetic: W ~ N(0,0.02) in Q4_K blocks (min/max-fit quantizer), x ~ N(0,1) f32, "
+                f"{args.copies} distinct layer copies cycled",
+        "config": {"workload": "configs[1]: Q4_K decode GEMV batch 1, one layer's 7 projections "
+                               "(4096/14336/32q/8kv), one grouped launch per layer",
+                   "bytes_per_step": step_bytes, "launches_per_step": 1, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": "tship::gemv_kernel<12, R> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
+                     "bytes_per_launch": step_bytes},
+    }
+
+    # ---- secondary workloads (reported, not the headline) ---------------------------------------
+    if not args.no_extra:
+        extra = {}
+        n_it = max(200, args.steps // 4)
+
+        def one_matrix(t, n, k, copies):
+            ws = [QuantizedWeight(synth.random_weight(t, n, k, dev, seed=77 + c), t, k, n) for c in range(copies)]
+            x = torch.randn((1, k), device=dev, dtype=torch.float32)
+            y = torch.empty((1, n), device=dev, dtype=torch.float32)
+
+            def f(i):
+                w = ws[i % copies]
+                HipBasicOps.AddmmQuantDevice(y, x, w.ptr, t, k, n, w.raw_bytes)
+            for i in range(50):
+                f(i)
+            ev, wall = time_region(f, n_it, torch)
+            b = algorithmic_bytes(t, n, k)
+            return {"us_per_launch_events": round(ev * 1e3 / n_it, 3), "GBps": round(b / (ev * 1e-3 / n_it) / 1e9, 1),
+                    "pct_hbm_peak": round(100 * b / (ev * 1e-3 / n_it) / 1e9 / HBM_PEAK_GBS, 1), "bytes": b}
+
+        extra["cfg1_q8_0_gemv_9728x2560"] = one_matrix(Q8_0, 9728, 2560, 12)
+        for name, n, k in (("gate", 14336, 4096), ("down", 4096, 14336), ("wq", 4096, 4096), ("wk", 1024, 4096)):
+            extra[f"cfg2_q4_k_gemv_{name}_{n}x{k}"] = one_matrix(Q4_K, n, k, max(2, int(300e6 // (n * row_bytes(Q4_K, k))) + 1))
+        extra["cfg4_mxfp4_gemv_gate_up_5760x2880"] = one_matrix(MXFP4, 5760, 2880, 32)
+        extra["cfg4_mxfp4_gemv_down_2880x2880"] = one_matrix(MXFP4, 2880, 2880, 64)
+        out["extra"] = extra
+
+    if not args.no_cpu:
+        n_threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1)
+        n_threads = min(n_threads, os.cpu_count() or 1)
+        layer_host = [w.data.cpu().numpy() for w in layers[0]]
+        xs_host = [x.cpu().numpy() for x in xs]
+        out["cpu_baseline"] = cpu_baseline(layer_host, xs_host, n_threads)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -115,6 +115,16 @@ TSHIP_EXPORT int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensor
                                            int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1,
                                            int64_t m2_raw_bytes);
 
+/* No counterpart in the bridge: the reference issues one AddmmQuant per projection from C#
+ * (ModelBase.LinearForward, TensorSharp.Models/ModelBase.cs:875-905).  `count` independent
+ * AddmmQuantF32Device problems of one block type; when every problem is a decode GEMV (M == 1) and
+ * count <= 8 they are served by ONE kernel launch, otherwise they run back to back.  Results equal those of
+ * one TSHip_AddmmQuantF32Device call per problem up to fp32 summation order. */
+TSHIP_EXPORT int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView2D* results,
+                                                const TSHipTensorView2D* m1s, const void* const* m2_datas,
+                                                int m2_ggml_type, const int64_t* m2_ne0s, const int64_t* m2_ne1s,
+                                                const int64_t* m2_raw_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -198,11 +198,9 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
     return true;
 }
 
-// result/m1/w are device pointers here.
-bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
-                       int64_t N, hipStream_t stream)
+// alignment the kernels assume for device operands
+bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
 {
-    const size_t w_bytes = row_size(type, K) * (size_t)N;
     const uintptr_t wa = reinterpret_cast<uintptr_t>(w);
     const uintptr_t need_align = type == kTypeQ4_K ? 16 : type == kTypeQ8_0 ? 2 : 1;
     if (wa % need_align != 0) {
@@ -213,6 +211,15 @@ bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D&
         set_last_error("Activation rows must be 16-byte aligned on the device.");
         return false;
     }
+    return true;
+}
+
+// result/m1/w are device pointers here.
+bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
+                       int64_t N, hipStream_t stream)
+{
+    const size_t w_bytes = row_size(type, K) * (size_t)N;
+    if (!check_device_operands(m1, w, type)) return false;
     const int M = m1.dim0;
     if (K <= gemv_max_k(type)) {
         // decode / small batch: one GEMV per activation row
@@ -422,6 +429,50 @@ int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D m1, co
             return 0;
         }
         if (!run_matmul_device(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load())) return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView2D* results, const TSHipTensorView2D* m1s,
+                                   const void* const* m2_datas, int m2_ggml_type, const int64_t* m2_ne0s,
+                                   const int64_t* m2_ne1s, const int64_t* m2_raw_bytes)
+{
+    return guarded(0, "addmm_quant_group", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (count <= 0 || !results || !m1s || !m2_datas || !m2_ne0s || !m2_ne1s || !m2_raw_bytes) {
+            set_last_error("Invalid arguments for addmm_quant_group.");
+            return 0;
+        }
+        bool decode = count <= gemv_max_group();
+        for (int i = 0; i < count; ++i) {
+            if (!validate_addmm_quant(results[i], m1s[i], m2_datas[i], m2_ggml_type, m2_ne0s[i], m2_ne1s[i],
+                                      m2_raw_bytes[i]))
+                return 0;
+            if (!is_standard_view(results[i]) || m1s[i].stride1 != 1) {
+                set_last_error("Device addmm_quant needs stride1 == 1 views.");
+                return 0;
+            }
+            if (!check_device_operands(m1s[i], m2_datas[i], m2_ggml_type)) return 0;
+            decode = decode && m1s[i].dim0 == 1 && m2_ne0s[i] <= gemv_max_k(m2_ggml_type);
+        }
+        hipStream_t stream = g_stream.load();
+        if (decode) {
+            GemvArgs args[16];
+            for (int i = 0; i < count; ++i) {
+                args[i].w = m2_datas[i];
+                args[i].w_bytes = (int64_t)(row_size(m2_ggml_type, m2_ne0s[i]) * (size_t)m2_ne1s[i]);
+                args[i].x = static_cast<const float*>(m1s[i].data);
+                args[i].y = static_cast<float*>(results[i].data);
+                args[i].N = (int)m2_ne1s[i];
+                args[i].K = (int)m2_ne0s[i];
+            }
+            if (!launch_gemv_group(m2_ggml_type, count, args, stream)) return 0;
+        } else {
+            for (int i = 0; i < count; ++i)
+                if (!run_matmul_device(results[i], m1s[i], m2_datas[i], m2_ggml_type, m2_ne0s[i], m2_ne1s[i], stream))
+                    return 0;
+        }
         clear_last_error();
         return 1;
     });

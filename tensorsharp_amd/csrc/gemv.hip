@@ -22,6 +22,9 @@
 // 4-bit formats (power-of-two pre-scaled so that no value overflows or underflows).
 #include "tship_internal.h"
 
+#include <algorithm>
+#include <cstring>
+
 namespace tship {
 namespace {
 
@@ -29,6 +32,25 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
+constexpr int kMaxGroup = 8;
+
+// one GEMV
+struct GemvProblem {
+    const uint8_t* w;
+    int64_t w_bytes;
+    const float* x;
+    float* y;
+    int N;
+    int K;
+};
+
+// up to kMaxGroup independent GEMVs served by one launch; workgroups [wg_begin[i], wg_begin[i+1])
+// work on problem i.  Passed by value as the kernel argument (no device-side descriptor memory).
+struct GemvGroup {
+    GemvProblem p[kMaxGroup];
+    int wg_begin[kMaxGroup + 1];
+    int count;
+};
 
 union H2U {
     uint32_t u;
@@ -154,11 +176,12 @@ __device__ void stage_x_q4k(const float* __restrict__ x, int K, uint32_t* lds, f
 }
 
 template <int R>
-__global__ void __launch_bounds__(kThreads) gemv_q4k_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x,
-                                                            float* __restrict__ y, int N, int K)
+__device__ __forceinline__ void gemv_q4k_body(const GemvProblem& P, int wg, int nwg, uint32_t* lds, float* red)
 {
-    extern __shared__ uint32_t lds[];
-    __shared__ float red[kWaves];
+    const uint8_t* __restrict__ W = P.w;
+    const float* __restrict__ x = P.x;
+    float* __restrict__ y = P.y;
+    const int N = P.N, K = P.K;
     float xscale;
     const float inv = block_prescale(x, K, red, &xscale);
     stage_x_q4k(x, K, lds, inv);
@@ -168,8 +191,8 @@ __global__ void __launch_bounds__(kThreads) gemv_q4k_kernel(const uint8_t* __res
     const int upr = K >> 6;  // units per row
     const int64_t row_bytes = (int64_t)(K >> 8) * 144;
     const int nrb = (N + R - 1) / R;
-    const int wave_stride = gridDim.x * kWaves;
-    for (int rb = blockIdx.x * kWaves + (threadIdx.x >> 6); rb < nrb; rb += wave_stride) {
+    const int wave_stride = nwg * kWaves;
+    for (int rb = wg * kWaves + (threadIdx.x >> 6); rb < nrb; rb += wave_stride) {
         const int row0 = rb * R;
         const int rows = min(R, N - row0);
         const int total = rows * upr;
@@ -270,12 +293,13 @@ __device__ __forceinline__ uint32_t fp4_pair(uint32_t w)
 }
 
 template <int R>
-__global__ void __launch_bounds__(kThreads) gemv_mxfp4_kernel(const uint8_t* __restrict__ W, int64_t w_bytes,
-                                                              const float* __restrict__ x, float* __restrict__ y, int N,
-                                                              int K)
+__device__ __forceinline__ void gemv_mxfp4_body(const GemvProblem& P, int wg, int nwg, uint32_t* lds, float* red)
 {
-    extern __shared__ uint32_t lds[];
-    __shared__ float red[kWaves];
+    const uint8_t* __restrict__ W = P.w;
+    const int64_t w_bytes = P.w_bytes;
+    const float* __restrict__ x = P.x;
+    float* __restrict__ y = P.y;
+    const int N = P.N, K = P.K;
     float xscale;
     const float inv = block_prescale(x, K, red, &xscale);
     stage_x_mxfp4(x, K, lds, inv);
@@ -285,9 +309,9 @@ __global__ void __launch_bounds__(kThreads) gemv_mxfp4_kernel(const uint8_t* __r
     const int upr = K >> 5;
     const int64_t row_bytes = (int64_t)upr * 17;
     const int nrb = (N + R - 1) / R;
-    const int wave_stride = gridDim.x * kWaves;
+    const int wave_stride = nwg * kWaves;
     const uintptr_t w_end = reinterpret_cast<uintptr_t>(W) + (uintptr_t)w_bytes;
-    for (int rb = blockIdx.x * kWaves + (threadIdx.x >> 6); rb < nrb; rb += wave_stride) {
+    for (int rb = wg * kWaves + (threadIdx.x >> 6); rb < nrb; rb += wave_stride) {
         const int row0 = rb * R;
         const int rows = min(R, N - row0);
         const int total = rows * upr;
@@ -374,11 +398,13 @@ __device__ __forceinline__ float dot4_i8(uint32_t q, float4 xv, float acc)
 }
 
 template <int R>
-__global__ void __launch_bounds__(kThreads) gemv_q80_kernel(const uint8_t* __restrict__ W, int64_t w_bytes,
-                                                            const float* __restrict__ x, float* __restrict__ y, int N,
-                                                            int K)
+__device__ __forceinline__ void gemv_q80_body(const GemvProblem& P, int wg, int nwg, uint32_t* lds, float* /*red*/)
 {
-    extern __shared__ uint32_t lds[];
+    const uint8_t* __restrict__ W = P.w;
+    const int64_t w_bytes = P.w_bytes;
+    const float* __restrict__ x = P.x;
+    float* __restrict__ y = P.y;
+    const int N = P.N, K = P.K;
     float* xl = reinterpret_cast<float*>(lds);
     stage_x_q80(x, K, xl);
     __syncthreads();
@@ -387,9 +413,9 @@ __global__ void __launch_bounds__(kThreads) gemv_q80_kernel(const uint8_t* __res
     const int upr = K >> 5;
     const int64_t row_bytes = (int64_t)upr * 34;
     const int nrb = (N + R - 1) / R;
-    const int wave_stride = gridDim.x * kWaves;
+    const int wave_stride = nwg * kWaves;
     const uintptr_t w_end = reinterpret_cast<uintptr_t>(W) + (uintptr_t)w_bytes;
-    for (int rb = blockIdx.x * kWaves + (threadIdx.x >> 6); rb < nrb; rb += wave_stride) {
+    for (int rb = wg * kWaves + (threadIdx.x >> 6); rb < nrb; rb += wave_stride) {
         const int row0 = rb * R;
         const int rows = min(R, N - row0);
         const int total = rows * upr;
@@ -441,6 +467,22 @@ __global__ void __launch_bounds__(kThreads) gemv_q80_kernel(const uint8_t* __res
     }
 }
 
+template <int TYPE, int R>
+__global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
+{
+    extern __shared__ uint32_t lds[];
+    __shared__ float red[kWaves];
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxGroup; ++j)
+        if (j < G.count && (int)blockIdx.x >= G.wg_begin[j]) i = j;
+    const int wg = (int)blockIdx.x - G.wg_begin[i];
+    const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
+    if (TYPE == kTypeQ4_K) gemv_q4k_body<R>(G.p[i], wg, nwg, lds, red);
+    else if (TYPE == kTypeMXFP4) gemv_mxfp4_body<R>(G.p[i], wg, nwg, lds, red);
+    else gemv_q80_body<R>(G.p[i], wg, nwg, lds, red);
+}
+
 size_t lds_bytes_for(int type, int K)
 {
     switch (type) {
@@ -453,14 +495,25 @@ size_t lds_bytes_for(int type, int K)
 
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 
-template <typename Kern>
-bool prepare(Kern kern, size_t lds)
+template <int TYPE, int R>
+bool launch_instance(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    if (lds > 64 * 1024)
-        return hip_ok(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                      "gemv: raising the dynamic LDS limit");
-    return true;
+    auto kern = gemv_kernel<TYPE, R>;
+    if (lds > 64 * 1024 &&
+        !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds),
+                "gemv: raising the dynamic LDS limit"))
+        return false;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g);
+    return hip_ok(hipGetLastError(), "gemv launch");
+}
+
+template <int TYPE>
+bool launch_type(const GemvGroup& g, int R, int grid, size_t lds, hipStream_t stream)
+{
+    if (R == 4) return launch_instance<TYPE, 4>(g, grid, lds, stream);
+    if (R == 2) return launch_instance<TYPE, 2>(g, grid, lds, stream);
+    return launch_instance<TYPE, 1>(g, grid, lds, stream);
 }
 
 }  // namespace
@@ -475,52 +528,70 @@ int gemv_max_k(int type)
     }
 }
 
-bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream)
+int gemv_max_group() { return kMaxGroup; }
+
+bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream)
 {
-    if (K > gemv_max_k(type)) {
-        set_last_error("gemv: K exceeds what one workgroup can stage in LDS.");
+    if (count < 1 || count > kMaxGroup) {
+        set_last_error("gemv: group size out of range.");
         return false;
     }
-    const size_t lds = lds_bytes_for(type, K);
-    const DeviceInfo& di = device_info();
-    // rows per wavefront step: keep at least ~8 waves per CU worth of row blocks
-    int R = 4;
-    while (R > 1 && (int64_t)N / R < (int64_t)di.num_cus * 16) R >>= 1;
-    const int nrb = (N + R - 1) / R;
-    const int wg_needed = (nrb + kWaves - 1) / kWaves;
-    int per_cu = (int)std::min<size_t>(8, (160 * 1024) / (lds + 256));
-    if (per_cu < 1) per_cu = 1;
-    const int grid = std::max(1, std::min(wg_needed, di.num_cus * per_cu));
-    const uint8_t* W = static_cast<const uint8_t*>(w);
-
-#define TSHIP_GEMV_LAUNCH(KERN, ...)                                                        \
-    do {                                                                                    \
-        if (!prepare(KERN, lds)) return false;                                              \
-        hipLaunchKernelGGL(KERN, dim3(grid), dim3(kThreads), lds, stream, __VA_ARGS__);      \
-    } while (0)
-
-    switch (type) {
-    case kTypeQ4_K:
-        if (R == 4) TSHIP_GEMV_LAUNCH(gemv_q4k_kernel<4>, W, x, y, N, K);
-        else if (R == 2) TSHIP_GEMV_LAUNCH(gemv_q4k_kernel<2>, W, x, y, N, K);
-        else TSHIP_GEMV_LAUNCH(gemv_q4k_kernel<1>, W, x, y, N, K);
-        break;
-    case kTypeMXFP4:
-        if (R == 4) TSHIP_GEMV_LAUNCH(gemv_mxfp4_kernel<4>, W, w_bytes, x, y, N, K);
-        else if (R == 2) TSHIP_GEMV_LAUNCH(gemv_mxfp4_kernel<2>, W, w_bytes, x, y, N, K);
-        else TSHIP_GEMV_LAUNCH(gemv_mxfp4_kernel<1>, W, w_bytes, x, y, N, K);
-        break;
-    case kTypeQ8_0:
-        if (R == 4) TSHIP_GEMV_LAUNCH(gemv_q80_kernel<4>, W, w_bytes, x, y, N, K);
-        else if (R == 2) TSHIP_GEMV_LAUNCH(gemv_q80_kernel<2>, W, w_bytes, x, y, N, K);
-        else TSHIP_GEMV_LAUNCH(gemv_q80_kernel<1>, W, w_bytes, x, y, N, K);
-        break;
-    default:
+    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4) {
         set_last_error("gemv: unsupported type.");
         return false;
     }
-#undef TSHIP_GEMV_LAUNCH
-    return hip_ok(hipGetLastError(), "gemv launch");
+    const DeviceInfo& di = device_info();
+    size_t lds = 0;
+    int64_t total_rows = 0;
+    double total_bytes = 0;
+    for (int i = 0; i < count; ++i) {
+        if (args[i].K > gemv_max_k(type)) {
+            set_last_error("gemv: K exceeds what one workgroup can stage in LDS.");
+            return false;
+        }
+        lds = std::max(lds, lds_bytes_for(type, args[i].K));
+        total_rows += args[i].N;
+        total_bytes += (double)args[i].w_bytes;
+    }
+    // rows per wavefront step: keep at least ~16 waves per CU worth of row blocks
+    int R = 4;
+    while (R > 1 && total_rows / R < (int64_t)di.num_cus * 16) R >>= 1;
+    int per_cu = (int)std::min<size_t>(8, (160 * 1024) / (lds + 256));
+    if (per_cu < 1) per_cu = 1;
+    const int budget = di.num_cus * per_cu;
+
+    GemvGroup g;
+    std::memset(&g, 0, sizeof(g));
+    g.count = count;
+    int begin = 0;
+    for (int i = 0; i < count; ++i) {
+        g.p[i].w = static_cast<const uint8_t*>(args[i].w);
+        g.p[i].w_bytes = args[i].w_bytes;
+        g.p[i].x = args[i].x;
+        g.p[i].y = args[i].y;
+        g.p[i].N = args[i].N;
+        g.p[i].K = args[i].K;
+        const int nrb = (args[i].N + R - 1) / R;
+        const int wg_needed = (nrb + kWaves - 1) / kWaves;
+        // workgroups in proportion to the bytes each problem streams
+        int share = (int)((double)budget * (double)args[i].w_bytes / total_bytes + 0.5);
+        share = std::max(1, std::min(share, wg_needed));
+        g.wg_begin[i] = begin;
+        begin += share;
+    }
+    for (int i = count; i <= kMaxGroup; ++i) g.wg_begin[i] = begin;
+    const int grid = begin;
+    switch (type) {
+    case kTypeQ4_K: return launch_type<kTypeQ4_K>(g, R, grid, lds, stream);
+    case kTypeMXFP4: return launch_type<kTypeMXFP4>(g, R, grid, lds, stream);
+    default: return launch_type<kTypeQ8_0>(g, R, grid, lds, stream);
+    }
+}
+
+bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream)
+{
+    GemvArgs a{w, w_bytes, x, y, N, K};
+    return launch_gemv_group(type, 1, &a, stream);
 }
 
 }  // namespace tship

@@ -61,4 +61,16 @@ bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float
 // largest K the GEMV kernel stages in LDS for this type
 int gemv_max_k(int type);
 
+// `count` independent GEMVs of one block type in a single launch (count <= gemv_max_group()).
+struct GemvArgs {
+    const void* w;
+    int64_t w_bytes;
+    const float* x;
+    float* y;
+    int N;
+    int K;
+};
+int gemv_max_group();
+bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);
+
 }  // namespace tship

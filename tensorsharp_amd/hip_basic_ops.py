@@ -130,6 +130,30 @@ class HipBasicOps:
         N.check_result(ok, "addmm_quant")
 
     @staticmethod
+    def PrepareGroup(results, m1s, weights):
+        """Marshal a list of (result, m1, QuantizedWeight) problems once; returns the argument pack
+        that AddmmQuantGroupDevice launches (decode loops reuse the pack every token)."""
+        n = len(weights)
+        if not (n == len(results) == len(m1s)) or n == 0:
+            raise ValueError("results, m1s and weights must be equally long and non-empty.")
+        t = weights[0].ggml_type
+        if any(w.ggml_type != t for w in weights):
+            raise ValueError("all weights of a group must share one block type.")
+        rv = (N.TensorView2D * n)(*[_device_view(r) for r in results])
+        mv = (N.TensorView2D * n)(*[_device_view(m) for m in m1s])
+        wp = (C.c_void_p * n)(*[w.ptr for w in weights])
+        ne0 = (C.c_int64 * n)(*[w.ne0 for w in weights])
+        ne1 = (C.c_int64 * n)(*[w.ne1 for w in weights])
+        rb = (C.c_int64 * n)(*[w.raw_bytes for w in weights])
+        return (n, rv, mv, wp, t, ne0, ne1, rb)
+
+    @staticmethod
+    def AddmmQuantGroupDevice(pack):
+        """count independent AddmmQuantDevice problems; one launch when all are decode GEMVs."""
+        ok = N.lib().TSHip_AddmmQuantGroupF32Device(*pack)
+        N.check_result(ok, "addmm_quant_group")
+
+    @staticmethod
     def AddmmQuantBatch(result, m1, weight_data, ggml_type, ne0, raw_bytes, weight_offsets, weight_ne1):
         """Row b of m1 times the sub-weight at weight_offsets[b] (GgmlBasicOps.cs:689-704)."""
         rv = _host_view(result, standard=True)

@@ -1,0 +1,90 @@
+"""Synthetic GGUF block generators (torch, run on whatever device the input lives on).
+
+Benchmarks need W ~ N(0, 0.02) in raw Q8_0 / Q4_K / MXFP4 blocks without touching the CPU
+oracle.  Q8_0 and MXFP4 follow the reference quantizers exactly (closed forms,
+ggml-quants.c:199-222 and :260-305).  Q4_K uses a plain min/max affine fit per 32-weight
+sub-block instead of the reference's iterative scale search (ggml-quants.c:622-701): the
+bytes are valid Q4_K super-blocks of the same statistics, not the reference's bytes.
+"""
+import torch
+
+MXFP4_TABLE = [0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12]
+
+
+def _half_bytes(v):
+    """fp32 tensor [n] -> uint8 [n, 2] little-endian fp16 (round to nearest even)."""
+    return v.to(torch.float16).view(torch.uint8).reshape(-1, 2)
+
+
+def quantize_q8_0(w):
+    x = w.reshape(-1, 32).float()
+    amax = x.abs().amax(dim=1)
+    d = amax / 127.0
+    inv = torch.where(d != 0, 1.0 / d, torch.zeros_like(d))
+    s = x * inv[:, None]
+    q = torch.where(s >= 0, torch.floor(s + 0.5), torch.ceil(s - 0.5)).to(torch.int8)   # roundf: half away from zero
+    out = torch.empty((x.shape[0], 34), dtype=torch.uint8, device=w.device)
+    out[:, :2] = _half_bytes(d)
+    out[:, 2:] = q.view(torch.uint8)
+    return out.reshape(-1)
+
+
+def quantize_mxfp4(w):
+    x = w.reshape(-1, 32).float()
+    amax = x.abs().amax(dim=1)
+    e = torch.where(amax > 0, torch.floor(torch.log2(amax.clamp_min(1e-38))) - 2 + 127, torch.zeros_like(amax))
+    e = e.clamp(0, 255)
+    d = torch.pow(torch.tensor(2.0, device=w.device), e - 128.0)
+    table = torch.tensor(MXFP4_TABLE, dtype=torch.float32, device=w.device)
+    err = (table[None, None, :] * d[:, None, None] - x[:, :, None]).abs()
+    idx = torch.argmin(err, dim=2).to(torch.uint8)
+    out = torch.empty((x.shape[0], 17), dtype=torch.uint8, device=w.device)
+    out[:, 0] = e.to(torch.uint8)
+    out[:, 1:] = idx[:, :16] | (idx[:, 16:] << 4)
+    return out.reshape(-1)
+
+
+def quantize_q4_k_simple(w):
+    x = w.reshape(-1, 8, 32).float()                     # [blocks, sub-blocks, 32]
+    lo = x.amin(dim=2).clamp_max(0.0)
+    hi = x.amax(dim=2)
+    scale = (hi - lo) / 15.0                             # per sub-block step
+    mn = -lo                                             # per sub-block offset (>= 0)
+    d = scale.amax(dim=1) / 63.0
+    dmin = mn.amax(dim=1) / 63.0
+    d16 = d.to(torch.float16).float()
+    dmin16 = dmin.to(torch.float16).float()
+    ls = torch.where(d16[:, None] > 0, torch.round(scale / d16[:, None].clamp_min(1e-30)), torch.zeros_like(scale)).clamp(0, 63)
+    lm = torch.where(dmin16[:, None] > 0, torch.round(mn / dmin16[:, None].clamp_min(1e-30)), torch.zeros_like(mn)).clamp(0, 63)
+    eff_d = d16[:, None] * ls
+    eff_m = dmin16[:, None] * lm
+    q = torch.where(eff_d[:, :, None] > 0, torch.round((x + eff_m[:, :, None]) / eff_d[:, :, None].clamp_min(1e-30)),
+                    torch.zeros_like(x)).clamp(0, 15).to(torch.uint8)
+    ls = ls.to(torch.uint8)
+    lm = lm.to(torch.uint8)
+    nb = x.shape[0]
+    out = torch.zeros((nb, 144), dtype=torch.uint8, device=w.device)
+    out[:, 0:2] = _half_bytes(d)
+    out[:, 2:4] = _half_bytes(dmin)
+    sc = out[:, 4:16]
+    sc[:, 0:4] = ls[:, 0:4] | ((ls[:, 4:8] >> 4) << 6)
+    sc[:, 4:8] = lm[:, 0:4] | ((lm[:, 4:8] >> 4) << 6)
+    sc[:, 8:12] = (ls[:, 4:8] & 0x0F) | ((lm[:, 4:8] & 0x0F) << 4)
+    qq = q.reshape(nb, 4, 2, 32)
+    out[:, 16:] = (qq[:, :, 0, :] | (qq[:, :, 1, :] << 4)).reshape(nb, 128)
+    return out.reshape(-1)
+
+
+QUANTIZERS = {8: quantize_q8_0, 12: quantize_q4_k_simple, 39: quantize_mxfp4}
+
+
+def random_weight(ggml_type, n_rows, n_cols, device, seed, sigma=0.02, chunk_rows=4096):
+    """Raw blocks of an [n_rows x n_cols] weight ~ N(0, sigma), generated in row chunks."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    parts = []
+    for r0 in range(0, n_rows, chunk_rows):
+        rows = min(chunk_rows, n_rows - r0)
+        w = torch.randn((rows, n_cols), generator=g, device=device, dtype=torch.float32) * sigma
+        parts.append(QUANTIZERS[ggml_type](w))
+    return torch.cat(parts)

@@ -164,3 +164,51 @@ def test_error_paths(hip, oracle):
     hip.AddmmQuant(y, x, wq.ctypes.data, Q4_K, K, Nn, wq.size)
     assert N.get_last_error() == ""
     hip.ClearHostBufferCache()
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+def test_grouped_launch_equals_single_launches(hip, oracle, name):
+    """TSHip_AddmmQuantGroupF32Device: several independent decode GEMVs in one launch."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(41)
+    shapes = [(96, 1024), (33, 2048), (700, 512), (1, 256), (260, 3072), (64, 1024), (17, 768)]
+    if name == "q4_k":
+        shapes = [(n, k) for n, k in shapes if k % 256 == 0]
+    ws, xs, ys, refs = [], [], [], []
+    for n, k in shapes:
+        wq = oracle.quantize(T[name], (rng.standard_normal(n * k) * 0.02).astype(np.float32))
+        x = rng.standard_normal((1, k)).astype(np.float32)
+        refs.append(oracle.matmul_f64(T[name], wq, n, k, x))
+        ws.append(QuantizedWeight(torch.from_numpy(wq).cuda(), T[name], k, n))
+        xs.append(torch.from_numpy(x).cuda())
+        ys.append(torch.full((1, n), float("nan"), device="cuda"))
+    hip.UseCurrentStream()
+    pack = hip.PrepareGroup(ys, xs, ws)
+    hip.AddmmQuantGroupDevice(pack)
+    torch.cuda.synchronize()
+    for y, ref, w, x in zip(ys, refs, ws, xs):
+        check(name, y.cpu().numpy(), ref)
+        single = hip.LinearForward(x, w)
+        torch.cuda.synchronize()
+        assert inputs.row_l2_err(y.cpu().numpy(), single.cpu().numpy()) < 1e-5
+
+
+def test_grouped_full_layer(hip, oracle):
+    """configs[1] at full size: the seven Q4_K projections of one layer in one launch."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    ws, xs, ys, refs = [], [], [], []
+    for tname, (fmt, n, k) in inputs.CFG2.items():
+        tag = f"cfg2.{tname}"
+        wq = oracle.quantize(T[fmt], inputs.weights(tag, n * k))
+        x = inputs.activations(tag, 1, k)
+        refs.append(oracle.matmul_f64(T[fmt], wq, n, k, x))
+        ws.append(QuantizedWeight(torch.from_numpy(wq).cuda(), T[fmt], k, n))
+        xs.append(torch.from_numpy(x).cuda())
+        ys.append(torch.empty((1, n), device="cuda"))
+    hip.UseCurrentStream()
+    hip.AddmmQuantGroupDevice(hip.PrepareGroup(ys, xs, ws))
+    torch.cuda.synchronize()
+    for y, ref in zip(ys, refs):
+        check("q4_k", y.cpu().numpy(), ref)
