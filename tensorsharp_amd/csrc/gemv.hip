@@ -4,10 +4,11 @@
 //   * persistent workgroups of 8 wavefronts (two per CU); each workgroup stages x once into LDS
 //     in the layout its format's unpack order wants (fp16 pairs for Q4_K / MXFP4, fp32 for
 //     Q8_0), padded so that a ds_read_b128 per lane is bank-conflict free;
-//   * a wavefront owns one weight row at a time.  The row is cut into "units" (Q8_0: one
-//     34-byte block, Q4_K: one 64-weight group = 32 quant bytes + the super-block header,
-//     MXFP4: one 17-byte block); lane l takes units l, l+64, ... so consecutive lanes read
-//     consecutive bytes of the raw blocks with 128-bit loads, everything that depends only on
+//   * a wavefront owns four consecutive weight rows at a time, one row per 16 lanes.  A row is
+//     cut into "units" (Q8_0: one 34-byte block, Q4_K: one 64-weight group = 32 quant bytes +
+//     the super-block header, MXFP4: one 17-byte block); lane l of a row takes units l, l+16,
+//     ... so consecutive lanes read consecutive bytes of the raw blocks with 128-bit loads,
+//     everything that depends only on
 //     the lane (block offset, scale bit positions, LDS address of its activations) is computed
 //     once, and the row / slot part of every address is a scalar.  Unaligned units (34 B / 17 B) are fetched as aligned dwords through a
 //     range-checked buffer resource and re-aligned in registers with v_alignbyte;
@@ -18,8 +19,8 @@
 //     Q4_K nibbles masked in place are fp16 subnormals (q * 2^-24) feeding v_dot2_f32_f16,
 //     MXFP4 E2M1 pairs -> fp16 with v_cvt_scalef32_pk_f16_fp4 feeding v_dot2_f32_f16;
 //     block scales (fp16 d, 6-bit K-quant scales/mins, E8M0) are applied once per unit in fp32;
-//   * the per-lane row sum is reduced with DPP inside each row of 16 lanes and four
-//     v_readlane across rows.
+//   * the per-lane sums of a row are reduced with four DPP adds inside its 16 lanes; the four
+//     results of a group leave as one store instruction.
 //
 // Arithmetic restated from TensorSharp.Models/ManagedQuantizedOps.cs:156-200 (dot of a
 // dequantised row with the activation row); for the 4-bit formats the activations of each
@@ -35,10 +36,23 @@ namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kWaves = 8;
+// tuning constants (overridable at build time for experiments)
+#ifndef TSHIP_GEMV_WAVES
+#define TSHIP_GEMV_WAVES 8
+#endif
+#ifndef TSHIP_GEMV_KU
+#define TSHIP_GEMV_KU 1
+#endif
+#ifndef TSHIP_GEMV_WG_PER_CU
+#define TSHIP_GEMV_WG_PER_CU 2
+#endif
+#ifndef TSHIP_GEMV_XFIRST
+#define TSHIP_GEMV_XFIRST 0
+#endif
+constexpr int kWaves = TSHIP_GEMV_WAVES;
 constexpr int kThreads = kWaves * 64;
 constexpr int kMaxGroup = 8;
-constexpr int kU = 2;      // units per lane whose loads are in flight together
+constexpr int kU = TSHIP_GEMV_KU;      // steps per wavefront fetched together, one fetch ahead of the compute
 
 // one GEMV
 struct GemvProblem {
@@ -88,18 +102,6 @@ constexpr int kDppXor2 = 0x4e;         // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7-i inside each 8
 constexpr int kDppMirror = 0x140;      // lane i <-> 15-i inside each 16
 
-// sum over the 64 lanes; result valid in every lane
-__device__ __forceinline__ float wave_sum(float v)
-{
-    v += TSHIP_DPP_F(v, kDppXor1);
-    v += TSHIP_DPP_F(v, kDppXor2);
-    v += TSHIP_DPP_F(v, kDppHalfMirror);
-    v += TSHIP_DPP_F(v, kDppMirror);
-    const int iv = __float_as_int(v);
-    return __int_as_float(__builtin_amdgcn_readlane(iv, 0)) + __int_as_float(__builtin_amdgcn_readlane(iv, 16)) +
-           __int_as_float(__builtin_amdgcn_readlane(iv, 32)) + __int_as_float(__builtin_amdgcn_readlane(iv, 48));
-}
-
 // Power-of-two pair (inverse, scale) that brings amax into [2^13, 2^14): fp16 keeps 11 bits for
 // everything down to 2^-27 of the unit's largest magnitude and nothing overflows.
 __device__ __forceinline__ void pow2_scale(float amax, float* inv, float* scale)
@@ -147,73 +149,64 @@ struct FmtQ4K {
 
     static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 8) * 144; }
 
+    static constexpr int kStageF4 = 1;   // float4 loads per work item
+
+    // work item `it` = activations [4*it, 4*it+4): byte offset of its float4
+    static __device__ __forceinline__ void stage_offsets(int it, uint32_t (&off)[kStageF4]) { off[0] = (uint32_t)it * 16u; }
+
     // one work item = one float4; the 16 lanes of a DPP row share a unit
-    static __device__ __forceinline__ void stage(const float* __restrict__ x, int K, uint32_t* lds)
+    static __device__ __forceinline__ void stage_store(const float4 (&vv)[kStageF4], int it, bool live, uint32_t* lds)
     {
-        const int items = K >> 2;
-        constexpr int kChunk = 4;
-        for (int base = 0; base < items; base += kThreads * kChunk) {
-            float4 v[kChunk];
-#pragma unroll
-            for (int c = 0; c < kChunk; ++c) {
-                const int it = base + c * kThreads + threadIdx.x;
-                v[c] = it < items ? reinterpret_cast<const float4*>(x)[it] : float4{0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int c = 0; c < kChunk; ++c) {
-                const int it = base + c * kThreads + threadIdx.x;
-                if (base + c * kThreads >= items) break;  // uniform
-                float amax = fmaxf(fmaxf(fabsf(v[c].x), fabsf(v[c].y)), fmaxf(fabsf(v[c].z), fabsf(v[c].w)));
-                amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
-                amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
-                amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppHalfMirror));
-                amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppMirror));
-                float inv, scale;
-                pow2_scale(amax, &inv, &scale);
-                const _Float16 h0 = (_Float16)(v[c].x * inv), h1 = (_Float16)(v[c].y * inv);
-                const _Float16 h2 = (_Float16)(v[c].z * inv), h3 = (_Float16)(v[c].w * inv);
-                float s = ((float)h0 + (float)h1) + ((float)h2 + (float)h3);
-                // sum over the 8 lanes of one 32-weight sub-block
-                s += TSHIP_DPP_F(s, kDppXor1);
-                s += TSHIP_DPP_F(s, kDppXor2);
-                s += TSHIP_DPP_F(s, kDppHalfMirror);
-                if (it < items) {
-                    const int e = it << 2;
-                    const int g = e >> 6, r = e & 63;
-                    const int sub = r >> 5, j = (r & 31) >> 2;
-                    uint32_t* unit = lds + g * kLdsDwords;
-                    H2U a, b;
-                    a.h = half2_t{h0, h2};
-                    b.h = half2_t{h1, h3};
-                    uint2 w2;
-                    w2.x = a.u;
-                    w2.y = b.u;
-                    *reinterpret_cast<uint2*>(unit + 4 * j + 2 * sub) = w2;
-                    if ((threadIdx.x & 7) == 0) reinterpret_cast<float*>(unit)[32 + sub] = s;
-                    if ((threadIdx.x & 15) == 0) reinterpret_cast<float*>(unit)[34] = scale;
-                }
-            }
+        const float4 v = vv[0];
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppHalfMirror));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppMirror));
+        float inv, scale;
+        pow2_scale(amax, &inv, &scale);
+        const _Float16 h0 = (_Float16)(v.x * inv), h1 = (_Float16)(v.y * inv);
+        const _Float16 h2 = (_Float16)(v.z * inv), h3 = (_Float16)(v.w * inv);
+        float s = ((float)h0 + (float)h1) + ((float)h2 + (float)h3);
+        // sum over the 8 lanes of one 32-weight sub-block
+        s += TSHIP_DPP_F(s, kDppXor1);
+        s += TSHIP_DPP_F(s, kDppXor2);
+        s += TSHIP_DPP_F(s, kDppHalfMirror);
+        if (live) {
+            const int e = it << 2;
+            const int g = e >> 6, r = e & 63;
+            const int sub = r >> 5, j = (r & 31) >> 2;
+            uint32_t* unit = lds + g * kLdsDwords;
+            H2U a, b;
+            a.h = half2_t{h0, h2};
+            b.h = half2_t{h1, h3};
+            uint2 w2;
+            w2.x = a.u;
+            w2.y = b.u;
+            *reinterpret_cast<uint2*>(unit + 4 * j + 2 * sub) = w2;
+            if ((threadIdx.x & 7) == 0) reinterpret_cast<float*>(unit)[32 + sub] = s;
+            if ((threadIdx.x & 15) == 0) reinterpret_cast<float*>(unit)[34] = scale;
         }
     }
+    static __device__ __forceinline__ int stage_items(int K) { return K >> 2; }
 
+    static constexpr int kSlotBytes = 4 * 144;   // 16 consecutive units of a row
 
-    static constexpr int kSlotBytes = 16 * 144;   // 64 consecutive units of a row
-
-    // Lane-invariant part of the addressing: unit g = lane + 64*slot lives in super-block g/4 at
-    // quant bytes (g & 3)*32; only the slot/row part (a scalar) changes from step to step.
+    // Lane-invariant part of the addressing: unit g = l16 + 16*step lives in super-block g/4 at
+    // quant bytes (g & 3)*32; only the step / row-group part (a scalar) changes from step to step.
     struct Lane {
-        uint32_t voff;    // byte offset of the lane's super-block inside a slot
+        uint32_t voff;    // byte offset of the lane's super-block: its row inside the group + inside the step
         uint32_t qoff;    // byte offset of the lane's 32 quant bytes inside the super-block
         int sh;           // bit position of the lane's scale pair inside the packed scale dwords
         bool upper;       // sub-blocks 4..7 use the split 4+2 bit encoding
     };
-    static __device__ __forceinline__ Lane lane_setup(int lane)
+    static __device__ __forceinline__ Lane lane_setup(int sub, int l16, uint32_t row_bytes)
     {
         Lane L;
-        L.voff = (uint32_t)(lane >> 2) * 144u;
-        L.qoff = 16u + (uint32_t)(lane & 3) * 32u;
-        L.sh = (lane & 1) * 16;
-        L.upper = (lane & 2) != 0;
+        L.voff = (uint32_t)sub * row_bytes + (uint32_t)(l16 >> 2) * 144u;
+        L.qoff = 16u + (uint32_t)(l16 & 3) * 32u;
+        L.sh = (l16 & 1) * 16;
+        L.upper = (l16 & 2) != 0;
         return L;
     }
 
@@ -232,6 +225,9 @@ struct FmtQ4K {
     static __device__ __forceinline__ float dot(const uint32_t (&w)[kRegs], const Lane& L, uint32_t /*aux*/,
                                                 const uint32_t* xu_dw)
     {
+#ifdef TSHIP_GEMV_DEBUG_NOCOMPUTE
+        return __uint_as_float((w[0] ^ w[1] ^ w[2] ^ w[3] ^ w[4] ^ w[5] ^ w[6] ^ w[7] ^ w[8] ^ w[9] ^ w[10] ^ w[11]) & 0x3fffffffu) * (float)xu_dw[0];
+#endif
         const uint4* xu = reinterpret_cast<const uint4*>(xu_dw);
         float lo = 0.f, hi = 0.f;
 #pragma unroll
@@ -275,55 +271,48 @@ struct FmtMXFP4 {
 
     static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 5) * 17; }
 
+    static constexpr int kStageF4 = 2;
+
     // one work item = x[b*32 + 4i .. +3] and x[b*32 + 16 + 4i .. +3]; the 4 lanes of a quad share a unit
-    static __device__ __forceinline__ void stage(const float* __restrict__ x, int K, uint32_t* lds)
+    static __device__ __forceinline__ void stage_offsets(int it, uint32_t (&off)[kStageF4])
     {
-        const int items = K >> 3;
-        constexpr int kChunk = 2;
-        for (int base = 0; base < items; base += kThreads * kChunk) {
-            float4 lo[kChunk], hi[kChunk];
-#pragma unroll
-            for (int c = 0; c < kChunk; ++c) {
-                const int it = base + c * kThreads + threadIdx.x;
-                const int b = it >> 2, i = it & 3;
-                const bool live = it < items;
-                lo[c] = live ? *reinterpret_cast<const float4*>(x + b * 32 + 4 * i) : float4{0.f, 0.f, 0.f, 0.f};
-                hi[c] = live ? *reinterpret_cast<const float4*>(x + b * 32 + 16 + 4 * i) : float4{0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int c = 0; c < kChunk; ++c) {
-                const int it = base + c * kThreads + threadIdx.x;
-                if (base + c * kThreads >= items) break;  // uniform
-                float amax = fmaxf(fmaxf(fmaxf(fabsf(lo[c].x), fabsf(lo[c].y)), fmaxf(fabsf(lo[c].z), fabsf(lo[c].w))),
-                                   fmaxf(fmaxf(fabsf(hi[c].x), fabsf(hi[c].y)), fmaxf(fabsf(hi[c].z), fabsf(hi[c].w))));
-                amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
-                amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
-                float inv, scale;
-                pow2_scale(amax, &inv, &scale);
-                if (it < items) {
-                    const int b = it >> 2, i = it & 3;
-                    uint4 o;
-                    o.x = pack_half2(lo[c].x * inv, hi[c].x * inv);
-                    o.y = pack_half2(lo[c].y * inv, hi[c].y * inv);
-                    o.z = pack_half2(lo[c].z * inv, hi[c].z * inv);
-                    o.w = pack_half2(lo[c].w * inv, hi[c].w * inv);
-                    uint32_t* unit = lds + b * kLdsDwords;
-                    *reinterpret_cast<uint4*>(unit + 4 * i) = o;
-                    if (i == 0) reinterpret_cast<float*>(unit)[16] = scale;
-                }
-            }
-        }
+        const uint32_t b = (uint32_t)it >> 2, i = (uint32_t)it & 3u;
+        off[0] = (b * 32u + 4u * i) * 4u;
+        off[1] = off[0] + 64u;
     }
 
-    static constexpr int kSlotBytes = 64 * 17;
+    static __device__ __forceinline__ void stage_store(const float4 (&vv)[kStageF4], int it, bool live, uint32_t* lds)
+    {
+        const float4 lo = vv[0], hi = vv[1];
+        float amax = fmaxf(fmaxf(fmaxf(fabsf(lo.x), fabsf(lo.y)), fmaxf(fabsf(lo.z), fabsf(lo.w))),
+                           fmaxf(fmaxf(fabsf(hi.x), fabsf(hi.y)), fmaxf(fabsf(hi.z), fabsf(hi.w))));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
+        float inv, scale;
+        pow2_scale(amax, &inv, &scale);
+        if (live) {
+            const int b = it >> 2, i = it & 3;
+            uint4 o;
+            o.x = pack_half2(lo.x * inv, hi.x * inv);
+            o.y = pack_half2(lo.y * inv, hi.y * inv);
+            o.z = pack_half2(lo.z * inv, hi.z * inv);
+            o.w = pack_half2(lo.w * inv, hi.w * inv);
+            uint32_t* unit = lds + b * kLdsDwords;
+            *reinterpret_cast<uint4*>(unit + 4 * i) = o;
+            if (i == 0) reinterpret_cast<float*>(unit)[16] = scale;
+        }
+    }
+    static __device__ __forceinline__ int stage_items(int K) { return K >> 3; }
+
+    static constexpr int kSlotBytes = 16 * 17;
 
     struct Lane {
-        uint32_t voff;   // byte offset of the lane's block inside a slot (before alignment)
+        uint32_t voff;   // byte offset of the lane's block: row inside the group + inside the step (before alignment)
     };
-    static __device__ __forceinline__ Lane lane_setup(int lane)
+    static __device__ __forceinline__ Lane lane_setup(int sub, int l16, uint32_t row_bytes)
     {
         Lane L;
-        L.voff = (uint32_t)lane * 17u;
+        L.voff = (uint32_t)sub * row_bytes + (uint32_t)l16 * 17u;
         return L;
     }
 
@@ -388,34 +377,25 @@ struct FmtQ80 {
 
     static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 5) * 34; }
 
-    static __device__ __forceinline__ void stage(const float* __restrict__ x, int K, uint32_t* lds)
-    {
-        const int items = K >> 2;
-        constexpr int kChunk = 4;
-        for (int base = 0; base < items; base += kThreads * kChunk) {
-            float4 v[kChunk];
-#pragma unroll
-            for (int c = 0; c < kChunk; ++c) {
-                const int it = base + c * kThreads + threadIdx.x;
-                v[c] = it < items ? reinterpret_cast<const float4*>(x)[it] : float4{0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int c = 0; c < kChunk; ++c) {
-                const int it = base + c * kThreads + threadIdx.x;
-                if (it < items) *reinterpret_cast<float4*>(lds + (it >> 3) * kLdsDwords + (it & 7) * 4) = v[c];
-            }
-        }
-    }
+    static constexpr int kStageF4 = 1;
 
-    static constexpr int kSlotBytes = 64 * 34;
+    static __device__ __forceinline__ void stage_offsets(int it, uint32_t (&off)[kStageF4]) { off[0] = (uint32_t)it * 16u; }
+
+    static __device__ __forceinline__ void stage_store(const float4 (&vv)[kStageF4], int it, bool live, uint32_t* lds)
+    {
+        if (live) *reinterpret_cast<float4*>(lds + (it >> 3) * kLdsDwords + (it & 7) * 4) = vv[0];
+    }
+    static __device__ __forceinline__ int stage_items(int K) { return K >> 2; }
+
+    static constexpr int kSlotBytes = 16 * 34;
 
     struct Lane {
         uint32_t voff;
     };
-    static __device__ __forceinline__ Lane lane_setup(int lane)
+    static __device__ __forceinline__ Lane lane_setup(int sub, int l16, uint32_t row_bytes)
     {
         Lane L;
-        L.voff = (uint32_t)lane * 34u;
+        L.voff = (uint32_t)sub * row_bytes + (uint32_t)l16 * 34u;
         return L;
     }
 
@@ -464,23 +444,26 @@ struct FmtQ80 {
 // ==========================================================================================
 // The kernel body shared by all formats.
 // ==========================================================================================
-// One step = one slot (64 consecutive units) of one row.  Steps of a wavefront are numbered
-// row-major over (row, slot); kU steps are fetched together, one fetch ahead of the compute.
+// A wavefront works on a group of 4 consecutive rows at a time, one row per 16 lanes.
+// One step = 16 consecutive units of each of the 4 rows.  Steps of a wavefront are numbered
+// group-major over (group, step); kU steps are fetched together, one fetch ahead of the compute.
 template <typename F>
 struct Step {
     uint32_t w[F::kRegs];
     uint32_t aux;     // format-specific lane datum produced by the load (byte position in its window)
-    int slot;         // uniform
-    int row;          // uniform; >= N marks a step past the end (its loads read zeros)
+    int step;         // uniform
+    int group;        // uniform; >= ngroups marks a step past the end (its loads read zeros)
 };
 
 template <typename F>
 __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, uint32_t* lds)
 {
     const int lane = threadIdx.x & 63;
+    const int sub = lane >> 4, l16 = lane & 15;
     const int N = P.N, K = P.K;
     const int upr = K / F::kUnitElems;          // units per row
-    const int nslots = (upr + 63) >> 6;         // steps per row
+    const int nsteps = (upr + 15) >> 4;         // steps per row group
+    const int ngroups = (N + 3) >> 2;
     const uint32_t row_bytes = (uint32_t)F::row_bytes(K);
     const int wave_stride = nwg * kWaves;
     const int gw = __builtin_amdgcn_readfirstlane(wg * kWaves + (int)(threadIdx.x >> 6));
@@ -492,54 +475,101 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const uint32_t extent = ((uint32_t)P.w_bytes + base_delta + 3u) & ~3u;
     const __amdgpu_buffer_rsrc_t rs =
         __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, (int)extent, 0x00020000);
-    const typename F::Lane L = F::lane_setup(lane);
-    const uint32_t lds_lane = (uint32_t)lane * F::kLdsDwords;
+    const typename F::Lane L = F::lane_setup(sub, l16, row_bytes);
+    const uint32_t lds_lane = (uint32_t)l16 * F::kLdsDwords;
 
-    // issue the loads of step (row, slot); no waiting, no branches
-    auto fetch = [&](int row, int slot, Step<F>& st) {
-        const bool row_ok = row < N;                                   // uniform
-        const uint32_t start = base_delta + (row_ok ? (uint32_t)row * row_bytes : 0u) + (uint32_t)slot * F::kSlotBytes;
+    // issue the loads of step (group, step); no waiting, no branches
+    auto fetch = [&](int group, int step, Step<F>& st) {
+        const bool group_ok = group < ngroups;                         // uniform
+        const int row0 = group_ok ? group * 4 : 0;
+        const uint32_t start = base_delta + (uint32_t)row0 * row_bytes + (uint32_t)step * F::kSlotBytes;
         const uint32_t soff = start & ~3u;                             // scalar part of the address
-        const bool live = row_ok && (lane + (slot << 6) < upr);
-        st.slot = slot;
-        st.row = row;
-        st.aux = F::load(rs, L, soff, start & 3u, slot, live, st.w);
+        const bool live = group_ok && (row0 + sub < N) && (l16 + (step << 4) < upr);
+        st.step = step;
+        st.group = group;
+        st.aux = F::load(rs, L, soff, start & 3u, step, live, st.w);
     };
-    auto advance = [&](int& row, int& slot) {
-        if (++slot == nslots) {
-            slot = 0;
-            row += wave_stride;
+    auto advance = [&](int& group, int& step) {
+        if (++step == nsteps) {
+            step = 0;
+            group += wave_stride;
         }
     };
 
+    // x is requested first (it mostly hits L2 and memory answers a wavefront in order), then the
+    // first weight steps, and only then is x converted into LDS - with the weights already in flight.
+    const int items = F::stage_items(K);
+    const __amdgpu_buffer_rsrc_t xrs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(P.x), 0, K * 4, 0x00020000);
+    constexpr int kStageChunk = 8 / F::kStageF4;           // work items per thread per pass
+    float4 xv[kStageChunk][F::kStageF4];
+    auto stage_issue = [&](int base) {
+#pragma unroll
+        for (int c = 0; c < kStageChunk; ++c) {
+            const int it = base + c * kThreads + (int)threadIdx.x;
+            uint32_t off[F::kStageF4];
+            F::stage_offsets(it, off);
+#pragma unroll
+            for (int q = 0; q < F::kStageF4; ++q) {
+                // items past the end fall outside the resource and read as zeros
+                const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
+                xv[c][q] = float4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+            }
+        }
+    };
+    auto stage_commit = [&](int base) {
+#pragma unroll
+        for (int c = 0; c < kStageChunk; ++c) {
+            if (base + c * kThreads < items) {   // uniform
+                const int it = base + c * kThreads + (int)threadIdx.x;
+                F::stage_store(xv[c], it, it < items, lds);
+            }
+        }
+    };
+
+    if (TSHIP_GEMV_XFIRST) stage_issue(0);
+    // kU steps per wavefront are requested before x is staged, so weight latency overlaps the
+    // prologue; in the loop the next kU steps are requested before the current ones are consumed.
     Step<F> cur[kU], nxt[kU];
-    int frow = gw, fslot = 0;                  // next step to fetch
+    int fgroup = gw, fstep = 0;                // next step to fetch
 #pragma unroll
     for (int i = 0; i < kU; ++i) {
-        fetch(frow, fslot, cur[i]);            // in flight while x is staged
-        advance(frow, fslot);
+        fetch(fgroup, fstep, cur[i]);
+        advance(fgroup, fstep);
     }
-
-    F::stage(P.x, K, lds);
-    // lanes past the end of a row read their activations from the zero-filled tail of the last slot
-    for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nslots * 64 * F::kLdsDwords; i += kThreads) lds[i] = 0u;
+    if (!TSHIP_GEMV_XFIRST) stage_issue(0);
+#ifdef TSHIP_GEMV_DEBUG_NOSTAGE
+    if (P.N < 0)
+#endif
+    stage_commit(0);
+    for (int base = kThreads * kStageChunk; base < items; base += kThreads * kStageChunk) {
+        stage_issue(base);
+        stage_commit(base);
+    }
+    // lanes past the end of a row read their activations from the zero-filled tail of the last step
+    for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nsteps * 16 * F::kLdsDwords; i += kThreads) lds[i] = 0u;
     __syncthreads();
 
     float acc = 0.f;
-    while (cur[0].row < N) {
+    while (cur[0].group < ngroups) {
 #pragma unroll
         for (int i = 0; i < kU; ++i) {
-            fetch(frow, fslot, nxt[i]);
-            advance(frow, fslot);
+            fetch(fgroup, fstep, nxt[i]);
+            advance(fgroup, fstep);
         }
 #pragma unroll
         for (int i = 0; i < kU; ++i) {
-            // lanes past the end of a row (and steps past the last row) hold zeros, zero scales included
-            const uint32_t* xu = lds + lds_lane + (uint32_t)cur[i].slot * (64u * F::kLdsDwords);
+            // lanes past the end of a row (and steps past the last group) hold zeros, zero scales included
+            const uint32_t* xu = lds + lds_lane + (uint32_t)cur[i].step * (16u * F::kLdsDwords);
             acc += F::dot(cur[i].w, L, cur[i].aux, xu);
-            if (cur[i].slot == nslots - 1) {   // uniform: row complete
-                const float t = wave_sum(acc);
-                if (lane == 0 && cur[i].row < N) P.y[cur[i].row] = t;
+            if (cur[i].step == nsteps - 1) {   // uniform: the 4 rows of the group are complete
+                float t = acc;
+                t += TSHIP_DPP_F(t, kDppXor1);
+                t += TSHIP_DPP_F(t, kDppXor2);
+                t += TSHIP_DPP_F(t, kDppHalfMirror);
+                t += TSHIP_DPP_F(t, kDppMirror);
+                const int row = cur[i].group * 4 + sub;
+                if (l16 == 0 && cur[i].group < ngroups && row < N) P.y[row] = t;
                 acc = 0.f;
             }
         }
@@ -565,10 +595,10 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
 
 int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
 
-// x staged as whole slots of 64 units (the tail of the last slot is zero-filled)
+// x staged as whole steps of 16 units (the tail of the last step is zero-filled)
 size_t lds_bytes_for(int type, int K)
 {
-    const size_t units = (size_t)((K / unit_elems(type) + 63) / 64) * 64;
+    const size_t units = (size_t)((K / unit_elems(type) + 15) / 16) * 16;
     return units * (type == kTypeMXFP4 ? 80 : 144);
 }
 
@@ -592,9 +622,9 @@ bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 int gemv_max_k(int type)
 {
     switch (type) {
-    case kTypeQ8_0: return (int)(kMaxLds / 144 / 64) * 64 * 32;
-    case kTypeQ4_K: return (int)(kMaxLds / 144 / 64) * 64 * 64;
-    case kTypeMXFP4: return (int)(kMaxLds / 80 / 64) * 64 * 32;
+    case kTypeQ8_0: return (int)(kMaxLds / 144 / 16) * 16 * 32;
+    case kTypeQ4_K: return (int)(kMaxLds / 144 / 16) * 16 * 64;
+    case kTypeMXFP4: return (int)(kMaxLds / 80 / 16) * 16 * 32;
     default: return 0;
     }
 }
@@ -626,7 +656,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         lds = std::max(lds, lds_bytes_for(type, args[i].K));
         total_bytes += (double)args[i].w_bytes;
     }
-    int per_cu = (int)std::min<size_t>(2, (160 * 1024) / (lds + 256));
+    int per_cu = (int)std::min<size_t>(TSHIP_GEMV_WG_PER_CU, (160 * 1024) / (lds + 256));
     if (per_cu < 1) per_cu = 1;
     const int budget = di.num_cus * per_cu;
 
@@ -637,7 +667,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     for (int i = 0; i < count; ++i) {
         // workgroups in proportion to the bytes each problem streams
         int share = std::max(1, (int)((double)budget * (double)args[i].w_bytes / total_bytes + 0.5));
-        share = std::min(share, (args[i].N + kWaves - 1) / kWaves);
+        share = std::min(share, ((args[i].N + 3) / 4 + kWaves - 1) / kWaves);
         g.p[i].w = static_cast<const uint8_t*>(args[i].w);
         g.p[i].w_bytes = args[i].w_bytes;
         g.p[i].x = args[i].x;
