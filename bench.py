@@ -176,6 +176,28 @@ def main():
             extra[f"cfg2_q4_k_gemv_{name}_{n}x{k}"] = one_matrix(Q4_K, n, k, max(2, int(300e6 // (n * row_bytes(Q4_K, k))) + 1))
         extra["cfg4_mxfp4_gemv_gate_up_5760x2880"] = one_matrix(MXFP4, 5760, 2880, 32)
         extra["cfg4_mxfp4_gemv_down_2880x2880"] = one_matrix(MXFP4, 2880, 2880, 64)
+
+        # prefill GEMMs (configs[2] and configs[4]): TFLOP/s = 2*M*N*K / time of the whole call
+        # (activation convert kernel + MFMA GEMM), fp16 operands -> priced against 2516.6 TFLOP/s
+        def prefill(t, m, n, k, iters=20):
+            w = QuantizedWeight(synth.random_weight(t, n, k, dev, seed=91), t, k, n)
+            x = torch.randn((m, k), device=dev, dtype=torch.float32)
+            y = torch.empty((m, n), device=dev, dtype=torch.float32)
+
+            def f(i):
+                HipBasicOps.AddmmQuantDevice(y, x, w.ptr, t, k, n, w.raw_bytes)
+            for i in range(3):
+                f(i)
+            ev, wall = time_region(f, iters, torch)
+            us = ev * 1e3 / iters
+            tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
+            return {"us_per_call_events": round(us, 1), "TFLOPs": round(tf, 1), "pct_mfma_fp16_peak": round(100 * tf / 2516.6, 1)}
+
+        extra["cfg3_q4_k_gemm_512x14336x4096"] = prefill(Q4_K, 512, 14336, 4096)
+        extra["cfg5_q4_k_gemm_2048x21504x5376"] = prefill(Q4_K, 2048, 21504, 5376, 10)
+        extra["cfg5_q8_0_gemm_2048x21504x5376"] = prefill(Q8_0, 2048, 21504, 5376, 10)
+        extra["cfg5_q4_k_gemm_2048x5376x21504"] = prefill(Q4_K, 2048, 5376, 21504, 10)
+        extra["cfg5_q8_0_gemm_2048x5376x21504"] = prefill(Q8_0, 2048, 5376, 21504, 10)
         out["extra"] = extra
 
     if not args.no_cpu:

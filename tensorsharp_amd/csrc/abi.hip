@@ -99,6 +99,29 @@ struct Workspace {
 };
 Workspace g_ws;
 
+// Scratch of the *Device entry points (converted activations of the prefill GEMM).  Grow-only:
+// after the first call of a given size nothing is allocated any more.
+std::mutex g_dev_ws_mutex;
+void* g_dev_ws = nullptr;
+size_t g_dev_ws_bytes = 0;
+
+void* dev_ws_reserve(size_t bytes)
+{
+    std::lock_guard<std::mutex> lock(g_dev_ws_mutex);
+    if (bytes > g_dev_ws_bytes) {
+        if (g_dev_ws) {
+            if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return nullptr;
+            (void)hipFree(g_dev_ws);
+        }
+        g_dev_ws = nullptr;
+        g_dev_ws_bytes = 0;
+        const size_t want = bytes + bytes / 4;
+        if (!hip_ok(hipMalloc(&g_dev_ws, want), "hipMalloc(gemm workspace)")) return nullptr;
+        g_dev_ws_bytes = want;
+    }
+    return g_dev_ws;
+}
+
 bool ws_reserve(size_t dev_bytes, size_t pinned_bytes)
 {
     if (dev_bytes > g_ws.dev_bytes) {
@@ -221,9 +244,8 @@ bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D&
     const size_t w_bytes = row_size(type, K) * (size_t)N;
     if (!check_device_operands(m1, w, type)) return false;
     const int M = m1.dim0;
-    if (K <= gemv_max_k(type)) {
-        // decode / small batch: one GEMV per activation row
-        // TODO(prefill): M > 1 goes to the MFMA GEMM once it lands
+    if (M <= 3 && K <= gemv_max_k(type)) {
+        // decode / tiny batch: one bandwidth-bound GEMV per activation row
         for (int m = 0; m < M; ++m) {
             const float* x = static_cast<const float*>(m1.data) + (int64_t)m * m1.stride0;
             float* y = static_cast<float*>(result.data) + (int64_t)m * result.stride0;
@@ -231,8 +253,12 @@ bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D&
         }
         return true;
     }
-    set_last_error("addmm_quant: K is too large for this build.");
-    return false;
+    // prefill: activations -> fp16 workspace, then the MFMA GEMM
+    void* ws = dev_ws_reserve(gemm_workspace_bytes(M, (int)K));
+    if (!ws) return false;
+    if (!launch_convert_x(type, static_cast<const float*>(m1.data), m1.stride0, nullptr, M, (int)K, ws, stream)) return false;
+    return launch_gemm(type, w, (int64_t)w_bytes, ws, static_cast<float*>(result.data), result.stride0, nullptr, M, (int)N,
+                       (int)K, nullptr, stream);
 }
 
 // device pointer for m2_data: preloaded key, cached host pointer, or upload now

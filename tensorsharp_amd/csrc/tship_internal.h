@@ -73,4 +73,29 @@ struct GemvArgs {
 int gemv_max_group();
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);
 
+// ---- prefill GEMM ---------------------------------------------------------------------------
+// Workspace layout: [M floats of row scales, padded to 256 B][M x Kp fp16 activations].
+size_t gemm_workspace_bytes(int M, int K);
+int gemm_tile_m(int M);   // rows of activations per tile for a plain (ungrouped) launch
+
+// fp32 activations -> workspace (fp16 in the weight format's unpack order + per-row scales);
+// row_map (device, optional) gathers source rows.
+bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
+                      hipStream_t stream);
+
+// Grouped launches (MoE): m-tiles enumerated by device tables; weights of expert e start at
+// w + e * expert_stride and span w_bytes each.
+struct GemmTiles {
+    const int* expert;
+    const int* row0;
+    const int* rows;
+    int count;
+    int bm;
+    int64_t expert_stride;
+};
+
+// c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
+bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc,
+                 const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream);
+
 }  // namespace tship

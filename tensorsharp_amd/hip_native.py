@@ -67,6 +67,14 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise NativeLibraryMissing(
                 f"{LIB_PATH} not found: build it with `python -m tensorsharp_amd.build` (needs hipcc).")
+        # PyTorch wheels ship their own copy of the HIP runtime.  Two HIP runtimes in one process cannot
+        # both open the GPU, so when torch is installed its runtime is loaded first and this library
+        # (which only asks for libamdhip64.so.7) binds to the same copy.  Without torch the system
+        # runtime under /opt/rocm is used.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             f = getattr(L, name)
