@@ -5,12 +5,12 @@
 //      magnitude overflows or underflows fp16), written in the k-order in which the weight
 //      format unpacks (so the dequantizer never has to shuffle lanes), zero-padded to a
 //      multiple of the k-tile.  Optionally gathers rows through an index (MoE).
-//   2. gemm_kernel: BM x BN x 64 tiles, 4 wavefronts (2 x 2).  Per k-tile the raw quantized bytes
-//      of BN weight rows are loaded (Q4_K: 32 quant bytes + the super-block header per row,
-//      Q8_0 / MXFP4: two blocks per row through a range-checked buffer resource), dequantized
+//   2. gemm_kernel: BM x BN x 64 tiles (256 x 256 with 8 wavefronts for large M).  Per k-tile the raw
+//      quantized bytes of BN weight rows are loaded (Q4_K: 32 quant bytes + the super-block header per
+//      row, Q8_0 / MXFP4: two blocks per row through a range-checked buffer resource), dequantized
 //      ONCE to fp16 with packed-fp16 VALU and written to LDS next to the activation tile; the
-//      wavefronts then run v_mfma_f32_32x32x16_f16 out of LDS with fp32 accumulation.  The
-//      global loads of tile t+1 are in flight while tile t is multiplied.
+//      wavefronts then run v_mfma_f32_32x32x16_f16 out of LDS with fp32 accumulation.  LDS is
+//      double-buffered, the global loads run two tiles ahead, and the tile order is XCD-aware.
 //   3. epilogue: fp32 accumulators times the row scale -> C (optionally scattered through a row
 //      index).
 //
@@ -31,7 +31,6 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kBK = 64;                 // k-tile
 constexpr int kLdsRow = kBK + 8;        // fp16 per LDS row: 144 B keeps ds_read_b128 conflict-free
-constexpr int kThreads = 256;
 constexpr uint32_t kDeadOffset = 0x80000000u;
 
 union H2U {
@@ -257,44 +256,82 @@ struct GQ80 {
 };
 
 struct GemmArgs {
-    const uint8_t* w;        // weight bytes (of the expert for grouped launches: see tiles)
-    int64_t w_bytes;
+    const uint8_t* w;        // weight bytes (of expert 0 for grouped launches)
+    int64_t w_bytes;         // bytes of one weight matrix (per expert for grouped launches)
     const _Float16* x16;     // [rows x Kp] converted activations
     const float* xscale;     // [rows]
     float* c;                // result
     int64_t ldc;
     const int* c_rows;       // optional: result row index per activation row (scatter)
     int M, N, K, Kp;
-    // grouped (MoE) launches: blockIdx.y enumerates m-tiles through this table
-    const int* tile_expert;  // [tiles] expert id
-    const int* tile_row0;    // [tiles] first activation row
-    const int* tile_rows;    // [tiles] rows in the tile (<= BM)
+    int m_tiles, n_tiles;
+    // grouped (MoE) launches: m-tiles enumerated through this table
+    const int* tile_expert;  // [m_tiles] expert id
+    const int* tile_row0;    // [m_tiles] first activation row
+    const int* tile_rows;    // [m_tiles] rows in the tile (<= BM)
     int64_t expert_stride;   // bytes between experts
 };
 
-template <typename G, int BM, int BN>
-__global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmArgs A)
+// One k-tile of MFMA work for a wavefront: TM x TN tiles of 32x32, four k-steps of 16.
+template <int TM, int TN>
+__device__ __forceinline__ void mma_tile(const _Float16* xs, const _Float16* ws, float16_t (&acc)[TM][TN])
 {
-    constexpr int TM = BM / 64, TN = BN / 64;        // 32x32 MFMA tiles per wavefront along m / n
-    constexpr int XCH = BM * 8 / kThreads;           // 16-byte activation chunks per thread per k-tile
-    constexpr int WIT = BN * 2 / kThreads;           // weight items per thread per k-tile
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+        half8_t a[TM], b[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kLdsRow + ks * 16);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const half8_t*>(ws + j * 32 * kLdsRow + ks * 16);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+}
+
+// BM x BN x 64 tiles, WM x WN wavefronts.  LDS holds two k-tiles (activations + dequantized weights);
+// per iteration every wavefront (a) dequantizes the raw bytes it fetched for tile kt+1 into the idle
+// buffer, (b) requests the raw bytes of tile kt+2, (c) multiplies tile kt.  Wavefronts that share a
+// SIMD run (a)(b) and (c) in opposite order so that the VALU dequantization of one overlaps the MFMA
+// phase of the other.  One barrier per k-tile.
+template <typename G, int BM, int BN, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64) gemm_kernel(const GemmArgs A)
+{
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int XCH = BM * 8 / NT;                 // 16-byte activation chunks per thread per k-tile
+    constexpr int WIT = BN * 2 / NT;                 // weight items per thread per k-tile
+    constexpr int kBufElems = (BM + BN) * kLdsRow;
+    static_assert(XCH >= 1 && WIT >= 1, "tile too small for the workgroup");
     extern __shared__ _Float16 smem[];
-    _Float16* Xs = smem;                             // [BM][kLdsRow]
-    _Float16* Ws = smem + BM * kLdsRow;              // [BN][kLdsRow]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs, so each XCD gets a contiguous
+    // run of tiles; consecutive tiles share the activation rows (same m-tile), which then stay in that
+    // XCD's L2 while its CUs walk over the weight columns.
+    const int total = A.m_tiles * A.n_tiles;
+    int t = blockIdx.x;
+    {
+        const int per = (total + 7) >> 3;
+        const int xcd = t & 7, slot = t >> 3;
+        t = xcd * per + slot;
+        if (slot >= per || t >= total) return;
+    }
+    const int mt = t / A.n_tiles, nt = t - mt * A.n_tiles;
     int m0, m_rows;
     const uint8_t* wbase = A.w;
     if (A.tile_expert) {
-        m0 = A.tile_row0[blockIdx.y];
-        m_rows = A.tile_rows[blockIdx.y];
-        wbase += (int64_t)A.tile_expert[blockIdx.y] * A.expert_stride;
+        m0 = A.tile_row0[mt];
+        m_rows = A.tile_rows[mt];
+        wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
     } else {
-        m0 = blockIdx.y * BM;
+        m0 = mt * BM;
         m_rows = min(BM, A.M - m0);
     }
-    const int n0 = blockIdx.x * BN;
+    const int n0 = nt * BN;
 
     WTensor W;
     const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
@@ -304,45 +341,43 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmArgs A)
     W.K = A.K;
     W.row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
 
-    // per-thread assignments
-    int x_row[XCH], x_chunk[XCH];
+    // per-thread sources / destinations (constant over the k loop)
+    const _Float16* x_src[XCH];
+    int x_dst[XCH];
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
-        const int c = tid + i * kThreads;
-        x_row[i] = c >> 3;
-        x_chunk[i] = c & 7;
+        const int c = tid + i * NT;
+        const int row = c >> 3, chunk = c & 7;
+        x_src[i] = A.x16 + (int64_t)(m0 + min(row, m_rows - 1)) * A.Kp + chunk * 8;
+        x_dst[i] = row * kLdsRow + chunk * 8;
     }
-    int w_row[WIT], w_part[WIT];
     uint32_t w_off[WIT];
+    int w_part[WIT], w_dst[WIT];
 #pragma unroll
     for (int i = 0; i < WIT; ++i) {
-        const int it = tid + i * kThreads;
-        w_row[i] = it >> 1;
+        const int it = tid + i * NT;
+        const int row = it >> 1;
         w_part[i] = it & 1;
-        const int n = min(n0 + w_row[i], A.N - 1);
-        w_off[i] = W.base_delta + (uint32_t)n * W.row_bytes;
+        w_off[i] = W.base_delta + (uint32_t)min(n0 + row, A.N - 1) * W.row_bytes;
+        w_dst[i] = (BM + row) * kLdsRow;
     }
 
-    uint4 xr[XCH];
+    uint4_t xr[XCH];
     uint32_t wr[WIT][G::kRegs];
-    auto load_tile = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < XCH; ++i) {
-            const int m = m0 + min(x_row[i], m_rows - 1);
-            xr[i] = *reinterpret_cast<const uint4*>(A.x16 + (int64_t)m * A.Kp + kt * kBK + x_chunk[i] * 8);
-        }
-#pragma unroll
-        for (int i = 0; i < WIT; ++i) G::load(W, w_off[i], kt, w_part[i], wr[i]);
-    };
-    auto store_tile = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < XCH; ++i) *reinterpret_cast<uint4*>(Xs + x_row[i] * kLdsRow + x_chunk[i] * 8) = xr[i];
-#pragma unroll
-        for (int i = 0; i < WIT; ++i) {
-            const bool live = G::kWholeTile || (kt * 2 + w_part[i]) * 32 < A.K;
-            G::store(wr[i], w_off[i], kt, w_part[i], live, Ws + w_row[i] * kLdsRow);
-        }
-    };
+#define TSHIP_GEMM_LOAD(kt)                                                                        \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < XCH; ++i) xr[i] = *reinterpret_cast<const uint4_t*>(x_src[i] + (kt) * kBK); \
+        _Pragma("unroll") for (int i = 0; i < WIT; ++i) G::load(W, w_off[i], (kt), w_part[i], wr[i]);  \
+    } while (0)
+#define TSHIP_GEMM_STORE(kt, buf)                                                                  \
+    do {                                                                                           \
+        _Float16* dstb = smem + (buf) * kBufElems;                                                 \
+        _Pragma("unroll") for (int i = 0; i < XCH; ++i) *reinterpret_cast<uint4_t*>(dstb + x_dst[i]) = xr[i]; \
+        _Pragma("unroll") for (int i = 0; i < WIT; ++i) {                                          \
+            const bool live = G::kWholeTile || ((kt) * 2 + w_part[i]) * 32 < A.K;                  \
+            G::store(wr[i], w_off[i], (kt), w_part[i], live, dstb + w_dst[i]);                     \
+        }                                                                                          \
+    } while (0)
 
     float16_t acc[TM][TN];
 #pragma unroll
@@ -353,42 +388,42 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmArgs A)
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const int nkt = A.Kp / kBK;
-    const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-    load_tile(0);
+    const int frag = (lane & 31) * kLdsRow + (lane >> 5) * 8;
+    const int xs_off = wm * (BM / WM) * kLdsRow + frag;
+    const int ws_off = (BM + wn * (BN / WN)) * kLdsRow + frag;
+    // wavefronts w and w + 4 share a SIMD: one of them multiplies first, the other dequantizes first
+    const bool mma_first = (wave & 4) != 0 && NT > 256;
+
+    TSHIP_GEMM_LOAD(0);
+    TSHIP_GEMM_STORE(0, 0);
+    if (nkt > 1) TSHIP_GEMM_LOAD(1);
+    __syncthreads();
     for (int kt = 0; kt < nkt; ++kt) {
-        store_tile(kt);
-        __syncthreads();
-        if (kt + 1 < nkt) load_tile(kt + 1);
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            half8_t a[TM], b[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                a[i] = *reinterpret_cast<const half8_t*>(Xs + (wm * (BM / 2) + i * 32 + frag_row) * kLdsRow + ks * 16 + frag_k);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                b[j] = *reinterpret_cast<const half8_t*>(Ws + (wn * (BN / 2) + j * 32 + frag_row) * kLdsRow + ks * 16 + frag_k);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
+        const int cur = kt & 1;
+        const _Float16* bufc = smem + cur * kBufElems;
+        if (mma_first) mma_tile<TM, TN>(bufc + xs_off, bufc + ws_off, acc);
+        if (kt + 1 < nkt) TSHIP_GEMM_STORE(kt + 1, cur ^ 1);
+        // past the last tile the loads wrap to tile 0: harmless, and the loop body stays branch-free
+        TSHIP_GEMM_LOAD(kt + 2 < nkt ? kt + 2 : 0);
+        if (!mma_first) mma_tile<TM, TN>(bufc + xs_off, bufc + ws_off, acc);
         __syncthreads();
     }
+#undef TSHIP_GEMM_LOAD
+#undef TSHIP_GEMM_STORE
 
     // epilogue: D[row = 8*(r/4) + 4*(lane/32) + r%4][col = lane%32]
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int ml = wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int ml = wm * (BM / WM) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             if (ml < m_rows) {
                 const int m = m0 + ml;
                 const float s = A.xscale[m];
                 float* crow = A.c + (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
-                    const int n = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
+                    const int n = n0 + wn * (BN / WN) + j * 32 + (lane & 31);
                     if (n < A.N) crow[n] = acc[i][j][r] * s;
                 }
             }
@@ -396,25 +431,29 @@ __global__ void __launch_bounds__(kThreads) gemm_kernel(const GemmArgs A)
     }
 }
 
-template <typename G, int BM, int BN>
-bool launch_tiles(const GemmArgs& a, int m_tiles, hipStream_t stream)
+template <typename G, int BM, int BN, int WM, int WN>
+bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    auto kern = gemm_kernel<G, BM, BN>;
-    const size_t lds = (size_t)(BM + BN) * kLdsRow * sizeof(_Float16);
+    auto kern = gemm_kernel<G, BM, BN, WM, WN>;
+    const size_t lds = (size_t)2 * (BM + BN) * kLdsRow * sizeof(_Float16);
     if (lds > 64 * 1024 &&
         !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                 "gemm: raising the dynamic LDS limit"))
         return false;
-    const dim3 grid((unsigned)((a.N + BN - 1) / BN), (unsigned)m_tiles);
-    hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds, stream, a);
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + BN - 1) / BN;
+    const int total = a.m_tiles * a.n_tiles;
+    const int grid = ((total + 7) / 8) * 8;          // whole rounds over the 8 XCDs
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, stream, a);
     return hip_ok(hipGetLastError(), "gemm launch");
 }
 
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-    if (bm == 128) return launch_tiles<G, 128, 128>(a, m_tiles, stream);
-    return launch_tiles<G, 64, 128>(a, m_tiles, stream);
+    if (bm == 256) return launch_tiles<G, 256, 256, 2, 4>(a, m_tiles, stream);
+    if (bm == 128) return launch_tiles<G, 128, 256, 2, 4>(a, m_tiles, stream);
+    return launch_tiles<G, 64, 128, 1, 4>(a, m_tiles, stream);
 }
 
 }  // namespace
@@ -425,7 +464,7 @@ size_t gemm_workspace_bytes(int M, int K)
     return (size_t)M * kp * sizeof(_Float16) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255) + 256;
 }
 
-int gemm_tile_m(int M) { return M > 64 ? 128 : 64; }
+int gemm_tile_m(int M) { return M > 1024 ? 256 : M > 64 ? 128 : 64; }
 
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
                       hipStream_t stream)
