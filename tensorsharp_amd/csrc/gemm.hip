@@ -272,21 +272,32 @@ struct GemmArgs {
     int64_t expert_stride;   // bytes between experts
 };
 
-// One k-tile of MFMA work for a wavefront: TM x TN tiles of 32x32, four k-steps of 16.
+// One k-tile of MFMA work for a wavefront: TM x TN tiles of 32x32, four k-steps of 16.  The LDS
+// fragments of k-step s+1 are requested before the MFMAs of k-step s are issued, so the matrix
+// pipe covers the LDS latency.
 template <int TM, int TN>
 __device__ __forceinline__ void mma_tile(const _Float16* xs, const _Float16* ws, float16_t (&acc)[TM][TN])
 {
+    half8_t a[2][TM], b[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a[0][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kLdsRow);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b[0][j] = *reinterpret_cast<const half8_t*>(ws + j * 32 * kLdsRow);
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
-        half8_t a[TM], b[TN];
+        const int c = ks & 1, n = c ^ 1;
+        if (ks + 1 < kBK / 16) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kLdsRow + ks * 16);
+            for (int i = 0; i < TM; ++i) a[n][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kLdsRow + (ks + 1) * 16);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const half8_t*>(ws + j * 32 * kLdsRow + ks * 16);
+            for (int j = 0; j < TN; ++j) b[n][j] = *reinterpret_cast<const half8_t*>(ws + j * 32 * kLdsRow + (ks + 1) * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // keep the requests above the MFMAs they are meant to overlap
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[c][i], b[c][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -451,7 +462,10 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-    if (bm == 256) return launch_tiles<G, 256, 256, 2, 4>(a, m_tiles, stream);
+#ifdef TSHIP_GEMM_VARIANT
+    if (bm == 256) return launch_tiles<G, TSHIP_GEMM_VARIANT>(a, m_tiles, stream);
+#endif
+    if (bm == 256) return launch_tiles<G, 256, 256, 4, 2>(a, m_tiles, stream);
     if (bm == 128) return launch_tiles<G, 128, 256, 2, 4>(a, m_tiles, stream);
     return launch_tiles<G, 64, 128, 1, 4>(a, m_tiles, stream);
 }
