@@ -82,6 +82,9 @@ def main():
     ap.add_argument("--copies", type=int, default=6, help="distinct layer copies cycled (6 x 123 MB > Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 1 GiB device-to-device copy (20 times): the known-size kernel against "
+                         "which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU kernel path only: this build has no multi-GPU code; run with --gpus 1.",
@@ -101,6 +104,16 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     HipBasicOps.UseCurrentStream()
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)       # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "calibrate_copy_bytes_written": src.numel() * 4,
+                          "launches": 20}))
+        return
 
     # ---- workload: `copies` layers of seven Q4_K matrices, device resident -------------------
     layers = []
