@@ -22,6 +22,9 @@ sys.path.insert(0, ROOT)
 
 Q8_0, Q4_K, MXFP4 = 8, 12, 39
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the grouped Q4_K GEMV from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the
+# reading of a 1 GiB copy (profiles/gemv_q4k_layer_hbm_traffic.txt); not measured by this script.
+MEASURED_TRAFFIC_BYTES = 124520000
 
 LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
     ("wq", 4096, 4096), ("wk", 1024, 4096), ("wv", 1024, 4096), ("wo", 4096, 4096),
@@ -140,13 +143,7 @@ def main():
     kern_us = ev_ms * 1e3 / args.steps          # one launch per step: HIP-event time per launch
     achieved = step_bytes / (kern_us * 1e-6) / 1e9
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("q4k_layer_group_gemv")
-        except (OSError, ValueError):
-            traffic = None
+    traffic = MEASURED_TRAFFIC_BYTES
 
     out = {
         "metric": "Q4_K/Q8_0/MXFP4 matmul: decode GB/s (% HBM peak), prefill TFLOP/s (% MFMA)",
