@@ -125,6 +125,27 @@ TSHIP_EXPORT int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView
                                                 int m2_ggml_type, const int64_t* m2_ne0s, const int64_t* m2_ne1s,
                                                 const int64_t* m2_raw_bytes);
 
+/* ---- MoE (GPT-OSS expert stage), device pointers ------------------------------------------ */
+
+/* No bridge export: the reference routes in C# (GptOssModel.MoERoute, TensorSharp.Models/Models/GptOss/GptOssModel.cs:814-865,
+ * the part after the router linear).  logits [T x E] -> ids / weights [T x k]: top-k by repeated argmax (first
+ * maximum wins ties), softmax over the k selected logits.  1 <= k <= 16. */
+TSHIP_EXPORT int TSHip_MoERouteF32Device(TSHipTensorView2D logits, int k, int32_t* ids, float* weights);
+
+/* No bridge export: replaces the per-expert C# loop GptOssModel.MoEForwardSingleToken / MoEForwardBatched / ExpertFFN
+ * (GptOssModel.cs:718-812, :867-934) that issues two AddmmQuant calls per expert.
+ *   result[t] = sum_s weights[t,s] * ( W_down[e] * swiglu_oai( W_gate_up[e] * hidden[t] + b_gate_up[e] ) + b_down[e] ),
+ *   e = ids[t,s]
+ * gate_up_w: [E][2F rows][H] raw blocks (gate rows, then up rows), down_w: [E][H rows][F]; biases [E][2F] / [E][H] or
+ * NULL.  Few assignments (T*k <= 8) run as grouped decode GEMVs with the expert picked on the device; otherwise the
+ * assignments are counting-sorted by expert on the device and each linear is ONE grouped MFMA GEMM launch.
+ * Accumulation order over experts: ascending expert id for T > 1, selection order for T == 1 (as the reference). */
+TSHIP_EXPORT int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D hidden, const int32_t* ids,
+                                                  const float* weights, int k, const void* gate_up_w,
+                                                  const float* gate_up_bias, const void* down_w, const float* down_bias,
+                                                  int ggml_type, int n_experts, int64_t H, int64_t F, float alpha,
+                                                  float limit);
+
 #ifdef __cplusplus
 }
 #endif

@@ -504,6 +504,110 @@ int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView2D* results, 
     });
 }
 
+int TSHip_MoERouteF32Device(TSHipTensorView2D logits, int k, int32_t* ids, float* weights)
+{
+    return guarded(0, "moe_route", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_desc(logits, "logits")) return 0;
+        if (ids == nullptr || weights == nullptr || logits.stride1 != 1) {
+            set_last_error("Invalid arguments for moe_route.");
+            return 0;
+        }
+        if (!launch_moe_route(static_cast<const float*>(logits.data), logits.stride0, logits.dim0, logits.dim1, k, ids, weights,
+                              g_stream.load()))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D hidden, const int32_t* ids,
+                                     const float* weights, int k, const void* gate_up_w, const float* gate_up_bias,
+                                     const void* down_w, const float* down_bias, int ggml_type, int n_experts, int64_t H,
+                                     int64_t F, float alpha, float limit)
+{
+    return guarded(0, "moe_experts_forward", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_desc(result, "result") || !validate_desc(hidden, "hidden")) return 0;
+        if (!ids || !weights || !gate_up_w || !down_w || k < 1 || k > 16 || n_experts < 1 || H <= 0 || F <= 0) {
+            set_last_error("Invalid arguments for moe_experts_forward.");
+            return 0;
+        }
+        if (hidden.dim1 != H || result.dim1 != H || hidden.dim0 != result.dim0 || hidden.stride1 != 1 || !is_standard_view(result)) {
+            set_last_error("Size mismatch: hidden / result must be [T x H] row-contiguous views in moe_experts_forward.");
+            return 0;
+        }
+        const size_t rs_h = row_size(ggml_type, H), rs_f = row_size(ggml_type, F);
+        if (!is_quant_type(ggml_type) || rs_h == 0 || rs_f == 0) {
+            set_last_error("Unsupported quantized weight type or row length for moe_experts_forward.");
+            return 0;
+        }
+        if (!check_device_operands(hidden, gate_up_w, ggml_type) || !check_device_operands(hidden, down_w, ggml_type)) return 0;
+        const int T = hidden.dim0;
+        const int64_t A64 = (int64_t)T * k;
+        if (A64 > (1 << 24)) {
+            set_last_error("moe_experts_forward: too many (token, expert) assignments for one call.");
+            return 0;
+        }
+        const int A = (int)A64, E = n_experts;
+        const int64_t gu_bytes = (int64_t)rs_h * 2 * F, dn_bytes = (int64_t)rs_f * H;   // per expert
+        hipStream_t stream = g_stream.load();
+        auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+        const bool small = A <= gemv_max_group() && H <= gemv_max_k(ggml_type) && F <= gemv_max_k(ggml_type);
+        const int bm = (A / E) > 96 ? 128 : 64;
+        const int max_tiles = A / bm + E;
+        // carve the workspace
+        size_t off = 0;
+        auto take = [&](size_t b) { const size_t o = off; off += al(b); return o; };
+        const size_t o_offsets = take((size_t)(E + 1) * 4), o_token = take((size_t)A * 4), o_expert = take((size_t)A * 4);
+        const size_t o_pos = take((size_t)A * 4), o_te = take((size_t)max_tiles * 4), o_tr0 = take((size_t)max_tiles * 4);
+        const size_t o_trn = take((size_t)max_tiles * 4);
+        const size_t o_ws1 = take(gemm_workspace_bytes(A, (int)H)), o_ws2 = take(gemm_workspace_bytes(A, (int)F));
+        const size_t o_gu = take((size_t)A * 2 * F * 4), o_act = take((size_t)A * F * 4), o_dn = take((size_t)A * H * 4);
+        char* ws = static_cast<char*>(dev_ws_reserve(off));
+        if (!ws) return 0;
+        float* gu = reinterpret_cast<float*>(ws + o_gu);
+        float* act = reinterpret_cast<float*>(ws + o_act);
+        float* dn = reinterpret_cast<float*>(ws + o_dn);
+        const float* hid = static_cast<const float*>(hidden.data);
+        if (small) {
+            // decode: one GEMV per (token, slot), expert chosen on the device through ids
+            GemvArgs args[16];
+            for (int a = 0; a < A; ++a) {
+                args[a] = GemvArgs{gate_up_w, gu_bytes, hid + (int64_t)(a / k) * hidden.stride0, gu + (int64_t)a * 2 * F,
+                                   (int)(2 * F), (int)H, ids + a, gu_bytes};
+            }
+            if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
+            if (!launch_moe_swiglu(gu, gate_up_bias, ids, A, (int)F, alpha, limit, act, stream)) return 0;
+            for (int a = 0; a < A; ++a)
+                args[a] = GemvArgs{down_w, dn_bytes, act + (int64_t)a * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes};
+            if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
+            if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, (int)H, T == 1, static_cast<float*>(result.data),
+                                    result.stride0, stream))
+                return 0;
+        } else {
+            MoeMaps maps{reinterpret_cast<int*>(ws + o_offsets), reinterpret_cast<int*>(ws + o_token),
+                         reinterpret_cast<int*>(ws + o_expert), reinterpret_cast<int*>(ws + o_pos),
+                         reinterpret_cast<int*>(ws + o_te),      reinterpret_cast<int*>(ws + o_tr0),
+                         reinterpret_cast<int*>(ws + o_trn)};
+            if (!launch_moe_group(ids, A, k, E, bm, max_tiles, maps, stream)) return 0;
+            GemmTiles tiles{maps.tile_expert, maps.tile_row0, maps.tile_rows, max_tiles, bm, gu_bytes};
+            if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream)) return 0;
+            if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream))
+                return 0;
+            if (!launch_moe_swiglu(gu, gate_up_bias, maps.expert_of, A, (int)F, alpha, limit, act, stream)) return 0;
+            if (!launch_convert_x(ggml_type, act, F, nullptr, A, (int)F, ws + o_ws2, stream)) return 0;
+            tiles.expert_stride = dn_bytes;
+            if (!launch_gemm(ggml_type, down_w, dn_bytes, ws + o_ws2, dn, H, nullptr, A, (int)H, (int)F, &tiles, stream)) return 0;
+            if (!launch_moe_combine(dn, down_bias, ids, weights, maps.pos_of, T, k, (int)H, false,
+                                    static_cast<float*>(result.data), result.stride0, stream))
+                return 0;
+        }
+        clear_last_error();
+        return 1;
+    });
+}
+
 int TSHip_AddmmQuantF32(TSHipTensorView2D result, TSHipTensorView2D m1, void* m2_data, int m2_ggml_type, int64_t m2_ne0,
                         int64_t m2_ne1, int64_t m2_raw_bytes)
 {

@@ -337,6 +337,7 @@ __global__ void __launch_bounds__(WM * WN * 64) gemm_kernel(const GemmArgs A)
     if (A.tile_expert) {
         m0 = A.tile_row0[mt];
         m_rows = A.tile_rows[mt];
+        if (m_rows <= 0) return;          // table entries past the last tile
         wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
     } else {
         m0 = mt * BM;

@@ -60,6 +60,8 @@ struct GemvProblem {
     int64_t w_bytes;
     const float* x;
     float* y;
+    const int* expert_id;     // optional (MoE): the weight is w + expert_id[0] * expert_stride
+    int64_t expert_stride;
     int N;
     int K;
 };
@@ -467,7 +469,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const uint32_t row_bytes = (uint32_t)F::row_bytes(K);
     const int wave_stride = nwg * kWaves;
     const int gw = __builtin_amdgcn_readfirstlane(wg * kWaves + (int)(threadIdx.x >> 6));
-    const uintptr_t w_begin = reinterpret_cast<uintptr_t>(P.w);
+    const uintptr_t w_begin = reinterpret_cast<uintptr_t>(P.w) + (P.expert_id ? (uintptr_t)((int64_t)P.expert_id[0] * P.expert_stride) : 0);
     // one range-checked resource for the whole tensor (host guarantees w_bytes < 2 GiB); the extent is
     // rounded up to whole dwords, which stay inside the last 4-byte word the tensor touches
     const uintptr_t base = w_begin & ~(uintptr_t)3;
@@ -674,6 +676,8 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         g.p[i].y = args[i].y;
         g.p[i].N = args[i].N;
         g.p[i].K = args[i].K;
+        g.p[i].expert_id = args[i].expert_id;
+        g.p[i].expert_stride = args[i].expert_stride;
         g.wg_begin[i] = begin;
         begin += share;
     }
@@ -687,7 +691,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
 
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream)
 {
-    GemvArgs a{w, w_bytes, x, y, N, K};
+    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0};
     return launch_gemv_group(type, 1, &a, stream);
 }
 

@@ -69,6 +69,8 @@ struct GemvArgs {
     float* y;
     int N;
     int K;
+    const int* expert_id = nullptr;   // optional device pointer (MoE): weight = w + expert_id[0] * expert_stride
+    int64_t expert_stride = 0;
 };
 int gemv_max_group();
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);
@@ -97,5 +99,27 @@ struct GemmTiles {
 // c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc,
                  const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream);
+
+// ---- MoE (GPT-OSS expert stage) -------------------------------------------------------------
+// ids / weights: [T x k] device; top-k by repeated argmax (first maximum wins), softmax over the k logits.
+bool launch_moe_route(const float* logits, int64_t ld, int T, int E, int k, int* ids, float* weights, hipStream_t stream);
+
+struct MoeMaps {            // all device pointers, A = T * k assignments
+    int* offsets;           // [E + 1]
+    int* token_of;          // [A] token of sorted row
+    int* expert_of;         // [A] expert of sorted row
+    int* pos_of;            // [A] sorted row of assignment (t, s); -1 for an invalid expert id
+    int* tile_expert;       // [max_tiles]
+    int* tile_row0;         // [max_tiles]
+    int* tile_rows;         // [max_tiles], 0 past the last tile
+};
+// stable counting sort of the assignments by expert + m-tile table for the grouped GEMM
+bool launch_moe_group(const int* ids, int A, int k, int E, int bm, int max_tiles, const MoeMaps& maps, hipStream_t stream);
+// act[r][f] = swiglu_oai(gu[r][f] + b[e][f], gu[r][F + f] + b[e][F + f]); e = expert_of[r]
+bool launch_moe_swiglu(const float* gu, const float* bias, const int* expert_of, int rows, int F, float alpha, float limit,
+                       float* act, hipStream_t stream);
+// out[t][h] = sum_s w[t][s] * (dn[pos_of[t*k+s]][h] + b[e][h]); order: ascending expert (or slot order)
+bool launch_moe_combine(const float* dn, const float* bias, const int* ids, const float* weights, const int* pos_of, int T,
+                        int k, int H, bool slot_order, float* out, int64_t ldo, hipStream_t stream);
 
 }  // namespace tship

@@ -181,6 +181,34 @@ class HipBasicOps:
     def ClearHostBufferCache():
         N.lib().TSHip_ClearHostBufferCache()
 
+    # -- MoE (GptOssModel.MoERoute / MoEForward twins, device tensors) --------------------------
+    @staticmethod
+    def MoERoute(logits, k):
+        """logits [T x E] (CUDA fp32) -> (weights [T x k] fp32, ids [T x k] int32)."""
+        import torch
+        T = logits.shape[0]
+        ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+        wts = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+        HipBasicOps.UseCurrentStream()
+        ok = N.lib().TSHip_MoERouteF32Device(_device_view(logits), int(k), ids.data_ptr(), wts.data_ptr())
+        N.check_result(ok, "moe_route")
+        return wts, ids
+
+    @staticmethod
+    def MoEExpertsForward(hidden, ids, weights, gate_up_w, gate_up_b, down_w, down_b, ggml_type, n_experts, H, F,
+                          alpha=1.702, limit=7.0):
+        """Expert stage of GptOssModel.MoEForward for routed tokens; all tensors on the device."""
+        import torch
+        out = torch.empty((hidden.shape[0], H), dtype=torch.float32, device=hidden.device)
+        HipBasicOps.UseCurrentStream()
+        ok = N.lib().TSHip_MoEExpertsForwardF32Device(
+            _device_view(out), _device_view(hidden), ids.data_ptr(), weights.data_ptr(), int(ids.shape[1]),
+            gate_up_w.data_ptr(), None if gate_up_b is None else gate_up_b.data_ptr(), down_w.data_ptr(),
+            None if down_b is None else down_b.data_ptr(), int(ggml_type), int(n_experts), int(H), int(F), float(alpha),
+            float(limit))
+        N.check_result(ok, "moe_experts_forward")
+        return out
+
     # -- LinearForward twin (ModelBase.cs:875-905): allocate result, route by residency -----
     @staticmethod
     def LinearForward(m1, qw: QuantizedWeight):
