@@ -208,6 +208,39 @@ def main():
         extra["cfg5_q8_0_gemm_2048x21504x5376"] = prefill(Q8_0, 2048, 21504, 5376, 10)
         extra["cfg5_q4_k_gemm_2048x5376x21504"] = prefill(Q4_K, 2048, 5376, 21504, 10)
         extra["cfg5_q8_0_gemm_2048x5376x21504"] = prefill(Q8_0, 2048, 5376, 21504, 10)
+        # MoE expert stage (configs[3]): 32 MXFP4 experts, top-4, hidden 2880; T = 1 (decode, HBM-bound:
+        # bytes of the 4 selected experts' gate_up + down blocks) and T = 256 (prefill, grouped GEMM)
+        def moe(T, iters):
+            E, H, F, k = 32, 2880, 2880, 4
+            sets = [(synth.random_weight(MXFP4, E * 2 * F, H, dev, seed=500 + c),
+                     synth.random_weight(MXFP4, E * H, F, dev, seed=600 + c)) for c in range(2)]
+            hidden = torch.randn((T, H), device=dev, dtype=torch.float32)
+            gi = torch.Generator(device="cpu")
+            gi.manual_seed(11)
+            idsets = [torch.stack([torch.randperm(E, generator=gi)[:k] for _ in range(T)]).to(torch.int32).to(dev)
+                      for _ in range(8)]
+            wts = torch.softmax(torch.randn((T, k), device=dev), dim=1).contiguous()
+
+            def f(i):
+                gu, dn = sets[i % 2]
+                HipBasicOps.MoEExpertsForward(hidden, idsets[i % 8], wts, gu, None, dn, None, MXFP4, E, H, F)
+            for i in range(5):
+                f(i)
+            ev, wall = time_region(f, iters, torch)
+            us = ev * 1e3 / iters
+            res = {"us_per_call_events": round(us, 1)}
+            if T == 1:
+                b = k * (2 * F + H) * row_bytes(MXFP4, H)
+                res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                            "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)})
+            else:
+                fl = 2.0 * T * k * (2 * F * H + H * F)
+                res.update({"TFLOPs": round(fl / (us * 1e-6) / 1e12, 1),
+                            "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / 2516.6, 1)})
+            return res
+
+        extra["cfg4_mxfp4_moe_experts_T1"] = moe(1, n_it)
+        extra["cfg4_mxfp4_moe_experts_T256"] = moe(256, 30)
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -5,12 +5,14 @@
 //      magnitude overflows or underflows fp16), written in the k-order in which the weight
 //      format unpacks (so the dequantizer never has to shuffle lanes), zero-padded to a
 //      multiple of the k-tile.  Optionally gathers rows through an index (MoE).
-//   2. gemm_kernel: BM x BN x 64 tiles (256 x 256 with 8 wavefronts for large M).  Per k-tile the raw
-//      quantized bytes of BN weight rows are loaded (Q4_K: 32 quant bytes + the super-block header per
-//      row, Q8_0 / MXFP4: two blocks per row through a range-checked buffer resource), dequantized
-//      ONCE to fp16 with packed-fp16 VALU and written to LDS next to the activation tile; the
-//      wavefronts then run v_mfma_f32_32x32x16_f16 out of LDS with fp32 accumulation.  LDS is
-//      double-buffered, the global loads run two tiles ahead, and the tile order is XCD-aware.
+//   2. gemm_kernel: BM x 256 x 64 tiles, eight wavefronts, each owning 32 output columns.  The fp16
+//      activation k-tiles and the RAW quantized bytes of 256 weight rows (one 144-byte window per row
+//      covering four k-tiles of Q4_K / MXFP4 or two of Q8_0) are copied from global memory straight
+//      into LDS (buffer_load ... lds, range-checked), double-buffered.  Every lane unpacks its own
+//      MFMA B operands from those raw bytes into registers with packed-fp16 VALU, one k-tile ahead
+//      and in the shadow of the matrix pipe, so a weight is unpacked exactly once per tile and
+//      dequantized weights never pass through LDS; A operands come from LDS one MFMA ahead.
+//      v_mfma_f32_32x32x16_f16, fp32 accumulation, XCD-aware tile order, one barrier per k-tile.
 //   3. epilogue: fp32 accumulators times the row scale -> C (optionally scattered through a row
 //      index).
 //
@@ -70,21 +72,27 @@ __device__ __forceinline__ uint32_t pack2(float a, float b)
 }
 __device__ __forceinline__ uint32_t splat(float a) { return pack2(a, a); }
 
-// position inside a k-tile at which activation k (0..63) is stored, per weight format
+// Position inside a k-tile at which activation k (0..63) is stored, per weight format.  MFMA k-step ks
+// (0..3) takes positions [16 ks, 16 ks + 16): the first eight from the lanes with k-half h = 0, the
+// next eight from h = 1, and element e of those eight pairs with element e of the lane's B operand,
+// i.e. half (e & 1) of dword (4 ks + e / 2) in the order in which dequant() unpacks the raw bytes.
 template <int TYPE>
 __device__ __forceinline__ int k_slot(int k)
 {
     if (TYPE == kTypeQ4_K) {
-        // quant dword -> (e0,e2),(e1,e3): order [0,2,1,3] inside every 4
-        const int q = k & 3;
-        return (k & ~3) | ((q & 1) << 1) | (q >> 1);
+        // sub-block k/32; quant byte c of the lane's 16-byte chunk; dword c/4 unpacks as (b0,b2),(b1,b3)
+        const int sub = k >> 5, hh = (k >> 4) & 1, c = k & 15, b = c & 3;
+        const int idx = sub * 8 + 2 * (c >> 2) + (b & 1);
+        return (idx >> 2) * 16 + hh * 8 + 2 * (idx & 3) + (b >> 1);
     }
     if (TYPE == kTypeMXFP4) {
-        // quant byte j -> (e_j, e_{j+16}) inside every 32
-        const int j = k & 15, hi = (k >> 4) & 1;
-        return (k & ~31) | (j << 1) | hi;
+        // block k/32; quant byte i = k%16 holds elements i (low nibble) and i + 16 (high nibble)
+        const int hh = k >> 5, i = k & 15, hi = (k >> 4) & 1;
+        return (i >> 2) * 16 + hh * 8 + 2 * (i & 3) + hi;
     }
-    return k;
+    // Q8_0: block k/32, natural order
+    const int hh = k >> 5, tt = k & 31;
+    return (tt >> 3) * 16 + hh * 8 + (tt & 7);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -121,73 +129,64 @@ __global__ void __launch_bounds__(256) convert_x_kernel(const float* __restrict_
 }
 
 // ------------------------------------------------------------------------------------------
-// weight tile loaders: ITEMS work items per row and k-tile, each yielding 32 fp16 for LDS
+// weight formats: a "super-tile" is kSup consecutive k-tiles of one weight row, kept RAW in LDS as a
+// 144-byte window (nine 16-byte chunks copied from a 4-byte aligned address at or just below the
+// first block).  `delta` (0..3) is the distance from the window start to that first block.
+//   fetch():   the raw dwords one lane needs for its (row, k-half) of k-tile j of the super-tile
+//   dequant(): those dwords -> 16 packed fp16 pairs, o[4 ks .. 4 ks + 3] being the lane's B operand
+//              of MFMA k-step ks
 // ------------------------------------------------------------------------------------------
-struct WTensor {
-    __amdgpu_buffer_rsrc_t rs;   // range-checked view of the weight bytes
-    uint32_t base_delta;         // (weight address) & 3
-    uint32_t row_bytes;
-    int K;
-};
+constexpr int kRawRow = 144;
 
-// Q4_K: item (row, h) = quant bytes [16h, 16h+16) of the k-tile's 64-group
 struct GQ4K {
     static constexpr int kRegs = 8;
-    static constexpr bool kWholeTile = true;    // K is a multiple of 256: every k-tile is complete
-    static __device__ __forceinline__ void load(const WTensor& W, uint32_t row_off, int kt, int h, uint32_t (&r)[kRegs])
+    static constexpr int kSup = 4;            // one 256-element super-block
+    static constexpr int kSupBytes = 144;
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t /*delta*/, uint32_t (&r)[kRegs])
     {
-        const uint32_t blk = row_off + (uint32_t)(kt >> 2) * 144u;
-        const uint4_t hdr = __builtin_amdgcn_raw_buffer_load_b128(W.rs, (int)blk, 0, 0);
-        const uint4_t q = __builtin_amdgcn_raw_buffer_load_b128(W.rs, (int)(blk + 16u + (uint32_t)(kt & 3) * 32u + (uint32_t)h * 16u), 0, 0);
+        const uint4_t hdr = *reinterpret_cast<const uint4_t*>(rp);
+        const uint4_t q = *reinterpret_cast<const uint4_t*>(rp + 16 + j * 32 + h * 16);
         r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
         r[4] = q.x; r[5] = q.y; r[6] = q.z; r[7] = q.w;
     }
-    // writes k' [16h, 16h+16) (low nibbles) and [32+16h, ...) (high nibbles) of LDS row `dst`
-    static __device__ __forceinline__ void store(const uint32_t (&r)[kRegs], uint32_t /*row_off*/, int kt, int h, bool live, _Float16* dst)
+    // o[0..7]: low nibbles (sub-block 2j, elements 16h..16h+15), o[8..15]: high nibbles (sub-block 2j+1)
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int /*h*/, uint32_t /*delta*/, bool /*live*/,
+                                                   uint32_t (&o)[16])
     {
-        const int g4 = kt & 3;
-        const int sh = (g4 & 1) * 16;
+        const int sh = (j & 1) * 16;
         const uint32_t a = r[1] >> sh, b = r[2] >> sh, c = r[3] >> sh;
         const uint32_t sc_lo = a & 0x3f3fu, m_lo = b & 0x3f3fu;
         const uint32_t sc_hi = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
         const uint32_t m_hi = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
-        const uint32_t sc = (g4 & 2) ? sc_hi : sc_lo, mn = (g4 & 2) ? m_hi : m_lo;
+        const uint32_t sc = (j & 2) ? sc_hi : sc_lo, mn = (j & 2) ? m_hi : m_lo;
         H2U dm;
         dm.u = r[0];
-        const float d = live ? (float)dm.h.x : 0.f, dmin = live ? (float)dm.h.y : 0.f;
+        const float d = (float)dm.h.x, dmin = (float)dm.h.y;
         const uint32_t s1 = splat(d * (float)(sc & 0xffu)), o1 = splat(-(dmin * (float)(mn & 0xffu)));
         const uint32_t s2 = splat(d * (float)(sc >> 8) * 0.0625f), o2 = splat(-(dmin * (float)(mn >> 8)));
         const uint32_t magic = 0x64006400u, neg1024 = 0xe400e400u;   // 1024.0, -1024.0
-        uint32_t lo[8], hi[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t q = r[4 + j], q8 = q >> 8;
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t q = r[4 + i], q8 = q >> 8;
             // 0x6400 | nibble = 1024 + q (low) or 1024 + 16 q (high): exact after subtracting 1024
-            lo[2 * j] = pk_fma(pk_add((q & 0x000f000fu) | magic, neg1024), s1, o1);
-            lo[2 * j + 1] = pk_fma(pk_add((q8 & 0x000f000fu) | magic, neg1024), s1, o1);
-            hi[2 * j] = pk_fma(pk_add((q & 0x00f000f0u) | magic, neg1024), s2, o2);
-            hi[2 * j + 1] = pk_fma(pk_add((q8 & 0x00f000f0u) | magic, neg1024), s2, o2);
+            o[2 * i] = pk_fma(pk_add((q & 0x000f000fu) | magic, neg1024), s1, o1);
+            o[2 * i + 1] = pk_fma(pk_add((q8 & 0x000f000fu) | magic, neg1024), s1, o1);
+            o[8 + 2 * i] = pk_fma(pk_add((q & 0x00f000f0u) | magic, neg1024), s2, o2);
+            o[8 + 2 * i + 1] = pk_fma(pk_add((q8 & 0x00f000f0u) | magic, neg1024), s2, o2);
         }
-        uint4* p = reinterpret_cast<uint4*>(dst + 16 * h);
-        p[0] = uint4{lo[0], lo[1], lo[2], lo[3]};
-        p[1] = uint4{lo[4], lo[5], lo[6], lo[7]};
-        p[4] = uint4{hi[0], hi[1], hi[2], hi[3]};
-        p[5] = uint4{hi[4], hi[5], hi[6], hi[7]};
     }
 };
 
-// MXFP4: item (row, b) = block b (0/1) of the k-tile, 17 bytes inside a 20-byte aligned window
 struct GMXFP4 {
     static constexpr int kRegs = 5;
-    static constexpr bool kWholeTile = false;   // K % 64 may be 32: the last tile's second block is absent
-    static __device__ __forceinline__ void load(const WTensor& W, uint32_t row_off, int kt, int b, uint32_t (&r)[kRegs])
+    static constexpr int kSup = 4;            // eight 17-byte blocks
+    static constexpr int kSupBytes = 136;
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t delta, uint32_t (&r)[kRegs])
     {
-        const int blk = kt * 2 + b;
-        const uint32_t p = row_off + (uint32_t)blk * 17u;
-        const uint32_t al = (blk * 32 < W.K) ? (p & ~3u) : kDeadOffset;
-        const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(W.rs, (int)al, 0, 0);
-        r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
-        r[4] = __builtin_amdgcn_raw_buffer_load_b32(W.rs, (int)(al + 16u), 0, 0);
+        const uint32_t off = delta + (uint32_t)(2 * j + h) * 17u;
+        const uint32_t* p = reinterpret_cast<const uint32_t*>(rp + (off & ~3u));
+#pragma unroll
+        for (int i = 0; i < kRegs; ++i) r[i] = p[i];
     }
     template <int SEL>
     static __device__ __forceinline__ uint32_t cvt(uint32_t q, float scale)
@@ -196,48 +195,46 @@ struct GMXFP4 {
         c.h = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, scale, SEL);
         return c.u;
     }
-    static __device__ __forceinline__ void store(const uint32_t (&r)[kRegs], uint32_t row_off, int kt, int b, bool live, _Float16* dst)
+    // quant byte i of the block -> (element i, element i + 16); o[4 w + s] holds byte 4 w + s
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int h, uint32_t delta, bool live, uint32_t (&o)[16])
     {
-        const uint32_t o = (row_off + (uint32_t)(kt * 2 + b) * 17u) & 3u;
-        const uint32_t e = (r[0] >> (8 * o)) & 0xffu;
-        const bool wrap = o == 3;
+        const uint32_t sft = (delta + (uint32_t)(2 * j + h) * 17u) & 3u;
+        const uint32_t e = (r[0] >> (8 * sft)) & 0xffu;
+        const bool wrap = sft == 3;
         const uint32_t b0 = wrap ? r[1] : r[0], b1 = wrap ? r[2] : r[1], b2 = wrap ? r[3] : r[2];
         const uint32_t b3 = wrap ? r[4] : r[3], b4 = r[4];
-        const uint32_t shb = (o + 1) & 3;
-        const uint32_t q0 = __builtin_amdgcn_alignbyte(b1, b0, shb), q1 = __builtin_amdgcn_alignbyte(b2, b1, shb);
-        const uint32_t q2 = __builtin_amdgcn_alignbyte(b3, b2, shb), q3 = __builtin_amdgcn_alignbyte(b4, b3, shb);
-        // doubled E2M1 * 2^(e-128) = E2M1 * 2^(e-127); an absent block (K tail) stores zeros
+        const uint32_t shb = (sft + 1) & 3;
+        const uint32_t q[4] = {__builtin_amdgcn_alignbyte(b1, b0, shb), __builtin_amdgcn_alignbyte(b2, b1, shb),
+                               __builtin_amdgcn_alignbyte(b3, b2, shb), __builtin_amdgcn_alignbyte(b4, b3, shb)};
+        // doubled E2M1 * 2^(e-128) = E2M1 * 2^(e-127); a block past the end of K contributes zeros
         const float scale = live ? __uint_as_float(e == 0 ? 0x00400000u : (e << 23)) : 0.f;
-        uint4* p = reinterpret_cast<uint4*>(dst + 32 * b);
-        p[0] = uint4{cvt<0>(q0, scale), cvt<1>(q0, scale), cvt<2>(q0, scale), cvt<3>(q0, scale)};
-        p[1] = uint4{cvt<0>(q1, scale), cvt<1>(q1, scale), cvt<2>(q1, scale), cvt<3>(q1, scale)};
-        p[2] = uint4{cvt<0>(q2, scale), cvt<1>(q2, scale), cvt<2>(q2, scale), cvt<3>(q2, scale)};
-        p[3] = uint4{cvt<0>(q3, scale), cvt<1>(q3, scale), cvt<2>(q3, scale), cvt<3>(q3, scale)};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            o[4 * w] = cvt<0>(q[w], scale);
+            o[4 * w + 1] = cvt<1>(q[w], scale);
+            o[4 * w + 2] = cvt<2>(q[w], scale);
+            o[4 * w + 3] = cvt<3>(q[w], scale);
+        }
     }
 };
 
-// Q8_0: item (row, b) = block b (0/1) of the k-tile, 34 bytes inside a 36-byte aligned window
 struct GQ80 {
     static constexpr int kRegs = 9;
-    static constexpr bool kWholeTile = false;
-    static __device__ __forceinline__ void load(const WTensor& W, uint32_t row_off, int kt, int b, uint32_t (&r)[kRegs])
+    static constexpr int kSup = 2;            // four 34-byte blocks
+    static constexpr int kSupBytes = 136;
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t delta, uint32_t (&r)[kRegs])
     {
-        const int blk = kt * 2 + b;
-        const uint32_t p = row_off + (uint32_t)blk * 34u;
-        const uint32_t al = (blk * 32 < W.K) ? (p & ~3u) : kDeadOffset;
-        const uint4_t v0 = __builtin_amdgcn_raw_buffer_load_b128(W.rs, (int)al, 0, 0);
-        const uint4_t v1 = __builtin_amdgcn_raw_buffer_load_b128(W.rs, (int)(al + 16u), 0, 0);
-        r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
-        r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
-        r[8] = __builtin_amdgcn_raw_buffer_load_b32(W.rs, (int)(al + 32u), 0, 0);
+        const uint32_t off = delta + (uint32_t)(2 * j + h) * 34u;
+        const uint32_t* p = reinterpret_cast<const uint32_t*>(rp + (off & ~3u));
+#pragma unroll
+        for (int i = 0; i < kRegs; ++i) r[i] = p[i];
     }
-    static __device__ __forceinline__ void store(const uint32_t (&r)[kRegs], uint32_t row_off, int kt, int b, bool live, _Float16* dst)
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int h, uint32_t delta, bool live, uint32_t (&o)[16])
     {
-        const bool odd = ((row_off + (uint32_t)(kt * 2 + b) * 34u) & 2u) != 0;
+        const bool odd = ((delta + (uint32_t)(2 * j + h) * 34u) & 2u) != 0;
         const uint32_t dbits = odd ? (r[0] >> 16) : (r[0] & 0xffffu);
         const uint32_t d2 = live ? (dbits | (dbits << 16)) : 0u;      // fp16 d in both halves
         const uint32_t bias = 0xe480e480u;                              // -1152.0 = -(1024 + 128)
-        uint32_t o[16];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t q = (odd ? r[i + 1] : __builtin_amdgcn_alignbyte(r[i + 1], r[i], 2)) ^ 0x80808080u;
@@ -247,11 +244,6 @@ struct GQ80 {
             o[2 * i] = pk_mul(pk_add(p0, bias), d2);
             o[2 * i + 1] = pk_mul(pk_add(p1, bias), d2);
         }
-        uint4* p = reinterpret_cast<uint4*>(dst + 32 * b);
-        p[0] = uint4{o[0], o[1], o[2], o[3]};
-        p[1] = uint4{o[4], o[5], o[6], o[7]};
-        p[2] = uint4{o[8], o[9], o[10], o[11]};
-        p[3] = uint4{o[12], o[13], o[14], o[15]};
     }
 };
 
@@ -259,6 +251,7 @@ struct GemmArgs {
     const uint8_t* w;        // weight bytes (of expert 0 for grouped launches)
     int64_t w_bytes;         // bytes of one weight matrix (per expert for grouped launches)
     const _Float16* x16;     // [rows x Kp] converted activations
+    int64_t x16_bytes;
     const float* xscale;     // [rows]
     float* c;                // result
     int64_t ldc;
@@ -272,53 +265,40 @@ struct GemmArgs {
     int64_t expert_stride;   // bytes between experts
 };
 
-// One k-tile of MFMA work for a wavefront: TM x TN tiles of 32x32, four k-steps of 16.  The LDS
-// fragments of k-step s+1 are requested before the MFMAs of k-step s are issued, so the matrix
-// pipe covers the LDS latency.
-template <int TM, int TN>
-__device__ __forceinline__ void mma_tile(const _Float16* xs, const _Float16* ws, float16_t (&acc)[TM][TN])
+constexpr int kBN = 256;                     // weight rows (output columns) per tile: 32 per wavefront
+constexpr int kWaves = 8;
+constexpr int kRawTile = kBN * kRawRow;      // bytes of one raw super-tile in LDS
+constexpr int kRawInstrs = kRawTile / 1024;  // wavefront-wide 1 KiB copies per raw super-tile
+
+// LDS-direct copy: 64 lanes x 16 bytes land at lds + 16 * lane; out-of-range offsets deliver zeros
+__device__ __forceinline__ void copy16_to_lds(__amdgpu_buffer_rsrc_t rs, uint8_t* lds, uint32_t voffset, uint32_t soffset)
 {
-    half8_t a[2][TM], b[2][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) a[0][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kLdsRow);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) b[0][j] = *reinterpret_cast<const half8_t*>(ws + j * 32 * kLdsRow);
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-        const int c = ks & 1, n = c ^ 1;
-        if (ks + 1 < kBK / 16) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i) a[n][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kLdsRow + (ks + 1) * 16);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) b[n][j] = *reinterpret_cast<const half8_t*>(ws + j * 32 * kLdsRow + (ks + 1) * 16);
-        }
-        __builtin_amdgcn_sched_barrier(0);   // keep the requests above the MFMAs they are meant to overlap
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[c][i], b[c][j], acc[i][j], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-    }
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)lds, 16, (int)voffset, (int)soffset, 0, 0);
 }
 
-// BM x BN x 64 tiles, WM x WN wavefronts.  LDS holds two k-tiles (activations + dequantized weights);
-// per iteration every wavefront (a) dequantizes the raw bytes it fetched for tile kt+1 into the idle
-// buffer, (b) requests the raw bytes of tile kt+2, (c) multiplies tile kt.  Wavefronts that share a
-// SIMD run (a)(b) and (c) in opposite order so that the VALU dequantization of one overlaps the MFMA
-// phase of the other.  One barrier per k-tile.
-template <typename G, int BM, int BN, int WM, int WN>
-__global__ void __launch_bounds__(WM * WN * 64) gemm_kernel(const GemmArgs A)
+// BM x 256 x 64 tiles, eight wavefronts, each owning all BM rows of 32 output columns.
+//   * Activation k-tiles (fp16) and raw weight super-tiles go from global memory straight into LDS
+//     (buffer_load ... lds, range-checked: rows past M or N and the row padding arrive as zeros), one
+//     k-tile / one super-tile ahead of their use, both double-buffered.
+//   * A lane (column n, k-half h) unpacks ITS OWN B operands from the raw bytes into registers one
+//     k-tile ahead, so dequantized weights never travel through LDS and every weight is unpacked by
+//     exactly one lane of the workgroup.
+//   * A operands are read from LDS one MFMA ahead of their use.  One barrier per k-tile.
+template <typename G, int BM>
+__global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
 {
-    constexpr int NT = WM * WN * 64;
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int XCH = BM * 8 / NT;                 // 16-byte activation chunks per thread per k-tile
-    constexpr int WIT = BN * 2 / NT;                 // weight items per thread per k-tile
-    constexpr int kBufElems = (BM + BN) * kLdsRow;
-    static_assert(XCH >= 1 && WIT >= 1, "tile too small for the workgroup");
-    extern __shared__ _Float16 smem[];
+    constexpr int TM = BM / 32;
+    constexpr int kXTile = BM * kRawRow;                 // fp16 activation tile: 64 values + 8 padding per row = 144 B
+    constexpr int kXInstrs = kXTile / 1024;
+    constexpr int XI = (kXInstrs + kWaves - 1) / kWaves;
+    constexpr int WI = (kRawInstrs + kWaves - 1) / kWaves;
+    extern __shared__ uint8_t smem[];
+    uint8_t* const xbuf = smem;                          // 2 x kXTile
+    uint8_t* const rbuf = smem + 2 * kXTile;             // 2 x kRawTile
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, h = lane >> 5;
 
     // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs, so each XCD gets a contiguous
     // run of tiles; consecutive tiles share the activation rows (same m-tile), which then stay in that
@@ -343,132 +323,152 @@ __global__ void __launch_bounds__(WM * WN * 64) gemm_kernel(const GemmArgs A)
         m0 = mt * BM;
         m_rows = min(BM, A.M - m0);
     }
-    const int n0 = nt * BN;
+    const int n0 = nt * kBN;
 
-    WTensor W;
     const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
-    W.base_delta = (uint32_t)(wa & 3);
-    W.rs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0,
-                                             (int)(((uint32_t)A.w_bytes + W.base_delta + 3u) & ~3u), 0x00020000);
-    W.K = A.K;
-    W.row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const uint32_t base_delta = (uint32_t)(wa & 3);
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
 
-    // per-thread sources / destinations (constant over the k loop)
-    const _Float16* x_src[XCH];
-    int x_dst[XCH];
+    // per-lane source offsets of the LDS-direct copies (constant over the k loop)
+    uint32_t x_off[XI], w_off[WI];
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-        const int c = tid + i * NT;
-        const int row = c >> 3, chunk = c & 7;
-        x_src[i] = A.x16 + (int64_t)(m0 + min(row, m_rows - 1)) * A.Kp + chunk * 8;
-        x_dst[i] = row * kLdsRow + chunk * 8;
+    for (int i = 0; i < XI; ++i) {
+        const int c = (wave + kWaves * i) * 64 + lane;
+        const int row = c / 9, chunk = c - row * 9;
+        x_off[i] = (chunk < 8 && row < m_rows) ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
     }
-    uint32_t w_off[WIT];
-    int w_part[WIT], w_dst[WIT];
 #pragma unroll
-    for (int i = 0; i < WIT; ++i) {
-        const int it = tid + i * NT;
-        const int row = it >> 1;
-        w_part[i] = it & 1;
-        w_off[i] = W.base_delta + (uint32_t)min(n0 + row, A.N - 1) * W.row_bytes;
-        w_dst[i] = (BM + row) * kLdsRow;
+    for (int i = 0; i < WI; ++i) {
+        const int c = (wave + kWaves * i) * 64 + lane;
+        const int row = c / 9, chunk = c - row * 9;
+        w_off[i] = (n0 + row < A.N) ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u : kDeadOffset;
     }
+    // this lane's weight row for the matrix pipe
+    const int my_n = n0 + wave * 32 + col;
+    const uint32_t my_delta = my_n < A.N ? (base_delta + (uint32_t)my_n * row_bytes) & 3u : 0u;
+    const int my_raw = (wave * 32 + col) * kRawRow;
 
-    uint4_t xr[XCH];
-    uint32_t wr[WIT][G::kRegs];
-#define TSHIP_GEMM_LOAD(kt)                                                                        \
-    do {                                                                                           \
-        _Pragma("unroll") for (int i = 0; i < XCH; ++i) xr[i] = *reinterpret_cast<const uint4_t*>(x_src[i] + (kt) * kBK); \
-        _Pragma("unroll") for (int i = 0; i < WIT; ++i) G::load(W, w_off[i], (kt), w_part[i], wr[i]);  \
-    } while (0)
-#define TSHIP_GEMM_STORE(kt, buf)                                                                  \
-    do {                                                                                           \
-        _Float16* dstb = smem + (buf) * kBufElems;                                                 \
-        _Pragma("unroll") for (int i = 0; i < XCH; ++i) *reinterpret_cast<uint4_t*>(dstb + x_dst[i]) = xr[i]; \
-        _Pragma("unroll") for (int i = 0; i < WIT; ++i) {                                          \
-            const bool live = G::kWholeTile || ((kt) * 2 + w_part[i]) * 32 < A.K;                  \
-            G::store(wr[i], w_off[i], (kt), w_part[i], live, dstb + w_dst[i]);                     \
-        }                                                                                          \
-    } while (0)
+    auto issue_x = [&](int kt, int buf) {
+#pragma unroll
+        for (int i = 0; i < XI; ++i)
+            if (wave + kWaves * i < kXInstrs)
+                copy16_to_lds(xrs, xbuf + buf * kXTile + (wave + kWaves * i) * 1024, x_off[i], (uint32_t)kt * (kBK * 2));
+    };
+    auto issue_w = [&](int s, int buf) {
+#pragma unroll
+        for (int i = 0; i < WI; ++i)
+            if (wave + kWaves * i < kRawInstrs)
+                copy16_to_lds(wrs, rbuf + buf * kRawTile + (wave + kWaves * i) * 1024, w_off[i], (uint32_t)s * G::kSupBytes);
+    };
 
-    float16_t acc[TM][TN];
+    float16_t acc[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
     const int nkt = A.Kp / kBK;
-    const int frag = (lane & 31) * kLdsRow + (lane >> 5) * 8;
-    const int xs_off = wm * (BM / WM) * kLdsRow + frag;
-    const int ws_off = (BM + wn * (BN / WN)) * kLdsRow + frag;
-    // wavefronts w and w + 4 share a SIMD: one of them multiplies first, the other dequantizes first
-    const bool mma_first = (wave & 4) != 0 && NT > 256;
+    const int frag = col * kRawRow + h * 16;       // byte offset of this lane's A operand inside a 32-row block
 
-    TSHIP_GEMM_LOAD(0);
-    TSHIP_GEMM_STORE(0, 0);
-    if (nkt > 1) TSHIP_GEMM_LOAD(1);
+    issue_x(0, 0);
+    issue_w(0, 0);
     __syncthreads();
-    for (int kt = 0; kt < nkt; ++kt) {
-        const int cur = kt & 1;
-        const _Float16* bufc = smem + cur * kBufElems;
-        if (mma_first) mma_tile<TM, TN>(bufc + xs_off, bufc + ws_off, acc);
-        if (kt + 1 < nkt) TSHIP_GEMM_STORE(kt + 1, cur ^ 1);
-        // past the last tile the loads wrap to tile 0: harmless, and the loop body stays branch-free
-        TSHIP_GEMM_LOAD(kt + 2 < nkt ? kt + 2 : 0);
-        if (!mma_first) mma_tile<TM, TN>(bufc + xs_off, bufc + ws_off, acc);
-        __syncthreads();
+    uint32_t oc[16], on[16];
+    {
+        uint32_t r[G::kRegs];
+        G::fetch(rbuf + my_raw, 0, h, my_delta, r);
+        G::dequant(r, 0, h, my_delta, h * 32 < A.K, oc);
     }
-#undef TSHIP_GEMM_LOAD
-#undef TSHIP_GEMM_STORE
+    int s = 0, j = 0;                               // super-tile and k-tile inside it of `kt`
+    for (int kt = 0; kt < nkt; ++kt) {
+#ifndef TSHIP_GEMM_DEBUG_NOX
+        if (kt + 1 < nkt) issue_x(kt + 1, (kt + 1) & 1);
+#endif
+#ifndef TSHIP_GEMM_DEBUG_NOW
+        if (j == 0 && (s + 1) * G::kSup < nkt) issue_w(s + 1, (s + 1) & 1);
+#endif
+        int jn = j + 1, sn = s;
+        if (jn == G::kSup) { jn = 0; sn = s + 1; }
+        // raw bytes of this lane's operands for k-tile kt + 1 (past the last k-tile: stale LDS, result unused)
+        uint32_t r[G::kRegs];
+        G::fetch(rbuf + (sn & 1) * kRawTile + my_raw, jn, h, my_delta, r);
+        const uint8_t* xs = xbuf + (kt & 1) * kXTile + frag;
+        half8_t a[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kRawRow);
+        __builtin_amdgcn_sched_barrier(0);       // all LDS requests of the k-tile's first step go out before any use
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint4_t bb = {oc[4 * ks], oc[4 * ks + 1], oc[4 * ks + 2], oc[4 * ks + 3]};
+            const half8_t b = __builtin_bit_cast(half8_t, bb);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#ifndef TSHIP_GEMM_DEBUG_NOMMA
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b, acc[i], 0, 0, 0);
+#else
+                acc[i][0] += (float)a[i][0] * (float)b[0];
+#endif
+                if (ks + 1 < 4) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kRawRow + (ks + 1) * 32);
+                // matrix and LDS instructions keep this order (each operand is requested TM - 1 MFMAs
+                // before its use); vector and scalar ALU work may move across
+                __builtin_amdgcn_sched_barrier(0x6);
+            }
+            // unpack the next k-tile's operands in the shadow of the matrix pipe
+#ifndef TSHIP_GEMM_DEBUG_NODEQ
+            if (ks == 0) G::dequant(r, jn, h, my_delta, ((kt + 1) * 2 + h) * 32 < A.K, on);
+#else
+            if (ks == 0) { _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs]; }
+#endif
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oc[i] = on[i];
+        j = jn;
+        s = sn;
+    }
 
     // epilogue: D[row = 8*(r/4) + 4*(lane/32) + r%4][col = lane%32]
+    if (my_n < A.N) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int ml = wm * (BM / WM) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (ml < m_rows) {
-                const int m = m0 + ml;
-                const float s = A.xscale[m];
-                float* crow = A.c + (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const int n = n0 + wn * (BN / WN) + j * 32 + (lane & 31);
-                    if (n < A.N) crow[n] = acc[i][j][r] * s;
+            for (int r = 0; r < 16; ++r) {
+                const int ml = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (ml < m_rows) {
+                    const int m = m0 + ml;
+                    A.c[(int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc + my_n] = acc[i][r] * A.xscale[m];
                 }
             }
         }
     }
 }
 
-template <typename G, int BM, int BN, int WM, int WN>
+template <typename G, int BM>
 bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    auto kern = gemm_kernel<G, BM, BN, WM, WN>;
-    const size_t lds = (size_t)2 * (BM + BN) * kLdsRow * sizeof(_Float16);
+    auto kern = gemm_kernel<G, BM>;
+    const size_t lds = (size_t)2 * BM * kRawRow + 2 * kRawTile;
     if (lds > 64 * 1024 &&
         !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
                 "gemm: raising the dynamic LDS limit"))
         return false;
     a.m_tiles = m_tiles;
-    a.n_tiles = (a.N + BN - 1) / BN;
+    a.n_tiles = (a.N + kBN - 1) / kBN;
     const int total = a.m_tiles * a.n_tiles;
     const int grid = ((total + 7) / 8) * 8;          // whole rounds over the 8 XCDs
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), lds, stream, a);
     return hip_ok(hipGetLastError(), "gemm launch");
 }
 
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-#ifdef TSHIP_GEMM_VARIANT
-    if (bm == 256) return launch_tiles<G, TSHIP_GEMM_VARIANT>(a, m_tiles, stream);
-#endif
-    if (bm == 256) return launch_tiles<G, 256, 256, 4, 2>(a, m_tiles, stream);
-    if (bm == 128) return launch_tiles<G, 128, 256, 2, 4>(a, m_tiles, stream);
-    return launch_tiles<G, 64, 128, 1, 4>(a, m_tiles, stream);
+    if (bm == 256) return launch_tiles<G, 256>(a, m_tiles, stream);
+    if (bm == 128) return launch_tiles<G, 128>(a, m_tiles, stream);
+    return launch_tiles<G, 64>(a, m_tiles, stream);
 }
 
 }  // namespace
@@ -515,6 +515,11 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     a.N = N;
     a.K = K;
     a.Kp = (K + kBK - 1) / kBK * kBK;
+    a.x16_bytes = (int64_t)M * a.Kp * (int64_t)sizeof(_Float16);
+    if (a.x16_bytes >= ((int64_t)1 << 31)) {
+        set_last_error("gemm: the converted activations of one call must stay below 2 GiB; split the rows.");
+        return false;
+    }
     int bm, m_tiles;
     if (tiles) {
         a.tile_expert = tiles->expert;
