@@ -27,6 +27,28 @@ bool hip_ok(hipError_t e, const char* what)
     return false;
 }
 
+// Dynamic LDS above 64 KiB has to be allowed per kernel and device; the attribute call costs tens of
+// microseconds on the host, so the largest size granted so far is remembered.
+bool raise_lds_limit(const void* kern, size_t lds)
+{
+    if (lds <= 64 * 1024) return true;
+    struct Granted { const void* kern; int dev; size_t bytes; };
+    static std::mutex mu;
+    static std::vector<Granted> granted;
+    int dev = 0;
+    if (!hip_ok(hipGetDevice(&dev), "current device")) return false;
+    std::lock_guard<std::mutex> lock(mu);
+    Granted* slot = nullptr;
+    for (auto& g : granted)
+        if (g.kern == kern && g.dev == dev) slot = &g;
+    if (slot && slot->bytes >= lds) return true;
+    if (!hip_ok(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), "raising the dynamic LDS limit"))
+        return false;
+    if (slot) slot->bytes = lds;
+    else granted.push_back({kern, dev, lds});
+    return true;
+}
+
 // ---- backend state ----------------------------------------------------------------------------
 namespace {
 

@@ -5,7 +5,8 @@
 //      magnitude overflows or underflows fp16), written in the k-order in which the weight
 //      format unpacks (so the dequantizer never has to shuffle lanes), zero-padded to a
 //      multiple of the k-tile.  Optionally gathers rows through an index (MoE).
-//   2. gemm_kernel: BM x 256 x 64 tiles, eight wavefronts, each owning 32 output columns.  The fp16
+//   2. gemm_kernel (M > 64 per tile) / gemm_few_rows_kernel (M <= 64 per tile, persistent workgroups):
+//      BM x 256 x 64 tiles, eight wavefronts, each owning 32 output columns.  The fp16
 //      activation k-tiles and the RAW quantized bytes of 256 weight rows (one 144-byte window per row
 //      covering four k-tiles of Q4_K / MXFP4 or two of Q8_0) are copied from global memory straight
 //      into LDS (buffer_load ... lds, range-checked), double-buffered.  Every lane unpacks its own
@@ -268,7 +269,9 @@ struct GemmArgs {
 constexpr int kBN = 256;                     // weight rows (output columns) per tile: 32 per wavefront
 constexpr int kWaves = 8;
 constexpr int kRawTile = kBN * kRawRow;      // bytes of one raw super-tile in LDS
-constexpr int kRawInstrs = kRawTile / 1024;  // wavefront-wide 1 KiB copies per raw super-tile
+constexpr int kRawInstrs = kRawTile / 1024;  // wavefront-wide 1 KiB copies per raw super-tile (36)
+constexpr int kWI = (kRawInstrs + kWaves - 1) / kWaves;   // copies per wavefront, the surplus goes to a dump area
+constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
 
 // LDS-direct copy: 64 lanes x 16 bytes land at lds + 16 * lane; out-of-range offsets deliver zeros
 __device__ __forceinline__ void copy16_to_lds(__amdgpu_buffer_rsrc_t rs, uint8_t* lds, uint32_t voffset, uint32_t soffset)
@@ -276,25 +279,68 @@ __device__ __forceinline__ void copy16_to_lds(__amdgpu_buffer_rsrc_t rs, uint8_t
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)lds, 16, (int)voffset, (int)soffset, 0, 0);
 }
 
+// All but the N youngest LDS-direct copies of this wavefront have landed and its own LDS reads are done;
+// then the workgroup barrier.  (A __syncthreads() would wait for every copy in flight.)
+template <int N>
+__device__ __forceinline__ void wait_copies_and_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// Epilogue of one wavefront: D[row = 32 i + 8 (r / 4) + 4 h + r % 4][column my_n] times the row scale.
+// The scales (and scatter indices) of a 32-row block are loaded before its stores: the result may
+// alias them as far as the compiler knows, so a load placed after a store would wait for it.
+template <int TM>
+__device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&acc)[TM], int m0, int m_rows, int my_n, int h)
+{
+    if (my_n >= A.N) return;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        float sc[16];
+        int64_t off[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int ml = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int m = m0 + min(ml, m_rows - 1);
+            sc[r] = A.xscale[m];
+            off[r] = (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc + my_n;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int ml = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (ml < m_rows) A.c[off[r]] = acc[i][r] * sc[r];
+        }
+    }
+}
+
 // BM x 256 x 64 tiles, eight wavefronts, each owning all BM rows of 32 output columns.
 //   * Activation k-tiles (fp16) and raw weight super-tiles go from global memory straight into LDS
-//     (buffer_load ... lds, range-checked: rows past M or N and the row padding arrive as zeros), one
-//     k-tile / one super-tile ahead of their use, both double-buffered.
+//     (buffer_load ... lds, range-checked: rows past M or N arrive as zeros).  Activation rows are 128
+//     bytes in LDS with the 16-byte chunk index XORed with (row / 2) % 8, which keeps the ds_read_b128 of
+//     the A operands conflict-free without padding, so a k-tile is exactly BM / 8 copies.
+//   * Activations run XST - 1 k-tiles ahead in XST LDS stages, weight super-tiles RL super-tiles ahead in
+//     RL + 1 buffers.  Every wavefront issues the same number of copies per iteration (surplus copies use
+//     an out-of-range source and a dump area), so the wait before the barrier is a vmcnt that leaves the
+//     younger copies in flight: the few-row tiles (XST = 4), whose speed is the speed of streaming the
+//     weights, keep three k-tiles of requests outstanding.
 //   * A lane (column n, k-half h) unpacks ITS OWN B operands from the raw bytes into registers one
 //     k-tile ahead, so dequantized weights never travel through LDS and every weight is unpacked by
-//     exactly one lane of the workgroup.
-//   * A operands are read from LDS one MFMA ahead of their use.  One barrier per k-tile.
-template <typename G, int BM>
+//     exactly one lane of the workgroup.  One barrier per k-tile.
+template <typename G, int BM, int XST>
 __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
 {
     constexpr int TM = BM / 32;
-    constexpr int kXTile = BM * kRawRow;                 // fp16 activation tile: 64 values + 8 padding per row = 144 B
-    constexpr int kXInstrs = kXTile / 1024;
-    constexpr int XI = (kXInstrs + kWaves - 1) / kWaves;
-    constexpr int WI = (kRawInstrs + kWaves - 1) / kWaves;
+    constexpr int D = XST - 1;                           // k-tiles of activation lookahead
+    constexpr int RL = (D > 1 && G::kSup == 2) ? 2 : 1;  // weight lookahead in super-tiles
+    constexpr int RB = RL + 1;
+    constexpr int kXTile = BM * kXRow;
+    constexpr int XI = kXTile / 1024 / kWaves;           // activation copies per wavefront and k-tile
+    static_assert(XI >= 1 && XI * kWaves * 1024 == kXTile, "activation tile must split evenly over the wavefronts");
+    static_assert(D == 1 || D == 3, "lookahead of one or three k-tiles");
     extern __shared__ uint8_t smem[];
-    uint8_t* const xbuf = smem;                          // 2 x kXTile
-    uint8_t* const rbuf = smem + 2 * kXTile;             // 2 x kRawTile
+    uint8_t* const xbuf = smem;                          // XST x kXTile
+    uint8_t* const rbuf = smem + XST * kXTile;           // RB x kRawTile
+    uint8_t* const dump = rbuf + RB * kRawTile;          // 1 KiB
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -331,37 +377,53 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
         reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
     const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int nkt = A.Kp / kBK;
 
     // per-lane source offsets of the LDS-direct copies (constant over the k loop)
-    uint32_t x_off[XI], w_off[WI];
+    uint32_t x_off[XI], w_off[kWI];
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
-        const int c = (wave + kWaves * i) * 64 + lane;
-        const int row = c / 9, chunk = c - row * 9;
-        x_off[i] = (chunk < 8 && row < m_rows) ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+        const int q = (wave + kWaves * i) * 64 + lane;           // LDS chunk slot: row q / 8, position q % 8
+        const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
+        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
     }
 #pragma unroll
-    for (int i = 0; i < WI; ++i) {
+    for (int i = 0; i < kWI; ++i) {
         const int c = (wave + kWaves * i) * 64 + lane;
         const int row = c / 9, chunk = c - row * 9;
-        w_off[i] = (n0 + row < A.N) ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u : kDeadOffset;
+        w_off[i] = (row < kBN && n0 + row < A.N) ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
+                                                  : kDeadOffset;
     }
     // this lane's weight row for the matrix pipe
     const int my_n = n0 + wave * 32 + col;
     const uint32_t my_delta = my_n < A.N ? (base_delta + (uint32_t)my_n * row_bytes) & 3u : 0u;
     const int my_raw = (wave * 32 + col) * kRawRow;
 
-    auto issue_x = [&](int kt, int buf) {
+    // every call issues XI (activations) or kWI (weights) copies from every wavefront
+    auto issue_x = [&](int kt) {
+        uint8_t* stage = xbuf + (kt % XST) * kXTile;
+        const bool any = kt < nkt;
 #pragma unroll
-        for (int i = 0; i < XI; ++i)
-            if (wave + kWaves * i < kXInstrs)
-                copy16_to_lds(xrs, xbuf + buf * kXTile + (wave + kWaves * i) * 1024, x_off[i], (uint32_t)kt * (kBK * 2));
+        for (int i = 0; i < XI; ++i) {
+#ifdef TSHIP_GEMM_DEBUG_NOX
+            copy16_to_lds(xrs, stage + (wave + kWaves * i) * 1024, kDeadOffset, (uint32_t)kt * kXRow);
+#else
+            copy16_to_lds(xrs, stage + (wave + kWaves * i) * 1024, any ? x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
+#endif
+        }
     };
-    auto issue_w = [&](int s, int buf) {
+    auto issue_w = [&](int s) {
+        uint8_t* buf = rbuf + (s % RB) * kRawTile;
+        const bool any = s * G::kSup < nkt;
 #pragma unroll
-        for (int i = 0; i < WI; ++i)
-            if (wave + kWaves * i < kRawInstrs)
-                copy16_to_lds(wrs, rbuf + buf * kRawTile + (wave + kWaves * i) * 1024, w_off[i], (uint32_t)s * G::kSupBytes);
+        for (int i = 0; i < kWI; ++i) {
+            const int id = wave + kWaves * i;
+#ifdef TSHIP_GEMM_DEBUG_NOW
+            copy16_to_lds(wrs, id < kRawInstrs ? buf + id * 1024 : dump, kDeadOffset, (uint32_t)s * G::kSupBytes);
+#else
+            copy16_to_lds(wrs, id < kRawInstrs ? buf + id * 1024 : dump, any ? w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
+#endif
+        }
     };
 
     float16_t acc[TM];
@@ -370,11 +432,16 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
-    const int nkt = A.Kp / kBK;
-    const int frag = col * kRawRow + h * 16;       // byte offset of this lane's A operand inside a 32-row block
+    // A operand of k-step ks: chunk 2 ks + h of row (32 i + col), at its swizzled position
+    const int sw = (col >> 1) & 7;
+    int a_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) a_off[ks] = col * kXRow + ((2 * ks + h) ^ sw) * 16;
 
-    issue_x(0, 0);
-    issue_w(0, 0);
+#pragma unroll
+    for (int s = 0; s < RL; ++s) issue_w(s);
+#pragma unroll
+    for (int kt = 0; kt < D; ++kt) issue_x(kt);
     __syncthreads();
     uint32_t oc[16], on[16];
     {
@@ -383,78 +450,94 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
         G::dequant(r, 0, h, my_delta, h * 32 < A.K, oc);
     }
     int s = 0, j = 0;                               // super-tile and k-tile inside it of `kt`
+    int xst = 0, rb = 0;                            // LDS stage of k-tile kt, raw buffer of super-tile s
     for (int kt = 0; kt < nkt; ++kt) {
-#ifndef TSHIP_GEMM_DEBUG_NOX
-        if (kt + 1 < nkt) issue_x(kt + 1, (kt + 1) & 1);
-#endif
-#ifndef TSHIP_GEMM_DEBUG_NOW
-        if (j == 0 && (s + 1) * G::kSup < nkt) issue_w(s + 1, (s + 1) & 1);
-#endif
-        int jn = j + 1, sn = s;
-        if (jn == G::kSup) { jn = 0; sn = s + 1; }
+        if (j == 0) issue_w(s + RL);
+        issue_x(kt + D);
+        int jn = j + 1, sn = s, rbn = rb;
+        if (jn == G::kSup) { jn = 0; sn = s + 1; rbn = rb + 1 == RB ? 0 : rb + 1; }
         // raw bytes of this lane's operands for k-tile kt + 1 (past the last k-tile: stale LDS, result unused)
         uint32_t r[G::kRegs];
-        G::fetch(rbuf + (sn & 1) * kRawTile + my_raw, jn, h, my_delta, r);
-        const uint8_t* xs = xbuf + (kt & 1) * kXTile + frag;
-        half8_t a[TM];
+        G::fetch(rbuf + rbn * kRawTile + my_raw, jn, h, my_delta, r);
+        const uint8_t* xs = xbuf + xst * kXTile;
+        if constexpr (TM <= 2) {
+            // few rows: every A operand of the k-tile is requested up front
+            half8_t a[4][TM];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kRawRow);
-        __builtin_amdgcn_sched_barrier(0);       // all LDS requests of the k-tile's first step go out before any use
+            for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const uint4_t bb = {oc[4 * ks], oc[4 * ks + 1], oc[4 * ks + 2], oc[4 * ks + 3]};
-            const half8_t b = __builtin_bit_cast(half8_t, bb);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#ifndef TSHIP_GEMM_DEBUG_NOMMA
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b, acc[i], 0, 0, 0);
-#else
-                acc[i][0] += (float)a[i][0] * (float)b[0];
-#endif
-                if (ks + 1 < 4) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kRawRow + (ks + 1) * 32);
-                // matrix and LDS instructions keep this order (each operand is requested TM - 1 MFMAs
-                // before its use); vector and scalar ALU work may move across
-                __builtin_amdgcn_sched_barrier(0x6);
-            }
-            // unpack the next k-tile's operands in the shadow of the matrix pipe
+                for (int i = 0; i < TM; ++i) a[ks][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[ks]);
+            __builtin_amdgcn_sched_barrier(0);
 #ifndef TSHIP_GEMM_DEBUG_NODEQ
-            if (ks == 0) G::dequant(r, jn, h, my_delta, ((kt + 1) * 2 + h) * 32 < A.K, on);
+            G::dequant(r, jn, h, my_delta, ((kt + 1) * 2 + h) * 32 < A.K, on);
 #else
-            if (ks == 0) { _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs]; }
+            _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs];
 #endif
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const uint4_t bb = {oc[4 * ks], oc[4 * ks + 1], oc[4 * ks + 2], oc[4 * ks + 3]};
+                const half8_t b = __builtin_bit_cast(half8_t, bb);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#ifndef TSHIP_GEMM_DEBUG_NOMMA
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks][i], b, acc[i], 0, 0, 0);
+#else
+                    acc[i][0] += (float)a[ks][i][0] * (float)b[0];
+#endif
+            }
+        } else {
+            half8_t a[TM];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[0]);
+            __builtin_amdgcn_sched_barrier(0);       // all LDS requests of the k-tile's first step go out before any use
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const uint4_t bb = {oc[4 * ks], oc[4 * ks + 1], oc[4 * ks + 2], oc[4 * ks + 3]};
+                const half8_t b = __builtin_bit_cast(half8_t, bb);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+#ifndef TSHIP_GEMM_DEBUG_NOMMA
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b, acc[i], 0, 0, 0);
+#else
+                    acc[i][0] += (float)a[i][0] * (float)b[0];
+#endif
+                    if (ks + 1 < 4) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[(ks + 1) & 3]);
+                    // matrix and LDS instructions keep this order (each operand is requested TM - 1 MFMAs
+                    // before its use); vector and scalar ALU work may move across
+                    __builtin_amdgcn_sched_barrier(0x6);
+                }
+                // unpack the next k-tile's operands in the shadow of the matrix pipe
+#ifndef TSHIP_GEMM_DEBUG_NODEQ
+                if (ks == 0) G::dequant(r, jn, h, my_delta, ((kt + 1) * 2 + h) * 32 < A.K, on);
+#else
+                if (ks == 0) { _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs]; }
+#endif
+            }
         }
-        __syncthreads();
+        // Copies that may stay in flight: the activations requested in the last D - 1 iterations and a
+        // weight super-tile requested in one of them.
+        if constexpr (D == 1) wait_copies_and_barrier<0>();
+        else if constexpr (G::kSup == 2) wait_copies_and_barrier<2 * XI + kWI>();
+        else if (j < 2) wait_copies_and_barrier<2 * XI + kWI>();
+        else wait_copies_and_barrier<2 * XI>();
 #pragma unroll
         for (int i = 0; i < 16; ++i) oc[i] = on[i];
         j = jn;
         s = sn;
+        rb = rbn;
+        xst = xst + 1 == XST ? 0 : xst + 1;
     }
 
-    // epilogue: D[row = 8*(r/4) + 4*(lane/32) + r%4][col = lane%32]
-    if (my_n < A.N) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ml = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (ml < m_rows) {
-                    const int m = m0 + ml;
-                    A.c[(int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc + my_n] = acc[i][r] * A.xscale[m];
-                }
-            }
-        }
-    }
+    store_tile<TM>(A, acc, m0, m_rows, my_n, h);
 }
 
-template <typename G, int BM>
+template <typename G, int BM, int XST>
 bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    auto kern = gemm_kernel<G, BM>;
-    const size_t lds = (size_t)2 * BM * kRawRow + 2 * kRawTile;
-    if (lds > 64 * 1024 &&
-        !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                "gemm: raising the dynamic LDS limit"))
-        return false;
+    auto kern = gemm_kernel<G, BM, XST>;
+    constexpr int RB = (XST > 2 && G::kSup == 2) ? 3 : 2;
+    const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * kRawTile + 1024;
+    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
     a.n_tiles = (a.N + kBN - 1) / kBN;
     const int total = a.m_tiles * a.n_tiles;
@@ -463,12 +546,206 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
     return hip_ok(hipGetLastError(), "gemm launch");
 }
 
+// ------------------------------------------------------------------------------------------
+// Few activation rows (at most 64 per tile: small batches, MoE experts).  The weights are read once, so
+// the speed limit is streaming them and what counts is bytes in flight.  Same 64-row x 256-column tile
+// and operand scheme as above, but one iteration covers TWO k-tiles, the activations live in a ring of
+// three such pairs (requested two iterations ahead) and the raw weight super-tiles in three buffers
+// (requested two super-tiles ahead).  Per iteration a wavefront issues its LDS-direct copies after its
+// LDS reads and leaves this iteration's copies in flight at the barrier (counted vmcnt).
+// ------------------------------------------------------------------------------------------
+// per-tile state of a persistent workgroup
+struct FewRowsTile {
+    int m0, m_rows, my_n;
+    uint32_t my_delta;
+    __amdgpu_buffer_rsrc_t wrs;
+    uint32_t x_off;
+    uint32_t w_off[kWI];
+};
+
+template <typename G>
+__global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmArgs A)
+{
+    constexpr int BM = 64, TM = 2, KS = G::kSup;
+    constexpr int kXTile = BM * kXRow;                   // one k-tile of activations: 8 KiB, one copy per wavefront
+    constexpr int kXPair = 2 * kXTile;
+    constexpr int HPS = KS / 2;                          // iterations (k-tile pairs) per weight super-tile: 2 or 1
+    extern __shared__ uint8_t smem[];
+    uint8_t* const xbuf = smem;                          // 3 x kXPair
+    uint8_t* const rbuf = smem + 3 * kXPair;             // 3 x kRawTile
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, h = lane >> 5;
+
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int nkt = A.Kp / kBK;
+    const int npair = (nkt + 1) / 2;
+    const int my_raw = (wave * 32 + col) * kRawRow;
+    // the 36 copies of a raw super-tile: wavefronts 0..3 issue five, 4..7 four
+    const bool five = wave + kWaves * (kWI - 1) < kRawInstrs;
+    const int sw = (col >> 1) & 7;
+    int a_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) a_off[ks] = col * kXRow + ((2 * ks + h) ^ sw) * 16;
+
+    // Persistent workgroups: the tiles of an XCD (a contiguous run, so that neighbours share the activation
+    // rows in that XCD's L2) are dealt round-robin to the workgroups that landed on it.
+    const int total = A.m_tiles * A.n_tiles;
+    const int per = (total + 7) >> 3;
+    const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
+    int slot = blockIdx.x >> 3;
+
+    // next tile with work at or after `slot` (grouped launches may list empty tiles); false when none is left
+    auto setup = [&](FewRowsTile& T) -> bool {
+        for (; slot < per; slot += stride) {
+            const int t = xcd * per + slot;
+            if (t >= total) return false;
+            const int mt = t / A.n_tiles, nt = t - mt * A.n_tiles;
+            const uint8_t* wbase = A.w;
+            if (A.tile_expert) {
+                T.m0 = A.tile_row0[mt];
+                T.m_rows = A.tile_rows[mt];
+                if (T.m_rows <= 0) continue;
+                wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+            } else {
+                T.m0 = mt * BM;
+                T.m_rows = min(BM, A.M - T.m0);
+            }
+            const int n0 = nt * kBN;
+            const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
+            const uint32_t base_delta = (uint32_t)(wa & 3);
+            T.wrs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0,
+                                                      (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
+            {
+                const int q = wave * 64 + lane;
+                const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
+                T.x_off = row < T.m_rows ? (uint32_t)(T.m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+            }
+#pragma unroll
+            for (int i = 0; i < kWI; ++i) {
+                const int c = (wave + kWaves * i) * 64 + lane;
+                const int row = c / 9, chunk = c - row * 9;
+                T.w_off[i] = (row < kBN && n0 + row < A.N)
+                                 ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
+                                 : kDeadOffset;
+            }
+            T.my_n = n0 + wave * 32 + col;
+            T.my_delta = T.my_n < A.N ? (base_delta + (uint32_t)T.my_n * row_bytes) & 3u : 0u;
+            slot += stride;
+            return true;
+        }
+        return false;
+    };
+    // always the same number of copies per wavefront (sources past the end are out of range: zeros)
+    auto issue_x = [&](const FewRowsTile& T, int p) {            // k-tile pair p -> ring slot p % 3
+        uint8_t* dst = xbuf + (p % 3) * kXPair + wave * 1024;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int kt = 2 * p + e;
+            copy16_to_lds(xrs, dst + e * kXTile, kt < nkt ? T.x_off : kDeadOffset, (uint32_t)kt * kXRow);
+        }
+    };
+    auto issue_w = [&](const FewRowsTile& T, int s) {            // super-tile s -> buffer s % 3
+        uint8_t* buf = rbuf + (s % 3) * kRawTile;
+        const bool any = s * KS < nkt;
+#pragma unroll
+        for (int i = 0; i < kWI; ++i) {
+            const int id = wave + kWaves * i;
+            if (id < kRawInstrs) copy16_to_lds(T.wrs, buf + id * 1024, any ? T.w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
+        }
+    };
+    auto issue_first = [&](const FewRowsTile& T) {
+        issue_x(T, 0);
+        issue_x(T, 1);
+        issue_w(T, 0);
+        issue_w(T, 1);
+    };
+
+    FewRowsTile T;
+    if (!setup(T)) return;
+    issue_first(T);
+    for (;;) {
+        __syncthreads();                   // the first two k-tile pairs and super-tiles of this tile have landed
+        float16_t acc[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+
+        for (int p = 0; p < npair; ++p) {
+            const int s = p / HPS, e0 = (p % HPS) * 2;           // super-tile and first k-tile inside it
+            const uint8_t* raw = rbuf + (s % 3) * kRawTile + my_raw;
+            const uint8_t* xs = xbuf + (p % 3) * kXPair;
+            uint32_t r[2][G::kRegs];
+            half8_t a[2][4][TM];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                G::fetch(raw, e0 + e, h, T.my_delta, r[e]);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        a[e][ks][i] = *reinterpret_cast<const half8_t*>(xs + e * kXTile + i * 32 * kXRow + a_off[ks]);
+            }
+            // Requests for two iterations / two super-tiles ahead, activations first (the wait below then
+            // never has to cover a weight super-tile younger than one iteration).
+            issue_x(T, p + 2);
+            if (HPS == 1 || (p & 1) == 0) issue_w(T, s + 2);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                uint32_t o[16];
+                G::dequant(r[e], e0 + e, h, T.my_delta, ((2 * p + e) * 2 + h) * 32 < A.K, o);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
+                    const half8_t b = __builtin_bit_cast(half8_t, bb);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[e][ks][i], b, acc[i], 0, 0, 0);
+                }
+            }
+            // in flight may stay: this iteration's two activation copies and the youngest weight super-tile
+            if (five) wait_copies_and_barrier<2 + kWI>();
+            else wait_copies_and_barrier<2 + kWI - 1>();
+        }
+
+        // The next tile's first requests go out before this tile's results are stored, so their latency
+        // is covered by the epilogue (every wavefront is past its last LDS read of this tile).
+        const int m0 = T.m0, m_rows = T.m_rows, my_n = T.my_n;
+        const bool more = setup(T);
+        if (more) issue_first(T);
+        store_tile<TM>(A, acc, m0, m_rows, my_n, h);
+        if (!more) break;
+    }
+}
+
+template <typename G>
+bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
+{
+    auto kern = gemm_few_rows_kernel<G>;
+    const size_t lds = (size_t)3 * 2 * 64 * kXRow + (size_t)3 * kRawTile;
+    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + kBN - 1) / kBN;
+    const int total = a.m_tiles * a.n_tiles;
+    // one persistent workgroup per CU (the LDS footprint allows no more), whole rounds over the 8 XCDs
+    const int grid = std::min(((total + 7) / 8) * 8, std::max(8, device_info().num_cus / 8 * 8));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), lds, stream, a);
+    return hip_ok(hipGetLastError(), "gemm launch");
+}
+
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-    if (bm == 256) return launch_tiles<G, 256>(a, m_tiles, stream);
-    if (bm == 128) return launch_tiles<G, 128>(a, m_tiles, stream);
-    return launch_tiles<G, 64>(a, m_tiles, stream);
+    if (bm == 256) return launch_tiles<G, 256, 2>(a, m_tiles, stream);
+    if (bm == 128) return launch_tiles<G, 128, G::kSup == 2 ? 2 : 4>(a, m_tiles, stream);
+#ifdef TSHIP_GEMM_NO_FEW_ROWS
+    return launch_tiles<G, 64, 4>(a, m_tiles, stream);
+#else
+    return launch_few_rows<G>(a, m_tiles, stream);
+#endif
 }
 
 }  // namespace

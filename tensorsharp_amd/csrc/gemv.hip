@@ -610,11 +610,7 @@ template <int TYPE>
 bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
     auto kern = gemv_kernel<TYPE>;
-    if (lds > 64 * 1024 &&
-        !hip_ok(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)lds),
-                "gemv: raising the dynamic LDS limit"))
-        return false;
+    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g);
     return hip_ok(hipGetLastError(), "gemv launch");
 }

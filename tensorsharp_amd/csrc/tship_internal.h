@@ -43,6 +43,7 @@ inline bool is_quant_type(int type) { return type == kTypeQ8_0 || type == kTypeQ
 void set_last_error(const std::string& msg);
 void clear_last_error();
 bool hip_ok(hipError_t e, const char* what);   // sets last error on failure
+bool raise_lds_limit(const void* kernel, size_t dynamic_lds_bytes);   // remembered per kernel and device
 
 struct DeviceInfo {
     int num_cus;
