@@ -94,3 +94,43 @@ def test_config3_q4_k_prefill(hip, oracle):
     e = check(y[rows], ref, "cfg3")
     print("cfg3 row-L2 err %.2e rms err %.2e" % e)
     assert np.all(np.isfinite(y))
+
+
+@pytest.mark.parametrize("name,M", [("q4_k", 40), ("mxfp4", 64), ("q8_0", 9)])
+def test_more_tiles_than_workgroups(hip, oracle, name, M):
+    # few rows x very many columns: the persistent workgroups each walk over several tiles
+    rng = np.random.default_rng(57 + M)
+    N, K = 256 * 300 + 77, 256
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, T[name], wq, N, K, x)
+    check(y, oracle.matmul_f64(T[name], wq, N, K, x), (name, M))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+def test_tall_activations(hip, oracle, name):
+    # M > 1024 takes the 256-row tiles; the last tile is ragged in both directions
+    rng = np.random.default_rng(59)
+    M, N, K = 1100, 300, 768
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, T[name], wq, N, K, x)
+    check(y, oracle.matmul_f64(T[name], wq, N, K, x), name)
+
+
+@pytest.mark.parametrize("name,row_bytes", [("mxfp4", 17 * 3), ("q8_0", 34 * 3)])
+@pytest.mark.parametrize("M", [8, 100])
+def test_weight_view_at_odd_address(hip, oracle, name, row_bytes, M):
+    # a sub-matrix that starts at row 1: its first byte is 1- or 2-byte aligned only
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(61 + M)
+    N, K = 301, 96
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    assert wq.size == N * row_bytes
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    dev = torch.from_numpy(wq).cuda()
+    sub = dev[row_bytes:]
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(sub, T[name], K, N - 1))
+    torch.cuda.synchronize()
+    check(y.cpu().numpy(), oracle.matmul_f64(T[name], wq[row_bytes:], N - 1, K, x), (name, M))
