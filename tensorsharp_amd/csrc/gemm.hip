@@ -326,21 +326,26 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
 //   * A lane (column n, k-half h) unpacks ITS OWN B operands from the raw bytes into registers one
 //     k-tile ahead, so dequantized weights never travel through LDS and every weight is unpacked by
 //     exactly one lane of the workgroup.  One barrier per k-tile.
-template <typename G, int BM, int XST>
-__global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
+template <typename G, int BM, int XST, int NW>
+__global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
 {
+    constexpr int BN = NW * 32;                          // output columns per tile
+    constexpr int RT = BN * kRawRow;                     // bytes of one raw super-tile in LDS
+    constexpr int RIN = RT / 1024;                       // wavefront-wide 1 KiB copies per raw super-tile
+    constexpr int WI = (RIN + NW - 1) / NW;              // per wavefront; the surplus goes to a dump area
+    static_assert(RIN * 1024 == RT, "raw tile must be whole KiB");
     constexpr int TM = BM / 32;
     constexpr int D = XST - 1;                           // k-tiles of activation lookahead
     constexpr int RL = (D > 1 && G::kSup == 2) ? 2 : 1;  // weight lookahead in super-tiles
     constexpr int RB = RL + 1;
     constexpr int kXTile = BM * kXRow;
-    constexpr int XI = kXTile / 1024 / kWaves;           // activation copies per wavefront and k-tile
-    static_assert(XI >= 1 && XI * kWaves * 1024 == kXTile, "activation tile must split evenly over the wavefronts");
+    constexpr int XI = kXTile / 1024 / NW;           // activation copies per wavefront and k-tile
+    static_assert(XI >= 1 && XI * NW * 1024 == kXTile, "activation tile must split evenly over the wavefronts");
     static_assert(D == 1 || D == 3, "lookahead of one or three k-tiles");
     extern __shared__ uint8_t smem[];
     uint8_t* const xbuf = smem;                          // XST x kXTile
-    uint8_t* const rbuf = smem + XST * kXTile;           // RB x kRawTile
-    uint8_t* const dump = rbuf + RB * kRawTile;          // 1 KiB
+    uint8_t* const rbuf = smem + XST * kXTile;           // RB x RT
+    uint8_t* const dump = rbuf + RB * RT;          // 1 KiB
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -369,7 +374,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
         m0 = mt * BM;
         m_rows = min(BM, A.M - m0);
     }
-    const int n0 = nt * kBN;
+    const int n0 = nt * BN;
 
     const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
     const uint32_t base_delta = (uint32_t)(wa & 3);
@@ -380,18 +385,18 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
     const int nkt = A.Kp / kBK;
 
     // per-lane source offsets of the LDS-direct copies (constant over the k loop)
-    uint32_t x_off[XI], w_off[kWI];
+    uint32_t x_off[XI], w_off[WI];
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
-        const int q = (wave + kWaves * i) * 64 + lane;           // LDS chunk slot: row q / 8, position q % 8
+        const int q = (wave + NW * i) * 64 + lane;           // LDS chunk slot: row q / 8, position q % 8
         const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
         x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
     }
 #pragma unroll
-    for (int i = 0; i < kWI; ++i) {
-        const int c = (wave + kWaves * i) * 64 + lane;
+    for (int i = 0; i < WI; ++i) {
+        const int c = (wave + NW * i) * 64 + lane;
         const int row = c / 9, chunk = c - row * 9;
-        w_off[i] = (row < kBN && n0 + row < A.N) ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
+        w_off[i] = (row < BN && n0 + row < A.N) ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
                                                   : kDeadOffset;
     }
     // this lane's weight row for the matrix pipe
@@ -399,29 +404,29 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
     const uint32_t my_delta = my_n < A.N ? (base_delta + (uint32_t)my_n * row_bytes) & 3u : 0u;
     const int my_raw = (wave * 32 + col) * kRawRow;
 
-    // every call issues XI (activations) or kWI (weights) copies from every wavefront
+    // every call issues XI (activations) or WI (weights) copies from every wavefront
     auto issue_x = [&](int kt) {
         uint8_t* stage = xbuf + (kt % XST) * kXTile;
         const bool any = kt < nkt;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
 #ifdef TSHIP_GEMM_DEBUG_NOX
-            copy16_to_lds(xrs, stage + (wave + kWaves * i) * 1024, kDeadOffset, (uint32_t)kt * kXRow);
+            copy16_to_lds(xrs, stage + (wave + NW * i) * 1024, kDeadOffset, (uint32_t)kt * kXRow);
 #else
-            copy16_to_lds(xrs, stage + (wave + kWaves * i) * 1024, any ? x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
+            copy16_to_lds(xrs, stage + (wave + NW * i) * 1024, any ? x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
 #endif
         }
     };
     auto issue_w = [&](int s) {
-        uint8_t* buf = rbuf + (s % RB) * kRawTile;
+        uint8_t* buf = rbuf + (s % RB) * RT;
         const bool any = s * G::kSup < nkt;
 #pragma unroll
-        for (int i = 0; i < kWI; ++i) {
-            const int id = wave + kWaves * i;
+        for (int i = 0; i < WI; ++i) {
+            const int id = wave + NW * i;
 #ifdef TSHIP_GEMM_DEBUG_NOW
-            copy16_to_lds(wrs, id < kRawInstrs ? buf + id * 1024 : dump, kDeadOffset, (uint32_t)s * G::kSupBytes);
+            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, kDeadOffset, (uint32_t)s * G::kSupBytes);
 #else
-            copy16_to_lds(wrs, id < kRawInstrs ? buf + id * 1024 : dump, any ? w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
+            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, any ? w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
 #endif
         }
     };
@@ -458,7 +463,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
         if (jn == G::kSup) { jn = 0; sn = s + 1; rbn = rb + 1 == RB ? 0 : rb + 1; }
         // raw bytes of this lane's operands for k-tile kt + 1 (past the last k-tile: stale LDS, result unused)
         uint32_t r[G::kRegs];
-        G::fetch(rbuf + rbn * kRawTile + my_raw, jn, h, my_delta, r);
+        G::fetch(rbuf + rbn * RT + my_raw, jn, h, my_delta, r);
         const uint8_t* xs = xbuf + xst * kXTile;
         if constexpr (TM <= 2) {
             // few rows: every A operand of the k-tile is requested up front
@@ -517,8 +522,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
         // Copies that may stay in flight: the activations requested in the last D - 1 iterations and a
         // weight super-tile requested in one of them.
         if constexpr (D == 1) wait_copies_and_barrier<0>();
-        else if constexpr (G::kSup == 2) wait_copies_and_barrier<2 * XI + kWI>();
-        else if (j < 2) wait_copies_and_barrier<2 * XI + kWI>();
+        else if constexpr (G::kSup == 2) wait_copies_and_barrier<2 * XI + WI>();
+        else if (j < 2) wait_copies_and_barrier<2 * XI + WI>();
         else wait_copies_and_barrier<2 * XI>();
 #pragma unroll
         for (int i = 0; i < 16; ++i) oc[i] = on[i];
@@ -531,18 +536,19 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_kernel(const GemmArgs A)
     store_tile<TM>(A, acc, m0, m_rows, my_n, h);
 }
 
-template <typename G, int BM, int XST>
+template <typename G, int BM, int XST, int NW>
 bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    auto kern = gemm_kernel<G, BM, XST>;
+    constexpr int BN = NW * 32, RT = BN * kRawRow;
+    auto kern = gemm_kernel<G, BM, XST, NW>;
     constexpr int RB = (XST > 2 && G::kSup == 2) ? 3 : 2;
-    const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * kRawTile + 1024;
+    const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * RT + 1024;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
-    a.n_tiles = (a.N + kBN - 1) / kBN;
+    a.n_tiles = (a.N + BN - 1) / BN;
     const int total = a.m_tiles * a.n_tiles;
     const int grid = ((total + 7) / 8) * 8;          // whole rounds over the 8 XCDs
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
     return hip_ok(hipGetLastError(), "gemm launch");
 }
 
@@ -739,10 +745,12 @@ bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-    if (bm == 256) return launch_tiles<G, 256, 2>(a, m_tiles, stream);
-    if (bm == 128) return launch_tiles<G, 128, G::kSup == 2 ? 2 : 4>(a, m_tiles, stream);
+    if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
+    // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
+    // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 the other way round
+    if (bm == 128) return G::kSup == 2 ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream) : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream);
 #ifdef TSHIP_GEMM_NO_FEW_ROWS
-    return launch_tiles<G, 64, 4>(a, m_tiles, stream);
+    return launch_tiles<G, 64, 4, 8>(a, m_tiles, stream);
 #else
     return launch_few_rows<G>(a, m_tiles, stream);
 #endif
