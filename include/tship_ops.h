@@ -127,6 +127,19 @@ TSHIP_EXPORT int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView
 
 /* ---- MoE (GPT-OSS expert stage), device pointers ------------------------------------------ */
 
+/* replaces TSGgml_GetRowsQuantF32 (ggml_ops_matmul.cpp:519-668, :1339-1368; GgmlNative.cs:324, :1003-1006; caller
+ * ModelBase.cs:826-856 embedding lookup): result[i, 0..ne0) = dequantized row indices[i] of the [ne1 x ne0] source
+ * (type F32 copies rows).  Host pointers; the source is cached on the device by pointer / preload key like the
+ * matmul weight.  result must be a standard view [num_indices x ne0]; indices I32 (or F32, truncated).  An index
+ * outside [0, ne1) is an error (the bridge's ggml_get_rows asserts). */
+TSHIP_EXPORT int TSHip_GetRowsQuantF32(TSHipTensorView2D result, void* src_data, int src_ggml_type, int64_t src_ne0,
+                                       int64_t src_ne1, int64_t src_raw_bytes, TSHipContiguousTensor indices);
+
+/* device-pointer form of the same: asynchronous on the selected stream; rows of out-of-range indices are zero. */
+TSHIP_EXPORT int TSHip_GetRowsQuantF32Device(TSHipTensorView2D result, const void* src_data, int src_ggml_type,
+                                             int64_t src_ne0, int64_t src_ne1, int64_t src_raw_bytes,
+                                             const int32_t* indices, int64_t num_indices);
+
 /* No bridge export: the reference routes in C# (GptOssModel.MoERoute, TensorSharp.Models/Models/GptOss/GptOssModel.cs:814-865,
  * the part after the router linear).  logits [T x E] -> ids / weights [T x k]: top-k by repeated argmax (first
  * maximum wins ties), softmax over the k selected logits.  1 <= k <= 16. */

@@ -748,4 +748,127 @@ int TSHip_SyncHostBuffer(void* ptr, size_t size)
     return 1;
 }
 
+/* ---- embedding gather ----------------------------------------------------------------- */
+
+int TSHip_GetRowsQuantF32Device(TSHipTensorView2D result, const void* src_data, int src_ggml_type, int64_t src_ne0,
+                                int64_t src_ne1, int64_t src_raw_bytes, const int32_t* indices, int64_t num_indices)
+{
+    return guarded(0, "get_rows_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_desc(result, "result")) return 0;
+        if (src_data == nullptr || src_ne0 <= 0 || src_ne1 <= 0 || src_raw_bytes <= 0) {
+            set_last_error("Invalid quantized weight descriptor for get_rows_quant.");
+            return 0;
+        }
+        if (indices == nullptr || num_indices <= 0) {
+            set_last_error("Invalid element count passed for indices.");
+            return 0;
+        }
+        if (result.dim0 != num_indices || result.dim1 != src_ne0) {
+            set_last_error("Shape mismatch in get_rows_quant: result must be [num_indices, ne0].");
+            return 0;
+        }
+        const size_t rs = row_size(src_ggml_type, src_ne0);
+        if ((src_ggml_type != kTypeF32 && !is_quant_type(src_ggml_type)) || rs == 0 || src_ne0 % 4 != 0) {
+            set_last_error("Unsupported source type or row length for get_rows_quant.");
+            return 0;
+        }
+        if ((size_t)src_raw_bytes < rs * (size_t)src_ne1) {
+            set_last_error("Quantized weight bytes are smaller than ne0 x ne1 for get_rows_quant.");
+            return 0;
+        }
+        if (result.stride1 != 1) {
+            set_last_error("result must be a standard (stride1 == 1) view in get_rows_quant.");
+            return 0;
+        }
+        if (!launch_get_rows(src_ggml_type, src_data, (int64_t)rs, src_ne1, indices, num_indices, src_ne0,
+                             static_cast<float*>(result.data), result.stride0, g_stream.load()))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_GetRowsQuantF32(TSHipTensorView2D result, void* src_data, int src_ggml_type, int64_t src_ne0, int64_t src_ne1,
+                          int64_t src_raw_bytes, TSHipContiguousTensor indices)
+{
+    return guarded(0, "get_rows_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_desc(result, "result")) return 0;
+        if (indices.data == nullptr) {
+            set_last_error("Null pointer passed for indices.");
+            return 0;
+        }
+        if (indices.element_count <= 0) {
+            set_last_error("Invalid element count passed for indices.");
+            return 0;
+        }
+        if (indices.element_type != 0 && indices.element_type != 3) {
+            set_last_error("Unsupported contiguous tensor element type passed for indices.");
+            return 0;
+        }
+        if (src_data == nullptr || src_ne0 <= 0 || src_ne1 <= 0 || src_raw_bytes <= 0) {
+            set_last_error("Invalid quantized weight descriptor for get_rows_quant.");
+            return 0;
+        }
+        const int64_t n = indices.element_count;
+        if (result.dim0 != n || result.dim1 != src_ne0) {
+            set_last_error("Shape mismatch in get_rows_quant: result must be [num_indices, ne0].");
+            return 0;
+        }
+        const size_t rs = row_size(src_ggml_type, src_ne0);
+        if ((src_ggml_type != kTypeF32 && !is_quant_type(src_ggml_type)) || rs == 0 || src_ne0 % 4 != 0) {
+            set_last_error("Unsupported source type or row length for get_rows_quant.");
+            return 0;
+        }
+        if ((size_t)src_raw_bytes < rs * (size_t)src_ne1) {
+            set_last_error("Quantized weight bytes are smaller than ne0 x ne1 for get_rows_quant.");
+            return 0;
+        }
+        if (!is_standard_view(result)) {
+            set_last_error("result must be a standard (stride1 == 1, non-overlapping) view in get_rows_quant.");
+            return 0;
+        }
+        // indices as int32 (F32 indices are truncated like the bridge's read_i32_values, ggml_ops_core.cpp:419-437)
+        std::vector<int32_t> ids((size_t)n);
+        if (indices.element_type == 3) {
+            std::memcpy(ids.data(), indices.data, (size_t)n * sizeof(int32_t));
+        } else {
+            const float* f = static_cast<const float*>(indices.data);
+            for (int64_t i = 0; i < n; ++i) ids[(size_t)i] = (int32_t)f[i];
+        }
+        for (int64_t i = 0; i < n; ++i)
+            if (ids[(size_t)i] < 0 || ids[(size_t)i] >= src_ne1) {
+                set_last_error("Index out of range in get_rows_quant.");
+                return 0;
+            }
+        const void* w_dev = resolve_weight(src_data, rs * (size_t)src_ne1);
+        if (!w_dev) return 0;
+
+        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        const size_t K = (size_t)src_ne0;
+        const size_t y_bytes = (size_t)n * K * sizeof(float);
+        const size_t id_bytes = ((size_t)n * sizeof(int32_t) + 255) & ~(size_t)255;
+        if (!ws_reserve(id_bytes + y_bytes, std::max(id_bytes, y_bytes))) return 0;
+        int32_t* ids_dev = static_cast<int32_t*>(g_ws.dev);
+        float* y_dev = reinterpret_cast<float*>(static_cast<char*>(g_ws.dev) + id_bytes);
+        hipStream_t stream = nullptr;
+        std::memcpy(g_ws.pinned, ids.data(), (size_t)n * sizeof(int32_t));
+        if (!hip_ok(hipMemcpyAsync(ids_dev, g_ws.pinned, (size_t)n * sizeof(int32_t), hipMemcpyHostToDevice, stream), "hipMemcpy(indices)")) return 0;
+        if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;       // the pinned block is reused below
+        for (int64_t i0 = 0; i0 < n; i0 += 65535) {
+            const int64_t cnt = std::min<int64_t>(65535, n - i0);
+            if (!launch_get_rows(src_ggml_type, w_dev, (int64_t)rs, src_ne1, ids_dev + i0, cnt, src_ne0, y_dev + (size_t)i0 * K, (int64_t)K, stream))
+                return 0;
+        }
+        if (!hip_ok(hipMemcpyAsync(g_ws.pinned, y_dev, y_bytes, hipMemcpyDeviceToHost, stream), "hipMemcpy(result)")) return 0;
+        if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+        float* dst = static_cast<float*>(result.data);
+        const float* stage = static_cast<const float*>(g_ws.pinned);
+        for (int64_t i = 0; i < n; ++i) std::memcpy(dst + (size_t)i * result.stride0, stage + (size_t)i * K, K * sizeof(float));
+        clear_last_error();
+        return 1;
+    });
+}
+
 }  // extern "C"

@@ -48,13 +48,9 @@ __device__ __forceinline__ float mxfp4_value(uint32_t nib)
     return (float)(int)(int8_t)((tab >> ((nib & 7u) * 8)) & 0xffu);
 }
 
-// one thread -> 4 consecutive outputs
-__global__ void __launch_bounds__(256) dequant_q8_0_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst,
-                                                           int64_t n4)
+// 4 consecutive outputs starting at element e0 (a multiple of 4) of the block sequence at src
+__device__ __forceinline__ float4 dequant4_q8_0(const uint8_t* src, int64_t e0)
 {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= n4) return;
-    const int64_t e0 = t * 4;
     const uint8_t* blk = src + (e0 >> 5) * 34;
     const int j = (int)(e0 & 31);
     const float d = half_bits_to_float((uint32_t)blk[0] | ((uint32_t)blk[1] << 8));
@@ -63,15 +59,11 @@ __global__ void __launch_bounds__(256) dequant_q8_0_kernel(const uint8_t* __rest
     o.y = (float)(int8_t)blk[3 + j] * d;
     o.z = (float)(int8_t)blk[4 + j] * d;
     o.w = (float)(int8_t)blk[5 + j] * d;
-    reinterpret_cast<float4*>(dst)[t] = o;
+    return o;
 }
 
-__global__ void __launch_bounds__(256) dequant_q4_K_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst,
-                                                           int64_t n4)
+__device__ __forceinline__ float4 dequant4_q4_K(const uint8_t* src, int64_t e0)
 {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= n4) return;
-    const int64_t e0 = t * 4;
     const uint8_t* blk = src + (e0 >> 8) * 144;
     const int r = (int)(e0 & 255);
     const int g = r >> 6;          // 64-group
@@ -98,15 +90,11 @@ __global__ void __launch_bounds__(256) dequant_q4_K_kernel(const uint8_t* __rest
     o.y = d1 * (float)((q[1] >> sh) & 0x0fu) - m1;
     o.z = d1 * (float)((q[2] >> sh) & 0x0fu) - m1;
     o.w = d1 * (float)((q[3] >> sh) & 0x0fu) - m1;
-    reinterpret_cast<float4*>(dst)[t] = o;
+    return o;
 }
 
-__global__ void __launch_bounds__(256) dequant_mxfp4_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst,
-                                                            int64_t n4)
+__device__ __forceinline__ float4 dequant4_mxfp4(const uint8_t* src, int64_t e0)
 {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= n4) return;
-    const int64_t e0 = t * 4;
     const uint8_t* blk = src + (e0 >> 5) * 17;
     const int j = (int)(e0 & 31);
     const int sh = (j >> 4) * 4;
@@ -117,7 +105,44 @@ __global__ void __launch_bounds__(256) dequant_mxfp4_kernel(const uint8_t* __res
     o.y = d * mxfp4_value((q[1] >> sh) & 0x0fu);
     o.z = d * mxfp4_value((q[2] >> sh) & 0x0fu);
     o.w = d * mxfp4_value((q[3] >> sh) & 0x0fu);
-    reinterpret_cast<float4*>(dst)[t] = o;
+    return o;
+}
+
+template <int TYPE>
+__device__ __forceinline__ float4 dequant4(const uint8_t* src, int64_t e0)
+{
+    if (TYPE == kTypeQ8_0) return dequant4_q8_0(src, e0);
+    if (TYPE == kTypeQ4_K) return dequant4_q4_K(src, e0);
+    if (TYPE == kTypeMXFP4) return dequant4_mxfp4(src, e0);
+    const float* f = reinterpret_cast<const float*>(src) + e0;      // F32 rows: plain copy
+    return float4{f[0], f[1], f[2], f[3]};
+}
+
+// one thread -> 4 consecutive outputs
+template <int TYPE>
+__global__ void __launch_bounds__(256) dequant_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst, int64_t n4)
+{
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n4) return;
+    reinterpret_cast<float4*>(dst)[t] = dequant4<TYPE>(src, t * 4);
+}
+
+// dst[i, :] = dequantized row ids[i] of the weight; rows with an index outside [0, ne1) become zeros
+template <int TYPE>
+__global__ void __launch_bounds__(256) get_rows_kernel(const uint8_t* __restrict__ src, int64_t row_bytes, int64_t ne1,
+                                                       const int32_t* __restrict__ ids, float* __restrict__ dst, int64_t ldd, int k4)
+{
+    const int t = (int)blockIdx.x * 256 + (int)threadIdx.x;
+    if (t >= k4) return;
+    const int64_t i = blockIdx.y;
+    const int64_t row = ids[i];
+    float4 o = float4{0.f, 0.f, 0.f, 0.f};
+    if (row >= 0 && row < ne1) o = dequant4<TYPE>(src + row * row_bytes, (int64_t)t * 4);
+    float* d = dst + i * ldd + (int64_t)t * 4;
+    d[0] = o.x;
+    d[1] = o.y;
+    d[2] = o.z;
+    d[3] = o.w;
 }
 
 }  // namespace
@@ -134,12 +159,35 @@ bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_
     const dim3 grid((unsigned)blocks), block(256);
     const uint8_t* s = static_cast<const uint8_t*>(src);
     switch (type) {
-    case kTypeQ8_0: hipLaunchKernelGGL(dequant_q8_0_kernel, grid, block, 0, stream, s, dst, n4); break;
-    case kTypeQ4_K: hipLaunchKernelGGL(dequant_q4_K_kernel, grid, block, 0, stream, s, dst, n4); break;
-    case kTypeMXFP4: hipLaunchKernelGGL(dequant_mxfp4_kernel, grid, block, 0, stream, s, dst, n4); break;
+    case kTypeQ8_0: hipLaunchKernelGGL(dequant_kernel<kTypeQ8_0>, grid, block, 0, stream, s, dst, n4); break;
+    case kTypeQ4_K: hipLaunchKernelGGL(dequant_kernel<kTypeQ4_K>, grid, block, 0, stream, s, dst, n4); break;
+    case kTypeMXFP4: hipLaunchKernelGGL(dequant_kernel<kTypeMXFP4>, grid, block, 0, stream, s, dst, n4); break;
     default: set_last_error("dequantize: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "dequantize launch");
+}
+
+// Embedding-style gather (ggml_get_rows on a quantized source, ggml_ops_matmul.cpp:519-668): n_ids rows of K
+// floats.  type kTypeF32 copies fp32 rows.
+bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, const int32_t* ids, int64_t n_ids, int64_t K,
+                     float* dst, int64_t ldd, hipStream_t stream)
+{
+    if (n_ids == 0 || K == 0) return true;
+    if (n_ids > 65535) {
+        set_last_error("get_rows: more than 65535 indices per call.");
+        return false;
+    }
+    const int k4 = (int)(K / 4);
+    const dim3 grid((unsigned)((k4 + 255) / 256), (unsigned)n_ids), block(256);
+    const uint8_t* s = static_cast<const uint8_t*>(src);
+    switch (type) {
+    case kTypeF32: hipLaunchKernelGGL(get_rows_kernel<kTypeF32>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
+    case kTypeQ8_0: hipLaunchKernelGGL(get_rows_kernel<kTypeQ8_0>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
+    case kTypeQ4_K: hipLaunchKernelGGL(get_rows_kernel<kTypeQ4_K>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
+    case kTypeMXFP4: hipLaunchKernelGGL(get_rows_kernel<kTypeMXFP4>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
+    default: set_last_error("get_rows: unsupported type."); return false;
+    }
+    return hip_ok(hipGetLastError(), "get_rows launch");
 }
 
 }  // namespace tship

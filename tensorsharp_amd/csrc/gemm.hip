@@ -284,7 +284,11 @@ __device__ __forceinline__ void copy16_to_lds(__amdgpu_buffer_rsrc_t rs, uint8_t
 template <int N>
 __device__ __forceinline__ void wait_copies_and_barrier()
 {
+#ifdef TSHIP_GEMM_DEBUG_NOBAR
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory");
+#else
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+#endif
 }
 
 // Epilogue of one wavefront: D[row = 32 i + 8 (r / 4) + 4 h + r % 4][column my_n] times the row scale.
@@ -561,24 +565,31 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 // LDS reads and leaves this iteration's copies in flight at the barrier (counted vmcnt).
 // ------------------------------------------------------------------------------------------
 // per-tile state of a persistent workgroup
+template <int NW>
 struct FewRowsTile {
     int m0, m_rows, my_n;
     uint32_t my_delta;
     __amdgpu_buffer_rsrc_t wrs;
-    uint32_t x_off;
-    uint32_t w_off[kWI];
+    uint32_t x_off[8 / NW];
+    uint32_t w_off[(NW * 32 * kRawRow / 1024 + NW - 1) / NW];
 };
 
-template <typename G>
-__global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmArgs A)
+// NW wavefronts (32 columns each), RING buffers for activations (in k-tile pairs) and for raw super-tiles:
+// 8 / 3 is one workgroup per CU with requests two iterations ahead, 4 / 2 two workgroups per CU with
+// requests one iteration ahead (the two workgroups drift apart, so one computes while the other waits).
+template <typename G, int NW, int RING>
+__global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A)
 {
     constexpr int BM = 64, TM = 2, KS = G::kSup;
+    constexpr int BN = NW * 32, RT = BN * kRawRow, RIN = RT / 1024, WI = (RIN + NW - 1) / NW, XI = 8 / NW;
+    static_assert(RIN * 1024 == RT && XI * NW == 8, "tile must split into whole copies");
+    static_assert(RING == 2 || RING == 3, "ring of two or three");
     constexpr int kXTile = BM * kXRow;                   // one k-tile of activations: 8 KiB, one copy per wavefront
     constexpr int kXPair = 2 * kXTile;
     constexpr int HPS = KS / 2;                          // iterations (k-tile pairs) per weight super-tile: 2 or 1
     extern __shared__ uint8_t smem[];
-    uint8_t* const xbuf = smem;                          // 3 x kXPair
-    uint8_t* const rbuf = smem + 3 * kXPair;             // 3 x kRawTile
+    uint8_t* const xbuf = smem;                          // RING x kXPair
+    uint8_t* const rbuf = smem + RING * kXPair;          // RING x RT
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -589,8 +600,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
     const int nkt = A.Kp / kBK;
     const int npair = (nkt + 1) / 2;
     const int my_raw = (wave * 32 + col) * kRawRow;
-    // the 36 copies of a raw super-tile: wavefronts 0..3 issue five, 4..7 four
-    const bool five = wave + kWaves * (kWI - 1) < kRawInstrs;
+    // the copies of a raw super-tile do not divide evenly: the first wavefronts issue WI, the others WI - 1
+    const bool five = wave + NW * (WI - 1) < RIN;
     const int sw = (col >> 1) & 7;
     int a_off[4];
 #pragma unroll
@@ -604,7 +615,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
     int slot = blockIdx.x >> 3;
 
     // next tile with work at or after `slot` (grouped launches may list empty tiles); false when none is left
-    auto setup = [&](FewRowsTile& T) -> bool {
+    auto setup = [&](FewRowsTile<NW>& T) -> bool {
         for (; slot < per; slot += stride) {
             const int t = xcd * per + slot;
             if (t >= total) return false;
@@ -619,21 +630,22 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
                 T.m0 = mt * BM;
                 T.m_rows = min(BM, A.M - T.m0);
             }
-            const int n0 = nt * kBN;
+            const int n0 = nt * BN;
             const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
             const uint32_t base_delta = (uint32_t)(wa & 3);
             T.wrs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0,
                                                       (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
-            {
-                const int q = wave * 64 + lane;
+#pragma unroll
+            for (int i = 0; i < XI; ++i) {
+                const int q = (wave + NW * i) * 64 + lane;
                 const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
-                T.x_off = row < T.m_rows ? (uint32_t)(T.m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+                T.x_off[i] = row < T.m_rows ? (uint32_t)(T.m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
             }
 #pragma unroll
-            for (int i = 0; i < kWI; ++i) {
-                const int c = (wave + kWaves * i) * 64 + lane;
+            for (int i = 0; i < WI; ++i) {
+                const int c = (wave + NW * i) * 64 + lane;
                 const int row = c / 9, chunk = c - row * 9;
-                T.w_off[i] = (row < kBN && n0 + row < A.N)
+                T.w_off[i] = (row < BN && n0 + row < A.N)
                                  ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
                                  : kDeadOffset;
             }
@@ -645,31 +657,33 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
         return false;
     };
     // always the same number of copies per wavefront (sources past the end are out of range: zeros)
-    auto issue_x = [&](const FewRowsTile& T, int p) {            // k-tile pair p -> ring slot p % 3
-        uint8_t* dst = xbuf + (p % 3) * kXPair + wave * 1024;
+    auto issue_x = [&](const FewRowsTile<NW>& T, int p) {            // k-tile pair p -> ring slot p % RING
+        uint8_t* dst = xbuf + (p % RING) * kXPair;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int kt = 2 * p + e;
-            copy16_to_lds(xrs, dst + e * kXTile, kt < nkt ? T.x_off : kDeadOffset, (uint32_t)kt * kXRow);
+#pragma unroll
+            for (int i = 0; i < XI; ++i)
+                copy16_to_lds(xrs, dst + e * kXTile + (wave + NW * i) * 1024, kt < nkt ? T.x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
         }
     };
-    auto issue_w = [&](const FewRowsTile& T, int s) {            // super-tile s -> buffer s % 3
-        uint8_t* buf = rbuf + (s % 3) * kRawTile;
+    auto issue_w = [&](const FewRowsTile<NW>& T, int s) {            // super-tile s -> buffer s % RING
+        uint8_t* buf = rbuf + (s % RING) * RT;
         const bool any = s * KS < nkt;
 #pragma unroll
-        for (int i = 0; i < kWI; ++i) {
-            const int id = wave + kWaves * i;
-            if (id < kRawInstrs) copy16_to_lds(T.wrs, buf + id * 1024, any ? T.w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
+        for (int i = 0; i < WI; ++i) {
+            const int id = wave + NW * i;
+            if (id < RIN) copy16_to_lds(T.wrs, buf + id * 1024, any ? T.w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
         }
     };
-    auto issue_first = [&](const FewRowsTile& T) {
-        issue_x(T, 0);
-        issue_x(T, 1);
-        issue_w(T, 0);
-        issue_w(T, 1);
+    auto issue_first = [&](const FewRowsTile<NW>& T) {
+#pragma unroll
+        for (int i = 0; i < RING - 1; ++i) issue_x(T, i);
+#pragma unroll
+        for (int i = 0; i < RING - 1; ++i) issue_w(T, i);
     };
 
-    FewRowsTile T;
+    FewRowsTile<NW> T;
     if (!setup(T)) return;
     issue_first(T);
     for (;;) {
@@ -682,8 +696,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
 
         for (int p = 0; p < npair; ++p) {
             const int s = p / HPS, e0 = (p % HPS) * 2;           // super-tile and first k-tile inside it
-            const uint8_t* raw = rbuf + (s % 3) * kRawTile + my_raw;
-            const uint8_t* xs = xbuf + (p % 3) * kXPair;
+            const uint8_t* raw = rbuf + (s % RING) * RT + my_raw;
+            const uint8_t* xs = xbuf + (p % RING) * kXPair;
             uint32_t r[2][G::kRegs];
             half8_t a[2][4][TM];
 #pragma unroll
@@ -695,10 +709,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
                     for (int i = 0; i < TM; ++i)
                         a[e][ks][i] = *reinterpret_cast<const half8_t*>(xs + e * kXTile + i * 32 * kXRow + a_off[ks]);
             }
-            // Requests for two iterations / two super-tiles ahead, activations first (the wait below then
-            // never has to cover a weight super-tile younger than one iteration).
-            issue_x(T, p + 2);
-            if (HPS == 1 || (p & 1) == 0) issue_w(T, s + 2);
+            // Requests RING - 1 iterations / super-tiles ahead, activations first (the counted wait below
+            // then never has to cover a weight super-tile younger than one iteration).
+            issue_x(T, p + RING - 1);
+            if (HPS == 1 || (p & 1) == 0) issue_w(T, s + RING - 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
@@ -712,9 +726,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
                     for (int i = 0; i < TM; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[e][ks][i], b, acc[i], 0, 0, 0);
                 }
             }
-            // in flight may stay: this iteration's two activation copies and the youngest weight super-tile
-            if (five) wait_copies_and_barrier<2 + kWI>();
-            else wait_copies_and_barrier<2 + kWI - 1>();
+            // RING 3: this iteration's activation copies and the youngest weight super-tile may stay in flight
+            if constexpr (RING == 2) wait_copies_and_barrier<0>();
+            else if (five) wait_copies_and_barrier<2 * XI + WI>();
+            else wait_copies_and_barrier<2 * XI + WI - 1>();
         }
 
         // The next tile's first requests go out before this tile's results are stored, so their latency
@@ -727,18 +742,20 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_few_rows_kernel(const GemmAr
     }
 }
 
-template <typename G>
+template <typename G, int NW, int RING>
 bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    auto kern = gemm_few_rows_kernel<G>;
-    const size_t lds = (size_t)3 * 2 * 64 * kXRow + (size_t)3 * kRawTile;
+    constexpr int BN = NW * 32, RT = BN * kRawRow;
+    auto kern = gemm_few_rows_kernel<G, NW, RING>;
+    const size_t lds = (size_t)RING * 2 * 64 * kXRow + (size_t)RING * RT;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
-    a.n_tiles = (a.N + kBN - 1) / kBN;
+    a.n_tiles = (a.N + BN - 1) / BN;
     const int total = a.m_tiles * a.n_tiles;
-    // one persistent workgroup per CU (the LDS footprint allows no more), whole rounds over the 8 XCDs
-    const int grid = std::min(((total + 7) / 8) * 8, std::max(8, device_info().num_cus / 8 * 8));
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), lds, stream, a);
+    // persistent workgroups, as many per CU as the LDS footprint allows, whole rounds over the 8 XCDs
+    const int per_cu = std::max(1, (int)((160 * 1024) / (lds + 512)));
+    const int grid = std::min(((total + 7) / 8) * 8, std::max(8, device_info().num_cus * per_cu / 8 * 8));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
     return hip_ok(hipGetLastError(), "gemm launch");
 }
 
@@ -752,7 +769,11 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 #ifdef TSHIP_GEMM_NO_FEW_ROWS
     return launch_tiles<G, 64, 4, 8>(a, m_tiles, stream);
 #else
-    return launch_few_rows<G>(a, m_tiles, stream);
+#ifdef TSHIP_GEMM_FEW_ROWS_ONE_WG
+    return launch_few_rows<G, 8, 3>(a, m_tiles, stream);
+#else
+    return launch_few_rows<G, 4, 2>(a, m_tiles, stream);
+#endif
 #endif
 }
 

@@ -55,6 +55,9 @@ const DeviceInfo& device_info();
 
 // dst[n] fp32 = dequant(src); bit-exact with the managed dequantizers.
 bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_t stream);
+// dst[i, 0..K) = row ids[i] of the weight (type F32 or quantized), rows of bad indices are zero-filled; n_ids <= 65535
+bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, const int32_t* ids, int64_t n_ids, int64_t K,
+                     float* dst, int64_t ldd, hipStream_t stream);
 
 // y[N] = W[N x K] * x[K]; W raw GGUF blocks, row-major; w_bytes = N * row_size.
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K,

@@ -110,6 +110,29 @@ class HipBasicOps:
             raise RuntimeError(f"Native HIP dequantization failed (code {rc}): {N.get_last_error()}")
         return dst
 
+    # -- embedding gather ------------------------------------------------------------------
+    @staticmethod
+    def GetRowsQuant(result, weight_data, ggml_type, ne0, ne1, raw_bytes, indices):
+        """result[i] = dequantized row indices[i] (GgmlBasicOps.cs:565-579). Host tensors; weight_data: address."""
+        if not isinstance(result, np.ndarray) or result.ndim != 2 or result.dtype != np.float32:
+            raise ValueError("GetRowsQuant requires a 2D Float32 result tensor.")
+        idx = np.asarray(indices)
+        if idx.dtype != np.int32 or not idx.flags["C_CONTIGUOUS"]:
+            raise NotImplementedError("HIP GetRowsQuant requires a standard-layout result and contiguous Int32 indices.")
+        rv = _host_view(result, standard=True)
+        desc = N.ContiguousTensor(idx.ctypes.data, int(idx.size), 3)
+        ok = N.lib().TSHip_GetRowsQuantF32(rv, C.c_void_p(weight_data), int(ggml_type), int(ne0), int(ne1),
+                                           int(raw_bytes), desc)
+        N.check_result(ok, "get_rows_quant")
+
+    @staticmethod
+    def GetRowsQuantDevice(result, weight, indices):
+        """Device form: result [n x K] fp32 CUDA tensor, weight a device QuantizedWeight, indices int32 CUDA tensor."""
+        rv = _device_view(result)
+        ok = N.lib().TSHip_GetRowsQuantF32Device(rv, C.c_void_p(weight.ptr), weight.ggml_type, weight.ne0, weight.ne1,
+                                                 weight.raw_bytes, C.c_void_p(indices.data_ptr()), int(indices.numel()))
+        N.check_result(ok, "get_rows_quant")
+
     # -- matmul ---------------------------------------------------------------------------
     @staticmethod
     def AddmmQuant(result, m1, weight_data, ggml_type, ne0, ne1, raw_bytes):

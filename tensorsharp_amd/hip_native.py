@@ -58,6 +58,10 @@ SIGNATURES = {
     "TSHip_AddmmQuantGroupF32Device": (C.c_int, [C.c_int, C.POINTER(TensorView2D), C.POINTER(TensorView2D),
                                                  C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int64),
                                                  C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "TSHip_GetRowsQuantF32": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                        ContiguousTensor]),
+    "TSHip_GetRowsQuantF32Device": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                              C.c_void_p, C.c_int64]),
     "TSHip_MoERouteF32Device": (C.c_int, [TensorView2D, C.c_int, C.c_void_p, C.c_void_p]),
     "TSHip_MoEExpertsForwardF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int64,
