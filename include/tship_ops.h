@@ -127,6 +127,44 @@ TSHIP_EXPORT int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView
 
 /* ---- MoE (GPT-OSS expert stage), device pointers ------------------------------------------ */
 
+/* ---- fused wrappers around the matmul ------------------------------------------------------ */
+
+/* replaces TSGgml_FusedRmsNormMatMulQuantF32 (ggml_ops_fused.cpp:21-217, :1380-1400; GgmlNative.cs:243-253, :903-912;
+ * caller Qwen35Model.cs:1492): result[M x ne1] = (RMSNorm(input, eps) * norm_weight) * W^T, RMSNorm as ggml_rms_norm
+ * (sum of squares in double, 1/sqrtf(mean + eps)).  Host pointers, weight cached like TSHip_AddmmQuantF32. */
+TSHIP_EXPORT int TSHip_FusedRmsNormMatMulQuantF32(TSHipTensorView2D result, TSHipTensorView2D input, void* norm_weight_data,
+                                                  int norm_weight_count, float eps, void* m2_data, int m2_ggml_type,
+                                                  int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes);
+
+/* replaces TSGgml_FusedMatMulQuantAddF32 (ggml_ops_fused.cpp:219-388, :1410-1430; GgmlNative.cs:256-263, :914-920; caller
+ * Qwen35Model.cs:1615): residual[M x ne1] += input * W^T, in place. */
+TSHIP_EXPORT int TSHip_FusedMatMulQuantAddF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* m2_data,
+                                              int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes);
+
+/* replaces TSGgml_FusedFFNSwiGLUQuantF32 (ggml_ops_fused.cpp:390-640, :1440-1480; GgmlNative.cs:266-283, :922-937; caller
+ * Qwen35Model.cs:1663): residual += W_down * ( silu(g) * u ), [g | u] = W_gate_up * (RMSNorm(input, eps) * norm_weight),
+ * g the first half_dim outputs, u the next half_dim; silu(g) = g / (1 + expf(-g)). */
+TSHIP_EXPORT int TSHip_FusedFFNSwiGLUQuantF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* norm_weight_data,
+                                              int norm_weight_count, float eps, void* gate_up_data, int gate_up_ggml_type,
+                                              int64_t gate_up_ne0, int64_t gate_up_ne1, int64_t gate_up_raw_bytes,
+                                              void* down_data, int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                              int64_t down_raw_bytes, int half_dim);
+
+/* device-pointer forms of the three (every pointer in device memory, asynchronous on the selected stream; they use the
+ * grow-only device workspace). */
+TSHIP_EXPORT int TSHip_FusedRmsNormMatMulQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D input,
+                                                        const float* norm_weight, int norm_weight_count, float eps,
+                                                        const void* m2_data, int m2_ggml_type, int64_t m2_ne0,
+                                                        int64_t m2_ne1, int64_t m2_raw_bytes);
+TSHIP_EXPORT int TSHip_FusedMatMulQuantAddF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, const void* m2_data,
+                                                    int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes);
+TSHIP_EXPORT int TSHip_FusedFFNSwiGLUQuantF32Device(TSHipTensorView2D residual, TSHipTensorView2D input,
+                                                    const float* norm_weight, int norm_weight_count, float eps,
+                                                    const void* gate_up_data, int gate_up_ggml_type, int64_t gate_up_ne0,
+                                                    int64_t gate_up_ne1, int64_t gate_up_raw_bytes, const void* down_data,
+                                                    int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                                    int64_t down_raw_bytes, int half_dim);
+
 /* replaces TSGgml_GetRowsQuantF32 (ggml_ops_matmul.cpp:519-668, :1339-1368; GgmlNative.cs:324, :1003-1006; caller
  * ModelBase.cs:826-856 embedding lookup): result[i, 0..ne0) = dequantized row indices[i] of the [ne1 x ne0] source
  * (type F32 copies rows).  Host pointers; the source is cached on the device by pointer / preload key like the

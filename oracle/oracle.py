@@ -80,6 +80,10 @@ class Oracle:
         L.tso_moe_route.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, _i32p, _f32p]
         L.tso_moe_group.restype = None
         L.tso_moe_group.argtypes = [_i32p, _f32p, C.c_int, C.c_int, C.c_int, _i32p, _i32p, _f32p]
+        L.tso_rms_norm_mul.restype = None
+        L.tso_rms_norm_mul.argtypes = [_f32p, C.c_int64, C.c_int64, C.c_int64, _f32p, C.c_float, _f32p]
+        L.tso_silu_mul.restype = None
+        L.tso_silu_mul.argtypes = [_f32p, C.c_int64, C.c_int64, _f32p]
         L.tso_swiglu_oai.restype = None
         L.tso_swiglu_oai.argtypes = [_f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
         L.tso_moe_forward.restype = C.c_int
@@ -160,6 +164,21 @@ class Oracle:
         self.lib.tso_moe_group(_ptr(ids, _i32p), _ptr(wts, _f32p), T, E, k, _ptr(offs, _i32p),
                                _ptr(tmap, _i32p), _ptr(wmap, _f32p))
         return offs, tmap, wmap
+
+    def rms_norm_mul(self, x, w, eps):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        rows, K = x.shape
+        out = np.empty((rows, K), dtype=np.float32)
+        self.lib.tso_rms_norm_mul(_ptr(x, _f32p), rows, K, K, _ptr(w, _f32p), eps, _ptr(out, _f32p))
+        return out
+
+    def silu_mul(self, gate_up):
+        gu = np.ascontiguousarray(gate_up, dtype=np.float32)
+        rows, two_f = gu.shape
+        out = np.empty((rows, two_f // 2), dtype=np.float32)
+        self.lib.tso_silu_mul(_ptr(gu, _f32p), rows, two_f // 2, _ptr(out, _f32p))
+        return out
 
     def swiglu_oai(self, gate_up, alpha=1.702, limit=7.0):
         gu = np.ascontiguousarray(gate_up, dtype=np.float32)

@@ -742,6 +742,35 @@ void tso_swiglu_oai(float* gate_up, int rows, int half_dim, float alpha, float l
     }
 }
 
+/* ---- fused wrappers of the bridge (ggml graphs of ggml_ops_fused.cpp:21-640) ------------------- */
+
+/* ggml_rms_norm followed by ggml_mul with the norm weight.
+ * Reference: ggml-cpu/ops.cpp:3646-3695 (ggml_compute_forward_rms_norm_f32: squares in fp32, summed in
+ * ggml_float = double in index order, mean = sum/ne00 and scale = 1.0f/sqrtf(mean + eps) in fp32,
+ * y = x * scale), then the graph's ggml_mul (ggml_ops_fused.cpp:161-162): (x * scale) * w. */
+void tso_rms_norm_mul(const float* x, int64_t rows, int64_t K, int64_t ldx, const float* w, float eps, float* out)
+{
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* xr = x + r * ldx;
+        double sum = 0.0;
+        for (int64_t i = 0; i < K; ++i) sum += (double)(xr[i] * xr[i]);
+        const float mean = (float)(sum / (double)K);
+        const float scale = 1.0f / sqrtf(mean + eps);
+        for (int64_t i = 0; i < K; ++i) out[r * K + i] = (xr[i] * scale) * w[i];
+    }
+}
+
+/* ggml_silu on the first half of each row times the second half.
+ * Reference: ggml-cpu/vec.h:958-960 (ggml_silu_f32 = x / (1 + expf(-x))), graph ggml_ops_fused.cpp:577-588. */
+void tso_silu_mul(const float* gate_up, int64_t rows, int64_t half_dim, float* out)
+{
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* g = gate_up + r * 2 * half_dim;
+        const float* u = g + half_dim;
+        for (int64_t i = 0; i < half_dim; ++i) out[r * half_dim + i] = (g[i] / (1.0f + expf(-g[i]))) * u[i];
+    }
+}
+
 static void linear_bias(int type, const void* w, const float* bias, int64_t N, int64_t K,
                         const float* x, int64_t M, float* out)
 {

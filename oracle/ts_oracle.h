@@ -66,6 +66,10 @@ int tso_moe_forward(int type, const void* gate_up_w, const float* gate_up_b,
                     int E, int H, int F, const float* hidden, int T, int k,
                     const int32_t* ids, const float* weights, float* out);
 
+/* fused wrappers: RMSNorm * weight, SiLU-gated product (ggml semantics) */
+void tso_rms_norm_mul(const float* x, int64_t rows, int64_t K, int64_t ldx, const float* w, float eps, float* out);
+void tso_silu_mul(const float* gate_up, int64_t rows, int64_t half_dim, float* out);
+
 int tso_max_threads(void);
 
 #ifdef __cplusplus

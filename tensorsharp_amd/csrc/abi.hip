@@ -259,28 +259,75 @@ bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
     return true;
 }
 
-// result/m1/w are device pointers here.
-bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
-                       int64_t N, hipStream_t stream)
+// bytes of device workspace one matmul needs (norm: RMSNorm prologue on the activations)
+size_t matmul_ws_bytes(int type, int M, int64_t K, bool norm)
+{
+    if (M <= 3 && K <= gemv_max_k(type)) return norm ? (((size_t)M * (size_t)K * sizeof(float) + 255) & ~(size_t)255) : 0;
+    return (gemm_workspace_bytes(M, (int)K) + 255) & ~(size_t)255;
+}
+
+// result (+)= f(m1) * W^T with f = identity or RMSNorm(eps) * norm_w.  All pointers are device pointers; `ws` has
+// matmul_ws_bytes() bytes.
+bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
+                          int64_t N, hipStream_t stream, void* ws, const float* norm_w, float eps, bool accumulate)
 {
     const size_t w_bytes = row_size(type, K) * (size_t)N;
     if (!check_device_operands(m1, w, type)) return false;
     const int M = m1.dim0;
     if (M <= 3 && K <= gemv_max_k(type)) {
         // decode / tiny batch: one bandwidth-bound GEMV per activation row
+        const float* xs = static_cast<const float*>(m1.data);
+        int64_t ldx = m1.stride0;
+        if (norm_w) {
+            if (!launch_rms_norm_rows(xs, ldx, norm_w, eps, M, (int)K, static_cast<float*>(ws), stream)) return false;
+            xs = static_cast<const float*>(ws);
+            ldx = K;
+        }
         for (int m = 0; m < M; ++m) {
-            const float* x = static_cast<const float*>(m1.data) + (int64_t)m * m1.stride0;
             float* y = static_cast<float*>(result.data) + (int64_t)m * result.stride0;
-            if (!launch_gemv(type, w, (int64_t)w_bytes, x, y, (int)N, (int)K, stream)) return false;
+            if (!launch_gemv(type, w, (int64_t)w_bytes, xs + (int64_t)m * ldx, y, (int)N, (int)K, stream, accumulate ? y : nullptr))
+                return false;
         }
         return true;
     }
     // prefill: activations -> fp16 workspace, then the MFMA GEMM
-    void* ws = dev_ws_reserve(gemm_workspace_bytes(M, (int)K));
-    if (!ws) return false;
-    if (!launch_convert_x(type, static_cast<const float*>(m1.data), m1.stride0, nullptr, M, (int)K, ws, stream)) return false;
+    if (!launch_convert_x(type, static_cast<const float*>(m1.data), m1.stride0, nullptr, M, (int)K, ws, stream, norm_w, eps)) return false;
     return launch_gemm(type, w, (int64_t)w_bytes, ws, static_cast<float*>(result.data), result.stride0, nullptr, M, (int)N,
-                       (int)K, nullptr, stream);
+                       (int)K, nullptr, stream, accumulate);
+}
+
+bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
+                       int64_t N, hipStream_t stream)
+{
+    const size_t need = matmul_ws_bytes(type, m1.dim0, K, false);
+    void* ws = nullptr;
+    if (need) {
+        ws = dev_ws_reserve(need);
+        if (!ws) return false;
+    }
+    return run_matmul_device_ws(result, m1, w, type, K, N, stream, ws, nullptr, 0.f, false);
+}
+
+// FFN of the fused entry points on device operands (ggml_ops_fused.cpp:390-640):
+//   residual += W_down * ( silu(g) * u ),  [g | u] = W_gate_up * (RMSNorm(input) * norm_w)
+bool run_ffn_swiglu_device(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const float* norm_w, float eps,
+                           const void* gate_up, int gu_type, const void* down, int dn_type, int hidden, int half,
+                           hipStream_t stream)
+{
+    const int M = input.dim0;
+    const size_t gu_bytes = ((size_t)M * 2 * half * sizeof(float) + 255) & ~(size_t)255;
+    const size_t act_bytes = ((size_t)M * half * sizeof(float) + 255) & ~(size_t)255;
+    const size_t ws1 = matmul_ws_bytes(gu_type, M, hidden, true), ws2 = matmul_ws_bytes(dn_type, M, half, false);
+    char* ws = static_cast<char*>(dev_ws_reserve(gu_bytes + act_bytes + std::max(ws1, ws2)));
+    if (!ws) return false;
+    float* gu = reinterpret_cast<float*>(ws);
+    float* act = reinterpret_cast<float*>(ws + gu_bytes);
+    void* mm_ws = ws + gu_bytes + act_bytes;
+    const TSHipTensorView2D gu_view{gu, M, 2 * half, 2 * half, 1, (int64_t)((size_t)M * 2 * half * sizeof(float))};
+    if (!run_matmul_device_ws(gu_view, input, gate_up, gu_type, hidden, 2 * half, stream, mm_ws, norm_w, eps, false)) return false;
+    if (!launch_silu_mul(gu, 2 * half, M, half, act, stream)) return false;
+    const TSHipTensorView2D act_view{act, M, half, half, 1, (int64_t)((size_t)M * half * sizeof(float))};
+    return run_matmul_device_ws(residual, act_view, down, dn_type, half, hidden, stream, mm_ws, nullptr, 0.f, true);
 }
 
 // device pointer for m2_data: preloaded key, cached host pointer, or upload now
@@ -377,6 +424,143 @@ static int guarded(int fallback, const char* what, F&& body)
         return fallback;
     }
 }
+
+// ---- helpers of the fused entry points ---------------------------------------------------------
+namespace {
+
+bool validate_weight(const void* data, int type, int64_t ne0, int64_t ne1, int64_t raw_bytes, const char* what)
+{
+    if (data == nullptr || ne0 <= 0 || ne1 <= 0 || raw_bytes <= 0) {
+        set_last_error(std::string("Invalid quantized weight descriptor for ") + what + ".");
+        return false;
+    }
+    if (!is_quant_type(type)) {
+        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, MXFP4).");
+        return false;
+    }
+    const size_t rs = row_size(type, ne0);
+    if (rs == 0) {
+        set_last_error("Quantized weight row length is not a multiple of the block size.");
+        return false;
+    }
+    if ((size_t)raw_bytes < rs * (size_t)ne1) {
+        set_last_error("Quantized weight byte span is too small for its dimensions.");
+        return false;
+    }
+    return true;
+}
+
+bool validate_fused_matmul(const TSHipTensorView2D& out, const TSHipTensorView2D& input, const void* norm_w, int norm_count,
+                           bool with_norm, const void* w, int type, int64_t ne0, int64_t ne1, int64_t raw_bytes, const char* what,
+                           const char* out_name)
+{
+    if (!validate_desc(out, out_name) || !validate_desc(input, "input")) return false;
+    if (with_norm && (norm_w == nullptr || norm_count <= 0)) {
+        set_last_error("Invalid norm weight data.");
+        return false;
+    }
+    if (!validate_weight(w, type, ne0, ne1, raw_bytes, what)) return false;
+    if (out.dim0 != input.dim0) {
+        set_last_error(std::string("Size mismatch: ") + out_name + ".dim0 != input.dim0 in " + what + ".");
+        return false;
+    }
+    if (ne0 != input.dim1 || ne1 != out.dim1 || (with_norm && norm_count != input.dim1)) {
+        set_last_error(std::string("Size mismatch: weight dims don't match in ") + what + ".");
+        return false;
+    }
+    if (out.stride1 != 1) {
+        set_last_error(std::string(out_name) + " must be a standard (stride1 == 1) view in " + what + ".");
+        return false;
+    }
+    return true;
+}
+
+bool validate_ffn(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const void* norm_w, int norm_count,
+                  const void* gu, int gu_type, int64_t gu_ne0, int64_t gu_ne1, int64_t gu_bytes, const void* dn, int dn_type,
+                  int64_t dn_ne0, int64_t dn_ne1, int64_t dn_bytes, int half_dim)
+{
+    if (!validate_desc(residual, "residual") || !validate_desc(input, "input")) return false;
+    if (norm_w == nullptr || norm_count <= 0) {
+        set_last_error("fused_ffn_swiglu: invalid norm weight.");
+        return false;
+    }
+    if (!validate_weight(gu, gu_type, gu_ne0, gu_ne1, gu_bytes, "fused_ffn_swiglu gate_up")) return false;
+    if (!validate_weight(dn, dn_type, dn_ne0, dn_ne1, dn_bytes, "fused_ffn_swiglu down")) return false;
+    const int hidden = input.dim1;
+    if (residual.dim0 != input.dim0 || residual.dim1 != hidden) {
+        set_last_error("fused_ffn_swiglu: residual shape mismatch.");
+        return false;
+    }
+    if (norm_count != hidden) {
+        set_last_error("fused_ffn_swiglu: norm_weight_count != hidden.");
+        return false;
+    }
+    if (gu_ne0 != hidden) {
+        set_last_error("fused_ffn_swiglu: gate_up.ne0 != hidden.");
+        return false;
+    }
+    if (half_dim <= 0 || gu_ne1 != 2 * (int64_t)half_dim) {
+        set_last_error("fused_ffn_swiglu: gate_up.ne1 != 2*half_dim.");
+        return false;
+    }
+    if (dn_ne0 != half_dim || dn_ne1 != hidden) {
+        set_last_error("fused_ffn_swiglu: down weight shape mismatch.");
+        return false;
+    }
+    if (residual.stride1 != 1) {
+        set_last_error("fused_ffn_swiglu: residual must be a standard (stride1 == 1) view.");
+        return false;
+    }
+    return true;
+}
+
+// Host tensors around a device computation: `input` (any non-negative-stride view) and optionally the current
+// contents of `inout` go up, `inout` comes back.  body(input_dev_view, inout_dev_view, norm_dev, stream).
+template <typename Body>
+int with_host_tensors(const TSHipTensorView2D& inout, bool upload_inout, const TSHipTensorView2D& input, const void* norm_w,
+                      int norm_count, Body&& body)
+{
+    if (!is_standard_view(inout)) {
+        set_last_error("The result / residual tensor must be a standard (stride1 == 1, non-overlapping) view.");
+        return 0;
+    }
+    std::lock_guard<std::mutex> lock(g_host_call_mutex);
+    const int M = input.dim0;
+    const size_t K = (size_t)input.dim1, N = (size_t)inout.dim1;
+    const size_t x_bytes = ((size_t)M * K * sizeof(float) + 255) & ~(size_t)255;
+    const size_t y_bytes = ((size_t)M * N * sizeof(float) + 255) & ~(size_t)255;
+    const size_t n_bytes = ((size_t)std::max(norm_count, 0) * sizeof(float) + 255) & ~(size_t)255;
+    if (!ws_reserve(x_bytes + y_bytes + n_bytes, x_bytes + y_bytes + n_bytes)) return 0;
+    char* dev = static_cast<char*>(g_ws.dev);
+    char* pin = static_cast<char*>(g_ws.pinned);
+    float* stage_x = reinterpret_cast<float*>(pin);
+    float* stage_y = reinterpret_cast<float*>(pin + x_bytes);
+    float* stage_n = reinterpret_cast<float*>(pin + x_bytes + y_bytes);
+    const float* src = static_cast<const float*>(input.data);
+    for (int m = 0; m < M; ++m)
+        for (size_t k = 0; k < K; ++k) stage_x[(size_t)m * K + k] = src[(size_t)m * input.stride0 + k * (size_t)input.stride1];
+    float* io = static_cast<float*>(inout.data);
+    if (upload_inout)
+        for (int m = 0; m < M; ++m) std::memcpy(stage_y + (size_t)m * N, io + (size_t)m * inout.stride0, N * sizeof(float));
+    if (norm_w) std::memcpy(stage_n, norm_w, (size_t)norm_count * sizeof(float));
+    hipStream_t stream = nullptr;
+    const size_t up = upload_inout ? x_bytes + y_bytes + (norm_w ? n_bytes : 0) : x_bytes;
+    if (!hip_ok(hipMemcpyAsync(dev, pin, up, hipMemcpyHostToDevice, stream), "hipMemcpy(inputs)")) return 0;
+    if (!upload_inout && norm_w &&
+        !hip_ok(hipMemcpyAsync(dev + x_bytes + y_bytes, stage_n, n_bytes, hipMemcpyHostToDevice, stream), "hipMemcpy(norm weight)"))
+        return 0;
+    const TSHipTensorView2D x_dev{dev, M, (int)K, (int)K, 1, (int64_t)((size_t)M * K * sizeof(float))};
+    const TSHipTensorView2D y_dev{dev + x_bytes, M, (int)N, (int)N, 1, (int64_t)((size_t)M * N * sizeof(float))};
+    if (!body(x_dev, y_dev, norm_w ? reinterpret_cast<const float*>(dev + x_bytes + y_bytes) : nullptr, stream)) return 0;
+    if (!hip_ok(hipMemcpyAsync(stage_y, dev + x_bytes, (size_t)M * N * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpy(result)"))
+        return 0;
+    if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+    for (int m = 0; m < M; ++m) std::memcpy(io + (size_t)m * inout.stride0, stage_y + (size_t)m * N, N * sizeof(float));
+    clear_last_error();
+    return 1;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -868,6 +1052,124 @@ int TSHip_GetRowsQuantF32(TSHipTensorView2D result, void* src_data, int src_ggml
         for (int64_t i = 0; i < n; ++i) std::memcpy(dst + (size_t)i * result.stride0, stage + (size_t)i * K, K * sizeof(float));
         clear_last_error();
         return 1;
+    });
+}
+
+/* ---- fused wrappers (ggml_ops_fused.cpp) ---------------------------------------------------- */
+
+int TSHip_FusedRmsNormMatMulQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D input, const float* norm_weight,
+                                           int norm_weight_count, float eps, const void* m2_data, int m2_ggml_type,
+                                           int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "fused_rms_norm_matmul_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_fused_matmul(result, input, norm_weight, norm_weight_count, true, m2_data, m2_ggml_type, m2_ne0, m2_ne1,
+                                   m2_raw_bytes, "fused rms_norm_matmul", "result"))
+            return 0;
+        const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, true);
+        void* ws = dev_ws_reserve(std::max<size_t>(need, 256));
+        if (!ws) return 0;
+        if (!run_matmul_device_ws(result, input, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load(), ws, norm_weight, eps, false))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_FusedMatMulQuantAddF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, const void* m2_data,
+                                       int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "fused_matmul_quant_add", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_fused_matmul(residual, input, nullptr, 0, false, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes,
+                                   "fused matmul_add", "residual"))
+            return 0;
+        const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, false);
+        void* ws = need ? dev_ws_reserve(need) : nullptr;
+        if (need && !ws) return 0;
+        if (!run_matmul_device_ws(residual, input, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load(), ws, nullptr, 0.f, true))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_FusedFFNSwiGLUQuantF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, const float* norm_weight,
+                                       int norm_weight_count, float eps, const void* gate_up_data, int gate_up_ggml_type,
+                                       int64_t gate_up_ne0, int64_t gate_up_ne1, int64_t gate_up_raw_bytes,
+                                       const void* down_data, int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                       int64_t down_raw_bytes, int half_dim)
+{
+    return guarded(0, "fused_ffn_swiglu_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_ffn(residual, input, norm_weight, norm_weight_count, gate_up_data, gate_up_ggml_type, gate_up_ne0,
+                          gate_up_ne1, gate_up_raw_bytes, down_data, down_ggml_type, down_ne0, down_ne1, down_raw_bytes, half_dim))
+            return 0;
+        if (!run_ffn_swiglu_device(residual, input, norm_weight, eps, gate_up_data, gate_up_ggml_type, down_data, down_ggml_type,
+                                   input.dim1, half_dim, g_stream.load()))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_FusedRmsNormMatMulQuantF32(TSHipTensorView2D result, TSHipTensorView2D input, void* norm_weight_data,
+                                     int norm_weight_count, float eps, void* m2_data, int m2_ggml_type, int64_t m2_ne0,
+                                     int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "fused_rms_norm_matmul_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_fused_matmul(result, input, norm_weight_data, norm_weight_count, true, m2_data, m2_ggml_type, m2_ne0,
+                                   m2_ne1, m2_raw_bytes, "fused rms_norm_matmul", "result"))
+            return 0;
+        const void* w = resolve_weight(m2_data, row_size(m2_ggml_type, m2_ne0) * (size_t)m2_ne1);
+        if (!w) return 0;
+        return with_host_tensors(result, false, input, norm_weight_data, norm_weight_count,
+                                 [&](const TSHipTensorView2D& x, const TSHipTensorView2D& y, const float* nw, hipStream_t st) {
+                                     const size_t need = matmul_ws_bytes(m2_ggml_type, x.dim0, m2_ne0, true);
+                                     void* ws = dev_ws_reserve(std::max<size_t>(need, 256));
+                                     return ws && run_matmul_device_ws(y, x, w, m2_ggml_type, m2_ne0, m2_ne1, st, ws, nw, eps, false);
+                                 });
+    });
+}
+
+int TSHip_FusedMatMulQuantAddF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* m2_data, int m2_ggml_type,
+                                 int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "fused_matmul_quant_add", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_fused_matmul(residual, input, nullptr, 0, false, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes,
+                                   "fused matmul_add", "residual"))
+            return 0;
+        const void* w = resolve_weight(m2_data, row_size(m2_ggml_type, m2_ne0) * (size_t)m2_ne1);
+        if (!w) return 0;
+        return with_host_tensors(residual, true, input, nullptr, 0,
+                                 [&](const TSHipTensorView2D& x, const TSHipTensorView2D& y, const float*, hipStream_t st) {
+                                     const size_t need = matmul_ws_bytes(m2_ggml_type, x.dim0, m2_ne0, false);
+                                     void* ws = need ? dev_ws_reserve(need) : nullptr;
+                                     return (!need || ws) && run_matmul_device_ws(y, x, w, m2_ggml_type, m2_ne0, m2_ne1, st, ws, nullptr, 0.f, true);
+                                 });
+    });
+}
+
+int TSHip_FusedFFNSwiGLUQuantF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* norm_weight_data,
+                                 int norm_weight_count, float eps, void* gate_up_data, int gate_up_ggml_type,
+                                 int64_t gate_up_ne0, int64_t gate_up_ne1, int64_t gate_up_raw_bytes, void* down_data,
+                                 int down_ggml_type, int64_t down_ne0, int64_t down_ne1, int64_t down_raw_bytes, int half_dim)
+{
+    return guarded(0, "fused_ffn_swiglu_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_ffn(residual, input, norm_weight_data, norm_weight_count, gate_up_data, gate_up_ggml_type, gate_up_ne0,
+                          gate_up_ne1, gate_up_raw_bytes, down_data, down_ggml_type, down_ne0, down_ne1, down_raw_bytes, half_dim))
+            return 0;
+        const void* gu = resolve_weight(gate_up_data, row_size(gate_up_ggml_type, gate_up_ne0) * (size_t)gate_up_ne1);
+        if (!gu) return 0;
+        const void* dn = resolve_weight(down_data, row_size(down_ggml_type, down_ne0) * (size_t)down_ne1);
+        if (!dn) return 0;
+        return with_host_tensors(residual, true, input, norm_weight_data, norm_weight_count,
+                                 [&](const TSHipTensorView2D& x, const TSHipTensorView2D& y, const float* nw, hipStream_t st) {
+                                     return run_ffn_swiglu_device(y, x, nw, eps, gu, gate_up_ggml_type, dn, down_ggml_type, x.dim1, half_dim, st);
+                                 });
     });
 }
 

@@ -33,7 +33,6 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kBK = 64;                 // k-tile
-constexpr int kLdsRow = kBK + 8;        // fp16 per LDS row: 144 B keeps ds_read_b128 conflict-free
 constexpr uint32_t kDeadOffset = 0x80000000u;
 
 union H2U {
@@ -101,15 +100,36 @@ __device__ __forceinline__ int k_slot(int k)
 // ------------------------------------------------------------------------------------------
 template <int TYPE>
 __global__ void __launch_bounds__(256) convert_x_kernel(const float* __restrict__ x, int64_t ldx, const int* __restrict__ row_map,
-                                                        int K, int Kp, _Float16* __restrict__ out, float* __restrict__ scales)
+                                                        int K, int Kp, _Float16* __restrict__ out, float* __restrict__ scales,
+                                                        const float* __restrict__ norm_w, float eps)
 {
     const int m = blockIdx.x;
     const float* src = x + (int64_t)(row_map ? row_map[m] : m) * ldx;
     __shared__ float red[4];
+    __shared__ double redd[4];
+    // optional RMSNorm prologue (ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1/sqrtf(mean + eps))
+    float rms = 1.f;
+    if (norm_w) {
+        double ss = 0.0;
+        for (int k = threadIdx.x * 4; k < K; k += 1024) {
+            const float4 v = *reinterpret_cast<const float4*>(src + k);
+            ss += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+        }
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((threadIdx.x & 63) == 0) redd[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        const float mean = (float)(((redd[0] + redd[1]) + (redd[2] + redd[3])) / (double)K);
+        rms = 1.0f / sqrtf(mean + eps);
+    }
+    auto value = [&](int k) { return norm_w ? (src[k] * rms) * norm_w[k] : src[k]; };
     float amax = 0.f;
-    for (int k = threadIdx.x * 4; k < K; k += 1024) {
-        const float4 v = *reinterpret_cast<const float4*>(src + k);
-        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    if (norm_w) {
+        for (int k = threadIdx.x; k < K; k += 256) amax = fmaxf(amax, fabsf(value(k)));
+    } else {
+        for (int k = threadIdx.x * 4; k < K; k += 1024) {
+            const float4 v = *reinterpret_cast<const float4*>(src + k);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
     }
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
@@ -124,7 +144,7 @@ __global__ void __launch_bounds__(256) convert_x_kernel(const float* __restrict_
     if (threadIdx.x == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
     _Float16* dst = out + (int64_t)m * Kp;
     for (int k = threadIdx.x; k < Kp; k += 256) {
-        const float v = k < K ? src[k] * inv : 0.f;
+        const float v = k < K ? value(k) * inv : 0.f;
         dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)v;
     }
 }
@@ -264,13 +284,13 @@ struct GemmArgs {
     const int* tile_row0;    // [m_tiles] first activation row
     const int* tile_rows;    // [m_tiles] rows in the tile (<= BM)
     int64_t expert_stride;   // bytes between experts
+    int accumulate;          // c += ... instead of c = ...
 };
 
 constexpr int kBN = 256;                     // weight rows (output columns) per tile: 32 per wavefront
 constexpr int kWaves = 8;
 constexpr int kRawTile = kBN * kRawRow;      // bytes of one raw super-tile in LDS
 constexpr int kRawInstrs = kRawTile / 1024;  // wavefront-wide 1 KiB copies per raw super-tile (36)
-constexpr int kWI = (kRawInstrs + kWaves - 1) / kWaves;   // copies per wavefront, the surplus goes to a dump area
 constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
 
 // LDS-direct copy: 64 lanes x 16 bytes land at lds + 16 * lane; out-of-range offsets deliver zeros
@@ -300,7 +320,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
     if (my_n >= A.N) return;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        float sc[16];
+        float sc[16], old[16];
         int64_t off[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -310,9 +330,11 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
             off[r] = (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc + my_n;
         }
 #pragma unroll
+        for (int r = 0; r < 16; ++r) old[r] = A.accumulate ? A.c[off[r]] : 0.f;
+#pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int ml = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (ml < m_rows) A.c[off[r]] = acc[i][r] * sc[r];
+            if (ml < m_rows) A.c[off[r]] = A.accumulate ? old[r] + acc[i][r] * sc[r] : acc[i][r] * sc[r];
         }
     }
 }
@@ -788,22 +810,22 @@ size_t gemm_workspace_bytes(int M, int K)
 int gemm_tile_m(int M) { return M > 1024 ? 256 : M > 64 ? 128 : 64; }
 
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
-                      hipStream_t stream)
+                      hipStream_t stream, const float* norm_w, float eps)
 {
     const int kp = (K + kBK - 1) / kBK * kBK;
     float* scales = static_cast<float*>(workspace);
     _Float16* x16 = reinterpret_cast<_Float16*>(static_cast<char*>(workspace) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
     switch (type) {
-    case kTypeQ4_K: hipLaunchKernelGGL(convert_x_kernel<kTypeQ4_K>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales); break;
-    case kTypeMXFP4: hipLaunchKernelGGL(convert_x_kernel<kTypeMXFP4>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales); break;
-    case kTypeQ8_0: hipLaunchKernelGGL(convert_x_kernel<kTypeQ8_0>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales); break;
+    case kTypeQ4_K: hipLaunchKernelGGL(convert_x_kernel<kTypeQ4_K>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
+    case kTypeMXFP4: hipLaunchKernelGGL(convert_x_kernel<kTypeMXFP4>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
+    case kTypeQ8_0: hipLaunchKernelGGL(convert_x_kernel<kTypeQ8_0>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
     default: set_last_error("gemm: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "activation convert launch");
 }
 
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
-                 int M, int N, int K, const GemmTiles* tiles, hipStream_t stream)
+                 int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate)
 {
     if (w_bytes >= ((int64_t)1 << 31) - 64 && !tiles) {
         set_last_error("gemm: a single weight of 2 GiB or more must be split by rows.");
@@ -817,6 +839,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     a.c = c;
     a.ldc = ldc;
     a.c_rows = c_rows;
+    a.accumulate = accumulate ? 1 : 0;
     a.M = M;
     a.N = N;
     a.K = K;

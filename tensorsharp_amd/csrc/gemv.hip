@@ -60,6 +60,7 @@ struct GemvProblem {
     int64_t w_bytes;
     const float* x;
     float* y;
+    const float* add;         // optional: y = add + W x (may be y itself: residual accumulation)
     const int* expert_id;     // optional (MoE): the weight is w + expert_id[0] * expert_stride
     int64_t expert_stride;
     int N;
@@ -571,7 +572,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
                 t += TSHIP_DPP_F(t, kDppHalfMirror);
                 t += TSHIP_DPP_F(t, kDppMirror);
                 const int row = cur[i].group * 4 + sub;
-                if (l16 == 0 && cur[i].group < ngroups && row < N) P.y[row] = t;
+                if (l16 == 0 && cur[i].group < ngroups && row < N) P.y[row] = P.add ? P.add[row] + t : t;
                 acc = 0.f;
             }
         }
@@ -670,6 +671,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         g.p[i].w_bytes = args[i].w_bytes;
         g.p[i].x = args[i].x;
         g.p[i].y = args[i].y;
+        g.p[i].add = args[i].add;
         g.p[i].N = args[i].N;
         g.p[i].K = args[i].K;
         g.p[i].expert_id = args[i].expert_id;
@@ -685,9 +687,10 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     }
 }
 
-bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream)
+bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream,
+                 const float* add)
 {
-    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0};
+    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, add};
     return launch_gemv_group(type, 1, &a, stream);
 }
 

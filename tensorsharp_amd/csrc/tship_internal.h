@@ -59,9 +59,9 @@ bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_
 bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, const int32_t* ids, int64_t n_ids, int64_t K,
                      float* dst, int64_t ldd, hipStream_t stream);
 
-// y[N] = W[N x K] * x[K]; W raw GGUF blocks, row-major; w_bytes = N * row_size.
+// y[N] = W[N x K] * x[K] (+ add[N] when given; add may be y); W raw GGUF blocks, row-major; w_bytes = N * row_size.
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K,
-                 hipStream_t stream);
+                 hipStream_t stream, const float* add = nullptr);
 // largest K the GEMV kernel stages in LDS for this type
 int gemv_max_k(int type);
 
@@ -75,6 +75,7 @@ struct GemvArgs {
     int K;
     const int* expert_id = nullptr;   // optional device pointer (MoE): weight = w + expert_id[0] * expert_stride
     int64_t expert_stride = 0;
+    const float* add = nullptr;       // optional: y = add + W x (add may be y)
 };
 int gemv_max_group();
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);
@@ -86,8 +87,9 @@ int gemm_tile_m(int M);   // rows of activations per tile for a plain (ungrouped
 
 // fp32 activations -> workspace (fp16 in the weight format's unpack order + per-row scales);
 // row_map (device, optional) gathers source rows.
+// norm_w (device, optional) applies RMSNorm first: x <- x / sqrt(mean(x^2) + eps) * norm_w.
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
-                      hipStream_t stream);
+                      hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f);
 
 // Grouped launches (MoE): m-tiles enumerated by device tables; weights of expert e start at
 // w + e * expert_stride and span w_bytes each.
@@ -101,8 +103,15 @@ struct GemmTiles {
 };
 
 // c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
+// accumulate: c[row] += ... instead of c[row] = ...
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc,
-                 const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream);
+                 const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate = false);
+
+// ---- fused wrappers around the matmul (RMSNorm prologue, SiLU-gated FFN) ------------------------
+// out[m, 0..K) = x[m] / sqrt(mean(x[m]^2) + eps) * w   (ggml_rms_norm then ggml_mul), contiguous rows
+bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps, int M, int K, float* out, hipStream_t stream);
+// out[m, j] = silu(gu[m, j]) * gu[m, half + j], j < half
+bool launch_silu_mul(const float* gu, int64_t ldgu, int M, int half, float* out, hipStream_t stream);
 
 // ---- MoE (GPT-OSS expert stage) -------------------------------------------------------------
 // ids / weights: [T x k] device; top-k by repeated argmax (first maximum wins), softmax over the k logits.

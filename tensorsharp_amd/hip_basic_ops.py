@@ -110,6 +110,45 @@ class HipBasicOps:
             raise RuntimeError(f"Native HIP dequantization failed (code {rc}): {N.get_last_error()}")
         return dst
 
+    # -- fused wrappers (GgmlBasicOps.FusedRmsNormMatMulQuant / FusedMatMulQuantAdd / FusedFFNSwiGLUQuant) ------
+    @staticmethod
+    def _views(out, inp):
+        """host (numpy) or device (torch) views of the in/out pair and the export suffix that takes them"""
+        if isinstance(out, np.ndarray):
+            return _host_view(out, standard=True), _host_view(inp, standard=False), ""
+        return _device_view(out), _device_view(inp), "Device"
+
+    @staticmethod
+    def _addr(a):
+        return a.ctypes.data if isinstance(a, np.ndarray) else a.data_ptr()
+
+    @staticmethod
+    def FusedRmsNormMatMulQuant(result, input, norm_weight, eps, weight):
+        """result = (RMSNorm(input) * norm_weight) * W^T; all host (numpy) or all device (torch) tensors."""
+        rv, iv, sfx = HipBasicOps._views(result, input)
+        fn = getattr(N.lib(), "TSHip_FusedRmsNormMatMulQuantF32" + sfx)
+        ok = fn(rv, iv, C.c_void_p(HipBasicOps._addr(norm_weight)), int(norm_weight.shape[0]), float(eps),
+                C.c_void_p(weight.ptr), weight.ggml_type, weight.ne0, weight.ne1, weight.raw_bytes)
+        N.check_result(ok, "fused_rms_norm_matmul_quant")
+
+    @staticmethod
+    def FusedMatMulQuantAdd(residual, input, weight):
+        """residual += input * W^T, in place."""
+        rv, iv, sfx = HipBasicOps._views(residual, input)
+        fn = getattr(N.lib(), "TSHip_FusedMatMulQuantAddF32" + sfx)
+        ok = fn(rv, iv, C.c_void_p(weight.ptr), weight.ggml_type, weight.ne0, weight.ne1, weight.raw_bytes)
+        N.check_result(ok, "fused_matmul_quant_add")
+
+    @staticmethod
+    def FusedFFNSwiGLUQuant(residual, input, norm_weight, eps, gate_up, down, half_dim):
+        """residual += W_down * (silu(g) * u), [g | u] = W_gate_up * (RMSNorm(input) * norm_weight)."""
+        rv, iv, sfx = HipBasicOps._views(residual, input)
+        fn = getattr(N.lib(), "TSHip_FusedFFNSwiGLUQuantF32" + sfx)
+        ok = fn(rv, iv, C.c_void_p(HipBasicOps._addr(norm_weight)), int(norm_weight.shape[0]), float(eps),
+                C.c_void_p(gate_up.ptr), gate_up.ggml_type, gate_up.ne0, gate_up.ne1, gate_up.raw_bytes,
+                C.c_void_p(down.ptr), down.ggml_type, down.ne0, down.ne1, down.raw_bytes, int(half_dim))
+        N.check_result(ok, "fused_ffn_swiglu_quant")
+
     # -- embedding gather ------------------------------------------------------------------
     @staticmethod
     def GetRowsQuant(result, weight_data, ggml_type, ne0, ne1, raw_bytes, indices):

@@ -58,6 +58,20 @@ SIGNATURES = {
     "TSHip_AddmmQuantGroupF32Device": (C.c_int, [C.c_int, C.POINTER(TensorView2D), C.POINTER(TensorView2D),
                                                  C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int64),
                                                  C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "TSHip_FusedRmsNormMatMulQuantF32": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_float, C.c_void_p,
+                                                   C.c_int, C.c_int64, C.c_int64, C.c_int64]),
+    "TSHip_FusedMatMulQuantAddF32": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64,
+                                               C.c_int64]),
+    "TSHip_FusedFFNSwiGLUQuantF32": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_float,
+                                               C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                               C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
+    "TSHip_FusedRmsNormMatMulQuantF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_float,
+                                                         C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64]),
+    "TSHip_FusedMatMulQuantAddF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_int64,
+                                                     C.c_int64, C.c_int64]),
+    "TSHip_FusedFFNSwiGLUQuantF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_float,
+                                                     C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                     C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
     "TSHip_GetRowsQuantF32": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
                                         ContiguousTensor]),
     "TSHip_GetRowsQuantF32Device": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,

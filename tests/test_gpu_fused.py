@@ -1,0 +1,131 @@
+"""GPU parity: the bridge's fused wrappers around the quantized matmul (ggml_ops_fused.cpp:21-640) through the
+C ABI, host-pointer and device forms, decode (GEMV) and prefill (GEMM) row counts.
+
+Reference value: oracle RMSNorm / SiLU restatements (fp32, ggml order) around the fp64 product with the bit-exact
+dequantized weights.  Bar: max_j |y - ref| <= 1e-3 * ||matmul part of the row||_2 (the residual that is added
+is exact and must not loosen the bound)."""
+import numpy as np
+import pytest
+
+from oracle.oracle import Q8_0, Q4_K, MXFP4
+
+pytestmark = pytest.mark.gpu
+T_ = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
+EPS = 1e-6
+
+
+def make(oracle, name, N, K, rng, sigma=0.03):
+    return oracle.quantize(T_[name], (rng.standard_normal(N * K) * sigma).astype(np.float32))
+
+
+def bound_ok(got, ref, mm):
+    tol = 1e-3 * np.linalg.norm(mm.astype(np.float64), axis=1, keepdims=True)
+    return np.all(np.abs(got.astype(np.float64) - ref) <= tol + 1e-30), float(np.max(np.abs(got - ref) / (tol + 1e-30)))
+
+
+def qweights(name, arrs, device):
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    out = []
+    for wq, K, N in arrs:
+        out.append(QuantizedWeight(torch.from_numpy(wq).cuda() if device else wq, T_[name], K, N))
+    return out
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+@pytest.mark.parametrize("M", [1, 3, 40])
+@pytest.mark.parametrize("device", [False, True])
+def test_rms_norm_matmul(hip, oracle, name, M, device):
+    import torch
+    rng = np.random.default_rng(91 + M)
+    N, K = 384, 1024
+    wq = make(oracle, name, N, K, rng)
+    x = (rng.standard_normal((M, K)) * 3).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    xn = oracle.rms_norm_mul(x, nw, EPS)
+    ref = oracle.matmul_f64(T_[name], wq, N, K, xn)
+    (qw,) = qweights(name, [(wq, K, N)], device)
+    if device:
+        res = torch.empty((M, N), device="cuda")
+        hip.FusedRmsNormMatMulQuant(res, torch.from_numpy(x).cuda(), torch.from_numpy(nw).cuda(), EPS, qw)
+        torch.cuda.synchronize()
+        got = res.cpu().numpy()
+    else:
+        got = np.full((M, N), np.nan, dtype=np.float32)
+        hip.FusedRmsNormMatMulQuant(got, x, nw, EPS, qw)
+        hip.ClearHostBufferCache()
+    ok, worst = bound_ok(got, ref, ref)
+    assert ok, (name, M, device, worst)
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+@pytest.mark.parametrize("M", [1, 2, 70, 300])
+@pytest.mark.parametrize("device", [False, True])
+def test_matmul_add_in_place(hip, oracle, name, M, device):
+    import torch
+    rng = np.random.default_rng(93 + M)
+    N, K = 320, 768
+    wq = make(oracle, name, N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    resid = (rng.standard_normal((M, N)) * 5).astype(np.float32)
+    mm = oracle.matmul_f64(T_[name], wq, N, K, x)
+    ref = resid.astype(np.float64) + mm
+    (qw,) = qweights(name, [(wq, K, N)], device)
+    if device:
+        r = torch.from_numpy(resid.copy()).cuda()
+        hip.FusedMatMulQuantAdd(r, torch.from_numpy(x).cuda(), qw)
+        torch.cuda.synchronize()
+        got = r.cpu().numpy()
+    else:
+        got = resid.copy()
+        hip.FusedMatMulQuantAdd(got, x, qw)
+        hip.ClearHostBufferCache()
+    ok, worst = bound_ok(got, ref, mm)
+    assert ok, (name, M, device, worst)
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+@pytest.mark.parametrize("M", [1, 3, 48])
+@pytest.mark.parametrize("device", [False, True])
+def test_ffn_swiglu(hip, oracle, name, M, device):
+    import torch
+    rng = np.random.default_rng(95 + M)
+    H, F = 512, 768
+    gu = make(oracle, name, 2 * F, H, rng, 0.05)
+    dn = make(oracle, name, H, F, rng, 0.05)
+    x = (rng.standard_normal((M, H)) * 2).astype(np.float32)
+    resid = rng.standard_normal((M, H)).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    xn = oracle.rms_norm_mul(x, nw, EPS)
+    g = oracle.matmul_f64(T_[name], gu, 2 * F, H, xn).astype(np.float32)
+    act = oracle.silu_mul(g)
+    mm = oracle.matmul_f64(T_[name], dn, H, F, act)
+    ref = resid.astype(np.float64) + mm
+    qgu, qdn = qweights(name, [(gu, H, 2 * F), (dn, F, H)], device)
+    if device:
+        r = torch.from_numpy(resid.copy()).cuda()
+        hip.FusedFFNSwiGLUQuant(r, torch.from_numpy(x).cuda(), torch.from_numpy(nw).cuda(), EPS, qgu, qdn, F)
+        torch.cuda.synchronize()
+        got = r.cpu().numpy()
+    else:
+        got = resid.copy()
+        hip.FusedFFNSwiGLUQuant(got, x, nw, EPS, qgu, qdn, F)
+        hip.ClearHostBufferCache()
+    # two chained fp16-operand matmuls: the first one's error passes through SiLU and the second matmul
+    tol = 2e-3 * np.linalg.norm(mm, axis=1, keepdims=True)
+    assert np.all(np.abs(got - ref) <= tol), (name, M, device, float(np.max(np.abs(got - ref) / tol)))
+
+
+def test_fused_argument_errors(hip, oracle):
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(97)
+    wq = make(oracle, "q8_0", 64, 128, rng)
+    qw = QuantizedWeight(wq, Q8_0, 128, 64)
+    x = np.zeros((2, 128), np.float32)
+    with pytest.raises(RuntimeError, match="Size mismatch"):
+        hip.FusedMatMulQuantAdd(np.zeros((3, 64), np.float32), x, qw)
+    with pytest.raises(RuntimeError, match="Size mismatch"):
+        hip.FusedRmsNormMatMulQuant(np.zeros((2, 64), np.float32), x, np.ones(100, np.float32), EPS, qw)
+    with pytest.raises(RuntimeError, match="gate_up.ne1 != 2\\*half_dim"):
+        hip.FusedFFNSwiGLUQuant(np.zeros((2, 128), np.float32), x, np.ones(128, np.float32), EPS, qw, qw, 48)
+    hip.ClearHostBufferCache()
