@@ -241,6 +241,29 @@ def main():
 
         extra["cfg4_mxfp4_moe_experts_T1"] = moe(1, n_it)
         extra["cfg4_mxfp4_moe_experts_T256"] = moe(256, 30)
+        # fused SwiGLU FFN at decode (configs[1] shapes: hidden 4096, intermediate 14336, Q4_K, one token):
+        # RMSNorm -> gate_up GEMV -> SiLU*up -> down GEMV + residual, one ABI call (4 launches)
+        def fused_ffn(copies=3):
+            Hd, Fd = 4096, 14336
+            ws = [(QuantizedWeight(synth.random_weight(Q4_K, 2 * Fd, Hd, dev, seed=700 + c), Q4_K, Hd, 2 * Fd),
+                   QuantizedWeight(synth.random_weight(Q4_K, Hd, Fd, dev, seed=800 + c), Q4_K, Fd, Hd)) for c in range(copies)]
+            x = torch.randn((1, Hd), device=dev)
+            nw = torch.ones(Hd, device=dev)
+            res = torch.zeros((1, Hd), device=dev)
+
+            def f(i):
+                gu, dn = ws[i % copies]
+                HipBasicOps.FusedFFNSwiGLUQuant(res, x, nw, 1e-6, gu, dn, Fd)
+            for i in range(20):
+                f(i)
+            ev, wall = time_region(f, n_it, torch)
+            us = ev * 1e3 / n_it
+            b = (2 * Fd + Hd) * row_bytes(Q4_K, Hd) + 0  # gate_up rows of K=4096 ...
+            b = 2 * Fd * row_bytes(Q4_K, Hd) + Hd * row_bytes(Q4_K, Fd)
+            return {"us_per_call_events": round(us, 2), "bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                    "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)}
+
+        extra["cfg2_q4_k_fused_ffn_decode_4096x14336"] = fused_ffn()
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -273,6 +273,10 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
 {
     const size_t w_bytes = row_size(type, K) * (size_t)N;
     if (!check_device_operands(m1, w, type)) return false;
+    if (norm_w && (reinterpret_cast<uintptr_t>(norm_w) & 15) != 0) {
+        set_last_error("The norm weight must be 16-byte aligned on the device.");
+        return false;
+    }
     const int M = m1.dim0;
     if (M <= 3 && K <= gemv_max_k(type)) {
         // decode / tiny batch: one bandwidth-bound GEMV per activation row

@@ -98,55 +98,86 @@ __device__ __forceinline__ int k_slot(int k)
 // ------------------------------------------------------------------------------------------
 // activations: fp32 [M x K] (row stride ldx) -> fp16 [M x Kp] in unpack order, per-row scale
 // ------------------------------------------------------------------------------------------
+constexpr int kCvtThreads = 1024;
+constexpr int kCvtHold = 8;      // float4 per thread kept in registers: rows up to 32768 elements are read once
+
 template <int TYPE>
-__global__ void __launch_bounds__(256) convert_x_kernel(const float* __restrict__ x, int64_t ldx, const int* __restrict__ row_map,
-                                                        int K, int Kp, _Float16* __restrict__ out, float* __restrict__ scales,
-                                                        const float* __restrict__ norm_w, float eps)
+__global__ void __launch_bounds__(kCvtThreads) convert_x_kernel(const float* __restrict__ x, int64_t ldx, const int* __restrict__ row_map,
+                                                                int K, int Kp, _Float16* __restrict__ out, float* __restrict__ scales,
+                                                                const float* __restrict__ norm_w, float eps)
 {
     const int m = blockIdx.x;
+    const int tid = threadIdx.x;
     const float* src = x + (int64_t)(row_map ? row_map[m] : m) * ldx;
-    __shared__ float red[4];
-    __shared__ double redd[4];
-    // optional RMSNorm prologue (ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1/sqrtf(mean + eps))
+    __shared__ float red[kCvtThreads / 64];
+    __shared__ double redd[kCvtThreads / 64];
+    const int k4 = K >> 2;                       // K is a multiple of 32
+    constexpr int kHeld = kCvtHold * kCvtThreads * 4;
+    float4 hold[kCvtHold];
+#pragma unroll
+    for (int i = 0; i < kCvtHold; ++i) {
+        const int q = tid + i * kCvtThreads;
+        hold[i] = q < k4 ? reinterpret_cast<const float4*>(src)[q] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    // optional RMSNorm prologue (ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1/sqrtf(mean + eps),
+    // then the multiply by the norm weight: (x * scale) * w)
     float rms = 1.f;
     if (norm_w) {
         double ss = 0.0;
-        for (int k = threadIdx.x * 4; k < K; k += 1024) {
-            const float4 v = *reinterpret_cast<const float4*>(src + k);
-            ss += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
-        }
+#pragma unroll
+        for (int i = 0; i < kCvtHold; ++i)
+            ss += (double)(hold[i].x * hold[i].x) + (double)(hold[i].y * hold[i].y) + (double)(hold[i].z * hold[i].z) +
+                  (double)(hold[i].w * hold[i].w);
+        for (int k = kHeld + tid; k < K; k += kCvtThreads) ss += (double)(src[k] * src[k]);
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-        if ((threadIdx.x & 63) == 0) redd[threadIdx.x >> 6] = ss;
+        if ((tid & 63) == 0) redd[tid >> 6] = ss;
         __syncthreads();
-        const float mean = (float)(((redd[0] + redd[1]) + (redd[2] + redd[3])) / (double)K);
-        rms = 1.0f / sqrtf(mean + eps);
-    }
-    auto value = [&](int k) { return norm_w ? (src[k] * rms) * norm_w[k] : src[k]; };
-    float amax = 0.f;
-    if (norm_w) {
-        for (int k = threadIdx.x; k < K; k += 256) amax = fmaxf(amax, fabsf(value(k)));
-    } else {
-        for (int k = threadIdx.x * 4; k < K; k += 1024) {
-            const float4 v = *reinterpret_cast<const float4*>(src + k);
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        double tot = 0.0;
+#pragma unroll
+        for (int i = 0; i < kCvtThreads / 64; ++i) tot += redd[i];
+        rms = 1.0f / sqrtf((float)(tot / (double)K) + eps);
+#pragma unroll
+        for (int i = 0; i < kCvtHold; ++i) {
+            const int q = tid + i * kCvtThreads;
+            if (q < k4) {
+                const float4 wv = reinterpret_cast<const float4*>(norm_w)[q];
+                hold[i] = float4{(hold[i].x * rms) * wv.x, (hold[i].y * rms) * wv.y, (hold[i].z * rms) * wv.z, (hold[i].w * rms) * wv.w};
+            }
         }
     }
+    auto tail_value = [&](int k) { return norm_w ? (src[k] * rms) * norm_w[k] : src[k]; };
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < kCvtHold; ++i)
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(hold[i].x), fabsf(hold[i].y)), fmaxf(fabsf(hold[i].z), fabsf(hold[i].w))));
+    for (int k = kHeld + tid; k < K; k += kCvtThreads) amax = fmaxf(amax, fabsf(tail_value(k)));
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < kCvtThreads / 64; ++i) amax = fmaxf(amax, red[i]);
     // power-of-two scale bringing amax into [2^13, 2^14)
     int e = (int)((__float_as_uint(amax) >> 23) & 0xffu);
     if (e == 255) e = 127;
     if (e < 14) e = 14;
     const int se = e - 13;
     const float inv = __uint_as_float((uint32_t)(254 - se) << 23);
-    if (threadIdx.x == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
+    if (tid == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
     _Float16* dst = out + (int64_t)m * Kp;
-    for (int k = threadIdx.x; k < Kp; k += 256) {
-        const float v = k < K ? value(k) * inv : 0.f;
-        dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)v;
+    auto put = [&](int k, float v) { dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)(v * inv); };
+#pragma unroll
+    for (int i = 0; i < kCvtHold; ++i) {
+        const int q = tid + i * kCvtThreads;
+        if (q < k4) {
+            put(4 * q, hold[i].x);
+            put(4 * q + 1, hold[i].y);
+            put(4 * q + 2, hold[i].z);
+            put(4 * q + 3, hold[i].w);
+        }
     }
+    for (int k = kHeld + tid; k < K; k += kCvtThreads) put(k, tail_value(k));
+    for (int k = K + tid; k < Kp; k += kCvtThreads) dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)0.f;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -816,9 +847,9 @@ bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map,
     float* scales = static_cast<float*>(workspace);
     _Float16* x16 = reinterpret_cast<_Float16*>(static_cast<char*>(workspace) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
     switch (type) {
-    case kTypeQ4_K: hipLaunchKernelGGL(convert_x_kernel<kTypeQ4_K>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
-    case kTypeMXFP4: hipLaunchKernelGGL(convert_x_kernel<kTypeMXFP4>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
-    case kTypeQ8_0: hipLaunchKernelGGL(convert_x_kernel<kTypeQ8_0>, dim3(M), dim3(256), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
+    case kTypeQ4_K: hipLaunchKernelGGL(convert_x_kernel<kTypeQ4_K>, dim3(M), dim3(kCvtThreads), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
+    case kTypeMXFP4: hipLaunchKernelGGL(convert_x_kernel<kTypeMXFP4>, dim3(M), dim3(kCvtThreads), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
+    case kTypeQ8_0: hipLaunchKernelGGL(convert_x_kernel<kTypeQ8_0>, dim3(M), dim3(kCvtThreads), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
     default: set_last_error("gemm: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "activation convert launch");
