@@ -282,14 +282,17 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
         // decode / tiny batch: one bandwidth-bound GEMV per activation row
         const float* xs = static_cast<const float*>(m1.data);
         int64_t ldx = m1.stride0;
-        if (norm_w) {
+        // RMSNorm is formed by the GEMV while it stages x (rows up to gemv_rms_max_k()), else by a kernel of its own
+        const bool norm_in_gemv = norm_w && K <= gemv_rms_max_k();
+        if (norm_w && !norm_in_gemv) {
             if (!launch_rms_norm_rows(xs, ldx, norm_w, eps, M, (int)K, static_cast<float*>(ws), stream)) return false;
             xs = static_cast<const float*>(ws);
             ldx = K;
         }
         for (int m = 0; m < M; ++m) {
             float* y = static_cast<float*>(result.data) + (int64_t)m * result.stride0;
-            if (!launch_gemv(type, w, (int64_t)w_bytes, xs + (int64_t)m * ldx, y, (int)N, (int)K, stream, accumulate ? y : nullptr))
+            if (!launch_gemv(type, w, (int64_t)w_bytes, xs + (int64_t)m * ldx, y, (int)N, (int)K, stream, accumulate ? y : nullptr,
+                             norm_in_gemv ? 1 : 0, norm_w, eps))
                 return false;
         }
         return true;
@@ -329,6 +332,17 @@ bool run_ffn_swiglu_device(const TSHipTensorView2D& residual, const TSHipTensorV
     void* mm_ws = ws + gu_bytes + act_bytes;
     const TSHipTensorView2D gu_view{gu, M, 2 * half, 2 * half, 1, (int64_t)((size_t)M * 2 * half * sizeof(float))};
     if (!run_matmul_device_ws(gu_view, input, gate_up, gu_type, hidden, 2 * half, stream, mm_ws, norm_w, eps, false)) return false;
+    if (M <= 3 && half <= gemv_max_k(dn_type)) {
+        // decode: the down GEMV forms silu(gate) * up while it stages its activations and adds the residual in its store
+        if (!check_device_operands(gu_view, down, dn_type)) return false;
+        const size_t dn_bytes = row_size(dn_type, half) * (size_t)hidden;
+        for (int m = 0; m < M; ++m) {
+            float* y = static_cast<float*>(residual.data) + (int64_t)m * residual.stride0;
+            if (!launch_gemv(dn_type, down, (int64_t)dn_bytes, gu + (size_t)m * 2 * half, y, hidden, half, stream, y, 2, nullptr, 0.f))
+                return false;
+        }
+        return true;
+    }
     if (!launch_silu_mul(gu, 2 * half, M, half, act, stream)) return false;
     const TSHipTensorView2D act_view{act, M, half, half, 1, (int64_t)((size_t)M * half * sizeof(float))};
     return run_matmul_device_ws(residual, act_view, down, dn_type, half, hidden, stream, mm_ws, nullptr, 0.f, true);

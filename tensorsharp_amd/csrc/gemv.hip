@@ -55,12 +55,20 @@ constexpr int kMaxGroup = 8;
 constexpr int kU = TSHIP_GEMV_KU;      // steps per wavefront fetched together, one fetch ahead of the compute
 
 // one GEMV
+// activation modes: what the workgroup stages as x
+constexpr int kActPlain = 0;      // x[k]
+constexpr int kActRmsNorm = 1;    // (x[k] / sqrt(mean(x^2) + eps)) * norm_w[k]        (ggml_rms_norm, ggml_mul)
+constexpr int kActSiluMul = 2;    // silu(x[k]) * x[K + k]: x is a [2K] gate|up row    (ggml_silu, ggml_mul)
+
 struct GemvProblem {
     const uint8_t* w;
     int64_t w_bytes;
     const float* x;
     float* y;
     const float* add;         // optional: y = add + W x (may be y itself: residual accumulation)
+    const float* norm_w;      // activation mode kActRmsNorm: the norm weight [K]
+    float eps;
+    int act;                  // how x is formed while it is staged (kAct*)
     const int* expert_id;     // optional (MoE): the weight is w + expert_id[0] * expert_stride
     int64_t expert_stride;
     int N;
@@ -458,7 +466,9 @@ struct Step {
     int group;        // uniform; >= ngroups marks a step past the end (its loads read zeros)
 };
 
-template <typename F>
+// ACT: the activation mode of every problem of the launch (compile time: the plain kernel carries none of
+// the other modes' code or registers)
+template <typename F, int ACT>
 __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, uint32_t* lds)
 {
     const int lane = threadIdx.x & 63;
@@ -506,6 +516,11 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(P.x), 0, K * 4, 0x00020000);
     constexpr int kStageChunk = 8 / F::kStageF4;           // work items per thread per pass
     float4 xv[kStageChunk][F::kStageF4];
+    // second operand of the activation modes: the norm weight (same offsets) or the "up" half (offsets + 4 K)
+    constexpr int act = ACT;
+    const __amdgpu_buffer_rsrc_t x2rs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(act == kActRmsNorm ? P.norm_w : P.x + K), 0, K * 4, 0x00020000);
+    float4 x2[kStageChunk][F::kStageF4];
     auto stage_issue = [&](int base) {
 #pragma unroll
         for (int c = 0; c < kStageChunk; ++c) {
@@ -517,10 +532,50 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
                 // items past the end fall outside the resource and read as zeros
                 const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
                 xv[c][q] = float4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+                if (act != kActPlain) {
+                    const uint4_t u = __builtin_amdgcn_raw_buffer_load_b128(x2rs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
+                    x2[c][q] = float4{__uint_as_float(u.x), __uint_as_float(u.y), __uint_as_float(u.z), __uint_as_float(u.w)};
+                }
             }
         }
     };
+    // kActRmsNorm: the whole row is in the registers of the workgroup after ONE pass (the host guarantees it);
+    // sum of squares in double over the workgroup, then (x * scale) * w in place
+    double* red = reinterpret_cast<double*>(lds + nsteps * 16 * F::kLdsDwords);      // [kWaves], after the x area
+    auto apply_act = [&]() {
+        if (act == kActRmsNorm) {
+            double ss = 0.0;
+#pragma unroll
+            for (int c = 0; c < kStageChunk; ++c)
+#pragma unroll
+                for (int q = 0; q < F::kStageF4; ++q)
+                    ss += (double)(xv[c][q].x * xv[c][q].x) + (double)(xv[c][q].y * xv[c][q].y) +
+                          (double)(xv[c][q].z * xv[c][q].z) + (double)(xv[c][q].w * xv[c][q].w);
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+            if (lane == 0) red[threadIdx.x >> 6] = ss;
+            __syncthreads();
+            double tot = 0.0;
+#pragma unroll
+            for (int i = 0; i < kWaves; ++i) tot += red[i];
+            const float scale = 1.0f / sqrtf((float)(tot / (double)K) + P.eps);
+#pragma unroll
+            for (int c = 0; c < kStageChunk; ++c)
+#pragma unroll
+                for (int q = 0; q < F::kStageF4; ++q)
+                    xv[c][q] = float4{(xv[c][q].x * scale) * x2[c][q].x, (xv[c][q].y * scale) * x2[c][q].y,
+                                      (xv[c][q].z * scale) * x2[c][q].z, (xv[c][q].w * scale) * x2[c][q].w};
+        } else if (act == kActSiluMul) {
+            auto silu = [](float g) { return g / (1.0f + expf(-g)); };
+#pragma unroll
+            for (int c = 0; c < kStageChunk; ++c)
+#pragma unroll
+                for (int q = 0; q < F::kStageF4; ++q)
+                    xv[c][q] = float4{silu(xv[c][q].x) * x2[c][q].x, silu(xv[c][q].y) * x2[c][q].y,
+                                      silu(xv[c][q].z) * x2[c][q].z, silu(xv[c][q].w) * x2[c][q].w};
+        }
+    };
     auto stage_commit = [&](int base) {
+        if (act != kActPlain) apply_act();
 #pragma unroll
         for (int c = 0; c < kStageChunk; ++c) {
             if (base + c * kThreads < items) {   // uniform
@@ -581,7 +636,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     }
 }
 
-template <int TYPE>
+template <int TYPE, int ACT>
 __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
 {
     extern __shared__ uint32_t lds[];
@@ -591,9 +646,9 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
         if (j < G.count && (int)blockIdx.x >= G.wg_begin[j]) i = j;
     const int wg = (int)blockIdx.x - G.wg_begin[i];
     const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
-    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K>(G.p[i], wg, nwg, lds);
-    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4>(G.p[i], wg, nwg, lds);
-    else gemv_body<FmtQ80>(G.p[i], wg, nwg, lds);
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT>(G.p[i], wg, nwg, lds);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT>(G.p[i], wg, nwg, lds);
+    else gemv_body<FmtQ80, ACT>(G.p[i], wg, nwg, lds);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
@@ -602,15 +657,15 @@ int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
 size_t lds_bytes_for(int type, int K)
 {
     const size_t units = (size_t)((K / unit_elems(type) + 15) / 16) * 16;
-    return units * (type == kTypeMXFP4 ? 80 : 144);
+    return units * (type == kTypeMXFP4 ? 80 : 144) + kWaves * sizeof(double);   // + the RMSNorm reduction slots
 }
 
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 
-template <int TYPE>
+template <int TYPE, int ACT>
 bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    auto kern = gemv_kernel<TYPE>;
+    auto kern = gemv_kernel<TYPE, ACT>;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g);
     return hip_ok(hipGetLastError(), "gemv launch");
@@ -629,6 +684,9 @@ int gemv_max_k(int type)
 }
 
 int gemv_max_group() { return kMaxGroup; }
+
+// one staging pass covers 8 float4 per thread
+int gemv_rms_max_k() { return kThreads * 8 * 4; }
 
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream)
 {
@@ -672,6 +730,13 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         g.p[i].x = args[i].x;
         g.p[i].y = args[i].y;
         g.p[i].add = args[i].add;
+        g.p[i].act = args[i].act;
+        g.p[i].norm_w = args[i].norm_w;
+        g.p[i].eps = args[i].eps;
+        if (args[i].act == kActRmsNorm && args[i].K > gemv_rms_max_k()) {
+            set_last_error("gemv: the RMSNorm activation mode stages the row in one pass; K is too large.");
+            return false;
+        }
         g.p[i].N = args[i].N;
         g.p[i].K = args[i].K;
         g.p[i].expert_id = args[i].expert_id;
@@ -680,17 +745,32 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         begin += share;
     }
     for (int i = count; i <= kMaxGroup; ++i) g.wg_begin[i] = begin;
-    switch (type) {
-    case kTypeQ4_K: return launch_type<kTypeQ4_K>(g, begin, lds, stream);
-    case kTypeMXFP4: return launch_type<kTypeMXFP4>(g, begin, lds, stream);
-    default: return launch_type<kTypeQ8_0>(g, begin, lds, stream);
+    const int act = args[0].act;
+    for (int i = 1; i < count; ++i)
+        if (args[i].act != act) {
+            set_last_error("gemv: the problems of one launch must share the activation mode.");
+            return false;
+        }
+    if (act < kActPlain || act > kActSiluMul) {
+        set_last_error("gemv: unknown activation mode.");
+        return false;
     }
+#define TSHIP_GEMV_DISPATCH(T)                                                           \
+    (act == kActPlain     ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
+     : act == kActRmsNorm ? launch_type<T, kActRmsNorm>(g, begin, lds, stream)           \
+                          : launch_type<T, kActSiluMul>(g, begin, lds, stream))
+    switch (type) {
+    case kTypeQ4_K: return TSHIP_GEMV_DISPATCH(kTypeQ4_K);
+    case kTypeMXFP4: return TSHIP_GEMV_DISPATCH(kTypeMXFP4);
+    default: return TSHIP_GEMV_DISPATCH(kTypeQ8_0);
+    }
+#undef TSHIP_GEMV_DISPATCH
 }
 
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream,
-                 const float* add)
+                 const float* add, int act, const float* norm_w, float eps)
 {
-    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, add};
+    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, add, act, norm_w, eps};
     return launch_gemv_group(type, 1, &a, stream);
 }
 

@@ -60,8 +60,11 @@ bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, 
                      float* dst, int64_t ldd, hipStream_t stream);
 
 // y[N] = W[N x K] * x[K] (+ add[N] when given; add may be y); W raw GGUF blocks, row-major; w_bytes = N * row_size.
+// act: 0 plain x; 1 RMSNorm(x, eps) * norm_w formed while x is staged (K <= gemv_rms_max_k()); 2 x is a [2K] row
+// gate|up and the staged activation is silu(gate) * up.
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K,
-                 hipStream_t stream, const float* add = nullptr);
+                 hipStream_t stream, const float* add = nullptr, int act = 0, const float* norm_w = nullptr, float eps = 0.f);
+int gemv_rms_max_k();
 // largest K the GEMV kernel stages in LDS for this type
 int gemv_max_k(int type);
 
@@ -76,6 +79,9 @@ struct GemvArgs {
     const int* expert_id = nullptr;   // optional device pointer (MoE): weight = w + expert_id[0] * expert_stride
     int64_t expert_stride = 0;
     const float* add = nullptr;       // optional: y = add + W x (add may be y)
+    int act = 0;                      // activation mode, see launch_gemv
+    const float* norm_w = nullptr;
+    float eps = 0.f;
 };
 int gemv_max_group();
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);

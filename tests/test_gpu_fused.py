@@ -129,3 +129,21 @@ def test_fused_argument_errors(hip, oracle):
     with pytest.raises(RuntimeError, match="gate_up.ne1 != 2\\*half_dim"):
         hip.FusedFFNSwiGLUQuant(np.zeros((2, 128), np.float32), x, np.ones(128, np.float32), EPS, qw, qw, 48)
     hip.ClearHostBufferCache()
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q8_0"])
+def test_rms_norm_matmul_row_longer_than_one_staging_pass(hip, oracle, name):
+    # K above what the decode kernel stages in one pass: RMSNorm runs as a kernel of its own
+    import torch
+    rng = np.random.default_rng(99)
+    N, K, M = 64, 16384 + 512, 2
+    wq = make(oracle, name, N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    ref = oracle.matmul_f64(T_[name], wq, N, K, oracle.rms_norm_mul(x, nw, EPS))
+    (qw,) = qweights(name, [(wq, K, N)], True)
+    res = torch.empty((M, N), device="cuda")
+    hip.FusedRmsNormMatMulQuant(res, torch.from_numpy(x).cuda(), torch.from_numpy(nw).cuda(), EPS, qw)
+    torch.cuda.synchronize()
+    ok, worst = bound_ok(res.cpu().numpy(), ref, ref)
+    assert ok, (name, worst)
