@@ -802,9 +802,14 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
                                    (int)(2 * F), (int)H, ids + a, gu_bytes};
             }
             if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
-            if (!launch_moe_swiglu(gu, gate_up_bias, ids, A, (int)F, alpha, limit, act, stream)) return 0;
-            for (int a = 0; a < A; ++a)
-                args[a] = GemvArgs{down_w, dn_bytes, act + (int64_t)a * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes};
+            // the down GEMVs form bias + SwiGLU-OAI from the gate|up rows while they stage their activations
+            for (int a = 0; a < A; ++a) {
+                args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * 2 * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes};
+                args[a].act = 3;
+                args[a].norm_w = gate_up_bias;
+                args[a].eps = alpha;
+                args[a].limit = limit;
+            }
             if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
             if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, (int)H, T == 1, static_cast<float*>(result.data),
                                     result.stride0, stream))

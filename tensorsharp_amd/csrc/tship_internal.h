@@ -79,9 +79,11 @@ struct GemvArgs {
     const int* expert_id = nullptr;   // optional device pointer (MoE): weight = w + expert_id[0] * expert_stride
     int64_t expert_stride = 0;
     const float* add = nullptr;       // optional: y = add + W x (add may be y)
-    int act = 0;                      // activation mode, see launch_gemv
+    int act = 0;                      // activation mode, see launch_gemv; 3 = GPT-OSS SwiGLU (x is a gate|up row of 2K,
+                                      // norm_w the optional [E][2K] bias indexed by expert_id, eps = alpha, limit = clamp)
     const float* norm_w = nullptr;
     float eps = 0.f;
+    float limit = 0.f;
 };
 int gemv_max_group();
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);
