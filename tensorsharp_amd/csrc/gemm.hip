@@ -23,6 +23,7 @@
 #include "tship_internal.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace tship {
 namespace {
@@ -716,8 +717,12 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
         for (int e = 0; e < 2; ++e) {
             const int kt = 2 * p + e;
 #pragma unroll
-            for (int i = 0; i < XI; ++i)
+            for (int i = 0; i < XI; ++i) {
+                // a copy covers 8 activation rows; with at most 32 live rows the upper half of the tile is never
+                // read (only where no copy count is kept: RING 2 waits for every copy)
+                if (RING == 2 && T.m_rows <= 32 && (wave + NW * i) * 8 >= 32) continue;
                 copy16_to_lds(xrs, dst + e * kXTile + (wave + NW * i) * 1024, kt < nkt ? T.x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
+            }
         }
     };
     auto issue_w = [&](const FewRowsTile<NW>& T, int s) {            // super-tile s -> buffer s % RING
@@ -747,43 +752,66 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
-        for (int p = 0; p < npair; ++p) {
-            const int s = p / HPS, e0 = (p % HPS) * 2;           // super-tile and first k-tile inside it
-            const uint8_t* raw = rbuf + (s % RING) * RT + my_raw;
-            const uint8_t* xs = xbuf + (p % RING) * kXPair;
-            uint32_t r[2][G::kRegs];
-            half8_t a[2][4][TM];
+        // tiles with at most 32 live rows skip the upper 32 x 32 accumulator block (its copies, LDS reads and MFMAs)
+        auto run = [&](auto rows_tag) {
+            constexpr int TMX = decltype(rows_tag)::value;
+            for (int p = 0; p < npair; ++p) {
+                const int s = p / HPS, e0 = (p % HPS) * 2;           // super-tile and first k-tile inside it
+                const uint8_t* raw = rbuf + (s % RING) * RT + my_raw;
+                const uint8_t* xs = xbuf + (p % RING) * kXPair;
+                uint32_t r[2][G::kRegs];
+                half8_t a[2][4][TMX];
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                G::fetch(raw, e0 + e, h, T.my_delta, r[e]);
+                for (int e = 0; e < 2; ++e) {
+#ifdef TSHIP_FR_NOFETCH
+                    _Pragma("unroll") for (int q = 0; q < G::kRegs; ++q) r[e][q] = 0x3c003c00u + q + p;
+#else
+                    G::fetch(raw, e0 + e, h, T.my_delta, r[e]);
+#endif
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
+                    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-                    for (int i = 0; i < TM; ++i)
-                        a[e][ks][i] = *reinterpret_cast<const half8_t*>(xs + e * kXTile + i * 32 * kXRow + a_off[ks]);
-            }
-            // Requests RING - 1 iterations / super-tiles ahead, activations first (the counted wait below
-            // then never has to cover a weight super-tile younger than one iteration).
-            issue_x(T, p + RING - 1);
-            if (HPS == 1 || (p & 1) == 0) issue_w(T, s + RING - 1);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                uint32_t o[16];
-                G::dequant(r[e], e0 + e, h, T.my_delta, ((2 * p + e) * 2 + h) * 32 < A.K, o);
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks) {
-                    const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
-                    const half8_t b = __builtin_bit_cast(half8_t, bb);
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[e][ks][i], b, acc[i], 0, 0, 0);
+                        for (int i = 0; i < TMX; ++i)
+                            a[e][ks][i] = *reinterpret_cast<const half8_t*>(xs + e * kXTile + i * 32 * kXRow + a_off[ks]);
                 }
+                // Requests RING - 1 iterations / super-tiles ahead, activations first (the counted wait below
+                // then never has to cover a weight super-tile younger than one iteration).
+#ifndef TSHIP_FR_NOX
+                issue_x(T, p + RING - 1);
+#endif
+#ifndef TSHIP_FR_NOW
+                if (HPS == 1 || (p & 1) == 0) issue_w(T, s + RING - 1);
+#endif
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    uint32_t o[16];
+#ifdef TSHIP_FR_NODEQ
+                    _Pragma("unroll") for (int q = 0; q < 16; ++q) o[q] = r[e][q % G::kRegs];
+#else
+                    G::dequant(r[e], e0 + e, h, T.my_delta, ((2 * p + e) * 2 + h) * 32 < A.K, o);
+#endif
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) {
+                        const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
+                        const half8_t b = __builtin_bit_cast(half8_t, bb);
+#pragma unroll
+                        for (int i = 0; i < TMX; ++i)
+#ifdef TSHIP_FR_NOMMA
+                            acc[i][0] += (float)a[e][ks][i][0] * (float)b[0];
+#else
+                            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[e][ks][i], b, acc[i], 0, 0, 0);
+#endif
+                    }
+                }
+                // RING 3: this iteration's activation copies and the youngest weight super-tile may stay in flight
+                if constexpr (RING == 2) wait_copies_and_barrier<0>();
+                else if (five) wait_copies_and_barrier<2 * XI + WI>();
+                else wait_copies_and_barrier<2 * XI + WI - 1>();
             }
-            // RING 3: this iteration's activation copies and the youngest weight super-tile may stay in flight
-            if constexpr (RING == 2) wait_copies_and_barrier<0>();
-            else if (five) wait_copies_and_barrier<2 * XI + WI>();
-            else wait_copies_and_barrier<2 * XI + WI - 1>();
-        }
+        };
+        if (RING == 2 && T.m_rows <= 32) run(std::integral_constant<int, 1>{});
+        else run(std::integral_constant<int, TM>{});
 
         // The next tile's first requests go out before this tile's results are stored, so their latency
         // is covered by the epilogue (every wavefront is past its last LDS read of this tile).
