@@ -778,7 +778,10 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
         hipStream_t stream = g_stream.load();
         auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
         const bool small = A <= gemv_max_group() && H <= gemv_max_k(ggml_type) && F <= gemv_max_k(ggml_type);
-        const int bm = (A / E) > 96 ? 128 : 64;
+        // rows per tile of the grouped GEMMs: with few tokens per expert the 32-row register-resident kernel
+        // streams the weights fastest, even though experts with 33..64 rows then take two tiles
+        const int per_expert = A / E;
+        const int bm = per_expert > 96 ? 128 : per_expert > 40 ? 64 : 32;
         const int max_tiles = A / bm + E;
         // carve the workspace
         size_t off = 0;

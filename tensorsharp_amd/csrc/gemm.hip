@@ -5,7 +5,8 @@
 //      magnitude overflows or underflows fp16), written in the k-order in which the weight
 //      format unpacks (so the dequantizer never has to shuffle lanes), zero-padded to a
 //      multiple of the k-tile.  Optionally gathers rows through an index (MoE).
-//   2. gemm_kernel (M > 64 per tile) / gemm_few_rows_kernel (M <= 64 per tile, persistent workgroups):
+//   2. gemm_kernel (M > 64 per tile) / gemm_few_rows_kernel (M <= 64 per tile, persistent workgroups) /
+//      gemm_slim_kernel (M <= 32 per tile and K <= 4096: activations in registers, K split over the wavefronts):
 //      BM x 256 x 64 tiles, eight wavefronts, each owning 32 output columns.  The fp16
 //      activation k-tiles and the RAW quantized bytes of 256 weight rows (one 144-byte window per row
 //      covering four k-tiles of Q4_K / MXFP4 or two of Q8_0) are copied from global memory straight
@@ -195,6 +196,9 @@ struct GQ4K {
     static constexpr int kRegs = 8;
     static constexpr int kSup = 4;            // one 256-element super-block
     static constexpr int kSupBytes = 144;
+    static constexpr int kTileBytes = 36;     // bytes of one k-tile of a row
+    static constexpr int kSlack = 0;          // bytes fetch() may touch past the last k-tile of a window
+    static constexpr bool kSuperBlocks = true;   // fetch() addresses a k-tile through its super-block header
     static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t /*delta*/, uint32_t (&r)[kRegs])
     {
         const uint4_t hdr = *reinterpret_cast<const uint4_t*>(rp);
@@ -234,6 +238,9 @@ struct GMXFP4 {
     static constexpr int kRegs = 5;
     static constexpr int kSup = 4;            // eight 17-byte blocks
     static constexpr int kSupBytes = 136;
+    static constexpr int kTileBytes = 34;
+    static constexpr int kSlack = 6;
+    static constexpr bool kSuperBlocks = false;
     static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t delta, uint32_t (&r)[kRegs])
     {
         const uint32_t off = delta + (uint32_t)(2 * j + h) * 17u;
@@ -275,6 +282,9 @@ struct GQ80 {
     static constexpr int kRegs = 9;
     static constexpr int kSup = 2;            // four 34-byte blocks
     static constexpr int kSupBytes = 136;
+    static constexpr int kTileBytes = 68;
+    static constexpr int kSlack = 4;
+    static constexpr bool kSuperBlocks = false;
     static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t delta, uint32_t (&r)[kRegs])
     {
         const uint32_t off = delta + (uint32_t)(2 * j + h) * 34u;
@@ -840,9 +850,246 @@ bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
     return hip_ok(hipGetLastError(), "gemm launch");
 }
 
+// ------------------------------------------------------------------------------------------
+// At most 32 activation rows per tile and K of at most 64 k-tiles * 8 (small batches, MoE experts with few
+// tokens).  The activations stay in REGISTERS: the eight wavefronts of a workgroup split K between them
+// (KTW k-tiles each), every wavefront keeps the MFMA A operands of its K range for all 32 rows, and the
+// workgroup walks over 32-column weight tiles.  Per tile a wavefront needs only its own K range of the 32
+// raw weight rows, which it copies itself (global -> LDS, two private buffers, requested two tiles ahead),
+// so the main loop has no barrier and no activation traffic at all; the eight partial 32 x 32 sums meet in
+// LDS (in the raw buffer the wavefront has just consumed), are added in a fixed order and stored.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// LDS layout of one wavefront of the register-resident kernel: RING raw buffers of 32 rows x CH 16-byte chunks
+// (the bytes of KTW k-tiles plus the up to three bytes between the 4-byte aligned window start and the first
+// block; the unpackers may read a few bytes further, into the next row, and ignore them)
+template <typename G, int KTW>
+struct SlimLayout {
+    static constexpr int CH = (KTW * G::kTileBytes + (G::kSlack ? 3 : 0) + 15) / 16;
+    static constexpr int DI = (32 * CH + 63) / 64;                       // LDS-direct copies per buffer
+    static constexpr int RAW = 32 * CH * 16;
+    static constexpr int BUF = RAW > 4096 ? RAW : 4096;                  // raw rows, later the 32 x 32 fp32 partial sums
+    static constexpr int RING = 8 * 3 * BUF + 1024 <= 160 * 1024 ? 3 : 2;
+};
+
+template <typename G, int KTW>
+__global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
+{
+    using L = SlimLayout<G, KTW>;
+    constexpr int CH = L::CH, DI = L::DI, BUF = L::BUF, RING = L::RING;
+    static_assert(!G::kSuperBlocks || KTW % G::kSup == 0, "a wavefront's K range must start at a super-block");
+    extern __shared__ uint8_t smem[];                                   // 8 wavefronts x RING x BUF
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, h = lane >> 5;
+    uint8_t* const my_buf = smem + wave * RING * BUF;
+
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int nkt = A.Kp / kBK;
+    const int kt0 = wave * KTW;
+    const int kcnt = max(0, min(KTW, nkt - kt0));                      // k-tiles of this wavefront
+    const int n32 = (A.N + 31) >> 5;
+
+    // grouped launches: the table may end in empty tiles
+    int live_tiles = A.m_tiles;
+    if (A.tile_expert) {
+        int c = 0;
+        for (int i = lane; i < A.m_tiles; i += 64) c += A.tile_rows[i] > 0 ? 1 : 0;
+        for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+        live_tiles = __builtin_amdgcn_readfirstlane(c);
+    }
+    // units = (row tile, 32-column tile), row tile major; every workgroup takes one contiguous run
+    const int64_t units = (int64_t)live_tiles * n32;
+    int u = (int)(units * blockIdx.x / gridDim.x);
+    const int u_end = (int)(units * (blockIdx.x + 1) / gridDim.x);
+
+    while (u < u_end) {
+        const int mt = u / n32, nt0 = u - mt * n32, cnt = min(n32 - nt0, u_end - u);
+        u += cnt;
+        int m0, m_rows;
+        const uint8_t* wbase = A.w;
+        if (A.tile_expert) {
+            m0 = A.tile_row0[mt];
+            m_rows = min(32, A.tile_rows[mt]);
+            wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+        } else {
+            m0 = mt * 32;
+            m_rows = min(32, A.M - m0);
+        }
+        const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
+        const uint32_t base_delta = (uint32_t)(wa & 3);
+        const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+            reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
+
+        // MFMA A operands of this wavefront's K range: row `col`, k-half h of every k-step
+        half8_t a[KTW][4];
+        {
+            const _Float16* xr = A.x16 + (int64_t)(m0 + min(col, m_rows - 1)) * A.Kp + h * 8;
+            const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < KTW; ++t) {
+                const int kt = min(kt0 + t, nkt - 1);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    const half8_t v = *reinterpret_cast<const half8_t*>(xr + kt * kBK + ks * 16);
+                    a[t][ks] = (col < m_rows && t < kcnt) ? v : zero;
+                }
+            }
+        }
+        // Source offsets of the raw copies.  32 rows are a multiple of four bytes, so a row's alignment
+        // inside its window is the same in every column tile.
+        const uint32_t koff = (uint32_t)kt0 * G::kTileBytes;
+        uint32_t w_off[DI];
+#pragma unroll
+        for (int i = 0; i < DI; ++i) {
+            const int q = i * 64 + lane;
+            const int row = q / CH, chunk = q - row * CH;
+            w_off[i] = (row < 32 && kcnt > 0) ? ((base_delta + (uint32_t)row * row_bytes + koff) & ~3u) + (uint32_t)chunk * 16u : kDeadOffset;
+        }
+        const uint32_t my_delta = (base_delta + (uint32_t)col * row_bytes + koff) & 3u;
+        auto issue = [&](int i, int b) {                // column tile nt0 + i -> buffer b
+            uint8_t* dst = my_buf + b * BUF;
+            const bool any = i < cnt;
+            const uint32_t so = any ? (uint32_t)(nt0 + i) * 32u * row_bytes : 0u;
+#pragma unroll
+            for (int q = 0; q < DI; ++q) {
+                // an odd number of chunks per row leaves the last copy half full: its upper lanes stay out (they would
+                // write into the next buffer)
+                if (q * 64 + 32 < 32 * CH || lane < 32) copy16_to_lds(wrs, dst + q * 1024, any ? w_off[q] : kDeadOffset, so);
+            }
+        };
+        // result rows of this thread in the reduction: accumulator registers `wave` and `wave + 8`
+        float sc[2];
+        int64_t coff[2];
+        bool ok[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int r = wave + 8 * q;
+            const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
+            const int m = m0 + min(ml, m_rows - 1);
+            sc[q] = A.xscale[m];
+            coff[q] = (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
+            ok[q] = ml < m_rows;
+        }
+
+#pragma unroll
+        for (int b = 0; b < RING; ++b) issue(b, b);
+        int b = 0;                                      // buffer of column tile i
+        float pend[2] = {0.f, 0.f};
+        int pend_n = -1;
+        auto flush = [&]() {
+            if (pend_n >= 0 && pend_n < A.N) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+                    if (ok[q]) A.c[coff[q] + pend_n] = pend[q];
+            }
+        };
+        for (int i = 0; i < cnt; ++i) {
+            // the copies of tile i have landed; those of the RING - 1 tiles after it stay in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RING - 1) * DI) : "memory");
+            // the previous tile's results leave here, after the wait: a store in flight at the wait would be
+            // counted against it
+            flush();
+            float16_t acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            const uint8_t* raw = my_buf + b * BUF + col * (CH * 16);
+            // a wavefront with a full K range runs the k-tiles as one branch-free block, so the unpacking of one
+            // k-tile is scheduled into the matrix instructions of the previous one
+            auto k_tiles = [&](auto full_tag) {
+                constexpr bool kFull = decltype(full_tag)::value;
+#pragma unroll
+                for (int t = 0; t < KTW; ++t) {
+                    if (kFull || t < kcnt) {
+                        uint32_t r[G::kRegs], o[16];
+                        if constexpr (G::kSuperBlocks) G::fetch(raw + (t / G::kSup) * G::kSupBytes, t % G::kSup, h, my_delta, r);
+                        else G::fetch(raw, t, h, my_delta, r);
+                        G::dequant(r, G::kSuperBlocks ? t % G::kSup : t, h, my_delta, ((kt0 + t) * 2 + h) * 32 < A.K, o);
+#pragma unroll
+                        for (int ks = 0; ks < 4; ++ks) {
+                            const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
+                            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][ks], __builtin_bit_cast(half8_t, bb), acc, 0, 0, 0);
+                        }
+                    }
+                }
+            };
+            if (kcnt == KTW) k_tiles(std::true_type{});
+            else k_tiles(std::false_type{});
+            // partial sums of this wavefront's K range -> the buffer it has just consumed
+            float* part = reinterpret_cast<float*>(my_buf + b * BUF);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) part[r * 64 + lane] = acc[r];
+            lds_barrier();
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float* pv = reinterpret_cast<const float*>(smem + (v * RING + b) * BUF);
+                s0 += pv[wave * 64 + lane];
+                s1 += pv[(wave + 8) * 64 + lane];
+            }
+            pend[0] = s0 * sc[0];
+            pend[1] = s1 * sc[1];
+            pend_n = (nt0 + i) * 32 + col;
+            lds_barrier();                              // every partial sum has been read: the buffers may be refilled
+            issue(i + RING, b);
+            b = b + 1 == RING ? 0 : b + 1;
+        }
+        flush();
+    }
+}
+
+template <typename G, int KTW>
+bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream)
+{
+    using L = SlimLayout<G, KTW>;
+    auto kern = gemm_slim_kernel<G, KTW>;
+    const size_t lds = (size_t)8 * L::RING * L::BUF + 64;     // the unpackers may read a few bytes past the last row
+    static_assert((size_t)8 * L::RING * L::BUF + 64 <= 160 * 1024, "raw buffers must fit LDS");
+    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + 31) / 32;
+    const int64_t units = (int64_t)m_tiles * a.n_tiles;
+    const int grid = (int)std::min<int64_t>(units, device_info().num_cus);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
+    return hip_ok(hipGetLastError(), "gemm launch");
+}
+
+// k-tiles per wavefront for which the register-resident kernel is built (0: K too long for it)
+template <typename G>
+int slim_ktw(int nkt)
+{
+    const int need = (nkt + 7) / 8;
+    constexpr int kStep = G::kSuperBlocks ? G::kSup : 2;
+    constexpr int kMax = G::kTileBytes > 40 ? 4 : 8;       // LDS: 16 raw buffers of 32 rows
+    const int ktw = (need + kStep - 1) / kStep * kStep;
+    return ktw <= kMax ? ktw : 0;
+}
+
+template <typename G>
+bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream)
+{
+    if constexpr (!G::kSuperBlocks) {
+        if (ktw == 2) return launch_slim<G, 2>(a, m_tiles, stream);
+        if constexpr (G::kTileBytes <= 40)
+            if (ktw == 6) return launch_slim<G, 6>(a, m_tiles, stream);
+    }
+    if (ktw == 4) return launch_slim<G, 4>(a, m_tiles, stream);
+    if constexpr (G::kTileBytes <= 40)
+        if (ktw == 8) return launch_slim<G, 8>(a, m_tiles, stream);
+    set_last_error("gemm: no register-resident kernel for this K.");
+    return false;
+}
+
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
+    if (bm == 32) {
+        const int ktw = a.accumulate ? 0 : slim_ktw<G>(a.Kp / kBK);
+        if (ktw) return launch_slim_for<G>(a, ktw, m_tiles, stream);
+        // longer K: the 64-row kernel takes 32-row tiles as half-empty ones
+    }
     if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
     // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
     // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 the other way round
@@ -866,7 +1113,7 @@ size_t gemm_workspace_bytes(int M, int K)
     return (size_t)M * kp * sizeof(_Float16) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255) + 256;
 }
 
-int gemm_tile_m(int M) { return M > 1024 ? 256 : M > 64 ? 128 : 64; }
+int gemm_tile_m(int M) { return M > 1024 ? 256 : M > 64 ? 128 : M > 32 ? 64 : 32; }
 
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
                       hipStream_t stream, const float* norm_w, float eps)

@@ -134,3 +134,27 @@ def test_weight_view_at_odd_address(hip, oracle, name, row_bytes, M):
     y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(sub, T[name], K, N - 1))
     torch.cuda.synchronize()
     check(y.cpu().numpy(), oracle.matmul_f64(T[name], wq[row_bytes:], N - 1, K, x), (name, M))
+
+
+@pytest.mark.parametrize("name,M,N,K", [
+    ("mxfp4", 32, 5000, 2880),    # six k-tiles per wavefront, three raw buffers, half-filled last copy
+    ("mxfp4", 17, 9001, 4096),    # eight k-tiles per wavefront, two raw buffers
+    ("mxfp4", 5, 3000, 1024),     # two k-tiles per wavefront
+    ("mxfp4", 31, 2000, 2048),    # four
+    ("mxfp4", 9, 1500, 4160),     # K too long for the register-resident kernel: 64-row kernel
+    ("q4_k", 32, 9000, 2048),
+    ("q4_k", 12, 14336, 4096),
+    ("q4_k", 20, 1000, 4352),     # too long
+    ("q4_k", 6, 333, 256),        # a single k-tile group: seven of the eight wavefronts have no K range
+    ("q8_0", 32, 3000, 1024),
+    ("q8_0", 11, 7000, 2048),
+    ("q8_0", 25, 900, 2080),      # too long
+    ("q8_0", 4, 40, 32),          # one block per row
+])
+def test_at_most_32_rows(hip, oracle, name, M, N, K):
+    # M <= 32: the activations stay in registers and the wavefronts of a workgroup split K
+    rng = np.random.default_rng(M * 17 + N + K)
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, T[name], wq, N, K, x)
+    check(y, oracle.matmul_f64(T[name], wq, N, K, x), (name, M, N, K))
