@@ -790,11 +790,10 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
         const size_t o_pos = take((size_t)A * 4), o_te = take((size_t)max_tiles * 4), o_tr0 = take((size_t)max_tiles * 4);
         const size_t o_trn = take((size_t)max_tiles * 4);
         const size_t o_ws1 = take(gemm_workspace_bytes(A, (int)H)), o_ws2 = take(gemm_workspace_bytes(A, (int)F));
-        const size_t o_gu = take((size_t)A * 2 * F * 4), o_act = take((size_t)A * F * 4), o_dn = take((size_t)A * H * 4);
+        const size_t o_gu = take((size_t)A * 2 * F * 4), o_dn = take((size_t)A * H * 4);
         char* ws = static_cast<char*>(dev_ws_reserve(off));
         if (!ws) return 0;
         float* gu = reinterpret_cast<float*>(ws + o_gu);
-        float* act = reinterpret_cast<float*>(ws + o_act);
         float* dn = reinterpret_cast<float*>(ws + o_dn);
         const float* hid = static_cast<const float*>(hidden.data);
         if (small) {
@@ -827,8 +826,9 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
             if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream)) return 0;
             if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream))
                 return 0;
-            if (!launch_moe_swiglu(gu, gate_up_bias, maps.expert_of, A, (int)F, alpha, limit, act, stream)) return 0;
-            if (!launch_convert_x(ggml_type, act, F, nullptr, A, (int)F, ws + o_ws2, stream)) return 0;
+            // bias + SwiGLU-OAI are formed while the down projection's activations are converted
+            if (!launch_convert_x_swiglu(ggml_type, gu, gate_up_bias, maps.expert_of, alpha, limit, A, (int)F, ws + o_ws2, stream))
+                return 0;
             tiles.expert_stride = dn_bytes;
             if (!launch_gemm(ggml_type, down_w, dn_bytes, ws + o_ws2, dn, H, nullptr, A, (int)H, (int)F, &tiles, stream)) return 0;
             if (!launch_moe_combine(dn, down_bias, ids, weights, maps.pos_of, T, k, (int)H, false,

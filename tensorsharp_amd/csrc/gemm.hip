@@ -100,26 +100,66 @@ __device__ __forceinline__ int k_slot(int k)
 // ------------------------------------------------------------------------------------------
 // activations: fp32 [M x K] (row stride ldx) -> fp16 [M x Kp] in unpack order, per-row scale
 // ------------------------------------------------------------------------------------------
-constexpr int kCvtThreads = 1024;
-constexpr int kCvtHold = 8;      // float4 per thread kept in registers: rows up to 32768 elements are read once
+constexpr int kCvtHold = 8;      // float4 per thread kept in registers: rows up to THREADS * 32 elements are read once
 
-template <int TYPE>
-__global__ void __launch_bounds__(kCvtThreads) convert_x_kernel(const float* __restrict__ x, int64_t ldx, const int* __restrict__ row_map,
-                                                                int K, int Kp, _Float16* __restrict__ out, float* __restrict__ scales,
-                                                                const float* __restrict__ norm_w, float eps)
+// How a row of activations is formed while it is read.
+struct ConvertSrc {
+    const float* x;          // rows (kSrcSwiglu: gate | up rows of 2 K floats)
+    int64_t ldx;
+    const int* row_map;      // optional gather: source row of activation row m
+    const float* norm_w;     // kSrcPlain: optional RMSNorm weight
+    float eps;
+    const float* bias;       // kSrcSwiglu: optional [experts x 2 K] bias, picked through expert_of
+    const int* expert_of;
+    float alpha, limit;
+};
+constexpr int kSrcPlain = 0, kSrcSwiglu = 1;
+
+// SwiGLU of the gpt-oss experts (ggml-cpu/ops.cpp swiglu_oai: x = min(gate, limit), y = clamp(up, +-limit),
+// x / (1 + exp(-alpha x)) * (y + 1))
+__device__ __forceinline__ float swiglu_oai(float gate, float up, float alpha, float limit)
+{
+    const float x = fminf(gate, limit);
+    const float y = fminf(fmaxf(up, -limit), limit);
+    return x / (1.0f + expf(alpha * (-x))) * (y + 1.0f);
+}
+
+template <int TYPE, int THREADS, int SRC>
+__global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, int K, int Kp, _Float16* __restrict__ out,
+                                                            float* __restrict__ scales)
 {
     const int m = blockIdx.x;
     const int tid = threadIdx.x;
-    const float* src = x + (int64_t)(row_map ? row_map[m] : m) * ldx;
-    __shared__ float red[kCvtThreads / 64];
-    __shared__ double redd[kCvtThreads / 64];
+    const float* src = S.x + (int64_t)(S.row_map ? S.row_map[m] : m) * S.ldx;
+    const float* norm_w = SRC == kSrcPlain ? S.norm_w : nullptr;
+    const float* bias = (SRC == kSrcSwiglu && S.bias) ? S.bias + (int64_t)S.expert_of[m] * 2 * K : nullptr;
+    __shared__ float red[THREADS / 64];
+    __shared__ double redd[THREADS / 64];
     const int k4 = K >> 2;                       // K is a multiple of 32
-    constexpr int kHeld = kCvtHold * kCvtThreads * 4;
+    constexpr int kHeld = kCvtHold * THREADS * 4;
+    // element k of the row as it enters the product (before the optional RMSNorm)
+    auto raw4 = [&](int q) -> float4 {
+        if (SRC == kSrcSwiglu) {
+            float4 g = reinterpret_cast<const float4*>(src)[q], u = reinterpret_cast<const float4*>(src + K)[q];
+            if (bias) {
+                const float4 bg = reinterpret_cast<const float4*>(bias)[q], bu = reinterpret_cast<const float4*>(bias + K)[q];
+                g = float4{g.x + bg.x, g.y + bg.y, g.z + bg.z, g.w + bg.w};
+                u = float4{u.x + bu.x, u.y + bu.y, u.z + bu.z, u.w + bu.w};
+            }
+            return float4{swiglu_oai(g.x, u.x, S.alpha, S.limit), swiglu_oai(g.y, u.y, S.alpha, S.limit),
+                          swiglu_oai(g.z, u.z, S.alpha, S.limit), swiglu_oai(g.w, u.w, S.alpha, S.limit)};
+        }
+        return reinterpret_cast<const float4*>(src)[q];
+    };
+    auto raw1 = [&](int k) -> float {
+        if (SRC == kSrcSwiglu) return swiglu_oai(src[k] + (bias ? bias[k] : 0.f), src[K + k] + (bias ? bias[K + k] : 0.f), S.alpha, S.limit);
+        return src[k];
+    };
     float4 hold[kCvtHold];
 #pragma unroll
     for (int i = 0; i < kCvtHold; ++i) {
-        const int q = tid + i * kCvtThreads;
-        hold[i] = q < k4 ? reinterpret_cast<const float4*>(src)[q] : float4{0.f, 0.f, 0.f, 0.f};
+        const int q = tid + i * THREADS;
+        hold[i] = q < k4 ? raw4(q) : float4{0.f, 0.f, 0.f, 0.f};
     }
     // optional RMSNorm prologue (ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1/sqrtf(mean + eps),
     // then the multiply by the norm weight: (x * scale) * w)
@@ -130,35 +170,35 @@ __global__ void __launch_bounds__(kCvtThreads) convert_x_kernel(const float* __r
         for (int i = 0; i < kCvtHold; ++i)
             ss += (double)(hold[i].x * hold[i].x) + (double)(hold[i].y * hold[i].y) + (double)(hold[i].z * hold[i].z) +
                   (double)(hold[i].w * hold[i].w);
-        for (int k = kHeld + tid; k < K; k += kCvtThreads) ss += (double)(src[k] * src[k]);
+        for (int k = kHeld + tid; k < K; k += THREADS) ss += (double)(src[k] * src[k]);
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
         if ((tid & 63) == 0) redd[tid >> 6] = ss;
         __syncthreads();
         double tot = 0.0;
 #pragma unroll
-        for (int i = 0; i < kCvtThreads / 64; ++i) tot += redd[i];
-        rms = 1.0f / sqrtf((float)(tot / (double)K) + eps);
+        for (int i = 0; i < THREADS / 64; ++i) tot += redd[i];
+        rms = 1.0f / sqrtf((float)(tot / (double)K) + S.eps);
 #pragma unroll
         for (int i = 0; i < kCvtHold; ++i) {
-            const int q = tid + i * kCvtThreads;
+            const int q = tid + i * THREADS;
             if (q < k4) {
                 const float4 wv = reinterpret_cast<const float4*>(norm_w)[q];
                 hold[i] = float4{(hold[i].x * rms) * wv.x, (hold[i].y * rms) * wv.y, (hold[i].z * rms) * wv.z, (hold[i].w * rms) * wv.w};
             }
         }
     }
-    auto tail_value = [&](int k) { return norm_w ? (src[k] * rms) * norm_w[k] : src[k]; };
+    auto tail_value = [&](int k) { return norm_w ? (src[k] * rms) * norm_w[k] : raw1(k); };
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < kCvtHold; ++i)
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(hold[i].x), fabsf(hold[i].y)), fmaxf(fabsf(hold[i].z), fabsf(hold[i].w))));
-    for (int k = kHeld + tid; k < K; k += kCvtThreads) amax = fmaxf(amax, fabsf(tail_value(k)));
+    for (int k = kHeld + tid; k < K; k += THREADS) amax = fmaxf(amax, fabsf(tail_value(k)));
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
     amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < kCvtThreads / 64; ++i) amax = fmaxf(amax, red[i]);
+    for (int i = 0; i < THREADS / 64; ++i) amax = fmaxf(amax, red[i]);
     // power-of-two scale bringing amax into [2^13, 2^14)
     int e = (int)((__float_as_uint(amax) >> 23) & 0xffu);
     if (e == 255) e = 127;
@@ -170,7 +210,7 @@ __global__ void __launch_bounds__(kCvtThreads) convert_x_kernel(const float* __r
     auto put = [&](int k, float v) { dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)(v * inv); };
 #pragma unroll
     for (int i = 0; i < kCvtHold; ++i) {
-        const int q = tid + i * kCvtThreads;
+        const int q = tid + i * THREADS;
         if (q < k4) {
             put(4 * q, hold[i].x);
             put(4 * q + 1, hold[i].y);
@@ -178,8 +218,8 @@ __global__ void __launch_bounds__(kCvtThreads) convert_x_kernel(const float* __r
             put(4 * q + 3, hold[i].w);
         }
     }
-    for (int k = kHeld + tid; k < K; k += kCvtThreads) put(k, tail_value(k));
-    for (int k = K + tid; k < Kp; k += kCvtThreads) dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)0.f;
+    for (int k = kHeld + tid; k < K; k += THREADS) put(k, tail_value(k));
+    for (int k = K + tid; k < Kp; k += THREADS) dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)0.f;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1115,19 +1155,58 @@ size_t gemm_workspace_bytes(int M, int K)
 
 int gemm_tile_m(int M) { return M > 1024 ? 256 : M > 64 ? 128 : M > 32 ? 64 : 32; }
 
-bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
-                      hipStream_t stream, const float* norm_w, float eps)
+namespace {
+
+template <int TYPE, int SRC>
+void launch_convert_typed(const ConvertSrc& src, int M, int K, int kp, _Float16* x16, float* scales, hipStream_t stream)
+{
+    // short rows: 256 threads hold the whole row and eight workgroups share a CU
+    if (K <= 256 * kCvtHold * 4)
+        hipLaunchKernelGGL((convert_x_kernel<TYPE, 256, SRC>), dim3(M), dim3(256), 0, stream, src, K, kp, x16, scales);
+    else
+        hipLaunchKernelGGL((convert_x_kernel<TYPE, 1024, SRC>), dim3(M), dim3(1024), 0, stream, src, K, kp, x16, scales);
+}
+
+template <int SRC>
+bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspace, hipStream_t stream)
 {
     const int kp = (K + kBK - 1) / kBK * kBK;
     float* scales = static_cast<float*>(workspace);
     _Float16* x16 = reinterpret_cast<_Float16*>(static_cast<char*>(workspace) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
     switch (type) {
-    case kTypeQ4_K: hipLaunchKernelGGL(convert_x_kernel<kTypeQ4_K>, dim3(M), dim3(kCvtThreads), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
-    case kTypeMXFP4: hipLaunchKernelGGL(convert_x_kernel<kTypeMXFP4>, dim3(M), dim3(kCvtThreads), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
-    case kTypeQ8_0: hipLaunchKernelGGL(convert_x_kernel<kTypeQ8_0>, dim3(M), dim3(kCvtThreads), 0, stream, x, ldx, row_map, K, kp, x16, scales, norm_w, eps); break;
+    case kTypeQ4_K: launch_convert_typed<kTypeQ4_K, SRC>(src, M, K, kp, x16, scales, stream); break;
+    case kTypeMXFP4: launch_convert_typed<kTypeMXFP4, SRC>(src, M, K, kp, x16, scales, stream); break;
+    case kTypeQ8_0: launch_convert_typed<kTypeQ8_0, SRC>(src, M, K, kp, x16, scales, stream); break;
     default: set_last_error("gemm: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "activation convert launch");
+}
+
+}  // namespace
+
+bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
+                      hipStream_t stream, const float* norm_w, float eps)
+{
+    ConvertSrc src{};
+    src.x = x;
+    src.ldx = ldx;
+    src.row_map = row_map;
+    src.norm_w = norm_w;
+    src.eps = eps;
+    return launch_convert<kSrcPlain>(type, src, M, K, workspace, stream);
+}
+
+bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, const int* expert_of, float alpha, float limit,
+                             int M, int F, void* workspace, hipStream_t stream)
+{
+    ConvertSrc src{};
+    src.x = gate_up;
+    src.ldx = 2 * (int64_t)F;
+    src.bias = bias;
+    src.expert_of = expert_of;
+    src.alpha = alpha;
+    src.limit = limit;
+    return launch_convert<kSrcSwiglu>(type, src, M, F, workspace, stream);
 }
 
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,

@@ -11,6 +11,7 @@ namespace tship {
 namespace {
 
 constexpr int kMaxK = 16;
+constexpr int kGroupLdsIds = 8192;     // assignments whose ids the grouping kernel keeps in LDS (32 KiB)
 
 // one wavefront per token
 __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__ logits, int64_t ld, int E, int k,
@@ -75,33 +76,54 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const float* __restrict__
         }
 }
 
-// single workgroup: histogram, exclusive scan, stable placement (one wavefront per expert at a time), tile table
+// single workgroup: histogram, exclusive scan, placement, tile table
 __global__ void __launch_bounds__(1024) moe_group_kernel(const int* __restrict__ ids, int A, int k, int E, int bm, int max_tiles,
                                                          MoeMaps M)
 {
-    extern __shared__ int sh[];      // cnt[E], off[E + 1], tbeg[E + 1]
+    extern __shared__ int sh[];      // cnt[E], off[E + 1], tbeg[E + 1], then a copy of the ids if it fits
     int* cnt = sh;
     int* off = sh + E;
     int* tbeg = sh + 2 * E + 1;
+    int* ids_lds = sh + 3 * E + 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+    const bool in_lds = A <= kGroupLdsIds;       // the placement pass below reads every id once per expert
     for (int e = tid; e < E; e += blockDim.x) cnt[e] = 0;
     __syncthreads();
     for (int i = tid; i < A; i += blockDim.x) {
         const int e = ids[i];
+        if (in_lds) ids_lds[i] = e;
         if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
         else M.pos_of[i] = -1;
     }
     __syncthreads();
-    if (tid == 0) {
-        int o = 0, tb = 0;
-        for (int e = 0; e < E; ++e) {
-            off[e] = o;
-            tbeg[e] = tb;
-            o += cnt[e];
-            tb += (cnt[e] + bm - 1) / bm;
+    // exclusive scans of the row counts and of the tile counts: one wavefront, 64 experts per step
+    const int bm_shift = __ffs(bm) - 1;          // bm is a power of two
+    if (wave == 0) {
+        int carry_o = 0, carry_t = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int c = e < E ? cnt[e] : 0;
+            const int nt = (c + bm - 1) >> bm_shift;
+            int so = c, st = nt;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int vo = __shfl_up(so, d), vt = __shfl_up(st, d);
+                if (lane >= d) {
+                    so += vo;
+                    st += vt;
+                }
+            }
+            if (e < E) {
+                off[e] = carry_o + so - c;
+                tbeg[e] = carry_t + st - nt;
+            }
+            carry_o += __shfl(so, 63);
+            carry_t += __shfl(st, 63);
         }
-        off[E] = o;
-        tbeg[E] = tb;
+        if (lane == 0) {
+            off[E] = carry_o;
+            tbeg[E] = carry_t;
+        }
     }
     __syncthreads();
     for (int e = tid; e <= E; e += blockDim.x) M.offsets[e] = off[e];
@@ -110,91 +132,99 @@ __global__ void __launch_bounds__(1024) moe_group_kernel(const int* __restrict__
         M.tile_row0[j] = 0;
         M.tile_rows[j] = 0;
     }
-    for (int e = wave; e < E; e += nw) {
-        int base = off[e];
-        for (int c = 0; c < A; c += 64) {
-            const int i = c + lane;
-            const bool match = i < A && ids[i] == e;
-            const unsigned long long mask = __ballot(match);
-            if (match) {
-                const int pos = base + __popcll(mask & ((1ull << lane) - 1ull));
-                M.token_of[pos] = i / k;
-                M.expert_of[pos] = e;
-                M.pos_of[i] = pos;
-            }
-            base += __popcll(mask);
+    // Placement: the rows of an expert are handed out by an LDS counter, in no particular order (every result row
+    // depends on its own activation row only, so the order inside an expert does not show in the output).
+    __syncthreads();
+    for (int e = tid; e < E; e += blockDim.x) cnt[e] = 0;            // reused as the fill counters
+    __syncthreads();
+    for (int i = tid; i < A; i += blockDim.x) {
+        const int e = in_lds ? ids_lds[i] : ids[i];
+        if (e >= 0 && e < E) {
+            const int pos = off[e] + atomicAdd(&cnt[e], 1);
+            M.token_of[pos] = i / k;
+            M.expert_of[pos] = e;
+            M.pos_of[i] = pos;
         }
-        const int nt = (cnt[e] + bm - 1) / bm;
+    }
+    for (int e = wave; e < E; e += nw) {
+        const int rows = off[e + 1] - off[e];
+        const int nt = (rows + bm - 1) >> bm_shift;
         for (int j = lane; j < nt; j += 64) {
             M.tile_expert[tbeg[e] + j] = e;
             M.tile_row0[tbeg[e] + j] = off[e] + j * bm;
-            M.tile_rows[tbeg[e] + j] = min(bm, cnt[e] - j * bm);
+            M.tile_rows[tbeg[e] + j] = min(bm, rows - j * bm);
         }
     }
 }
 
-__global__ void __launch_bounds__(256) moe_swiglu_kernel(const float* __restrict__ gu, const float* __restrict__ bias,
-                                                         const int* __restrict__ expert_of, int F, float alpha, float limit,
-                                                         float* __restrict__ act)
-{
-    const int r = blockIdx.y;
-    const int f = blockIdx.x * 256 + threadIdx.x;
-    if (f >= F) return;
-    const float* g = gu + (int64_t)r * 2 * F;
-    float gate = g[f], up = g[F + f];
-    if (bias) {
-        const float* b = bias + (int64_t)expert_of[r] * 2 * F;
-        gate += b[f];
-        up += b[F + f];
-    }
-    const float x = fminf(gate, limit);
-    const float y = fminf(fmaxf(up, -limit), limit);
-    const float glu = x / (1.0f + expf(alpha * (-x)));
-    act[(int64_t)r * F + f] = glu * (y + 1.0f);
-}
-
+// VEC consecutive columns per thread (4: rows and pointers 16-byte aligned)
+template <int VEC>
 __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ dn, const float* __restrict__ bias,
                                                           const int* __restrict__ ids, const float* __restrict__ weights,
                                                           const int* __restrict__ pos_of, int k, int H, int slot_order,
                                                           float* __restrict__ out, int64_t ldo)
 {
     const int t = blockIdx.y;
-    const int h = blockIdx.x * 256 + threadIdx.x;
+    const int h = (blockIdx.x * 256 + threadIdx.x) * VEC;
     if (h >= H) return;
-    int order[kMaxK];
+    // the token's (expert, slot) pairs in registers
+    int id[kMaxK], slot[kMaxK];
 #pragma unroll
-    for (int s = 0; s < kMaxK; ++s) order[s] = s;
+    for (int s = 0; s < kMaxK; ++s) {
+        id[s] = s < k ? ids[(int64_t)t * k + s] : 0x7fffffff;
+        slot[s] = s;
+    }
     if (!slot_order) {
         // ascending expert id, ties in slot order (insertion sort, k <= 16)
 #pragma unroll
         for (int a = 1; a < kMaxK; ++a) {
             if (a < k) {
 #pragma unroll
-                for (int b = kMaxK - 1; b > 0; --b) {
-                    if (b <= a && ids[(int64_t)t * k + order[b]] < ids[(int64_t)t * k + order[b - 1]]) {
-                        const int tmp = order[b];
-                        order[b] = order[b - 1];
-                        order[b - 1] = tmp;
+                for (int b = a; b > 0; --b) {
+                    if (id[b] < id[b - 1]) {
+                        const int ti = id[b], ts = slot[b];
+                        id[b] = id[b - 1];
+                        slot[b] = slot[b - 1];
+                        id[b - 1] = ti;
+                        slot[b - 1] = ts;
                     }
                 }
             }
         }
     }
-    float acc = 0.f;
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
 #pragma unroll
     for (int j = 0; j < kMaxK; ++j) {
         if (j < k) {
-            const int s = order[j];
-            const int64_t a = (int64_t)t * k + s;
+            const int64_t a = (int64_t)t * k + slot[j];
             const int pos = pos_of ? pos_of[a] : (int)a;
             if (pos >= 0) {
-                float v = dn[(int64_t)pos * H + h];
-                if (bias) v += bias[(int64_t)ids[a] * H + h];
-                acc += weights[a] * v;
+                const float w = weights[a];
+                const float* dp = dn + (int64_t)pos * H + h;
+                const float* bp = bias ? bias + (int64_t)id[j] * H + h : nullptr;
+                if constexpr (VEC == 4) {
+                    float4 v = *reinterpret_cast<const float4*>(dp);
+                    if (bp) {
+                        const float4 bv = *reinterpret_cast<const float4*>(bp);
+                        v = float4{v.x + bv.x, v.y + bv.y, v.z + bv.z, v.w + bv.w};
+                    }
+                    acc[0] += w * v.x;
+                    acc[1] += w * v.y;
+                    acc[2] += w * v.z;
+                    acc[3] += w * v.w;
+                } else {
+                    float v = dp[0];
+                    if (bp) v += bp[0];
+                    acc[0] += w * v;
+                }
             }
         }
     }
-    out[(int64_t)t * ldo + h] = acc;
+    float* op = out + (int64_t)t * ldo + h;
+    if constexpr (VEC == 4) *reinterpret_cast<float4*>(op) = float4{acc[0], acc[1], acc[2], acc[3]};
+    else op[0] = acc[0];
 }
 
 }  // namespace
@@ -215,16 +245,9 @@ bool launch_moe_group(const int* ids, int A, int k, int E, int bm, int max_tiles
         set_last_error("moe_group: more than 4096 experts.");
         return false;
     }
-    const size_t lds = (size_t)(3 * E + 2) * sizeof(int);
+    const size_t lds = (size_t)(3 * E + 2 + (A <= kGroupLdsIds ? A : 0)) * sizeof(int);
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), lds, stream, ids, A, k, E, bm, max_tiles, maps);
     return hip_ok(hipGetLastError(), "moe_group launch");
-}
-
-bool launch_moe_swiglu(const float* gu, const float* bias, const int* expert_of, int rows, int F, float alpha, float limit,
-                       float* act, hipStream_t stream)
-{
-    hipLaunchKernelGGL(moe_swiglu_kernel, dim3((F + 255) / 256, rows), dim3(256), 0, stream, gu, bias, expert_of, F, alpha, limit, act);
-    return hip_ok(hipGetLastError(), "moe_swiglu launch");
 }
 
 bool launch_moe_combine(const float* dn, const float* bias, const int* ids, const float* weights, const int* pos_of, int T,
@@ -234,8 +257,14 @@ bool launch_moe_combine(const float* dn, const float* bias, const int* ids, cons
         set_last_error("moe_combine: k > 16.");
         return false;
     }
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((H + 255) / 256, T), dim3(256), 0, stream, dn, bias, ids, weights, pos_of, k, H,
-                       slot_order ? 1 : 0, out, ldo);
+    const bool vec = H % 4 == 0 && ldo % 4 == 0 && ((reinterpret_cast<uintptr_t>(dn) | reinterpret_cast<uintptr_t>(bias) |
+                                                    reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL(moe_combine_kernel<4>, dim3((H / 4 + 255) / 256, T), dim3(256), 0, stream, dn, bias, ids, weights, pos_of, k,
+                           H, slot_order ? 1 : 0, out, ldo);
+    else
+        hipLaunchKernelGGL(moe_combine_kernel<1>, dim3((H + 255) / 256, T), dim3(256), 0, stream, dn, bias, ids, weights, pos_of, k, H,
+                           slot_order ? 1 : 0, out, ldo);
     return hip_ok(hipGetLastError(), "moe_combine launch");
 }
 

@@ -98,6 +98,10 @@ int gemm_tile_m(int M);   // rows of activations per tile for a plain (ungrouped
 // norm_w (device, optional) applies RMSNorm first: x <- x / sqrt(mean(x^2) + eps) * norm_w.
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
                       hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f);
+// The same for the activations of an expert's down projection: row m is SwiGLU-OAI of (gate | up)[m] (+ the bias
+// row of expert_of[m]), formed while it is read.
+bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, const int* expert_of, float alpha, float limit,
+                             int M, int F, void* workspace, hipStream_t stream);
 
 // Grouped launches (MoE): m-tiles enumerated by device tables; weights of expert e start at
 // w + e * expert_stride and span w_bytes each.
@@ -134,11 +138,8 @@ struct MoeMaps {            // all device pointers, A = T * k assignments
     int* tile_row0;         // [max_tiles]
     int* tile_rows;         // [max_tiles], 0 past the last tile
 };
-// stable counting sort of the assignments by expert + m-tile table for the grouped GEMM
+// counting sort of the assignments by expert (row order inside an expert is unspecified) + m-tile table for the grouped GEMM
 bool launch_moe_group(const int* ids, int A, int k, int E, int bm, int max_tiles, const MoeMaps& maps, hipStream_t stream);
-// act[r][f] = swiglu_oai(gu[r][f] + b[e][f], gu[r][F + f] + b[e][F + f]); e = expert_of[r]
-bool launch_moe_swiglu(const float* gu, const float* bias, const int* expert_of, int rows, int F, float alpha, float limit,
-                       float* act, hipStream_t stream);
 // out[t][h] = sum_s w[t][s] * (dn[pos_of[t*k+s]][h] + b[e][h]); order: ascending expert (or slot order)
 bool launch_moe_combine(const float* dn, const float* bias, const int* ids, const float* weights, const int* pos_of, int T,
                         int k, int H, bool slot_order, float* out, int64_t ldo, hipStream_t stream);
