@@ -234,8 +234,13 @@ def main():
                 res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
                             "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)})
             else:
+                # weight-streaming bound (about 120 FLOP per weight byte): bytes of all 32 experts are the figure
+                # of merit, TFLOP/s beside it
+                b = E * (2 * F + H) * row_bytes(MXFP4, H)
                 fl = 2.0 * T * k * (2 * F * H + H * F)
-                res.update({"TFLOPs": round(fl / (us * 1e-6) / 1e12, 1),
+                res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                            "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1),
+                            "TFLOPs": round(fl / (us * 1e-6) / 1e12, 1),
                             "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / 2516.6, 1)})
             return res
 
