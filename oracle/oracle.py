@@ -13,8 +13,13 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 F32, Q8_0, Q4_K, MXFP4 = 0, 8, 12, 39
+F16, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q6_K, IQ4_NL, BF16 = 1, 2, 3, 6, 7, 13, 14, 20, 30
 TYPES = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
-BLOCK = {F32: (1, 4), Q8_0: (32, 34), Q4_K: (256, 144), MXFP4: (32, 17)}
+# formats with a dequantizer only (embedding gather, DequantizeToF32); Q6_K also has matmuls on the GPU
+MORE_TYPES = {"f16": F16, "bf16": BF16, "q4_0": Q4_0, "q4_1": Q4_1, "q5_0": Q5_0, "q5_1": Q5_1, "q5_k": Q5_K,
+              "q6_k": Q6_K, "iq4_nl": IQ4_NL}
+BLOCK = {F32: (1, 4), Q8_0: (32, 34), Q4_K: (256, 144), MXFP4: (32, 17), F16: (1, 2), BF16: (1, 2), Q4_0: (32, 18),
+         Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176), Q6_K: (256, 210), IQ4_NL: (32, 18)}
 
 _f32p = C.POINTER(C.c_float)
 _f64p = C.POINTER(C.c_double)

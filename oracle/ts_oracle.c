@@ -108,6 +108,9 @@ int64_t tso_block_size(int type)
     case TSO_TYPE_Q8_0: return Q8_0_ELEMS;
     case TSO_TYPE_Q4_K: return Q4_K_ELEMS;
     case TSO_TYPE_MXFP4: return MXFP4_ELEMS;
+    case TSO_TYPE_F16: case TSO_TYPE_BF16: return 1;
+    case TSO_TYPE_Q4_0: case TSO_TYPE_Q4_1: case TSO_TYPE_Q5_0: case TSO_TYPE_Q5_1: case TSO_TYPE_IQ4_NL: return 32;
+    case TSO_TYPE_Q5_K: case TSO_TYPE_Q6_K: return 256;
     default: return 0;
     }
 }
@@ -119,6 +122,14 @@ int64_t tso_type_size(int type)
     case TSO_TYPE_Q8_0: return Q8_0_BYTES;
     case TSO_TYPE_Q4_K: return Q4_K_BYTES;
     case TSO_TYPE_MXFP4: return MXFP4_BYTES;
+    case TSO_TYPE_F16: case TSO_TYPE_BF16: return 2;
+    case TSO_TYPE_Q4_0: return 18;
+    case TSO_TYPE_Q4_1: return 20;
+    case TSO_TYPE_Q5_0: return 22;
+    case TSO_TYPE_Q5_1: return 24;
+    case TSO_TYPE_IQ4_NL: return 18;
+    case TSO_TYPE_Q5_K: return 176;
+    case TSO_TYPE_Q6_K: return 210;
     default: return 0;
     }
 }
@@ -443,6 +454,137 @@ static void dequant_mxfp4(const uint8_t* src, int64_t n, float* y)
     }
 }
 
+
+/* ---- the other formats the managed code reads (dequantize / embedding gather only, plus Q6_K matmuls) ---- */
+
+/* Reference: ManagedQuantizedOps.cs:268-281 (F16: exact widening; BF16: bits << 16). */
+static void dequant_f16(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t i = 0; i < n; ++i) y[i] = tso_fp16_to_fp32(rd16(src + 2 * i));
+}
+static void dequant_bf16(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t i = 0; i < n; ++i) y[i] = bits_f32((uint32_t)rd16(src + 2 * i) << 16);
+}
+
+/* y[j] = (q - 8) * d, low nibble -> j, high nibble -> j + 16.
+ * Reference: ManagedQuantizedOps.cs:313-333, ggml-quants.c dequantize_row_q4_0. */
+static void dequant_q4_0(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 32; ++b, src += 18, y += 32) {
+        const float d = tso_fp16_to_fp32(rd16(src));
+        for (int j = 0; j < 16; ++j) {
+            y[j] = ((src[2 + j] & 0x0f) - 8) * d;
+            y[j + 16] = ((src[2 + j] >> 4) - 8) * d;
+        }
+    }
+}
+
+/* y[j] = q * d + m (a product and a separately rounded sum).
+ * Reference: ManagedQuantizedOps.cs:335-356, ggml-quants.c dequantize_row_q4_1. */
+static void dequant_q4_1(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 32; ++b, src += 20, y += 32) {
+        const float d = tso_fp16_to_fp32(rd16(src)), m = tso_fp16_to_fp32(rd16(src + 2));
+        for (int j = 0; j < 16; ++j) {
+            y[j] = (src[4 + j] & 0x0f) * d + m;
+            y[j + 16] = (src[4 + j] >> 4) * d + m;
+        }
+    }
+}
+
+/* fifth bit of element j from bit j of qh (elements 16.. from bits 16..).
+ * Reference: ManagedQuantizedOps.cs:358-382, ggml-quants.c dequantize_row_q5_0. */
+static void dequant_q5_0(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 32; ++b, src += 22, y += 32) {
+        const float d = tso_fp16_to_fp32(rd16(src));
+        const uint32_t qh = (uint32_t)src[2] | ((uint32_t)src[3] << 8) | ((uint32_t)src[4] << 16) | ((uint32_t)src[5] << 24);
+        for (int j = 0; j < 16; ++j) {
+            const int xh0 = (int)(((qh >> j) << 4) & 0x10), xh1 = (int)((qh >> (j + 12)) & 0x10);
+            y[j] = (((src[6 + j] & 0x0f) | xh0) - 16) * d;
+            y[j + 16] = (((src[6 + j] >> 4) | xh1) - 16) * d;
+        }
+    }
+}
+
+/* Reference: ManagedQuantizedOps.cs:384-409, ggml-quants.c dequantize_row_q5_1. */
+static void dequant_q5_1(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 32; ++b, src += 24, y += 32) {
+        const float d = tso_fp16_to_fp32(rd16(src)), m = tso_fp16_to_fp32(rd16(src + 2));
+        const uint32_t qh = (uint32_t)src[4] | ((uint32_t)src[5] << 8) | ((uint32_t)src[6] << 16) | ((uint32_t)src[7] << 24);
+        for (int j = 0; j < 16; ++j) {
+            const int xh0 = (int)(((qh >> j) << 4) & 0x10), xh1 = (int)((qh >> (j + 12)) & 0x10);
+            y[j] = ((src[8 + j] & 0x0f) | xh0) * d + m;
+            y[j + 16] = ((src[8 + j] >> 4) | xh1) * d + m;
+        }
+    }
+}
+
+/* Q4_K with a fifth bit per weight: block = d, dmin, scales[12], qh[32], ql[128];
+ * y = (d*sc) * (nibble + 16*bit) - (dmin*m).
+ * Reference: ManagedQuantizedOps.cs:481-518, ggml-quants.c dequantize_row_q5_K. */
+static void dequant_q5_K(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 256; ++b, src += 176, y += 256) {
+        const float d = tso_fp16_to_fp32(rd16(src)), dmin = tso_fp16_to_fp32(rd16(src + 2));
+        const uint8_t* packed = src + 4;
+        const uint8_t* qh = src + 16;
+        const uint8_t* ql = src + 48;
+        uint8_t u1 = 1, u2 = 2;
+        for (int g = 0; g < 4; ++g, ql += 32, u1 <<= 2, u2 <<= 2) {
+            uint8_t sc1, m1, sc2, m2;
+            unpack_scale_min(2 * g, packed, &sc1, &m1);
+            unpack_scale_min(2 * g + 1, packed, &sc2, &m2);
+            const float d1 = d * sc1, d2 = d * sc2;
+            const float o1 = dmin * m1, o2 = dmin * m2;
+            for (int l = 0; l < 32; ++l) y[64 * g + l] = d1 * ((ql[l] & 0x0f) + ((qh[l] & u1) ? 16 : 0)) - o1;
+            for (int l = 0; l < 32; ++l) y[64 * g + 32 + l] = d2 * ((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - o2;
+        }
+    }
+}
+
+/* block = ql[128], qh[64], int8 scales[16], fp16 d; per 128 weights: 4 groups of 32 taken from the low / high
+ * nibbles of ql[l], ql[l + 32] and two bits of qh[l]; y = d * scale * (q - 32), exact in fp32.
+ * Reference: ManagedQuantizedOps.cs:520-557, ggml-quants.c:1762-1791. */
+static void dequant_q6_K(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 256; ++b, src += 210, y += 256) {
+        const uint8_t* ql = src;
+        const uint8_t* qh = src + 128;
+        const int8_t* sc = (const int8_t*)(src + 192);
+        const float d = tso_fp16_to_fp32(rd16(src + 208));
+        for (int half = 0; half < 2; ++half, ql += 64, qh += 32, sc += 8) {
+            float* o = y + 128 * half;
+            for (int l = 0; l < 32; ++l) {
+                const int is = l / 16;
+                const int8_t q1 = (int8_t)(((ql[l] & 0x0f) | (((qh[l] >> 0) & 3) << 4)) - 32);
+                const int8_t q2 = (int8_t)(((ql[l + 32] & 0x0f) | (((qh[l] >> 2) & 3) << 4)) - 32);
+                const int8_t q3 = (int8_t)(((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+                const int8_t q4 = (int8_t)(((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+                o[l] = d * sc[is] * q1;
+                o[l + 32] = d * sc[is + 2] * q2;
+                o[l + 64] = d * sc[is + 4] * q3;
+                o[l + 96] = d * sc[is + 6] * q4;
+            }
+        }
+    }
+}
+
+/* y = d * table[nibble].  Reference: ManagedQuantizedOps.cs:30-33, :559-577. */
+static const int8_t k_iq4nl_values[16] = { -127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113 };
+static void dequant_iq4_nl(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 32; ++b, src += 18, y += 32) {
+        const float d = tso_fp16_to_fp32(rd16(src));
+        for (int j = 0; j < 16; ++j) {
+            y[j] = d * k_iq4nl_values[src[2 + j] & 0x0f];
+            y[j + 16] = d * k_iq4nl_values[src[2 + j] >> 4];
+        }
+    }
+}
+
 /* Return codes follow TSGgml_DequantizeToF32: 0 ok, -1 bad args, -2 unsupported type.
  * Reference: ggml_ops_core.cpp:1331-1354. */
 int tso_dequantize(int type, const void* src, int64_t n, float* dst)
@@ -456,6 +598,15 @@ int tso_dequantize(int type, const void* src, int64_t n, float* dst)
     case TSO_TYPE_Q8_0: dequant_q8_0((const uint8_t*)src, n, dst); return 0;
     case TSO_TYPE_Q4_K: dequant_q4_K((const uint8_t*)src, n, dst); return 0;
     case TSO_TYPE_MXFP4: dequant_mxfp4((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_F16: dequant_f16((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_BF16: dequant_bf16((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q4_0: dequant_q4_0((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q4_1: dequant_q4_1((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q5_0: dequant_q5_0((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q5_1: dequant_q5_1((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q5_K: dequant_q5_K((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q6_K: dequant_q6_K((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_IQ4_NL: dequant_iq4_nl((const uint8_t*)src, n, dst); return 0;
     default: return -2;
     }
 }
@@ -468,7 +619,7 @@ static int check_mm(int type, const void* w, int64_t N, int64_t K, const float* 
                     int64_t x_stride, const void* out)
 {
     if (!w || !x || !out || N <= 0 || M <= 0 || K <= 0 || x_stride < K) return -1;
-    if (type != TSO_TYPE_Q8_0 && type != TSO_TYPE_Q4_K && type != TSO_TYPE_MXFP4) return -2;
+    if (tso_block_size(type) == 0 || type == TSO_TYPE_F32) return -2;
     if (K % tso_block_size(type) != 0) return -1;
     return 0;
 }
@@ -641,6 +792,7 @@ int tso_matmul_ggml(int type, const void* w, int64_t N, int64_t K, const float* 
 {
     int rc = check_mm(type, w, N, K, x, M, x_stride, out);
     if (rc) return rc;
+    if (type != TSO_TYPE_Q8_0 && type != TSO_TYPE_Q4_K && type != TSO_TYPE_MXFP4) return -2;
     const int64_t row_bytes = tso_row_size(type, K);
     const int64_t act_bytes = type == TSO_TYPE_Q4_K ? K / 256 * Q8_K_BYTES : K / 32 * Q8_0_BYTES;
     uint8_t* act = (uint8_t*)malloc((size_t)(act_bytes * M));

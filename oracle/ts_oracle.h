@@ -2,7 +2,7 @@
  * TEST INFRASTRUCTURE — not part of the shipped library.
  *
  * CPU restatement of the reference arithmetic for the GGUF quantized-matmul
- * path (Q8_0 / Q4_K / MXFP4).  Only tests, the smoke check and the
+ * path (Q8_0 / Q4_K / MXFP4 matmuls; dequantizers also for the other formats the managed code reads).  Only tests, the smoke check and the
  * cpu_baseline leg of the benchmark may load this library; the HIP library
  * never links or calls it.
  *
@@ -20,7 +20,11 @@ extern "C" {
 #endif
 
 /* GGUF tensor type ids: TensorSharp.Runtime/GgufReader.cs:26-37 */
-enum { TSO_TYPE_F32 = 0, TSO_TYPE_Q8_0 = 8, TSO_TYPE_Q4_K = 12, TSO_TYPE_MXFP4 = 39 };
+enum {
+    TSO_TYPE_F32 = 0, TSO_TYPE_F16 = 1, TSO_TYPE_Q4_0 = 2, TSO_TYPE_Q4_1 = 3, TSO_TYPE_Q5_0 = 6, TSO_TYPE_Q5_1 = 7,
+    TSO_TYPE_Q8_0 = 8, TSO_TYPE_Q4_K = 12, TSO_TYPE_Q5_K = 13, TSO_TYPE_Q6_K = 14, TSO_TYPE_IQ4_NL = 20,
+    TSO_TYPE_BF16 = 30, TSO_TYPE_MXFP4 = 39
+};
 
 /* scalar helpers */
 float    tso_fp16_to_fp32(uint16_t h);

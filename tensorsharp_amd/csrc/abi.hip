@@ -228,7 +228,7 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
         return false;
     }
     if (!is_quant_type(type)) {
-        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, MXFP4).");
+        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, Q6_K, MXFP4).");
         return false;
     }
     const size_t rs = row_size(type, ne0);
@@ -247,7 +247,7 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
 bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
 {
     const uintptr_t wa = reinterpret_cast<uintptr_t>(w);
-    const uintptr_t need_align = type == kTypeQ4_K ? 16 : type == kTypeQ8_0 ? 2 : 1;
+    const uintptr_t need_align = type == kTypeQ4_K ? 16 : (type == kTypeQ8_0 || type == kTypeQ6_K) ? 2 : 1;
     if (wa % need_align != 0) {
         set_last_error("Quantized weight pointer is not aligned for its block type.");
         return false;
@@ -453,7 +453,7 @@ bool validate_weight(const void* data, int type, int64_t ne0, int64_t ne1, int64
         return false;
     }
     if (!is_quant_type(type)) {
-        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, MXFP4).");
+        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, Q6_K, MXFP4).");
         return false;
     }
     const size_t rs = row_size(type, ne0);
@@ -631,7 +631,7 @@ int TSHip_DequantizeToF32Device(int ggml_type, const void* src, int64_t num_elem
     return guarded(-1, "dequantize", [&]() -> int {
         if (src == nullptr || dst == nullptr || num_elements < 0) return -1;
         if (num_elements == 0) return 0;
-        if (ggml_type != kTypeF32 && !is_quant_type(ggml_type)) return -2;
+        if (ggml_type != kTypeF32 && !is_dequant_type(ggml_type)) return -2;
         if (!ensure_backend()) return -1;
         if (ggml_type == kTypeF32)
             return hip_ok(hipMemcpyAsync(dst, src, (size_t)num_elements * 4, hipMemcpyDeviceToDevice, g_stream.load()),
@@ -652,7 +652,7 @@ int TSHip_DequantizeToF32(int ggml_type, const void* src, int64_t num_elements, 
             std::memcpy(dst, src, (size_t)num_elements * sizeof(float));
             return 0;
         }
-        if (!is_quant_type(ggml_type)) return -2;
+        if (!is_dequant_type(ggml_type)) return -2;
         if (num_elements % block_elems(ggml_type) != 0) return -1;
         if (!ensure_backend()) return -1;
         const size_t in_bytes = row_size(ggml_type, num_elements);
@@ -979,7 +979,7 @@ int TSHip_GetRowsQuantF32Device(TSHipTensorView2D result, const void* src_data, 
             return 0;
         }
         const size_t rs = row_size(src_ggml_type, src_ne0);
-        if ((src_ggml_type != kTypeF32 && !is_quant_type(src_ggml_type)) || rs == 0 || src_ne0 % 4 != 0) {
+        if ((src_ggml_type != kTypeF32 && !is_dequant_type(src_ggml_type)) || rs == 0 || src_ne0 % 4 != 0) {
             set_last_error("Unsupported source type or row length for get_rows_quant.");
             return 0;
         }
@@ -1027,7 +1027,7 @@ int TSHip_GetRowsQuantF32(TSHipTensorView2D result, void* src_data, int src_ggml
             return 0;
         }
         const size_t rs = row_size(src_ggml_type, src_ne0);
-        if ((src_ggml_type != kTypeF32 && !is_quant_type(src_ggml_type)) || rs == 0 || src_ne0 % 4 != 0) {
+        if ((src_ggml_type != kTypeF32 && !is_dequant_type(src_ggml_type)) || rs == 0 || src_ne0 % 4 != 0) {
             set_last_error("Unsupported source type or row length for get_rows_quant.");
             return 0;
         }

@@ -1,7 +1,8 @@
 // Bit-exact dequantization of raw GGUF blocks to fp32 on gfx950.
 //
 // The arithmetic is the managed dequantizers' (TensorSharp.Models/ManagedQuantizedOps.cs:411-427 Q8_0,
-// :447-479 Q4_K, :579-598 MXFP4): every product is exact in fp32, the Q4_K subtract is the one rounding.
+// :447-479 Q4_K, :579-598 MXFP4; :268-409 and :481-577 for F16, BF16, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q6_K, IQ4_NL):
+// every product is exact in fp32, the subtract of Q4_K / Q5_K and the add of Q4_1 / Q5_1 are the one rounding.
 // Contraction is switched off so the multiply and the subtract stay separately rounded operations.
 // fp16 scales are widened with integer arithmetic, so the result does not depend on the wave's
 // denormal mode.
@@ -108,12 +109,119 @@ __device__ __forceinline__ float4 dequant4_mxfp4(const uint8_t* src, int64_t e0)
     return o;
 }
 
+
+// ---- formats used for dequantization / embedding gather only (ManagedQuantizedOps.cs:268-409, :481-577) ----
+__device__ __forceinline__ uint32_t rd16u(const uint8_t* p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
+__device__ __forceinline__ uint32_t rd32u(const uint8_t* p) { return rd16u(p) | (rd16u(p + 2) << 16); }
+
+__device__ __forceinline__ float4 dequant4_f16(const uint8_t* src, int64_t e0)
+{
+    const uint8_t* p = src + e0 * 2;
+    return float4{half_bits_to_float(rd16u(p)), half_bits_to_float(rd16u(p + 2)), half_bits_to_float(rd16u(p + 4)),
+                  half_bits_to_float(rd16u(p + 6))};
+}
+
+__device__ __forceinline__ float4 dequant4_bf16(const uint8_t* src, int64_t e0)
+{
+    const uint8_t* p = src + e0 * 2;
+    return float4{__uint_as_float(rd16u(p) << 16), __uint_as_float(rd16u(p + 2) << 16), __uint_as_float(rd16u(p + 4) << 16),
+                  __uint_as_float(rd16u(p + 6) << 16)};
+}
+
+// Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL: 32 weights, low nibbles are elements 0..15, high nibbles 16..31;
+// HDR bytes of scales (and the 32 fifth bits) in front of the 16 quant bytes
+template <int TYPE>
+__device__ __forceinline__ float4 dequant4_legacy(const uint8_t* src, int64_t e0)
+{
+    constexpr int kHdr = TYPE == kTypeQ4_0 || TYPE == kTypeIQ4_NL ? 2 : TYPE == kTypeQ4_1 ? 4 : TYPE == kTypeQ5_0 ? 6 : 8;
+    constexpr bool kMin = TYPE == kTypeQ4_1 || TYPE == kTypeQ5_1;
+    constexpr bool kFive = TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1;
+    const uint8_t* blk = src + (e0 >> 5) * (kHdr + 16);
+    const int j = (int)(e0 & 31);
+    const int sh = (j >> 4) * 4;
+    const uint8_t* q = blk + kHdr + (j & 15);
+    const float d = half_bits_to_float(rd16u(blk));
+    const float m = kMin ? half_bits_to_float(rd16u(blk + 2)) : 0.f;
+    const uint32_t qh = kFive ? rd32u(blk + kHdr - 4) : 0u;
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int v = (q[i] >> sh) & 0x0f;
+        if (kFive) v |= (int)((qh >> (j + i)) & 1u) << 4;
+        if (TYPE == kTypeIQ4_NL) {
+            // {-127,-104,-83,-65,-49,-35,-22,-10, 1,13,25,38,53,69,89,113} as signed bytes (ManagedQuantizedOps.cs:30-33)
+            const uint64_t tab = (v & 8) ? 0x7159453526190d01ull : 0xf6eaddcfbfad9881ull;
+            o[i] = d * (float)(int)(int8_t)((tab >> ((v & 7) * 8)) & 0xffu);
+        } else if (kMin) {
+            o[i] = (float)v * d + m;
+        } else {
+            o[i] = (float)(v - (kFive ? 16 : 8)) * d;
+        }
+    }
+    return float4{o[0], o[1], o[2], o[3]};
+}
+
+// Q5_K: d, dmin, scales[12], qh[32], ql[128]; y = (d*sc) * (nibble + 16*bit) - (dmin*m)
+__device__ __forceinline__ float4 dequant4_q5_K(const uint8_t* src, int64_t e0)
+{
+    const uint8_t* blk = src + (e0 >> 8) * 176;
+    const int r = (int)(e0 & 255);
+    const int g = r >> 6, hi = (r >> 5) & 1, l = r & 31;
+    const int j = 2 * g + hi;
+    const float d = half_bits_to_float(rd16u(blk));
+    const float dmin = half_bits_to_float(rd16u(blk + 2));
+    const uint8_t* p = blk + 4;
+    uint32_t sc, mn;
+    if (j < 4) {
+        sc = p[j] & 63u;
+        mn = p[j + 4] & 63u;
+    } else {
+        sc = (p[j + 4] & 0x0fu) | ((uint32_t)(p[j - 4] >> 6) << 4);
+        mn = (uint32_t)(p[j + 4] >> 4) | ((uint32_t)(p[j] >> 6) << 4);
+    }
+    const float d1 = d * (float)sc;
+    const float m1 = dmin * (float)mn;
+    const uint8_t* qh = blk + 16 + l;
+    const uint8_t* q = blk + 48 + 32 * g + l;
+    const int sh = hi * 4;
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = d1 * (float)(((q[i] >> sh) & 0x0fu) + (((qh[i] >> j) & 1u) << 4)) - m1;
+    return float4{o[0], o[1], o[2], o[3]};
+}
+
+// Q6_K: ql[128], qh[64], int8 scales[16], fp16 d; y = d * scale * (q - 32)
+__device__ __forceinline__ float4 dequant4_q6_K(const uint8_t* src, int64_t e0)
+{
+    const uint8_t* blk = src + (e0 >> 8) * 210;
+    const int r = (int)(e0 & 255);
+    const int half = r >> 7, grp = (r >> 5) & 3, l = r & 31;
+    const uint8_t* ql = blk + 64 * half + 32 * (grp & 1) + l;
+    const uint8_t* qh = blk + 128 + 32 * half + l;
+    const float d = half_bits_to_float(rd16u(blk + 208));
+    const float ds = d * (float)(int)(int8_t)blk[192 + 8 * half + 2 * grp + (l >> 4)];
+    const int sh = (grp >> 1) * 4;
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int q = (int)(((ql[i] >> sh) & 0x0fu) | (((qh[i] >> (2 * grp)) & 3u) << 4)) - 32;
+        o[i] = ds * (float)q;
+    }
+    return float4{o[0], o[1], o[2], o[3]};
+}
+
 template <int TYPE>
 __device__ __forceinline__ float4 dequant4(const uint8_t* src, int64_t e0)
 {
     if (TYPE == kTypeQ8_0) return dequant4_q8_0(src, e0);
     if (TYPE == kTypeQ4_K) return dequant4_q4_K(src, e0);
     if (TYPE == kTypeMXFP4) return dequant4_mxfp4(src, e0);
+    if (TYPE == kTypeF16) return dequant4_f16(src, e0);
+    if (TYPE == kTypeBF16) return dequant4_bf16(src, e0);
+    if (TYPE == kTypeQ4_0 || TYPE == kTypeQ4_1 || TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1 || TYPE == kTypeIQ4_NL)
+        return dequant4_legacy<TYPE>(src, e0);
+    if (TYPE == kTypeQ5_K) return dequant4_q5_K(src, e0);
+    if (TYPE == kTypeQ6_K) return dequant4_q6_K(src, e0);
     const float* f = reinterpret_cast<const float*>(src) + e0;      // F32 rows: plain copy
     return float4{f[0], f[1], f[2], f[3]};
 }
@@ -162,6 +270,11 @@ bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_
     case kTypeQ8_0: hipLaunchKernelGGL(dequant_kernel<kTypeQ8_0>, grid, block, 0, stream, s, dst, n4); break;
     case kTypeQ4_K: hipLaunchKernelGGL(dequant_kernel<kTypeQ4_K>, grid, block, 0, stream, s, dst, n4); break;
     case kTypeMXFP4: hipLaunchKernelGGL(dequant_kernel<kTypeMXFP4>, grid, block, 0, stream, s, dst, n4); break;
+#define TSHIP_DEQUANT_CASE(T) case T: hipLaunchKernelGGL(dequant_kernel<T>, grid, block, 0, stream, s, dst, n4); break;
+    TSHIP_DEQUANT_CASE(kTypeF16) TSHIP_DEQUANT_CASE(kTypeBF16) TSHIP_DEQUANT_CASE(kTypeQ4_0) TSHIP_DEQUANT_CASE(kTypeQ4_1)
+    TSHIP_DEQUANT_CASE(kTypeQ5_0) TSHIP_DEQUANT_CASE(kTypeQ5_1) TSHIP_DEQUANT_CASE(kTypeQ5_K) TSHIP_DEQUANT_CASE(kTypeQ6_K)
+    TSHIP_DEQUANT_CASE(kTypeIQ4_NL)
+#undef TSHIP_DEQUANT_CASE
     default: set_last_error("dequantize: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "dequantize launch");
@@ -185,6 +298,11 @@ bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, 
     case kTypeQ8_0: hipLaunchKernelGGL(get_rows_kernel<kTypeQ8_0>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
     case kTypeQ4_K: hipLaunchKernelGGL(get_rows_kernel<kTypeQ4_K>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
     case kTypeMXFP4: hipLaunchKernelGGL(get_rows_kernel<kTypeMXFP4>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
+#define TSHIP_ROWS_CASE(T) case T: hipLaunchKernelGGL(get_rows_kernel<T>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
+    TSHIP_ROWS_CASE(kTypeF16) TSHIP_ROWS_CASE(kTypeBF16) TSHIP_ROWS_CASE(kTypeQ4_0) TSHIP_ROWS_CASE(kTypeQ4_1)
+    TSHIP_ROWS_CASE(kTypeQ5_0) TSHIP_ROWS_CASE(kTypeQ5_1) TSHIP_ROWS_CASE(kTypeQ5_K) TSHIP_ROWS_CASE(kTypeQ6_K)
+    TSHIP_ROWS_CASE(kTypeIQ4_NL)
+#undef TSHIP_ROWS_CASE
     default: set_last_error("get_rows: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "get_rows launch");

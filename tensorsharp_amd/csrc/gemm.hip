@@ -6,7 +6,7 @@
 //      format unpacks (so the dequantizer never has to shuffle lanes), zero-padded to a
 //      multiple of the k-tile.  Optionally gathers rows through an index (MoE).
 //   2. gemm_kernel (M > 64 per tile) / gemm_few_rows_kernel (M <= 64 per tile, persistent workgroups) /
-//      gemm_slim_kernel (M <= 32 per tile and K <= 4096: activations in registers, K split over the wavefronts):
+//      gemm_slim_kernel (M <= 32 per tile: activations in registers, K split over the wavefronts, long K in chunks):
 //      BM x 256 x 64 tiles, eight wavefronts, each owning 32 output columns.  The fp16
 //      activation k-tiles and the RAW quantized bytes of 256 weight rows (one 144-byte window per row
 //      covering four k-tiles of Q4_K / MXFP4 or two of Q8_0) are copied from global memory straight
@@ -24,6 +24,7 @@
 #include "tship_internal.h"
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 namespace tship {
@@ -92,7 +93,7 @@ __device__ __forceinline__ int k_slot(int k)
         const int hh = k >> 5, i = k & 15, hi = (k >> 4) & 1;
         return (i >> 2) * 16 + hh * 8 + 2 * (i & 3) + hi;
     }
-    // Q8_0: block k/32, natural order
+    // Q8_0 and Q6_K: 32-element group k/32, natural order
     const int hh = k >> 5, tt = k & 31;
     return (tt >> 3) * 16 + hh * 8 + (tt & 7);
 }
@@ -223,24 +224,30 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
 }
 
 // ------------------------------------------------------------------------------------------
-// weight formats: a "super-tile" is kSup consecutive k-tiles of one weight row, kept RAW in LDS as a
-// 144-byte window (nine 16-byte chunks copied from a 4-byte aligned address at or just below the
-// first block).  `delta` (0..3) is the distance from the window start to that first block.
-//   fetch():   the raw dwords one lane needs for its (row, k-half) of k-tile j of the super-tile
+// weight formats: a "super-tile" is kSup consecutive k-tiles of one weight row, kept RAW in LDS as a window of
+// kRawRow bytes (16-byte chunks copied from a 4-byte aligned address at or just below the first block).  `delta`
+// is the distance from the window start to that first block.
+//   fetch():   the raw dwords one lane needs for its (row, k-half) of k-tile t of the window
 //   dequant(): those dwords -> 16 packed fp16 pairs, o[4 ks .. 4 ks + 3] being the lane's B operand
 //              of MFMA k-step ks
+//   sup_offset() / sup_delta(): where super-tile s starts (4-byte aligned) relative to the row's first window and
+//              the delta inside that window; window_bytes() / tile_offset(): the same for windows of any number
+//              of k-tiles (the register-resident kernel)
 // ------------------------------------------------------------------------------------------
-constexpr int kRawRow = 144;
-
 struct GQ4K {
     static constexpr int kRegs = 8;
     static constexpr int kSup = 4;            // one 256-element super-block
     static constexpr int kSupBytes = 144;
-    static constexpr int kTileBytes = 36;     // bytes of one k-tile of a row
-    static constexpr int kSlack = 0;          // bytes fetch() may touch past the last k-tile of a window
-    static constexpr bool kSuperBlocks = true;   // fetch() addresses a k-tile through its super-block header
-    static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t /*delta*/, uint32_t (&r)[kRegs])
+    static constexpr int kRawRow = 144;       // LDS bytes of one row's super-tile window
+    static constexpr int kTileStep = 4;       // a wavefront's K range starts at a multiple of this many k-tiles
+    static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 144u; }            // window start of super-tile s
+    static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int /*s*/) { return delta; }
+    static constexpr int window_bytes(int ktw) { return ktw * 36; }                       // of ktw consecutive k-tiles
+    static constexpr uint32_t tile_offset(int kt0) { return (uint32_t)kt0 * 36u; }        // kt0 a multiple of kTileStep
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int t, int h, uint32_t /*delta*/, uint32_t (&r)[kRegs])
     {
+        rp += (t >> 2) * 144;
+        const int j = t & 3;
         const uint4_t hdr = *reinterpret_cast<const uint4_t*>(rp);
         const uint4_t q = *reinterpret_cast<const uint4_t*>(rp + 16 + j * 32 + h * 16);
         r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
@@ -278,9 +285,12 @@ struct GMXFP4 {
     static constexpr int kRegs = 5;
     static constexpr int kSup = 4;            // eight 17-byte blocks
     static constexpr int kSupBytes = 136;
-    static constexpr int kTileBytes = 34;
-    static constexpr int kSlack = 6;
-    static constexpr bool kSuperBlocks = false;
+    static constexpr int kRawRow = 144;
+    static constexpr int kTileStep = 2;
+    static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 136u; }
+    static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int /*s*/) { return delta; }
+    static constexpr int window_bytes(int ktw) { return ktw * 34 + 3; }
+    static constexpr uint32_t tile_offset(int kt0) { return (uint32_t)kt0 * 34u; }
     static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t delta, uint32_t (&r)[kRegs])
     {
         const uint32_t off = delta + (uint32_t)(2 * j + h) * 17u;
@@ -322,9 +332,12 @@ struct GQ80 {
     static constexpr int kRegs = 9;
     static constexpr int kSup = 2;            // four 34-byte blocks
     static constexpr int kSupBytes = 136;
-    static constexpr int kTileBytes = 68;
-    static constexpr int kSlack = 4;
-    static constexpr bool kSuperBlocks = false;
+    static constexpr int kRawRow = 144;
+    static constexpr int kTileStep = 2;
+    static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 136u; }
+    static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int /*s*/) { return delta; }
+    static constexpr int window_bytes(int ktw) { return ktw * 68 + 3; }
+    static constexpr uint32_t tile_offset(int kt0) { return (uint32_t)kt0 * 68u; }
     static __device__ __forceinline__ void fetch(const uint8_t* rp, int j, int h, uint32_t delta, uint32_t (&r)[kRegs])
     {
         const uint32_t off = delta + (uint32_t)(2 * j + h) * 34u;
@@ -350,6 +363,64 @@ struct GQ80 {
     }
 };
 
+// Q6_K (ggml-common.h block_q6_K: ql[128], qh[64], int8 scales[16], fp16 d = 210 bytes, 2-byte aligned): k-tile
+// t & 3 of a block takes, for k-half h, 32 quant bytes ql[64 (j / 2) + 32 h ..] (low nibbles for even j, high for
+// odd), the two bits (2 (j & 1) + h) of qh[32 (j / 2) ..] and two scales.  Values d * scale * (q - 32)
+// (ManagedQuantizedOps.cs:520-557) enter the matrix cores as fp16(d * scale) * (q - 32).  Blocks alternate
+// between 4-byte aligned and 2 bytes off, so every piece is fetched as aligned dwords and shifted by 0 or 2 bytes.
+struct GQ6K {
+    static constexpr int kRegs = 20;
+    static constexpr int kSup = 4;            // one 256-element block
+    static constexpr int kSupBytes = 210;
+    static constexpr int kRawRow = 224;
+    static constexpr int kTileStep = 4;
+    static constexpr uint32_t sup_offset(int s) { return ((uint32_t)s * 210u) & ~3u; }
+    static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int s) { return delta + ((uint32_t)(s & 1) << 1); }
+    static constexpr int window_bytes(int ktw) { return ktw / 4 * 210 + 2; }
+    static constexpr uint32_t tile_offset(int kt0) { return (uint32_t)(kt0 >> 2) * 210u; }
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int t, int h, uint32_t delta, uint32_t (&r)[kRegs])
+    {
+        const uint32_t blk = delta + (uint32_t)(t >> 2) * 210u;        // block start inside the window (even)
+        const int j = t & 3, nh = j >> 1;
+        const uint32_t* a = reinterpret_cast<const uint32_t*>(rp + ((blk + 64u * nh + 32u * h) & ~3u));
+        const uint32_t* b = reinterpret_cast<const uint32_t*>(rp + ((blk + 128u + 32u * nh) & ~3u));
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+            r[i] = a[i];
+            r[9 + i] = b[i];
+        }
+        r[18] = *reinterpret_cast<const uint32_t*>(rp + ((blk + 192u + 8u * nh + 2u * (2 * (j & 1) + h)) & ~3u));
+        r[19] = *reinterpret_cast<const uint32_t*>(rp + ((blk + 208u) & ~3u));
+    }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int h, uint32_t delta, bool live, uint32_t (&o)[16])
+    {
+        const uint32_t blk = delta + (uint32_t)(t >> 2) * 210u;
+        const int j = t & 3, g4 = 2 * (j & 1) + h;
+        const uint32_t sh = (blk & 2u) ? 2u : 0u;                       // byte shift of the block's dwords
+        const uint32_t ps = blk + 192u + 8u * (j >> 1) + 2u * g4;
+        const uint32_t scw = r[18] >> ((ps & 2u) * 8u);
+        const float sc0 = (float)(int)(int8_t)(scw & 0xffu), sc1 = (float)(int)(int8_t)((scw >> 8) & 0xffu);
+        H2U dd;
+        dd.u = (r[19] >> ((blk & 2u) * 8u)) & 0xffffu;
+        const float d = live ? (float)dd.h.x : 0.f;
+        const uint32_t s0 = splat(d * sc0), s1 = splat(d * sc1);
+        const uint32_t bias = 0xe420e420u;                              // -(1024 + 32)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t ql = __builtin_amdgcn_alignbyte(r[i + 1], r[i], sh);
+            const uint32_t qh = __builtin_amdgcn_alignbyte(r[10 + i], r[9 + i], sh);
+            const uint32_t nib = ((j & 1) ? (ql >> 4) : ql) & 0x0f0f0f0fu;
+            const uint32_t q6 = nib | (((qh >> (2 * g4)) & 0x03030303u) << 4);
+            // bytes u = q become fp16 1024 + u: (0x64, u) pairs picked with v_perm; minus 1056 leaves q - 32 exactly
+            const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, q6, 0x04010400u);
+            const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, q6, 0x04030402u);
+            const uint32_t sc = i < 4 ? s0 : s1;                         // elements 0..15 / 16..31 of the group
+            o[2 * i] = pk_mul(pk_add(p0, bias), sc);
+            o[2 * i + 1] = pk_mul(pk_add(p1, bias), sc);
+        }
+    }
+};
+
 struct GemmArgs {
     const uint8_t* w;        // weight bytes (of expert 0 for grouped launches)
     int64_t w_bytes;         // bytes of one weight matrix (per expert for grouped launches)
@@ -367,12 +438,13 @@ struct GemmArgs {
     const int* tile_rows;    // [m_tiles] rows in the tile (<= BM)
     int64_t expert_stride;   // bytes between experts
     int accumulate;          // c += ... instead of c = ...
+    // register-resident kernel with K cut into chunks: chunk kc of a row tile writes its sums (already scaled) to
+    // partial[kc][activation row][column]; a second kernel adds the chunks in order into c
+    float* partial;          // null: one chunk, results go straight to c
+    int k_chunks;
+    int chunk_kt;            // k-tiles per chunk (8 wavefronts x KTW)
 };
 
-constexpr int kBN = 256;                     // weight rows (output columns) per tile: 32 per wavefront
-constexpr int kWaves = 8;
-constexpr int kRawTile = kBN * kRawRow;      // bytes of one raw super-tile in LDS
-constexpr int kRawInstrs = kRawTile / 1024;  // wavefront-wide 1 KiB copies per raw super-tile (36)
 constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
 
 // LDS-direct copy: 64 lanes x 16 bytes land at lds + 16 * lane; out-of-range offsets deliver zeros
@@ -438,6 +510,7 @@ template <typename G, int BM, int XST, int NW>
 __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
 {
     constexpr int BN = NW * 32;                          // output columns per tile
+    constexpr int kRawRow = G::kRawRow, kRowChunks = kRawRow / 16;
     constexpr int RT = BN * kRawRow;                     // bytes of one raw super-tile in LDS
     constexpr int RIN = RT / 1024;                       // wavefront-wide 1 KiB copies per raw super-tile
     constexpr int WI = (RIN + NW - 1) / NW;              // per wavefront; the surplus goes to a dump area
@@ -503,7 +576,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
         const int c = (wave + NW * i) * 64 + lane;
-        const int row = c / 9, chunk = c - row * 9;
+        const int row = c / kRowChunks, chunk = c - row * kRowChunks;
         w_off[i] = (row < BN && n0 + row < A.N) ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
                                                   : kDeadOffset;
     }
@@ -532,9 +605,9 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         for (int i = 0; i < WI; ++i) {
             const int id = wave + NW * i;
 #ifdef TSHIP_GEMM_DEBUG_NOW
-            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, kDeadOffset, (uint32_t)s * G::kSupBytes);
+            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, kDeadOffset, G::sup_offset(s));
 #else
-            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, any ? w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
+            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, any ? w_off[i] : kDeadOffset, G::sup_offset(s));
 #endif
         }
     };
@@ -559,8 +632,8 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
     uint32_t oc[16], on[16];
     {
         uint32_t r[G::kRegs];
-        G::fetch(rbuf + my_raw, 0, h, my_delta, r);
-        G::dequant(r, 0, h, my_delta, h * 32 < A.K, oc);
+        G::fetch(rbuf + my_raw, 0, h, G::sup_delta(my_delta, 0), r);
+        G::dequant(r, 0, h, G::sup_delta(my_delta, 0), h * 32 < A.K, oc);
     }
     int s = 0, j = 0;                               // super-tile and k-tile inside it of `kt`
     int xst = 0, rb = 0;                            // LDS stage of k-tile kt, raw buffer of super-tile s
@@ -571,7 +644,8 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         if (jn == G::kSup) { jn = 0; sn = s + 1; rbn = rb + 1 == RB ? 0 : rb + 1; }
         // raw bytes of this lane's operands for k-tile kt + 1 (past the last k-tile: stale LDS, result unused)
         uint32_t r[G::kRegs];
-        G::fetch(rbuf + rbn * RT + my_raw, jn, h, my_delta, r);
+        const uint32_t dn = G::sup_delta(my_delta, sn);
+        G::fetch(rbuf + rbn * RT + my_raw, jn, h, dn, r);
         const uint8_t* xs = xbuf + xst * kXTile;
         if constexpr (TM <= 2) {
             // few rows: every A operand of the k-tile is requested up front
@@ -582,7 +656,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
                 for (int i = 0; i < TM; ++i) a[ks][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[ks]);
             __builtin_amdgcn_sched_barrier(0);
 #ifndef TSHIP_GEMM_DEBUG_NODEQ
-            G::dequant(r, jn, h, my_delta, ((kt + 1) * 2 + h) * 32 < A.K, on);
+            G::dequant(r, jn, h, dn, ((kt + 1) * 2 + h) * 32 < A.K, on);
 #else
             _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs];
 #endif
@@ -621,7 +695,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
                 }
                 // unpack the next k-tile's operands in the shadow of the matrix pipe
 #ifndef TSHIP_GEMM_DEBUG_NODEQ
-                if (ks == 0) G::dequant(r, jn, h, my_delta, ((kt + 1) * 2 + h) * 32 < A.K, on);
+                if (ks == 0) G::dequant(r, jn, h, dn, ((kt + 1) * 2 + h) * 32 < A.K, on);
 #else
                 if (ks == 0) { _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs]; }
 #endif
@@ -647,7 +721,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
 template <typename G, int BM, int XST, int NW>
 bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    constexpr int BN = NW * 32, RT = BN * kRawRow;
+    constexpr int BN = NW * 32, RT = BN * G::kRawRow;
     auto kern = gemm_kernel<G, BM, XST, NW>;
     constexpr int RB = (XST > 2 && G::kSup == 2) ? 3 : 2;
     const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * RT + 1024;
@@ -669,13 +743,13 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 // LDS reads and leaves this iteration's copies in flight at the barrier (counted vmcnt).
 // ------------------------------------------------------------------------------------------
 // per-tile state of a persistent workgroup
-template <int NW>
+template <int NW, int RAW_ROW>
 struct FewRowsTile {
     int m0, m_rows, my_n;
     uint32_t my_delta;
     __amdgpu_buffer_rsrc_t wrs;
     uint32_t x_off[8 / NW];
-    uint32_t w_off[(NW * 32 * kRawRow / 1024 + NW - 1) / NW];
+    uint32_t w_off[(NW * 32 * RAW_ROW / 1024 + NW - 1) / NW];
 };
 
 // NW wavefronts (32 columns each), RING buffers for activations (in k-tile pairs) and for raw super-tiles:
@@ -685,6 +759,8 @@ template <typename G, int NW, int RING>
 __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A)
 {
     constexpr int BM = 64, TM = 2, KS = G::kSup;
+    constexpr int kRawRow = G::kRawRow, kRowChunks = kRawRow / 16;
+    using Tile = FewRowsTile<NW, G::kRawRow>;
     constexpr int BN = NW * 32, RT = BN * kRawRow, RIN = RT / 1024, WI = (RIN + NW - 1) / NW, XI = 8 / NW;
     static_assert(RIN * 1024 == RT && XI * NW == 8, "tile must split into whole copies");
     static_assert(RING == 2 || RING == 3, "ring of two or three");
@@ -719,7 +795,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
     int slot = blockIdx.x >> 3;
 
     // next tile with work at or after `slot` (grouped launches may list empty tiles); false when none is left
-    auto setup = [&](FewRowsTile<NW>& T) -> bool {
+    auto setup = [&](Tile& T) -> bool {
         for (; slot < per; slot += stride) {
             const int t = xcd * per + slot;
             if (t >= total) return false;
@@ -748,7 +824,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
 #pragma unroll
             for (int i = 0; i < WI; ++i) {
                 const int c = (wave + NW * i) * 64 + lane;
-                const int row = c / 9, chunk = c - row * 9;
+                const int row = c / kRowChunks, chunk = c - row * kRowChunks;
                 T.w_off[i] = (row < BN && n0 + row < A.N)
                                  ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
                                  : kDeadOffset;
@@ -761,7 +837,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
         return false;
     };
     // always the same number of copies per wavefront (sources past the end are out of range: zeros)
-    auto issue_x = [&](const FewRowsTile<NW>& T, int p) {            // k-tile pair p -> ring slot p % RING
+    auto issue_x = [&](const Tile& T, int p) {            // k-tile pair p -> ring slot p % RING
         uint8_t* dst = xbuf + (p % RING) * kXPair;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -775,23 +851,23 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
             }
         }
     };
-    auto issue_w = [&](const FewRowsTile<NW>& T, int s) {            // super-tile s -> buffer s % RING
+    auto issue_w = [&](const Tile& T, int s) {            // super-tile s -> buffer s % RING
         uint8_t* buf = rbuf + (s % RING) * RT;
         const bool any = s * KS < nkt;
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             const int id = wave + NW * i;
-            if (id < RIN) copy16_to_lds(T.wrs, buf + id * 1024, any ? T.w_off[i] : kDeadOffset, (uint32_t)s * G::kSupBytes);
+            if (id < RIN) copy16_to_lds(T.wrs, buf + id * 1024, any ? T.w_off[i] : kDeadOffset, G::sup_offset(s));
         }
     };
-    auto issue_first = [&](const FewRowsTile<NW>& T) {
+    auto issue_first = [&](const Tile& T) {
 #pragma unroll
         for (int i = 0; i < RING - 1; ++i) issue_x(T, i);
 #pragma unroll
         for (int i = 0; i < RING - 1; ++i) issue_w(T, i);
     };
 
-    FewRowsTile<NW> T;
+    Tile T;
     if (!setup(T)) return;
     issue_first(T);
     for (;;) {
@@ -816,7 +892,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
 #ifdef TSHIP_FR_NOFETCH
                     _Pragma("unroll") for (int q = 0; q < G::kRegs; ++q) r[e][q] = 0x3c003c00u + q + p;
 #else
-                    G::fetch(raw, e0 + e, h, T.my_delta, r[e]);
+                    G::fetch(raw, e0 + e, h, G::sup_delta(T.my_delta, s), r[e]);
 #endif
 #pragma unroll
                     for (int ks = 0; ks < 4; ++ks)
@@ -839,7 +915,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
 #ifdef TSHIP_FR_NODEQ
                     _Pragma("unroll") for (int q = 0; q < 16; ++q) o[q] = r[e][q % G::kRegs];
 #else
-                    G::dequant(r[e], e0 + e, h, T.my_delta, ((2 * p + e) * 2 + h) * 32 < A.K, o);
+                    G::dequant(r[e], e0 + e, h, G::sup_delta(T.my_delta, s), ((2 * p + e) * 2 + h) * 32 < A.K, o);
 #endif
 #pragma unroll
                     for (int ks = 0; ks < 4; ++ks) {
@@ -876,7 +952,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A
 template <typename G, int NW, int RING>
 bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
 {
-    constexpr int BN = NW * 32, RT = BN * kRawRow;
+    constexpr int BN = NW * 32, RT = BN * G::kRawRow;
     auto kern = gemm_few_rows_kernel<G, NW, RING>;
     const size_t lds = (size_t)RING * 2 * 64 * kXRow + (size_t)RING * RT;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
@@ -891,8 +967,8 @@ bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
 }
 
 // ------------------------------------------------------------------------------------------
-// At most 32 activation rows per tile and K of at most 64 k-tiles * 8 (small batches, MoE experts with few
-// tokens).  The activations stay in REGISTERS: the eight wavefronts of a workgroup split K between them
+// At most 32 activation rows per tile (small batches, MoE experts with few tokens; also single rows of formats
+// without a GEMV kernel).  The activations stay in REGISTERS: the eight wavefronts of a workgroup split K between them
 // (KTW k-tiles each), every wavefront keeps the MFMA A operands of its K range for all 32 rows, and the
 // workgroup walks over 32-column weight tiles.  Per tile a wavefront needs only its own K range of the 32
 // raw weight rows, which it copies itself (global -> LDS, two private buffers, requested two tiles ahead),
@@ -906,7 +982,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // block; the unpackers may read a few bytes further, into the next row, and ignore them)
 template <typename G, int KTW>
 struct SlimLayout {
-    static constexpr int CH = (KTW * G::kTileBytes + (G::kSlack ? 3 : 0) + 15) / 16;
+    static constexpr int CH = (G::window_bytes(KTW) + 15) / 16;
     static constexpr int DI = (32 * CH + 63) / 64;                       // LDS-direct copies per buffer
     static constexpr int RAW = 32 * CH * 16;
     static constexpr int BUF = RAW > 4096 ? RAW : 4096;                  // raw rows, later the 32 x 32 fp32 partial sums
@@ -918,7 +994,7 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
 {
     using L = SlimLayout<G, KTW>;
     constexpr int CH = L::CH, DI = L::DI, BUF = L::BUF, RING = L::RING;
-    static_assert(!G::kSuperBlocks || KTW % G::kSup == 0, "a wavefront's K range must start at a super-block");
+    static_assert(KTW % G::kTileStep == 0, "a wavefront's K range must start at a block");
     extern __shared__ uint8_t smem[];                                   // 8 wavefronts x RING x BUF
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -928,9 +1004,8 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
 
     const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
     const int nkt = A.Kp / kBK;
-    const int kt0 = wave * KTW;
-    const int kcnt = max(0, min(KTW, nkt - kt0));                      // k-tiles of this wavefront
     const int n32 = (A.N + 31) >> 5;
+    const int per_tile = A.k_chunks * n32;                              // units of one row tile
 
     // grouped launches: the table may end in empty tiles
     int live_tiles = A.m_tiles;
@@ -940,14 +1015,17 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
         for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
         live_tiles = __builtin_amdgcn_readfirstlane(c);
     }
-    // units = (row tile, 32-column tile), row tile major; every workgroup takes one contiguous run
-    const int64_t units = (int64_t)live_tiles * n32;
+    // units = (row tile, K chunk, 32-column tile), column tile fastest; every workgroup takes one contiguous run
+    const int64_t units = (int64_t)live_tiles * per_tile;
     int u = (int)(units * blockIdx.x / gridDim.x);
     const int u_end = (int)(units * (blockIdx.x + 1) / gridDim.x);
 
     while (u < u_end) {
-        const int mt = u / n32, nt0 = u - mt * n32, cnt = min(n32 - nt0, u_end - u);
+        const int mt = u / per_tile, rem = u - mt * per_tile;
+        const int kc = rem / n32, nt0 = rem - kc * n32, cnt = min(n32 - nt0, u_end - u);
         u += cnt;
+        const int kt0 = kc * A.chunk_kt + wave * KTW;
+        const int kcnt = max(0, min(KTW, nkt - kt0));                  // k-tiles of this wavefront in this chunk
         int m0, m_rows;
         const uint8_t* wbase = A.w;
         if (A.tile_expert) {
@@ -980,7 +1058,7 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
         }
         // Source offsets of the raw copies.  32 rows are a multiple of four bytes, so a row's alignment
         // inside its window is the same in every column tile.
-        const uint32_t koff = (uint32_t)kt0 * G::kTileBytes;
+        const uint32_t koff = G::tile_offset(kt0);
         uint32_t w_off[DI];
 #pragma unroll
         for (int i = 0; i < DI; ++i) {
@@ -1010,7 +1088,7 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
             const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
             const int m = m0 + min(ml, m_rows - 1);
             sc[q] = A.xscale[m];
-            coff[q] = (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
+            coff[q] = A.partial ? ((int64_t)kc * A.M + m) * A.N : (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
             ok[q] = ml < m_rows;
         }
 
@@ -1019,11 +1097,12 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
         int b = 0;                                      // buffer of column tile i
         float pend[2] = {0.f, 0.f};
         int pend_n = -1;
+        float* const dst = A.partial ? A.partial : A.c;
         auto flush = [&]() {
             if (pend_n >= 0 && pend_n < A.N) {
 #pragma unroll
                 for (int q = 0; q < 2; ++q)
-                    if (ok[q]) A.c[coff[q] + pend_n] = pend[q];
+                    if (ok[q]) dst[coff[q] + pend_n] = pend[q];
             }
         };
         for (int i = 0; i < cnt; ++i) {
@@ -1044,9 +1123,8 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
                 for (int t = 0; t < KTW; ++t) {
                     if (kFull || t < kcnt) {
                         uint32_t r[G::kRegs], o[16];
-                        if constexpr (G::kSuperBlocks) G::fetch(raw + (t / G::kSup) * G::kSupBytes, t % G::kSup, h, my_delta, r);
-                        else G::fetch(raw, t, h, my_delta, r);
-                        G::dequant(r, G::kSuperBlocks ? t % G::kSup : t, h, my_delta, ((kt0 + t) * 2 + h) * 32 < A.K, o);
+                        G::fetch(raw, t, h, my_delta, r);
+                        G::dequant(r, t, h, my_delta, ((kt0 + t) * 2 + h) * 32 < A.K, o);
 #pragma unroll
                         for (int ks = 0; ks < 4; ++ks) {
                             const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
@@ -1080,6 +1158,41 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
     }
 }
 
+// c[row][n] (+)= sum over the K chunks of partial[kc][m][n], chunks added in order
+__global__ void __launch_bounds__(256) gemm_chunk_sum_kernel(const float* __restrict__ partial, int k_chunks, int M, int N,
+                                                             const int* __restrict__ c_rows, float* __restrict__ c, int64_t ldc,
+                                                             int accumulate)
+{
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    const int m = blockIdx.y;
+    if (n >= N) return;
+    float* out = c + (int64_t)(c_rows ? c_rows[m] : m) * ldc + n;
+    float s = accumulate ? *out : 0.f;
+    for (int kc = 0; kc < k_chunks; ++kc) s += partial[((int64_t)kc * M + m) * N + n];
+    *out = s;
+}
+
+// grow-only device buffer for the K-chunk sums
+float* chunk_buffer(size_t bytes)
+{
+    static std::mutex mu;
+    static void* buf = nullptr;
+    static size_t have = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (bytes > have) {
+        if (buf) {
+            if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return nullptr;
+            (void)hipFree(buf);
+        }
+        buf = nullptr;
+        have = 0;
+        const size_t want = bytes + bytes / 4;
+        if (!hip_ok(hipMalloc(&buf, want), "hipMalloc(K-chunk sums)")) return nullptr;
+        have = want;
+    }
+    return static_cast<float*>(buf);
+}
+
 template <typename G, int KTW>
 bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream)
 {
@@ -1090,33 +1203,53 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream)
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
     a.n_tiles = (a.N + 31) / 32;
-    const int64_t units = (int64_t)m_tiles * a.n_tiles;
+    a.chunk_kt = 8 * KTW;
+    a.k_chunks = (a.Kp / kBK + a.chunk_kt - 1) / a.chunk_kt;
+    a.partial = nullptr;
+    const bool two_pass = a.k_chunks > 1 || a.accumulate;
+    if (two_pass) {
+        a.partial = chunk_buffer((size_t)a.k_chunks * a.M * a.N * sizeof(float));
+        if (!a.partial) return false;
+    }
+    const int64_t units = (int64_t)m_tiles * a.k_chunks * a.n_tiles;
     const int grid = (int)std::min<int64_t>(units, device_info().num_cus);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
-    return hip_ok(hipGetLastError(), "gemm launch");
+    if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
+    if (two_pass) {
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, a.M), dim3(256), 0, stream, a.partial, a.k_chunks, a.M, a.N,
+                           a.c_rows, a.c, a.ldc, a.accumulate);
+        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+    }
+    return true;
 }
 
-// k-tiles per wavefront for which the register-resident kernel is built (0: K too long for it)
+// k-tiles per wavefront of the register-resident kernel: a multiple of the format's block step, at most what two
+// raw buffers per wavefront fit into LDS; a longer K is cut into chunks of 8 x that many k-tiles
+template <typename G, int KTW>
+constexpr bool slim_fits()
+{
+    return (size_t)8 * SlimLayout<G, KTW>::RING * SlimLayout<G, KTW>::BUF + 64 <= 160 * 1024;
+}
+
 template <typename G>
 int slim_ktw(int nkt)
 {
     const int need = (nkt + 7) / 8;
-    constexpr int kStep = G::kSuperBlocks ? G::kSup : 2;
-    constexpr int kMax = G::kTileBytes > 40 ? 4 : 8;       // LDS: 16 raw buffers of 32 rows
-    const int ktw = (need + kStep - 1) / kStep * kStep;
-    return ktw <= kMax ? ktw : 0;
+    const int ktw = (need + G::kTileStep - 1) / G::kTileStep * G::kTileStep;
+    const int limit = slim_fits<G, 8>() ? 8 : slim_fits<G, 6>() && G::kTileStep == 2 ? 6 : 4;
+    return ktw <= limit ? ktw : limit;       // longer K: chunks of 8 * limit k-tiles
 }
 
 template <typename G>
 bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream)
 {
-    if constexpr (!G::kSuperBlocks) {
+    if constexpr (G::kTileStep == 2) {
         if (ktw == 2) return launch_slim<G, 2>(a, m_tiles, stream);
-        if constexpr (G::kTileBytes <= 40)
+        if constexpr (slim_fits<G, 6>())
             if (ktw == 6) return launch_slim<G, 6>(a, m_tiles, stream);
     }
     if (ktw == 4) return launch_slim<G, 4>(a, m_tiles, stream);
-    if constexpr (G::kTileBytes <= 40)
+    if constexpr (slim_fits<G, 8>())
         if (ktw == 8) return launch_slim<G, 8>(a, m_tiles, stream);
     set_last_error("gemm: no register-resident kernel for this K.");
     return false;
@@ -1125,22 +1258,24 @@ bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-    if (bm == 32) {
-        const int ktw = a.accumulate ? 0 : slim_ktw<G>(a.Kp / kBK);
-        if (ktw) return launch_slim_for<G>(a, ktw, m_tiles, stream);
-        // longer K: the 64-row kernel takes 32-row tiles as half-empty ones
+    if (bm == 32 && a.M <= 65535) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream);
+    if constexpr (G::kRawRow <= 144) {
+        if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
     }
-    if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
     // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
     // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 the other way round
-    if (bm == 128) return G::kSup == 2 ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream) : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream);
+    if (bm == 128)
+        return (G::kSup == 2 || G::kRawRow > 144) ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream)
+                                                   : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream);
 #ifdef TSHIP_GEMM_NO_FEW_ROWS
     return launch_tiles<G, 64, 4, 8>(a, m_tiles, stream);
 #else
 #ifdef TSHIP_GEMM_FEW_ROWS_ONE_WG
     return launch_few_rows<G, 8, 3>(a, m_tiles, stream);
 #else
-    return launch_few_rows<G, 4, 2>(a, m_tiles, stream);
+    // wide raw rows (Q6_K): one 8-wavefront workgroup per CU instead of two 4-wavefront ones
+    if constexpr (G::kRawRow > 144) return launch_few_rows<G, 8, 2>(a, m_tiles, stream);
+    else return launch_few_rows<G, 4, 2>(a, m_tiles, stream);
 #endif
 #endif
 }
@@ -1177,6 +1312,7 @@ bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspa
     case kTypeQ4_K: launch_convert_typed<kTypeQ4_K, SRC>(src, M, K, kp, x16, scales, stream); break;
     case kTypeMXFP4: launch_convert_typed<kTypeMXFP4, SRC>(src, M, K, kp, x16, scales, stream); break;
     case kTypeQ8_0: launch_convert_typed<kTypeQ8_0, SRC>(src, M, K, kp, x16, scales, stream); break;
+    case kTypeQ6_K: launch_convert_typed<kTypeQ6_K, SRC>(src, M, K, kp, x16, scales, stream); break;
     default: set_last_error("gemm: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "activation convert launch");
@@ -1244,6 +1380,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
         m_tiles = tiles->count;
     } else {
         bm = gemm_tile_m(M);
+        if (type == kTypeQ6_K && bm == 256) bm = 128;     // two raw Q6_K super-tiles of 256 rows do not fit LDS
         m_tiles = (M + bm - 1) / bm;
     }
     if (m_tiles == 0) return true;
@@ -1251,6 +1388,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     case kTypeQ4_K: return launch_for_type<GQ4K>(a, bm, m_tiles, stream);
     case kTypeMXFP4: return launch_for_type<GMXFP4>(a, bm, m_tiles, stream);
     case kTypeQ8_0: return launch_for_type<GQ80>(a, bm, m_tiles, stream);
+    case kTypeQ6_K: return launch_for_type<GQ6K>(a, bm, m_tiles, stream);
     default: set_last_error("gemm: unsupported type."); return false;
     }
 }

@@ -9,9 +9,19 @@
 
 namespace tship {
 
+// GGUF tensor type ids (TensorSharp.Runtime/GgufReader.cs:26-37)
 constexpr int kTypeF32 = 0;
+constexpr int kTypeF16 = 1;
+constexpr int kTypeQ4_0 = 2;
+constexpr int kTypeQ4_1 = 3;
+constexpr int kTypeQ5_0 = 6;
+constexpr int kTypeQ5_1 = 7;
 constexpr int kTypeQ8_0 = 8;
 constexpr int kTypeQ4_K = 12;
+constexpr int kTypeQ5_K = 13;
+constexpr int kTypeQ6_K = 14;
+constexpr int kTypeIQ4_NL = 20;
+constexpr int kTypeBF16 = 30;
 constexpr int kTypeMXFP4 = 39;
 
 // elements per block / bytes per block; 0 for unsupported types
@@ -23,6 +33,9 @@ inline int64_t block_elems(int type)
     case kTypeQ8_0: return 32;
     case kTypeQ4_K: return 256;
     case kTypeMXFP4: return 32;
+    case kTypeF16: case kTypeBF16: return 1;
+    case kTypeQ4_0: case kTypeQ4_1: case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL: return 32;
+    case kTypeQ5_K: case kTypeQ6_K: return 256;
     default: return 0;
     }
 }
@@ -34,11 +47,23 @@ inline int64_t block_bytes(int type)
     case kTypeQ8_0: return 34;
     case kTypeQ4_K: return 144;
     case kTypeMXFP4: return 17;
+    case kTypeF16: case kTypeBF16: return 2;
+    case kTypeQ4_0: case kTypeIQ4_NL: return 18;
+    case kTypeQ4_1: return 20;
+    case kTypeQ5_0: return 22;
+    case kTypeQ5_1: return 24;
+    case kTypeQ5_K: return 176;
+    case kTypeQ6_K: return 210;
     default: return 0;
     }
 }
 
-inline bool is_quant_type(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4; }
+// formats the matmul kernels read (Q6_K through the matrix-core kernels only: no GEMV specialisation)
+inline bool is_quant_type(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4 || type == kTypeQ6_K; }
+inline bool has_gemv(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4; }
+// formats with a dequantizer (DequantizeToF32, embedding gather): every block format the managed code reads
+// (ManagedQuantizedOps.cs:40-59) except Q8_1
+inline bool is_dequant_type(int type) { return type != kTypeF32 && block_elems(type) != 0; }
 
 void set_last_error(const std::string& msg);
 void clear_last_error();

@@ -14,6 +14,7 @@ LIB_PATH = os.environ.get("TSHIP_LIBRARY") or os.path.join(HERE, "libTsHipOps.so
 
 BACKEND_HIP = 4
 TYPE_F32, TYPE_Q8_0, TYPE_Q4_K, TYPE_MXFP4 = 0, 8, 12, 39
+TYPE_F16, TYPE_Q4_0, TYPE_Q4_1, TYPE_Q5_0, TYPE_Q5_1, TYPE_Q5_K, TYPE_Q6_K, TYPE_IQ4_NL, TYPE_BF16 = 1, 2, 3, 6, 7, 13, 14, 20, 30
 DTYPE_F32, DTYPE_I32 = 0, 3
 
 

@@ -1,6 +1,6 @@
 """Synthetic GGUF block generators (torch, run on whatever device the input lives on).
 
-Benchmarks need W ~ N(0, 0.02) in raw Q8_0 / Q4_K / MXFP4 blocks without touching the CPU
+Benchmarks need W ~ N(0, 0.02) in raw Q8_0 / Q4_K / Q6_K / MXFP4 blocks without touching the CPU
 oracle.  Q8_0 and MXFP4 follow the reference quantizers exactly (closed forms,
 ggml-quants.c:199-222 and :260-305).  Q4_K uses a plain min/max affine fit per 32-weight
 sub-block instead of the reference's iterative scale search (ggml-quants.c:622-701): the
@@ -75,7 +75,30 @@ def quantize_q4_k_simple(w):
     return out.reshape(-1)
 
 
-QUANTIZERS = {8: quantize_q8_0, 12: quantize_q4_k_simple, 39: quantize_mxfp4}
+def quantize_q6_k_simple(w):
+    """Valid Q6_K blocks (ggml-common.h block_q6_K) from a plain absmax fit per 16-weight group, not the reference's
+    iterative search (ggml-quants.c quantize_row_q6_K_ref): same layout and statistics, not the reference's bytes."""
+    x = w.reshape(-1, 16, 16).float()                    # [blocks, groups, 16]
+    nb = x.shape[0]
+    scale = x.abs().amax(dim=2) / 31.0                   # per group step
+    d = scale.amax(dim=1) / 127.0
+    d16 = d.to(torch.float16).float()
+    sc = torch.where(d16[:, None] > 0, torch.round(scale / d16[:, None].clamp_min(1e-30)), torch.zeros_like(scale)).clamp(1, 127)
+    eff = d16[:, None] * sc
+    q = torch.where(eff[:, :, None] > 0, torch.round(x / eff[:, :, None].clamp_min(1e-30)), torch.zeros_like(x)).clamp(-32, 31)
+    q = (q + 32).to(torch.uint8).reshape(nb, 2, 4, 32)   # [block, half, group of 32, l]
+    out = torch.zeros((nb, 210), dtype=torch.uint8, device=w.device)
+    lo, hi = q & 0x0F, q >> 4
+    ql = out[:, 0:128].reshape(nb, 2, 2, 32)             # [block, half, l / 32, l % 32]
+    ql[:, :, 0, :] = lo[:, :, 0, :] | (lo[:, :, 2, :] << 4)
+    ql[:, :, 1, :] = lo[:, :, 1, :] | (lo[:, :, 3, :] << 4)
+    out[:, 128:192] = (hi[:, :, 0, :] | (hi[:, :, 1, :] << 2) | (hi[:, :, 2, :] << 4) | (hi[:, :, 3, :] << 6)).reshape(nb, 64)
+    out[:, 192:208] = sc.to(torch.int8).view(torch.uint8)
+    out[:, 208:210] = _half_bytes(d)
+    return out.reshape(-1)
+
+
+QUANTIZERS = {8: quantize_q8_0, 12: quantize_q4_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
 
 
 def random_weight(ggml_type, n_rows, n_cols, device, seed, sigma=0.02, chunk_rows=4096):

@@ -74,8 +74,50 @@ def test_codes(hip):
     out = np.zeros(256, dtype=np.float32)
     assert lib.TSHip_DequantizeToF32(Q4_K, None, 256, out.ctypes.data) == -1
     assert lib.TSHip_DequantizeToF32(Q4_K, buf.ctypes.data, 255, out.ctypes.data) == -1
-    assert lib.TSHip_DequantizeToF32(14, buf.ctypes.data, 256, out.ctypes.data) == -2     # Q6_K: not on this path
+    assert lib.TSHip_DequantizeToF32(10, buf.ctypes.data, 256, out.ctypes.data) == -2     # Q2_K: no dequantizer here
     assert lib.TSHip_DequantizeToF32(Q4_K, buf.ctypes.data, 0, out.ctypes.data) == 0
     src = np.arange(8, dtype=np.float32)
     dst = np.zeros(8, dtype=np.float32)
     assert lib.TSHip_DequantizeToF32(0, src.ctypes.data, 8, dst.ctypes.data) == 0 and np.array_equal(src, dst)
+
+
+# ---- the other block formats the managed code reads (ManagedQuantizedOps.cs:40-59) ----------------------------
+from oracle.oracle import MORE_TYPES, BLOCK  # noqa: E402
+import os  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def formats():
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "formats.npz"))
+
+
+@pytest.mark.parametrize("name", sorted(MORE_TYPES))
+def test_more_formats_reference_known_answers(hip, formats, name):
+    # bytes and floats written by the reference's own quantizers / dequantizers (tests/golden/make_golden_formats.py)
+    t = MORE_TYPES[name]
+    for q, want in ((formats[f"{name}_q"], formats[f"{name}_deq"]), (formats[f"{name}_rq"], formats[f"{name}_rdeq"])):
+        assert bits_equal(hip.DequantizeToFloat32(t, q, want.size), want), name
+
+
+@pytest.mark.parametrize("name", sorted(MORE_TYPES))
+def test_more_formats_random_bytes_and_row_gather(hip, oracle, name):
+    import torch
+    t = MORE_TYPES[name]
+    bs, bb = BLOCK[t]
+    rng = np.random.default_rng(23 + t)
+    K = 512
+    rows = 300
+    raw = rng.integers(0, 256, size=rows * (K // bs) * bb, dtype=np.uint8)
+    want = oracle.dequantize(t, raw)
+    dev = torch.from_numpy(raw).cuda()
+    out = hip.DequantizeToFloat32Device(t, dev, want.size)
+    torch.cuda.synchronize()
+    assert bits_equal(out.cpu().numpy(), want)
+    # embedding gather of the same rows
+    idx = np.array([299, 0, 17, 150, 17], dtype=np.int32)
+    res = np.full((idx.size, K), 7.0, dtype=np.float32)
+    hip.GetRowsQuant(res, raw.ctypes.data, t, K, rows, raw.size, idx)
+    w = want.reshape(rows, K)
+    for i, r in enumerate(idx):
+        assert bits_equal(res[i], w[r]), (name, i)
+    hip.ClearHostBufferCache()

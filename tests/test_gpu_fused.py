@@ -33,7 +33,7 @@ def qweights(name, arrs, device):
 
 
 @pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
-@pytest.mark.parametrize("M", [1, 3, 40])
+@pytest.mark.parametrize("M", [1, 3, 9, 40])
 @pytest.mark.parametrize("device", [False, True])
 def test_rms_norm_matmul(hip, oracle, name, M, device):
     import torch
@@ -85,7 +85,7 @@ def test_matmul_add_in_place(hip, oracle, name, M, device):
 
 
 @pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
-@pytest.mark.parametrize("M", [1, 3, 48])
+@pytest.mark.parametrize("M", [1, 3, 9, 48])
 @pytest.mark.parametrize("device", [False, True])
 def test_ffn_swiglu(hip, oracle, name, M, device):
     import torch
@@ -147,3 +147,32 @@ def test_rms_norm_matmul_row_longer_than_one_staging_pass(hip, oracle, name):
     torch.cuda.synchronize()
     ok, worst = bound_ok(res.cpu().numpy(), ref, ref)
     assert ok, (name, worst)
+
+
+@pytest.mark.parametrize("M", [1, 40])
+def test_ffn_swiglu_q4_k_gate_up_q6_k_down(hip, oracle, M):
+    # the mix of a Q4_K_M file: gate/up in Q4_K, down in Q6_K (no GEMV specialisation: matrix-core path at M = 1 too)
+    import torch
+    from oracle.oracle import Q6_K
+    from tensorsharp_amd import QuantizedWeight, synth
+    rng = np.random.default_rng(97 + M)
+    H, F = 512, 768
+    gu = make(oracle, "q4_k", 2 * F, H, rng, 0.05)
+    g = torch.Generator()
+    g.manual_seed(9)
+    dn = synth.quantize_q6_k_simple(torch.randn((H, F), generator=g) * 0.05).numpy()
+    x = (rng.standard_normal((M, H)) * 2).astype(np.float32)
+    resid = rng.standard_normal((M, H)).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    xn = oracle.rms_norm_mul(x, nw, EPS)
+    act = oracle.silu_mul(oracle.matmul_f64(Q4_K, gu, 2 * F, H, xn).astype(np.float32))
+    mm = oracle.matmul_f64(Q6_K, dn, H, F, act)
+    ref = resid.astype(np.float64) + mm
+    r = torch.from_numpy(resid.copy()).cuda()
+    hip.FusedFFNSwiGLUQuant(r, torch.from_numpy(x).cuda(), torch.from_numpy(nw).cuda(), EPS,
+                            QuantizedWeight(torch.from_numpy(gu).cuda(), Q4_K, H, 2 * F),
+                            QuantizedWeight(torch.from_numpy(dn).cuda(), Q6_K, F, H), F)
+    torch.cuda.synchronize()
+    tol = 2e-3 * np.linalg.norm(mm, axis=1, keepdims=True)
+    got = r.cpu().numpy()
+    assert np.all(np.abs(got - ref) <= tol), (M, float(np.max(np.abs(got - ref) / tol)))

@@ -141,14 +141,17 @@ def test_weight_view_at_odd_address(hip, oracle, name, row_bytes, M):
     ("mxfp4", 17, 9001, 4096),    # eight k-tiles per wavefront, two raw buffers
     ("mxfp4", 5, 3000, 1024),     # two k-tiles per wavefront
     ("mxfp4", 31, 2000, 2048),    # four
-    ("mxfp4", 9, 1500, 4160),     # K too long for the register-resident kernel: 64-row kernel
+    ("mxfp4", 9, 1500, 4160),     # K longer than one chunk of the register-resident kernel: two chunks, summed
+    ("mxfp4", 30, 700, 8192 + 64),
     ("q4_k", 32, 9000, 2048),
     ("q4_k", 12, 14336, 4096),
-    ("q4_k", 20, 1000, 4352),     # too long
+    ("q4_k", 20, 1000, 4352),     # two chunks
+    ("q4_k", 8, 4096, 14336),     # four chunks, few columns
     ("q4_k", 6, 333, 256),        # a single k-tile group: seven of the eight wavefronts have no K range
     ("q8_0", 32, 3000, 1024),
     ("q8_0", 11, 7000, 2048),
-    ("q8_0", 25, 900, 2080),      # too long
+    ("q8_0", 25, 900, 2080),      # two chunks
+    ("q8_0", 5, 300, 6176),       # four chunks, the last one a single block
     ("q8_0", 4, 40, 32),          # one block per row
 ])
 def test_at_most_32_rows(hip, oracle, name, M, N, K):
@@ -158,3 +161,42 @@ def test_at_most_32_rows(hip, oracle, name, M, N, K):
     x = rng.standard_normal((M, K)).astype(np.float32)
     y = run_device(hip, T[name], wq, N, K, x)
     check(y, oracle.matmul_f64(T[name], wq, N, K, x), (name, M, N, K))
+
+
+# ---- Q6_K (the format Q4_K_M files use for the output matrix and some projections): matrix-core kernels only ----
+def q6k_weight(N, K, seed):
+    import torch
+    from tensorsharp_amd import synth
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return synth.quantize_q6_k_simple(torch.randn((N, K), generator=g) * 0.02).numpy()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 2048), (3, 333, 256), (4, 128, 256), (32, 3000, 2048), (17, 700, 4096),
+                                   (1, 4096, 14336), (2, 600, 2304),
+                                   (33, 130, 768), (64, 600, 1024), (65, 257, 2304), (128, 256, 1024), (200, 77, 2048),
+                                   (1100, 300, 768)])
+def test_q6_k_shapes(hip, oracle, M, N, K):
+    from oracle.oracle import Q6_K
+    rng = np.random.default_rng(M * 31 + N + K)
+    wq = q6k_weight(N, K, M + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, Q6_K, wq, N, K, x)
+    check(y, oracle.matmul_f64(Q6_K, wq, N, K, x), ("q6_k", M, N, K))
+
+
+@pytest.mark.parametrize("M", [2, 40, 150])
+def test_q6_k_rows_two_bytes_off(hip, oracle, M):
+    # K = 256 * odd and a view from row 1: rows start 2 bytes off a dword, and so does every second block
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    from oracle.oracle import Q6_K
+    rng = np.random.default_rng(73 + M)
+    N, K = 200, 256 * 3
+    wq = q6k_weight(N, K, 5)
+    row_bytes = 210 * 3
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    dev = torch.from_numpy(wq).cuda()
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(dev[row_bytes:], Q6_K, K, N - 1))
+    torch.cuda.synchronize()
+    check(y.cpu().numpy(), oracle.matmul_f64(Q6_K, wq[row_bytes:], N - 1, K, x), ("q6_k view", M))

@@ -116,3 +116,117 @@ def test_error_codes(oracle):
     assert oracle.lib.tso_dequantize(77, C.c_void_p(buf.ctypes.data), 32, out.ctypes.data_as(f32p)) == -2
     assert oracle.lib.tso_dequantize(8, C.c_void_p(buf.ctypes.data), 33, out.ctypes.data_as(f32p)) == -1
     assert oracle.lib.tso_dequantize(8, C.c_void_p(buf.ctypes.data), 0, out.ctypes.data_as(f32p)) == 0
+
+
+# ---- formats beyond the three matmul formats (ManagedQuantizedOps.cs:268-409, :481-577) -------------------
+from oracle.oracle import MORE_TYPES, BLOCK, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q6_K, IQ4_NL, F16, BF16  # noqa: E402
+import os  # noqa: E402
+import pytest  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def formats():
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "formats.npz"))
+
+
+@pytest.mark.parametrize("name", sorted(MORE_TYPES))
+def test_more_formats_match_the_reference_build(oracle, formats, name):
+    # known answers written by the reference's own dequantizers (tests/golden/make_golden_formats.py)
+    t = MORE_TYPES[name]
+    for q, want in ((formats[f"{name}_q"], formats[f"{name}_deq"]), (formats[f"{name}_rq"], formats[f"{name}_rdeq"])):
+        y = oracle.dequantize(t, q)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), name
+
+
+def _f16(raw2):
+    return np.ascontiguousarray(raw2).view(np.float16).astype(np.float64)[:, 0]
+
+
+def test_q6_k_closed_form(oracle):
+    # every value is d * scale * (q - 32) with an 11-bit d, an 8-bit scale and a 6-bit q: exact in fp32, so an
+    # fp64 evaluation of the layout (ggml-common.h block_q6_K) must agree to the bit
+    rng = np.random.default_rng(5)
+    nb = 2048
+    raw = rng.integers(0, 256, size=(nb, 210), dtype=np.uint8)
+    raw[:, 209] &= 0x7B
+    y = oracle.dequantize(Q6_K, raw.reshape(-1)).reshape(nb, 256)
+    d = _f16(raw[:, 208:210])
+    sc = raw[:, 192:208].view(np.int8).astype(np.float64)
+    want = np.empty((nb, 256))
+    for e in range(256):
+        half, r = divmod(e, 128)
+        grp, l = divmod(r, 32)
+        qlb = raw[:, 64 * half + 32 * (grp & 1) + l]
+        nib = (qlb >> 4) if grp >= 2 else (qlb & 0x0F)
+        hi = (raw[:, 128 + 32 * half + l] >> (2 * grp)) & 3
+        q = (nib | (hi << 4)).astype(np.float64) - 32
+        want[:, e] = d * sc[:, 8 * half + 2 * grp + l // 16] * q
+    assert np.array_equal(y.astype(np.float64), want)
+
+
+def test_q5_k_closed_form(oracle):
+    rng = np.random.default_rng(6)
+    nb = 2048
+    raw = rng.integers(0, 256, size=(nb, 176), dtype=np.uint8)
+    raw[:, 1] &= 0x7B
+    raw[:, 3] &= 0x7B
+    y = oracle.dequantize(Q5_K, raw.reshape(-1)).reshape(nb, 256)
+    d = _f16(raw[:, 0:2]).astype(np.float32)
+    dmin = _f16(raw[:, 2:4]).astype(np.float32)
+    p = raw[:, 4:16]
+    want = np.empty((nb, 256), dtype=np.float32)
+    for j in range(8):
+        sc, mn = _scale_min(j, p)
+        d1 = d * sc.astype(np.float32)
+        m1 = dmin * mn.astype(np.float32)
+        g, hi = divmod(j, 2)
+        qb = raw[:, 48 + 32 * g:48 + 32 * g + 32]
+        nib = (qb >> 4) if hi else (qb & 0x0F)
+        bit = (raw[:, 16:48] >> j) & 1
+        q = (nib + 16 * bit).astype(np.float32)
+        want[:, 32 * j:32 * j + 32] = d1[:, None] * q - m1[:, None]
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("t,hdr,bias,has_min", [(Q4_0, 2, 8, False), (Q4_1, 4, 0, True), (Q5_0, 6, 16, False), (Q5_1, 8, 0, True)])
+def test_legacy_32_blocks_closed_form(oracle, t, hdr, bias, has_min):
+    rng = np.random.default_rng(7 + t)
+    nb = 4096
+    bb = BLOCK[t][1]
+    raw = rng.integers(0, 256, size=(nb, bb), dtype=np.uint8)
+    raw[:, 1] &= 0x7B
+    if has_min:
+        raw[:, 3] &= 0x7B
+    y = oracle.dequantize(t, raw.reshape(-1)).reshape(nb, 32)
+    d = _f16(raw[:, 0:2]).astype(np.float32)
+    m = _f16(raw[:, 2:4]).astype(np.float32) if has_min else None
+    qs = raw[:, hdr:hdr + 16]
+    q = np.concatenate([qs & 0x0F, qs >> 4], axis=1).astype(np.int32)
+    if t in (Q5_0, Q5_1):
+        qh = raw[:, hdr - 4:hdr].copy().view(np.uint32)[:, 0]
+        bits = (qh[:, None] >> np.arange(32)[None, :]) & 1
+        q = q + 16 * bits.astype(np.int32)
+    want = (q - bias).astype(np.float32) * d[:, None]
+    if has_min:
+        want = want + m[:, None]
+    assert np.array_equal(y.view(np.uint32), want.astype(np.float32).view(np.uint32))
+
+
+def test_iq4_nl_f16_bf16_closed_form(oracle):
+    rng = np.random.default_rng(8)
+    table = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
+    raw = rng.integers(0, 256, size=(4096, 18), dtype=np.uint8)
+    raw[:, 1] &= 0x7B
+    y = oracle.dequantize(IQ4_NL, raw.reshape(-1)).reshape(-1, 32)
+    d = _f16(raw[:, 0:2]).astype(np.float32)
+    qs = raw[:, 2:]
+    want = d[:, None] * table[np.concatenate([qs & 0x0F, qs >> 4], axis=1)]
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    # every fp16 / bf16 code
+    codes = np.arange(65536, dtype=np.uint16)
+    y = oracle.dequantize(F16, codes.view(np.uint8))
+    want = codes.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(want)
+    assert np.array_equal(y.view(np.uint32)[ok], want.view(np.uint32)[ok])
+    y = oracle.dequantize(BF16, codes.view(np.uint8))
+    assert np.array_equal(y.view(np.uint32), codes.astype(np.uint32) << 16)
