@@ -778,10 +778,10 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
         hipStream_t stream = g_stream.load();
         auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
         const bool small = A <= gemv_max_group() && H <= gemv_max_k(ggml_type) && F <= gemv_max_k(ggml_type);
-        // rows per tile of the grouped GEMMs: with few tokens per expert the 32-row register-resident kernel
-        // streams the weights fastest, even though experts with 33..64 rows then take two tiles
+        // rows per tile of the grouped GEMMs: up to about 160 tokens per expert the 32-row register-resident kernel
+        // is fastest (measured at 32 experts of 2880 x 2880: T = 256 ... 1024), beyond that 128-row tiles
         const int per_expert = A / E;
-        const int bm = per_expert > 96 ? 128 : per_expert > 40 ? 64 : 32;
+        const int bm = per_expert > 160 ? 128 : 32;
         const int max_tiles = A / bm + E;
         // carve the workspace
         size_t off = 0;

@@ -5,8 +5,8 @@
 //      magnitude overflows or underflows fp16), written in the k-order in which the weight
 //      format unpacks (so the dequantizer never has to shuffle lanes), zero-padded to a
 //      multiple of the k-tile.  Optionally gathers rows through an index (MoE).
-//   2. gemm_kernel (M > 64 per tile) / gemm_few_rows_kernel (M <= 64 per tile, persistent workgroups) /
-//      gemm_slim_kernel (M <= 32 per tile: activations in registers, K split over the wavefronts, long K in chunks):
+//   2. gemm_slim_kernel (32 rows per tile: activations in registers, K split over the wavefronts, long K in
+//      chunks; used up to a few hundred rows, see gemm_tile_m) and gemm_kernel (128 / 256 rows per tile):
 //      BM x 256 x 64 tiles, eight wavefronts, each owning 32 output columns.  The fp16
 //      activation k-tiles and the RAW quantized bytes of 256 weight rows (one 144-byte window per row
 //      covering four k-tiles of Q4_K / MXFP4 or two of Q8_0) are copied from global memory straight
@@ -501,8 +501,8 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
 //   * Activations run XST - 1 k-tiles ahead in XST LDS stages, weight super-tiles RL super-tiles ahead in
 //     RL + 1 buffers.  Every wavefront issues the same number of copies per iteration (surplus copies use
 //     an out-of-range source and a dump area), so the wait before the barrier is a vmcnt that leaves the
-//     younger copies in flight: the few-row tiles (XST = 4), whose speed is the speed of streaming the
-//     weights, keep three k-tiles of requests outstanding.
+//     younger copies in flight (XST = 4 keeps three k-tiles of requests outstanding; the configurations in use
+//     are double-buffered, XST = 2).
 //   * A lane (column n, k-half h) unpacks ITS OWN B operands from the raw bytes into registers one
 //     k-tile ahead, so dequantized weights never travel through LDS and every weight is unpacked by
 //     exactly one lane of the workgroup.  One barrier per k-tile.
@@ -647,32 +647,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         const uint32_t dn = G::sup_delta(my_delta, sn);
         G::fetch(rbuf + rbn * RT + my_raw, jn, h, dn, r);
         const uint8_t* xs = xbuf + xst * kXTile;
-        if constexpr (TM <= 2) {
-            // few rows: every A operand of the k-tile is requested up front
-            half8_t a[4][TM];
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int i = 0; i < TM; ++i) a[ks][i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[ks]);
-            __builtin_amdgcn_sched_barrier(0);
-#ifndef TSHIP_GEMM_DEBUG_NODEQ
-            G::dequant(r, jn, h, dn, ((kt + 1) * 2 + h) * 32 < A.K, on);
-#else
-            _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs];
-#endif
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const uint4_t bb = {oc[4 * ks], oc[4 * ks + 1], oc[4 * ks + 2], oc[4 * ks + 3]};
-                const half8_t b = __builtin_bit_cast(half8_t, bb);
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#ifndef TSHIP_GEMM_DEBUG_NOMMA
-                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks][i], b, acc[i], 0, 0, 0);
-#else
-                    acc[i][0] += (float)a[ks][i][0] * (float)b[0];
-#endif
-            }
-        } else {
+        {
             half8_t a[TM];
 #pragma unroll
             for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[0]);
@@ -735,245 +710,14 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
 }
 
 // ------------------------------------------------------------------------------------------
-// Few activation rows (at most 64 per tile: small batches, MoE experts).  The weights are read once, so
-// the speed limit is streaming them and what counts is bytes in flight.  Same 64-row x 256-column tile
-// and operand scheme as above, but one iteration covers TWO k-tiles, the activations live in a ring of
-// three such pairs (requested two iterations ahead) and the raw weight super-tiles in three buffers
-// (requested two super-tiles ahead).  Per iteration a wavefront issues its LDS-direct copies after its
-// LDS reads and leaves this iteration's copies in flight at the barrier (counted vmcnt).
-// ------------------------------------------------------------------------------------------
-// per-tile state of a persistent workgroup
-template <int NW, int RAW_ROW>
-struct FewRowsTile {
-    int m0, m_rows, my_n;
-    uint32_t my_delta;
-    __amdgpu_buffer_rsrc_t wrs;
-    uint32_t x_off[8 / NW];
-    uint32_t w_off[(NW * 32 * RAW_ROW / 1024 + NW - 1) / NW];
-};
-
-// NW wavefronts (32 columns each), RING buffers for activations (in k-tile pairs) and for raw super-tiles:
-// 8 / 3 is one workgroup per CU with requests two iterations ahead, 4 / 2 two workgroups per CU with
-// requests one iteration ahead (the two workgroups drift apart, so one computes while the other waits).
-template <typename G, int NW, int RING>
-__global__ void __launch_bounds__(NW * 64) gemm_few_rows_kernel(const GemmArgs A)
-{
-    constexpr int BM = 64, TM = 2, KS = G::kSup;
-    constexpr int kRawRow = G::kRawRow, kRowChunks = kRawRow / 16;
-    using Tile = FewRowsTile<NW, G::kRawRow>;
-    constexpr int BN = NW * 32, RT = BN * kRawRow, RIN = RT / 1024, WI = (RIN + NW - 1) / NW, XI = 8 / NW;
-    static_assert(RIN * 1024 == RT && XI * NW == 8, "tile must split into whole copies");
-    static_assert(RING == 2 || RING == 3, "ring of two or three");
-    constexpr int kXTile = BM * kXRow;                   // one k-tile of activations: 8 KiB, one copy per wavefront
-    constexpr int kXPair = 2 * kXTile;
-    constexpr int HPS = KS / 2;                          // iterations (k-tile pairs) per weight super-tile: 2 or 1
-    extern __shared__ uint8_t smem[];
-    uint8_t* const xbuf = smem;                          // RING x kXPair
-    uint8_t* const rbuf = smem + RING * kXPair;          // RING x RT
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int col = lane & 31, h = lane >> 5;
-
-    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
-    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
-    const int nkt = A.Kp / kBK;
-    const int npair = (nkt + 1) / 2;
-    const int my_raw = (wave * 32 + col) * kRawRow;
-    // the copies of a raw super-tile do not divide evenly: the first wavefronts issue WI, the others WI - 1
-    const bool five = wave + NW * (WI - 1) < RIN;
-    const int sw = (col >> 1) & 7;
-    int a_off[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) a_off[ks] = col * kXRow + ((2 * ks + h) ^ sw) * 16;
-
-    // Persistent workgroups: the tiles of an XCD (a contiguous run, so that neighbours share the activation
-    // rows in that XCD's L2) are dealt round-robin to the workgroups that landed on it.
-    const int total = A.m_tiles * A.n_tiles;
-    const int per = (total + 7) >> 3;
-    const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
-    int slot = blockIdx.x >> 3;
-
-    // next tile with work at or after `slot` (grouped launches may list empty tiles); false when none is left
-    auto setup = [&](Tile& T) -> bool {
-        for (; slot < per; slot += stride) {
-            const int t = xcd * per + slot;
-            if (t >= total) return false;
-            const int mt = t / A.n_tiles, nt = t - mt * A.n_tiles;
-            const uint8_t* wbase = A.w;
-            if (A.tile_expert) {
-                T.m0 = A.tile_row0[mt];
-                T.m_rows = A.tile_rows[mt];
-                if (T.m_rows <= 0) continue;
-                wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
-            } else {
-                T.m0 = mt * BM;
-                T.m_rows = min(BM, A.M - T.m0);
-            }
-            const int n0 = nt * BN;
-            const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
-            const uint32_t base_delta = (uint32_t)(wa & 3);
-            T.wrs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0,
-                                                      (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
-#pragma unroll
-            for (int i = 0; i < XI; ++i) {
-                const int q = (wave + NW * i) * 64 + lane;
-                const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
-                T.x_off[i] = row < T.m_rows ? (uint32_t)(T.m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
-            }
-#pragma unroll
-            for (int i = 0; i < WI; ++i) {
-                const int c = (wave + NW * i) * 64 + lane;
-                const int row = c / kRowChunks, chunk = c - row * kRowChunks;
-                T.w_off[i] = (row < BN && n0 + row < A.N)
-                                 ? ((base_delta + (uint32_t)(n0 + row) * row_bytes) & ~3u) + (uint32_t)chunk * 16u
-                                 : kDeadOffset;
-            }
-            T.my_n = n0 + wave * 32 + col;
-            T.my_delta = T.my_n < A.N ? (base_delta + (uint32_t)T.my_n * row_bytes) & 3u : 0u;
-            slot += stride;
-            return true;
-        }
-        return false;
-    };
-    // always the same number of copies per wavefront (sources past the end are out of range: zeros)
-    auto issue_x = [&](const Tile& T, int p) {            // k-tile pair p -> ring slot p % RING
-        uint8_t* dst = xbuf + (p % RING) * kXPair;
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const int kt = 2 * p + e;
-#pragma unroll
-            for (int i = 0; i < XI; ++i) {
-                // a copy covers 8 activation rows; with at most 32 live rows the upper half of the tile is never
-                // read (only where no copy count is kept: RING 2 waits for every copy)
-                if (RING == 2 && T.m_rows <= 32 && (wave + NW * i) * 8 >= 32) continue;
-                copy16_to_lds(xrs, dst + e * kXTile + (wave + NW * i) * 1024, kt < nkt ? T.x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
-            }
-        }
-    };
-    auto issue_w = [&](const Tile& T, int s) {            // super-tile s -> buffer s % RING
-        uint8_t* buf = rbuf + (s % RING) * RT;
-        const bool any = s * KS < nkt;
-#pragma unroll
-        for (int i = 0; i < WI; ++i) {
-            const int id = wave + NW * i;
-            if (id < RIN) copy16_to_lds(T.wrs, buf + id * 1024, any ? T.w_off[i] : kDeadOffset, G::sup_offset(s));
-        }
-    };
-    auto issue_first = [&](const Tile& T) {
-#pragma unroll
-        for (int i = 0; i < RING - 1; ++i) issue_x(T, i);
-#pragma unroll
-        for (int i = 0; i < RING - 1; ++i) issue_w(T, i);
-    };
-
-    Tile T;
-    if (!setup(T)) return;
-    issue_first(T);
-    for (;;) {
-        __syncthreads();                   // the first two k-tile pairs and super-tiles of this tile have landed
-        float16_t acc[TM];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
-
-        // tiles with at most 32 live rows skip the upper 32 x 32 accumulator block (its copies, LDS reads and MFMAs)
-        auto run = [&](auto rows_tag) {
-            constexpr int TMX = decltype(rows_tag)::value;
-            for (int p = 0; p < npair; ++p) {
-                const int s = p / HPS, e0 = (p % HPS) * 2;           // super-tile and first k-tile inside it
-                const uint8_t* raw = rbuf + (s % RING) * RT + my_raw;
-                const uint8_t* xs = xbuf + (p % RING) * kXPair;
-                uint32_t r[2][G::kRegs];
-                half8_t a[2][4][TMX];
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-#ifdef TSHIP_FR_NOFETCH
-                    _Pragma("unroll") for (int q = 0; q < G::kRegs; ++q) r[e][q] = 0x3c003c00u + q + p;
-#else
-                    G::fetch(raw, e0 + e, h, G::sup_delta(T.my_delta, s), r[e]);
-#endif
-#pragma unroll
-                    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                        for (int i = 0; i < TMX; ++i)
-                            a[e][ks][i] = *reinterpret_cast<const half8_t*>(xs + e * kXTile + i * 32 * kXRow + a_off[ks]);
-                }
-                // Requests RING - 1 iterations / super-tiles ahead, activations first (the counted wait below
-                // then never has to cover a weight super-tile younger than one iteration).
-#ifndef TSHIP_FR_NOX
-                issue_x(T, p + RING - 1);
-#endif
-#ifndef TSHIP_FR_NOW
-                if (HPS == 1 || (p & 1) == 0) issue_w(T, s + RING - 1);
-#endif
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    uint32_t o[16];
-#ifdef TSHIP_FR_NODEQ
-                    _Pragma("unroll") for (int q = 0; q < 16; ++q) o[q] = r[e][q % G::kRegs];
-#else
-                    G::dequant(r[e], e0 + e, h, G::sup_delta(T.my_delta, s), ((2 * p + e) * 2 + h) * 32 < A.K, o);
-#endif
-#pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) {
-                        const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
-                        const half8_t b = __builtin_bit_cast(half8_t, bb);
-#pragma unroll
-                        for (int i = 0; i < TMX; ++i)
-#ifdef TSHIP_FR_NOMMA
-                            acc[i][0] += (float)a[e][ks][i][0] * (float)b[0];
-#else
-                            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[e][ks][i], b, acc[i], 0, 0, 0);
-#endif
-                    }
-                }
-                // RING 3: this iteration's activation copies and the youngest weight super-tile may stay in flight
-                if constexpr (RING == 2) wait_copies_and_barrier<0>();
-                else if (five) wait_copies_and_barrier<2 * XI + WI>();
-                else wait_copies_and_barrier<2 * XI + WI - 1>();
-            }
-        };
-        if (RING == 2 && T.m_rows <= 32) run(std::integral_constant<int, 1>{});
-        else run(std::integral_constant<int, TM>{});
-
-        // The next tile's first requests go out before this tile's results are stored, so their latency
-        // is covered by the epilogue (every wavefront is past its last LDS read of this tile).
-        const int m0 = T.m0, m_rows = T.m_rows, my_n = T.my_n;
-        const bool more = setup(T);
-        if (more) issue_first(T);
-        store_tile<TM>(A, acc, m0, m_rows, my_n, h);
-        if (!more) break;
-    }
-}
-
-template <typename G, int NW, int RING>
-bool launch_few_rows(GemmArgs a, int m_tiles, hipStream_t stream)
-{
-    constexpr int BN = NW * 32, RT = BN * G::kRawRow;
-    auto kern = gemm_few_rows_kernel<G, NW, RING>;
-    const size_t lds = (size_t)RING * 2 * 64 * kXRow + (size_t)RING * RT;
-    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
-    a.m_tiles = m_tiles;
-    a.n_tiles = (a.N + BN - 1) / BN;
-    const int total = a.m_tiles * a.n_tiles;
-    // persistent workgroups, as many per CU as the LDS footprint allows, whole rounds over the 8 XCDs
-    const int per_cu = std::max(1, (int)((160 * 1024) / (lds + 512)));
-    const int grid = std::min(((total + 7) / 8) * 8, std::max(8, device_info().num_cus * per_cu / 8 * 8));
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
-    return hip_ok(hipGetLastError(), "gemm launch");
-}
-
-// ------------------------------------------------------------------------------------------
 // At most 32 activation rows per tile (small batches, MoE experts with few tokens; also single rows of formats
-// without a GEMV kernel).  The activations stay in REGISTERS: the eight wavefronts of a workgroup split K between them
-// (KTW k-tiles each), every wavefront keeps the MFMA A operands of its K range for all 32 rows, and the
-// workgroup walks over 32-column weight tiles.  Per tile a wavefront needs only its own K range of the 32
-// raw weight rows, which it copies itself (global -> LDS, two private buffers, requested two tiles ahead),
-// so the main loop has no barrier and no activation traffic at all; the eight partial 32 x 32 sums meet in
-// LDS (in the raw buffer the wavefront has just consumed), are added in a fixed order and stored.
+// without a GEMV kernel).  The activations stay in REGISTERS: the eight wavefronts of a workgroup split K between
+// them (KTW k-tiles each), every wavefront keeps the MFMA A operands of its K range for all 32 rows, and the
+// workgroup walks over 32-column weight tiles.  Per tile a wavefront needs only its own K range of the 32 raw
+// weight rows, which it copies itself (global -> LDS, a private ring of buffers, requested RING tiles ahead), so
+// the main loop has no barrier and no activation traffic at all; the eight partial 32 x 32 sums meet in LDS (in
+// the raw buffer the wavefront has just consumed), are added in a fixed order and stored.  A K longer than
+// 8 * KTW k-tiles is cut into chunks whose sums a second kernel adds.
 // ------------------------------------------------------------------------------------------
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -1164,12 +908,13 @@ __global__ void __launch_bounds__(256) gemm_chunk_sum_kernel(const float* __rest
                                                              int accumulate)
 {
     const int n = blockIdx.x * 256 + threadIdx.x;
-    const int m = blockIdx.y;
     if (n >= N) return;
-    float* out = c + (int64_t)(c_rows ? c_rows[m] : m) * ldc + n;
-    float s = accumulate ? *out : 0.f;
-    for (int kc = 0; kc < k_chunks; ++kc) s += partial[((int64_t)kc * M + m) * N + n];
-    *out = s;
+    for (int m = blockIdx.y; m < M; m += gridDim.y) {
+        float* out = c + (int64_t)(c_rows ? c_rows[m] : m) * ldc + n;
+        float s = accumulate ? *out : 0.f;
+        for (int kc = 0; kc < k_chunks; ++kc) s += partial[((int64_t)kc * M + m) * N + n];
+        *out = s;
+    }
 }
 
 // grow-only device buffer for the K-chunk sums
@@ -1216,7 +961,7 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream)
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (two_pass) {
-        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, a.M), dim3(256), 0, stream, a.partial, a.k_chunks, a.M, a.N,
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial, a.k_chunks, a.M, a.N,
                            a.c_rows, a.c, a.ldc, a.accumulate);
         return hip_ok(hipGetLastError(), "gemm chunk sum launch");
     }
@@ -1258,26 +1003,17 @@ bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
-    if (bm == 32 && a.M <= 65535) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream);
+    if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream);
     if constexpr (G::kRawRow <= 144) {
         if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
     }
     // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
-    // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 the other way round
+    // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 and Q6_K the other way round
     if (bm == 128)
         return (G::kSup == 2 || G::kRawRow > 144) ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream)
                                                    : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream);
-#ifdef TSHIP_GEMM_NO_FEW_ROWS
-    return launch_tiles<G, 64, 4, 8>(a, m_tiles, stream);
-#else
-#ifdef TSHIP_GEMM_FEW_ROWS_ONE_WG
-    return launch_few_rows<G, 8, 3>(a, m_tiles, stream);
-#else
-    // wide raw rows (Q6_K): one 8-wavefront workgroup per CU instead of two 4-wavefront ones
-    if constexpr (G::kRawRow > 144) return launch_few_rows<G, 8, 2>(a, m_tiles, stream);
-    else return launch_few_rows<G, 4, 2>(a, m_tiles, stream);
-#endif
-#endif
+    set_last_error("gemm: unsupported tile height.");
+    return false;
 }
 
 }  // namespace
@@ -1288,7 +1024,17 @@ size_t gemm_workspace_bytes(int M, int K)
     return (size_t)M * kp * sizeof(_Float16) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255) + 256;
 }
 
-int gemm_tile_m(int M) { return M > 1024 ? 256 : M > 64 ? 128 : M > 32 ? 64 : 32; }
+// Rows of activations per tile for a plain (ungrouped) launch.  The 32-row register-resident kernel streams the
+// weights once per 32 rows, but at a much higher rate than the LDS-tiled kernels and mostly out of the memory-side
+// cache, so it wins well past 32 rows (measured crossovers: 4-bit formats about 128 rows, or up to 512 when the
+// big tiles would leave CUs idle; Q8_0 about 64; Q6_K, whose big tiles are limited to 128 rows, about 256).
+int gemm_tile_m(int type, int M, int N)
+{
+    const int slim_rows = type == kTypeQ8_0 ? 64 : type == kTypeQ6_K ? 256 : 128;
+    if (M <= slim_rows) return 32;
+    if ((type == kTypeQ4_K || type == kTypeMXFP4) && M <= 512 && ((M + 127) / 128) * ((N + 127) / 128) <= 128) return 32;
+    return M > 1024 ? 256 : 128;
+}
 
 namespace {
 
@@ -1379,7 +1125,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
         bm = tiles->bm;
         m_tiles = tiles->count;
     } else {
-        bm = gemm_tile_m(M);
+        bm = gemm_tile_m(type, M, N);
         if (type == kTypeQ6_K && bm == 256) bm = 128;     // two raw Q6_K super-tiles of 256 rows do not fit LDS
         m_tiles = (M + bm - 1) / bm;
     }

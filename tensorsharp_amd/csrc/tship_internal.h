@@ -116,7 +116,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
 // ---- prefill GEMM ---------------------------------------------------------------------------
 // Workspace layout: [M floats of row scales, padded to 256 B][M x Kp fp16 activations].
 size_t gemm_workspace_bytes(int M, int K);
-int gemm_tile_m(int M);   // rows of activations per tile for a plain (ungrouped) launch
+int gemm_tile_m(int type, int M, int N);   // rows of activations per tile for a plain (ungrouped) launch
 
 // fp32 activations -> workspace (fp16 in the weight format's unpack order + per-row scales);
 // row_map (device, optional) gathers source rows.

@@ -200,3 +200,23 @@ def test_q6_k_rows_two_bytes_off(hip, oracle, M):
     y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(dev[row_bytes:], Q6_K, K, N - 1))
     torch.cuda.synchronize()
     check(y.cpu().numpy(), oracle.matmul_f64(Q6_K, wq[row_bytes:], N - 1, K, x), ("q6_k view", M))
+
+
+@pytest.mark.parametrize("name,M,N,K", [("mxfp4", 600, 300, 768), ("q4_k", 520, 1000, 1024), ("q8_0", 70, 500, 1088),
+                                       ("mxfp4", 300, 17000, 512)])
+def test_128_row_tiles(hip, oracle, name, M, N, K):
+    # row counts past the register-resident kernel's range: 128-row tiles, ragged last tile
+    rng = np.random.default_rng(M + N + K)
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, T[name], wq, N, K, x)
+    check(y, oracle.matmul_f64(T[name], wq, N, K, x), (name, M, N, K))
+
+
+def test_q6_k_128_row_tiles(hip, oracle):
+    from oracle.oracle import Q6_K
+    rng = np.random.default_rng(77)
+    M, N, K = 300, 520, 1024
+    wq = q6k_weight(N, K, 11)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    check(run_device(hip, Q6_K, wq, N, K, x), oracle.matmul_f64(Q6_K, wq, N, K, x), "q6_k 300")
