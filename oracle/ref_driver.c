@@ -53,3 +53,50 @@ int ref_mul_mat(int type, const void* w, int64_t N, int64_t K, const float* x, i
     ggml_free(ctx);
     return st == GGML_STATUS_SUCCESS ? 0 : -3;
 }
+
+/* A small GGUF file written by the reference's own writer (gguf.cpp): fixed metadata of every value kind the
+ * managed reader handles, plus the given 2-D tensors (raw block bytes, ne0 = row length).  Pins the GGUF reader. */
+#include "gguf.h"
+
+int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** names, const int* types,
+                   const int64_t* ne0, const int64_t* ne1, const void** data)
+{
+    size_t total = 1u << 20;
+    for (int i = 0; i < n_tensors; ++i) total += ggml_row_size((enum ggml_type)types[i], ne0[i]) * (size_t)ne1[i] + 4096;
+    struct ggml_init_params ip = { total, NULL, false };
+    struct ggml_context* ctx = ggml_init(ip);
+    if (!ctx) return -1;
+    struct gguf_context* g = gguf_init_empty();
+    gguf_set_val_str(g, "general.architecture", "llama");
+    gguf_set_val_str(g, "general.name", "tiny \xe2\x9c\x93 model");          /* non-ASCII UTF-8 */
+    if (alignment != 32) gguf_set_val_u32(g, "general.alignment", (uint32_t)alignment);
+    gguf_set_val_u32(g, "llama.block_count", 2);
+    gguf_set_val_i32(g, "test.i32", -7);
+    gguf_set_val_u8(g, "test.u8", 200);
+    gguf_set_val_i8(g, "test.i8", -100);
+    gguf_set_val_u16(g, "test.u16", 65000);
+    gguf_set_val_i16(g, "test.i16", -30000);
+    gguf_set_val_u64(g, "test.u64", 1ull << 40);
+    gguf_set_val_i64(g, "test.i64", -(1ll << 41));
+    gguf_set_val_f32(g, "llama.attention.layer_norm_rms_epsilon", 1e-5f);
+    gguf_set_val_f64(g, "test.f64", 0.1);
+    gguf_set_val_bool(g, "test.flag", true);
+    const char* toks[4] = { "<s>", "</s>", "hello", "w\xc3\xb6rld" };
+    gguf_set_arr_str(g, "tokenizer.ggml.tokens", toks, 4);
+    const float scores[4] = { 0.0f, -1.5f, 2.25f, -1000.0f };
+    gguf_set_arr_data(g, "tokenizer.ggml.scores", GGUF_TYPE_FLOAT32, scores, 4);
+    const int32_t ttypes[4] = { 3, 3, 1, 1 };
+    gguf_set_arr_data(g, "tokenizer.ggml.token_type", GGUF_TYPE_INT32, ttypes, 4);
+    const uint32_t u32s[3] = { 1, 2, 4000000000u };
+    gguf_set_arr_data(g, "test.u32s", GGUF_TYPE_UINT32, u32s, 3);
+    for (int i = 0; i < n_tensors; ++i) {
+        struct ggml_tensor* t = ggml_new_tensor_2d(ctx, (enum ggml_type)types[i], ne0[i], ne1[i]);
+        ggml_set_name(t, names[i]);
+        memcpy(t->data, data[i], ggml_nbytes(t));
+        gguf_add_tensor(g, t);
+    }
+    const int ok = gguf_write_to_file(g, path, false) ? 0 : -2;
+    gguf_free(g);
+    ggml_free(ctx);
+    return ok;
+}
