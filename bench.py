@@ -20,7 +20,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-Q8_0, Q4_K, MXFP4 = 8, 12, 39
+Q8_0, Q4_K, Q6_K, MXFP4 = 8, 12, 14, 39
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the grouped Q4_K GEMV from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the
 # reading of a 1 GiB copy (profiles/gemv_q4k_layer_hbm_traffic.txt); not measured by this script.
@@ -33,7 +33,7 @@ LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
 
 
 def row_bytes(t, k):
-    return {Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), MXFP4: 17 * (k // 32)}[t]
+    return {Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), Q6_K: 210 * (k // 256), MXFP4: 17 * (k // 32)}[t]
 
 
 def algorithmic_bytes(t, n, k, m=1):
@@ -186,6 +186,13 @@ def main():
             extra[f"cfg2_q4_k_gemv_{name}_{n}x{k}"] = one_matrix(Q4_K, n, k, max(2, int(300e6 // (n * row_bytes(Q4_K, k))) + 1))
         extra["cfg4_mxfp4_gemv_gate_up_5760x2880"] = one_matrix(MXFP4, 5760, 2880, 32)
         extra["cfg4_mxfp4_gemv_down_2880x2880"] = one_matrix(MXFP4, 2880, 2880, 64)
+        # output projection of a 128k-vocabulary model (the largest single GEMV of a decode step): Q8_0 through the
+        # GEMV kernel, Q6_K (what Q4_K_M files store it in) through the register-resident matrix-core kernel
+        n_it_save, n_it = n_it, 50
+        extra["lm_head_q8_0_gemv_128256x4096"] = one_matrix(Q8_0, 128256, 4096, 2)
+        extra["lm_head_q6_k_128256x4096"] = one_matrix(Q6_K, 128256, 4096, 2)
+        extra["q6_k_ffn_down_4096x14336"] = one_matrix(Q6_K, 4096, 14336, 8)
+        n_it = n_it_save
 
         # prefill GEMMs (configs[2] and configs[4]): TFLOP/s = 2*M*N*K / time of the whole call
         # (activation convert kernel + MFMA GEMM), fp16 operands -> priced against 2516.6 TFLOP/s
@@ -208,6 +215,13 @@ def main():
         extra["cfg5_q8_0_gemm_2048x21504x5376"] = prefill(Q8_0, 2048, 21504, 5376, 10)
         extra["cfg5_q4_k_gemm_2048x5376x21504"] = prefill(Q4_K, 2048, 5376, 21504, 10)
         extra["cfg5_q8_0_gemm_2048x5376x21504"] = prefill(Q8_0, 2048, 5376, 21504, 10)
+        # small batches (speculative decoding / few concurrent sequences): weight streaming, GB/s is the figure of merit
+        for m in (8, 32, 128):
+            r = prefill(Q4_K, m, 14336, 4096)
+            b = algorithmic_bytes(Q4_K, 14336, 4096, m)
+            r.update({"bytes": b, "GBps": round(b / (r["us_per_call_events"] * 1e-6) / 1e9, 1)})
+            extra[f"q4_k_gemm_{m}x14336x4096"] = r
+        extra["q6_k_gemm_512x14336x4096"] = prefill(Q6_K, 512, 14336, 4096)
         # MoE expert stage (configs[3]): 32 MXFP4 experts, top-4, hidden 2880; T = 1 (decode, HBM-bound:
         # bytes of the 4 selected experts' gate_up + down blocks) and T = 256 (prefill, grouped GEMM)
         def moe(T, iters):

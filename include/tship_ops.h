@@ -9,7 +9,8 @@
  *     (thread-local, valid until the next call on that thread) — except
  *     TSHip_DequantizeToF32*, which keeps the bridge's 0 / -1 / -2 codes;
  *   - nothing throws across the boundary; the caller owns every buffer.
- * Supported weight types: Q8_0 (8), Q4_K (12), MXFP4 (39)
+ * Matmul weight types: Q8_0 (8), Q4_K (12), Q6_K (14), MXFP4 (39).  Dequantize / row gather additionally read F16 (1),
+ * Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q5_K (13), IQ4_NL (20), BF16 (30): the block formats of ManagedQuantizedOps.cs:40-59
  * (ids: TensorSharp.Runtime/GgufReader.cs:26-37).
  *
  * Two families:
@@ -33,7 +34,11 @@ extern "C" {
 /* Backend ids. 1..3 are the bridge's (TensorSharp.Backends.GGML/GgmlNative.cs:20-25); 4 is new. */
 enum { TSHIP_BACKEND_METAL = 1, TSHIP_BACKEND_CPU = 2, TSHIP_BACKEND_CUDA = 3, TSHIP_BACKEND_HIP = 4 };
 
-enum { TSHIP_TYPE_F32 = 0, TSHIP_TYPE_Q8_0 = 8, TSHIP_TYPE_Q4_K = 12, TSHIP_TYPE_MXFP4 = 39 };
+enum {
+    TSHIP_TYPE_F32 = 0, TSHIP_TYPE_F16 = 1, TSHIP_TYPE_Q4_0 = 2, TSHIP_TYPE_Q4_1 = 3, TSHIP_TYPE_Q5_0 = 6, TSHIP_TYPE_Q5_1 = 7,
+    TSHIP_TYPE_Q8_0 = 8, TSHIP_TYPE_Q4_K = 12, TSHIP_TYPE_Q5_K = 13, TSHIP_TYPE_Q6_K = 14, TSHIP_TYPE_IQ4_NL = 20,
+    TSHIP_TYPE_BF16 = 30, TSHIP_TYPE_MXFP4 = 39
+};
 
 /* TensorSharp.GGML.Native/ggml_ops_internal.h:69-77 == GgmlNative.cs:27-45 (GgmlTensorView2D). */
 typedef struct TSHipTensorView2D {

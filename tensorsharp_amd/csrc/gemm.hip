@@ -372,7 +372,7 @@ struct GQ6K {
     static constexpr int kRegs = 20;
     static constexpr int kSup = 4;            // one 256-element block
     static constexpr int kSupBytes = 210;
-    static constexpr int kRawRow = 224;
+    static constexpr int kRawRow = 240;       // 60 dwords: the dword reads of 32 rows spread over 16 banks (224 bytes: 8)
     static constexpr int kTileStep = 4;
     static constexpr uint32_t sup_offset(int s) { return ((uint32_t)s * 210u) & ~3u; }
     static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int s) { return delta + ((uint32_t)(s & 1) << 1); }
@@ -726,7 +726,14 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // block; the unpackers may read a few bytes further, into the next row, and ignore them)
 template <typename G, int KTW>
 struct SlimLayout {
-    static constexpr int CH = (G::window_bytes(KTW) + 15) / 16;
+    static constexpr int kNeed = (G::window_bytes(KTW) + 15) / 16;
+    static constexpr int buf_of(int ch) { return 32 * ch * 16 > 4096 ? 32 * ch * 16 : 4096; }
+    static constexpr int ring_of(int ch) { return 8 * 3 * buf_of(ch) + 1024 <= 160 * 1024 ? 3 : 2; }
+    // an odd chunk count spreads the dword reads of the 32 rows over twice as many LDS banks; taken when it costs no
+    // ring depth and still fits
+    static constexpr bool kOdd = (kNeed & 1) == 0 && ring_of(kNeed + 1) == ring_of(kNeed) &&
+                                 8 * ring_of(kNeed + 1) * buf_of(kNeed + 1) + 64 <= 160 * 1024;
+    static constexpr int CH = kNeed + (kOdd ? 1 : 0);
     static constexpr int DI = (32 * CH + 63) / 64;                       // LDS-direct copies per buffer
     static constexpr int RAW = 32 * CH * 16;
     static constexpr int BUF = RAW > 4096 ? RAW : 4096;                  // raw rows, later the 32 x 32 fp32 partial sums
