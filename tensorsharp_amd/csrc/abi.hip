@@ -228,7 +228,7 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
         return false;
     }
     if (!is_quant_type(type)) {
-        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, Q6_K, MXFP4).");
+        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, MXFP4).");
         return false;
     }
     const size_t rs = row_size(type, ne0);
@@ -247,7 +247,7 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
 bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
 {
     const uintptr_t wa = reinterpret_cast<uintptr_t>(w);
-    const uintptr_t need_align = type == kTypeQ4_K ? 16 : (type == kTypeQ8_0 || type == kTypeQ6_K) ? 2 : 1;
+    const uintptr_t need_align = (type == kTypeQ4_K || type == kTypeQ5_K) ? 16 : (type == kTypeMXFP4) ? 1 : 2;
     if (wa % need_align != 0) {
         set_last_error("Quantized weight pointer is not aligned for its block type.");
         return false;
@@ -453,7 +453,7 @@ bool validate_weight(const void* data, int type, int64_t ne0, int64_t ne1, int64
         return false;
     }
     if (!is_quant_type(type)) {
-        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q8_0, Q4_K, Q6_K, MXFP4).");
+        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, MXFP4).");
         return false;
     }
     const size_t rs = row_size(type, ne0);

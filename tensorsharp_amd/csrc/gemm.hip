@@ -82,13 +82,13 @@ __device__ __forceinline__ uint32_t splat(float a) { return pack2(a, a); }
 template <int TYPE>
 __device__ __forceinline__ int k_slot(int k)
 {
-    if (TYPE == kTypeQ4_K) {
+    if (TYPE == kTypeQ4_K) {      // also the order of Q5_K
         // sub-block k/32; quant byte c of the lane's 16-byte chunk; dword c/4 unpacks as (b0,b2),(b1,b3)
         const int sub = k >> 5, hh = (k >> 4) & 1, c = k & 15, b = c & 3;
         const int idx = sub * 8 + 2 * (c >> 2) + (b & 1);
         return (idx >> 2) * 16 + hh * 8 + 2 * (idx & 3) + (b >> 1);
     }
-    if (TYPE == kTypeMXFP4) {
+    if (TYPE == kTypeMXFP4) {     // also the order of Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL
         // block k/32; quant byte i = k%16 holds elements i (low nibble) and i + 16 (high nibble)
         const int hh = k >> 5, i = k & 15, hi = (k >> 4) & 1;
         return (i >> 2) * 16 + hh * 8 + 2 * (i & 3) + hi;
@@ -417,6 +417,132 @@ struct GQ6K {
             const uint32_t sc = i < 4 ? s0 : s1;                         // elements 0..15 / 16..31 of the group
             o[2 * i] = pk_mul(pk_add(p0, bias), sc);
             o[2 * i + 1] = pk_mul(pk_add(p1, bias), sc);
+        }
+    }
+};
+
+// Q5_K (ggml-common.h block_q5_K: d, dmin, scales[12], qh[32], ql[128] = 176 bytes): Q4_K with a fifth bit per weight,
+// bit 2j (low nibbles) / 2j + 1 (high nibbles) of qh[l] for the 64-weight group j (ManagedQuantizedOps.cs:481-518).
+struct GQ5K {
+    static constexpr int kRegs = 12;
+    static constexpr int kSup = 4;
+    static constexpr int kSupBytes = 176;
+    static constexpr int kRawRow = 176;
+    static constexpr int kTileStep = 4;
+    static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 176u; }
+    static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int /*s*/) { return delta; }
+    static constexpr int window_bytes(int ktw) { return ktw * 44; }
+    static constexpr uint32_t tile_offset(int kt0) { return (uint32_t)kt0 * 44u; }
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int t, int h, uint32_t /*delta*/, uint32_t (&r)[kRegs])
+    {
+        rp += (t >> 2) * 176;
+        const int j = t & 3;
+        const uint4_t hdr = *reinterpret_cast<const uint4_t*>(rp);
+        const uint4_t qh = *reinterpret_cast<const uint4_t*>(rp + 16 + h * 16);
+        const uint4_t q = *reinterpret_cast<const uint4_t*>(rp + 48 + j * 32 + h * 16);
+        r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
+        r[4] = q.x; r[5] = q.y; r[6] = q.z; r[7] = q.w;
+        r[8] = qh.x; r[9] = qh.y; r[10] = qh.z; r[11] = qh.w;
+    }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int /*h*/, uint32_t /*delta*/, bool /*live*/,
+                                                   uint32_t (&o)[16])
+    {
+        const int j = t & 3;
+        const int sh = (j & 1) * 16;
+        const uint32_t a = r[1] >> sh, b = r[2] >> sh, c = r[3] >> sh;
+        const uint32_t sc_lo = a & 0x3f3fu, m_lo = b & 0x3f3fu;
+        const uint32_t sc_hi = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+        const uint32_t m_hi = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+        const uint32_t sc = (j & 2) ? sc_hi : sc_lo, mn = (j & 2) ? m_hi : m_lo;
+        H2U dm;
+        dm.u = r[0];
+        const float d = (float)dm.h.x, dmin = (float)dm.h.y;
+        const uint32_t s1 = splat(d * (float)(sc & 0xffu)), o1 = splat(-(dmin * (float)(mn & 0xffu)));
+        const uint32_t s2 = splat(d * (float)(sc >> 8) * 0.0625f), o2 = splat(-(dmin * (float)(mn >> 8)));
+        const uint32_t magic = 0x64006400u, neg1024 = 0xe400e400u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t q = r[4 + i], q8 = q >> 8;
+            const uint32_t bl = r[8 + i] >> (2 * j), bh = r[8 + i] >> (2 * j + 1);    // fifth bits at bit 0 of every byte
+            // low group: nibble + 16 bit; high group (kept as 16 * nibble): + 256 bit; both exact above 1024
+            o[2 * i] = pk_fma(pk_add((q & 0x000f000fu) | ((bl & 0x00010001u) << 4) | magic, neg1024), s1, o1);
+            o[2 * i + 1] = pk_fma(pk_add((q8 & 0x000f000fu) | (((bl >> 8) & 0x00010001u) << 4) | magic, neg1024), s1, o1);
+            o[8 + 2 * i] = pk_fma(pk_add((q & 0x00f000f0u) | ((bh & 0x00010001u) << 8) | magic, neg1024), s2, o2);
+            o[8 + 2 * i + 1] = pk_fma(pk_add((q8 & 0x00f000f0u) | (((bh >> 8) & 0x00010001u) << 8) | magic, neg1024), s2, o2);
+        }
+    }
+};
+
+// The 32-weight block formats with 16 quant bytes (low nibble = element j, high nibble = element j + 16) behind a
+// header: Q4_0 (d), Q4_1 (d, m), Q5_0 (d, 32 fifth bits), Q5_1 (d, m, fifth bits), IQ4_NL (d, table lookup)
+// (ManagedQuantizedOps.cs:313-409, :559-577).  Values enter the matrix cores as fp16(d) * q (+ fp16(m)).
+template <int TYPE>
+struct GLegacy {
+    static constexpr int kHdr = TYPE == kTypeQ4_0 || TYPE == kTypeIQ4_NL ? 2 : TYPE == kTypeQ4_1 ? 4 : TYPE == kTypeQ5_0 ? 6 : 8;
+    static constexpr int kBlock = kHdr + 16;
+    static constexpr bool kMin = TYPE == kTypeQ4_1 || TYPE == kTypeQ5_1;
+    static constexpr bool kFive = TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1;
+    static constexpr int kWords = (kBlock + 3) / 4;        // aligned dwords of one block
+    static constexpr int kRegs = kWords + 1;
+    static constexpr int kSup = 2;                          // four blocks
+    static constexpr int kSupBytes = 4 * kBlock;
+    static constexpr int kRawRow = 112;
+    static constexpr int kTileStep = 2;
+    static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * (4u * kBlock); }
+    static __device__ __forceinline__ uint32_t sup_delta(uint32_t delta, int /*s*/) { return delta; }
+    static constexpr int window_bytes(int ktw) { return ktw * 2 * kBlock + 3; }
+    static constexpr uint32_t tile_offset(int kt0) { return (uint32_t)kt0 * (2u * kBlock); }
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int t, int h, uint32_t delta, uint32_t (&r)[kRegs])
+    {
+        const uint32_t off = delta + (uint32_t)(2 * t + h) * kBlock;
+        const uint32_t* p = reinterpret_cast<const uint32_t*>(rp + (off & ~3u));
+#pragma unroll
+        for (int i = 0; i < kRegs; ++i) r[i] = p[i];
+    }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int h, uint32_t delta, bool live, uint32_t (&o)[16])
+    {
+        const uint32_t sft = (delta + (uint32_t)(2 * t + h) * kBlock) & 3u;
+        uint32_t b[kWords];                                  // the block from its first byte
+#pragma unroll
+        for (int i = 0; i < kWords; ++i) b[i] = __builtin_amdgcn_alignbyte(r[i + 1], r[i], sft);
+        const uint32_t dbits = live ? b[0] & 0xffffu : 0u;
+        const uint32_t d2 = dbits | (dbits << 16);
+        uint32_t m2 = 0u;
+        if (kMin) {
+            const uint32_t mbits = live ? b[0] >> 16 : 0u;
+            m2 = mbits | (mbits << 16);
+        }
+        uint32_t qh = 0u;
+        if (kFive) qh = (kHdr & 3) ? __builtin_amdgcn_alignbyte(b[kHdr / 4], b[kHdr / 4 - 1], 2) : b[kHdr / 4 - 1];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            // quant bytes 4 w .. 4 w + 3 of the block
+            const uint32_t q = (kHdr & 3) ? __builtin_amdgcn_alignbyte(b[kHdr / 4 + w + 1], b[kHdr / 4 + w], 2) : b[kHdr / 4 + w];
+            uint32_t lo = q & 0x0f0f0f0fu, hi = (q >> 4) & 0x0f0f0f0fu;
+            if (kFive) {
+                // bits 4 w .. 4 w + 3 (elements j) and 16 + 4 w .. (elements j + 16) of qh, one per byte, at bit 4
+                lo |= ((((qh >> (4 * w)) & 0xfu) * 0x00204081u) & 0x01010101u) << 4;
+                hi |= ((((qh >> (16 + 4 * w)) & 0xfu) * 0x00204081u) & 0x01010101u) << 4;
+            }
+            uint32_t bias;
+            if (TYPE == kTypeIQ4_NL) {
+                // {-127,-104,-83,-65,-49,-35,-22,-10, 1,13,25,38,53,69,89,113} + 128 as bytes, looked up with v_perm
+                const uint32_t t0 = 0x3f2d1801u, t1 = 0x766a5d4fu, t2 = 0xa6998d81u, t3 = 0xf1d9c5b5u;
+                const uint32_t ml = ((lo >> 3) & 0x01010101u) * 0xffu, mh = ((hi >> 3) & 0x01010101u) * 0xffu;
+                const uint32_t sl = lo & 0x07070707u, shh = hi & 0x07070707u;
+                lo = (__builtin_amdgcn_perm(t3, t2, sl) & ml) | (__builtin_amdgcn_perm(t1, t0, sl) & ~ml);
+                hi = (__builtin_amdgcn_perm(t3, t2, shh) & mh) | (__builtin_amdgcn_perm(t1, t0, shh) & ~mh);
+                bias = 0xe480e480u;                          // -(1024 + 128)
+            } else {
+                bias = kMin ? 0xe400e400u : kFive ? 0xe410e410u : 0xe408e408u;   // -1024, -(1024 + 16), -(1024 + 8)
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) {
+                // (element 4 w + s2, element 4 w + s2 + 16) as fp16 1024 + value
+                const uint32_t sel = (uint32_t)s2 | 0x0c00u | ((uint32_t)(4 + s2) << 16) | 0x0c000000u;
+                const uint32_t pair = __builtin_amdgcn_perm(hi, lo, sel) | 0x64006400u;
+                o[4 * w + s2] = pk_fma(pk_add(pair, bias), d2, m2);
+            }
         }
     }
 };
@@ -1011,7 +1137,7 @@ template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
     if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream);
-    if constexpr (G::kRawRow <= 144) {
+    if constexpr (2 * 256 * kXRow + 2 * 256 * G::kRawRow + 1024 <= 160 * 1024) {
         if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
     }
     // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
@@ -1061,11 +1187,13 @@ bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspa
     const int kp = (K + kBK - 1) / kBK * kBK;
     float* scales = static_cast<float*>(workspace);
     _Float16* x16 = reinterpret_cast<_Float16*>(static_cast<char*>(workspace) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
+    // three activation orders: the K-quant nibble order, the split-nibble order of the 32-weight blocks, natural
     switch (type) {
-    case kTypeQ4_K: launch_convert_typed<kTypeQ4_K, SRC>(src, M, K, kp, x16, scales, stream); break;
-    case kTypeMXFP4: launch_convert_typed<kTypeMXFP4, SRC>(src, M, K, kp, x16, scales, stream); break;
-    case kTypeQ8_0: launch_convert_typed<kTypeQ8_0, SRC>(src, M, K, kp, x16, scales, stream); break;
-    case kTypeQ6_K: launch_convert_typed<kTypeQ6_K, SRC>(src, M, K, kp, x16, scales, stream); break;
+    case kTypeQ4_K: case kTypeQ5_K: launch_convert_typed<kTypeQ4_K, SRC>(src, M, K, kp, x16, scales, stream); break;
+    case kTypeMXFP4: case kTypeQ4_0: case kTypeQ4_1: case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL:
+        launch_convert_typed<kTypeMXFP4, SRC>(src, M, K, kp, x16, scales, stream);
+        break;
+    case kTypeQ8_0: case kTypeQ6_K: launch_convert_typed<kTypeQ8_0, SRC>(src, M, K, kp, x16, scales, stream); break;
     default: set_last_error("gemm: unsupported type."); return false;
     }
     return hip_ok(hipGetLastError(), "activation convert launch");
@@ -1133,7 +1261,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
         m_tiles = tiles->count;
     } else {
         bm = gemm_tile_m(type, M, N);
-        if (type == kTypeQ6_K && bm == 256) bm = 128;     // two raw Q6_K super-tiles of 256 rows do not fit LDS
+        if (type == kTypeQ6_K && bm == 256) bm = 128;     // two raw Q6_K super-tiles of 256 columns do not fit LDS
         m_tiles = (M + bm - 1) / bm;
     }
     if (m_tiles == 0) return true;
@@ -1142,6 +1270,12 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     case kTypeMXFP4: return launch_for_type<GMXFP4>(a, bm, m_tiles, stream);
     case kTypeQ8_0: return launch_for_type<GQ80>(a, bm, m_tiles, stream);
     case kTypeQ6_K: return launch_for_type<GQ6K>(a, bm, m_tiles, stream);
+    case kTypeQ5_K: return launch_for_type<GQ5K>(a, bm, m_tiles, stream);
+    case kTypeQ4_0: return launch_for_type<GLegacy<kTypeQ4_0>>(a, bm, m_tiles, stream);
+    case kTypeQ4_1: return launch_for_type<GLegacy<kTypeQ4_1>>(a, bm, m_tiles, stream);
+    case kTypeQ5_0: return launch_for_type<GLegacy<kTypeQ5_0>>(a, bm, m_tiles, stream);
+    case kTypeQ5_1: return launch_for_type<GLegacy<kTypeQ5_1>>(a, bm, m_tiles, stream);
+    case kTypeIQ4_NL: return launch_for_type<GLegacy<kTypeIQ4_NL>>(a, bm, m_tiles, stream);
     default: set_last_error("gemm: unsupported type."); return false;
     }
 }

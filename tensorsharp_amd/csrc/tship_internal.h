@@ -58,8 +58,17 @@ inline int64_t block_bytes(int type)
     }
 }
 
-// formats the matmul kernels read (Q6_K through the matrix-core kernels only: no GEMV specialisation)
-inline bool is_quant_type(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4 || type == kTypeQ6_K; }
+// formats the matmul kernels read: every block format of ManagedQuantizedOps.cs:40-59 except Q8_1; the ones without
+// a GEMV specialisation take the matrix-core kernels for single rows too
+inline bool is_quant_type(int type)
+{
+    switch (type) {
+    case kTypeQ8_0: case kTypeQ4_K: case kTypeMXFP4: case kTypeQ6_K: case kTypeQ5_K: case kTypeQ4_0: case kTypeQ4_1:
+    case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL:
+        return true;
+    default: return false;
+    }
+}
 inline bool has_gemv(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4; }
 // formats with a dequantizer (DequantizeToF32, embedding gather): every block format the managed code reads
 // (ManagedQuantizedOps.cs:40-59) except Q8_1

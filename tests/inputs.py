@@ -54,3 +54,25 @@ def rms_err(y, ref):
     rms = np.sqrt(np.mean(ref * ref, axis=1))
     rms[rms == 0] = 1.0
     return float(np.max(np.max(np.abs(y - ref), axis=1) / rms))
+
+
+def random_blocks(name, rows, k, rng):
+    """Valid raw blocks of a [rows x k] weight with random quants and small finite scales, for the formats whose
+    reference quantizer is not restated here (the layouts: ggml-common.h block_q4_0 ... block_q5_K)."""
+    def f16(lo, hi, n):
+        return rng.uniform(lo, hi, n).astype(np.float16).view(np.uint8).reshape(n, 2)
+    hdr = {"q4_0": 2, "iq4_nl": 2, "q4_1": 4, "q5_0": 6, "q5_1": 8}
+    if name in hdr:
+        nb = rows * (k // 32)
+        raw = rng.integers(0, 256, size=(nb, hdr[name] + 16), dtype=np.uint8)
+        raw[:, 0:2] = f16(2e-3, 8e-3, nb) if name != "iq4_nl" else f16(2e-4, 6e-4, nb)
+        if name in ("q4_1", "q5_1"):
+            raw[:, 2:4] = f16(-0.06, 0.0, nb)
+        return raw.reshape(-1)
+    if name == "q5_k":
+        nb = rows * (k // 256)
+        raw = rng.integers(0, 256, size=(nb, 176), dtype=np.uint8)
+        raw[:, 0:2] = f16(5e-5, 2e-4, nb)
+        raw[:, 2:4] = f16(5e-5, 2e-4, nb)
+        return raw.reshape(-1)
+    raise KeyError(name)

@@ -220,3 +220,35 @@ def test_q6_k_128_row_tiles(hip, oracle):
     wq = q6k_weight(N, K, 11)
     x = rng.standard_normal((M, K)).astype(np.float32)
     check(run_device(hip, Q6_K, wq, N, K, x), oracle.matmul_f64(Q6_K, wq, N, K, x), "q6_k 300")
+
+
+# ---- the remaining block formats of the managed code (ManagedQuantizedOps.cs:40-59): matrix-core kernels only ----
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "q5_k"])
+@pytest.mark.parametrize("M,N,K", [(1, 700, 1024), (5, 130, 256), (32, 2000, 2304), (40, 300, 4352), (300, 520, 768),
+                                   (1100, 260, 512)])
+def test_more_formats_matmul(hip, oracle, name, M, N, K):
+    from oracle.oracle import MORE_TYPES
+    t = MORE_TYPES[name]
+    rng = np.random.default_rng(M * 7 + N + K + t)
+    wq = inputs.random_blocks(name, N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, t, wq, N, K, x)
+    check(y, oracle.matmul_f64(t, wq, N, K, x), (name, M, N, K))
+
+
+@pytest.mark.parametrize("name,row_bytes", [("q4_0", 18 * 3), ("q5_0", 22 * 3), ("q5_1", 24 * 5)])
+def test_more_formats_rows_two_bytes_off(hip, oracle, name, row_bytes):
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    from oracle.oracle import MORE_TYPES
+    t = MORE_TYPES[name]
+    rng = np.random.default_rng(91)
+    K = 96 if name != "q5_1" else 160
+    N = 150
+    wq = inputs.random_blocks(name, N, K, rng)
+    assert wq.size == N * row_bytes
+    x = rng.standard_normal((12, K)).astype(np.float32)
+    dev = torch.from_numpy(wq).cuda()
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(dev[row_bytes:], t, K, N - 1))
+    torch.cuda.synchronize()
+    check(y.cpu().numpy(), oracle.matmul_f64(t, wq[row_bytes:], N - 1, K, x), (name, "view"))
