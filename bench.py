@@ -88,6 +88,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy (20 times): the known-size kernel against "
                          "which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
+    ap.add_argument("--matmul", metavar="TYPE,M,N,K",
+                    help="time only one matmul shape (GGUF type id, rows, out features, in features) through "
+                         "TSHip_AddmmQuantF32Device, --steps calls after --warmup; for profiling a single kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU kernel path only: this build has no multi-GPU code; run with --gpus 1.",
@@ -116,6 +119,23 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "calibrate_copy_bytes_written": src.numel() * 4,
                           "launches": 20}))
+        return
+
+    if args.matmul:
+        t, m, n, k = (int(v) for v in args.matmul.split(","))
+        w = QuantizedWeight(synth.random_weight(t, n, k, dev, seed=91), t, k, n)
+        x = torch.randn((m, k), device=dev, dtype=torch.float32)
+        y = torch.empty((m, n), device=dev, dtype=torch.float32)
+
+        def one(i):
+            HipBasicOps.AddmmQuantDevice(y, x, w.ptr, t, k, n, w.raw_bytes)
+        for i in range(args.warmup):
+            one(i)
+        ev, wall = time_region(one, args.steps, torch)
+        us = ev * 1e3 / args.steps
+        b = algorithmic_bytes(t, n, k, m)
+        print(json.dumps({"matmul": {"type": t, "M": m, "N": n, "K": k}, "us_per_call_events": round(us, 2), "bytes": b,
+                          "GBps": round(b / (us * 1e-6) / 1e9, 1), "TFLOPs": round(2.0 * m * n * k / (us * 1e-6) / 1e12, 2)}))
         return
 
     # ---- workload: `copies` layers of seven Q4_K matrices, device resident -------------------
