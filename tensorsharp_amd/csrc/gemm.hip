@@ -619,6 +619,10 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
     }
 }
 
+float* chunk_buffer(size_t bytes);
+__global__ void gemm_chunk_sum_kernel(const float* __restrict__ partial, int k_chunks, int M, int N, const int* __restrict__ c_rows,
+                                      float* __restrict__ c, int64_t ldc, int accumulate);
+
 // BM x 256 x 64 tiles, eight wavefronts, each owning all BM rows of 32 output columns.
 //   * Activation k-tiles (fp16) and raw weight super-tiles go from global memory straight into LDS
 //     (buffer_load ... lds, range-checked: rows past M or N arrive as zeros).  Activation rows are 128
@@ -661,7 +665,9 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
     // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs, so each XCD gets a contiguous
     // run of tiles; consecutive tiles share the activation rows (same m-tile), which then stay in that
     // XCD's L2 while its CUs walk over the weight columns.
-    const int total = A.m_tiles * A.n_tiles;
+    // With K cut into chunks (few tiles, long K: the chunks fill the idle CUs) chunk kc of every tile is one unit.
+    const int tiles = A.m_tiles * A.n_tiles;
+    const int total = tiles * A.k_chunks;
     int t = blockIdx.x;
     {
         const int per = (total + 7) >> 3;
@@ -669,6 +675,8 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         t = xcd * per + slot;
         if (slot >= per || t >= total) return;
     }
+    const int kc = t / tiles;
+    t -= kc * tiles;
     const int mt = t / A.n_tiles, nt = t - mt * A.n_tiles;
     int m0, m_rows;
     const uint8_t* wbase = A.w;
@@ -689,7 +697,8 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
     const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
-    const int nkt = A.Kp / kBK;
+    const int kt_begin = kc * A.chunk_kt;                               // a multiple of 4: whole super-tiles and stage pairs
+    const int nkt = min(A.Kp / kBK, kt_begin + A.chunk_kt);            // end of this unit's K range
 
     // per-lane source offsets of the LDS-direct copies (constant over the k loop)
     uint32_t x_off[XI], w_off[WI];
@@ -750,20 +759,20 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) a_off[ks] = col * kXRow + ((2 * ks + h) ^ sw) * 16;
 
+    int s = kt_begin / G::kSup, j = 0;              // super-tile and k-tile inside it of `kt`
+    int xst = kt_begin % XST, rb = s % RB;          // LDS stage of k-tile kt, raw buffer of super-tile s
 #pragma unroll
-    for (int s = 0; s < RL; ++s) issue_w(s);
+    for (int i = 0; i < RL; ++i) issue_w(s + i);
 #pragma unroll
-    for (int kt = 0; kt < D; ++kt) issue_x(kt);
+    for (int i = 0; i < D; ++i) issue_x(kt_begin + i);
     __syncthreads();
     uint32_t oc[16], on[16];
     {
         uint32_t r[G::kRegs];
-        G::fetch(rbuf + my_raw, 0, h, G::sup_delta(my_delta, 0), r);
-        G::dequant(r, 0, h, G::sup_delta(my_delta, 0), h * 32 < A.K, oc);
+        G::fetch(rbuf + rb * RT + my_raw, 0, h, G::sup_delta(my_delta, s), r);
+        G::dequant(r, 0, h, G::sup_delta(my_delta, s), (kt_begin * 2 + h) * 32 < A.K, oc);
     }
-    int s = 0, j = 0;                               // super-tile and k-tile inside it of `kt`
-    int xst = 0, rb = 0;                            // LDS stage of k-tile kt, raw buffer of super-tile s
-    for (int kt = 0; kt < nkt; ++kt) {
+    for (int kt = kt_begin; kt < nkt; ++kt) {
         if (j == 0) issue_w(s + RL);
         issue_x(kt + D);
         int jn = j + 1, sn = s, rbn = rb;
@@ -816,7 +825,35 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         xst = xst + 1 == XST ? 0 : xst + 1;
     }
 
-    store_tile<TM>(A, acc, m0, m_rows, my_n, h);
+    if (A.partial) {
+        // chunk sums: [kc][activation row][column], already scaled; a second kernel adds the chunks
+        GemmArgs P = A;
+        P.c = A.partial + (int64_t)kc * A.M * A.N;
+        P.ldc = A.N;
+        P.c_rows = nullptr;
+        P.accumulate = 0;
+        store_tile<TM>(P, acc, m0, m_rows, my_n, h);
+    } else {
+        store_tile<TM>(A, acc, m0, m_rows, my_n, h);
+    }
+}
+
+// Number of K chunks for a plain launch: with few tiles and a long K, chunks of K fill the CUs that a whole-K launch
+// leaves idle.  Model: rounds of workgroups x k-tiles per chunk, plus writing and re-reading the chunk sums.
+inline int pick_k_chunks(int tiles, int nkt, int slots, int64_t out_elems, double us_per_ktile)
+{
+    int best = 1;
+    double best_t = (double)((tiles + slots - 1) / slots) * nkt * us_per_ktile;
+    for (int sc = 2; sc <= 4; ++sc) {
+        const int chunk = ((nkt + sc - 1) / sc + 3) / 4 * 4;
+        if (chunk < 48) break;
+        const double t = (double)((tiles * sc + slots - 1) / slots) * chunk * us_per_ktile + 2.0 * sc * out_elems * 4 / 4.5e6;
+        if (t < 0.9 * best_t) {
+            best = sc;
+            best_t = t;
+        }
+    }
+    return best;
 }
 
 template <typename G, int BM, int XST, int NW>
@@ -829,10 +866,32 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
     a.n_tiles = (a.N + BN - 1) / BN;
-    const int total = a.m_tiles * a.n_tiles;
+    const int nkt = a.Kp / kBK;
+    a.k_chunks = 1;
+    a.chunk_kt = (nkt + 3) / 4 * 4;
+    a.partial = nullptr;
+    if (!a.tile_expert) {
+        const int per_cu = std::max(1, (int)((160 * 1024) / (lds + 512)));
+        // measured: about 1.7 us per k-tile of a 256 x 256 tile when all CUs are busy
+        a.k_chunks = pick_k_chunks(a.m_tiles * a.n_tiles, nkt, device_info().num_cus * per_cu, (int64_t)a.M * a.N,
+                                   1.7 * BM * BN / 65536.0 * per_cu);
+        if (a.k_chunks > 1) {
+            a.chunk_kt = ((nkt + a.k_chunks - 1) / a.k_chunks + 3) / 4 * 4;
+            a.k_chunks = (nkt + a.chunk_kt - 1) / a.chunk_kt;
+            a.partial = chunk_buffer((size_t)a.k_chunks * a.M * a.N * sizeof(float));
+            if (!a.partial) return false;
+        }
+    }
+    const int total = a.m_tiles * a.n_tiles * a.k_chunks;
     const int grid = ((total + 7) / 8) * 8;          // whole rounds over the 8 XCDs
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
-    return hip_ok(hipGetLastError(), "gemm launch");
+    if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
+    if (a.partial) {
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
+                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
+        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+    }
+    return true;
 }
 
 // ------------------------------------------------------------------------------------------
