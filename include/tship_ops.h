@@ -202,6 +202,38 @@ TSHIP_EXPORT int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHi
                                                   int ggml_type, int n_experts, int64_t H, int64_t F, float alpha,
                                                   float limit);
 
+/* replaces TSGgml_TransformerLayerDecode (TensorSharp.GGML.Native/ggml_ops_transformer.cpp:318-470, :572-600;
+ * GgmlNative.cs:518-531): one token through one transformer layer with every pointer in DEVICE memory.
+ *   x   = RMSNorm(hidden) * attn_norm;  [q | k | v] = W_qkv x            (q: num_heads heads, k / v: num_kv_heads)
+ *   q, k: per-head RMSNorm * q_norm / k_norm (skipped when the pointer is NULL), RoPE at `position`
+ *         (rope_mode 0: adjacent pairs, 2: NeoX halves; n_dims = head_dim)
+ *   k, v -> row `position` of the fp32 caches [num_kv_heads][max_seq_len][head_dim]
+ *   a   = softmax(q K^T / sqrt(head_dim)) V over rows 0..position, grouped-query heads sharing their KV head
+ *   hidden += W_o a;  hidden += W_down( silu(g) * u ), [g | u] = W_gate_up (RMSNorm(hidden) * ffn_norm)
+ * hidden [hidden_size] is updated in place.  Same argument list as the bridge export. */
+TSHIP_EXPORT int TSHip_TransformerLayerDecodeDevice(float* hidden, int hidden_size, const float* attn_norm, const void* qkv_data,
+                                                    int qkv_type, int64_t qkv_ne0, int64_t qkv_ne1, int64_t qkv_bytes,
+                                                    const float* q_norm, const float* k_norm, int head_dim, const void* o_data,
+                                                    int o_type, int64_t o_ne0, int64_t o_ne1, int64_t o_bytes, const float* ffn_norm,
+                                                    const void* gu_data, int gu_type, int64_t gu_ne0, int64_t gu_ne1, int64_t gu_bytes,
+                                                    const void* down_data, int down_type, int64_t down_ne0, int64_t down_ne1,
+                                                    int64_t down_bytes, float* k_cache, float* v_cache, int num_heads,
+                                                    int num_kv_heads, int max_seq_len, int position, float eps, float rope_base,
+                                                    float rope_freq_scale, int intermediate_size, int rope_mode);
+
+/* replaces TSGgml_TransformerModelDecode (ggml_ops_transformer.cpp:1040-1230; GgmlNative.cs:647-659): the same for
+ * num_layers layers in sequence; the arrays (host memory) hold one device pointer per layer, shapes and types are shared. */
+TSHIP_EXPORT int TSHip_TransformerModelDecodeDevice(float* hidden, int hidden_size, int num_layers, const float* const* attn_norm,
+                                                    const void* const* qkv, const float* const* q_norm, const float* const* k_norm,
+                                                    const void* const* o, const float* const* ffn_norm, const void* const* gu,
+                                                    const void* const* down, float* const* k_cache, float* const* v_cache,
+                                                    int qkv_type, int64_t qkv_ne0, int64_t qkv_ne1, int64_t qkv_bytes, int o_type,
+                                                    int64_t o_ne0, int64_t o_ne1, int64_t o_bytes, int gu_type, int64_t gu_ne0,
+                                                    int64_t gu_ne1, int64_t gu_bytes, int down_type, int64_t down_ne0,
+                                                    int64_t down_ne1, int64_t down_bytes, int head_dim, int num_heads,
+                                                    int num_kv_heads, int max_seq_len, int position, float eps, float rope_base,
+                                                    float rope_freq_scale, int intermediate_size, int rope_mode);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,24 @@ _f64p = C.POINTER(C.c_double)
 _i32p = C.POINTER(C.c_int32)
 
 
+# argument list shared by tso_layer_decode and the reference driver's ref_layer_decode
+LAYER_ARGS = [_f32p, C.c_int, _f32p, C.c_void_p, C.c_int, _f32p, _f32p, C.c_int, C.c_void_p, C.c_int, _f32p, C.c_void_p, C.c_int,
+              C.c_void_p, C.c_int, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int,
+              C.c_int]
+
+
+def _layer_call(fn, hidden, layer, k_cache, v_cache, heads, kv_heads, head_dim, position, eps, rope_base, rope_freq_scale,
+                rope_mode):
+    """layer: dict attn_norm, qkv=(type, bytes), q_norm, k_norm, o=(type, bytes), ffn_norm, gate_up=(type, bytes),
+    down=(type, bytes), intermediate.  hidden / caches are updated in place (fp32, C-contiguous)."""
+    f = lambda a: None if a is None else _ptr(a, _f32p)
+    rc = fn(_ptr(hidden, _f32p), hidden.size, f(layer["attn_norm"]), _vp(layer["qkv"][1]), layer["qkv"][0], f(layer["q_norm"]),
+            f(layer["k_norm"]), head_dim, _vp(layer["o"][1]), layer["o"][0], f(layer["ffn_norm"]), _vp(layer["gate_up"][1]),
+            layer["gate_up"][0], _vp(layer["down"][1]), layer["down"][0], _ptr(k_cache, _f32p), _ptr(v_cache, _f32p), heads,
+            kv_heads, k_cache.shape[1], position, eps, rope_base, rope_freq_scale, layer["intermediate"], rope_mode)
+    assert rc == 0, rc
+
+
 def build(fast=True):
     """Compile the oracle libraries (gcc only)."""
     targets = ["liboracle.so"] + (["liboracle_fast.so"] if fast else [])
@@ -96,6 +114,12 @@ class Oracle:
                                       C.c_int, C.c_int, C.c_int, _f32p, C.c_int, C.c_int, _i32p,
                                       _f32p, _f32p]
         L.tso_max_threads.restype = C.c_int
+        L.tso_rope.restype = None
+        L.tso_rope.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float]
+        L.tso_attention_decode.restype = None
+        L.tso_attention_decode.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _f32p]
+        L.tso_layer_decode.restype = C.c_int
+        L.tso_layer_decode.argtypes = LAYER_ARGS
 
     # -- helpers ---------------------------------------------------------
     def row_size(self, t, ne):
@@ -192,6 +216,23 @@ class Oracle:
         self.lib.tso_swiglu_oai(_ptr(gu, _f32p), rows, two_f // 2, alpha, limit, _ptr(out, _f32p))
         return out
 
+    def rope(self, x, pos, mode, base, freq_scale=1.0):
+        y = np.ascontiguousarray(x, dtype=np.float32).copy()
+        self.lib.tso_rope(_ptr(y, _f32p), y.shape[0], y.shape[1], pos, mode, base, freq_scale)
+        return y
+
+    def attention_decode(self, q, k_cache, v_cache, total):
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        out = np.empty_like(q)
+        self.lib.tso_attention_decode(_ptr(q, _f32p), _ptr(k_cache, _f32p), _ptr(v_cache, _f32p), q.shape[0], k_cache.shape[0],
+                                      q.shape[1], k_cache.shape[1], total, _ptr(out, _f32p))
+        return out
+
+    def layer_decode(self, hidden, layer, k_cache, v_cache, heads, kv_heads, head_dim, position, eps, rope_base,
+                     rope_freq_scale=1.0, rope_mode=2):
+        _layer_call(self.lib.tso_layer_decode, hidden, layer, k_cache, v_cache, heads, kv_heads, head_dim, position, eps,
+                    rope_base, rope_freq_scale, rope_mode)
+
     def moe_forward(self, t, gu_w, gu_b, dn_w, dn_b, E, H, F, hidden, ids, wts):
         hidden = np.ascontiguousarray(hidden, dtype=np.float32)
         ids = np.ascontiguousarray(ids, dtype=np.int32)
@@ -233,6 +274,12 @@ class Reference:
                                   C.c_int]
         L.quantize_row_q8_K_ref.restype = None
         L.quantize_row_q8_K_ref.argtypes = [_f32p, C.c_void_p, C.c_int64]
+        L.ref_rope.restype = C.c_int
+        L.ref_rope.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
+        L.ref_flash_attn.restype = C.c_int
+        L.ref_flash_attn.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _f32p]
+        L.ref_layer_decode.restype = C.c_int
+        L.ref_layer_decode.argtypes = LAYER_ARGS
 
     def quantize(self, t, x, n_per_row=None):
         x = np.ascontiguousarray(x, dtype=np.float32)
@@ -259,6 +306,24 @@ class Reference:
         out = np.empty(n, dtype=np.float32)
         assert self.lib.ref_dequantize(t, _vp(raw), n, _ptr(out, _f32p)) == 0
         return out
+
+    def rope(self, x, pos, mode, base, freq_scale=1.0):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty_like(x)
+        assert self.lib.ref_rope(_ptr(x, _f32p), x.shape[0], x.shape[1], pos, mode, base, freq_scale, _ptr(out, _f32p)) == 0
+        return out
+
+    def flash_attn(self, q, k_cache, v_cache, total):
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        out = np.empty_like(q)
+        assert self.lib.ref_flash_attn(_ptr(q, _f32p), _ptr(k_cache, _f32p), _ptr(v_cache, _f32p), q.shape[0], k_cache.shape[0],
+                                       q.shape[1], k_cache.shape[1], total, _ptr(out, _f32p)) == 0
+        return out
+
+    def layer_decode(self, hidden, layer, k_cache, v_cache, heads, kv_heads, head_dim, position, eps, rope_base,
+                     rope_freq_scale=1.0, rope_mode=2):
+        _layer_call(self.lib.ref_layer_decode, hidden, layer, k_cache, v_cache, heads, kv_heads, head_dim, position, eps,
+                    rope_base, rope_freq_scale, rope_mode)
 
     def mul_mat(self, t, w, N, K, x, threads=4):
         x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)

@@ -10,6 +10,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#include <math.h>
 
 /* fp32 -> raw blocks with the reference quantizer (ggml_quantize_chunk, no imatrix). */
 size_t ref_quantize(int type, const float* src, void* dst, int64_t nrows, int64_t n_per_row)
@@ -99,4 +100,142 @@ int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** 
     gguf_free(g);
     ggml_free(ctx);
     return ok;
+}
+
+/* ---- known answers for the whole-layer decode, computed by the reference's ggml CPU ops ---------------- */
+
+static int run_graph(struct ggml_context* ctx, struct ggml_tensor* out)
+{
+    struct ggml_cgraph* g = ggml_new_graph(ctx);
+    ggml_build_forward_expand(g, out);
+    return ggml_graph_compute_with_ctx(ctx, g, 1) == GGML_STATUS_SUCCESS ? 0 : -3;
+}
+
+/* ggml_rope_ext as the bridge calls it (ggml_ops_transformer.cpp:403-406): n_dims = head_dim, n_ctx_orig 0,
+ * ext_factor 0, attn_factor 1, beta 0 / 0. */
+int ref_rope(const float* x, int n_heads, int head_dim, int pos, int mode, float base, float freq_scale, float* out)
+{
+    struct ggml_init_params ip = { 16u << 20, NULL, false };
+    struct ggml_context* ctx = ggml_init(ip);
+    if (!ctx) return -1;
+    struct ggml_tensor* t = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, head_dim, n_heads, 1);
+    memcpy(t->data, x, (size_t)n_heads * head_dim * sizeof(float));
+    struct ggml_tensor* p = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, 1);
+    ((int32_t*)p->data)[0] = pos;
+    struct ggml_tensor* r = ggml_rope_ext(ctx, t, p, NULL, head_dim, mode, 0, base, freq_scale, 0, 1, 0, 0);
+    int rc = run_graph(ctx, r);
+    if (rc == 0) memcpy(out, r->data, (size_t)n_heads * head_dim * sizeof(float));
+    ggml_free(ctx);
+    return rc;
+}
+
+/* ggml_flash_attn_ext as the bridge calls it (ggml_ops_transformer.cpp:436-441) on fp32 caches
+ * [kv_heads][max_seq][head_dim], one query row per head, rows [0, total), no mask. */
+int ref_flash_attn(const float* q, const float* kc, const float* vc, int heads, int kv_heads, int head_dim, int max_seq,
+                   int total, float* out)
+{
+    const size_t cache = (size_t)kv_heads * max_seq * head_dim * sizeof(float);
+    struct ggml_init_params ip = { 2 * cache + (64u << 20), NULL, false };
+    struct ggml_context* ctx = ggml_init(ip);
+    if (!ctx) return -1;
+    struct ggml_tensor* tq = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, head_dim, 1, heads);
+    memcpy(tq->data, q, (size_t)heads * head_dim * sizeof(float));
+    struct ggml_tensor* tk = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, head_dim, max_seq, kv_heads);
+    struct ggml_tensor* tv = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, head_dim, max_seq, kv_heads);
+    memcpy(tk->data, kc, cache);
+    memcpy(tv->data, vc, cache);
+    struct ggml_tensor* kw = ggml_view_3d(ctx, tk, head_dim, total, kv_heads, tk->nb[1], tk->nb[2], 0);
+    struct ggml_tensor* vw = ggml_view_3d(ctx, tv, head_dim, total, kv_heads, tv->nb[1], tv->nb[2], 0);
+    struct ggml_tensor* a = ggml_flash_attn_ext(ctx, tq, kw, vw, NULL, 1.0f / sqrtf((float)head_dim), 0.0f, 0.0f);
+    int rc = run_graph(ctx, a);
+    if (rc == 0) memcpy(out, a->data, (size_t)heads * head_dim * sizeof(float));   /* [head_dim, heads, 1] */
+    ggml_free(ctx);
+    return rc;
+}
+
+/* The layer graph of transformer_layer_decode_impl (ggml_ops_transformer.cpp:379-470), op for op through ggml's public
+ * API, computed by the reference's CPU backend (its mul_mat quantizes the activations to int8 blocks, so this is a
+ * coarse known answer: it pins the wiring of the graph, not the last digits).  hidden is updated in place; the caches
+ * [kv_heads][max_seq][head_dim] receive row `position`. */
+int ref_layer_decode(float* hidden, int hidden_size, const float* attn_norm, const void* qkv_w, int qkv_type,
+                     const float* q_norm, const float* k_norm, int head_dim, const void* o_w, int o_type,
+                     const float* ffn_norm, const void* gu_w, int gu_type, const void* down_w, int down_type,
+                     float* k_cache, float* v_cache, int heads, int kv_heads, int max_seq, int position, float eps,
+                     float rope_base, float rope_freq_scale, int inter, int rope_mode)
+{
+    const int q_dim = heads * head_dim, k_dim = kv_heads * head_dim, total = position + 1;
+    const size_t cache = (size_t)kv_heads * max_seq * head_dim * sizeof(float);
+    const size_t wb = ggml_row_size((enum ggml_type)qkv_type, hidden_size) * (size_t)(q_dim + 2 * k_dim) +
+                      ggml_row_size((enum ggml_type)o_type, q_dim) * (size_t)hidden_size +
+                      ggml_row_size((enum ggml_type)gu_type, hidden_size) * (size_t)(2 * inter) +
+                      ggml_row_size((enum ggml_type)down_type, inter) * (size_t)hidden_size;
+    struct ggml_init_params ip = { wb + 2 * cache + (128u << 20), NULL, false };
+    struct ggml_context* ctx = ggml_init(ip);
+    if (!ctx) return -1;
+#define NEW1(n) ggml_new_tensor_1d(ctx, GGML_TYPE_F32, n)
+    struct ggml_tensor* input = NEW1(hidden_size);
+    struct ggml_tensor* an = NEW1(hidden_size);
+    struct ggml_tensor* qn = NEW1(head_dim);
+    struct ggml_tensor* kn = NEW1(head_dim);
+    struct ggml_tensor* fn = NEW1(hidden_size);
+    memcpy(input->data, hidden, (size_t)hidden_size * 4);
+    memcpy(an->data, attn_norm, (size_t)hidden_size * 4);
+    memcpy(qn->data, q_norm, (size_t)head_dim * 4);
+    memcpy(kn->data, k_norm, (size_t)head_dim * 4);
+    memcpy(fn->data, ffn_norm, (size_t)hidden_size * 4);
+    struct ggml_tensor* wqkv = ggml_new_tensor_2d(ctx, (enum ggml_type)qkv_type, hidden_size, q_dim + 2 * k_dim);
+    struct ggml_tensor* wo = ggml_new_tensor_2d(ctx, (enum ggml_type)o_type, q_dim, hidden_size);
+    struct ggml_tensor* wgu = ggml_new_tensor_2d(ctx, (enum ggml_type)gu_type, hidden_size, 2 * inter);
+    struct ggml_tensor* wdn = ggml_new_tensor_2d(ctx, (enum ggml_type)down_type, inter, hidden_size);
+    memcpy(wqkv->data, qkv_w, ggml_nbytes(wqkv));
+    memcpy(wo->data, o_w, ggml_nbytes(wo));
+    memcpy(wgu->data, gu_w, ggml_nbytes(wgu));
+    memcpy(wdn->data, down_w, ggml_nbytes(wdn));
+    struct ggml_tensor* pos = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, 1);
+    ((int32_t*)pos->data)[0] = position;
+    struct ggml_tensor* kcb = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, head_dim, max_seq, kv_heads);
+    struct ggml_tensor* vcb = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, head_dim, max_seq, kv_heads);
+    memcpy(kcb->data, k_cache, cache);
+    memcpy(vcb->data, v_cache, cache);
+
+    struct ggml_tensor* normed = ggml_mul(ctx, ggml_rms_norm(ctx, input, eps), an);
+    struct ggml_tensor* qkv = ggml_reshape_1d(ctx, ggml_mul_mat(ctx, wqkv, ggml_reshape_2d(ctx, normed, hidden_size, 1)), q_dim + 2 * k_dim);
+    struct ggml_tensor* q_raw = ggml_view_1d(ctx, qkv, q_dim, 0);
+    struct ggml_tensor* k_raw = ggml_view_1d(ctx, qkv, k_dim, (size_t)q_dim * 4);
+    struct ggml_tensor* v_raw = ggml_view_1d(ctx, qkv, k_dim, (size_t)(q_dim + k_dim) * 4);
+    struct ggml_tensor* q_n = ggml_mul(ctx, ggml_rms_norm(ctx, ggml_reshape_2d(ctx, q_raw, head_dim, heads), eps), qn);
+    struct ggml_tensor* k_n = ggml_mul(ctx, ggml_rms_norm(ctx, ggml_reshape_2d(ctx, k_raw, head_dim, kv_heads), eps), kn);
+    struct ggml_tensor* q_r = ggml_rope_ext(ctx, ggml_reshape_3d(ctx, q_n, head_dim, heads, 1), pos, NULL, head_dim, rope_mode, 0, rope_base, rope_freq_scale, 0, 1, 0, 0);
+    struct ggml_tensor* k_r = ggml_rope_ext(ctx, ggml_reshape_3d(ctx, k_n, head_dim, kv_heads, 1), pos, NULL, head_dim, rope_mode, 0, rope_base, rope_freq_scale, 0, 1, 0, 0);
+    struct ggml_tensor* q_attn = ggml_permute(ctx, q_r, 0, 2, 1, 3);
+    struct ggml_tensor* k_write = ggml_cont(ctx, ggml_permute(ctx, k_r, 0, 2, 1, 3));
+    struct ggml_tensor* v_write = ggml_cont(ctx, ggml_permute(ctx, ggml_reshape_3d(ctx, v_raw, head_dim, kv_heads, 1), 0, 2, 1, 3));
+    const size_t off = (size_t)position * head_dim * 4;
+    struct ggml_tensor* k_cpy = ggml_cpy(ctx, k_write, ggml_view_3d(ctx, kcb, head_dim, 1, kv_heads, kcb->nb[1], kcb->nb[2], off));
+    struct ggml_tensor* v_cpy = ggml_cpy(ctx, v_write, ggml_view_3d(ctx, vcb, head_dim, 1, kv_heads, vcb->nb[1], vcb->nb[2], off));
+    struct ggml_tensor* k_full = ggml_view_3d(ctx, kcb, head_dim, total, kv_heads, kcb->nb[1], kcb->nb[2], 0);
+    struct ggml_tensor* v_full = ggml_view_3d(ctx, vcb, head_dim, total, kv_heads, vcb->nb[1], vcb->nb[2], 0);
+    struct ggml_tensor* attn = ggml_flash_attn_ext(ctx, q_attn, k_full, v_full, NULL, 1.0f / sqrtf((float)head_dim), 0.0f, 0.0f);
+    struct ggml_tensor* o_flat = ggml_reshape_1d(ctx, ggml_mul_mat(ctx, wo, ggml_reshape_2d(ctx, attn, q_dim, 1)), hidden_size);
+    struct ggml_tensor* res1 = ggml_add(ctx, input, o_flat);
+    struct ggml_tensor* normed2 = ggml_mul(ctx, ggml_rms_norm(ctx, res1, eps), fn);
+    struct ggml_tensor* gu = ggml_reshape_1d(ctx, ggml_mul_mat(ctx, wgu, ggml_reshape_2d(ctx, normed2, hidden_size, 1)), 2 * inter);
+    struct ggml_tensor* gate = ggml_view_1d(ctx, gu, inter, 0);
+    struct ggml_tensor* up = ggml_view_1d(ctx, gu, inter, (size_t)inter * 4);
+    struct ggml_tensor* ffn = ggml_mul(ctx, ggml_silu(ctx, gate), up);
+    struct ggml_tensor* down = ggml_reshape_1d(ctx, ggml_mul_mat(ctx, wdn, ggml_reshape_2d(ctx, ffn, inter, 1)), hidden_size);
+    struct ggml_tensor* result = ggml_add(ctx, res1, down);
+    struct ggml_cgraph* g = ggml_new_graph(ctx);
+    ggml_build_forward_expand(g, k_cpy);          /* cache writes first, as the bridge orders them */
+    ggml_build_forward_expand(g, v_cpy);
+    ggml_build_forward_expand(g, result);
+    const int rc = ggml_graph_compute_with_ctx(ctx, g, 1) == GGML_STATUS_SUCCESS ? 0 : -3;
+    if (rc == 0) {
+        memcpy(hidden, result->data, (size_t)hidden_size * 4);
+        memcpy(k_cache, kcb->data, cache);
+        memcpy(v_cache, vcb->data, cache);
+    }
+    ggml_free(ctx);
+    return rc;
+#undef NEW1
 }

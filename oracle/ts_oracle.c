@@ -990,3 +990,113 @@ int tso_moe_forward(int type, const void* gate_up_w, const float* gate_up_b, con
     free(offs); free(tmap); free(wmap); free(emap);
     return 0;
 }
+
+/* ---- whole-layer decode of the bridge (ggml graph of ggml_ops_transformer.cpp:379-470) ---------------- */
+
+/* ggml_rope_ext with n_dims = head_dim, ext_factor 0, attn_factor 1, no frequency factors, in place on
+ * x[n_heads][head_dim].  theta_scale = powf(base, -2/n_dims); theta starts at pos and is multiplied by theta_scale
+ * once per pair (fp32); the angle is freq_scale * theta.  mode 0 rotates (x[2i], x[2i+1]), mode 2 (NeoX)
+ * (x[i], x[i + n_dims/2]).
+ * Reference: ggml-cpu/ops.cpp:5532-5563 (rope_yarn, ggml_rope_cache_init), :5636-5652 (rotate_pairs), :5711, :5742-5775. */
+void tso_rope(float* x, int n_heads, int head_dim, int pos, int mode, float base, float freq_scale)
+{
+    const float theta_scale = powf(base, -2.0f / (float)head_dim);
+    const int half = head_dim / 2;
+    for (int h = 0; h < n_heads; ++h) {
+        float* v = x + (size_t)h * head_dim;
+        float theta = (float)pos;
+        for (int p = 0; p < half; ++p) {
+            const float ang = freq_scale * theta;
+            const float c = cosf(ang), s = sinf(ang);
+            const int i0 = mode == 2 ? p : 2 * p, i1 = mode == 2 ? p + half : 2 * p + 1;
+            const float x0 = v[i0], x1 = v[i1];
+            v[i0] = x0 * c - x1 * s;
+            v[i1] = x0 * s + x1 * c;
+            theta *= theta_scale;
+        }
+    }
+}
+
+/* One query row per head against cache rows [0, total): softmax(q . k * scale) v with scale = 1/sqrt(head_dim),
+ * query head h reads KV head h / (heads / kv_heads); caches are [kv_heads][max_seq][head_dim] fp32.  fp64 inside.
+ * Reference: the ggml_flash_attn_ext call of ggml_ops_transformer.cpp:436-441 (q [head_dim,1,heads], k/v windows of the
+ * caches, scale, no bias, no soft cap) — for one query row that is exactly this softmax-weighted sum. */
+void tso_attention_decode(const float* q, const float* kc, const float* vc, int heads, int kv_heads, int head_dim,
+                          int max_seq, int total, float* out)
+{
+    const double scale = 1.0 / sqrt((double)head_dim);
+    double* s = (double*)malloc((size_t)total * sizeof(double));
+    for (int h = 0; h < heads; ++h) {
+        const int kvh = h / (heads / kv_heads);
+        const float* qh = q + (size_t)h * head_dim;
+        double mx = -INFINITY;
+        for (int t = 0; t < total; ++t) {
+            const float* kr = kc + ((size_t)kvh * max_seq + t) * head_dim;
+            double d = 0.0;
+            for (int i = 0; i < head_dim; ++i) d += (double)qh[i] * (double)kr[i];
+            s[t] = d * scale;
+            if (s[t] > mx) mx = s[t];
+        }
+        double sum = 0.0;
+        for (int t = 0; t < total; ++t) { s[t] = exp(s[t] - mx); sum += s[t]; }
+        for (int i = 0; i < head_dim; ++i) {
+            double acc = 0.0;
+            for (int t = 0; t < total; ++t) acc += s[t] * (double)vc[((size_t)kvh * max_seq + t) * head_dim + i];
+            out[(size_t)h * head_dim + i] = (float)(acc / sum);
+        }
+    }
+    free(s);
+}
+
+static void linear_f32(int type, const void* w, int64_t N, int64_t K, const float* x, float* out)
+{
+    double* tmp = (double*)malloc((size_t)N * sizeof(double));
+    tso_matmul_f64(type, w, N, K, x, 1, K, tmp);
+    for (int64_t n = 0; n < N; ++n) out[n] = (float)tmp[n];
+    free(tmp);
+}
+
+/* One token through one layer, hidden [hidden_size] in place, K / V rows written at `position`.  Matmuls are the exact
+ * (fp64-accumulated) products with the dequantized weights; q_norm / k_norm may be NULL.
+ * Reference: ggml_ops_transformer.cpp:379-470 (steps 1-14 of transformer_layer_decode_impl). */
+int tso_layer_decode(float* hidden, int hidden_size, const float* attn_norm, const void* qkv_w, int qkv_type,
+                     const float* q_norm, const float* k_norm, int head_dim, const void* o_w, int o_type,
+                     const float* ffn_norm, const void* gu_w, int gu_type, const void* down_w, int down_type,
+                     float* k_cache, float* v_cache, int heads, int kv_heads, int max_seq, int position, float eps,
+                     float rope_base, float rope_freq_scale, int intermediate, int rope_mode)
+{
+    const int q_dim = heads * head_dim, k_dim = kv_heads * head_dim, qkv_n = q_dim + 2 * k_dim;
+    if (!hidden || !attn_norm || !qkv_w || !o_w || !ffn_norm || !gu_w || !down_w || !k_cache || !v_cache) return -1;
+    if (position < 0 || position >= max_seq || heads % kv_heads) return -1;
+    float* normed = (float*)malloc((size_t)hidden_size * sizeof(float));
+    float* qkv = (float*)malloc((size_t)qkv_n * sizeof(float));
+    float* attn = (float*)malloc((size_t)q_dim * sizeof(float));
+    float* o = (float*)malloc((size_t)hidden_size * sizeof(float));
+    float* gu = (float*)malloc((size_t)2 * intermediate * sizeof(float));
+    float* act = (float*)malloc((size_t)intermediate * sizeof(float));
+    tso_rms_norm_mul(hidden, 1, hidden_size, hidden_size, attn_norm, eps, normed);
+    linear_f32(qkv_type, qkv_w, qkv_n, hidden_size, normed, qkv);
+    float* q = qkv;
+    float* k = qkv + q_dim;
+    float* v = qkv + q_dim + k_dim;
+    if (q_norm)
+        for (int h = 0; h < heads; ++h) tso_rms_norm_mul(q + (size_t)h * head_dim, 1, head_dim, head_dim, q_norm, eps, q + (size_t)h * head_dim);
+    if (k_norm)
+        for (int h = 0; h < kv_heads; ++h) tso_rms_norm_mul(k + (size_t)h * head_dim, 1, head_dim, head_dim, k_norm, eps, k + (size_t)h * head_dim);
+    tso_rope(q, heads, head_dim, position, rope_mode, rope_base, rope_freq_scale);
+    tso_rope(k, kv_heads, head_dim, position, rope_mode, rope_base, rope_freq_scale);
+    for (int h = 0; h < kv_heads; ++h) {
+        memcpy(k_cache + ((size_t)h * max_seq + position) * head_dim, k + (size_t)h * head_dim, (size_t)head_dim * sizeof(float));
+        memcpy(v_cache + ((size_t)h * max_seq + position) * head_dim, v + (size_t)h * head_dim, (size_t)head_dim * sizeof(float));
+    }
+    tso_attention_decode(q, k_cache, v_cache, heads, kv_heads, head_dim, max_seq, position + 1, attn);
+    linear_f32(o_type, o_w, hidden_size, q_dim, attn, o);
+    for (int i = 0; i < hidden_size; ++i) hidden[i] = hidden[i] + o[i];
+    tso_rms_norm_mul(hidden, 1, hidden_size, hidden_size, ffn_norm, eps, normed);
+    linear_f32(gu_type, gu_w, 2 * (int64_t)intermediate, hidden_size, normed, gu);
+    tso_silu_mul(gu, 1, intermediate, act);
+    linear_f32(down_type, down_w, hidden_size, intermediate, act, o);
+    for (int i = 0; i < hidden_size; ++i) hidden[i] = hidden[i] + o[i];
+    free(normed); free(qkv); free(attn); free(o); free(gu); free(act);
+    return 0;
+}

@@ -70,6 +70,17 @@ int tso_moe_forward(int type, const void* gate_up_w, const float* gate_up_b,
                     int E, int H, int F, const float* hidden, int T, int k,
                     const int32_t* ids, const float* weights, float* out);
 
+/* whole-layer decode (ggml semantics): RoPE in place on x[n_heads][head_dim]; single-query attention over fp32 caches
+ * [kv_heads][max_seq][head_dim]; one token through one layer (hidden in place, caches written at `position`) */
+void tso_rope(float* x, int n_heads, int head_dim, int pos, int mode, float base, float freq_scale);
+void tso_attention_decode(const float* q, const float* kc, const float* vc, int heads, int kv_heads, int head_dim,
+                          int max_seq, int total, float* out);
+int tso_layer_decode(float* hidden, int hidden_size, const float* attn_norm, const void* qkv_w, int qkv_type,
+                     const float* q_norm, const float* k_norm, int head_dim, const void* o_w, int o_type,
+                     const float* ffn_norm, const void* gu_w, int gu_type, const void* down_w, int down_type,
+                     float* k_cache, float* v_cache, int heads, int kv_heads, int max_seq, int position, float eps,
+                     float rope_base, float rope_freq_scale, int intermediate, int rope_mode);
+
 /* fused wrappers: RMSNorm * weight, SiLU-gated product (ggml semantics) */
 void tso_rms_norm_mul(const float* x, int64_t rows, int64_t K, int64_t ldx, const float* w, float eps, float* out);
 void tso_silu_mul(const float* gate_up, int64_t rows, int64_t half_dim, float* out);

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libTsHipOps.so")
-SOURCES = ["abi.hip", "dequant.hip", "gemv.hip", "gemm.hip", "moe.hip", "fused.hip"]
+SOURCES = ["abi.hip", "dequant.hip", "gemv.hip", "gemm.hip", "moe.hip", "fused.hip", "layer.hip"]
 
 # packed-fp32 VALU forms stay off: the compiler must not form v_pk_{add,mul,fma}_f32.
 FLAGS = [

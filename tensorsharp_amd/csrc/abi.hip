@@ -1200,3 +1200,140 @@ int TSHip_FusedFFNSwiGLUQuantF32(TSHipTensorView2D residual, TSHipTensorView2D i
 }
 
 }  // extern "C"
+
+namespace {
+
+struct LayerShape {
+    int hidden, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate;
+    int qkv_type, o_type, gu_type, down_type;
+    int64_t qkv_bytes, o_bytes, gu_bytes, down_bytes;
+};
+
+bool validate_layer(const LayerShape& L, int64_t qkv_ne0, int64_t qkv_ne1, int64_t o_ne0, int64_t o_ne1, int64_t gu_ne0, int64_t gu_ne1,
+                    int64_t down_ne0, int64_t down_ne1, int position)
+{
+    const int64_t q_dim = (int64_t)L.num_heads * L.head_dim, k_dim = (int64_t)L.num_kv_heads * L.head_dim;
+    if (L.hidden <= 0 || L.head_dim <= 0 || L.num_heads <= 0 || L.num_kv_heads <= 0 || L.intermediate <= 0 || L.max_seq_len <= 0 ||
+        L.num_heads % L.num_kv_heads != 0) {
+        set_last_error("Invalid dimensions for transformer layer decode.");
+        return false;
+    }
+    if (position < 0 || position >= L.max_seq_len) {
+        set_last_error("transformer layer decode: position outside the KV cache.");
+        return false;
+    }
+    if (qkv_ne0 != L.hidden || qkv_ne1 != q_dim + 2 * k_dim || o_ne0 != q_dim || o_ne1 != L.hidden || gu_ne0 != L.hidden ||
+        gu_ne1 != 2 * (int64_t)L.intermediate || down_ne0 != L.intermediate || down_ne1 != L.hidden) {
+        set_last_error("Size mismatch: layer weight dims don't match in transformer layer decode.");
+        return false;
+    }
+    const struct { int type; int64_t ne0, ne1, bytes; } ws[4] = {{L.qkv_type, qkv_ne0, qkv_ne1, L.qkv_bytes}, {L.o_type, o_ne0, o_ne1, L.o_bytes},
+                                                                 {L.gu_type, gu_ne0, gu_ne1, L.gu_bytes}, {L.down_type, down_ne0, down_ne1, L.down_bytes}};
+    for (const auto& w : ws) {
+        const size_t rs = row_size(w.type, w.ne0);
+        if (!is_quant_type(w.type) || rs == 0 || (size_t)w.bytes < rs * (size_t)w.ne1) {
+            set_last_error("Unsupported quantized weight type, row length or byte span in transformer layer decode.");
+            return false;
+        }
+    }
+    return true;
+}
+
+// one token through one layer (ggml_ops_transformer.cpp:379-470); every pointer in device memory
+bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm, const void* qkv, const float* q_norm,
+                      const float* k_norm, const void* o, const float* ffn_norm, const void* gu, const void* down, float* k_cache,
+                      float* v_cache, int position, float eps, float rope_base, float rope_freq_scale, int rope_mode, hipStream_t stream)
+{
+    const int q_dim = L.num_heads * L.head_dim, k_dim = L.num_kv_heads * L.head_dim, qkv_n = q_dim + 2 * k_dim;
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t b_qkv = al((size_t)qkv_n * 4), b_q = al((size_t)q_dim * 4), b_attn = al((size_t)q_dim * 4);
+    const size_t b_part = al(attention_decode_ws_bytes(L.num_heads, position + 1));
+    const size_t b_mm = std::max(matmul_ws_bytes(L.qkv_type, 1, L.hidden, true), matmul_ws_bytes(L.o_type, 1, q_dim, false));
+    char* ws = static_cast<char*>(dev_ws_reserve(b_qkv + b_q + b_attn + b_part + b_mm + 256));
+    if (!ws) return false;
+    float* qkv_out = reinterpret_cast<float*>(ws);
+    float* q_rot = reinterpret_cast<float*>(ws + b_qkv);
+    float* attn = reinterpret_cast<float*>(ws + b_qkv + b_q);
+    float* part = reinterpret_cast<float*>(ws + b_qkv + b_q + b_attn);
+    void* mm_ws = ws + b_qkv + b_q + b_attn + b_part;
+    const TSHipTensorView2D h_view{hidden, 1, L.hidden, L.hidden, 1, (int64_t)L.hidden * 4};
+    const TSHipTensorView2D qkv_view{qkv_out, 1, qkv_n, qkv_n, 1, (int64_t)qkv_n * 4};
+    const TSHipTensorView2D attn_view{attn, 1, q_dim, q_dim, 1, (int64_t)q_dim * 4};
+    if (!run_matmul_device_ws(qkv_view, h_view, qkv, L.qkv_type, L.hidden, qkv_n, stream, mm_ws, attn_norm, eps, false)) return false;
+    if (!launch_qkv_post(qkv_out, L.num_heads, L.num_kv_heads, L.head_dim, q_norm, k_norm, eps, position, rope_base, rope_freq_scale,
+                         rope_mode, q_rot, k_cache, v_cache, L.max_seq_len, stream))
+        return false;
+    if (!launch_attention_decode(q_rot, k_cache, v_cache, L.num_heads, L.num_kv_heads, L.head_dim, L.max_seq_len, position + 1, part,
+                                 attn, stream))
+        return false;
+    // hidden += W_o attn
+    if (!run_matmul_device_ws(h_view, attn_view, o, L.o_type, q_dim, L.hidden, stream, mm_ws, nullptr, 0.f, true)) return false;
+    // hidden += W_down(silu(g) * u); the FFN reads hidden (RMSNorm) before its last kernel adds into it
+    return run_ffn_swiglu_device(h_view, h_view, ffn_norm, eps, gu, L.gu_type, down, L.down_type, L.hidden, L.intermediate, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int TSHip_TransformerLayerDecodeDevice(float* hidden, int hidden_size, const float* attn_norm, const void* qkv_data, int qkv_type,
+                                       int64_t qkv_ne0, int64_t qkv_ne1, int64_t qkv_bytes, const float* q_norm, const float* k_norm,
+                                       int head_dim, const void* o_data, int o_type, int64_t o_ne0, int64_t o_ne1, int64_t o_bytes,
+                                       const float* ffn_norm, const void* gu_data, int gu_type, int64_t gu_ne0, int64_t gu_ne1,
+                                       int64_t gu_bytes, const void* down_data, int down_type, int64_t down_ne0, int64_t down_ne1,
+                                       int64_t down_bytes, float* k_cache, float* v_cache, int num_heads, int num_kv_heads,
+                                       int max_seq_len, int position, float eps, float rope_base, float rope_freq_scale,
+                                       int intermediate_size, int rope_mode)
+{
+    return guarded(0, "transformer_layer_decode", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!hidden || !attn_norm || !qkv_data || !o_data || !ffn_norm || !gu_data || !down_data || !k_cache || !v_cache) {
+            set_last_error("Invalid arguments for transformer layer decode.");
+            return 0;
+        }
+        const LayerShape L{hidden_size, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate_size, qkv_type, o_type, gu_type,
+                           down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
+        if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
+        if (!run_layer_decode(hidden, L, attn_norm, qkv_data, q_norm, k_norm, o_data, ffn_norm, gu_data, down_data, k_cache, v_cache,
+                              position, eps, rope_base, rope_freq_scale, rope_mode, g_stream.load()))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_TransformerModelDecodeDevice(float* hidden, int hidden_size, int num_layers, const float* const* attn_norm,
+                                       const void* const* qkv, const float* const* q_norm, const float* const* k_norm,
+                                       const void* const* o, const float* const* ffn_norm, const void* const* gu,
+                                       const void* const* down, float* const* k_cache, float* const* v_cache, int qkv_type,
+                                       int64_t qkv_ne0, int64_t qkv_ne1, int64_t qkv_bytes, int o_type, int64_t o_ne0, int64_t o_ne1,
+                                       int64_t o_bytes, int gu_type, int64_t gu_ne0, int64_t gu_ne1, int64_t gu_bytes, int down_type,
+                                       int64_t down_ne0, int64_t down_ne1, int64_t down_bytes, int head_dim, int num_heads,
+                                       int num_kv_heads, int max_seq_len, int position, float eps, float rope_base,
+                                       float rope_freq_scale, int intermediate_size, int rope_mode)
+{
+    return guarded(0, "transformer_model_decode", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!hidden || num_layers <= 0 || !attn_norm || !qkv || !o || !ffn_norm || !gu || !down || !k_cache || !v_cache) {
+            set_last_error("Invalid arguments for transformer model decode.");
+            return 0;
+        }
+        const LayerShape L{hidden_size, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate_size, qkv_type, o_type, gu_type,
+                           down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
+        if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
+        for (int l = 0; l < num_layers; ++l) {
+            if (!attn_norm[l] || !qkv[l] || !o[l] || !ffn_norm[l] || !gu[l] || !down[l] || !k_cache[l] || !v_cache[l]) {
+                set_last_error("transformer model decode: a layer pointer is null.");
+                return 0;
+            }
+            if (!run_layer_decode(hidden, L, attn_norm[l], qkv[l], q_norm ? q_norm[l] : nullptr, k_norm ? k_norm[l] : nullptr, o[l],
+                                  ffn_norm[l], gu[l], down[l], k_cache[l], v_cache[l], position, eps, rope_base, rope_freq_scale,
+                                  rope_mode, g_stream.load()))
+                return 0;
+        }
+        clear_last_error();
+        return 1;
+    });
+}
+
+}  // extern "C"

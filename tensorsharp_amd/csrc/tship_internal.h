@@ -159,6 +159,17 @@ bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps
 // out[m, j] = silu(gu[m, j]) * gu[m, half + j], j < half
 bool launch_silu_mul(const float* gu, int64_t ldgu, int M, int half, float* out, hipStream_t stream);
 
+// ---- single-token attention of the whole-layer decode ---------------------------------------
+// qkv = [q heads | k heads | v heads], head_dim each: per-head RMSNorm (weights may be null) + RoPE; q -> q_out, k / v ->
+// row `position` of the caches [num_kv_heads][max_seq_len][head_dim]
+bool launch_qkv_post(const float* qkv, int num_heads, int num_kv_heads, int head_dim, const float* q_norm_w, const float* k_norm_w,
+                     float eps, int position, float rope_base, float rope_freq_scale, int rope_mode, float* q_out, float* k_cache,
+                     float* v_cache, int max_seq_len, hipStream_t stream);
+// out[h] = softmax(q[h] . K^T / sqrt(head_dim)) V over cache rows [0, total)
+size_t attention_decode_ws_bytes(int num_heads, int total);
+bool launch_attention_decode(const float* q, const float* k_cache, const float* v_cache, int num_heads, int num_kv_heads,
+                             int head_dim, int max_seq_len, int total, float* partial_ws, float* out, hipStream_t stream);
+
 // ---- MoE (GPT-OSS expert stage) -------------------------------------------------------------
 // ids / weights: [T x k] device; top-k by repeated argmax (first maximum wins), softmax over the k logits.
 bool launch_moe_route(const float* logits, int64_t ld, int T, int E, int k, int* ids, float* weights, hipStream_t stream);

@@ -271,6 +271,52 @@ class HipBasicOps:
         N.check_result(ok, "moe_experts_forward")
         return out
 
+    # -- whole-layer decode (GgmlBasicOps.TransformerLayerDecode / TransformerModelDecode twins) ----
+    @staticmethod
+    def TransformerLayerDecode(hidden, attn_norm, qkv, q_norm, k_norm, o, ffn_norm, gate_up, down, k_cache, v_cache,
+                               num_heads, num_kv_heads, head_dim, position, eps, rope_base, rope_freq_scale=1.0, rope_mode=2):
+        """One token through one layer, in place on `hidden` [hidden_size] (torch CUDA fp32).  qkv / o / gate_up / down are
+        device QuantizedWeights; k_cache / v_cache fp32 [num_kv_heads, max_seq_len, head_dim]; q_norm / k_norm may be None."""
+        HipBasicOps.UseCurrentStream()
+        p = lambda t: None if t is None else t.data_ptr()
+        ok = N.lib().TSHip_TransformerLayerDecodeDevice(
+            hidden.data_ptr(), int(hidden.numel()), attn_norm.data_ptr(),
+            qkv.ptr, qkv.ggml_type, qkv.ne0, qkv.ne1, qkv.raw_bytes, p(q_norm), p(k_norm), int(head_dim),
+            o.ptr, o.ggml_type, o.ne0, o.ne1, o.raw_bytes, ffn_norm.data_ptr(),
+            gate_up.ptr, gate_up.ggml_type, gate_up.ne0, gate_up.ne1, gate_up.raw_bytes,
+            down.ptr, down.ggml_type, down.ne0, down.ne1, down.raw_bytes,
+            k_cache.data_ptr(), v_cache.data_ptr(), int(num_heads), int(num_kv_heads), int(k_cache.shape[1]), int(position),
+            float(eps), float(rope_base), float(rope_freq_scale), int(gate_up.ne1 // 2), int(rope_mode))
+        N.check_result(ok, "transformer_layer_decode")
+
+    @staticmethod
+    def TransformerModelDecode(hidden, layers, num_heads, num_kv_heads, head_dim, position, eps, rope_base, rope_freq_scale=1.0,
+                               rope_mode=2):
+        """The same for a list of layers; each layer is a dict with the argument names of TransformerLayerDecode
+        (attn_norm, qkv, q_norm, k_norm, o, ffn_norm, gate_up, down, k_cache, v_cache); shapes and types are shared."""
+        import ctypes as C
+        HipBasicOps.UseCurrentStream()
+        n = len(layers)
+
+        def arr(key, weight=False):
+            vals = []
+            for L in layers:
+                t = L.get(key)
+                vals.append(None if t is None else (t.ptr if weight else t.data_ptr()))
+            if all(v is None for v in vals):
+                return None
+            return (C.c_void_p * n)(*vals)
+        l0 = layers[0]
+        qkv, o, gu, dn = l0["qkv"], l0["o"], l0["gate_up"], l0["down"]
+        ok = N.lib().TSHip_TransformerModelDecodeDevice(
+            hidden.data_ptr(), int(hidden.numel()), n, arr("attn_norm"), arr("qkv", True), arr("q_norm"), arr("k_norm"), arr("o", True),
+            arr("ffn_norm"), arr("gate_up", True), arr("down", True), arr("k_cache"), arr("v_cache"),
+            qkv.ggml_type, qkv.ne0, qkv.ne1, qkv.raw_bytes, o.ggml_type, o.ne0, o.ne1, o.raw_bytes,
+            gu.ggml_type, gu.ne0, gu.ne1, gu.raw_bytes, dn.ggml_type, dn.ne0, dn.ne1, dn.raw_bytes,
+            int(head_dim), int(num_heads), int(num_kv_heads), int(l0["k_cache"].shape[1]), int(position), float(eps),
+            float(rope_base), float(rope_freq_scale), int(gu.ne1 // 2), int(rope_mode))
+        N.check_result(ok, "transformer_model_decode")
+
     # -- LinearForward twin (ModelBase.cs:875-905): allocate result, route by residency -----
     @staticmethod
     def LinearForward(m1, qw: QuantizedWeight):

@@ -81,6 +81,22 @@ SIGNATURES = {
     "TSHip_MoEExpertsForwardF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int64,
                                                    C.c_int64, C.c_float, C.c_float]),
+    "TSHip_TransformerLayerDecodeDevice": (C.c_int, [
+        C.c_void_p, C.c_int, C.c_void_p,
+        C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+        C.c_void_p, C.c_void_p, C.c_int,
+        C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+        C.c_void_p,
+        C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+        C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+        C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
+    "TSHip_TransformerModelDecodeDevice": (C.c_int, [
+        C.c_void_p, C.c_int, C.c_int,
+        C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+        C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+        C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+        C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+        C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
 }
 
 
