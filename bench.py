@@ -280,6 +280,41 @@ def main():
 
         extra["cfg4_mxfp4_moe_experts_T1"] = moe(1, n_it)
         extra["cfg4_mxfp4_moe_experts_T256"] = moe(256, 30)
+        # whole-layer decode (TransformerLayerDecode) at configs[1] shapes: hidden 4096, 32 heads / 8 KV heads of 128,
+        # intermediate 14336, Q4_K weights (fused QKV 6144 x 4096 and gate_up 28672 x 4096), fp32 KV cache; 8 distinct
+        # layers cycled (984 MB of weights).  Bytes = weights + the KV rows read by the attention.
+        def layer_decode(context, iters):
+            hidden, heads, kvh, hd, inter, max_seq = 4096, 32, 8, 128, 14336, 4096
+            q_dim, k_dim = heads * hd, kvh * hd
+            mk = lambda n, k, sd: QuantizedWeight(synth.random_weight(Q4_K, n, k, dev, seed=sd), Q4_K, k, n)
+            layers = []
+            for c in range(8):
+                layers.append({"qkv": mk(q_dim + 2 * k_dim, hidden, 3000 + 10 * c), "o": mk(hidden, q_dim, 3001 + 10 * c),
+                               "gate_up": mk(2 * inter, hidden, 3002 + 10 * c), "down": mk(hidden, inter, 3003 + 10 * c),
+                               "attn_norm": torch.ones(hidden, device=dev), "ffn_norm": torch.ones(hidden, device=dev),
+                               "q_norm": torch.ones(hd, device=dev), "k_norm": torch.ones(hd, device=dev),
+                               "k_cache": torch.randn((kvh, max_seq, hd), device=dev), "v_cache": torch.randn((kvh, max_seq, hd), device=dev)})
+            h = torch.randn(hidden, device=dev)
+            pos = context - 1
+
+            def f(i):
+                L = layers[i % 8]
+                HipBasicOps.TransformerLayerDecode(h, L["attn_norm"], L["qkv"], L["q_norm"], L["k_norm"], L["o"], L["ffn_norm"],
+                                                   L["gate_up"], L["down"], L["k_cache"], L["v_cache"], heads, kvh, hd, pos, 1e-6,
+                                                   10000.0, 1.0, 2)
+                if i % 8 == 7:
+                    h.normal_()           # keep the running hidden state bounded
+            for i in range(16):
+                f(i)
+            ev, wall = time_region(f, iters, torch)
+            us = ev * 1e3 / iters
+            wbytes = sum(layers[0][k].raw_bytes for k in ("qkv", "o", "gate_up", "down"))
+            b = wbytes + 2 * kvh * context * hd * 4
+            return {"us_per_layer_events": round(us, 1), "bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                    "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1), "context": context}
+
+        extra["cfg2_q4_k_layer_decode_ctx512"] = layer_decode(512, 200)
+        extra["cfg2_q4_k_layer_decode_ctx4096"] = layer_decode(4096, 200)
         # fused SwiGLU FFN at decode (configs[1] shapes: hidden 4096, intermediate 14336, Q4_K, one token):
         # RMSNorm -> gate_up GEMV -> SiLU*up -> down GEMV + residual, one ABI call (4 launches)
         def fused_ffn(copies=3):

@@ -5,9 +5,10 @@
 //                        (ggml_rope_ext with n_dims = head_dim, ext_factor 0, attn_factor 1: ggml-cpu/ops.cpp:5549-5563,
 //                        :5636-5652); q heads go to a scratch row, k heads and the untouched v heads into the fp32 KV
 //                        cache [kv_head][max_seq_len][head_dim] at row `position`
-//   attn_decode_kernel   softmax(q . K^T / sqrt(head_dim)) V over positions 0..position for one query head, grouped-query
-//                        heads sharing their KV head (what ggml_flash_attn_ext computes for one query row); the positions
-//                        are cut into splits of 256, each split leaves (max, sum, weighted V) behind
+//   attn_decode_kernel   softmax(q . K^T / sqrt(head_dim)) V over positions 0..position (what ggml_flash_attn_ext computes
+//                        for one query row); a workgroup serves the query heads that share a KV head, so K / V rows are
+//                        loaded once per group; the positions are cut into splits of 256, each split leaves
+//                        (max, sum, weighted V) behind (a single split writes the result itself)
 //   attn_combine_kernel  merges the splits of a head
 //
 // HBM-bound on the KV cache: 2 * num_kv_heads * (position + 1) * head_dim * 4 bytes per call.
@@ -76,78 +77,129 @@ __global__ void __launch_bounds__(64) qkv_post_kernel(const float* __restrict__ 
     }
 }
 
-// grid (num_heads, splits): 4 wavefronts, wavefront w takes positions w, w + 4, ... of the split; lane l holds the
-// head dimensions l, l + 64, ...
-__global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ k_cache,
-                                                                       const float* __restrict__ v_cache, int head_dim, int group,
-                                                                       int max_seq_len, int total, float scale,
-                                                                       float* __restrict__ partial)
+// Merge of two online-softmax states (max, sum, weighted values).
+template <int N>
+__device__ __forceinline__ void softmax_merge(float& m, float& l, float (&acc)[N], float m2, float l2, const float (&acc2)[N])
 {
-    constexpr int kPer = kMaxHeadDim / 64;
-    __shared__ float sm[kAttnWaves], sl[kAttnWaves], sacc[kAttnWaves][kMaxHeadDim];
-    const int h = blockIdx.x, split = blockIdx.y;
+    const float mm = fmaxf(m, m2);
+    const float f1 = m == -INFINITY ? 0.f : expf(m - mm), f2 = m2 == -INFINITY ? 0.f : expf(m2 - mm);
+    l = l * f1 + l2 * f2;
+#pragma unroll
+    for (int j = 0; j < N; ++j) acc[j] = acc[j] * f1 + acc2[j] * f2;
+    m = mm;
+}
+
+// grid (num_kv_heads, splits, q-head chunks): one workgroup serves G query heads that share a KV head, so every K / V
+// row is loaded once for all of them.  4 wavefronts x 4 groups of 16 lanes; a group takes positions g, g + 16, ... of
+// the split, two at a time (both rows' loads are issued before either is used: the loop is latency bound), lane l of
+// a group holds the head dimensions l, l + 16, ... (PER of them).  Groups, then wavefronts, merge their softmax states.
+template <int PER, int G>
+__global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ k_cache,
+                                                                       const float* __restrict__ v_cache, int group, int max_seq_len,
+                                                                       int total, float scale, int splits, float* __restrict__ partial,
+                                                                       float* __restrict__ out_direct)
+{
+    constexpr int HD = 16 * PER;
+    __shared__ float sm[kAttnWaves][G], sl[kAttnWaves][G], sacc[kAttnWaves][G][HD];
+    const int kvh = blockIdx.x, split = blockIdx.y;
+    const int h0 = kvh * group + blockIdx.z * G;                     // first query head of this workgroup
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int kvh = h / group;
-    const float* kb = k_cache + (int64_t)kvh * max_seq_len * head_dim;
-    const float* vb = v_cache + (int64_t)kvh * max_seq_len * head_dim;
-    float qr[kPer], acc[kPer];
+    const int lg = lane & 15, grp = (wave << 2) | (lane >> 4);       // 16 groups per workgroup
+    const float* kb = k_cache + (int64_t)kvh * max_seq_len * HD;
+    const float* vb = v_cache + (int64_t)kvh * max_seq_len * HD;
+    float qr[G][PER], acc[G][PER], m[G], l[G];
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        const int d = lane + 64 * j;
-        qr[j] = d < head_dim ? q[(int64_t)h * head_dim + d] : 0.f;
-        acc[j] = 0.f;
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            qr[g][j] = q[(int64_t)(h0 + g) * HD + lg + 16 * j] * scale;
+            acc[g][j] = 0.f;
+        }
     }
-    float m = -INFINITY, l = 0.f;
     const int t_end = min(total, (split + 1) * kSplit);
-    for (int t = split * kSplit + wave; t < t_end; t += kAttnWaves) {
-        const float* kr = kb + (int64_t)t * head_dim;
-        float dot = 0.f;
+    for (int t = split * kSplit + grp; t < t_end; t += 32) {
+        const int t2 = t + 16;
+        const bool two = t2 < t_end;
+        const float* k1 = kb + (int64_t)t * HD + lg;
+        const float* v1 = vb + (int64_t)t * HD + lg;
+        const float* k2 = kb + (int64_t)(two ? t2 : t) * HD + lg;
+        const float* v2 = vb + (int64_t)(two ? t2 : t) * HD + lg;
+        float ka[PER], va[PER], kc[PER], vc[PER];
 #pragma unroll
-        for (int j = 0; j < kPer; ++j) {
-            const int d = lane + 64 * j;
-            if (d < head_dim) dot += qr[j] * kr[d];
+        for (int j = 0; j < PER; ++j) {
+            ka[j] = k1[16 * j];
+            kc[j] = k2[16 * j];
+            va[j] = v1[16 * j];
+            vc[j] = v2[16 * j];
         }
-        const float s = wave_sum(dot) * scale;
-        const float mn = fmaxf(m, s);
-        const float corr = expf(m - mn), p = expf(s - mn);       // exp(-inf) = 0 on the first position
-        const float* vr = vb + (int64_t)t * head_dim;
-        l = l * corr + p;
 #pragma unroll
-        for (int j = 0; j < kPer; ++j) {
-            const int d = lane + 64 * j;
-            if (d < head_dim) acc[j] = acc[j] * corr + p * vr[d];
+        for (int g = 0; g < G; ++g) {
+            float d1 = 0.f, d2 = 0.f;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                d1 += qr[g][j] * ka[j];
+                d2 += qr[g][j] * kc[j];
+            }
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) {
+                d1 += __shfl_xor(d1, o);
+                d2 += __shfl_xor(d2, o);
+            }
+            if (!two) d2 = -INFINITY;
+            const float mn = fmaxf(m[g], fmaxf(d1, d2));
+            const float corr = expf(m[g] - mn), p1 = expf(d1 - mn), p2 = expf(d2 - mn);      // exp(-inf) = 0
+            l[g] = l[g] * corr + p1 + p2;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) acc[g][j] = acc[g][j] * corr + p1 * va[j] + p2 * vc[j];
+            m[g] = mn;
         }
-        m = mn;
     }
-    if (lane == 0) {
-        sm[wave] = m;
-        sl[wave] = l;
-    }
+    // the four groups of a wavefront
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) sacc[wave][lane + 64 * j] = acc[j];
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int o = 16; o <= 32; o <<= 1) {
+            const float m2 = __shfl_xor(m[g], o), l2 = __shfl_xor(l[g], o);
+            float a2[PER];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) a2[j] = __shfl_xor(acc[g][j], o);
+            softmax_merge<PER>(m[g], l[g], acc[g], m2, l2, a2);
+        }
+        if (lane < 16) {
+            if (lane == 0) {
+                sm[wave][g] = m[g];
+                sl[wave][g] = l[g];
+            }
+#pragma unroll
+            for (int j = 0; j < PER; ++j) sacc[wave][g][lg + 16 * j] = acc[g][j];
+        }
+    }
     __syncthreads();
-    if (wave == 0) {
+    // the four wavefronts: thread (g, d) of the first G * HD threads
+    for (int i = threadIdx.x; i < G * HD; i += kAttnWaves * 64) {
+        const int g = i / HD, d = i - g * HD;
         float mm = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kAttnWaves; ++w) mm = fmaxf(mm, sm[w]);
-        float ll = 0.f;
-        float out[kPer];
-#pragma unroll
-        for (int j = 0; j < kPer; ++j) out[j] = 0.f;
+        for (int w = 0; w < kAttnWaves; ++w) mm = fmaxf(mm, sm[w][g]);
+        float ll = 0.f, out = 0.f;
 #pragma unroll
         for (int w = 0; w < kAttnWaves; ++w) {
-            const float f = sm[w] == -INFINITY ? 0.f : expf(sm[w] - mm);     // a wavefront without positions
-            ll += sl[w] * f;
-#pragma unroll
-            for (int j = 0; j < kPer; ++j) out[j] += sacc[w][lane + 64 * j] * f;
+            const float f = sm[w][g] == -INFINITY ? 0.f : expf(sm[w][g] - mm);
+            ll += sl[w][g] * f;
+            out += sacc[w][g][d] * f;
         }
-        float* dst = partial + ((int64_t)h * gridDim.y + split) * (kMaxHeadDim + 2);
-        if (lane == 0) {
+        if (out_direct) {
+            out_direct[(int64_t)(h0 + g) * HD + d] = out / ll;       // a single split: this is the result
+            continue;
+        }
+        float* dst = partial + ((int64_t)(h0 + g) * splits + split) * (kMaxHeadDim + 2);
+        if (d == 0) {
             dst[0] = mm;
             dst[1] = ll;
         }
-#pragma unroll
-        for (int j = 0; j < kPer; ++j) dst[2 + lane + 64 * j] = out[j];
+        dst[2 + d] = out;
     }
 }
 
@@ -213,9 +265,32 @@ bool launch_attention_decode(const float* q, const float* k_cache, const float* 
         return false;
     }
     const float scale = 1.0f / sqrtf((float)head_dim);
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(num_heads, splits), dim3(kAttnWaves * 64), 0, stream, q, k_cache, v_cache, head_dim,
-                       num_heads / num_kv_heads, max_seq_len, total, scale, partial_ws);
+    const int group = num_heads / num_kv_heads;
+    const int g = group % 8 == 0 ? 8 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;     // query heads per workgroup
+    const dim3 grid(num_kv_heads, splits, group / g), block(kAttnWaves * 64);
+#define TSHIP_ATTN_LAUNCH(PER, GG)                                                                                              \
+    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, q, k_cache, v_cache, group, max_seq_len, total, scale, \
+                       splits, partial_ws, splits == 1 ? out : nullptr)
+#define TSHIP_ATTN_G(PER)                                                    \
+    switch (g) {                                                             \
+    case 8: TSHIP_ATTN_LAUNCH(PER, 8); break;                                \
+    case 4: TSHIP_ATTN_LAUNCH(PER, 4); break;                                \
+    case 2: TSHIP_ATTN_LAUNCH(PER, 2); break;                                \
+    default: TSHIP_ATTN_LAUNCH(PER, 1); break;                               \
+    }
+    switch (head_dim) {
+    case 64: TSHIP_ATTN_G(4) break;
+    case 80: TSHIP_ATTN_G(5) break;
+    case 96: TSHIP_ATTN_G(6) break;
+    case 128: TSHIP_ATTN_G(8) break;
+    case 192: TSHIP_ATTN_G(12) break;
+    case 256: TSHIP_ATTN_G(16) break;
+    default: set_last_error("layer decode: head_dim must be one of 64, 80, 96, 128, 192, 256."); return false;
+    }
+#undef TSHIP_ATTN_G
+#undef TSHIP_ATTN_LAUNCH
     if (!hip_ok(hipGetLastError(), "attention launch")) return false;
+    if (splits == 1) return true;
     hipLaunchKernelGGL(attn_combine_kernel, dim3(num_heads), dim3(64), 0, stream, partial_ws, splits, head_dim, out);
     return hip_ok(hipGetLastError(), "attention combine launch");
 }
