@@ -18,7 +18,8 @@ namespace tship {
 namespace {
 
 constexpr int kMaxHeadDim = 256;
-constexpr int kSplit = 256;          // positions per workgroup of the attention kernel
+constexpr int kSplit = 128;          // positions per workgroup of the attention kernel
+constexpr int kInFlight = 4;         // K / V rows a 16-lane group loads before it uses the first
 constexpr int kAttnWaves = 4;
 
 __device__ __forceinline__ float wave_sum(float v)
@@ -91,7 +92,7 @@ __device__ __forceinline__ void softmax_merge(float& m, float& l, float (&acc)[N
 
 // grid (num_kv_heads, splits, q-head chunks): one workgroup serves G query heads that share a KV head, so every K / V
 // row is loaded once for all of them.  4 wavefronts x 4 groups of 16 lanes; a group takes positions g, g + 16, ... of
-// the split, two at a time (both rows' loads are issued before either is used: the loop is latency bound), lane l of
+// the split, kInFlight at a time (all their loads are issued before the first is used: the loop is latency bound), lane l of
 // a group holds the head dimensions l, l + 16, ... (PER of them).  Groups, then wavefronts, merge their softmax states.
 template <int PER, int G>
 __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ k_cache,
@@ -119,40 +120,55 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const floa
         }
     }
     const int t_end = min(total, (split + 1) * kSplit);
-    for (int t = split * kSplit + grp; t < t_end; t += 32) {
-        const int t2 = t + 16;
-        const bool two = t2 < t_end;
-        const float* k1 = kb + (int64_t)t * HD + lg;
-        const float* v1 = vb + (int64_t)t * HD + lg;
-        const float* k2 = kb + (int64_t)(two ? t2 : t) * HD + lg;
-        const float* v2 = vb + (int64_t)(two ? t2 : t) * HD + lg;
-        float ka[PER], va[PER], kc[PER], vc[PER];
+    for (int t0 = split * kSplit + grp; t0 < t_end; t0 += 16 * kInFlight) {
+        // kInFlight rows of K and of V per group: every load is issued before the first use
+        float kr[kInFlight][PER], vr[kInFlight][PER];
+        bool live[kInFlight];
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            ka[j] = k1[16 * j];
-            kc[j] = k2[16 * j];
-            va[j] = v1[16 * j];
-            vc[j] = v2[16 * j];
+        for (int u = 0; u < kInFlight; ++u) {
+            const int t = t0 + 16 * u;
+            live[u] = t < t_end;
+            const int64_t row = (int64_t)(live[u] ? t : t0) * HD + lg;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                kr[u][j] = kb[row + 16 * j];
+                vr[u][j] = vb[row + 16 * j];
+            }
         }
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            float d1 = 0.f, d2 = 0.f;
+            float d[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                d[u] = 0.f;
+#pragma unroll
+                for (int j = 0; j < PER; ++j) d[u] += qr[g][j] * kr[u][j];
+            }
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1)
+#pragma unroll
+                for (int u = 0; u < kInFlight; ++u) d[u] += __shfl_xor(d[u], o);
+            float mn = m[g];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                if (!live[u]) d[u] = -INFINITY;
+                mn = fmaxf(mn, d[u]);
+            }
+            const float corr = expf(m[g] - mn);                    // exp(-inf) = 0 on the first rows
+            float p[kInFlight], psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                p[u] = expf(d[u] - mn);
+                psum += p[u];
+            }
+            l[g] = l[g] * corr + psum;
 #pragma unroll
             for (int j = 0; j < PER; ++j) {
-                d1 += qr[g][j] * ka[j];
-                d2 += qr[g][j] * kc[j];
-            }
+                float a = acc[g][j] * corr;
 #pragma unroll
-            for (int o = 8; o > 0; o >>= 1) {
-                d1 += __shfl_xor(d1, o);
-                d2 += __shfl_xor(d2, o);
+                for (int u = 0; u < kInFlight; ++u) a += p[u] * vr[u][j];
+                acc[g][j] = a;
             }
-            if (!two) d2 = -INFINITY;
-            const float mn = fmaxf(m[g], fmaxf(d1, d2));
-            const float corr = expf(m[g] - mn), p1 = expf(d1 - mn), p2 = expf(d2 - mn);      // exp(-inf) = 0
-            l[g] = l[g] * corr + p1 + p2;
-#pragma unroll
-            for (int j = 0; j < PER; ++j) acc[g][j] = acc[g][j] * corr + p1 * va[j] + p2 * vc[j];
             m[g] = mn;
         }
     }
@@ -203,25 +219,61 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const floa
     }
 }
 
-__global__ void __launch_bounds__(64) attn_combine_kernel(const float* __restrict__ partial, int splits, int head_dim,
-                                                          float* __restrict__ out)
+// one workgroup per head: wavefront w merges splits w, w + 4, ... (four rows in flight), the wavefronts meet in LDS
+__global__ void __launch_bounds__(kAttnWaves * 64) attn_combine_kernel(const float* __restrict__ partial, int splits, int head_dim,
+                                                                        float* __restrict__ out)
 {
-    const int h = blockIdx.x, lane = threadIdx.x;
-    const float* base = partial + (int64_t)h * splits * (kMaxHeadDim + 2);
+    constexpr int kPer = kMaxHeadDim / 64, kRow = kMaxHeadDim + 2;
+    __shared__ float sacc[kAttnWaves][kMaxHeadDim], sl[kAttnWaves];
+    const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* base = partial + (int64_t)h * splits * kRow;
+    // the maximum over all splits: every wavefront computes it (independent loads, one pass)
     float mm = -INFINITY;
-    for (int s = 0; s < splits; ++s) mm = fmaxf(mm, base[(int64_t)s * (kMaxHeadDim + 2)]);
-    float ll = 0.f;
-    for (int s = 0; s < splits; ++s) {
-        const float* p = base + (int64_t)s * (kMaxHeadDim + 2);
-        ll += p[1] * expf(p[0] - mm);
-    }
-    for (int d = lane; d < head_dim; d += 64) {
-        float acc = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const float* p = base + (int64_t)s * (kMaxHeadDim + 2);
-            acc += p[2 + d] * expf(p[0] - mm);
+    for (int s = lane; s < splits; s += 64) mm = fmaxf(mm, base[(int64_t)s * kRow]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
+    float acc[kPer], ll = 0.f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) acc[j] = 0.f;
+    for (int s0 = wave; s0 < splits; s0 += 4 * kAttnWaves) {
+        float ms[4], ls[4], v[4][kPer];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = s0 + u * kAttnWaves;
+            const bool live = s < splits;
+            const float* p = base + (int64_t)(live ? s : s0) * kRow;
+            ms[u] = live ? p[0] : -INFINITY;
+            ls[u] = p[1];
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) {
+                const int d = lane + 64 * j;
+                v[u][j] = d < head_dim ? p[2 + d] : 0.f;
+            }
         }
-        out[(int64_t)h * head_dim + d] = acc / ll;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float f = ms[u] == -INFINITY ? 0.f : expf(ms[u] - mm);
+            ll += ls[u] * f;
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) acc[j] += v[u][j] * f;
+        }
+    }
+    if (lane == 0) sl[wave] = ll;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) sacc[wave][lane + 64 * j] = acc[j];
+    __syncthreads();
+    if (wave == 0) {
+        float lt = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) lt += sl[w];
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+            const int d = lane + 64 * j;
+            float a = 0.f;
+#pragma unroll
+            for (int w = 0; w < kAttnWaves; ++w) a += sacc[w][d];
+            if (d < head_dim) out[(int64_t)h * head_dim + d] = a / lt;
+        }
     }
 }
 
@@ -291,7 +343,7 @@ bool launch_attention_decode(const float* q, const float* k_cache, const float* 
 #undef TSHIP_ATTN_LAUNCH
     if (!hip_ok(hipGetLastError(), "attention launch")) return false;
     if (splits == 1) return true;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(num_heads), dim3(64), 0, stream, partial_ws, splits, head_dim, out);
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(num_heads), dim3(kAttnWaves * 64), 0, stream, partial_ws, splits, head_dim, out);
     return hip_ok(hipGetLastError(), "attention combine launch");
 }
 
