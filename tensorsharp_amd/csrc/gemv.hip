@@ -29,6 +29,7 @@
 #include "tship_internal.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 namespace tship {
@@ -471,7 +472,9 @@ struct Step {
 
 // ACT: the activation mode of every problem of the launch (compile time: the plain kernel carries none of
 // the other modes' code or registers)
-template <typename F, int ACT>
+// KS: wavefronts that share a row group, each taking 1/KS of its steps (few rows, long K: one group per wavefront would
+// leave most wavefronts without work); their sums meet in LDS.  KS = 1 is the plain scheme.
+template <typename F, int ACT, int KS>
 __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, uint32_t* lds)
 {
     const int lane = threadIdx.x & 63;
@@ -620,10 +623,29 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // prologue; in the loop the next kU steps are requested before the current ones are consumed.
     Step<F> cur[kU], nxt[kU];
     int fgroup = gw, fstep = 0;                // next step to fetch
+    // K-split scheme: rounds of kWaves / KS row groups per workgroup; wavefront (gslot, slice) takes steps
+    // [s_begin, s_end) of its group
+    constexpr int GPW = kWaves / KS;
+    const int wv = (int)(threadIdx.x >> 6), slice = wv % KS, gslot = wv / KS;
+    const int s_begin = slice * nsteps / KS, s_end = (slice + 1) * nsteps / KS;
+    const int rounds = (ngroups + nwg * GPW - 1) / (nwg * GPW);
+    auto group_of = [&](int r) { return r < rounds ? (r * nwg + wg) * GPW + gslot : ngroups; };
+    int fr = 0, fs = s_begin;
+    auto fetch_next = [&](Step<F>& st) {
+        fetch(group_of(fr), fs, st);
+        if (++fs >= s_end) {
+            fs = s_begin;
+            ++fr;
+        }
+    };
+    if constexpr (KS > 1) {
+        fetch_next(cur[0]);
+    } else {
 #pragma unroll
-    for (int i = 0; i < kU; ++i) {
-        fetch(fgroup, fstep, cur[i]);
-        advance(fgroup, fstep);
+        for (int i = 0; i < kU; ++i) {
+            fetch(fgroup, fstep, cur[i]);
+            advance(fgroup, fstep);
+        }
     }
     if (!TSHIP_GEMV_XFIRST) stage_issue(0);
 #ifdef TSHIP_GEMV_DEBUG_NOSTAGE
@@ -638,6 +660,35 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nsteps * 16 * F::kLdsDwords; i += kThreads) lds[i] = 0u;
     __syncthreads();
 
+    if constexpr (KS > 1) {
+        // Every wavefront of the workgroup runs every round (groups past the end read zeros), so the barrier is uniform.
+        float* part = reinterpret_cast<float*>(red + kWaves);        // [2][kWaves][4]
+        for (int r = 0; r < rounds; ++r) {
+            float acc = 0.f;
+            for (int st = s_begin; st < s_end; ++st) {
+                fetch_next(nxt[0]);
+                const uint32_t* xu = lds + lds_lane + (uint32_t)cur[0].step * (16u * F::kLdsDwords);
+                acc += F::dot(cur[0].w, L, cur[0].aux, xu);
+                cur[0] = nxt[0];
+            }
+            float t = acc;
+            t += TSHIP_DPP_F(t, kDppXor1);
+            t += TSHIP_DPP_F(t, kDppXor2);
+            t += TSHIP_DPP_F(t, kDppHalfMirror);
+            t += TSHIP_DPP_F(t, kDppMirror);
+            float* pr = part + (r & 1) * kWaves * 4;
+            if (l16 == 0) pr[wv * 4 + sub] = t;
+            __syncthreads();
+            const int group = group_of(r), row = group * 4 + sub;
+            if (slice == 0 && l16 == 0 && group < ngroups && row < N) {
+                float sum = 0.f;
+#pragma unroll
+                for (int k = 0; k < KS; ++k) sum += pr[(wv + k) * 4 + sub];
+                P.y[row] = P.add ? P.add[row] + sum : sum;
+            }
+        }
+        return;
+    }
     float acc = 0.f;
     while (cur[0].group < ngroups) {
 #pragma unroll
@@ -666,7 +717,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     }
 }
 
-template <int TYPE, int ACT>
+template <int TYPE, int ACT, int KS>
 __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
 {
     extern __shared__ uint32_t lds[];
@@ -676,9 +727,9 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
         if (j < G.count && (int)blockIdx.x >= G.wg_begin[j]) i = j;
     const int wg = (int)blockIdx.x - G.wg_begin[i];
     const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
-    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT>(G.p[i], wg, nwg, lds);
-    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT>(G.p[i], wg, nwg, lds);
-    else gemv_body<FmtQ80, ACT>(G.p[i], wg, nwg, lds);
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, KS>(G.p[i], wg, nwg, lds);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, lds);
+    else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, lds);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
@@ -687,15 +738,16 @@ int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
 size_t lds_bytes_for(int type, int K)
 {
     const size_t units = (size_t)((K / unit_elems(type) + 15) / 16) * 16;
-    return units * (type == kTypeMXFP4 ? 80 : 144) + kWaves * sizeof(double);   // + the RMSNorm reduction slots
+    // + the RMSNorm reduction slots + the partial row sums of the K-split scheme
+    return units * (type == kTypeMXFP4 ? 80 : 144) + kWaves * sizeof(double) + 2 * kWaves * 4 * sizeof(float);
 }
 
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 
-template <int TYPE, int ACT>
+template <int TYPE, int ACT, int KS = 1>
 bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    auto kern = gemv_kernel<TYPE, ACT>;
+    auto kern = gemv_kernel<TYPE, ACT, KS>;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g);
     return hip_ok(hipGetLastError(), "gemv launch");
@@ -746,6 +798,16 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     int per_cu = (int)std::min<size_t>(TSHIP_GEMV_WG_PER_CU, (160 * 1024) / (lds + 256));
     if (per_cu < 1) per_cu = 1;
     const int budget = di.num_cus * per_cu;
+    // A single matrix with so few rows that one row group per wavefront would keep less than half of the wavefronts
+    // busy, and rows long enough to cut: four wavefronts share a row group, each taking a quarter of its steps.
+    // Only with plain activations: four times as many workgroups stage x, and measured with the SiLU / RMSNorm
+    // staging modes that costs more than the extra wavefronts win (4096 x 14336 Q4_K: plain 14.7 -> 12.6 us,
+    // SiLU mode inside the fused FFN 32.7 -> 34.3 us).
+    int ksplit = 1;
+    if (count == 1 && args[0].act == kActPlain) {
+        const int ngroups = (args[0].N + 3) / 4, nsteps = (args[0].K / unit_elems(type) + 15) / 16;
+        if (ngroups * 2 <= budget * kWaves && nsteps >= 8) ksplit = 4;
+    }
 
     GemvGroup g;
     std::memset(&g, 0, sizeof(g));
@@ -754,7 +816,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     for (int i = 0; i < count; ++i) {
         // workgroups in proportion to the bytes each problem streams
         int share = std::max(1, (int)((double)budget * (double)args[i].w_bytes / total_bytes + 0.5));
-        share = std::min(share, ((args[i].N + 3) / 4 + kWaves - 1) / kWaves);
+        share = std::min(share, ((args[i].N + 3) / 4 + kWaves / ksplit - 1) / (kWaves / ksplit));
         g.p[i].w = static_cast<const uint8_t*>(args[i].w);
         g.p[i].w_bytes = args[i].w_bytes;
         g.p[i].x = args[i].x;
@@ -787,7 +849,8 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         return false;
     }
 #define TSHIP_GEMV_DISPATCH(T)                                                           \
-    (act == kActPlain     ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
+    (ksplit == 4          ? launch_type<T, kActPlain, 4>(g, begin, lds, stream)          \
+     : act == kActPlain   ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
      : act == kActRmsNorm ? launch_type<T, kActRmsNorm>(g, begin, lds, stream)           \
      : act == kActSiluMul ? launch_type<T, kActSiluMul>(g, begin, lds, stream)           \
                           : launch_type<T, kActSwigluOai>(g, begin, lds, stream))

@@ -212,3 +212,22 @@ def test_grouped_full_layer(hip, oracle):
     torch.cuda.synchronize()
     for y, ref in zip(ys, refs):
         check("q4_k", y.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("name,N,K", [("q4_k", 1001, 14336), ("q8_0", 515, 8192 + 32), ("mxfp4", 2880, 5760), ("q4_k", 6, 8192),
+                                      ("q8_0", 4096, 4096 + 64)])
+def test_few_rows_long_k_split_over_wavefronts(hip, oracle, name, N, K):
+    # few rows, long K: four wavefronts share a row group and each takes a quarter of its steps; also as y = add + W x
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(N + K)
+    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    ref = oracle.matmul_f64(T[name], wq, N, K, x)
+    check(name, run_device(hip, T[name], wq, N, K, x), ref)
+    resid = rng.standard_normal((1, N)).astype(np.float32)
+    r = torch.from_numpy(resid.copy()).cuda()
+    hip.FusedMatMulQuantAdd(r, torch.from_numpy(x).cuda(), QuantizedWeight(torch.from_numpy(wq).cuda(), T[name], K, N))
+    torch.cuda.synchronize()
+    got = r.cpu().numpy().astype(np.float64) - resid
+    assert np.max(np.abs(got - ref)) <= 1e-3 * np.linalg.norm(ref) + 1e-6 * np.max(np.abs(resid)), name
