@@ -177,7 +177,7 @@ def main():
                    "bytes_per_step": step_bytes, "launches_per_step": 1, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "tship::gemv_kernel<12, R> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
+                     "kernel": "tship::gemv_kernel<12, 0, 1> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
                      "bytes_per_launch": step_bytes},
     }
 
