@@ -237,7 +237,6 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
 struct GQ4K {
     static constexpr int kRegs = 8;
     static constexpr int kSup = 4;            // one 256-element super-block
-    static constexpr int kSupBytes = 144;
     static constexpr int kRawRow = 144;       // LDS bytes of one row's super-tile window
     static constexpr int kTileStep = 4;       // a wavefront's K range starts at a multiple of this many k-tiles
     static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 144u; }            // window start of super-tile s
@@ -284,7 +283,6 @@ struct GQ4K {
 struct GMXFP4 {
     static constexpr int kRegs = 5;
     static constexpr int kSup = 4;            // eight 17-byte blocks
-    static constexpr int kSupBytes = 136;
     static constexpr int kRawRow = 144;
     static constexpr int kTileStep = 2;
     static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 136u; }
@@ -331,7 +329,6 @@ struct GMXFP4 {
 struct GQ80 {
     static constexpr int kRegs = 9;
     static constexpr int kSup = 2;            // four 34-byte blocks
-    static constexpr int kSupBytes = 136;
     static constexpr int kRawRow = 144;
     static constexpr int kTileStep = 2;
     static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 136u; }
@@ -371,7 +368,6 @@ struct GQ80 {
 struct GQ6K {
     static constexpr int kRegs = 20;
     static constexpr int kSup = 4;            // one 256-element block
-    static constexpr int kSupBytes = 210;
     static constexpr int kRawRow = 240;       // 60 dwords: the dword reads of 32 rows spread over 16 banks (224 bytes: 8)
     static constexpr int kTileStep = 4;
     static constexpr uint32_t sup_offset(int s) { return ((uint32_t)s * 210u) & ~3u; }
@@ -426,7 +422,6 @@ struct GQ6K {
 struct GQ5K {
     static constexpr int kRegs = 12;
     static constexpr int kSup = 4;
-    static constexpr int kSupBytes = 176;
     static constexpr int kRawRow = 176;
     static constexpr int kTileStep = 4;
     static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * 176u; }
@@ -485,7 +480,6 @@ struct GLegacy {
     static constexpr int kWords = (kBlock + 3) / 4;        // aligned dwords of one block
     static constexpr int kRegs = kWords + 1;
     static constexpr int kSup = 2;                          // four blocks
-    static constexpr int kSupBytes = 4 * kBlock;
     static constexpr int kRawRow = 112;
     static constexpr int kTileStep = 2;
     static constexpr uint32_t sup_offset(int s) { return (uint32_t)s * (4u * kBlock); }
