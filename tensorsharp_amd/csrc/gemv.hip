@@ -158,7 +158,11 @@ constexpr uint32_t kDeadOffset = 0x80000000u;   // beyond any resource extent us
 //   dword 4j+1 = (x[4j+1], x[4j+3])        low nibbles of bytes 1 and 3
 //   dword 4j+2 = (x[32+4j], x[32+4j+2])    high nibbles
 //   dword 4j+3 = (x[32+4j+1], x[32+4j+3])
+#ifndef TSHIP_GEMV_Q4K_LPR
+#define TSHIP_GEMV_Q4K_LPR 32
+#endif
 struct FmtQ4K {
+    static constexpr int kLPR = TSHIP_GEMV_Q4K_LPR;   // lanes per row: a step covers kLPR consecutive units of 64 / kLPR rows
     static constexpr int kUnitElems = 64;
     static constexpr int kLdsDwords = 36;
     static constexpr int kRegs = 12;
@@ -206,7 +210,7 @@ struct FmtQ4K {
     }
     static __device__ __forceinline__ int stage_items(int K) { return K >> 2; }
 
-    static constexpr int kSlotBytes = 4 * 144;   // 16 consecutive units of a row
+    static constexpr int kSlotBytes = kLPR / 4 * 144;   // kLPR consecutive units of a row
 
     // Lane-invariant part of the addressing: unit g = l16 + 16*step lives in super-block g/4 at
     // quant bytes (g & 3)*32; only the step / row-group part (a scalar) changes from step to step.
@@ -281,6 +285,7 @@ struct FmtQ4K {
 // LDS unit (one 32-weight block, 80 B): 16 dwords (x[j], x[j+16]) as fp16 pairs, then the unit's
 // scale, then 12 B pad.
 struct FmtMXFP4 {
+    static constexpr int kLPR = 16;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 20;
     static constexpr int kRegs = 5;
@@ -387,6 +392,7 @@ struct FmtMXFP4 {
 // ---- Q8_0 ------------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 144 B): 32 fp32 activations, 16 B pad.  fp32 throughout.
 struct FmtQ80 {
+    static constexpr int kLPR = 16;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 36;
     static constexpr int kRegs = 9;
@@ -460,7 +466,29 @@ struct FmtQ80 {
 // ==========================================================================================
 // The kernel body shared by all formats.
 // ==========================================================================================
-// A wavefront works on a group of 4 consecutive rows at a time, one row per 16 lanes.
+// Sum of a value over the LPR lanes of a row (16, 32 or 64 consecutive lanes); every lane of the row gets it.
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v)
+{
+    typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+    float t = v;
+    t += TSHIP_DPP_F(t, kDppXor1);
+    t += TSHIP_DPP_F(t, kDppXor2);
+    t += TSHIP_DPP_F(t, kDppHalfMirror);
+    t += TSHIP_DPP_F(t, kDppMirror);
+    if (LPR >= 32) {     // 16-lane rows (r0 r1 r2 r3) swapped with themselves: (r0 r0 r2 r2) + (r1 r1 r3 r3)
+        const u2_t a = __builtin_amdgcn_permlane16_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+        t = __uint_as_float(a.x) + __uint_as_float(a.y);
+    }
+    if (LPR == 64) {     // halves (lo hi): (lo lo) + (hi hi)
+        const u2_t b = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+        t = __uint_as_float(b.x) + __uint_as_float(b.y);
+    }
+    return t;
+}
+
+// A wavefront works on a group of 64 / LPR consecutive rows at a time, one row per LPR lanes (LPR = 16 unless the
+// format says otherwise).
 // One step = 16 consecutive units of each of the 4 rows.  Steps of a wavefront are numbered
 // group-major over (group, step); kU steps are fetched together, one fetch ahead of the compute.
 template <typename F>
@@ -479,11 +507,12 @@ template <typename F, int ACT, int KS>
 __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, bool strict, uint32_t* lds)
 {
     const int lane = threadIdx.x & 63;
-    const int sub = lane >> 4, l16 = lane & 15;
+    constexpr int LPR = F::kLPR, RPG = 64 / LPR;     // lanes per row, rows per group
+    const int sub = lane / LPR, l16 = lane % LPR;    // row of the group, lane inside the row
     const int N = P.N, K = P.K;
     const int upr = K / F::kUnitElems;          // units per row
-    const int nsteps = (upr + 15) >> 4;         // steps per row group
-    const int ngroups = (N + 3) >> 2;
+    const int nsteps = (upr + LPR - 1) / LPR;   // steps per row group
+    const int ngroups = (N + RPG - 1) / RPG;
     const uint32_t row_bytes = (uint32_t)F::row_bytes(K);
     const int wave_stride = nwg * kWaves;
     const int gw = __builtin_amdgcn_readfirstlane(wg * kWaves + (int)(threadIdx.x >> 6));
@@ -501,10 +530,10 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // issue the loads of step (group, step); no waiting, no branches
     auto fetch = [&](int group, int step, Step<F>& st) {
         const bool group_ok = group < ngroups;                         // uniform
-        const int row0 = group_ok ? group * 4 : 0;
+        const int row0 = group_ok ? group * RPG : 0;
         const uint32_t start = base_delta + (uint32_t)row0 * row_bytes + (uint32_t)step * F::kSlotBytes;
         const uint32_t soff = start & ~3u;                             // scalar part of the address
-        const bool live = group_ok && (row0 + sub < N) && (l16 + (step << 4) < upr);
+        const bool live = group_ok && (row0 + sub < N) && (l16 + step * LPR < upr);
         st.step = step;
         st.group = group;
         st.aux = F::load(rs, L, soff, start & 3u, step, live, st.w);
@@ -562,7 +591,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     };
     // kActRmsNorm: the whole row is in the registers of the workgroup after ONE pass (the host guarantees it);
     // sum of squares in double over the workgroup, then (x * scale) * w in place
-    double* red = reinterpret_cast<double*>(lds + nsteps * 16 * F::kLdsDwords);      // [kWaves], after the x area
+    double* red = reinterpret_cast<double*>(lds + nsteps * LPR * F::kLdsDwords);      // [kWaves], after the x area
     auto apply_act = [&]() {
         if (act == kActRmsNorm) {
             double ss = 0.0;
@@ -658,7 +687,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         stage_commit(base);
     }
     // lanes past the end of a row read their activations from the zero-filled tail of the last step
-    for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nsteps * 16 * F::kLdsDwords; i += kThreads) lds[i] = 0u;
+    for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nsteps * LPR * F::kLdsDwords; i += kThreads) lds[i] = 0u;
     __syncthreads();
 
     if constexpr (KS > 1) {
@@ -668,19 +697,15 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             float acc = 0.f;
             for (int st = s_begin; st < s_end; ++st) {
                 fetch_next(nxt[0]);
-                const uint32_t* xu = lds + lds_lane + (uint32_t)cur[0].step * (16u * F::kLdsDwords);
+                const uint32_t* xu = lds + lds_lane + (uint32_t)cur[0].step * (uint32_t)(LPR * F::kLdsDwords);
                 acc += F::dot(cur[0].w, L, cur[0].aux, xu);
                 cur[0] = nxt[0];
             }
-            float t = acc;
-            t += TSHIP_DPP_F(t, kDppXor1);
-            t += TSHIP_DPP_F(t, kDppXor2);
-            t += TSHIP_DPP_F(t, kDppHalfMirror);
-            t += TSHIP_DPP_F(t, kDppMirror);
+            const float t = row_sum<LPR>(acc);
             float* pr = part + (r & 1) * kWaves * 4;
             if (l16 == 0) pr[wv * 4 + sub] = t;
             __syncthreads();
-            const int group = group_of(r), row = group * 4 + sub;
+            const int group = group_of(r), row = group * RPG + sub;
             if (slice == 0 && l16 == 0 && group < ngroups && row < N) {
                 float sum = 0.f;
 #pragma unroll
@@ -693,15 +718,11 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     float acc = 0.f;
     auto consume = [&](const Step<F>& st) {
         // lanes past the end of a row (and steps past the last group) hold zeros, zero scales included
-        const uint32_t* xu = lds + lds_lane + (uint32_t)st.step * (16u * F::kLdsDwords);
+        const uint32_t* xu = lds + lds_lane + (uint32_t)st.step * (uint32_t)(LPR * F::kLdsDwords);
         acc += F::dot(st.w, L, st.aux, xu);
         if (st.step == nsteps - 1) {   // uniform: the 4 rows of the group are complete
-            float t = acc;
-            t += TSHIP_DPP_F(t, kDppXor1);
-            t += TSHIP_DPP_F(t, kDppXor2);
-            t += TSHIP_DPP_F(t, kDppHalfMirror);
-            t += TSHIP_DPP_F(t, kDppMirror);
-            const int row = st.group * 4 + sub;
+            const float t = row_sum<LPR>(acc);
+            const int row = st.group * RPG + sub;
             if (l16 == 0 && st.group < ngroups && row < N) P.y[row] = P.add ? P.add[row] + t : t;
             acc = 0.f;
         }
@@ -743,11 +764,13 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
+int lanes_per_row(int type) { return type == kTypeQ4_K ? FmtQ4K::kLPR : 16; }
 
 // x staged as whole steps of 16 units (the tail of the last step is zero-filled)
 size_t lds_bytes_for(int type, int K)
 {
-    const size_t units = (size_t)((K / unit_elems(type) + 15) / 16) * 16;
+    const int lpr = lanes_per_row(type);
+    const size_t units = (size_t)((K / unit_elems(type) + lpr - 1) / lpr) * lpr;
     // + the RMSNorm reduction slots + the partial row sums of the K-split scheme
     return units * (type == kTypeMXFP4 ? 80 : 144) + kWaves * sizeof(double) + 2 * kWaves * 4 * sizeof(float);
 }
@@ -770,7 +793,7 @@ int gemv_max_k(int type)
 {
     switch (type) {
     case kTypeQ8_0: return (int)(kMaxLds / 144 / 16) * 16 * 32;
-    case kTypeQ4_K: return (int)(kMaxLds / 144 / 16) * 16 * 64;
+    case kTypeQ4_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
     case kTypeMXFP4: return (int)(kMaxLds / 80 / 16) * 16 * 32;
     default: return 0;
     }
@@ -809,15 +832,16 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     int per_cu = (int)std::min<size_t>(TSHIP_GEMV_WG_PER_CU, (160 * 1024) / (lds + 256));
     if (per_cu < 1) per_cu = 1;
     const int budget = di.num_cus * per_cu;
-    // A single matrix with so few rows that one row group per wavefront would keep less than half of the wavefronts
-    // busy, and rows long enough to cut: four wavefronts share a row group, each taking a quarter of its steps.
-    // Only with plain activations: four times as many workgroups stage x, and measured with the SiLU / RMSNorm
-    // staging modes that costs more than the extra wavefronts win (4096 x 14336 Q4_K: plain 14.7 -> 12.6 us,
+    // A single matrix with so few rows that one row group per wavefront would keep at most half of the wavefronts
+    // busy, and rows long enough to cut: two or four wavefronts share a row group, each taking a slice of at least two
+    // of its steps.  Only with plain activations: that many more workgroups stage x, and measured with the SiLU /
+    // RMSNorm staging modes that costs more than the extra wavefronts win (4096 x 14336 Q4_K: plain 14.7 -> 12.6 us,
     // SiLU mode inside the fused FFN 32.7 -> 34.3 us).
+    const int lpr = lanes_per_row(type), rpg = 64 / lpr;
     int ksplit = 1;
     if (count == 1 && args[0].act == kActPlain) {
-        const int ngroups = (args[0].N + 3) / 4, nsteps = (args[0].K / unit_elems(type) + 15) / 16;
-        if (ngroups * 2 <= budget * kWaves && nsteps >= 8) ksplit = 4;
+        const int ngroups = (args[0].N + rpg - 1) / rpg, nsteps = (args[0].K / unit_elems(type) + lpr - 1) / lpr;
+        while (ksplit < 4 && ngroups * ksplit * 2 <= budget * kWaves && nsteps / (ksplit * 2) >= 2) ksplit *= 2;
     }
 
     GemvGroup g;
@@ -828,7 +852,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     for (int i = 0; i < count; ++i) {
         // workgroups in proportion to the bytes each problem streams
         int share = std::max(1, (int)((double)budget * (double)args[i].w_bytes / total_bytes + 0.5));
-        share = std::min(share, ((args[i].N + 3) / 4 + kWaves / ksplit - 1) / (kWaves / ksplit));
+        share = std::min(share, ((args[i].N + rpg - 1) / rpg + kWaves / ksplit - 1) / (kWaves / ksplit));
         g.p[i].w = static_cast<const uint8_t*>(args[i].w);
         g.p[i].w_bytes = args[i].w_bytes;
         g.p[i].x = args[i].x;
@@ -862,6 +886,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     }
 #define TSHIP_GEMV_DISPATCH(T)                                                           \
     (ksplit == 4          ? launch_type<T, kActPlain, 4>(g, begin, lds, stream)          \
+     : ksplit == 2        ? launch_type<T, kActPlain, 2>(g, begin, lds, stream)          \
      : act == kActPlain   ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
      : act == kActRmsNorm ? launch_type<T, kActRmsNorm>(g, begin, lds, stream)           \
      : act == kActSiluMul ? launch_type<T, kActSiluMul>(g, begin, lds, stream)           \
