@@ -284,8 +284,11 @@ struct FmtQ4K {
 // ---- MXFP4 -----------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 80 B): 16 dwords (x[j], x[j+16]) as fp16 pairs, then the unit's
 // scale, then 12 B pad.
+#ifndef TSHIP_GEMV_MXFP4_LPR
+#define TSHIP_GEMV_MXFP4_LPR 16
+#endif
 struct FmtMXFP4 {
-    static constexpr int kLPR = 16;
+    static constexpr int kLPR = TSHIP_GEMV_MXFP4_LPR;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 20;
     static constexpr int kRegs = 5;
@@ -325,7 +328,7 @@ struct FmtMXFP4 {
     }
     static __device__ __forceinline__ int stage_items(int K) { return K >> 3; }
 
-    static constexpr int kSlotBytes = 16 * 17;
+    static constexpr int kSlotBytes = kLPR * 17;
 
     struct Lane {
         uint32_t voff;   // byte offset of the lane's block: row inside the group + inside the step (before alignment)
@@ -391,8 +394,11 @@ struct FmtMXFP4 {
 
 // ---- Q8_0 ------------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 144 B): 32 fp32 activations, 16 B pad.  fp32 throughout.
+#ifndef TSHIP_GEMV_Q80_LPR
+#define TSHIP_GEMV_Q80_LPR 16
+#endif
 struct FmtQ80 {
-    static constexpr int kLPR = 16;
+    static constexpr int kLPR = TSHIP_GEMV_Q80_LPR;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 36;
     static constexpr int kRegs = 9;
@@ -409,7 +415,7 @@ struct FmtQ80 {
     }
     static __device__ __forceinline__ int stage_items(int K) { return K >> 2; }
 
-    static constexpr int kSlotBytes = 16 * 34;
+    static constexpr int kSlotBytes = kLPR * 34;
 
     struct Lane {
         uint32_t voff;
@@ -764,7 +770,7 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
-int lanes_per_row(int type) { return type == kTypeQ4_K ? FmtQ4K::kLPR : 16; }
+int lanes_per_row(int type) { return type == kTypeQ4_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : FmtQ80::kLPR; }
 
 // x staged as whole steps of 16 units (the tail of the last step is zero-filled)
 size_t lds_bytes_for(int type, int K)
@@ -792,9 +798,9 @@ bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 int gemv_max_k(int type)
 {
     switch (type) {
-    case kTypeQ8_0: return (int)(kMaxLds / 144 / 16) * 16 * 32;
+    case kTypeQ8_0: return (int)(kMaxLds / 144 / FmtQ80::kLPR) * FmtQ80::kLPR * 32;
     case kTypeQ4_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
-    case kTypeMXFP4: return (int)(kMaxLds / 80 / 16) * 16 * 32;
+    case kTypeMXFP4: return (int)(kMaxLds / 80 / FmtMXFP4::kLPR) * FmtMXFP4::kLPR * 32;
     default: return 0;
     }
 }
