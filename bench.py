@@ -206,12 +206,12 @@ def main():
             extra[f"cfg2_q4_k_gemv_{name}_{n}x{k}"] = one_matrix(Q4_K, n, k, max(2, int(300e6 // (n * row_bytes(Q4_K, k))) + 1))
         extra["cfg4_mxfp4_gemv_gate_up_5760x2880"] = one_matrix(MXFP4, 5760, 2880, 32)
         extra["cfg4_mxfp4_gemv_down_2880x2880"] = one_matrix(MXFP4, 2880, 2880, 64)
-        # output projection of a 128k-vocabulary model (the largest single GEMV of a decode step): Q8_0 through the
-        # GEMV kernel, Q6_K (what Q4_K_M files store it in) through the register-resident matrix-core kernel
+        # output projection of a 128k-vocabulary model (the largest single GEMV of a decode step): Q8_0, and Q6_K (what
+        # Q4_K_M files store it in)
         n_it_save, n_it = n_it, 50
         extra["lm_head_q8_0_gemv_128256x4096"] = one_matrix(Q8_0, 128256, 4096, 2)
-        extra["lm_head_q6_k_128256x4096"] = one_matrix(Q6_K, 128256, 4096, 2)
-        extra["q6_k_ffn_down_4096x14336"] = one_matrix(Q6_K, 4096, 14336, 8)
+        extra["lm_head_q6_k_gemv_128256x4096"] = one_matrix(Q6_K, 128256, 4096, 2)
+        extra["q6_k_gemv_down_4096x14336"] = one_matrix(Q6_K, 4096, 14336, 8)
         n_it = n_it_save
 
         # prefill GEMMs (configs[2] and configs[4]): TFLOP/s = 2*M*N*K / time of the whole call

@@ -469,6 +469,145 @@ struct FmtQ80 {
     }
 };
 
+// ---- Q6_K ------------------------------------------------------------------------------------
+// Block of 256 weights, 210 bytes: ql[128] low nibbles, qh[64] 2-bit tops, 16 int8 scales (one per 16 weights), fp16 d
+// (ggml-quants.c dequantize_row_q6_K; ManagedQuantizedOps.cs:481-520).  Unit = 64 weights (n = half of the block,
+// j = which 16 of its 32 columns): weights 128 n + 16 j + t + 32 r for t = 0..15 and run r = 0..3, held in
+//   piece A = ql[64 n + 16 j + t]        low nibble -> run 0, high nibble -> run 2
+//   piece B = ql[64 n + 32 + 16 j + t]   low nibble -> run 1, high nibble -> run 3
+//   piece H = qh[32 n + 16 j + t]        bits 2r .. 2r+1 -> run r
+// and scale[8 n + j + 2 r] for run r.  Blocks are 2-byte aligned, so each 16-byte piece is fetched as a 20-byte
+// dword-aligned window and re-aligned in registers.
+// LDS unit (176 B): for quant dword i of piece A, dwords 4i .. 4i+3 = (x[t], x[t+2]), (x[t+1], x[t+3]) of run 0, then
+// the same of run 2 (t = 4 i); piece B (runs 1, 3) in dwords 16 .. 31; then the four runs' sums of the scaled fp16
+// activations, then the four runs' power-of-two scales, 16 B pad (a 44-dword stride keeps ds_read_b128 conflict-free).
+// A 6-bit value left in the low bits of an fp16 is the subnormal v * 2^-24, exact in v_dot2_f32_f16.
+#ifndef TSHIP_GEMV_Q6K_LPR
+#define TSHIP_GEMV_Q6K_LPR 32
+#endif
+struct FmtQ6K {
+    static constexpr int kLPR = TSHIP_GEMV_Q6K_LPR;
+    static constexpr int kUnitElems = 64;
+    static constexpr int kLdsDwords = 44;
+    static constexpr int kRegs = 19;
+
+    static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 8) * 210; }
+
+    static constexpr int kStageF4 = 1;
+    static __device__ __forceinline__ void stage_offsets(int it, uint32_t (&off)[kStageF4]) { off[0] = (uint32_t)it * 16u; }
+
+    // one work item = 4 consecutive activations of one run; the 4 lanes of a quad share the run
+    static __device__ __forceinline__ void stage_store(const float4 (&vv)[kStageF4], int it, bool live, uint32_t* lds)
+    {
+        const float4 v = vv[0];
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
+        float inv, scale;
+        pow2_scale(amax, &inv, &scale);
+        const _Float16 h0 = (_Float16)(v.x * inv), h1 = (_Float16)(v.y * inv);
+        const _Float16 h2 = (_Float16)(v.z * inv), h3 = (_Float16)(v.w * inv);
+        float s = ((float)h0 + (float)h1) + ((float)h2 + (float)h3);
+        s += TSHIP_DPP_F(s, kDppXor1);
+        s += TSHIP_DPP_F(s, kDppXor2);
+        if (live) {
+            const int e = it << 2;
+            const int b = e >> 8, n = (e >> 7) & 1, r = (e >> 5) & 3, j = (e >> 4) & 1, i = (e >> 2) & 3;
+            uint32_t* unit = lds + ((b * 2 + n) * 2 + j) * kLdsDwords;
+            H2U lo, hi;
+            lo.h = half2_t{h0, h2};
+            hi.h = half2_t{h1, h3};
+            uint2 w2;
+            w2.x = lo.u;
+            w2.y = hi.u;
+            *reinterpret_cast<uint2*>(unit + (r & 1) * 16 + i * 4 + (r >> 1) * 2) = w2;
+            if ((threadIdx.x & 3) == 0) {
+                reinterpret_cast<float*>(unit)[32 + r] = s;
+                reinterpret_cast<float*>(unit)[36 + r] = scale;
+            }
+        }
+    }
+    static __device__ __forceinline__ int stage_items(int K) { return K >> 2; }
+
+    static constexpr int kSlotBytes = kLPR / 4 * 210;
+
+    struct Lane {
+        uint32_t voff;    // the lane's block: its row inside the group + inside the step
+        uint32_t off_a;   // piece A inside the block (piece B is 32 bytes on)
+        uint32_t off_h;   // piece H
+        uint32_t off_s;   // the 8 scales of the lane's half
+        int sc_shift;     // bit position of the scales of runs 0 and 2 inside their dwords (runs 1 and 3: 16 bits on)
+    };
+    static __device__ __forceinline__ Lane lane_setup(int sub, int l16, uint32_t row_bytes)
+    {
+        const uint32_t n = (uint32_t)(l16 >> 1) & 1u, j = (uint32_t)l16 & 1u;
+        Lane L;
+        L.voff = (uint32_t)sub * row_bytes + (uint32_t)(l16 >> 2) * 210u;
+        L.off_a = 64u * n + 16u * j;
+        L.off_h = 128u + 32u * n + 16u * j;
+        L.off_s = 192u + 8u * n;
+        L.sc_shift = (int)j * 8;
+        return L;
+    }
+
+    // Every piece offset is a multiple of 4, so all windows share the block's byte position p & 3 (0 or 2), returned.
+    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t rs, const Lane& L, uint32_t soff,
+                                                    uint32_t row_delta, int /*slot*/, bool live, uint32_t (&w)[kRegs])
+    {
+        const uint32_t p = L.voff + row_delta;
+        const uint32_t al = live ? (p & ~3u) : kDeadOffset;
+        buf_load4(rs, al + L.off_a, soff, &w[0]);
+        w[4] = buf_load1(rs, al + L.off_a + 16u, soff);
+        buf_load4(rs, al + L.off_a + 32u, soff, &w[5]);
+        w[9] = buf_load1(rs, al + L.off_a + 48u, soff);
+        buf_load4(rs, al + L.off_h, soff, &w[10]);
+        w[14] = buf_load1(rs, al + L.off_h + 16u, soff);
+        w[15] = buf_load1(rs, al + L.off_s, soff);
+        w[16] = buf_load1(rs, al + L.off_s + 4u, soff);
+        w[17] = buf_load1(rs, al + L.off_s + 8u, soff);
+        w[18] = buf_load1(rs, al + 208u, soff);
+        return p & 3u;
+    }
+
+    static __device__ __forceinline__ float dot(const uint32_t (&w)[kRegs], const Lane& L, uint32_t o, const uint32_t* xu_dw)
+    {
+        const bool odd = (o & 2u) != 0;       // the block starts at byte 2 of its aligned window
+        const uint4* xu = reinterpret_cast<const uint4*>(xu_dw);
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        constexpr uint32_t kNib = 0x000f000fu, kTop = 0x00300030u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t qa = odd ? __builtin_amdgcn_alignbyte(w[i + 1], w[i], 2) : w[i];
+            const uint32_t qb = odd ? __builtin_amdgcn_alignbyte(w[i + 6], w[i + 5], 2) : w[i + 5];
+            const uint32_t h = odd ? __builtin_amdgcn_alignbyte(w[i + 11], w[i + 10], 2) : w[i + 10];
+            const uint4 xa = xu[i], xb = xu[4 + i];
+            a0 = dot2((qa & kNib) | ((h << 4) & kTop), xa.x, a0);
+            a0 = dot2(((qa >> 8) & kNib) | ((h >> 4) & kTop), xa.y, a0);
+            a2 = dot2(((qa >> 4) & kNib) | (h & kTop), xa.z, a2);
+            a2 = dot2(((qa >> 12) & kNib) | ((h >> 8) & kTop), xa.w, a2);
+            a1 = dot2((qb & kNib) | ((h << 2) & kTop), xb.x, a1);
+            a1 = dot2(((qb >> 8) & kNib) | ((h >> 6) & kTop), xb.y, a1);
+            a3 = dot2(((qb >> 4) & kNib) | ((h >> 2) & kTop), xb.z, a3);
+            a3 = dot2(((qb >> 12) & kNib) | ((h >> 10) & kTop), xb.w, a3);
+        }
+        // the half's 8 scale bytes: runs 0, 1 in bytes j, j + 2 of the first dword, runs 2, 3 of the second
+        const uint32_t s01 = odd ? __builtin_amdgcn_alignbyte(w[16], w[15], 2) : w[15];
+        const uint32_t s23 = odd ? __builtin_amdgcn_alignbyte(w[17], w[16], 2) : w[16];
+        const float sc0 = (float)(int8_t)(s01 >> L.sc_shift), sc1 = (float)(int8_t)(s01 >> (L.sc_shift + 16));
+        const float sc2 = (float)(int8_t)(s23 >> L.sc_shift), sc3 = (float)(int8_t)(s23 >> (L.sc_shift + 16));
+        H2U dh;
+        dh.u = odd ? (w[18] >> 16) : (w[18] & 0xffffu);
+        const float d = (float)dh.h.x;
+        const uint4 sums = xu[8], scl = xu[9];
+        // a_r carries v * 2^-24; the stored value is v - 32
+        const float t0 = (a0 * 16777216.f - 32.f * __uint_as_float(sums.x)) * __uint_as_float(scl.x);
+        const float t1 = (a1 * 16777216.f - 32.f * __uint_as_float(sums.y)) * __uint_as_float(scl.y);
+        const float t2 = (a2 * 16777216.f - 32.f * __uint_as_float(sums.z)) * __uint_as_float(scl.z);
+        const float t3 = (a3 * 16777216.f - 32.f * __uint_as_float(sums.w)) * __uint_as_float(scl.w);
+        return d * ((sc0 * t0 + sc1 * t1) + (sc2 * t2 + sc3 * t3));
+    }
+};
+
 // ==========================================================================================
 // The kernel body shared by all formats.
 // ==========================================================================================
@@ -766,11 +905,16 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
     const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
     if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
+    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
 }
 
-int unit_elems(int type) { return type == kTypeQ4_K ? 64 : 32; }
-int lanes_per_row(int type) { return type == kTypeQ4_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : FmtQ80::kLPR; }
+int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ6_K ? 64 : 32; }
+int unit_lds_bytes(int type) { return type == kTypeMXFP4 ? 80 : type == kTypeQ6_K ? 176 : 144; }
+int lanes_per_row(int type)
+{
+    return type == kTypeQ4_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : type == kTypeQ6_K ? FmtQ6K::kLPR : FmtQ80::kLPR;
+}
 
 // x staged as whole steps of 16 units (the tail of the last step is zero-filled)
 size_t lds_bytes_for(int type, int K)
@@ -778,7 +922,7 @@ size_t lds_bytes_for(int type, int K)
     const int lpr = lanes_per_row(type);
     const size_t units = (size_t)((K / unit_elems(type) + lpr - 1) / lpr) * lpr;
     // + the RMSNorm reduction slots + the partial row sums of the K-split scheme
-    return units * (type == kTypeMXFP4 ? 80 : 144) + kWaves * sizeof(double) + 2 * kWaves * 4 * sizeof(float);
+    return units * unit_lds_bytes(type) + kWaves * sizeof(double) + 2 * kWaves * 4 * sizeof(float);
 }
 
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
@@ -801,6 +945,7 @@ int gemv_max_k(int type)
     case kTypeQ8_0: return (int)(kMaxLds / 144 / FmtQ80::kLPR) * FmtQ80::kLPR * 32;
     case kTypeQ4_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
     case kTypeMXFP4: return (int)(kMaxLds / 80 / FmtMXFP4::kLPR) * FmtMXFP4::kLPR * 32;
+    case kTypeQ6_K: return (int)(kMaxLds / 176 / FmtQ6K::kLPR) * FmtQ6K::kLPR * 64;
     default: return 0;
     }
 }
@@ -816,7 +961,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         set_last_error("gemv: group size out of range.");
         return false;
     }
-    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4) {
+    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K) {
         set_last_error("gemv: unsupported type.");
         return false;
     }
@@ -900,6 +1045,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     switch (type) {
     case kTypeQ4_K: return TSHIP_GEMV_DISPATCH(kTypeQ4_K);
     case kTypeMXFP4: return TSHIP_GEMV_DISPATCH(kTypeMXFP4);
+    case kTypeQ6_K: return TSHIP_GEMV_DISPATCH(kTypeQ6_K);
     default: return TSHIP_GEMV_DISPATCH(kTypeQ8_0);
     }
 #undef TSHIP_GEMV_DISPATCH

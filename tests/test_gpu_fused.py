@@ -151,7 +151,7 @@ def test_rms_norm_matmul_row_longer_than_one_staging_pass(hip, oracle, name):
 
 @pytest.mark.parametrize("M", [1, 40])
 def test_ffn_swiglu_q4_k_gate_up_q6_k_down(hip, oracle, M):
-    # the mix of a Q4_K_M file: gate/up in Q4_K, down in Q6_K (no GEMV specialisation: matrix-core path at M = 1 too)
+    # the mix of a Q4_K_M file: gate/up in Q4_K, down in Q6_K (its GEMV at M = 1 with silu(gate) * up formed in the staging)
     import torch
     from oracle.oracle import Q6_K
     from tensorsharp_amd import QuantizedWeight, synth

@@ -231,3 +231,68 @@ def test_few_rows_long_k_split_over_wavefronts(hip, oracle, name, N, K):
     torch.cuda.synchronize()
     got = r.cpu().numpy().astype(np.float64) - resid
     assert np.max(np.abs(got - ref)) <= 1e-3 * np.linalg.norm(ref) + 1e-6 * np.max(np.abs(resid)), name
+
+
+# ---- Q6_K (output matrix and some projections of Q4_K_M files): 210-byte blocks, 2-byte aligned ----
+def q6k_weight(N, K, seed, std=0.02):
+    import torch
+    from tensorsharp_amd import synth
+    g = torch.Generator().manual_seed(seed)
+    return synth.quantize_q6_k_simple(torch.randn((N, K), generator=g) * std).numpy()
+
+
+@pytest.mark.parametrize("N,K", [(1, 256), (3, 512), (7, 1024), (130, 2560), (257, 4096), (1001, 2816), (4096, 14336), (6, 8192)])
+def test_q6_k_shapes(hip, oracle, N, K):
+    from oracle.oracle import Q6_K
+    wq = q6k_weight(N, K, N * 31 + K)
+    rng = np.random.default_rng(N + K)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    ref = oracle.matmul_f64(Q6_K, wq, N, K, x)
+    check("q4_k", run_device(hip, Q6_K, wq, N, K, x), ref)
+    for s in (1e-20, 3e4):
+        xs = (x * np.float32(s)).astype(np.float32)
+        check("q4_k", run_device(hip, Q6_K, wq, N, K, xs), oracle.matmul_f64(Q6_K, wq, N, K, xs))
+    assert np.all(run_device(hip, Q6_K, wq, N, K, np.zeros((1, K), np.float32)) == 0)
+
+
+def test_q6_k_extreme_quants_and_scales(hip, oracle):
+    # every 6-bit value and both signs of the int8 scales, in random order
+    from oracle.oracle import Q6_K
+    rng = np.random.default_rng(77)
+    N, K = 64, 1024
+    nb = N * K // 256
+    raw = rng.integers(0, 256, size=(nb, 210), dtype=np.uint8)
+    raw[:, 208:210] = rng.uniform(1e-4, 4e-4, nb).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    raw[0, 192:208] = np.array([-128, 127, -1, 1, 0, 64, -64, 5] * 2, dtype=np.int8).view(np.uint8)
+    wq = raw.reshape(-1)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    check("q4_k", run_device(hip, Q6_K, wq, N, K, x), oracle.matmul_f64(Q6_K, wq, N, K, x))
+
+
+def test_q6_k_views_two_bytes_off_and_grouped(hip, oracle):
+    # a weight that starts one row into an allocation (105 blocks per row: rows alternate between byte 0 and byte 2 of
+    # a dword), alone and as members of a grouped launch
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    from oracle.oracle import Q6_K
+    N, K = 48, 256 * 5
+    wq = q6k_weight(N + 3, K, 5)
+    rb = (K // 256) * 210
+    dev = torch.from_numpy(wq).cuda()
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    ws, ys, refs = [], [], []
+    for skip in (1, 2, 3):
+        view = dev[skip * rb:(skip + N) * rb]
+        refs.append(oracle.matmul_f64(Q6_K, wq[skip * rb:(skip + N) * rb], N, K, x))
+        ws.append(QuantizedWeight(view, Q6_K, K, N))
+        y = hip.LinearForward(xd, ws[-1])
+        torch.cuda.synchronize()
+        check("q4_k", y.cpu().numpy(), refs[-1])
+        ys.append(torch.full((1, N), float("nan"), device="cuda"))
+    hip.UseCurrentStream()
+    hip.AddmmQuantGroupDevice(hip.PrepareGroup(ys, [xd] * 3, ws))
+    torch.cuda.synchronize()
+    for y, ref in zip(ys, refs):
+        check("q4_k", y.cpu().numpy(), ref)

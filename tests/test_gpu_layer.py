@@ -93,7 +93,7 @@ def test_first_token_and_the_reference_graph_known_answer(hip, oracle):
 
 
 def test_model_decode_equals_layers_in_sequence_and_mixed_formats(hip, oracle):
-    # two layers through the model entry point; down projections in Q6_K (no GEMV kernel: matrix-core path inside the layer)
+    # two layers through the model entry point; down projections in Q6_K
     import torch
     from tensorsharp_amd import QuantizedWeight, synth
     rng = np.random.default_rng(107)
