@@ -20,7 +20,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-Q8_0, Q4_K, Q6_K, MXFP4 = 8, 12, 14, 39
+Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 8, 12, 13, 14, 39
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the grouped Q4_K GEMV from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the
 # reading of a 1 GiB copy (profiles/gemv_q4k_layer_hbm_traffic.txt); not measured by this script.
@@ -33,7 +33,7 @@ LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
 
 
 def row_bytes(t, k):
-    return {Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), Q6_K: 210 * (k // 256), MXFP4: 17 * (k // 32)}[t]
+    return {Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), Q5_K: 176 * (k // 256), Q6_K: 210 * (k // 256), MXFP4: 17 * (k // 32)}[t]
 
 
 def algorithmic_bytes(t, n, k, m=1):

@@ -281,6 +281,79 @@ struct FmtQ4K {
     }
 };
 
+// ---- Q5_K ------------------------------------------------------------------------------------
+// Q4_K with a fifth bit: block of 176 bytes = d, dmin, 12 scale bytes, qh[32], qs[128] (ggml-quants.c
+// dequantize_row_q5_K; ManagedQuantizedOps.cs:521-577).  Unit u = 64-weight group: its 32 quant bytes, and of every
+// qh byte l the bits 2u (weight 64u + l) and 2u + 1 (weight 64u + 32 + l).  x in LDS, scales and mins: as FmtQ4K.
+struct FmtQ5K : FmtQ4K {
+    static constexpr int kRegs = 20;
+
+    static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 8) * 176; }
+    static constexpr int kSlotBytes = kLPR / 4 * 176;
+
+    struct Lane {
+        uint32_t voff;    // the lane's super-block
+        uint32_t qoff;    // its 32 quant bytes inside the super-block
+        int sh;           // bit position of the lane's scale pair inside the packed scale dwords
+        bool upper;       // sub-blocks 4..7 use the split 4+2 bit encoding
+        int hsh;          // bit position of the group's pair of fifth bits inside a qh byte
+    };
+    static __device__ __forceinline__ Lane lane_setup(int sub, int l16, uint32_t row_bytes)
+    {
+        Lane L;
+        L.voff = (uint32_t)sub * row_bytes + (uint32_t)(l16 >> 2) * 176u;
+        L.qoff = 48u + (uint32_t)(l16 & 3) * 32u;
+        L.sh = (l16 & 1) * 16;
+        L.upper = (l16 & 2) != 0;
+        L.hsh = (l16 & 3) * 2;
+        return L;
+    }
+
+    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t rs, const Lane& L, uint32_t soff,
+                                                    uint32_t /*row_delta*/, int /*slot*/, bool live, uint32_t (&w)[kRegs])
+    {
+        const uint32_t hdr = live ? L.voff : kDeadOffset;
+        const uint32_t q = hdr + L.qoff;
+        buf_load4(rs, hdr, soff, &w[0]);
+        buf_load4(rs, hdr + 16, soff, &w[4]);      // qh, shared by the four groups of the super-block
+        buf_load4(rs, hdr + 32, soff, &w[8]);
+        buf_load4(rs, q, soff, &w[12]);
+        buf_load4(rs, q + 16, soff, &w[16]);
+        return 0;
+    }
+
+    static __device__ __forceinline__ float dot(const uint32_t (&w)[kRegs], const Lane& L, uint32_t /*aux*/,
+                                                const uint32_t* xu_dw)
+    {
+        const uint4* xu = reinterpret_cast<const uint4*>(xu_dw);
+        float lo = 0.f, hi = 0.f;
+        constexpr uint32_t kNib = 0x000f000fu, kFifth = 0x00100010u;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint4 xv = xu[j];
+            const uint32_t q = w[12 + j];
+            const uint32_t h = w[4 + j] >> L.hsh;      // bit 0 of every byte: low-nibble weight, bit 1: high-nibble weight
+            // a 5-bit value left in the low bits of an fp16 is the subnormal v * 2^-24
+            lo = dot2((q & kNib) | ((h << 4) & kFifth), xv.x, lo);
+            lo = dot2(((q >> 8) & kNib) | ((h >> 4) & kFifth), xv.y, lo);
+            hi = dot2(((q >> 4) & kNib) | ((h << 3) & kFifth), xv.z, hi);
+            hi = dot2(((q >> 12) & kNib) | ((h >> 5) & kFifth), xv.w, hi);
+        }
+        const uint4 tail = xu[8];
+        const float s1 = __uint_as_float(tail.x), s2 = __uint_as_float(tail.y), xscale = __uint_as_float(tail.z);
+        const uint32_t a = w[1] >> L.sh, b = w[2] >> L.sh, c = w[3] >> L.sh;
+        const uint32_t sc_lo = a & 0x3f3fu, m_lo = b & 0x3f3fu;
+        const uint32_t sc_hi = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+        const uint32_t m_hi = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+        const uint32_t sc = L.upper ? sc_hi : sc_lo, mn = L.upper ? m_hi : m_lo;
+        const float sc1 = (float)(sc & 0xffu), sc2 = (float)(sc >> 8);
+        const float m1 = (float)(mn & 0xffu), m2 = (float)(mn >> 8);
+        const half2_t dm = as_half2(w[0]);
+        const float d = (float)dm.x, dmin = (float)dm.y;
+        return (d * ((sc1 * lo + sc2 * hi) * 16777216.f) - dmin * (m1 * s1 + m2 * s2)) * xscale;
+    }
+};
+
 // ---- MXFP4 -----------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 80 B): 16 dwords (x[j], x[j+16]) as fp16 pairs, then the unit's
 // scale, then 12 B pad.
@@ -906,14 +979,15 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
     if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
+    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
 }
 
-int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ6_K ? 64 : 32; }
+int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
 int unit_lds_bytes(int type) { return type == kTypeMXFP4 ? 80 : type == kTypeQ6_K ? 176 : 144; }
 int lanes_per_row(int type)
 {
-    return type == kTypeQ4_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : type == kTypeQ6_K ? FmtQ6K::kLPR : FmtQ80::kLPR;
+    return type == kTypeQ4_K || type == kTypeQ5_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : type == kTypeQ6_K ? FmtQ6K::kLPR : FmtQ80::kLPR;
 }
 
 // x staged as whole steps of 16 units (the tail of the last step is zero-filled)
@@ -946,6 +1020,7 @@ int gemv_max_k(int type)
     case kTypeQ4_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
     case kTypeMXFP4: return (int)(kMaxLds / 80 / FmtMXFP4::kLPR) * FmtMXFP4::kLPR * 32;
     case kTypeQ6_K: return (int)(kMaxLds / 176 / FmtQ6K::kLPR) * FmtQ6K::kLPR * 64;
+    case kTypeQ5_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
     default: return 0;
     }
 }
@@ -961,7 +1036,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         set_last_error("gemv: group size out of range.");
         return false;
     }
-    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K) {
+    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K && type != kTypeQ5_K) {
         set_last_error("gemv: unsupported type.");
         return false;
     }
@@ -1046,6 +1121,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     case kTypeQ4_K: return TSHIP_GEMV_DISPATCH(kTypeQ4_K);
     case kTypeMXFP4: return TSHIP_GEMV_DISPATCH(kTypeMXFP4);
     case kTypeQ6_K: return TSHIP_GEMV_DISPATCH(kTypeQ6_K);
+    case kTypeQ5_K: return TSHIP_GEMV_DISPATCH(kTypeQ5_K);
     default: return TSHIP_GEMV_DISPATCH(kTypeQ8_0);
     }
 #undef TSHIP_GEMV_DISPATCH

@@ -98,7 +98,43 @@ def quantize_q6_k_simple(w):
     return out.reshape(-1)
 
 
-QUANTIZERS = {8: quantize_q8_0, 12: quantize_q4_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
+def quantize_q5_k_simple(w):
+    """Valid Q5_K blocks (ggml-common.h block_q5_K): the per-sub-block affine fit of quantize_q4_k_simple with 31 levels
+    instead of 15 (the fifth bits go to qh), for synthetic weights."""
+    x = w.reshape(-1, 8, 32).float()
+    lo = x.amin(dim=2).clamp_max(0.0)
+    hi = x.amax(dim=2)
+    scale = (hi - lo) / 31.0
+    mn = -lo
+    d = scale.amax(dim=1) / 63.0
+    dmin = mn.amax(dim=1) / 63.0
+    d16 = d.to(torch.float16).float()
+    dmin16 = dmin.to(torch.float16).float()
+    ls = torch.where(d16[:, None] > 0, torch.round(scale / d16[:, None].clamp_min(1e-30)), torch.zeros_like(scale)).clamp(0, 63)
+    lm = torch.where(dmin16[:, None] > 0, torch.round(mn / dmin16[:, None].clamp_min(1e-30)), torch.zeros_like(mn)).clamp(0, 63)
+    eff_d = d16[:, None] * ls
+    eff_m = dmin16[:, None] * lm
+    q = torch.where(eff_d[:, :, None] > 0, torch.round((x + eff_m[:, :, None]) / eff_d[:, :, None].clamp_min(1e-30)),
+                    torch.zeros_like(x)).clamp(0, 31).to(torch.uint8)
+    ls = ls.to(torch.uint8)
+    lm = lm.to(torch.uint8)
+    nb = x.shape[0]
+    out = torch.zeros((nb, 176), dtype=torch.uint8, device=w.device)
+    out[:, 0:2] = _half_bytes(d)
+    out[:, 2:4] = _half_bytes(dmin)
+    sc = out[:, 4:16]
+    sc[:, 0:4] = ls[:, 0:4] | ((ls[:, 4:8] >> 4) << 6)
+    sc[:, 4:8] = lm[:, 0:4] | ((lm[:, 4:8] >> 4) << 6)
+    sc[:, 8:12] = (ls[:, 4:8] & 0x0F) | ((lm[:, 4:8] & 0x0F) << 4)
+    qq = q.reshape(nb, 4, 2, 32)                         # [block, 64-weight group, low / high nibble half, 32]
+    qh = out[:, 16:48]
+    for u in range(4):
+        qh |= ((qq[:, u, 0, :] >> 4) << (2 * u)) | ((qq[:, u, 1, :] >> 4) << (2 * u + 1))
+    out[:, 48:] = ((qq[:, :, 0, :] & 15) | ((qq[:, :, 1, :] & 15) << 4)).reshape(nb, 128)
+    return out.reshape(-1)
+
+
+QUANTIZERS = {8: quantize_q8_0, 12: quantize_q4_k_simple, 13: quantize_q5_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
 
 
 def random_weight(ggml_type, n_rows, n_cols, device, seed, sigma=0.02, chunk_rows=4096):

@@ -296,3 +296,16 @@ def test_q6_k_views_two_bytes_off_and_grouped(hip, oracle):
     torch.cuda.synchronize()
     for y, ref in zip(ys, refs):
         check("q4_k", y.cpu().numpy(), ref)
+
+
+# ---- Q5_K: Q4_K with a fifth bit per weight (176-byte blocks) ----
+@pytest.mark.parametrize("N,K", [(1, 256), (5, 768), (130, 2560), (257, 4096), (4096, 14336), (6, 8192)])
+def test_q5_k_shapes(hip, oracle, N, K):
+    from oracle.oracle import Q5_K
+    rng = np.random.default_rng(N * 13 + K)
+    wq = inputs.random_blocks("q5_k", N, K, rng)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    check("q4_k", run_device(hip, Q5_K, wq, N, K, x), oracle.matmul_f64(Q5_K, wq, N, K, x))
+    xs = (x * np.float32(1e-20)).astype(np.float32)
+    check("q4_k", run_device(hip, Q5_K, wq, N, K, xs), oracle.matmul_f64(Q5_K, wq, N, K, xs))
+    assert np.all(run_device(hip, Q5_K, wq, N, K, np.zeros((1, K), np.float32)) == 0)

@@ -23,3 +23,15 @@ def test_q4_k_generator_makes_valid_blocks(oracle):
     deq = oracle.dequantize(Q4_K, raw)
     rms = float(np.sqrt(np.mean((deq - w.numpy().reshape(-1)) ** 2))) / 0.02
     assert rms < 0.12          # the reference's search reaches 0.071; a plain min/max fit stays close
+
+
+def test_q5_k_and_q6_k_generators_make_valid_blocks(oracle):
+    from oracle.oracle import Q5_K, Q6_K
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn((16, 1024), generator=g) * 0.02
+    for t, fn, size, bound in ((Q5_K, synth.quantize_q5_k_simple, 176, 0.06), (Q6_K, synth.quantize_q6_k_simple, 210, 0.04)):
+        raw = fn(w).numpy()
+        assert raw.size == 16 * 4 * size
+        deq = oracle.dequantize(t, raw)
+        rms = float(np.sqrt(np.mean((deq - w.numpy().reshape(-1)) ** 2))) / 0.02
+        assert rms < bound, (t, rms)
