@@ -7,7 +7,7 @@
 //                        cache [kv_head][max_seq_len][head_dim] at row `position`
 //   attn_decode_kernel   softmax(q . K^T / sqrt(head_dim)) V over positions 0..position (what ggml_flash_attn_ext computes
 //                        for one query row); a workgroup serves the query heads that share a KV head, so K / V rows are
-//                        loaded once per group; the positions are cut into splits of 256, each split leaves
+//                        loaded once per group; the positions are cut into splits of 64 or 128, each split leaves
 //                        (max, sum, weighted V) behind (a single split writes the result itself)
 //   attn_combine_kernel  merges the splits of a head
 //
@@ -18,7 +18,9 @@ namespace tship {
 namespace {
 
 constexpr int kMaxHeadDim = 256;
-constexpr int kSplit = 128;          // positions per workgroup of the attention kernel
+// positions per workgroup of the attention kernel: one trip of the 16 groups x kInFlight rows while the context is
+// short (the kernel is latency bound: more, shorter workgroups), two trips beyond
+int attn_split_len(int total) { return total <= 2048 ? 64 : 128; }
 constexpr int kInFlight = 4;         // K / V rows a 16-lane group loads before it uses the first
 constexpr int kAttnWaves = 4;
 
@@ -97,7 +99,7 @@ __device__ __forceinline__ void softmax_merge(float& m, float& l, float (&acc)[N
 template <int PER, int G>
 __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ k_cache,
                                                                        const float* __restrict__ v_cache, int group, int max_seq_len,
-                                                                       int total, float scale, int splits, float* __restrict__ partial,
+                                                                       int total, int split_len, float scale, int splits, float* __restrict__ partial,
                                                                        float* __restrict__ out_direct)
 {
     constexpr int HD = 16 * PER;
@@ -119,8 +121,8 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const floa
             acc[g][j] = 0.f;
         }
     }
-    const int t_end = min(total, (split + 1) * kSplit);
-    for (int t0 = split * kSplit + grp; t0 < t_end; t0 += 16 * kInFlight) {
+    const int t_end = min(total, (split + 1) * split_len);
+    for (int t0 = split * split_len + grp; t0 < t_end; t0 += 16 * kInFlight) {
         // kInFlight rows of K and of V per group: every load is issued before the first use
         float kr[kInFlight][PER], vr[kInFlight][PER];
         bool live[kInFlight];
@@ -281,7 +283,8 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_combine_kernel(const flo
 
 size_t attention_decode_ws_bytes(int num_heads, int total)
 {
-    const int splits = (total + kSplit - 1) / kSplit;
+    const int split_len = attn_split_len(total);
+    const int splits = (total + split_len - 1) / split_len;
     return (size_t)num_heads * splits * (kMaxHeadDim + 2) * sizeof(float);
 }
 
@@ -311,17 +314,21 @@ bool launch_attention_decode(const float* q, const float* k_cache, const float* 
         set_last_error("layer decode: bad head counts or position.");
         return false;
     }
-    const int splits = (total + kSplit - 1) / kSplit;
+    const int split_len = attn_split_len(total);
+    const int splits = (total + split_len - 1) / split_len;
     if (splits > 65535) {
         set_last_error("layer decode: context too long for one launch.");
         return false;
     }
     const float scale = 1.0f / sqrtf((float)head_dim);
     const int group = num_heads / num_kv_heads;
-    const int g = group % 8 == 0 ? 8 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;     // query heads per workgroup
+    // query heads per workgroup: as many as share the KV head (its rows are then loaded once), fewer while that leaves
+    // the launch with too few workgroups to hide its latency
+    int g = group % 8 == 0 ? 8 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    while (g > 2 && num_kv_heads * splits * (group / g) < 128) g >>= 1;
     const dim3 grid(num_kv_heads, splits, group / g), block(kAttnWaves * 64);
 #define TSHIP_ATTN_LAUNCH(PER, GG)                                                                                              \
-    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, q, k_cache, v_cache, group, max_seq_len, total, scale, \
+    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, q, k_cache, v_cache, group, max_seq_len, total, split_len, scale, \
                        splits, partial_ws, splits == 1 ? out : nullptr)
 #define TSHIP_ATTN_G(PER)                                                    \
     switch (g) {                                                             \
