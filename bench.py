@@ -24,7 +24,7 @@ Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 8, 12, 13, 14, 39
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the grouped Q4_K GEMV from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the
 # reading of a 1 GiB copy (profiles/gemv_q4k_layer_hbm_traffic.txt); not measured by this script.
-MEASURED_TRAFFIC_BYTES = 124520000
+MEASURED_TRAFFIC_BYTES = 124240000
 
 LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
     ("wq", 4096, 4096), ("wk", 1024, 4096), ("wv", 1024, 4096), ("wo", 4096, 4096),
