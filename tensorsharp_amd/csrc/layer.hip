@@ -54,29 +54,53 @@ __global__ void __launch_bounds__(64) qkv_post_kernel(const float* __restrict__ 
     }
     const bool is_q = b < num_heads;
     const float* nw = is_q ? q_norm_w : k_norm_w;
+    // the head's values are requested first; the rotation angles do not depend on them and are worked out while the
+    // loads are in flight
+    constexpr int kPer = kMaxHeadDim / 64, kPairs = kMaxHeadDim / 128;
+    float xv[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int d = lane + 64 * j;
+        xv[j] = d < head_dim ? src[d] : 0.f;
+    }
+    const int half = head_dim >> 1;
+    float cs[kPairs], sn[kPairs];
+#pragma unroll
+    for (int j = 0; j < kPairs; ++j) {
+        const int p = lane + 64 * j;
+        // the reference builds theta by repeated multiplication; the same float products in the same order
+        float theta = (float)position;
+        for (int i = 0; i < p && p < half; ++i) theta *= theta_scale;
+        const float ang = freq_scale * theta;
+        cs[j] = cosf(ang);
+        sn[j] = sinf(ang);
+    }
     float scale = 1.f;
     if (nw) {
         // ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1 / sqrtf(mean + eps)
         double ss = 0.0;
-        for (int d = lane; d < head_dim; d += 64) ss += (double)(src[d] * src[d]);
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) ss += (double)(xv[j] * xv[j]);
         ss = wave_sum(ss);
         scale = 1.0f / sqrtf((float)(ss / (double)head_dim) + eps);
     }
-    for (int d = lane; d < head_dim; d += 64) head[d] = nw ? (src[d] * scale) * nw[d] : src[d];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int d = lane + 64 * j;
+        if (d < head_dim) head[d] = nw ? (xv[j] * scale) * nw[d] : xv[j];
+    }
     __syncthreads();
     float* dst = is_q ? q_out + (int64_t)b * head_dim
                       : k_cache + ((int64_t)(b - num_heads) * max_seq_len + position) * head_dim;
-    const int half = head_dim >> 1;
-    for (int p = lane; p < half; p += 64) {
-        // the reference builds theta by repeated multiplication; the same float products in the same order
-        float theta = (float)position;
-        for (int i = 0; i < p; ++i) theta *= theta_scale;
-        const float ang = freq_scale * theta;
-        const float c = cosf(ang), s = sinf(ang);
-        const int i0 = neox ? p : 2 * p, i1 = neox ? p + half : 2 * p + 1;
-        const float x0 = head[i0], x1 = head[i1];
-        dst[i0] = x0 * c - x1 * s;
-        dst[i1] = x0 * s + x1 * c;
+#pragma unroll
+    for (int j = 0; j < kPairs; ++j) {
+        const int p = lane + 64 * j;
+        if (p < half) {
+            const int i0 = neox ? p : 2 * p, i1 = neox ? p + half : 2 * p + 1;
+            const float x0 = head[i0], x1 = head[i1];
+            dst[i0] = x0 * cs[j] - x1 * sn[j];
+            dst[i1] = x0 * sn[j] + x1 * cs[j];
+        }
     }
 }
 
