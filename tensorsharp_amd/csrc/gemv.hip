@@ -1,31 +1,29 @@
-// Decode GEMV  y[N] = W[N x K] * x[K]  over raw GGUF blocks (Q8_0 / Q4_K / MXFP4) for gfx950.
+// Decode GEMV  y[N] = W[N x K] * x[K]  over raw GGUF blocks (Q8_0 / Q4_K / Q5_K / Q6_K / MXFP4) for gfx950.
 //
-// Shape of the kernel (all three formats):
-//   * persistent workgroups of 8 wavefronts (two per CU); each workgroup stages x once into LDS
-//     in the layout its format's unpack order wants (fp16 pairs for Q4_K / MXFP4, fp32 for
-//     Q8_0), padded so that a ds_read_b128 per lane is bank-conflict free;
-//   * a wavefront owns four consecutive weight rows at a time, one row per 16 lanes.  A row is
-//     cut into "units" (Q8_0: one 34-byte block, Q4_K: one 64-weight group = 32 quant bytes +
-//     the super-block header, MXFP4: one 17-byte block); lane l of a row takes units l, l+16,
-//     ... so consecutive lanes read consecutive bytes of the raw blocks with 128-bit loads,
-//     everything that depends only on
-//     the lane (block offset, scale bit positions, LDS address of its activations) is computed
-//     once, and the row / slot part of every address is a scalar.  Unaligned units (34 B / 17 B) are fetched as aligned dwords through a
-//     range-checked buffer resource and re-aligned in registers with v_alignbyte;
-//   * the loads of the next batch of units are issued before the current batch is consumed,
-//     and the very first batch is issued before x is staged, so that weight latency overlaps
-//     the prologue;
-//   * dequantization happens in registers: Q8_0 int8 -> fp32 (sign-extending byte select),
-//     Q4_K nibbles masked in place are fp16 subnormals (q * 2^-24) feeding v_dot2_f32_f16,
-//     MXFP4 E2M1 pairs -> fp16 with v_cvt_scalef32_pk_f16_fp4 feeding v_dot2_f32_f16;
-//     block scales (fp16 d, 6-bit K-quant scales/mins, E8M0) are applied once per unit in fp32;
-//   * the per-lane sums of a row are reduced with four DPP adds inside its 16 lanes; the four
-//     results of a group leave as one store instruction.
+// Shape of the kernel (all formats):
+//   * persistent workgroups of 8 wavefronts (two per CU); each workgroup stages x once into LDS in the layout its
+//     format's unpack order wants (fp16 pairs for the K-quants and MXFP4, fp32 for Q8_0), padded so that a
+//     ds_read_b128 per lane is bank-conflict free;
+//   * a wavefront owns a group of consecutive weight rows at a time, one row per LPR lanes (Q8_0 / MXFP4: 4 rows x 16
+//     lanes, the K-quants: 2 rows x 32 lanes).  A row is cut into "units" (Q8_0: one 34-byte block, MXFP4: one 17-byte
+//     block, K-quants: one 64-weight group of a 256-weight block); lane l of a row takes units l, l + LPR, ... so
+//     consecutive lanes read consecutive bytes of the raw blocks with 128-bit loads, everything that depends only on
+//     the lane (block offset, scale bit positions, LDS address of its activations) is computed once, and the row /
+//     step part of every address is a scalar.  Unaligned units (34 B / 17 B blocks, pieces of the 210-byte Q6_K
+//     block) are fetched as aligned dwords through a range-checked buffer resource and re-aligned in registers with
+//     v_alignbyte;
+//   * the loads of the next step are issued before the current step is consumed (two register sets that swap roles),
+//     and the very first step is issued before x is staged, so that weight latency overlaps the prologue;
+//   * dequantization happens in registers: Q8_0 int8 -> fp32 (sign-extending byte select); 4-, 5- and 6-bit values
+//     assembled in the low bits of an fp16 are subnormals (v * 2^-24), exact operands of v_dot2_f32_f16; MXFP4 E2M1
+//     pairs -> fp16 with v_cvt_scalef32_pk_f16_fp4 feeding v_dot2_f32_f16; block scales (fp16 d, 6-bit K-quant
+//     scales / mins, int8 Q6_K scales, E8M0) are applied once per unit in fp32;
+//   * the per-lane sums of a row are reduced with four DPP adds inside 16 lanes (and a lane-swap add for 32-lane
+//     rows); the results of a group leave as one store instruction.
 //
-// Arithmetic restated from TensorSharp.Models/ManagedQuantizedOps.cs:156-200 (dot of a
-// dequantised row with the activation row); for the 4-bit formats the activations of each
-// unit are rounded to fp16 after a per-unit power-of-two scale, so no input magnitude
-// overflows or underflows fp16.
+// Arithmetic restated from TensorSharp.Models/ManagedQuantizedOps.cs:156-200 (dot of a dequantised row with the
+// activation row); except for Q8_0 the activations of each unit are rounded to fp16 after a power-of-two scale of
+// their own, so no input magnitude overflows or underflows fp16.
 #include "tship_internal.h"
 
 #include <algorithm>
