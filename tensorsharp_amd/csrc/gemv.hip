@@ -831,7 +831,9 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
                     xv[c][q] = float4{(xv[c][q].x * scale) * x2[c][q].x, (xv[c][q].y * scale) * x2[c][q].y,
                                       (xv[c][q].z * scale) * x2[c][q].z, (xv[c][q].w * scale) * x2[c][q].w};
         } else if (act == kActSiluMul) {
-            auto silu = [](float g) { return g / (1.0f + expf(-g)); };
+            // hardware exp2 / reciprocal: relative error below 1e-5, far under the fp16 rounding the staged value gets
+            // next (every workgroup evaluates the whole row, so the exact expf and division cost microseconds)
+            auto silu = [](float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); };
 #pragma unroll
             for (int c = 0; c < kStageChunk; ++c)
 #pragma unroll
@@ -843,7 +845,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             auto glu = [&](float g, float u, float b0, float b1) {      // GptOssModel.cs:901-934
                 const float x = fminf(g + b0, limit);
                 const float y = fminf(fmaxf(u + b1, -limit), limit);
-                return (x / (1.0f + expf(alpha * (-x)))) * (y + 1.0f);
+                return (x * __builtin_amdgcn_rcpf(1.0f + __expf(alpha * (-x)))) * (y + 1.0f);
             };
 #pragma unroll
             for (int c = 0; c < kStageChunk; ++c)
