@@ -39,19 +39,12 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 #ifndef TSHIP_GEMV_WAVES
 #define TSHIP_GEMV_WAVES 8
 #endif
-#ifndef TSHIP_GEMV_KU
-#define TSHIP_GEMV_KU 1
-#endif
 #ifndef TSHIP_GEMV_WG_PER_CU
 #define TSHIP_GEMV_WG_PER_CU 2
-#endif
-#ifndef TSHIP_GEMV_XFIRST
-#define TSHIP_GEMV_XFIRST 0
 #endif
 constexpr int kWaves = TSHIP_GEMV_WAVES;
 constexpr int kThreads = kWaves * 64;
 constexpr int kMaxGroup = 8;
-constexpr int kU = TSHIP_GEMV_KU;      // steps per wavefront fetched together, one fetch ahead of the compute
 
 // one GEMV
 // activation modes: what the workgroup stages as x
@@ -243,9 +236,6 @@ struct FmtQ4K {
     static __device__ __forceinline__ float dot(const uint32_t (&w)[kRegs], const Lane& L, uint32_t /*aux*/,
                                                 const uint32_t* xu_dw)
     {
-#ifdef TSHIP_GEMV_DEBUG_NOCOMPUTE
-        return __uint_as_float((w[0] ^ w[1] ^ w[2] ^ w[3] ^ w[4] ^ w[5] ^ w[6] ^ w[7] ^ w[8] ^ w[9] ^ w[10] ^ w[11]) & 0x3fffffffu) * (float)xu_dw[0];
-#endif
         const uint4* xu = reinterpret_cast<const uint4*>(xu_dw);
         float lo = 0.f, hi = 0.f;
 #pragma unroll
@@ -705,8 +695,8 @@ __device__ __forceinline__ float row_sum(float v)
 
 // A wavefront works on a group of 64 / LPR consecutive rows at a time, one row per LPR lanes (LPR = 16 unless the
 // format says otherwise).
-// One step = 16 consecutive units of each of the 4 rows.  Steps of a wavefront are numbered
-// group-major over (group, step); kU steps are fetched together, one fetch ahead of the compute.
+// One step = LPR consecutive units of each row of the group.  Steps of a wavefront are numbered group-major over
+// (group, step); a step is fetched one step ahead of the compute.
 template <typename F>
 struct Step {
     uint32_t w[F::kRegs];
@@ -866,10 +856,9 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         }
     };
 
-    if (TSHIP_GEMV_XFIRST) stage_issue(0);
-    // kU steps per wavefront are requested before x is staged, so weight latency overlaps the
-    // prologue; in the loop the next kU steps are requested before the current ones are consumed.
-    Step<F> cur[kU], nxt[kU];
+    // The first step of a wavefront is requested before x is staged, so weight latency overlaps the prologue; in the
+    // loop the next step is requested before the current one is consumed.
+    Step<F> cur, nxt;
     int fgroup = gw, fstep = 0;                // next step to fetch
     // K-split scheme: rounds of kWaves / KS row groups per workgroup; wavefront (gslot, slice) takes steps
     // [s_begin, s_end) of its group
@@ -887,18 +876,12 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         }
     };
     if constexpr (KS > 1) {
-        fetch_next(cur[0]);
+        fetch_next(cur);
     } else {
-#pragma unroll
-        for (int i = 0; i < kU; ++i) {
-            fetch(fgroup, fstep, cur[i]);
-            advance(fgroup, fstep);
-        }
+        fetch(fgroup, fstep, cur);
+        advance(fgroup, fstep);
     }
-    if (!TSHIP_GEMV_XFIRST) stage_issue(0);
-#ifdef TSHIP_GEMV_DEBUG_NOSTAGE
-    if (P.N < 0)
-#endif
+    stage_issue(0);
     stage_commit(0);
     for (int base = kThreads * kStageChunk; base < items; base += kThreads * kStageChunk) {
         stage_issue(base);
@@ -914,10 +897,10 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         for (int r = 0; r < rounds; ++r) {
             float acc = 0.f;
             for (int st = s_begin; st < s_end; ++st) {
-                fetch_next(nxt[0]);
-                const uint32_t* xu = lds + lds_lane + (uint32_t)cur[0].step * (uint32_t)(LPR * F::kLdsDwords);
-                acc += F::dot(cur[0].w, L, cur[0].aux, xu);
-                cur[0] = nxt[0];
+                fetch_next(nxt);
+                const uint32_t* xu = lds + lds_lane + (uint32_t)cur.step * (uint32_t)(LPR * F::kLdsDwords);
+                acc += F::dot(cur.w, L, cur.aux, xu);
+                cur = nxt;
             }
             const float t = row_sum<LPR>(acc);
             float* pr = part + (r & 1) * kWaves * 4;
@@ -945,7 +928,6 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             acc = 0.f;
         }
     };
-    static_assert(kU == 1, "the loop below alternates two single-step buffers");
     // Two steps per trip, the buffers swapping roles, so no step is ever copied between registers.
     // strict: a wavefront asks for its next step only once the previous one has arrived, so it never has more than
     // one step in flight and the wavefronts of the launch stay in step with each other.  Measured on one box
@@ -953,16 +935,16 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // FFN's two launches (66 + 33 MB) 31.7 / 30.6 us and a whole layer 67.1 / 65.8 us: long launches that saturate
     // HBM lose bandwidth when requests run ahead, short ones gain from the extra overlap.
     for (;;) {
-        if (cur[0].group >= ngroups) break;
+        if (cur.group >= ngroups) break;
         if (strict) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        fetch(fgroup, fstep, nxt[0]);
+        fetch(fgroup, fstep, nxt);
         advance(fgroup, fstep);
-        consume(cur[0]);
-        if (nxt[0].group >= ngroups) break;
+        consume(cur);
+        if (nxt.group >= ngroups) break;
         if (strict) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        fetch(fgroup, fstep, cur[0]);
+        fetch(fgroup, fstep, cur);
         advance(fgroup, fstep);
-        consume(nxt[0]);
+        consume(nxt);
     }
 }
 
