@@ -453,6 +453,119 @@ struct FmtMXFP4 {
     }
 };
 
+// ---- Q4_0 / Q4_1 -----------------------------------------------------------------------------
+// Blocks of 32 weights: fp16 d (Q4_1: also fp16 m), then 16 bytes whose low nibble is weight j and high nibble weight
+// j + 16; value d * (q - 8) (Q4_1: d * q + m) (ggml-quants.c dequantize_row_q4_0 / q4_1; ManagedQuantizedOps.cs:268-330).
+// LDS unit (80 B): for quant dword i, dwords 4i .. 4i+3 = (x[4i], x[4i+2]), (x[4i+1], x[4i+3]), then the same of
+// x[16 + ..]; then the sum of the scaled fp16 activations and the unit's power-of-two scale.  Nibbles masked in place
+// are fp16 subnormals (q * 2^-24, high nibbles 16 q * 2^-24) for v_dot2_f32_f16; the -8 / + m term leaves through the sum.
+template <bool HAS_MIN>
+struct FmtQ4Legacy {
+    static constexpr int kLPR = 16;
+    static constexpr int kUnitElems = 32;
+    static constexpr int kLdsDwords = 20;
+    static constexpr int kRegs = 6;
+    static constexpr int kBlock = HAS_MIN ? 20 : 18;
+
+    static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 5) * kBlock; }
+
+    static constexpr int kStageF4 = 2;
+    // one work item = x[b*32 + 4i .. +3] and x[b*32 + 16 + 4i .. +3]; the 4 lanes of a quad share a unit
+    static __device__ __forceinline__ void stage_offsets(int it, uint32_t (&off)[kStageF4])
+    {
+        const uint32_t b = (uint32_t)it >> 2, i = (uint32_t)it & 3u;
+        off[0] = (b * 32u + 4u * i) * 4u;
+        off[1] = off[0] + 64u;
+    }
+    static __device__ __forceinline__ void stage_store(const float4 (&vv)[kStageF4], int it, bool live, uint32_t* lds)
+    {
+        const float4 lo = vv[0], hi = vv[1];
+        float amax = fmaxf(fmaxf(fmaxf(fabsf(lo.x), fabsf(lo.y)), fmaxf(fabsf(lo.z), fabsf(lo.w))),
+                           fmaxf(fmaxf(fabsf(hi.x), fabsf(hi.y)), fmaxf(fabsf(hi.z), fabsf(hi.w))));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
+        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
+        float inv, scale;
+        pow2_scale(amax, &inv, &scale);
+        const _Float16 a0 = (_Float16)(lo.x * inv), a1 = (_Float16)(lo.y * inv), a2 = (_Float16)(lo.z * inv), a3 = (_Float16)(lo.w * inv);
+        const _Float16 b0 = (_Float16)(hi.x * inv), b1 = (_Float16)(hi.y * inv), b2 = (_Float16)(hi.z * inv), b3 = (_Float16)(hi.w * inv);
+        float s = (((float)a0 + (float)a1) + ((float)a2 + (float)a3)) + (((float)b0 + (float)b1) + ((float)b2 + (float)b3));
+        s += TSHIP_DPP_F(s, kDppXor1);
+        s += TSHIP_DPP_F(s, kDppXor2);
+        if (live) {
+            const int b = it >> 2, i = it & 3;
+            H2U p0, p1, p2, p3;
+            p0.h = half2_t{a0, a2};
+            p1.h = half2_t{a1, a3};
+            p2.h = half2_t{b0, b2};
+            p3.h = half2_t{b1, b3};
+            uint4 o;
+            o.x = p0.u;
+            o.y = p1.u;
+            o.z = p2.u;
+            o.w = p3.u;
+            uint32_t* unit = lds + b * kLdsDwords;
+            *reinterpret_cast<uint4*>(unit + 4 * i) = o;
+            if (i == 0) {
+                reinterpret_cast<float*>(unit)[16] = s;
+                reinterpret_cast<float*>(unit)[17] = scale;
+            }
+        }
+    }
+    static __device__ __forceinline__ int stage_items(int K) { return K >> 3; }
+
+    static constexpr int kSlotBytes = kLPR * kBlock;
+
+    struct Lane {
+        uint32_t voff;
+    };
+    static __device__ __forceinline__ Lane lane_setup(int sub, int l16, uint32_t row_bytes)
+    {
+        Lane L;
+        L.voff = (uint32_t)sub * row_bytes + (uint32_t)l16 * (uint32_t)kBlock;
+        return L;
+    }
+
+    // the block sits at byte 0 or 2 of a 24-byte dword-aligned window.  Returns p & 3.
+    static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t rs, const Lane& L, uint32_t soff,
+                                                    uint32_t row_delta, int /*slot*/, bool live, uint32_t (&w)[kRegs])
+    {
+        const uint32_t p = L.voff + row_delta;
+        const uint32_t al = live ? (p & ~3u) : kDeadOffset;
+        buf_load4(rs, al, soff, &w[0]);
+        w[4] = buf_load1(rs, al + 16, soff);
+        w[5] = HAS_MIN ? buf_load1(rs, al + 20, soff) : 0u;
+        return p & 3u;
+    }
+
+    static __device__ __forceinline__ float dot(const uint32_t (&w)[kRegs], const Lane& /*L*/, uint32_t o, const uint32_t* xu_dw)
+    {
+        const bool odd = (o & 2u) != 0;
+        H2U dh, mh;
+        dh.u = odd ? (w[0] >> 16) : (w[0] & 0xffffu);
+        mh.u = HAS_MIN ? (odd ? (w[1] & 0xffffu) : (w[0] >> 16)) : 0u;
+        const float d = (float)dh.h.x, m = (float)mh.h.x;
+        const uint4* xu = reinterpret_cast<const uint4*>(xu_dw);
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // quant bytes start 2 (Q4_1: 4) bytes into the block
+            uint32_t q;
+            if (HAS_MIN) q = odd ? __builtin_amdgcn_alignbyte(w[i + 2], w[i + 1], 2) : w[i + 1];
+            else q = odd ? w[i + 1] : __builtin_amdgcn_alignbyte(w[i + 1], w[i], 2);
+            const uint32_t q8 = q >> 8;
+            const uint4 xv = xu[i];
+            lo = dot2(q & 0x000f000fu, xv.x, lo);
+            lo = dot2(q8 & 0x000f000fu, xv.y, lo);
+            hi = dot2(q & 0x00f000f0u, xv.z, hi);
+            hi = dot2(q8 & 0x00f000f0u, xv.w, hi);
+        }
+        const uint4 tail = xu[4];
+        const float sum = __uint_as_float(tail.x), xscale = __uint_as_float(tail.y);
+        const float qx = lo * 16777216.f + hi * 1048576.f;
+        return (HAS_MIN ? d * qx + m * sum : d * (qx - 8.f * sum)) * xscale;
+    }
+};
+
 // ---- Q8_0 ------------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 144 B): 32 fp32 activations, 16 B pad.  fp32 throughout.
 #ifndef TSHIP_GEMV_Q80_LPR
@@ -962,11 +1075,13 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
     else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
+    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
+    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
     else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
-int unit_lds_bytes(int type) { return type == kTypeMXFP4 ? 80 : type == kTypeQ6_K ? 176 : 144; }
+int unit_lds_bytes(int type) { return type == kTypeMXFP4 || type == kTypeQ4_0 || type == kTypeQ4_1 ? 80 : type == kTypeQ6_K ? 176 : 144; }
 int lanes_per_row(int type)
 {
     return type == kTypeQ4_K || type == kTypeQ5_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : type == kTypeQ6_K ? FmtQ6K::kLPR : FmtQ80::kLPR;
@@ -1003,6 +1118,8 @@ int gemv_max_k(int type)
     case kTypeMXFP4: return (int)(kMaxLds / 80 / FmtMXFP4::kLPR) * FmtMXFP4::kLPR * 32;
     case kTypeQ6_K: return (int)(kMaxLds / 176 / FmtQ6K::kLPR) * FmtQ6K::kLPR * 64;
     case kTypeQ5_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
+    case kTypeQ4_0:
+    case kTypeQ4_1: return (int)(kMaxLds / 80 / 16) * 16 * 32;
     default: return 0;
     }
 }
@@ -1018,7 +1135,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         set_last_error("gemv: group size out of range.");
         return false;
     }
-    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K && type != kTypeQ5_K) {
+    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K && type != kTypeQ5_K && type != kTypeQ4_0 && type != kTypeQ4_1) {
         set_last_error("gemv: unsupported type.");
         return false;
     }
@@ -1104,6 +1221,8 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     case kTypeMXFP4: return TSHIP_GEMV_DISPATCH(kTypeMXFP4);
     case kTypeQ6_K: return TSHIP_GEMV_DISPATCH(kTypeQ6_K);
     case kTypeQ5_K: return TSHIP_GEMV_DISPATCH(kTypeQ5_K);
+    case kTypeQ4_0: return TSHIP_GEMV_DISPATCH(kTypeQ4_0);
+    case kTypeQ4_1: return TSHIP_GEMV_DISPATCH(kTypeQ4_1);
     default: return TSHIP_GEMV_DISPATCH(kTypeQ8_0);
     }
 #undef TSHIP_GEMV_DISPATCH

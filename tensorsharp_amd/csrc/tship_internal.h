@@ -69,7 +69,11 @@ inline bool is_quant_type(int type)
     default: return false;
     }
 }
-inline bool has_gemv(int type) { return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4 || type == kTypeQ6_K || type == kTypeQ5_K; }
+inline bool has_gemv(int type)
+{
+    return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4 || type == kTypeQ6_K || type == kTypeQ5_K ||
+           type == kTypeQ4_0 || type == kTypeQ4_1;
+}
 // formats with a dequantizer (DequantizeToF32, embedding gather): every block format the managed code reads
 // (ManagedQuantizedOps.cs:40-59) except Q8_1
 inline bool is_dequant_type(int type) { return type != kTypeF32 && block_elems(type) != 0; }

@@ -134,7 +134,34 @@ def quantize_q5_k_simple(w):
     return out.reshape(-1)
 
 
-QUANTIZERS = {8: quantize_q8_0, 12: quantize_q4_k_simple, 13: quantize_q5_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
+def quantize_q4_0_simple(w):
+    """Valid Q4_0 blocks (ggml-common.h block_q4_0): d = amax / 7, q = round(x / d) + 8, for synthetic weights."""
+    x = w.reshape(-1, 32).float()
+    d = x.abs().amax(dim=1) / 7.0
+    d16 = d.to(torch.float16).float()
+    q = torch.where(d16[:, None] > 0, torch.round(x / d16[:, None].clamp_min(1e-30)) + 8, torch.full_like(x, 8)).clamp(0, 15).to(torch.uint8)
+    out = torch.empty((x.shape[0], 18), dtype=torch.uint8, device=w.device)
+    out[:, 0:2] = _half_bytes(d)
+    out[:, 2:] = q[:, :16] | (q[:, 16:] << 4)
+    return out.reshape(-1)
+
+
+def quantize_q4_1_simple(w):
+    """Valid Q4_1 blocks (ggml-common.h block_q4_1): min / max fit with 15 steps, for synthetic weights."""
+    x = w.reshape(-1, 32).float()
+    lo = x.amin(dim=1)
+    d = (x.amax(dim=1) - lo) / 15.0
+    d16 = d.to(torch.float16).float()
+    m16 = lo.to(torch.float16).float()
+    q = torch.where(d16[:, None] > 0, torch.round((x - m16[:, None]) / d16[:, None].clamp_min(1e-30)), torch.zeros_like(x)).clamp(0, 15).to(torch.uint8)
+    out = torch.empty((x.shape[0], 20), dtype=torch.uint8, device=w.device)
+    out[:, 0:2] = _half_bytes(d)
+    out[:, 2:4] = _half_bytes(lo)
+    out[:, 4:] = q[:, :16] | (q[:, 16:] << 4)
+    return out.reshape(-1)
+
+
+QUANTIZERS = {2: quantize_q4_0_simple, 3: quantize_q4_1_simple, 8: quantize_q8_0, 12: quantize_q4_k_simple, 13: quantize_q5_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
 
 
 def random_weight(ggml_type, n_rows, n_cols, device, seed, sigma=0.02, chunk_rows=4096):

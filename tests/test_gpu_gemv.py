@@ -309,3 +309,38 @@ def test_q5_k_shapes(hip, oracle, N, K):
     xs = (x * np.float32(1e-20)).astype(np.float32)
     check("q4_k", run_device(hip, Q5_K, wq, N, K, xs), oracle.matmul_f64(Q5_K, wq, N, K, xs))
     assert np.all(run_device(hip, Q5_K, wq, N, K, np.zeros((1, K), np.float32)) == 0)
+
+
+# ---- Q4_0 / Q4_1: 18- and 20-byte blocks of 32 weights ----
+@pytest.mark.parametrize("name", ["q4_0", "q4_1"])
+@pytest.mark.parametrize("N,K", [(1, 32), (3, 96), (7, 1056), (130, 2560), (257, 4096), (1001, 2880), (4096, 14336)])
+def test_q4_legacy_shapes(hip, oracle, name, N, K):
+    from oracle.oracle import Q4_0, Q4_1
+    t = {"q4_0": Q4_0, "q4_1": Q4_1}[name]
+    rng = np.random.default_rng(N * 17 + K)
+    wq = inputs.random_blocks(name, N, K, rng)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    check("q4_k", run_device(hip, t, wq, N, K, x), oracle.matmul_f64(t, wq, N, K, x))
+    xs = (x * np.float32(3e4)).astype(np.float32)
+    check("q4_k", run_device(hip, t, wq, N, K, xs), oracle.matmul_f64(t, wq, N, K, xs))
+    assert np.all(run_device(hip, t, wq, N, K, np.zeros((1, K), np.float32)) == 0)
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q4_1"])
+def test_q4_legacy_views_at_odd_rows(hip, oracle, name):
+    # 35 blocks per row: Q4_0 rows alternate between byte 0 and byte 2 of a dword; views that start rows into a tensor
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    from oracle.oracle import Q4_0, Q4_1
+    t = {"q4_0": Q4_0, "q4_1": Q4_1}[name]
+    rng = np.random.default_rng(44)
+    N, K = 64, 1120
+    wq = inputs.random_blocks(name, N + 3, K, rng)
+    rs = oracle.row_size(t, K)
+    dev = torch.from_numpy(wq).cuda()
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    for rb in (1, 2, 3):
+        y = hip.LinearForward(xd, QuantizedWeight(dev[rb * rs:(rb + N) * rs], t, K, N))
+        torch.cuda.synchronize()
+        check("q4_k", y.cpu().numpy(), oracle.matmul_f64(t, wq[rb * rs:(rb + N) * rs], N, K, x))

@@ -25,11 +25,13 @@ def test_q4_k_generator_makes_valid_blocks(oracle):
     assert rms < 0.12          # the reference's search reaches 0.071; a plain min/max fit stays close
 
 
-def test_q5_k_and_q6_k_generators_make_valid_blocks(oracle):
+def test_other_generators_make_valid_blocks(oracle):
     from oracle.oracle import Q5_K, Q6_K
     g = torch.Generator().manual_seed(5)
     w = torch.randn((16, 1024), generator=g) * 0.02
-    for t, fn, size, bound in ((Q5_K, synth.quantize_q5_k_simple, 176, 0.06), (Q6_K, synth.quantize_q6_k_simple, 210, 0.04)):
+    from oracle.oracle import Q4_0, Q4_1
+    for t, fn, size, bound in ((Q5_K, synth.quantize_q5_k_simple, 176, 0.06), (Q6_K, synth.quantize_q6_k_simple, 210, 0.04),
+                               (Q4_0, synth.quantize_q4_0_simple, 8 * 18, 0.2), (Q4_1, synth.quantize_q4_1_simple, 8 * 20, 0.12)):
         raw = fn(w).numpy()
         assert raw.size == 16 * 4 * size
         deq = oracle.dequantize(t, raw)
