@@ -209,15 +209,33 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
     if (tid == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
     _Float16* dst = out + (int64_t)m * Kp;
     auto put = [&](int k, float v) { dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)(v * inv); };
+    // Four consecutive activations land in one aligned 8-byte piece of the k-tile: in the K-quant order as
+    // (x0, x2, x1, x3), in the natural order as they are, and in the split-nibble order interleaved with the four
+    // activations 16 further on, which the lane four to the right (left) holds - the pair swaps them and each stores
+    // one half of the 16 bytes.
 #pragma unroll
     for (int i = 0; i < kCvtHold; ++i) {
         const int q = tid + i * THREADS;
-        if (q < k4) {
-            put(4 * q, hold[i].x);
-            put(4 * q + 1, hold[i].y);
-            put(4 * q + 2, hold[i].z);
-            put(4 * q + 3, hold[i].w);
+        const float4 v = float4{hold[i].x * inv, hold[i].y * inv, hold[i].z * inv, hold[i].w * inv};
+        uint2 o;
+        int slot;
+        if (TYPE == kTypeQ4_K) {
+            o.x = pack2(v.x, v.z);
+            o.y = pack2(v.y, v.w);
+            slot = k_slot<TYPE>((4 * q) & (kBK - 1));
+        } else if (TYPE == kTypeMXFP4) {
+            // uniform trip count: lanes past the row take part in the exchange with zeros
+            const float4 p = float4{__shfl_xor(v.x, 4), __shfl_xor(v.y, 4), __shfl_xor(v.z, 4), __shfl_xor(v.w, 4)};
+            const bool upper = (q & 4) != 0;             // this lane holds the activations paired with high nibbles
+            o.x = upper ? pack2(p.z, v.z) : pack2(v.x, p.x);
+            o.y = upper ? pack2(p.w, v.w) : pack2(v.y, p.y);
+            slot = k_slot<TYPE>((4 * (q & ~4)) & (kBK - 1)) + (upper ? 4 : 0);
+        } else {
+            o.x = pack2(v.x, v.y);
+            o.y = pack2(v.z, v.w);
+            slot = k_slot<TYPE>((4 * q) & (kBK - 1));
         }
+        if (q < k4) *reinterpret_cast<uint2*>(dst + (((4 * q) & ~(kBK - 1)) | slot)) = o;
     }
     for (int k = kHeld + tid; k < K; k += THREADS) put(k, tail_value(k));
     for (int k = K + tid; k < Kp; k += THREADS) dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)0.f;
