@@ -1246,25 +1246,21 @@ bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm
 {
     const int q_dim = L.num_heads * L.head_dim, k_dim = L.num_kv_heads * L.head_dim, qkv_n = q_dim + 2 * k_dim;
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
-    const size_t b_qkv = al((size_t)qkv_n * 4), b_q = al((size_t)q_dim * 4), b_attn = al((size_t)q_dim * 4);
+    const size_t b_qkv = al((size_t)qkv_n * 4), b_attn = al((size_t)q_dim * 4);
     const size_t b_part = al(attention_decode_ws_bytes(L.num_heads, position + 1));
     const size_t b_mm = std::max(matmul_ws_bytes(L.qkv_type, 1, L.hidden, true), matmul_ws_bytes(L.o_type, 1, q_dim, false));
-    char* ws = static_cast<char*>(dev_ws_reserve(b_qkv + b_q + b_attn + b_part + b_mm + 256));
+    char* ws = static_cast<char*>(dev_ws_reserve(b_qkv + b_attn + b_part + b_mm + 256));
     if (!ws) return false;
     float* qkv_out = reinterpret_cast<float*>(ws);
-    float* q_rot = reinterpret_cast<float*>(ws + b_qkv);
-    float* attn = reinterpret_cast<float*>(ws + b_qkv + b_q);
-    float* part = reinterpret_cast<float*>(ws + b_qkv + b_q + b_attn);
-    void* mm_ws = ws + b_qkv + b_q + b_attn + b_part;
+    float* attn = reinterpret_cast<float*>(ws + b_qkv);
+    float* part = reinterpret_cast<float*>(ws + b_qkv + b_attn);
+    void* mm_ws = ws + b_qkv + b_attn + b_part;
     const TSHipTensorView2D h_view{hidden, 1, L.hidden, L.hidden, 1, (int64_t)L.hidden * 4};
     const TSHipTensorView2D qkv_view{qkv_out, 1, qkv_n, qkv_n, 1, (int64_t)qkv_n * 4};
     const TSHipTensorView2D attn_view{attn, 1, q_dim, q_dim, 1, (int64_t)q_dim * 4};
     if (!run_matmul_device_ws(qkv_view, h_view, qkv, L.qkv_type, L.hidden, qkv_n, stream, mm_ws, attn_norm, eps, false)) return false;
-    if (!launch_qkv_post(qkv_out, L.num_heads, L.num_kv_heads, L.head_dim, q_norm, k_norm, eps, position, rope_base, rope_freq_scale,
-                         rope_mode, q_rot, k_cache, v_cache, L.max_seq_len, stream))
-        return false;
-    if (!launch_attention_decode(q_rot, k_cache, v_cache, L.num_heads, L.num_kv_heads, L.head_dim, L.max_seq_len, position + 1, part,
-                                 attn, stream))
+    if (!launch_attention_decode(qkv_out, q_norm, k_norm, eps, rope_base, rope_freq_scale, rope_mode, k_cache, v_cache, L.num_heads,
+                                 L.num_kv_heads, L.head_dim, L.max_seq_len, position, part, attn, stream))
         return false;
     // hidden += W_o attn
     if (!run_matmul_device_ws(h_view, attn_view, o, L.o_type, q_dim, L.hidden, stream, mm_ws, nullptr, 0.f, true)) return false;

@@ -1,14 +1,15 @@
 // Single-token attention pieces of the whole-layer decode (TensorSharp.GGML.Native/ggml_ops_transformer.cpp:318-470):
 // what sits between the fused QKV projection and the output projection.
 //
-//   qkv_post_kernel      per head: optional RMSNorm over the head (ggml_rms_norm, then * weight), RoPE at `position`
-//                        (ggml_rope_ext with n_dims = head_dim, ext_factor 0, attn_factor 1: ggml-cpu/ops.cpp:5549-5563,
-//                        :5636-5652); q heads go to a scratch row, k heads and the untouched v heads into the fp32 KV
-//                        cache [kv_head][max_seq_len][head_dim] at row `position`
-//   attn_decode_kernel   softmax(q . K^T / sqrt(head_dim)) V over positions 0..position (what ggml_flash_attn_ext computes
-//                        for one query row); a workgroup serves the query heads that share a KV head, so K / V rows are
-//                        loaded once per group; the positions are cut into splits of 64 or 128, each split leaves
-//                        (max, sum, weighted V) behind (a single split writes the result itself)
+//   attn_decode_kernel   first finishes the projections for the heads it serves - optional RMSNorm over the head
+//                        (ggml_rms_norm, then * weight), RoPE at `position` (ggml_rope_ext with n_dims = head_dim,
+//                        ext_factor 0, attn_factor 1: ggml-cpu/ops.cpp:5549-5563, :5636-5652); the new k and the
+//                        untouched v row go into the fp32 KV cache [kv_head][max_seq_len][head_dim] at row `position`
+//                        (written by the workgroup of the last split, which uses them from LDS) - then computes
+//                        softmax(q . K^T / sqrt(head_dim)) V over positions 0..position (what ggml_flash_attn_ext
+//                        computes for one query row); a workgroup serves the query heads that share a KV head, so K / V
+//                        rows are loaded once per group; the positions are cut into splits of 64 or 128, each split
+//                        leaves (max, sum, weighted V) behind (a single split writes the result itself)
 //   attn_combine_kernel  merges the splits of a head
 //
 // HBM-bound on the KV cache: 2 * num_kv_heads * (position + 1) * head_dim * 4 bytes per call.
@@ -37,72 +38,19 @@ __device__ __forceinline__ double wave_sum(double v)
     return v;
 }
 
-// one wavefront per head: blocks [0, H) are query heads, [H, H + KV) key heads, [H + KV, H + 2 KV) value heads
-__global__ void __launch_bounds__(64) qkv_post_kernel(const float* __restrict__ qkv, int num_heads, int num_kv_heads, int head_dim,
-                                                      const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
-                                                      float eps, int position, float theta_scale, float freq_scale, int neox,
-                                                      float* __restrict__ q_out, float* __restrict__ k_cache,
-                                                      float* __restrict__ v_cache, int max_seq_len)
-{
-    __shared__ float head[kMaxHeadDim];
-    const int b = blockIdx.x, lane = threadIdx.x;
-    const float* src = qkv + (int64_t)b * head_dim;          // q heads, then k heads, then v heads, all head_dim wide
-    if (b >= num_heads + num_kv_heads) {
-        float* dst = v_cache + ((int64_t)(b - num_heads - num_kv_heads) * max_seq_len + position) * head_dim;
-        for (int d = lane; d < head_dim; d += 64) dst[d] = src[d];
-        return;
-    }
-    const bool is_q = b < num_heads;
-    const float* nw = is_q ? q_norm_w : k_norm_w;
-    // the head's values are requested first; the rotation angles do not depend on them and are worked out while the
-    // loads are in flight
-    constexpr int kPer = kMaxHeadDim / 64, kPairs = kMaxHeadDim / 128;
-    float xv[kPer];
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        const int d = lane + 64 * j;
-        xv[j] = d < head_dim ? src[d] : 0.f;
-    }
-    const int half = head_dim >> 1;
-    float cs[kPairs], sn[kPairs];
-#pragma unroll
-    for (int j = 0; j < kPairs; ++j) {
-        const int p = lane + 64 * j;
-        // the reference builds theta by repeated multiplication; the same float products in the same order
-        float theta = (float)position;
-        for (int i = 0; i < p && p < half; ++i) theta *= theta_scale;
-        const float ang = freq_scale * theta;
-        cs[j] = cosf(ang);
-        sn[j] = sinf(ang);
-    }
-    float scale = 1.f;
-    if (nw) {
-        // ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1 / sqrtf(mean + eps)
-        double ss = 0.0;
-#pragma unroll
-        for (int j = 0; j < kPer; ++j) ss += (double)(xv[j] * xv[j]);
-        ss = wave_sum(ss);
-        scale = 1.0f / sqrtf((float)(ss / (double)head_dim) + eps);
-    }
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        const int d = lane + 64 * j;
-        if (d < head_dim) head[d] = nw ? (xv[j] * scale) * nw[d] : xv[j];
-    }
-    __syncthreads();
-    float* dst = is_q ? q_out + (int64_t)b * head_dim
-                      : k_cache + ((int64_t)(b - num_heads) * max_seq_len + position) * head_dim;
-#pragma unroll
-    for (int j = 0; j < kPairs; ++j) {
-        const int p = lane + 64 * j;
-        if (p < half) {
-            const int i0 = neox ? p : 2 * p, i1 = neox ? p + half : 2 * p + 1;
-            const float x0 = head[i0], x1 = head[i1];
-            dst[i0] = x0 * cs[j] - x1 * sn[j];
-            dst[i1] = x0 * sn[j] + x1 * cs[j];
-        }
-    }
-}
+// What the attention kernel needs to finish the projections itself: the raw output of the QKV matmul
+// ([q heads | k heads | v heads], head_dim each), the optional per-head RMSNorm weights, the rotation, and the caches
+// whose row `position` it writes.
+struct AttnFront {
+    const float* qkv;
+    const float* q_norm_w;
+    const float* k_norm_w;
+    float eps, theta_scale, freq_scale;
+    int neox;
+    int num_heads, num_kv_heads;
+    float* k_cache;
+    float* v_cache;
+};
 
 // Merge of two online-softmax states (max, sum, weighted values).
 template <int N>
@@ -121,19 +69,99 @@ __device__ __forceinline__ void softmax_merge(float& m, float& l, float (&acc)[N
 // the split, kInFlight at a time (all their loads are issued before the first is used: the loop is latency bound), lane l of
 // a group holds the head dimensions l, l + 16, ... (PER of them).  Groups, then wavefronts, merge their softmax states.
 template <int PER, int G>
-__global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ k_cache,
-                                                                       const float* __restrict__ v_cache, int group, int max_seq_len,
-                                                                       int total, int split_len, float scale, int splits, float* __restrict__ partial,
-                                                                       float* __restrict__ out_direct)
+__global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const AttnFront F, int group, int max_seq_len, int total,
+                                                                       int split_len, float scale, int splits,
+                                                                       float* __restrict__ partial, float* __restrict__ out_direct)
 {
     constexpr int HD = 16 * PER;
     __shared__ float sm[kAttnWaves][G], sl[kAttnWaves][G], sacc[kAttnWaves][G][HD];
+    __shared__ float sq[G][HD], sk[HD], sv[HD], tmp[kAttnWaves][HD];
     const int kvh = blockIdx.x, split = blockIdx.y;
     const int h0 = kvh * group + blockIdx.z * G;                     // first query head of this workgroup
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lg = lane & 15, grp = (wave << 2) | (lane >> 4);       // 16 groups per workgroup
-    const float* kb = k_cache + (int64_t)kvh * max_seq_len * HD;
-    const float* vb = v_cache + (int64_t)kvh * max_seq_len * HD;
+    const float* kb = F.k_cache + (int64_t)kvh * max_seq_len * HD;
+    const float* vb = F.v_cache + (int64_t)kvh * max_seq_len * HD;
+    const int position = total - 1;
+    const bool last = split == splits - 1;                           // the split that holds the new position
+
+    // ---- the projections' last steps, per head: RMSNorm over the head (ggml_rms_norm, then * weight), RoPE at
+    // `position` (ggml_rope_ext with n_dims = head_dim: ggml-cpu/ops.cpp:5549-5563, :5636-5652).  Every workgroup
+    // prepares its own query heads; the workgroup of the last split also prepares the new key / value row, uses it
+    // from LDS and (query-head chunk 0 only) writes it to the caches.
+    {
+        constexpr int kPer = (HD + 63) / 64, kPairs = (HD / 2 + 63) / 64;
+        constexpr int half = HD / 2;
+        float cs[kPairs], sn[kPairs];
+#pragma unroll
+        for (int j = 0; j < kPairs; ++j) {
+            const int p = lane + 64 * j;
+            // the reference builds theta by repeated multiplication; the same float products in the same order
+            float theta = (float)position;
+            for (int i = 0; i < p && p < half; ++i) theta *= F.theta_scale;
+            const float ang = F.freq_scale * theta;
+            cs[j] = cosf(ang);
+            sn[j] = sinf(ang);
+        }
+        const int nprep = G + (last ? 1 : 0);
+        for (int hh = wave; hh < nprep; hh += kAttnWaves) {          // uniform per wavefront
+            const bool is_q = hh < G;
+            const float* src = F.qkv + (int64_t)(is_q ? h0 + hh : F.num_heads + kvh) * HD;
+            const float* nw = is_q ? F.q_norm_w : F.k_norm_w;
+            float xv[kPer];
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) {
+                const int d = lane + 64 * j;
+                xv[j] = d < HD ? src[d] : 0.f;
+            }
+            float rs = 1.f;
+            if (nw) {
+                // ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1 / sqrtf(mean + eps)
+                double ss = 0.0;
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) ss += (double)(xv[j] * xv[j]);
+                ss = wave_sum(ss);
+                rs = 1.0f / sqrtf((float)(ss / (double)HD) + F.eps);
+            }
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) {
+                const int d = lane + 64 * j;
+                if (d < HD) tmp[wave][d] = nw ? (xv[j] * rs) * nw[d] : xv[j];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the wavefront's own LDS writes before its reads
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            float* dst = is_q ? sq[hh] : sk;
+            float* cache = (!is_q && blockIdx.z == 0) ? F.k_cache + ((int64_t)kvh * max_seq_len + position) * HD : nullptr;
+#pragma unroll
+            for (int j = 0; j < kPairs; ++j) {
+                const int p = lane + 64 * j;
+                if (p < half) {
+                    const int i0 = F.neox ? p : 2 * p, i1 = F.neox ? p + half : 2 * p + 1;
+                    const float x0 = tmp[wave][i0], x1 = tmp[wave][i1];
+                    const float r0 = x0 * cs[j] - x1 * sn[j], r1 = x0 * sn[j] + x1 * cs[j];
+                    dst[i0] = r0;
+                    dst[i1] = r1;
+                    if (cache) {
+                        cache[i0] = r0;
+                        cache[i1] = r1;
+                    }
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // tmp is reused by this wavefront's next head
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (last) {
+            const float* src = F.qkv + (int64_t)(F.num_heads + F.num_kv_heads + kvh) * HD;
+            float* cache = blockIdx.z == 0 ? F.v_cache + ((int64_t)kvh * max_seq_len + position) * HD : nullptr;
+            for (int d = threadIdx.x; d < HD; d += kAttnWaves * 64) {
+                const float v = src[d];
+                sv[d] = v;
+                if (cache) cache[d] = v;
+            }
+        }
+        __syncthreads();
+    }
     float qr[G][PER], acc[G][PER], m[G], l[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -141,7 +169,7 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const floa
         l[g] = 0.f;
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            qr[g][j] = q[(int64_t)(h0 + g) * HD + lg + 16 * j] * scale;
+            qr[g][j] = sq[g][lg + 16 * j] * scale;
             acc[g][j] = 0.f;
         }
     }
@@ -159,6 +187,17 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const floa
             for (int j = 0; j < PER; ++j) {
                 kr[u][j] = kb[row + 16 * j];
                 vr[u][j] = vb[row + 16 * j];
+            }
+        }
+        if (last) {       // uniform: the new position's row is not in the caches yet (another workgroup may be writing it)
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                const bool fresh = t0 + 16 * u == position;
+#pragma unroll
+                for (int j = 0; j < PER; ++j) {
+                    kr[u][j] = fresh ? sk[lg + 16 * j] : kr[u][j];
+                    vr[u][j] = fresh ? sv[lg + 16 * j] : vr[u][j];
+                }
             }
         }
 #pragma unroll
@@ -312,32 +351,31 @@ size_t attention_decode_ws_bytes(int num_heads, int total)
     return (size_t)num_heads * splits * (kMaxHeadDim + 2) * sizeof(float);
 }
 
-bool launch_qkv_post(const float* qkv, int num_heads, int num_kv_heads, int head_dim, const float* q_norm_w, const float* k_norm_w,
-                     float eps, int position, float rope_base, float rope_freq_scale, int rope_mode, float* q_out, float* k_cache,
-                     float* v_cache, int max_seq_len, hipStream_t stream)
+bool launch_attention_decode(const float* qkv, const float* q_norm_w, const float* k_norm_w, float eps, float rope_base,
+                             float rope_freq_scale, int rope_mode, float* k_cache, float* v_cache, int num_heads, int num_kv_heads,
+                             int head_dim, int max_seq_len, int position, float* partial_ws, float* out, hipStream_t stream)
 {
-    if (head_dim <= 0 || head_dim > kMaxHeadDim || (head_dim & 1)) {
-        set_last_error("layer decode: head_dim must be even and at most 256.");
+    const int total = position + 1;
+    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || total <= 0 || total > max_seq_len) {
+        set_last_error("layer decode: bad head counts or position.");
         return false;
     }
     if (rope_mode != 0 && rope_mode != 2) {
         set_last_error("layer decode: rope mode must be 0 (adjacent pairs) or 2 (NeoX halves).");
         return false;
     }
-    const float theta_scale = powf(rope_base, -2.0f / (float)head_dim);           // ggml-cpu/ops.cpp:5711
-    hipLaunchKernelGGL(qkv_post_kernel, dim3(num_heads + 2 * num_kv_heads), dim3(64), 0, stream, qkv, num_heads, num_kv_heads, head_dim,
-                       q_norm_w, k_norm_w, eps, position, theta_scale, rope_freq_scale, rope_mode == 2 ? 1 : 0, q_out, k_cache,
-                       v_cache, max_seq_len);
-    return hip_ok(hipGetLastError(), "qkv post launch");
-}
-
-bool launch_attention_decode(const float* q, const float* k_cache, const float* v_cache, int num_heads, int num_kv_heads,
-                             int head_dim, int max_seq_len, int total, float* partial_ws, float* out, hipStream_t stream)
-{
-    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || total <= 0 || total > max_seq_len) {
-        set_last_error("layer decode: bad head counts or position.");
-        return false;
-    }
+    AttnFront front{};
+    front.qkv = qkv;
+    front.q_norm_w = q_norm_w;
+    front.k_norm_w = k_norm_w;
+    front.eps = eps;
+    front.theta_scale = powf(rope_base, -2.0f / (float)head_dim);           // ggml-cpu/ops.cpp:5711
+    front.freq_scale = rope_freq_scale;
+    front.neox = rope_mode == 2 ? 1 : 0;
+    front.num_heads = num_heads;
+    front.num_kv_heads = num_kv_heads;
+    front.k_cache = k_cache;
+    front.v_cache = v_cache;
     const int split_len = attn_split_len(total);
     const int splits = (total + split_len - 1) / split_len;
     if (splits > 65535) {
@@ -352,7 +390,7 @@ bool launch_attention_decode(const float* q, const float* k_cache, const float* 
     while (g > 2 && num_kv_heads * splits * (group / g) < 128) g >>= 1;
     const dim3 grid(num_kv_heads, splits, group / g), block(kAttnWaves * 64);
 #define TSHIP_ATTN_LAUNCH(PER, GG)                                                                                              \
-    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, q, k_cache, v_cache, group, max_seq_len, total, split_len, scale, \
+    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, front, group, max_seq_len, total, split_len, scale, \
                        splits, partial_ws, splits == 1 ? out : nullptr)
 #define TSHIP_ATTN_G(PER)                                                    \
     switch (g) {                                                             \

@@ -164,15 +164,13 @@ bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps
 bool launch_silu_mul(const float* gu, int64_t ldgu, int M, int half, float* out, hipStream_t stream);
 
 // ---- single-token attention of the whole-layer decode ---------------------------------------
-// qkv = [q heads | k heads | v heads], head_dim each: per-head RMSNorm (weights may be null) + RoPE; q -> q_out, k / v ->
-// row `position` of the caches [num_kv_heads][max_seq_len][head_dim]
-bool launch_qkv_post(const float* qkv, int num_heads, int num_kv_heads, int head_dim, const float* q_norm_w, const float* k_norm_w,
-                     float eps, int position, float rope_base, float rope_freq_scale, int rope_mode, float* q_out, float* k_cache,
-                     float* v_cache, int max_seq_len, hipStream_t stream);
-// out[h] = softmax(q[h] . K^T / sqrt(head_dim)) V over cache rows [0, total)
+// qkv = [q heads | k heads | v heads], head_dim each.  Per head: RMSNorm (weights may be null) + RoPE at `position`; the
+// new k / v row goes into row `position` of the caches [num_kv_heads][max_seq_len][head_dim];
+// out[h] = softmax(q[h] . K^T / sqrt(head_dim)) V over cache rows [0, position]
 size_t attention_decode_ws_bytes(int num_heads, int total);
-bool launch_attention_decode(const float* q, const float* k_cache, const float* v_cache, int num_heads, int num_kv_heads,
-                             int head_dim, int max_seq_len, int total, float* partial_ws, float* out, hipStream_t stream);
+bool launch_attention_decode(const float* qkv, const float* q_norm_w, const float* k_norm_w, float eps, float rope_base,
+                             float rope_freq_scale, int rope_mode, float* k_cache, float* v_cache, int num_heads, int num_kv_heads,
+                             int head_dim, int max_seq_len, int position, float* partial_ws, float* out, hipStream_t stream);
 
 // ---- MoE (GPT-OSS expert stage) -------------------------------------------------------------
 // ids / weights: [T x k] device; top-k by repeated argmax (first maximum wins), softmax over the k logits.

@@ -139,3 +139,29 @@ def test_layer_decode_argument_errors(hip, oracle):
     with pytest.raises(RuntimeError, match="rope mode"):
         call(mode=8)
     call()
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rope_mode,prefix", [(8, 1, 80, 0, 130), (8, 2, 256, 2, 63), (16, 2, 96, 2, 2100),
+                                                                      (6, 3, 192, 0, 0), (32, 4, 128, 2, 700)])
+def test_head_shapes_groupings_and_split_counts(hip, oracle, heads, kv_heads, head_dim, rope_mode, prefix):
+    # every head width the attention kernel is built for, 1 / 2 / 4 / 8 query heads per workgroup, one to many splits
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(heads * 1000 + head_dim)
+    hidden, inter, max_seq = 256, 512, prefix + 3
+    layer, dims = make_layer(oracle, rng, hidden, heads, kv_heads, head_dim, inter, (Q8_0, Q8_0, Q8_0, Q8_0), True)
+    dev = to_device_layer(layer, torch, QuantizedWeight, dims)
+    kc = np.zeros((kv_heads, max_seq, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    vc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    kd, vd = torch.from_numpy(kc.copy()).cuda(), torch.from_numpy(vc.copy()).cuda()
+    for pos in range(prefix, prefix + 3):
+        h = rng.standard_normal(hidden).astype(np.float32)
+        hd = torch.from_numpy(h.copy()).cuda()
+        oracle.layer_decode(h, layer, kc, vc, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, rope_mode)
+        hip.TransformerLayerDecode(hd, dev["attn_norm"], dev["qkv"], dev["q_norm"], dev["k_norm"], dev["o"], dev["ffn_norm"],
+                                   dev["gate_up"], dev["down"], kd, vd, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, rope_mode)
+        torch.cuda.synchronize()
+        assert rel(hd.cpu().numpy(), h) <= 3e-3, (pos, rel(hd.cpu().numpy(), h))
+        assert rel(kd.cpu().numpy()[:, pos], kc[:, pos]) <= 1e-5 and rel(vd.cpu().numpy()[:, pos], vc[:, pos]) <= 1e-5
