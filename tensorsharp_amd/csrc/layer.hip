@@ -84,6 +84,23 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
     const float* vb = F.v_cache + (int64_t)kvh * max_seq_len * HD;
     const int position = total - 1;
     const bool last = split == splits - 1;                           // the split that holds the new position
+    // kInFlight rows of K and of V per group, all requested before the first is used; the first set is requested
+    // here, ahead of the work on the projections below, which does not depend on it
+    const int t_end = min(total, (split + 1) * split_len);
+    float kr[kInFlight][PER], vr[kInFlight][PER];
+    auto load_rows = [&](int t0) {
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            const int64_t row = (int64_t)min(t0 + 16 * u, t_end - 1) * HD + lg;      // rows past the split: a valid row, unused
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                kr[u][j] = kb[row + 16 * j];
+                vr[u][j] = vb[row + 16 * j];
+            }
+        }
+    };
+    int t0 = split * split_len + grp;
+    load_rows(t0);
 
     // ---- the projections' last steps, per head: RMSNorm over the head (ggml_rms_norm, then * weight), RoPE at
     // `position` (ggml_rope_ext with n_dims = head_dim: ggml-cpu/ops.cpp:5549-5563, :5636-5652).  Every workgroup
@@ -173,22 +190,10 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
             acc[g][j] = 0.f;
         }
     }
-    const int t_end = min(total, (split + 1) * split_len);
-    for (int t0 = split * split_len + grp; t0 < t_end; t0 += 16 * kInFlight) {
-        // kInFlight rows of K and of V per group: every load is issued before the first use
-        float kr[kInFlight][PER], vr[kInFlight][PER];
+    for (; t0 < t_end; t0 += 16 * kInFlight) {
         bool live[kInFlight];
 #pragma unroll
-        for (int u = 0; u < kInFlight; ++u) {
-            const int t = t0 + 16 * u;
-            live[u] = t < t_end;
-            const int64_t row = (int64_t)(live[u] ? t : t0) * HD + lg;
-#pragma unroll
-            for (int j = 0; j < PER; ++j) {
-                kr[u][j] = kb[row + 16 * j];
-                vr[u][j] = vb[row + 16 * j];
-            }
-        }
+        for (int u = 0; u < kInFlight; ++u) live[u] = t0 + 16 * u < t_end;
         if (last) {       // uniform: the new position's row is not in the caches yet (another workgroup may be writing it)
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u) {
@@ -236,6 +241,7 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
             }
             m[g] = mn;
         }
+        if (t0 + 16 * kInFlight < t_end) load_rows(t0 + 16 * kInFlight);
     }
     // the four groups of a wavefront
 #pragma unroll
