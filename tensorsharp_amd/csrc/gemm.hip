@@ -1237,13 +1237,13 @@ int gemm_tile_m(int type, int M, int N)
     const int slim_rows = type == kTypeQ8_0 ? 64 : type == kTypeQ6_K ? 256 : 128;
     if (M <= slim_rows) return 32;
     if ((type == kTypeQ4_K || type == kTypeMXFP4) && M <= 512 && ((M + 127) / 128) * ((N + 127) / 128) <= 128) return 32;
-    // 256-row tiles: above 1024 rows, and from 449 rows when they still give most CUs a tile and pad the rows by at most
-    // 15 % more than 128-row tiles would (measured, Q4_K: 1024 x 14336 x 4096 196 -> 160 us, 512 x 28672 x 4096
+    // 256-row tiles: above 1024 rows, and from 385 rows when they still give most CUs a tile and pad the rows by at most
+    // a quarter more than 128-row tiles would (measured, Q4_K: 1024 x 14336 x 4096 196 -> 160 us, 512 x 28672 x 4096
     // 191 -> 158 us, 512 x 21504 x 5376 188 -> 169 us and Q8_0 232 -> 185 us; but 512 x 5760 x 2880 with its 46 tiles
-    // 52 -> 88 us, and 384 rows no better)
+    // 52 -> 88 us; 600 x 21504 x 5376 with 768 instead of 640 padded rows still 221 -> 198 us; 384 rows no better)
     const int64_t tiles256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
     const int pad256 = (M + 255) / 256 * 256, pad128 = (M + 127) / 128 * 128;
-    return (M > 1024 || (M > 448 && tiles256 >= 160 && pad256 * 100 <= pad128 * 115)) ? 256 : 128;
+    return (M > 1024 || (M > 384 && tiles256 >= 160 && pad256 * 100 <= pad128 * 125)) ? 256 : 128;
 }
 
 namespace {
