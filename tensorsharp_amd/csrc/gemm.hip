@@ -1204,6 +1204,10 @@ bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream
     return false;
 }
 
+// 128-row tiles are 128 x 256 (one workgroup per CU) for these formats, 128 x 128 (two per CU) for the others
+template <typename G>
+constexpr bool kWide128 = G::kSup == 2 || G::kRawRow > 144;
+
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
 {
@@ -1214,7 +1218,7 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
     // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
     // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 and Q6_K the other way round
     if (bm == 128)
-        return (G::kSup == 2 || G::kRawRow > 144) ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream)
+        return kWide128<G> ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream)
                                                    : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream);
     set_last_error("gemm: unsupported tile height.");
     return false;
@@ -1232,18 +1236,41 @@ size_t gemm_workspace_bytes(int M, int K)
 // weights once per 32 rows, but at a much higher rate than the LDS-tiled kernels and mostly out of the memory-side
 // cache, so it wins well past 32 rows (measured crossovers: 4-bit formats about 128 rows, or up to 512 when the
 // big tiles would leave CUs idle; Q8_0 about 64; Q6_K, whose big tiles are limited to 128 rows, about 256).
+namespace {
+bool wide_128_row_tiles(int type)
+{
+    switch (type) {
+    case kTypeQ4_K: return kWide128<GQ4K>;
+    case kTypeMXFP4: return kWide128<GMXFP4>;
+    case kTypeQ8_0: return kWide128<GQ80>;
+    case kTypeQ6_K: return kWide128<GQ6K>;
+    case kTypeQ5_K: return kWide128<GQ5K>;
+    case kTypeQ4_0: return kWide128<GLegacy<kTypeQ4_0>>;
+    case kTypeQ4_1: return kWide128<GLegacy<kTypeQ4_1>>;
+    case kTypeQ5_0: return kWide128<GLegacy<kTypeQ5_0>>;
+    case kTypeQ5_1: return kWide128<GLegacy<kTypeQ5_1>>;
+    default: return kWide128<GLegacy<kTypeIQ4_NL>>;
+    }
+}
+}  // namespace
+
 int gemm_tile_m(int type, int M, int N)
 {
     const int slim_rows = type == kTypeQ8_0 ? 64 : type == kTypeQ6_K ? 256 : 128;
     if (M <= slim_rows) return 32;
     if ((type == kTypeQ4_K || type == kTypeMXFP4) && M <= 512 && ((M + 127) / 128) * ((N + 127) / 128) <= 128) return 32;
-    // 256-row tiles: above 1024 rows, and from 385 rows when they still give most CUs a tile and pad the rows by at most
-    // a quarter more than 128-row tiles would (measured, Q4_K: 1024 x 14336 x 4096 196 -> 160 us, 512 x 28672 x 4096
-    // 191 -> 158 us, 512 x 21504 x 5376 188 -> 169 us and Q8_0 232 -> 185 us; but 512 x 5760 x 2880 with its 46 tiles
-    // 52 -> 88 us; 600 x 21504 x 5376 with 768 instead of 640 padded rows still 221 -> 198 us; 384 rows no better)
+    // 128- or 256-row tiles by rounds of workgroups x time per k-tile of a round (measured per k-tile: a 256 x 256 tile
+    // 2.0 us; two co-resident 128 x 128 tiles of the 4-bit formats 1.37 us; one 128 x 256 tile of the other formats
+    // 1.4 us).  The model reproduces the measured crossovers (Q4_K, us, 128 / 256 rows): 1024 x 14336 x 4096 196 / 160,
+    // 512 x 28672 x 4096 191 / 158, 600 x 21504 x 5376 221 / 198, 512 x 14336 x 4096 94 / 105, MXFP4 512 x 5760 x 2880
+    // 52 / 88.
+    const int cus = device_info().num_cus;
+    const bool two_per_cu = !wide_128_row_tiles(type);                    // 128 x 128 tiles, two workgroups per CU
     const int64_t tiles256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    const int pad256 = (M + 255) / 256 * 256, pad128 = (M + 127) / 128 * 128;
-    return (M > 1024 || (M > 384 && tiles256 >= 160 && pad256 * 100 <= pad128 * 125)) ? 256 : 128;
+    const int64_t tiles128 = (int64_t)((M + 127) / 128) * ((N + (two_per_cu ? 127 : 255)) / (two_per_cu ? 128 : 256));
+    const double t256 = (double)((tiles256 + cus - 1) / cus) * 2.0;
+    const double t128 = (double)((tiles128 + (two_per_cu ? 2 : 1) * cus - 1) / ((two_per_cu ? 2 : 1) * cus)) * (two_per_cu ? 1.37 : 1.4);
+    return t256 < t128 ? 256 : 128;
 }
 
 namespace {
