@@ -858,7 +858,7 @@ inline int pick_k_chunks(int tiles, int nkt, int slots, int64_t out_elems, doubl
     double best_t = (double)((tiles + slots - 1) / slots) * nkt * us_per_ktile;
     for (int sc = 2; sc <= 4; ++sc) {
         const int chunk = ((nkt + sc - 1) / sc + 3) / 4 * 4;
-        if (chunk < 48) break;
+        if (chunk < 32) break;
         const double t = (double)((tiles * sc + slots - 1) / slots) * chunk * us_per_ktile + 2.0 * sc * out_elems * 4 / 4.5e6;
         if (t < 0.9 * best_t) {
             best = sc;
