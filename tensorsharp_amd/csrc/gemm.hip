@@ -1259,6 +1259,8 @@ int gemm_tile_m(int type, int M, int N)
     const int slim_rows = type == kTypeQ8_0 ? 64 : type == kTypeQ6_K ? 256 : 128;
     if (M <= slim_rows) return 32;
     if ((type == kTypeQ4_K || type == kTypeMXFP4) && M <= 512 && ((M + 127) / 128) * ((N + 127) / 128) <= 128) return 32;
+    // the 128 x 256 tiles of the other formats: up to 128 rows when they would be very few (Q8_0 128 x 4096 x 4096: 48 -> 27 us)
+    if (wide_128_row_tiles(type) && M <= 128 && ((M + 127) / 128) * ((N + 255) / 256) <= 32) return 32;
     // 128- or 256-row tiles by rounds of workgroups x time per k-tile of a round (measured per k-tile: a 256 x 256 tile
     // 2.0 us; two co-resident 128 x 128 tiles of the 4-bit formats 1.37 us; one 128 x 256 tile of the other formats
     // 1.4 us).  The model reproduces the measured crossovers (Q4_K, us, 128 / 256 rows): 1024 x 14336 x 4096 196 / 160,
