@@ -99,40 +99,52 @@ def test_unaligned_sub_weight_views(hip, oracle, name):
         check(name, y.cpu().numpy(), ref)
 
 
-@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+def host_case_weight(oracle, name, N, K, rng):
+    """(ggml type, raw blocks) of a random weight in any format with a GEMV kernel."""
+    from oracle.oracle import Q6_K, Q5_K, Q4_0, Q4_1
+    if name in T:
+        return T[name], oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    if name == "q6_k":
+        return Q6_K, q6k_weight(N, K, 35)
+    return {"q5_k": Q5_K, "q4_0": Q4_0, "q4_1": Q4_1}[name], inputs.random_blocks(name, N, K, rng)
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4", "q6_k", "q5_k", "q4_0", "q4_1"])
 def test_host_entry_points(hip, oracle, name):
     """Drop-in path: host pointers, strided activation view, preload key, batch form."""
     rng = np.random.default_rng(35)
     N, K, M = 96, 1024, 3
-    wq = oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    t, wq = host_case_weight(oracle, name, N, K, rng)
+    T_ = dict(T)
+    T_[name] = t
     big = rng.standard_normal((M, K + 40)).astype(np.float32)
     x = big[:, 8:8 + K]                               # row stride K+40, stride1 == 1
-    ref = oracle.matmul_f64(T[name], wq, N, K, np.ascontiguousarray(x))
+    ref = oracle.matmul_f64(T_[name], wq, N, K, np.ascontiguousarray(x))
     out = np.full((M, N + 5), np.nan, dtype=np.float32)
     res = out[:, :N]                                  # strided result view
-    hip.AddmmQuant(res, x, wq.ctypes.data, T[name], K, N, wq.size)
-    check(name, res, ref)
+    hip.AddmmQuant(res, x, wq.ctypes.data, T_[name], K, N, wq.size)
+    check(name if name in RMS_TOL else "q4_k", res, ref)
     assert np.all(np.isnan(out[:, N:]))               # nothing outside the view was written
     # column-strided activations are packed by the shim
     xt = np.asfortranarray(np.ascontiguousarray(x))
     res2 = np.empty((M, N), dtype=np.float32)
-    hip.AddmmQuant(res2, xt, wq.ctypes.data, T[name], K, N, wq.size)
+    hip.AddmmQuant(res2, xt, wq.ctypes.data, T_[name], K, N, wq.size)
     assert np.array_equal(res2, res)
     # preload under an opaque key, then drop the host bytes
     key = 0x7000_0000_1234
     scratch = wq.copy()
-    hip.PreloadQuantizedWeight(key, scratch.ctypes.data, T[name], K, N, scratch.size)
+    hip.PreloadQuantizedWeight(key, scratch.ctypes.data, T_[name], K, N, scratch.size)
     scratch[:] = 0
     res3 = np.empty((M, N), dtype=np.float32)
-    hip.AddmmQuant(res3, np.ascontiguousarray(x), key, T[name], K, N, wq.size)
+    hip.AddmmQuant(res3, np.ascontiguousarray(x), key, T_[name], K, N, wq.size)
     assert np.array_equal(res3, res)
     hip.InvalidateHostBuffer(key)
     # batch form == per-row single calls on sub-weights
-    rs = oracle.row_size(T[name], K)
+    rs = oracle.row_size(T_[name], K)
     n_sub = N // 3
     offs = [0, n_sub * rs, 2 * n_sub * rs]
     resb = np.empty((M, n_sub), dtype=np.float32)
-    hip.AddmmQuantBatch(resb, np.ascontiguousarray(x), wq.ctypes.data, T[name], K, wq.size, offs, [n_sub] * 3)
+    hip.AddmmQuantBatch(resb, np.ascontiguousarray(x), wq.ctypes.data, T_[name], K, wq.size, offs, [n_sub] * 3)
     for b in range(3):
         assert np.array_equal(resb[b], res[b, b * n_sub:(b + 1) * n_sub])
     hip.ClearHostBufferCache()
