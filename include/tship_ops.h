@@ -234,6 +234,36 @@ TSHIP_EXPORT int TSHip_TransformerModelDecodeDevice(float* hidden, int hidden_si
                                                     int num_kv_heads, int max_seq_len, int position, float eps, float rope_base,
                                                     float rope_freq_scale, int intermediate_size, int rope_mode);
 
+/* replaces TSGgml_TransformerLayerDecode with the bridge's own HOST pointers (GgmlNative.cs:518-531; argument list of
+ * ggml_ops_transformer.cpp:572-600).  hidden [hidden_size] travels host -> device -> host on every call.  Every other
+ * buffer - norm weights, raw weight blocks, the two fp32 KV caches - is kept on the device under the host pointer
+ * passed (uploaded the first time that pointer is seen, the protocol of the bridge's cacheable buffers,
+ * ggml_ops_transformer.cpp:244-300).  The device copy of a KV cache is the one this call updates:
+ * TSHip_SyncHostBuffer(k_cache, bytes) copies it back to host memory, TSHip_InvalidateHostBuffer(ptr) drops a device
+ * copy so that the next call uploads the host bytes again (after the caller has edited or truncated the cache).
+ * Synchronous; runs on the default stream. */
+TSHIP_EXPORT int TSHip_TransformerLayerDecode(void* hidden, int hidden_size, void* attn_norm, void* qkv_data, int qkv_type,
+                                              int64_t qkv_ne0, int64_t qkv_ne1, int64_t qkv_bytes, void* q_norm, void* k_norm,
+                                              int head_dim, void* o_data, int o_type, int64_t o_ne0, int64_t o_ne1, int64_t o_bytes,
+                                              void* ffn_norm, void* gu_data, int gu_type, int64_t gu_ne0, int64_t gu_ne1,
+                                              int64_t gu_bytes, void* down_data, int down_type, int64_t down_ne0, int64_t down_ne1,
+                                              int64_t down_bytes, void* k_cache, void* v_cache, int num_heads, int num_kv_heads,
+                                              int max_seq_len, int position, float eps, float rope_base, float rope_freq_scale,
+                                              int intermediate_size, int rope_mode);
+
+/* replaces TSGgml_TransformerModelDecode with HOST pointers (GgmlNative.cs:647-659; ggml_ops_transformer.cpp:1040-1230):
+ * num_layers layers in sequence with ONE round trip of hidden; the arrays hold one host pointer per layer, cached on
+ * the device as above. */
+TSHIP_EXPORT int TSHip_TransformerModelDecode(void* hidden, int hidden_size, int num_layers, void* const* attn_norm,
+                                              void* const* qkv, void* const* q_norm, void* const* k_norm, void* const* o,
+                                              void* const* ffn_norm, void* const* gu, void* const* down, void* const* k_cache,
+                                              void* const* v_cache, int qkv_type, int64_t qkv_ne0, int64_t qkv_ne1,
+                                              int64_t qkv_bytes, int o_type, int64_t o_ne0, int64_t o_ne1, int64_t o_bytes,
+                                              int gu_type, int64_t gu_ne0, int64_t gu_ne1, int64_t gu_bytes, int down_type,
+                                              int64_t down_ne0, int64_t down_ne1, int64_t down_bytes, int head_dim, int num_heads,
+                                              int num_kv_heads, int max_seq_len, int position, float eps, float rope_base,
+                                              float rope_freq_scale, int intermediate_size, int rope_mode);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1270,6 +1270,62 @@ bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm
 
 }  // namespace
 
+// ---- host-pointer forms (the bridge's own argument lists) -------------------------------------
+// hidden travels per call; everything else - norm weights, raw weight blocks, the fp32 KV caches - lives in device
+// buffers kept under the host pointer the caller passes (uploaded on first use, like the bridge's cacheable buffers,
+// ggml_ops_transformer.cpp:244-300).  The device copy of a KV cache is the one that is updated: TSHip_SyncHostBuffer
+// brings it back to host memory, TSHip_InvalidateHostBuffer makes the next call upload the host bytes again.
+namespace {
+struct HostLayer {
+    const float* attn_norm;
+    const void* qkv;
+    const float* q_norm;
+    const float* k_norm;
+    const void* o;
+    const float* ffn_norm;
+    const void* gu;
+    const void* down;
+    float* k_cache;
+    float* v_cache;
+};
+
+bool resolve_layer(const LayerShape& L, void* attn_norm, void* qkv, void* q_norm, void* k_norm, void* o, void* ffn_norm, void* gu,
+                   void* down, void* k_cache, void* v_cache, HostLayer* out)
+{
+    const size_t kv_bytes = (size_t)L.num_kv_heads * L.max_seq_len * L.head_dim * sizeof(float);
+    auto f32 = [](void* p, size_t n) { return p ? static_cast<const float*>(resolve_weight(p, n * sizeof(float))) : nullptr; };
+    out->attn_norm = f32(attn_norm, (size_t)L.hidden);
+    out->ffn_norm = f32(ffn_norm, (size_t)L.hidden);
+    out->q_norm = f32(q_norm, (size_t)L.head_dim);
+    out->k_norm = f32(k_norm, (size_t)L.head_dim);
+    out->qkv = resolve_weight(qkv, (size_t)L.qkv_bytes);
+    out->o = resolve_weight(o, (size_t)L.o_bytes);
+    out->gu = resolve_weight(gu, (size_t)L.gu_bytes);
+    out->down = resolve_weight(down, (size_t)L.down_bytes);
+    out->k_cache = static_cast<float*>(const_cast<void*>(resolve_weight(k_cache, kv_bytes)));
+    out->v_cache = static_cast<float*>(const_cast<void*>(resolve_weight(v_cache, kv_bytes)));
+    return out->attn_norm && out->ffn_norm && (!q_norm || out->q_norm) && (!k_norm || out->k_norm) && out->qkv && out->o && out->gu &&
+           out->down && out->k_cache && out->v_cache;
+}
+
+// hidden: host -> device, `layers` layer steps, device -> host
+template <typename Layers>
+int decode_with_host_hidden(float* hidden, int hidden_size, Layers&& layers)
+{
+    const size_t h_bytes = ((size_t)hidden_size * sizeof(float) + 255) & ~(size_t)255;
+    if (!ws_reserve(h_bytes, h_bytes)) return 0;
+    hipStream_t stream = nullptr;
+    std::memcpy(g_ws.pinned, hidden, (size_t)hidden_size * sizeof(float));
+    if (!hip_ok(hipMemcpyAsync(g_ws.dev, g_ws.pinned, h_bytes, hipMemcpyHostToDevice, stream), "hipMemcpy(hidden)")) return 0;
+    if (!layers(static_cast<float*>(g_ws.dev), stream)) return 0;
+    if (!hip_ok(hipMemcpyAsync(g_ws.pinned, g_ws.dev, h_bytes, hipMemcpyDeviceToHost, stream), "hipMemcpy(hidden)")) return 0;
+    if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+    std::memcpy(hidden, g_ws.pinned, (size_t)hidden_size * sizeof(float));
+    clear_last_error();
+    return 1;
+}
+}  // namespace
+
 extern "C" {
 
 int TSHip_TransformerLayerDecodeDevice(float* hidden, int hidden_size, const float* attn_norm, const void* qkv_data, int qkv_type,
@@ -1329,6 +1385,71 @@ int TSHip_TransformerModelDecodeDevice(float* hidden, int hidden_size, int num_l
         }
         clear_last_error();
         return 1;
+    });
+}
+
+int TSHip_TransformerLayerDecode(void* hidden, int hidden_size, void* attn_norm, void* qkv_data, int qkv_type, int64_t qkv_ne0,
+                                 int64_t qkv_ne1, int64_t qkv_bytes, void* q_norm, void* k_norm, int head_dim, void* o_data, int o_type,
+                                 int64_t o_ne0, int64_t o_ne1, int64_t o_bytes, void* ffn_norm, void* gu_data, int gu_type,
+                                 int64_t gu_ne0, int64_t gu_ne1, int64_t gu_bytes, void* down_data, int down_type, int64_t down_ne0,
+                                 int64_t down_ne1, int64_t down_bytes, void* k_cache, void* v_cache, int num_heads, int num_kv_heads,
+                                 int max_seq_len, int position, float eps, float rope_base, float rope_freq_scale,
+                                 int intermediate_size, int rope_mode)
+{
+    return guarded(0, "transformer_layer_decode", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!hidden || !attn_norm || !qkv_data || !o_data || !ffn_norm || !gu_data || !down_data || !k_cache || !v_cache) {
+            set_last_error("Invalid arguments for transformer layer decode.");
+            return 0;
+        }
+        const LayerShape L{hidden_size, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate_size, qkv_type, o_type, gu_type,
+                           down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
+        if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
+        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        HostLayer d;
+        if (!resolve_layer(L, attn_norm, qkv_data, q_norm, k_norm, o_data, ffn_norm, gu_data, down_data, k_cache, v_cache, &d)) return 0;
+        return decode_with_host_hidden(static_cast<float*>(hidden), hidden_size, [&](float* h, hipStream_t stream) {
+            return run_layer_decode(h, L, d.attn_norm, d.qkv, d.q_norm, d.k_norm, d.o, d.ffn_norm, d.gu, d.down, d.k_cache, d.v_cache,
+                                    position, eps, rope_base, rope_freq_scale, rope_mode, stream);
+        });
+    });
+}
+
+int TSHip_TransformerModelDecode(void* hidden, int hidden_size, int num_layers, void* const* attn_norm, void* const* qkv,
+                                 void* const* q_norm, void* const* k_norm, void* const* o, void* const* ffn_norm, void* const* gu,
+                                 void* const* down, void* const* k_cache, void* const* v_cache, int qkv_type, int64_t qkv_ne0,
+                                 int64_t qkv_ne1, int64_t qkv_bytes, int o_type, int64_t o_ne0, int64_t o_ne1, int64_t o_bytes,
+                                 int gu_type, int64_t gu_ne0, int64_t gu_ne1, int64_t gu_bytes, int down_type, int64_t down_ne0,
+                                 int64_t down_ne1, int64_t down_bytes, int head_dim, int num_heads, int num_kv_heads, int max_seq_len,
+                                 int position, float eps, float rope_base, float rope_freq_scale, int intermediate_size, int rope_mode)
+{
+    return guarded(0, "transformer_model_decode", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!hidden || num_layers <= 0 || !attn_norm || !qkv || !o || !ffn_norm || !gu || !down || !k_cache || !v_cache) {
+            set_last_error("Invalid arguments for transformer model decode.");
+            return 0;
+        }
+        const LayerShape L{hidden_size, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate_size, qkv_type, o_type, gu_type,
+                           down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
+        if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
+        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        std::vector<HostLayer> d((size_t)num_layers);
+        for (int l = 0; l < num_layers; ++l) {
+            if (!attn_norm[l] || !qkv[l] || !o[l] || !ffn_norm[l] || !gu[l] || !down[l] || !k_cache[l] || !v_cache[l]) {
+                set_last_error("transformer model decode: a layer pointer is null.");
+                return 0;
+            }
+            if (!resolve_layer(L, attn_norm[l], qkv[l], q_norm ? q_norm[l] : nullptr, k_norm ? k_norm[l] : nullptr, o[l], ffn_norm[l],
+                               gu[l], down[l], k_cache[l], v_cache[l], &d[(size_t)l]))
+                return 0;
+        }
+        return decode_with_host_hidden(static_cast<float*>(hidden), hidden_size, [&](float* h, hipStream_t stream) {
+            for (const HostLayer& x : d)
+                if (!run_layer_decode(h, L, x.attn_norm, x.qkv, x.q_norm, x.k_norm, x.o, x.ffn_norm, x.gu, x.down, x.k_cache, x.v_cache,
+                                      position, eps, rope_base, rope_freq_scale, rope_mode, stream))
+                    return false;
+            return true;
+        });
     });
 }
 

@@ -243,6 +243,12 @@ class HipBasicOps:
     def ClearHostBufferCache():
         N.lib().TSHip_ClearHostBufferCache()
 
+    @staticmethod
+    def SyncHostBuffer(array):
+        """Copy the device copy kept for this host array (a KV cache the layer decode updates) back into it."""
+        ok = N.lib().TSHip_SyncHostBuffer(C.c_void_p(array.ctypes.data), int(array.nbytes))
+        N.check_result(ok, "sync_host_buffer")
+
     # -- MoE (GptOssModel.MoERoute / MoEForward twins, device tensors) --------------------------
     @staticmethod
     def MoERoute(logits, k):
@@ -275,17 +281,25 @@ class HipBasicOps:
     @staticmethod
     def TransformerLayerDecode(hidden, attn_norm, qkv, q_norm, k_norm, o, ffn_norm, gate_up, down, k_cache, v_cache,
                                num_heads, num_kv_heads, head_dim, position, eps, rope_base, rope_freq_scale=1.0, rope_mode=2):
-        """One token through one layer, in place on `hidden` [hidden_size] (torch CUDA fp32).  qkv / o / gate_up / down are
-        device QuantizedWeights; k_cache / v_cache fp32 [num_kv_heads, max_seq_len, head_dim]; q_norm / k_norm may be None."""
-        HipBasicOps.UseCurrentStream()
-        p = lambda t: None if t is None else t.data_ptr()
-        ok = N.lib().TSHip_TransformerLayerDecodeDevice(
-            hidden.data_ptr(), int(hidden.numel()), attn_norm.data_ptr(),
+        """One token through one layer, in place on `hidden` [hidden_size] fp32.  Either everything is on the device (torch
+        CUDA tensors, device QuantizedWeights; asynchronous on the current stream) or everything is in host memory (numpy
+        arrays, host QuantizedWeights; weights, norms and KV caches are kept on the device under their host address, and
+        SyncHostBuffer(k_cache) brings a cache back).  k_cache / v_cache fp32 [num_kv_heads, max_seq_len, head_dim];
+        q_norm / k_norm may be None."""
+        host = isinstance(hidden, np.ndarray)
+        if host:
+            fn = N.lib().TSHip_TransformerLayerDecode
+        else:
+            HipBasicOps.UseCurrentStream()
+            fn = N.lib().TSHip_TransformerLayerDecodeDevice
+        p = lambda t: None if t is None else HipBasicOps._addr(t)
+        ok = fn(
+            p(hidden), int(hidden.size if host else hidden.numel()), p(attn_norm),
             qkv.ptr, qkv.ggml_type, qkv.ne0, qkv.ne1, qkv.raw_bytes, p(q_norm), p(k_norm), int(head_dim),
-            o.ptr, o.ggml_type, o.ne0, o.ne1, o.raw_bytes, ffn_norm.data_ptr(),
+            o.ptr, o.ggml_type, o.ne0, o.ne1, o.raw_bytes, p(ffn_norm),
             gate_up.ptr, gate_up.ggml_type, gate_up.ne0, gate_up.ne1, gate_up.raw_bytes,
             down.ptr, down.ggml_type, down.ne0, down.ne1, down.raw_bytes,
-            k_cache.data_ptr(), v_cache.data_ptr(), int(num_heads), int(num_kv_heads), int(k_cache.shape[1]), int(position),
+            p(k_cache), p(v_cache), int(num_heads), int(num_kv_heads), int(k_cache.shape[1]), int(position),
             float(eps), float(rope_base), float(rope_freq_scale), int(gate_up.ne1 // 2), int(rope_mode))
         N.check_result(ok, "transformer_layer_decode")
 
@@ -293,23 +307,29 @@ class HipBasicOps:
     def TransformerModelDecode(hidden, layers, num_heads, num_kv_heads, head_dim, position, eps, rope_base, rope_freq_scale=1.0,
                                rope_mode=2):
         """The same for a list of layers; each layer is a dict with the argument names of TransformerLayerDecode
-        (attn_norm, qkv, q_norm, k_norm, o, ffn_norm, gate_up, down, k_cache, v_cache); shapes and types are shared."""
+        (attn_norm, qkv, q_norm, k_norm, o, ffn_norm, gate_up, down, k_cache, v_cache); shapes and types are shared.
+        Host arrays or device tensors throughout, as for TransformerLayerDecode."""
         import ctypes as C
-        HipBasicOps.UseCurrentStream()
+        host = isinstance(hidden, np.ndarray)
+        if host:
+            fn = N.lib().TSHip_TransformerModelDecode
+        else:
+            HipBasicOps.UseCurrentStream()
+            fn = N.lib().TSHip_TransformerModelDecodeDevice
         n = len(layers)
 
         def arr(key, weight=False):
             vals = []
             for L in layers:
                 t = L.get(key)
-                vals.append(None if t is None else (t.ptr if weight else t.data_ptr()))
+                vals.append(None if t is None else (t.ptr if weight else HipBasicOps._addr(t)))
             if all(v is None for v in vals):
                 return None
             return (C.c_void_p * n)(*vals)
         l0 = layers[0]
         qkv, o, gu, dn = l0["qkv"], l0["o"], l0["gate_up"], l0["down"]
-        ok = N.lib().TSHip_TransformerModelDecodeDevice(
-            hidden.data_ptr(), int(hidden.numel()), n, arr("attn_norm"), arr("qkv", True), arr("q_norm"), arr("k_norm"), arr("o", True),
+        ok = fn(
+            HipBasicOps._addr(hidden), int(hidden.size if host else hidden.numel()), n, arr("attn_norm"), arr("qkv", True), arr("q_norm"), arr("k_norm"), arr("o", True),
             arr("ffn_norm"), arr("gate_up", True), arr("down", True), arr("k_cache"), arr("v_cache"),
             qkv.ggml_type, qkv.ne0, qkv.ne1, qkv.raw_bytes, o.ggml_type, o.ne0, o.ne1, o.raw_bytes,
             gu.ggml_type, gu.ne0, gu.ne1, gu.raw_bytes, dn.ggml_type, dn.ne0, dn.ne1, dn.raw_bytes,

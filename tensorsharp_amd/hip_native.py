@@ -98,6 +98,9 @@ SIGNATURES = {
         C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
         C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
 }
+# the host-pointer forms take the same argument lists
+SIGNATURES["TSHip_TransformerLayerDecode"] = SIGNATURES["TSHip_TransformerLayerDecodeDevice"]
+SIGNATURES["TSHip_TransformerModelDecode"] = SIGNATURES["TSHip_TransformerModelDecodeDevice"]
 
 
 def lib():

@@ -1,4 +1,4 @@
-"""GPU parity: whole-layer decode (TSHip_TransformerLayerDecodeDevice / ModelDecodeDevice) against the oracle's restatement
+"""GPU parity: whole-layer decode (TSHip_TransformerLayerDecode / ModelDecode, device and host forms) against the oracle's restatement
 of the bridge's layer graph (ggml_ops_transformer.cpp:379-470) on the same weights, token by token with a growing KV cache.
 
 Bar: ||hidden - ref||_2 <= 3e-3 ||ref||_2 per token (four chained matmuls with fp16 operands, each held to 1e-3 of its
@@ -165,3 +165,89 @@ def test_head_shapes_groupings_and_split_counts(hip, oracle, heads, kv_heads, he
         torch.cuda.synchronize()
         assert rel(hd.cpu().numpy(), h) <= 3e-3, (pos, rel(hd.cpu().numpy(), h))
         assert rel(kd.cpu().numpy()[:, pos], kc[:, pos]) <= 1e-5 and rel(vd.cpu().numpy()[:, pos], vc[:, pos]) <= 1e-5
+
+
+def to_host_layer(layer, QuantizedWeight, dims):
+    d = {k: (None if layer[k] is None else np.ascontiguousarray(layer[k])) for k in ("attn_norm", "q_norm", "k_norm", "ffn_norm")}
+    for k, (ne0, ne1) in dims.items():
+        d[k] = QuantizedWeight(np.ascontiguousarray(layer[k][1]), layer[k][0], ne0, ne1)
+    return d
+
+
+def test_host_pointer_layer_decode_keeps_the_kv_cache_on_the_device(hip, oracle):
+    # the bridge's own argument list: host arrays throughout; the caches come back with SyncHostBuffer
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(113)
+    hidden, heads, kv_heads, head_dim, inter, max_seq, prefix = 512, 8, 2, 64, 1024, 160, 150
+    layer, dims = make_layer(oracle, rng, hidden, heads, kv_heads, head_dim, inter, (Q4_K, Q8_0, Q4_K, Q4_K))
+    host = to_host_layer(layer, QuantizedWeight, dims)
+    kc = np.zeros((kv_heads, max_seq, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    vc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    kh, vh = kc.copy(), vc.copy()
+    step = lambda h, pos: hip.TransformerLayerDecode(h, host["attn_norm"], host["qkv"], host["q_norm"], host["k_norm"], host["o"],
+                                                     host["ffn_norm"], host["gate_up"], host["down"], kh, vh, heads, kv_heads, head_dim,
+                                                     pos, 1e-6, 10000.0, 1.0, 2)
+    try:
+        for pos in range(prefix, prefix + 3):
+            h = rng.standard_normal(hidden).astype(np.float32)
+            got = h.copy()
+            oracle.layer_decode(h, layer, kc, vc, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, 2)
+            step(got, pos)
+            assert rel(got, h) <= 3e-3, (pos, rel(got, h))
+        # the host arrays were not written by the calls; the device copies hold the three new rows
+        assert not kh[:, prefix:].any() and not vh[:, prefix:].any()
+        hip.SyncHostBuffer(kh)
+        hip.SyncHostBuffer(vh)
+        assert np.array_equal(kh[:, :prefix], kc[:, :prefix]) and not kh[:, prefix + 3:].any()
+        assert rel(kh[:, prefix:prefix + 3], kc[:, prefix:prefix + 3]) <= 3e-3
+        assert rel(vh[:, prefix:prefix + 3], vc[:, prefix:prefix + 3]) <= 3e-3
+        # a caller that rewinds the cache on the host: invalidate, and the next call reads the host bytes again
+        kh[:, prefix:] = 0
+        vh[:, prefix:] = 0
+        kc[:, prefix:] = 0
+        vc[:, prefix:] = 0
+        hip.InvalidateHostBuffer(kh.ctypes.data)
+        hip.InvalidateHostBuffer(vh.ctypes.data)
+        h = rng.standard_normal(hidden).astype(np.float32)
+        got = h.copy()
+        oracle.layer_decode(h, layer, kc, vc, heads, kv_heads, head_dim, prefix, 1e-6, 10000.0, 1.0, 2)
+        step(got, prefix)
+        assert rel(got, h) <= 3e-3
+        with pytest.raises(RuntimeError, match="position outside the KV cache"):
+            step(got, max_seq)
+    finally:
+        hip.ClearHostBufferCache()
+
+
+def test_host_pointer_model_decode_equals_the_device_form(hip, oracle):
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(127)
+    hidden, heads, kv_heads, head_dim, inter, max_seq = 512, 4, 2, 128, 768, 6
+    hosts, devs = [], []
+    for li in range(3):
+        layer, dims = make_layer(oracle, rng, hidden, heads, kv_heads, head_dim, inter, (Q8_0, Q8_0, Q8_0, Q8_0), qk_norm=False)
+        hl = to_host_layer(layer, QuantizedWeight, dims)
+        hl["k_cache"] = np.zeros((kv_heads, max_seq, head_dim), np.float32)
+        hl["v_cache"] = np.zeros_like(hl["k_cache"])
+        hosts.append(hl)
+        d = to_device_layer(layer, torch, QuantizedWeight, dims)
+        d["k_cache"] = torch.zeros((kv_heads, max_seq, head_dim), dtype=torch.float32, device="cuda")
+        d["v_cache"] = torch.zeros_like(d["k_cache"])
+        devs.append(d)
+    try:
+        for pos in range(3):
+            h = rng.standard_normal(hidden).astype(np.float32)
+            hd = torch.from_numpy(h.copy()).cuda()
+            hip.TransformerModelDecode(h, hosts, heads, kv_heads, head_dim, pos, 1e-5, 1e6, 1.0, 0)
+            hip.TransformerModelDecode(hd, devs, heads, kv_heads, head_dim, pos, 1e-5, 1e6, 1.0, 0)
+            torch.cuda.synchronize()
+            assert np.array_equal(h, hd.cpu().numpy()), pos          # same kernels, same launch shapes: same bits
+        for hl, d in zip(hosts, devs):
+            hip.SyncHostBuffer(hl["k_cache"])
+            hip.SyncHostBuffer(hl["v_cache"])
+            assert np.array_equal(hl["k_cache"], d["k_cache"].cpu().numpy()) and np.array_equal(hl["v_cache"], d["v_cache"].cpu().numpy())
+    finally:
+        hip.ClearHostBufferCache()
