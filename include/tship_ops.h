@@ -9,15 +9,18 @@
  *     (thread-local, valid until the next call on that thread) — except
  *     TSHip_DequantizeToF32*, which keeps the bridge's 0 / -1 / -2 codes;
  *   - nothing throws across the boundary; the caller owns every buffer.
- * Matmul weight types: Q8_0 (8), Q4_K (12), Q6_K (14), MXFP4 (39).  Dequantize / row gather additionally read F16 (1),
- * Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q5_K (13), IQ4_NL (20), BF16 (30): the block formats of ManagedQuantizedOps.cs:40-59
- * (ids: TensorSharp.Runtime/GgufReader.cs:26-37).
+ * Matmul weight types: Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), IQ4_NL (20),
+ * MXFP4 (39) - the block formats of ManagedQuantizedOps.cs:40-59 without Q8_1.  Dequantize / row gather additionally
+ * read F16 (1) and BF16 (30).  (ids: TensorSharp.Runtime/GgufReader.cs:26-37)
  *
  * Two families:
  *   host-pointer entry points   drop-in for the bridge (activations/results in host
  *                               memory, weights device-resident after preload);
  *   *Device entry points        same contracts with every pointer in device memory;
  *                               pure kernel launches on the stream set by TSHip_SetStream.
+ * Concurrency: host-pointer entry points serialise on one lock.  The *Device entry points share one process-wide
+ * stream setting and one grow-only scratch buffer, so they are ordered by that stream: issue them from one thread at
+ * a time and do not let calls on two different streams overlap.
  */
 #ifndef TSHIP_OPS_H
 #define TSHIP_OPS_H

@@ -823,7 +823,7 @@ struct Step {
 // KS: wavefronts that share a row group, each taking 1/KS of its steps (few rows, long K: one group per wavefront would
 // leave most wavefronts without work); their sums meet in LDS.  KS = 1 is the plain scheme.
 template <typename F, int ACT, int KS>
-__device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, bool strict, uint32_t* lds)
+__device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, int mode, uint32_t* lds)
 {
     const int lane = threadIdx.x & 63;
     constexpr int LPR = F::kLPR, RPG = 64 / LPR;     // lanes per row, rows per group
@@ -988,11 +988,20 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             ++fr;
         }
     };
+    // deep: two steps requested before x is staged and two in flight afterwards.  Only the activation modes use it
+    // (their staging takes longer, and they are the short dependent launches of a decode step: fused FFN 33.9 -> 32.2 us,
+    // whole layer 66.5 -> 64.0 us in an A/B on one box; plain launches lose, 4096 x 14336 12.7 -> 14.2 us).
+    const bool strict = mode == 1, deep = ACT != kActPlain && !strict;
     if constexpr (KS > 1) {
         fetch_next(cur);
+        if (deep) fetch_next(nxt);
     } else {
         fetch(fgroup, fstep, cur);
         advance(fgroup, fstep);
+        if (deep) {
+            fetch(fgroup, fstep, nxt);
+            advance(fgroup, fstep);
+        }
     }
     stage_issue(0);
     stage_commit(0);
@@ -1007,13 +1016,19 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     if constexpr (KS > 1) {
         // Every wavefront of the workgroup runs every round (groups past the end read zeros), so the barrier is uniform.
         float* part = reinterpret_cast<float*>(red + kWaves);        // [2][kWaves][4]
+        bool flip = false;                                            // which buffer holds the step to consume
         for (int r = 0; r < rounds; ++r) {
             float acc = 0.f;
+            auto one = [&](Step<F>& a, Step<F>& b) {
+                if (!deep) fetch_next(b);
+                const uint32_t* xu = lds + lds_lane + (uint32_t)a.step * (uint32_t)(LPR * F::kLdsDwords);
+                acc += F::dot(a.w, L, a.aux, xu);
+                if (deep) fetch_next(a);
+            };
             for (int st = s_begin; st < s_end; ++st) {
-                fetch_next(nxt);
-                const uint32_t* xu = lds + lds_lane + (uint32_t)cur.step * (uint32_t)(LPR * F::kLdsDwords);
-                acc += F::dot(cur.w, L, cur.aux, xu);
-                cur = nxt;
+                if (flip) one(nxt, cur);
+                else one(cur, nxt);
+                flip = !flip;
             }
             const float t = row_sum<LPR>(acc);
             float* pr = part + (r & 1) * kWaves * 4;
@@ -1047,17 +1062,23 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // (strict / not): 123 MB grouped Q4_K launch 24.4 / 25.9 us, 559 MB Q8_0 matrix 92.0 / 98.7 us, but the fused
     // FFN's two launches (66 + 33 MB) 31.7 / 30.6 us and a whole layer 67.1 / 65.8 us: long launches that saturate
     // HBM lose bandwidth when requests run ahead, short ones gain from the extra overlap.
+    auto one = [&](Step<F>& a, Step<F>& b) {
+        if (strict) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (!deep) {
+            fetch(fgroup, fstep, b);
+            advance(fgroup, fstep);
+        }
+        consume(a);
+        if (deep) {
+            fetch(fgroup, fstep, a);
+            advance(fgroup, fstep);
+        }
+    };
     for (;;) {
         if (cur.group >= ngroups) break;
-        if (strict) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        fetch(fgroup, fstep, nxt);
-        advance(fgroup, fstep);
-        consume(cur);
+        one(cur, nxt);
         if (nxt.group >= ngroups) break;
-        if (strict) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        fetch(fgroup, fstep, cur);
-        advance(fgroup, fstep);
-        consume(nxt);
+        one(nxt, cur);
     }
 }
 
@@ -1071,13 +1092,13 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
         if (j < G.count && (int)blockIdx.x >= G.wg_begin[j]) i = j;
     const int wg = (int)blockIdx.x - G.wg_begin[i];
     const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
-    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
-    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
-    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
-    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
-    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
-    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
-    else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, G.strict != 0, lds);
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
