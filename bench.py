@@ -8,7 +8,7 @@ layer = seven GEMVs, issued through the C ABI as one grouped launch
 256 MB Infinity Cache cannot serve the weights.  `value` is algorithmic GB/s
 (weights + activations + outputs) over the timed region, inputs resident in HBM.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line.
 """
 import argparse
 import ctypes as C
