@@ -254,3 +254,37 @@ def test_more_formats_rows_two_bytes_off(hip, oracle, name, row_bytes):
     y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(dev[row_bytes:], t, K, N - 1))
     torch.cuda.synchronize()
     check(y.cpu().numpy(), oracle.matmul_f64(t, wq[row_bytes:], N - 1, K, x), (name, "view"))
+
+
+@pytest.mark.parametrize("N,K", [(21504, 5376), (5376, 21504)])
+@pytest.mark.parametrize("name", ["q8_0", "q4_k"])
+def test_config5_full_size(hip, oracle, name, N, K):
+    """BASELINE configs[4] at its full size: M = 2048, both the up shape and the transposed down shape.
+    The weights are valid blocks made on the device (a min/max-fit quantizer of N(0, 0.02) values; running the
+    reference's Q4_K quantizer over 115 M weights would take minutes).  Checked: a sample of output rows against the
+    oracle's fp64 product, a GEMM row against the decode GEMV of the same row (two different kernels), exact
+    linearity under a power-of-two scaling of the activations, and finiteness of every output."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight, synth
+    M = 2048
+    dev = torch.device("cuda:0")
+    wd = synth.random_weight(T[name], N, K, dev, seed=500 + N % 7)
+    w = QuantizedWeight(wd, T[name], K, N)
+    g = torch.Generator(device=dev)
+    g.manual_seed(501)
+    x = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32)
+    y = hip.LinearForward(x, w)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y).all())
+    rows = [0, 255, 256, 1023, 2047]
+    wq = wd.cpu().numpy()
+    ref = oracle.matmul_f64(T[name], wq, N, K, x[rows].cpu().numpy())
+    e = check(y[rows].cpu().numpy(), ref, (name, N, K))
+    print("cfg5 %s %dx%dx%d row-L2 err %.2e rms err %.2e" % ((name, M, N, K) + e))
+    # the decode kernel on one of the rows
+    y1 = hip.LinearForward(x[1023:1024].contiguous(), w)
+    check(y1.cpu().numpy(), ref[3:4], (name, "gemv row"))
+    # activations times 4: every row's power-of-two scale absorbs the factor, so the results are exactly 4 y
+    y4 = hip.LinearForward(x * 4.0, w)
+    torch.cuda.synchronize()
+    assert torch.equal(y4, y * 4.0)
