@@ -62,6 +62,28 @@ def cpu_baseline(layer_host, xs_host, n_threads):
             "seconds_per_layer": round(best, 4)}
 
 
+def cpu_reference_ggml(layer_host, xs_host, n_threads):
+    """The reference's own ggml CPU matmul (activations quantized to Q8_K, integer dot products) on the same
+    seven matrices, from the library built out of the reference's sources beside the oracle; None when that
+    library is not there.  Best of 3 passes over one layer."""
+    from oracle.oracle import Reference
+    if not Reference.available():
+        return None
+    ref = Reference()
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for (name, n, k), w, x in zip(LAYER, layer_host, xs_host):
+            ref.mul_mat(Q4_K, w, n, k, x, threads=n_threads)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    total = sum(algorithmic_bytes(Q4_K, n, k) for _, n, k in LAYER)
+    return {"value": round(total / best / 1e9, 3), "unit": "GB/s", "cores": n_threads, "kind": "reference",
+            "sample": "one full layer (7 Q4_K GEMVs, 123.0 MB) through ggml's CPU backend as the reference builds it "
+                      "(-O3, no -march), best of 3 passes",
+            "seconds_per_layer": round(best, 4)}
+
+
 def time_region(fn, steps, torch):
     """fn(i) launches step i on the current stream. Returns (event_ms, wall_ms)."""
     e0 = torch.cuda.Event(enable_timing=True)
@@ -346,6 +368,12 @@ def main():
         layer_host = [w.data.cpu().numpy() for w in layers[0]]
         xs_host = [x.cpu().numpy() for x in xs]
         out["cpu_baseline"] = cpu_baseline(layer_host, xs_host, n_threads)
+        try:
+            ggml = cpu_reference_ggml(layer_host, xs_host, n_threads)
+        except (OSError, AssertionError, AttributeError) as e:      # reported beside the port, never required
+            ggml = {"error": str(e)}
+        if ggml is not None:
+            out["cpu_baseline_ggml"] = ggml
 
     print(json.dumps(out))
 
