@@ -954,7 +954,7 @@ int tso_moe_forward(int type, const void* gate_up_w, const float* gate_up_b, con
     int32_t* offs = (int32_t*)malloc(((size_t)E + 1) * sizeof(int32_t));
     int32_t* tmap = (int32_t*)malloc((size_t)A * sizeof(int32_t));
     float* wmap = (float*)malloc((size_t)A * sizeof(float));
-    int32_t* emap = (int32_t*)malloc((size_t)A * sizeof(int32_t));
+    int32_t* emap = (int32_t*)malloc((size_t)(A > E ? A : E) * sizeof(int32_t));   /* T > 1 lists all E experts */
     int groups;
     if (T == 1) {
         groups = k;

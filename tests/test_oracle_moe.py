@@ -71,3 +71,17 @@ def test_grouped_forward_equals_per_token_loop(oracle):
     for t in range(T):
         one = oracle.moe_forward(MXFP4, gu_w, gu_b, dn_w, dn_b, E, H, F, hidden[t:t + 1], ids[t:t + 1], wts[t:t + 1])
         np.testing.assert_allclose(one[0], full[t], rtol=1e-5, atol=1e-6)
+
+
+def test_more_experts_than_assignments(oracle):
+    # T > 1 visits all E experts even when fewer (token, expert) pairs exist; most experts stay empty
+    rng = np.random.default_rng(14)
+    E, H, F, T, k = 64, 32, 32, 3, 1
+    gu_w = oracle.quantize(MXFP4, (rng.standard_normal(E * 2 * F * H) * 0.05).astype(np.float32))
+    dn_w = oracle.quantize(MXFP4, (rng.standard_normal(E * H * F) * 0.05).astype(np.float32))
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    full = oracle.moe_forward(MXFP4, gu_w, None, dn_w, None, E, H, F, hidden, ids, wts)
+    for t in range(T):
+        one = oracle.moe_forward(MXFP4, gu_w, None, dn_w, None, E, H, F, hidden[t:t + 1], ids[t:t + 1], wts[t:t + 1])
+        np.testing.assert_allclose(one[0], full[t], rtol=1e-5, atol=1e-6)
