@@ -123,6 +123,20 @@ TSHIP_EXPORT int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensor
                                            int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1,
                                            int64_t m2_raw_bytes);
 
+/* No counterpart in the reference.  TSHip_AddmmQuantF32Device for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same kernels and the same
+ * results, but the scratch of the prefill path (fp16 activations + row scales, sums of K chunks) lives in a static
+ * device array of TSHIP_NO_ALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends; the
+ * call makes no hipMalloc / hipFree.  A call whose converted activations (about 2 bytes per activation + 4 per row)
+ * exceed the array fails with an error; when only the sums of K chunks do not fit, the launch runs with whole K per
+ * tile (results then agree with TSHip_AddmmQuantF32Device to fp32 summation order) or, for the shapes that cannot
+ * do without chunks (at most 128 rows with K > 4096 ... 32768 depending on the format), fails with an error.
+ * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+#define TSHIP_NO_ALLOC_SCRATCH_BYTES (64u << 20)
+TSHIP_EXPORT int TSHip_AddmmQuantF32DeviceNoAlloc(TSHipTensorView2D result, TSHipTensorView2D m1, const void* m2_data,
+                                                  int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1,
+                                                  int64_t m2_raw_bytes);
+
 /* No counterpart in the bridge: the reference issues one AddmmQuant per projection from C#
  * (ModelBase.LinearForward, TensorSharp.Models/ModelBase.cs:875-905).  `count` independent
  * AddmmQuantF32Device problems of one block type; when every problem is a decode GEMV (M == 1) and

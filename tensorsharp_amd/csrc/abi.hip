@@ -269,7 +269,8 @@ size_t matmul_ws_bytes(int type, int M, int64_t K, bool norm)
 // result (+)= f(m1) * W^T with f = identity or RMSNorm(eps) * norm_w.  All pointers are device pointers; `ws` has
 // matmul_ws_bytes() bytes.
 bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
-                          int64_t N, hipStream_t stream, void* ws, const float* norm_w, float eps, bool accumulate)
+                          int64_t N, hipStream_t stream, void* ws, const float* norm_w, float eps, bool accumulate,
+                          void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0)
 {
     const size_t w_bytes = row_size(type, K) * (size_t)N;
     if (!check_device_operands(m1, w, type)) return false;
@@ -300,7 +301,7 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
     // prefill: activations -> fp16 workspace, then the MFMA GEMM
     if (!launch_convert_x(type, static_cast<const float*>(m1.data), m1.stride0, nullptr, M, (int)K, ws, stream, norm_w, eps)) return false;
     return launch_gemm(type, w, (int64_t)w_bytes, ws, static_cast<float*>(result.data), result.stride0, nullptr, M, (int)N,
-                       (int)K, nullptr, stream, accumulate);
+                       (int)K, nullptr, stream, accumulate, chunk_ws, chunk_ws_bytes);
 }
 
 bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
@@ -313,6 +314,35 @@ bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D&
         if (!ws) return false;
     }
     return run_matmul_device_ws(result, m1, w, type, K, N, stream, ws, nullptr, 0.f, false);
+}
+
+// ---- static device scratch of the entry point that allocates nothing ---------------------------
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.  In
+// host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use is looked up
+// once per device and kept in g_scratch_ptr.
+constexpr size_t kScratchBytes = (size_t)TSHIP_NO_ALLOC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device (looked up on the first call per device)
+unsigned char* scratch_ptr()
+{
+    int dev = 0;
+    if (!hip_ok(hipGetDevice(&dev), "current device")) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        set_last_error("Device index out of range for the static scratch buffer.");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (!hip_ok(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+    }
+    return g_scratch_ptr[dev];
 }
 
 // FFN of the fused entry points on device operands (ggml_ops_fused.cpp:390-640):
@@ -679,6 +709,35 @@ int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D m1, co
             return 0;
         }
         if (!run_matmul_device(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load())) return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_AddmmQuantF32DeviceNoAlloc(TSHipTensorView2D result, TSHipTensorView2D m1, const void* m2_data, int m2_ggml_type,
+                                     int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes)
+{
+    return guarded(0, "addmm_quant", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_addmm_quant(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes)) return 0;
+        if (!is_standard_view(result) || m1.stride1 != 1) {
+            set_last_error("Device addmm_quant needs stride1 == 1 views.");
+            return 0;
+        }
+        // [converted activations + row scales][sums of K chunks]: both live in the static array
+        const size_t need = matmul_ws_bytes(m2_ggml_type, m1.dim0, m2_ne0, false);
+        if (need > kScratchBytes) {
+            set_last_error("addmm_quant (no-alloc): the converted activations of this call (" + std::to_string(need) +
+                           " bytes) exceed the static scratch buffer of " + std::to_string(kScratchBytes) +
+                           " bytes; use fewer rows per call or TSHip_AddmmQuantF32Device.");
+            return 0;
+        }
+        unsigned char* ws = scratch_ptr();
+        if (!ws) return 0;
+        // need == 0: the decode GEMV uses no scratch, but a non-null chunk buffer keeps the matmul from allocating
+        if (!run_matmul_device_ws(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load(), ws, nullptr, 0.f, false,
+                                  ws + need, kScratchBytes - need))
+            return 0;
         clear_last_error();
         return 1;
     });

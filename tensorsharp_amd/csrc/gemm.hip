@@ -632,6 +632,18 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
 }
 
 float* chunk_buffer(size_t bytes);
+// K-chunk sums go to the caller's buffer when one is given (`fixed`: nothing is allocated; a launch that needs more
+// either runs with whole K or fails), else to the grow-only buffer above.
+struct ChunkScratch {
+    float* ptr;
+    size_t bytes;
+    bool fixed;
+};
+inline float* chunk_scratch(const ChunkScratch& cs, size_t bytes)
+{
+    if (!cs.fixed) return chunk_buffer(bytes);
+    return bytes <= cs.bytes ? cs.ptr : nullptr;
+}
 __global__ void gemm_chunk_sum_kernel(const float* __restrict__ partial, int k_chunks, int M, int N, const int* __restrict__ c_rows,
                                       float* __restrict__ c, int64_t ldc, int accumulate);
 
@@ -869,7 +881,7 @@ inline int pick_k_chunks(int tiles, int nkt, int slots, int64_t out_elems, doubl
 }
 
 template <typename G, int BM, int XST, int NW>
-bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
+bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
     constexpr int BN = NW * 32, RT = BN * G::kRawRow;
     auto kern = gemm_kernel<G, BM, XST, NW>;
@@ -890,8 +902,15 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream)
         if (a.k_chunks > 1) {
             a.chunk_kt = ((nkt + a.k_chunks - 1) / a.k_chunks + 3) / 4 * 4;
             a.k_chunks = (nkt + a.chunk_kt - 1) / a.chunk_kt;
-            a.partial = chunk_buffer((size_t)a.k_chunks * a.M * a.N * sizeof(float));
-            if (!a.partial) return false;
+            a.partial = chunk_scratch(cs, (size_t)a.k_chunks * a.M * a.N * sizeof(float));
+            if (!a.partial && cs.fixed) {
+                // the caller's scratch is too small for the chunk sums: whole K per tile (slower, same result up to
+                // fp32 summation order)
+                a.k_chunks = 1;
+                a.chunk_kt = (nkt + 3) / 4 * 4;
+            } else if (!a.partial) {
+                return false;
+            }
         }
     }
     const int total = a.m_tiles * a.n_tiles * a.k_chunks;
@@ -1143,7 +1162,7 @@ float* chunk_buffer(size_t bytes)
 }
 
 template <typename G, int KTW>
-bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream)
+bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
     using L = SlimLayout<G, KTW>;
     auto kern = gemm_slim_kernel<G, KTW>;
@@ -1157,8 +1176,11 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream)
     a.partial = nullptr;
     const bool two_pass = a.k_chunks > 1 || a.accumulate;
     if (two_pass) {
-        a.partial = chunk_buffer((size_t)a.k_chunks * a.M * a.N * sizeof(float));
-        if (!a.partial) return false;
+        a.partial = chunk_scratch(cs, (size_t)a.k_chunks * a.M * a.N * sizeof(float));
+        if (!a.partial) {
+            if (cs.fixed) set_last_error("gemm: the K-chunk sums of this shape do not fit the caller's scratch buffer.");
+            return false;
+        }
     }
     const int64_t units = (int64_t)m_tiles * a.k_chunks * a.n_tiles;
     const int grid = (int)std::min<int64_t>(units, device_info().num_cus);
@@ -1190,16 +1212,16 @@ int slim_ktw(int nkt)
 }
 
 template <typename G>
-bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream)
+bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
     if constexpr (G::kTileStep == 2) {
-        if (ktw == 2) return launch_slim<G, 2>(a, m_tiles, stream);
+        if (ktw == 2) return launch_slim<G, 2>(a, m_tiles, stream, cs);
         if constexpr (slim_fits<G, 6>())
-            if (ktw == 6) return launch_slim<G, 6>(a, m_tiles, stream);
+            if (ktw == 6) return launch_slim<G, 6>(a, m_tiles, stream, cs);
     }
-    if (ktw == 4) return launch_slim<G, 4>(a, m_tiles, stream);
+    if (ktw == 4) return launch_slim<G, 4>(a, m_tiles, stream, cs);
     if constexpr (slim_fits<G, 8>())
-        if (ktw == 8) return launch_slim<G, 8>(a, m_tiles, stream);
+        if (ktw == 8) return launch_slim<G, 8>(a, m_tiles, stream, cs);
     set_last_error("gemm: no register-resident kernel for this K.");
     return false;
 }
@@ -1209,17 +1231,17 @@ template <typename G>
 constexpr bool kWide128 = G::kSup == 2 || G::kRawRow > 144;
 
 template <typename G>
-bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream)
+bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
-    if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream);
+    if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream, cs);
     if constexpr (2 * 256 * kXRow + 2 * 256 * G::kRawRow + 1024 <= 160 * 1024) {
-        if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream);
+        if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream, cs);
     }
     // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
     // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 and Q6_K the other way round
     if (bm == 128)
-        return kWide128<G> ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream)
-                                                   : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream);
+        return kWide128<G> ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream, cs)
+                                                   : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream, cs);
     set_last_error("gemm: unsupported tile height.");
     return false;
 }
@@ -1333,8 +1355,10 @@ bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, 
 }
 
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
-                 int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate)
+                 int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, void* chunk_ws,
+                 size_t chunk_ws_bytes)
 {
+    const ChunkScratch cs{static_cast<float*>(chunk_ws), chunk_ws_bytes, chunk_ws != nullptr};
     if (w_bytes >= ((int64_t)1 << 31) - 64 && !tiles) {
         set_last_error("gemm: a single weight of 2 GiB or more must be split by rows.");
         return false;
@@ -1372,16 +1396,16 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     }
     if (m_tiles == 0) return true;
     switch (type) {
-    case kTypeQ4_K: return launch_for_type<GQ4K>(a, bm, m_tiles, stream);
-    case kTypeMXFP4: return launch_for_type<GMXFP4>(a, bm, m_tiles, stream);
-    case kTypeQ8_0: return launch_for_type<GQ80>(a, bm, m_tiles, stream);
-    case kTypeQ6_K: return launch_for_type<GQ6K>(a, bm, m_tiles, stream);
-    case kTypeQ5_K: return launch_for_type<GQ5K>(a, bm, m_tiles, stream);
-    case kTypeQ4_0: return launch_for_type<GLegacy<kTypeQ4_0>>(a, bm, m_tiles, stream);
-    case kTypeQ4_1: return launch_for_type<GLegacy<kTypeQ4_1>>(a, bm, m_tiles, stream);
-    case kTypeQ5_0: return launch_for_type<GLegacy<kTypeQ5_0>>(a, bm, m_tiles, stream);
-    case kTypeQ5_1: return launch_for_type<GLegacy<kTypeQ5_1>>(a, bm, m_tiles, stream);
-    case kTypeIQ4_NL: return launch_for_type<GLegacy<kTypeIQ4_NL>>(a, bm, m_tiles, stream);
+    case kTypeQ4_K: return launch_for_type<GQ4K>(a, bm, m_tiles, stream, cs);
+    case kTypeMXFP4: return launch_for_type<GMXFP4>(a, bm, m_tiles, stream, cs);
+    case kTypeQ8_0: return launch_for_type<GQ80>(a, bm, m_tiles, stream, cs);
+    case kTypeQ6_K: return launch_for_type<GQ6K>(a, bm, m_tiles, stream, cs);
+    case kTypeQ5_K: return launch_for_type<GQ5K>(a, bm, m_tiles, stream, cs);
+    case kTypeQ4_0: return launch_for_type<GLegacy<kTypeQ4_0>>(a, bm, m_tiles, stream, cs);
+    case kTypeQ4_1: return launch_for_type<GLegacy<kTypeQ4_1>>(a, bm, m_tiles, stream, cs);
+    case kTypeQ5_0: return launch_for_type<GLegacy<kTypeQ5_0>>(a, bm, m_tiles, stream, cs);
+    case kTypeQ5_1: return launch_for_type<GLegacy<kTypeQ5_1>>(a, bm, m_tiles, stream, cs);
+    case kTypeIQ4_NL: return launch_for_type<GLegacy<kTypeIQ4_NL>>(a, bm, m_tiles, stream, cs);
     default: set_last_error("gemm: unsupported type."); return false;
     }
 }

@@ -154,8 +154,12 @@ struct GemmTiles {
 
 // c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
 // accumulate: c[row] += ... instead of c[row] = ...
+// chunk_ws (device, optional): where the sums of K chunks go; with it the launch allocates nothing (a shape whose
+// chunk sums do not fit runs with whole K per tile, or fails when the kernel cannot do without chunks).  Without it
+// they go to a grow-only buffer of the library.
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc,
-                 const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate = false);
+                 const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate = false,
+                 void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0);
 
 // ---- fused wrappers around the matmul (RMSNorm prologue, SiLU-gated FFN) ------------------------
 // out[m, 0..K) = x[m] / sqrt(mean(x[m]^2) + eps) * w   (ggml_rms_norm then ggml_mul), contiguous rows

@@ -192,6 +192,15 @@ class HipBasicOps:
         N.check_result(ok, "addmm_quant")
 
     @staticmethod
+    def AddmmQuantDeviceNoAlloc(result, m1, weight_data, ggml_type, ne0, ne1, raw_bytes):
+        """AddmmQuantDevice for callers that cannot allocate device memory: scratch lives in a static device array."""
+        rv = _device_view(result)
+        mv = _device_view(m1)
+        ok = N.lib().TSHip_AddmmQuantF32DeviceNoAlloc(rv, mv, C.c_void_p(weight_data), int(ggml_type), int(ne0), int(ne1),
+                                                      int(raw_bytes))
+        N.check_result(ok, "addmm_quant")
+
+    @staticmethod
     def PrepareGroup(results, m1s, weights):
         """Marshal a list of (result, m1, QuantizedWeight) problems once; returns the argument pack
         that AddmmQuantGroupDevice launches (decode loops reuse the pack every token)."""

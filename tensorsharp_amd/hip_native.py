@@ -56,6 +56,8 @@ SIGNATURES = {
     "TSHip_DequantizeToF32Device": (C.c_int, [C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "TSHip_AddmmQuantF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64,
                                             C.c_int64]),
+    "TSHip_AddmmQuantF32DeviceNoAlloc": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64,
+                                                   C.c_int64]),
     "TSHip_AddmmQuantGroupF32Device": (C.c_int, [C.c_int, C.POINTER(TensorView2D), C.POINTER(TensorView2D),
                                                  C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int64),
                                                  C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
