@@ -18,9 +18,11 @@
  *                               memory, weights device-resident after preload);
  *   *Device entry points        same contracts with every pointer in device memory;
  *                               pure kernel launches on the stream set by TSHip_SetStream.
- * Concurrency: host-pointer entry points serialise on one lock.  The *Device entry points share one process-wide
- * stream setting and one grow-only scratch buffer, so they are ordered by that stream: issue them from one thread at
- * a time and do not let calls on two different streams overlap.
+ * Concurrency: host-pointer entry points serialise on one lock (which also orders them against Invalidate / Clear /
+ * Preload, so a device copy is never freed under a running call).  The *Device entry points launch on the calling
+ * THREAD's stream (TSHip_SetStream is per thread) and keep their scratch per stream: threads that use different
+ * streams run concurrently, threads that share a stream are serialised while they enqueue.
+ * Operands beyond 2 GiB (a weight, or the fp16 copy of a call's activations) are cut by rows inside the call.
  */
 #ifndef TSHIP_OPS_H
 #define TSHIP_OPS_H
@@ -92,7 +94,8 @@ TSHIP_EXPORT int TSHip_AddmmQuantF32(TSHipTensorView2D result, TSHipTensorView2D
                                      int m2_ggml_type, int64_t m2_ne0, int64_t m2_ne1, int64_t m2_raw_bytes);
 
 /* replaces TSGgml_AddmmQuantBatchF32 (ggml_ops_matmul.cpp:1370-1401, impl :672-729): row b of m1 times the
- * sub-weight at byte offset weight_offsets[b] with weight_ne1[b] rows -> row b of result. */
+ * sub-weight at byte offset weight_offsets[b] with weight_ne1[b] rows -> the first weight_ne1[b] columns of row b of
+ * result.  m2_data may be a preload key: sub-weights are then served from the device copy of the whole stack. */
 TSHIP_EXPORT int TSHip_AddmmQuantBatchF32(TSHipTensorView2D result, TSHipTensorView2D m1, void* m2_data,
                                           int m2_ggml_type, int64_t m2_ne0, int64_t m2_raw_bytes,
                                           int batch_count, int64_t* weight_offsets, int64_t* weight_ne1_arr);
@@ -103,7 +106,9 @@ TSHIP_EXPORT int TSHip_PreloadQuantizedWeight(void* cache_key, void* host_data, 
                                               int64_t ne1, int64_t raw_bytes);
 
 /* replace TSGgml_InvalidateHostBuffer / TSGgml_ClearHostBufferCache / TSGgml_SyncHostBuffer
- * (ggml_ops_core.cpp:1166-1197). */
+ * (ggml_ops_core.cpp:1166-1197).  SyncHostBuffer copies a device copy made from caller memory back to it; as in the
+ * bridge (ggml_ops_core.cpp:664-684) it succeeds without doing anything for a null pointer, a zero size, a pointer
+ * that was never cached or a preload key, and fails only when `size` exceeds the cached bytes or the copy fails. */
 TSHIP_EXPORT void TSHip_InvalidateHostBuffer(void* ptr);
 TSHIP_EXPORT void TSHip_ClearHostBufferCache(void);
 TSHIP_EXPORT int TSHip_SyncHostBuffer(void* ptr, size_t size);
@@ -111,7 +116,7 @@ TSHIP_EXPORT int TSHip_SyncHostBuffer(void* ptr, size_t size);
 /* ---- device-pointer entry points ---------------------------------------------------- */
 
 /* No counterpart in the bridge (its tensors are host memory): selects the HIP stream the *Device entry
- * points launch on (NULL = default stream).  Process-wide. */
+ * points launch on when called from THIS thread (NULL = default stream, the initial setting of every thread). */
 TSHIP_EXPORT int TSHip_SetStream(void* hip_stream);
 
 /* Device form of TSGgml_DequantizeToF32 (same codes). */

@@ -56,7 +56,8 @@ std::once_flag g_init_once;
 bool g_backend_ready = false;
 std::string g_init_error;
 DeviceInfo g_device_info{256, 64 * 1024};
-std::atomic<hipStream_t> g_stream{nullptr};
+// The stream of the *Device entry points is a property of the calling thread (two host threads can drive two streams).
+thread_local hipStream_t t_stream = nullptr;
 
 bool probe_device(std::string& err, DeviceInfo* info)
 {
@@ -110,8 +111,11 @@ struct CachedWeight {
 std::mutex g_cache_mutex;
 std::unordered_map<const void*, CachedWeight> g_weight_cache;
 
-// Serialises the host-pointer entry points: they share one staging workspace.
-std::mutex g_host_call_mutex;
+// Serialises the host-pointer entry points: they share one staging workspace, and a device copy may only be freed
+// (re-upload at another size, Invalidate, Clear) while no host call is between resolving its weights and the end of its
+// kernels.  Every host entry point takes it before it resolves a weight and holds it until its results are back.
+// Order: g_host_call_mutex, then g_cache_mutex.
+std::recursive_mutex g_host_call_mutex;
 
 struct Workspace {
     void* dev = nullptr;
@@ -121,28 +125,55 @@ struct Workspace {
 };
 Workspace g_ws;
 
-// Scratch of the *Device entry points (converted activations of the prefill GEMM).  Grow-only:
-// after the first call of a given size nothing is allocated any more.
-std::mutex g_dev_ws_mutex;
-void* g_dev_ws = nullptr;
-size_t g_dev_ws_bytes = 0;
+// Scratch of the *Device entry points (converted activations and K-chunk sums of the prefill GEMM, intermediate rows of
+// the fused wrappers, MoE tables): one grow-only buffer PER STREAM, so calls on different streams never share scratch.
+// A call holds its stream's buffer (WsLease) while it enqueues its kernels; since kernels of one stream run in order,
+// two threads that use the same stream are then safe too.  After the first call of a given size on a stream nothing
+// is allocated any more.  Growing waits for the stream's earlier work (it may still use the old buffer).
+struct StreamWs {
+    std::mutex mu;
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+std::mutex g_dev_ws_mutex;                                   // guards the map, not the buffers
+std::unordered_map<hipStream_t, StreamWs*> g_dev_ws;         // entries live until the process ends
 
-void* dev_ws_reserve(size_t bytes)
-{
-    std::lock_guard<std::mutex> lock(g_dev_ws_mutex);
-    if (bytes > g_dev_ws_bytes) {
-        if (g_dev_ws) {
-            if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return nullptr;
-            (void)hipFree(g_dev_ws);
+class WsLease {
+public:
+    WsLease(hipStream_t stream, size_t bytes)
+    {
+        {
+            std::lock_guard<std::mutex> lock(g_dev_ws_mutex);
+            StreamWs*& slot = g_dev_ws[stream];
+            if (!slot) slot = new StreamWs();
+            ws_ = slot;
         }
-        g_dev_ws = nullptr;
-        g_dev_ws_bytes = 0;
-        const size_t want = bytes + bytes / 4;
-        if (!hip_ok(hipMalloc(&g_dev_ws, want), "hipMalloc(gemm workspace)")) return nullptr;
-        g_dev_ws_bytes = want;
+        ws_->mu.lock();
+        if (bytes > ws_->bytes) {
+            if (ws_->ptr) {
+                if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return;
+                (void)hipFree(ws_->ptr);
+            }
+            ws_->ptr = nullptr;
+            ws_->bytes = 0;
+            const size_t want = bytes + bytes / 4;
+            if (!hip_ok(hipMalloc(&ws_->ptr, want), "hipMalloc(device workspace)")) return;
+            ws_->bytes = want;
+        }
+        ptr_ = static_cast<char*>(ws_->ptr);
+        ok_ = bytes == 0 || ptr_ != nullptr;
     }
-    return g_dev_ws;
-}
+    ~WsLease() { ws_->mu.unlock(); }
+    WsLease(const WsLease&) = delete;
+    WsLease& operator=(const WsLease&) = delete;
+    bool ok() const { return ok_; }
+    char* ptr() const { return ptr_; }
+
+private:
+    StreamWs* ws_ = nullptr;
+    char* ptr_ = nullptr;
+    bool ok_ = false;
+};
 
 bool ws_reserve(size_t dev_bytes, size_t pinned_bytes)
 {
@@ -259,61 +290,113 @@ bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
     return true;
 }
 
-// bytes of device workspace one matmul needs (norm: RMSNorm prologue on the activations)
-size_t matmul_ws_bytes(int type, int M, int64_t K, bool norm)
+// ---- one matmul on device operands ------------------------------------------------------------
+// The kernels address a weight, and the converted activations of a launch, with 32-bit offsets.  Larger operands are
+// cut by rows inside the call, as the bridge does when a buffer passes INT_MAX (ggml_ops_matmul.cpp:331-367): weight
+// rows (output columns) in slices below 2 GiB, activation rows in slices whose fp16 copy stays below 2 GiB.
+struct MatmulPlan {
+    bool gemv;            // decode / tiny batch: one bandwidth-bound GEMV per activation row
+    int m_step;           // activation rows per launch
+    int64_t n_step;       // weight rows per launch
+    size_t conv_bytes;    // [row scales][fp16 activations] of one slice of rows (prefill), or the RMSNorm rows (decode)
+    size_t chunk_bytes;   // sums of K chunks of one launch
+    size_t total() const { return conv_bytes + chunk_bytes; }
+};
+
+MatmulPlan plan_matmul(int type, int M, int64_t K, int64_t N, bool norm, bool accumulate)
 {
-    if (M <= 3 && K <= gemv_max_k(type)) return norm ? (((size_t)M * (size_t)K * sizeof(float) + 255) & ~(size_t)255) : 0;
-    return (gemm_workspace_bytes(M, (int)K) + 255) & ~(size_t)255;
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    MatmulPlan p{};
+    const size_t rs = row_size(type, K);
+    p.n_step = N;
+    if (rs * (size_t)N >= (size_t)kMaxOperandBytes) {
+        // slices of whole rows; a multiple of 256 rows keeps every slice's first row as aligned as the tensor itself
+        p.n_step = std::max<int64_t>(256, (int64_t)((size_t)(kMaxOperandBytes - 1) / rs) / 256 * 256);
+    }
+    p.gemv = M <= 3 && K <= gemv_max_k(type);
+    if (p.gemv) {
+        p.m_step = M;
+        // RMSNorm is formed by the GEMV while it stages x (rows up to gemv_rms_max_k()), else by a kernel of its own
+        p.conv_bytes = norm && K > gemv_rms_max_k() ? al((size_t)M * (size_t)K * sizeof(float)) : 0;
+        return p;
+    }
+    const size_t kp = (size_t)((K + 63) / 64) * 64;
+    p.m_step = (int)std::min<int64_t>(M, std::max<int64_t>(256, ((kMaxOperandBytes - 1) / (int64_t)(kp * 2)) / 256 * 256));
+    p.conv_bytes = al(gemm_workspace_bytes(p.m_step, (int)K));
+    // the launches of a call differ only in their last, smaller slices: the first one needs the most
+    p.chunk_bytes = al(gemm_chunk_ws_bytes(type, p.m_step, (int)std::min<int64_t>(N, p.n_step), (int)K, nullptr, accumulate));
+    return p;
+}
+
+// bytes of device workspace one matmul needs (norm: RMSNorm prologue on the activations)
+size_t matmul_ws_bytes(int type, int M, int64_t K, int64_t N, bool norm, bool accumulate)
+{
+    return plan_matmul(type, M, K, N, norm, accumulate).total();
 }
 
 // result (+)= f(m1) * W^T with f = identity or RMSNorm(eps) * norm_w.  All pointers are device pointers; `ws` has
-// matmul_ws_bytes() bytes.
+// ws_bytes >= matmul_ws_bytes() bytes (with fewer, the K-chunk sums are given up first: see launch_gemm).
 bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
-                          int64_t N, hipStream_t stream, void* ws, const float* norm_w, float eps, bool accumulate,
-                          void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0)
+                          int64_t N, hipStream_t stream, void* ws, size_t ws_bytes, const float* norm_w, float eps, bool accumulate)
 {
-    const size_t w_bytes = row_size(type, K) * (size_t)N;
+    const size_t rs = row_size(type, K);
     if (!check_device_operands(m1, w, type)) return false;
     if (norm_w && (reinterpret_cast<uintptr_t>(norm_w) & 15) != 0) {
         set_last_error("The norm weight must be 16-byte aligned on the device.");
         return false;
     }
     const int M = m1.dim0;
-    if (M <= 3 && K <= gemv_max_k(type)) {
-        // decode / tiny batch: one bandwidth-bound GEMV per activation row
+    const MatmulPlan plan = plan_matmul(type, M, K, N, norm_w != nullptr, accumulate);
+    if (plan.conv_bytes > ws_bytes) {
+        set_last_error("matmul: the device workspace is too small for the converted activations.");
+        return false;
+    }
+    const uint8_t* wb = static_cast<const uint8_t*>(w);
+    float* out = static_cast<float*>(result.data);
+    if (plan.gemv) {
         const float* xs = static_cast<const float*>(m1.data);
         int64_t ldx = m1.stride0;
-        // RMSNorm is formed by the GEMV while it stages x (rows up to gemv_rms_max_k()), else by a kernel of its own
         const bool norm_in_gemv = norm_w && K <= gemv_rms_max_k();
         if (norm_w && !norm_in_gemv) {
             if (!launch_rms_norm_rows(xs, ldx, norm_w, eps, M, (int)K, static_cast<float*>(ws), stream)) return false;
             xs = static_cast<const float*>(ws);
             ldx = K;
         }
-        for (int m = 0; m < M; ++m) {
-            float* y = static_cast<float*>(result.data) + (int64_t)m * result.stride0;
-            if (!launch_gemv(type, w, (int64_t)w_bytes, xs + (int64_t)m * ldx, y, (int)N, (int)K, stream, accumulate ? y : nullptr,
-                             norm_in_gemv ? 1 : 0, norm_w, eps))
-                return false;
+        for (int64_t n0 = 0; n0 < N; n0 += plan.n_step) {
+            const int64_t n = std::min<int64_t>(plan.n_step, N - n0);
+            for (int m = 0; m < M; ++m) {
+                float* y = out + (int64_t)m * result.stride0 + n0;
+                if (!launch_gemv(type, wb + (size_t)n0 * rs, (int64_t)(rs * (size_t)n), xs + (int64_t)m * ldx, y, (int)n, (int)K, stream,
+                                 accumulate ? y : nullptr, norm_in_gemv ? 1 : 0, norm_w, eps))
+                    return false;
+            }
         }
         return true;
     }
     // prefill: activations -> fp16 workspace, then the MFMA GEMM
-    if (!launch_convert_x(type, static_cast<const float*>(m1.data), m1.stride0, nullptr, M, (int)K, ws, stream, norm_w, eps)) return false;
-    return launch_gemm(type, w, (int64_t)w_bytes, ws, static_cast<float*>(result.data), result.stride0, nullptr, M, (int)N,
-                       (int)K, nullptr, stream, accumulate, chunk_ws, chunk_ws_bytes);
+    char* chunk_ws = static_cast<char*>(ws) + plan.conv_bytes;
+    const size_t chunk_bytes = ws_bytes - plan.conv_bytes;
+    for (int m0 = 0; m0 < M; m0 += plan.m_step) {
+        const int m = std::min(plan.m_step, M - m0);
+        const float* x = static_cast<const float*>(m1.data) + (int64_t)m0 * m1.stride0;
+        if (!launch_convert_x(type, x, m1.stride0, nullptr, m, (int)K, ws, stream, norm_w, eps)) return false;
+        for (int64_t n0 = 0; n0 < N; n0 += plan.n_step) {
+            const int64_t n = std::min<int64_t>(plan.n_step, N - n0);
+            if (!launch_gemm(type, wb + (size_t)n0 * rs, (int64_t)(rs * (size_t)n), ws, out + (int64_t)m0 * result.stride0 + n0,
+                             result.stride0, nullptr, m, (int)n, (int)K, nullptr, stream, accumulate, chunk_ws, chunk_bytes))
+                return false;
+        }
+    }
+    return true;
 }
 
 bool run_matmul_device(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* w, int type, int64_t K,
                        int64_t N, hipStream_t stream)
 {
-    const size_t need = matmul_ws_bytes(type, m1.dim0, K, false);
-    void* ws = nullptr;
-    if (need) {
-        ws = dev_ws_reserve(need);
-        if (!ws) return false;
-    }
-    return run_matmul_device_ws(result, m1, w, type, K, N, stream, ws, nullptr, 0.f, false);
+    const size_t need = matmul_ws_bytes(type, m1.dim0, K, N, false, false);
+    WsLease ws(stream, need);
+    if (!ws.ok()) return false;
+    return run_matmul_device_ws(result, m1, w, type, K, N, stream, ws.ptr(), need, nullptr, 0.f, false);
 }
 
 // ---- static device scratch of the entry point that allocates nothing ---------------------------
@@ -347,22 +430,28 @@ unsigned char* scratch_ptr()
 
 // FFN of the fused entry points on device operands (ggml_ops_fused.cpp:390-640):
 //   residual += W_down * ( silu(g) * u ),  [g | u] = W_gate_up * (RMSNorm(input) * norm_w)
+// `ws` has ffn_ws_bytes() bytes.
+size_t ffn_ws_bytes(int M, int gu_type, int dn_type, int hidden, int half)
+{
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    return al((size_t)M * 2 * half * sizeof(float)) + al((size_t)M * half * sizeof(float)) +
+           std::max(matmul_ws_bytes(gu_type, M, hidden, 2 * (int64_t)half, true, false), matmul_ws_bytes(dn_type, M, half, hidden, false, true));
+}
+
 bool run_ffn_swiglu_device(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const float* norm_w, float eps,
                            const void* gate_up, int gu_type, const void* down, int dn_type, int hidden, int half,
-                           hipStream_t stream)
+                           hipStream_t stream, char* ws)
 {
     const int M = input.dim0;
     const size_t gu_bytes = ((size_t)M * 2 * half * sizeof(float) + 255) & ~(size_t)255;
     const size_t act_bytes = ((size_t)M * half * sizeof(float) + 255) & ~(size_t)255;
-    const size_t ws1 = matmul_ws_bytes(gu_type, M, hidden, true), ws2 = matmul_ws_bytes(dn_type, M, half, false);
-    char* ws = static_cast<char*>(dev_ws_reserve(gu_bytes + act_bytes + std::max(ws1, ws2)));
-    if (!ws) return false;
+    const size_t mm_bytes = ffn_ws_bytes(M, gu_type, dn_type, hidden, half) - gu_bytes - act_bytes;
     float* gu = reinterpret_cast<float*>(ws);
     float* act = reinterpret_cast<float*>(ws + gu_bytes);
     void* mm_ws = ws + gu_bytes + act_bytes;
     const TSHipTensorView2D gu_view{gu, M, 2 * half, 2 * half, 1, (int64_t)((size_t)M * 2 * half * sizeof(float))};
-    if (!run_matmul_device_ws(gu_view, input, gate_up, gu_type, hidden, 2 * half, stream, mm_ws, norm_w, eps, false)) return false;
-    if (M <= 3 && half <= gemv_max_k(dn_type)) {
+    if (!run_matmul_device_ws(gu_view, input, gate_up, gu_type, hidden, 2 * half, stream, mm_ws, mm_bytes, norm_w, eps, false)) return false;
+    if (M <= 3 && half <= gemv_max_k(dn_type) && row_size(dn_type, half) * (size_t)hidden < (size_t)kMaxOperandBytes) {
         // decode: the down GEMV forms silu(gate) * up while it stages its activations and adds the residual in its store
         if (!check_device_operands(gu_view, down, dn_type)) return false;
         const size_t dn_bytes = row_size(dn_type, half) * (size_t)hidden;
@@ -375,20 +464,25 @@ bool run_ffn_swiglu_device(const TSHipTensorView2D& residual, const TSHipTensorV
     }
     if (!launch_silu_mul(gu, 2 * half, M, half, act, stream)) return false;
     const TSHipTensorView2D act_view{act, M, half, half, 1, (int64_t)((size_t)M * half * sizeof(float))};
-    return run_matmul_device_ws(residual, act_view, down, dn_type, half, hidden, stream, mm_ws, nullptr, 0.f, true);
+    return run_matmul_device_ws(residual, act_view, down, dn_type, half, hidden, stream, mm_ws, mm_bytes, nullptr, 0.f, true);
 }
 
-// device pointer for m2_data: preloaded key, cached host pointer, or upload now
+// Device pointer for m2_data: preloaded key, cached host pointer, or upload now.  The caller holds g_host_call_mutex.
+// Hit rules: a copy made from caller memory on first use is reused only for exactly the same byte count (the bridge's
+// rule, ggml_ops_core.cpp:604-640: a host address reused for a tensor of another size is uploaded again); a preloaded
+// entry serves any view that fits into the bytes it was given (preload takes the caller's raw byte span, which may
+// exceed rows x row size) and is never re-read from the key, which need not be readable memory.
 const void* resolve_weight(void* m2_data, size_t bytes)
 {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_weight_cache.find(m2_data);
     if (it != g_weight_cache.end()) {
-        if (it->second.bytes >= bytes) return it->second.dev;
         if (it->second.preloaded) {
+            if (bytes <= it->second.bytes) return it->second.dev;
             set_last_error("Preloaded quantized weight is smaller than the requested view.");
             return nullptr;
         }
+        if (it->second.bytes == bytes) return it->second.dev;
         (void)hipFree(it->second.dev);
         g_weight_cache.erase(it);
     }
@@ -403,8 +497,22 @@ const void* resolve_weight(void* m2_data, size_t bytes)
     return cw.dev;
 }
 
+// Sub-weight [offset, offset + bytes) of a stacked weight (AddmmQuantBatch): served from the device copy of the whole
+// stack when `base` is a preloaded key or an already cached host pointer that covers the range - a deliberate range
+// hit, the key need not be readable; otherwise the sub-weight is cached under its own host address like any weight.
+const void* resolve_weight_range(void* base, size_t offset, size_t bytes)
+{
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        auto it = g_weight_cache.find(base);
+        if (it != g_weight_cache.end() && offset + bytes <= it->second.bytes) return static_cast<const char*>(it->second.dev) + offset;
+    }
+    return resolve_weight(static_cast<char*>(base) + offset, bytes);
+}
+
+// w_dev_given: the device copy when the caller has resolved the weight already (sub-weights of a stack)
 int addmm_quant_host(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, void* m2_data, int type, int64_t ne0,
-                     int64_t ne1, int64_t raw_bytes)
+                     int64_t ne1, int64_t raw_bytes, const void* w_dev_given = nullptr)
 {
     if (!ensure_backend()) return 0;
     if (!validate_addmm_quant(result, m1, m2_data, type, ne0, ne1, raw_bytes)) return 0;
@@ -415,10 +523,9 @@ int addmm_quant_host(const TSHipTensorView2D& result, const TSHipTensorView2D& m
     const int M = m1.dim0;
     const int64_t K = ne0, N = ne1;
     const size_t w_bytes = row_size(type, K) * (size_t)N;
-    const void* w_dev = resolve_weight(m2_data, w_bytes);
+    std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
+    const void* w_dev = w_dev_given ? w_dev_given : resolve_weight(m2_data, w_bytes);
     if (!w_dev) return 0;
-
-    std::lock_guard<std::mutex> lock(g_host_call_mutex);
     const size_t x_bytes = (size_t)M * K * sizeof(float);
     const size_t y_bytes = (size_t)M * N * sizeof(float);
     const size_t x_off = 0, y_off = (x_bytes + 255) & ~(size_t)255;
@@ -572,7 +679,7 @@ int with_host_tensors(const TSHipTensorView2D& inout, bool upload_inout, const T
         set_last_error("The result / residual tensor must be a standard (stride1 == 1, non-overlapping) view.");
         return 0;
     }
-    std::lock_guard<std::mutex> lock(g_host_call_mutex);
+    std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
     const int M = input.dim0;
     const size_t K = (size_t)input.dim1, N = (size_t)inout.dim1;
     const size_t x_bytes = ((size_t)M * K * sizeof(float) + 255) & ~(size_t)255;
@@ -651,7 +758,7 @@ void TSHip_AlignedFree(void* ptr)
 
 int TSHip_SetStream(void* hip_stream)
 {
-    g_stream.store(static_cast<hipStream_t>(hip_stream));
+    t_stream = static_cast<hipStream_t>(hip_stream);
     clear_last_error();
     return 1;
 }
@@ -664,12 +771,12 @@ int TSHip_DequantizeToF32Device(int ggml_type, const void* src, int64_t num_elem
         if (ggml_type != kTypeF32 && !is_dequant_type(ggml_type)) return -2;
         if (!ensure_backend()) return -1;
         if (ggml_type == kTypeF32)
-            return hip_ok(hipMemcpyAsync(dst, src, (size_t)num_elements * 4, hipMemcpyDeviceToDevice, g_stream.load()),
+            return hip_ok(hipMemcpyAsync(dst, src, (size_t)num_elements * 4, hipMemcpyDeviceToDevice, t_stream),
                           "hipMemcpy")
                        ? 0
                        : -1;
         if (num_elements % block_elems(ggml_type) != 0) return -1;
-        return launch_dequant(ggml_type, src, num_elements, dst, g_stream.load()) ? 0 : -1;
+        return launch_dequant(ggml_type, src, num_elements, dst, t_stream) ? 0 : -1;
     });
 }
 
@@ -687,7 +794,7 @@ int TSHip_DequantizeToF32(int ggml_type, const void* src, int64_t num_elements, 
         if (!ensure_backend()) return -1;
         const size_t in_bytes = row_size(ggml_type, num_elements);
         const size_t out_bytes = (size_t)num_elements * sizeof(float);
-        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
         const size_t out_off = (in_bytes + 255) & ~(size_t)255;
         if (!ws_reserve(out_off + out_bytes, 0)) return -1;
         char* base = static_cast<char*>(g_ws.dev);
@@ -708,7 +815,7 @@ int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D m1, co
             set_last_error("Device addmm_quant needs stride1 == 1 views.");
             return 0;
         }
-        if (!run_matmul_device(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load())) return 0;
+        if (!run_matmul_device(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, t_stream)) return 0;
         clear_last_error();
         return 1;
     });
@@ -725,7 +832,7 @@ int TSHip_AddmmQuantF32DeviceNoAlloc(TSHipTensorView2D result, TSHipTensorView2D
             return 0;
         }
         // [converted activations + row scales][sums of K chunks]: both live in the static array
-        const size_t need = matmul_ws_bytes(m2_ggml_type, m1.dim0, m2_ne0, false);
+        const size_t need = plan_matmul(m2_ggml_type, m1.dim0, m2_ne0, m2_ne1, false, false).conv_bytes;
         if (need > kScratchBytes) {
             set_last_error("addmm_quant (no-alloc): the converted activations of this call (" + std::to_string(need) +
                            " bytes) exceed the static scratch buffer of " + std::to_string(kScratchBytes) +
@@ -734,9 +841,8 @@ int TSHip_AddmmQuantF32DeviceNoAlloc(TSHipTensorView2D result, TSHipTensorView2D
         }
         unsigned char* ws = scratch_ptr();
         if (!ws) return 0;
-        // need == 0: the decode GEMV uses no scratch, but a non-null chunk buffer keeps the matmul from allocating
-        if (!run_matmul_device_ws(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load(), ws, nullptr, 0.f, false,
-                                  ws + need, kScratchBytes - need))
+        // what the converted activations leave of the array takes the sums of K chunks
+        if (!run_matmul_device_ws(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, t_stream, ws, kScratchBytes, nullptr, 0.f, false))
             return 0;
         clear_last_error();
         return 1;
@@ -765,7 +871,7 @@ int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView2D* results, 
             if (!check_device_operands(m1s[i], m2_datas[i], m2_ggml_type)) return 0;
             decode = decode && m1s[i].dim0 == 1 && m2_ne0s[i] <= gemv_max_k(m2_ggml_type);
         }
-        hipStream_t stream = g_stream.load();
+        hipStream_t stream = t_stream;
         if (decode) {
             GemvArgs args[16];
             for (int i = 0; i < count; ++i) {
@@ -797,7 +903,7 @@ int TSHip_MoERouteF32Device(TSHipTensorView2D logits, int k, int32_t* ids, float
             return 0;
         }
         if (!launch_moe_route(static_cast<const float*>(logits.data), logits.stride0, logits.dim0, logits.dim1, k, ids, weights,
-                              g_stream.load()))
+                              t_stream))
             return 0;
         clear_last_error();
         return 1;
@@ -834,7 +940,7 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
         }
         const int A = (int)A64, E = n_experts;
         const int64_t gu_bytes = (int64_t)rs_h * 2 * F, dn_bytes = (int64_t)rs_f * H;   // per expert
-        hipStream_t stream = g_stream.load();
+        hipStream_t stream = t_stream;
         auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
         const bool small = A <= gemv_max_group() && H <= gemv_max_k(ggml_type) && F <= gemv_max_k(ggml_type);
         // rows per tile of the grouped GEMMs: up to about 160 tokens per expert the 32-row register-resident kernel
@@ -850,8 +956,14 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
         const size_t o_trn = take((size_t)max_tiles * 4);
         const size_t o_ws1 = take(gemm_workspace_bytes(A, (int)H)), o_ws2 = take(gemm_workspace_bytes(A, (int)F));
         const size_t o_gu = take((size_t)A * 2 * F * 4), o_dn = take((size_t)A * H * 4);
-        char* ws = static_cast<char*>(dev_ws_reserve(off));
-        if (!ws) return 0;
+        const GemmTiles plan_tiles{nullptr, nullptr, nullptr, max_tiles, bm, 0};
+        const size_t chunk_bytes = small ? 0
+                                         : std::max(gemm_chunk_ws_bytes(ggml_type, A, (int)(2 * F), (int)H, &plan_tiles, false),
+                                                    gemm_chunk_ws_bytes(ggml_type, A, (int)H, (int)F, &plan_tiles, false));
+        const size_t o_chunk = take(chunk_bytes);
+        WsLease lease(stream, off);
+        if (!lease.ok()) return 0;
+        char* ws = lease.ptr();
         float* gu = reinterpret_cast<float*>(ws + o_gu);
         float* dn = reinterpret_cast<float*>(ws + o_dn);
         const float* hid = static_cast<const float*>(hidden.data);
@@ -860,19 +972,19 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
             GemvArgs args[16];
             for (int a = 0; a < A; ++a) {
                 args[a] = GemvArgs{gate_up_w, gu_bytes, hid + (int64_t)(a / k) * hidden.stride0, gu + (int64_t)a * 2 * F,
-                                   (int)(2 * F), (int)H, ids + a, gu_bytes};
+                                   (int)(2 * F), (int)H, ids + a, gu_bytes, E};
             }
             if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
             // the down GEMVs form bias + SwiGLU-OAI from the gate|up rows while they stage their activations
             for (int a = 0; a < A; ++a) {
-                args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * 2 * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes};
+                args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * 2 * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes, E};
                 args[a].act = 3;
                 args[a].norm_w = gate_up_bias;
                 args[a].eps = alpha;
                 args[a].limit = limit;
             }
             if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
-            if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, (int)H, T == 1, static_cast<float*>(result.data),
+            if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, E, (int)H, T == 1, static_cast<float*>(result.data),
                                     result.stride0, stream))
                 return 0;
         } else {
@@ -883,14 +995,17 @@ int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D
             if (!launch_moe_group(ids, A, k, E, bm, max_tiles, maps, stream)) return 0;
             GemmTiles tiles{maps.tile_expert, maps.tile_row0, maps.tile_rows, max_tiles, bm, gu_bytes};
             if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream)) return 0;
-            if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream))
+            if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream, false,
+                             ws + o_chunk, chunk_bytes))
                 return 0;
             // bias + SwiGLU-OAI are formed while the down projection's activations are converted
             if (!launch_convert_x_swiglu(ggml_type, gu, gate_up_bias, maps.expert_of, alpha, limit, A, (int)F, ws + o_ws2, stream))
                 return 0;
             tiles.expert_stride = dn_bytes;
-            if (!launch_gemm(ggml_type, down_w, dn_bytes, ws + o_ws2, dn, H, nullptr, A, (int)H, (int)F, &tiles, stream)) return 0;
-            if (!launch_moe_combine(dn, down_bias, ids, weights, maps.pos_of, T, k, (int)H, false,
+            if (!launch_gemm(ggml_type, down_w, dn_bytes, ws + o_ws2, dn, H, nullptr, A, (int)H, (int)F, &tiles, stream, false,
+                             ws + o_chunk, chunk_bytes))
+                return 0;
+            if (!launch_moe_combine(dn, down_bias, ids, weights, maps.pos_of, T, k, E, (int)H, false,
                                     static_cast<float*>(result.data), result.stride0, stream))
                 return 0;
         }
@@ -934,8 +1049,13 @@ int TSHip_AddmmQuantBatchF32(TSHipTensorView2D result, TSHipTensorView2D m1, voi
                 set_last_error("addmm_quant_batch: sub-weight lies outside the weight bytes.");
                 return 0;
             }
+            if (ne1 > result.dim1) {
+                set_last_error("addmm_quant_batch: a sub-weight has more rows than the result has columns.");
+                return 0;
+            }
             TSHipTensorView2D r = result;
             r.dim0 = 1;
+            r.dim1 = (int)ne1;        // a sub-weight with fewer rows than result.dim1 fills the first ne1 columns of its row
             r.data = static_cast<char*>(result.data) + (size_t)b * result.stride0 * sizeof(float);
             r.raw_bytes = (int64_t)r.dim1 * (int64_t)sizeof(float);
             TSHipTensorView2D x = m1;
@@ -943,7 +1063,10 @@ int TSHip_AddmmQuantBatchF32(TSHipTensorView2D result, TSHipTensorView2D m1, voi
             x.data = static_cast<char*>(m1.data) + (size_t)b * m1.stride0 * sizeof(float);
             x.raw_bytes = (int64_t)required_raw_bytes(x);
             void* sub = static_cast<char*>(m2_data) + off;
-            if (!addmm_quant_host(r, x, sub, m2_ggml_type, m2_ne0, ne1, (int64_t)((size_t)ne1 * rs))) return 0;
+            std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
+            const void* sub_dev = resolve_weight_range(m2_data, (size_t)off, (size_t)ne1 * rs);
+            if (!sub_dev) return 0;
+            if (!addmm_quant_host(r, x, sub, m2_ggml_type, m2_ne0, ne1, (int64_t)((size_t)ne1 * rs), sub_dev)) return 0;
         }
         clear_last_error();
         return 1;
@@ -964,6 +1087,7 @@ int TSHip_PreloadQuantizedWeight(void* cache_key, void* host_data, int ggml_type
             set_last_error("Unsupported type or inconsistent size for quantized weight preload.");
             return 0;
         }
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
         std::lock_guard<std::mutex> lock(g_cache_mutex);
         auto it = g_weight_cache.find(cache_key);
         if (it != g_weight_cache.end()) {
@@ -990,6 +1114,7 @@ int TSHip_PreloadQuantizedWeight(void* cache_key, void* host_data, int ggml_type
 
 void TSHip_InvalidateHostBuffer(void* ptr)
 {
+    std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_weight_cache.find(ptr);
     if (it == g_weight_cache.end()) return;
@@ -999,22 +1124,31 @@ void TSHip_InvalidateHostBuffer(void* ptr)
 
 void TSHip_ClearHostBufferCache(void)
 {
+    std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     for (auto& kv : g_weight_cache) (void)hipFree(kv.second.dev);
     g_weight_cache.clear();
 }
 
+// ggml_ops_core.cpp:664-684: nothing to do (success) for a null pointer, a zero size, a pointer that is not cached or
+// an entry that is not a device copy of caller memory (here: a preloaded key); an error only when more bytes are
+// asked for than the copy holds, or when the copy fails.
 int TSHip_SyncHostBuffer(void* ptr, size_t size)
 {
-    std::lock_guard<std::mutex> lock(g_cache_mutex);
-    auto it = g_weight_cache.find(ptr);
-    if (it == g_weight_cache.end() || it->second.preloaded || ptr == nullptr || size > it->second.bytes) {
-        set_last_error("Failed to synchronize cached HIP device buffer back to host memory.");
-        return 0;
-    }
-    if (!hip_ok(hipMemcpy(ptr, it->second.dev, size, hipMemcpyDeviceToHost), "hipMemcpy(sync)")) return 0;
-    clear_last_error();
-    return 1;
+    return guarded(0, "sync_host_buffer", [&]() -> int {
+        clear_last_error();
+        if (ptr == nullptr || size == 0) return 1;
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        auto it = g_weight_cache.find(ptr);
+        if (it == g_weight_cache.end() || it->second.preloaded) return 1;
+        if (size > it->second.bytes) {
+            set_last_error("Failed to synchronize cached HIP device buffer back to host memory.");
+            return 0;
+        }
+        if (!hip_ok(hipMemcpy(ptr, it->second.dev, size, hipMemcpyDeviceToHost), "hipMemcpy(sync)")) return 0;
+        return 1;
+    });
 }
 
 /* ---- embedding gather ----------------------------------------------------------------- */
@@ -1050,9 +1184,13 @@ int TSHip_GetRowsQuantF32Device(TSHipTensorView2D result, const void* src_data, 
             set_last_error("result must be a standard (stride1 == 1) view in get_rows_quant.");
             return 0;
         }
-        if (!launch_get_rows(src_ggml_type, src_data, (int64_t)rs, src_ne1, indices, num_indices, src_ne0,
-                             static_cast<float*>(result.data), result.stride0, g_stream.load()))
-            return 0;
+        // one launch serves at most 65535 indices (grid dimension): more are served in slices, like the host form
+        for (int64_t i0 = 0; i0 < num_indices; i0 += 65535) {
+            const int64_t cnt = std::min<int64_t>(65535, num_indices - i0);
+            if (!launch_get_rows(src_ggml_type, src_data, (int64_t)rs, src_ne1, indices + i0, cnt, src_ne0,
+                                 static_cast<float*>(result.data) + i0 * result.stride0, result.stride0, t_stream))
+                return 0;
+        }
         clear_last_error();
         return 1;
     });
@@ -1111,10 +1249,10 @@ int TSHip_GetRowsQuantF32(TSHipTensorView2D result, void* src_data, int src_ggml
                 set_last_error("Index out of range in get_rows_quant.");
                 return 0;
             }
+        std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
         const void* w_dev = resolve_weight(src_data, rs * (size_t)src_ne1);
         if (!w_dev) return 0;
 
-        std::lock_guard<std::mutex> lock(g_host_call_mutex);
         const size_t K = (size_t)src_ne0;
         const size_t y_bytes = (size_t)n * K * sizeof(float);
         const size_t id_bytes = ((size_t)n * sizeof(int32_t) + 255) & ~(size_t)255;
@@ -1151,10 +1289,10 @@ int TSHip_FusedRmsNormMatMulQuantF32Device(TSHipTensorView2D result, TSHipTensor
         if (!validate_fused_matmul(result, input, norm_weight, norm_weight_count, true, m2_data, m2_ggml_type, m2_ne0, m2_ne1,
                                    m2_raw_bytes, "fused rms_norm_matmul", "result"))
             return 0;
-        const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, true);
-        void* ws = dev_ws_reserve(std::max<size_t>(need, 256));
-        if (!ws) return 0;
-        if (!run_matmul_device_ws(result, input, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load(), ws, norm_weight, eps, false))
+        const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, m2_ne1, true, false);
+        WsLease ws(t_stream, need);
+        if (!ws.ok()) return 0;
+        if (!run_matmul_device_ws(result, input, m2_data, m2_ggml_type, m2_ne0, m2_ne1, t_stream, ws.ptr(), need, norm_weight, eps, false))
             return 0;
         clear_last_error();
         return 1;
@@ -1169,10 +1307,10 @@ int TSHip_FusedMatMulQuantAddF32Device(TSHipTensorView2D residual, TSHipTensorVi
         if (!validate_fused_matmul(residual, input, nullptr, 0, false, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes,
                                    "fused matmul_add", "residual"))
             return 0;
-        const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, false);
-        void* ws = need ? dev_ws_reserve(need) : nullptr;
-        if (need && !ws) return 0;
-        if (!run_matmul_device_ws(residual, input, m2_data, m2_ggml_type, m2_ne0, m2_ne1, g_stream.load(), ws, nullptr, 0.f, true))
+        const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, m2_ne1, false, true);
+        WsLease ws(t_stream, need);
+        if (!ws.ok()) return 0;
+        if (!run_matmul_device_ws(residual, input, m2_data, m2_ggml_type, m2_ne0, m2_ne1, t_stream, ws.ptr(), need, nullptr, 0.f, true))
             return 0;
         clear_last_error();
         return 1;
@@ -1190,8 +1328,10 @@ int TSHip_FusedFFNSwiGLUQuantF32Device(TSHipTensorView2D residual, TSHipTensorVi
         if (!validate_ffn(residual, input, norm_weight, norm_weight_count, gate_up_data, gate_up_ggml_type, gate_up_ne0,
                           gate_up_ne1, gate_up_raw_bytes, down_data, down_ggml_type, down_ne0, down_ne1, down_raw_bytes, half_dim))
             return 0;
+        WsLease ws(t_stream, ffn_ws_bytes(input.dim0, gate_up_ggml_type, down_ggml_type, input.dim1, half_dim));
+        if (!ws.ok()) return 0;
         if (!run_ffn_swiglu_device(residual, input, norm_weight, eps, gate_up_data, gate_up_ggml_type, down_data, down_ggml_type,
-                                   input.dim1, half_dim, g_stream.load()))
+                                   input.dim1, half_dim, t_stream, ws.ptr()))
             return 0;
         clear_last_error();
         return 1;
@@ -1207,13 +1347,14 @@ int TSHip_FusedRmsNormMatMulQuantF32(TSHipTensorView2D result, TSHipTensorView2D
         if (!validate_fused_matmul(result, input, norm_weight_data, norm_weight_count, true, m2_data, m2_ggml_type, m2_ne0,
                                    m2_ne1, m2_raw_bytes, "fused rms_norm_matmul", "result"))
             return 0;
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
         const void* w = resolve_weight(m2_data, row_size(m2_ggml_type, m2_ne0) * (size_t)m2_ne1);
         if (!w) return 0;
         return with_host_tensors(result, false, input, norm_weight_data, norm_weight_count,
                                  [&](const TSHipTensorView2D& x, const TSHipTensorView2D& y, const float* nw, hipStream_t st) {
-                                     const size_t need = matmul_ws_bytes(m2_ggml_type, x.dim0, m2_ne0, true);
-                                     void* ws = dev_ws_reserve(std::max<size_t>(need, 256));
-                                     return ws && run_matmul_device_ws(y, x, w, m2_ggml_type, m2_ne0, m2_ne1, st, ws, nw, eps, false);
+                                     const size_t need = matmul_ws_bytes(m2_ggml_type, x.dim0, m2_ne0, m2_ne1, true, false);
+                                     WsLease ws(st, need);
+                                     return ws.ok() && run_matmul_device_ws(y, x, w, m2_ggml_type, m2_ne0, m2_ne1, st, ws.ptr(), need, nw, eps, false);
                                  });
     });
 }
@@ -1226,13 +1367,14 @@ int TSHip_FusedMatMulQuantAddF32(TSHipTensorView2D residual, TSHipTensorView2D i
         if (!validate_fused_matmul(residual, input, nullptr, 0, false, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes,
                                    "fused matmul_add", "residual"))
             return 0;
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
         const void* w = resolve_weight(m2_data, row_size(m2_ggml_type, m2_ne0) * (size_t)m2_ne1);
         if (!w) return 0;
         return with_host_tensors(residual, true, input, nullptr, 0,
                                  [&](const TSHipTensorView2D& x, const TSHipTensorView2D& y, const float*, hipStream_t st) {
-                                     const size_t need = matmul_ws_bytes(m2_ggml_type, x.dim0, m2_ne0, false);
-                                     void* ws = need ? dev_ws_reserve(need) : nullptr;
-                                     return (!need || ws) && run_matmul_device_ws(y, x, w, m2_ggml_type, m2_ne0, m2_ne1, st, ws, nullptr, 0.f, true);
+                                     const size_t need = matmul_ws_bytes(m2_ggml_type, x.dim0, m2_ne0, m2_ne1, false, true);
+                                     WsLease ws(st, need);
+                                     return ws.ok() && run_matmul_device_ws(y, x, w, m2_ggml_type, m2_ne0, m2_ne1, st, ws.ptr(), need, nullptr, 0.f, true);
                                  });
     });
 }
@@ -1247,13 +1389,16 @@ int TSHip_FusedFFNSwiGLUQuantF32(TSHipTensorView2D residual, TSHipTensorView2D i
         if (!validate_ffn(residual, input, norm_weight_data, norm_weight_count, gate_up_data, gate_up_ggml_type, gate_up_ne0,
                           gate_up_ne1, gate_up_raw_bytes, down_data, down_ggml_type, down_ne0, down_ne1, down_raw_bytes, half_dim))
             return 0;
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
         const void* gu = resolve_weight(gate_up_data, row_size(gate_up_ggml_type, gate_up_ne0) * (size_t)gate_up_ne1);
         if (!gu) return 0;
         const void* dn = resolve_weight(down_data, row_size(down_ggml_type, down_ne0) * (size_t)down_ne1);
         if (!dn) return 0;
         return with_host_tensors(residual, true, input, norm_weight_data, norm_weight_count,
                                  [&](const TSHipTensorView2D& x, const TSHipTensorView2D& y, const float* nw, hipStream_t st) {
-                                     return run_ffn_swiglu_device(y, x, nw, eps, gu, gate_up_ggml_type, dn, down_ggml_type, x.dim1, half_dim, st);
+                                     WsLease ws(st, ffn_ws_bytes(x.dim0, gate_up_ggml_type, down_ggml_type, x.dim1, half_dim));
+                                     return ws.ok() && run_ffn_swiglu_device(y, x, nw, eps, gu, gate_up_ggml_type, dn, down_ggml_type, x.dim1,
+                                                                             half_dim, st, ws.ptr());
                                  });
     });
 }
@@ -1307,9 +1452,11 @@ bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t b_qkv = al((size_t)qkv_n * 4), b_attn = al((size_t)q_dim * 4);
     const size_t b_part = al(attention_decode_ws_bytes(L.num_heads, position + 1));
-    const size_t b_mm = std::max(matmul_ws_bytes(L.qkv_type, 1, L.hidden, true), matmul_ws_bytes(L.o_type, 1, q_dim, false));
-    char* ws = static_cast<char*>(dev_ws_reserve(b_qkv + b_attn + b_part + b_mm + 256));
-    if (!ws) return false;
+    const size_t b_mm = al(std::max(matmul_ws_bytes(L.qkv_type, 1, L.hidden, qkv_n, true, false), matmul_ws_bytes(L.o_type, 1, q_dim, L.hidden, false, true)));
+    const size_t b_ffn = ffn_ws_bytes(1, L.gu_type, L.down_type, L.hidden, L.intermediate);
+    WsLease lease(stream, b_qkv + b_attn + b_part + b_mm + b_ffn);
+    if (!lease.ok()) return false;
+    char* ws = lease.ptr();
     float* qkv_out = reinterpret_cast<float*>(ws);
     float* attn = reinterpret_cast<float*>(ws + b_qkv);
     float* part = reinterpret_cast<float*>(ws + b_qkv + b_attn);
@@ -1317,14 +1464,15 @@ bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm
     const TSHipTensorView2D h_view{hidden, 1, L.hidden, L.hidden, 1, (int64_t)L.hidden * 4};
     const TSHipTensorView2D qkv_view{qkv_out, 1, qkv_n, qkv_n, 1, (int64_t)qkv_n * 4};
     const TSHipTensorView2D attn_view{attn, 1, q_dim, q_dim, 1, (int64_t)q_dim * 4};
-    if (!run_matmul_device_ws(qkv_view, h_view, qkv, L.qkv_type, L.hidden, qkv_n, stream, mm_ws, attn_norm, eps, false)) return false;
+    if (!run_matmul_device_ws(qkv_view, h_view, qkv, L.qkv_type, L.hidden, qkv_n, stream, mm_ws, b_mm, attn_norm, eps, false)) return false;
     if (!launch_attention_decode(qkv_out, q_norm, k_norm, eps, rope_base, rope_freq_scale, rope_mode, k_cache, v_cache, L.num_heads,
                                  L.num_kv_heads, L.head_dim, L.max_seq_len, position, part, attn, stream))
         return false;
     // hidden += W_o attn
-    if (!run_matmul_device_ws(h_view, attn_view, o, L.o_type, q_dim, L.hidden, stream, mm_ws, nullptr, 0.f, true)) return false;
+    if (!run_matmul_device_ws(h_view, attn_view, o, L.o_type, q_dim, L.hidden, stream, mm_ws, b_mm, nullptr, 0.f, true)) return false;
     // hidden += W_down(silu(g) * u); the FFN reads hidden (RMSNorm) before its last kernel adds into it
-    return run_ffn_swiglu_device(h_view, h_view, ffn_norm, eps, gu, L.gu_type, down, L.down_type, L.hidden, L.intermediate, stream);
+    return run_ffn_swiglu_device(h_view, h_view, ffn_norm, eps, gu, L.gu_type, down, L.down_type, L.hidden, L.intermediate, stream,
+                                 ws + b_qkv + b_attn + b_part + b_mm);
 }
 
 }  // namespace
@@ -1406,7 +1554,7 @@ int TSHip_TransformerLayerDecodeDevice(float* hidden, int hidden_size, const flo
                            down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
         if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
         if (!run_layer_decode(hidden, L, attn_norm, qkv_data, q_norm, k_norm, o_data, ffn_norm, gu_data, down_data, k_cache, v_cache,
-                              position, eps, rope_base, rope_freq_scale, rope_mode, g_stream.load()))
+                              position, eps, rope_base, rope_freq_scale, rope_mode, t_stream))
             return 0;
         clear_last_error();
         return 1;
@@ -1439,7 +1587,7 @@ int TSHip_TransformerModelDecodeDevice(float* hidden, int hidden_size, int num_l
             }
             if (!run_layer_decode(hidden, L, attn_norm[l], qkv[l], q_norm ? q_norm[l] : nullptr, k_norm ? k_norm[l] : nullptr, o[l],
                                   ffn_norm[l], gu[l], down[l], k_cache[l], v_cache[l], position, eps, rope_base, rope_freq_scale,
-                                  rope_mode, g_stream.load()))
+                                  rope_mode, t_stream))
                 return 0;
         }
         clear_last_error();
@@ -1464,7 +1612,7 @@ int TSHip_TransformerLayerDecode(void* hidden, int hidden_size, void* attn_norm,
         const LayerShape L{hidden_size, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate_size, qkv_type, o_type, gu_type,
                            down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
         if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
-        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
         HostLayer d;
         if (!resolve_layer(L, attn_norm, qkv_data, q_norm, k_norm, o_data, ffn_norm, gu_data, down_data, k_cache, v_cache, &d)) return 0;
         return decode_with_host_hidden(static_cast<float*>(hidden), hidden_size, [&](float* h, hipStream_t stream) {
@@ -1491,7 +1639,7 @@ int TSHip_TransformerModelDecode(void* hidden, int hidden_size, int num_layers, 
         const LayerShape L{hidden_size, head_dim, num_heads, num_kv_heads, max_seq_len, intermediate_size, qkv_type, o_type, gu_type,
                            down_type, qkv_bytes, o_bytes, gu_bytes, down_bytes};
         if (!validate_layer(L, qkv_ne0, qkv_ne1, o_ne0, o_ne1, gu_ne0, gu_ne1, down_ne0, down_ne1, position)) return 0;
-        std::lock_guard<std::mutex> lock(g_host_call_mutex);
+        std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
         std::vector<HostLayer> d((size_t)num_layers);
         for (int l = 0; l < num_layers; ++l) {
             if (!attn_norm[l] || !qkv[l] || !o[l] || !ffn_norm[l] || !gu[l] || !down[l] || !k_cache[l] || !v_cache[l]) {

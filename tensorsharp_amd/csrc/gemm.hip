@@ -631,19 +631,15 @@ __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&
     }
 }
 
-float* chunk_buffer(size_t bytes);
-// K-chunk sums go to the caller's buffer when one is given (`fixed`: nothing is allocated; a launch that needs more
-// either runs with whole K or fails), else to the grow-only buffer above.
+// Where the sums of K chunks go: a buffer of the caller (the kernels allocate nothing).  A launch whose chunk sums do
+// not fit runs with whole K per tile, or fails when the kernel cannot do without chunks.  `need_out` set: nothing is
+// launched, the launcher only reports how many bytes it would use.
 struct ChunkScratch {
     float* ptr;
     size_t bytes;
-    bool fixed;
+    size_t* need_out;
 };
-inline float* chunk_scratch(const ChunkScratch& cs, size_t bytes)
-{
-    if (!cs.fixed) return chunk_buffer(bytes);
-    return bytes <= cs.bytes ? cs.ptr : nullptr;
-}
+inline float* chunk_scratch(const ChunkScratch& cs, size_t bytes) { return bytes <= cs.bytes ? cs.ptr : nullptr; }
 __global__ void gemm_chunk_sum_kernel(const float* __restrict__ partial, int k_chunks, int M, int N, const int* __restrict__ c_rows,
                                       float* __restrict__ c, int64_t ldc, int accumulate);
 
@@ -887,7 +883,7 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratc
     auto kern = gemm_kernel<G, BM, XST, NW>;
     constexpr int RB = (XST > 2 && G::kSup == 2) ? 3 : 2;
     const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * RT + 1024;
-    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
     a.n_tiles = (a.N + BN - 1) / BN;
     const int nkt = a.Kp / kBK;
@@ -902,17 +898,18 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratc
         if (a.k_chunks > 1) {
             a.chunk_kt = ((nkt + a.k_chunks - 1) / a.k_chunks + 3) / 4 * 4;
             a.k_chunks = (nkt + a.chunk_kt - 1) / a.chunk_kt;
-            a.partial = chunk_scratch(cs, (size_t)a.k_chunks * a.M * a.N * sizeof(float));
-            if (!a.partial && cs.fixed) {
+            const size_t need = (size_t)a.k_chunks * a.M * a.N * sizeof(float);
+            if (cs.need_out) *cs.need_out = need;
+            a.partial = chunk_scratch(cs, need);
+            if (!a.partial) {
                 // the caller's scratch is too small for the chunk sums: whole K per tile (slower, same result up to
                 // fp32 summation order)
                 a.k_chunks = 1;
                 a.chunk_kt = (nkt + 3) / 4 * 4;
-            } else if (!a.partial) {
-                return false;
             }
         }
     }
+    if (cs.need_out) return true;
     const int total = a.m_tiles * a.n_tiles * a.k_chunks;
     const int grid = ((total + 7) / 8) * 8;          // whole rounds over the 8 XCDs
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
@@ -1140,27 +1137,6 @@ __global__ void __launch_bounds__(256) gemm_chunk_sum_kernel(const float* __rest
     }
 }
 
-// grow-only device buffer for the K-chunk sums
-float* chunk_buffer(size_t bytes)
-{
-    static std::mutex mu;
-    static void* buf = nullptr;
-    static size_t have = 0;
-    std::lock_guard<std::mutex> lock(mu);
-    if (bytes > have) {
-        if (buf) {
-            if (!hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize")) return nullptr;
-            (void)hipFree(buf);
-        }
-        buf = nullptr;
-        have = 0;
-        const size_t want = bytes + bytes / 4;
-        if (!hip_ok(hipMalloc(&buf, want), "hipMalloc(K-chunk sums)")) return nullptr;
-        have = want;
-    }
-    return static_cast<float*>(buf);
-}
-
 template <typename G, int KTW>
 bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
@@ -1168,7 +1144,7 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch
     auto kern = gemm_slim_kernel<G, KTW>;
     const size_t lds = (size_t)8 * L::RING * L::BUF + 64;     // the unpackers may read a few bytes past the last row
     static_assert((size_t)8 * L::RING * L::BUF + 64 <= 160 * 1024, "raw buffers must fit LDS");
-    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
     a.n_tiles = (a.N + 31) / 32;
     a.chunk_kt = 8 * KTW;
@@ -1176,12 +1152,15 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch
     a.partial = nullptr;
     const bool two_pass = a.k_chunks > 1 || a.accumulate;
     if (two_pass) {
-        a.partial = chunk_scratch(cs, (size_t)a.k_chunks * a.M * a.N * sizeof(float));
-        if (!a.partial) {
-            if (cs.fixed) set_last_error("gemm: the K-chunk sums of this shape do not fit the caller's scratch buffer.");
+        const size_t need = (size_t)a.k_chunks * a.M * a.N * sizeof(float);
+        if (cs.need_out) *cs.need_out = need;
+        a.partial = chunk_scratch(cs, need);
+        if (!a.partial && !cs.need_out) {
+            set_last_error("gemm: the K-chunk sums of this shape do not fit the scratch buffer.");
             return false;
         }
     }
+    if (cs.need_out) return true;
     const int64_t units = (int64_t)m_tiles * a.k_chunks * a.n_tiles;
     const int grid = (int)std::min<int64_t>(units, device_info().num_cus);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
@@ -1354,12 +1333,11 @@ bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, 
     return launch_convert<kSrcSwiglu>(type, src, M, F, workspace, stream);
 }
 
-bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
-                 int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, void* chunk_ws,
-                 size_t chunk_ws_bytes)
+namespace {
+bool gemm_dispatch(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
+                   int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, const ChunkScratch& cs)
 {
-    const ChunkScratch cs{static_cast<float*>(chunk_ws), chunk_ws_bytes, chunk_ws != nullptr};
-    if (w_bytes >= ((int64_t)1 << 31) - 64 && !tiles) {
+    if (w_bytes >= kMaxOperandBytes && !tiles) {
         set_last_error("gemm: a single weight of 2 GiB or more must be split by rows.");
         return false;
     }
@@ -1377,7 +1355,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     a.K = K;
     a.Kp = (K + kBK - 1) / kBK * kBK;
     a.x16_bytes = (int64_t)M * a.Kp * (int64_t)sizeof(_Float16);
-    if (a.x16_bytes >= ((int64_t)1 << 31)) {
+    if (a.x16_bytes >= kMaxOperandBytes) {
         set_last_error("gemm: the converted activations of one call must stay below 2 GiB; split the rows.");
         return false;
     }
@@ -1408,6 +1386,25 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     case kTypeIQ4_NL: return launch_for_type<GLegacy<kTypeIQ4_NL>>(a, bm, m_tiles, stream, cs);
     default: set_last_error("gemm: unsupported type."); return false;
     }
+}
+}  // namespace
+
+bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
+                 int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, void* chunk_ws,
+                 size_t chunk_ws_bytes)
+{
+    const ChunkScratch cs{static_cast<float*>(chunk_ws), chunk_ws ? chunk_ws_bytes : 0, nullptr};
+    return gemm_dispatch(type, w, w_bytes, workspace, c, ldc, c_rows, M, N, K, tiles, stream, accumulate, cs);
+}
+
+size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate)
+{
+    size_t need = 0;
+    // a buffer "large enough" so that the launchers make the choices they would make with the reported bytes at hand
+    const ChunkScratch cs{nullptr, ~(size_t)0, &need};
+    const int64_t w_bytes = tiles ? 0 : (int64_t)(block_bytes(type) * (K / block_elems(type))) * N;
+    if (!gemm_dispatch(type, nullptr, w_bytes, nullptr, nullptr, N, nullptr, M, N, K, tiles, nullptr, accumulate, cs)) return 0;
+    return need;
 }
 
 }  // namespace tship

@@ -66,6 +66,7 @@ struct GemvProblem {
     int act;                  // how x is formed while it is staged (kAct*)
     const int* expert_id;     // optional (MoE): the weight is w + expert_id[0] * expert_stride
     int64_t expert_stride;
+    int n_experts;            // ids outside [0, n_experts) select no weight: the problem reads zeros
     int N;
     int K;
 };
@@ -835,12 +836,16 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const uint32_t row_bytes = (uint32_t)F::row_bytes(K);
     const int wave_stride = nwg * kWaves;
     const int gw = __builtin_amdgcn_readfirstlane(wg * kWaves + (int)(threadIdx.x >> 6));
-    const uintptr_t w_begin = reinterpret_cast<uintptr_t>(P.w) + (P.expert_id ? (uintptr_t)((int64_t)P.expert_id[0] * P.expert_stride) : 0);
+    // an expert id from the device is not trusted: one outside the table gets an empty resource (every load reads
+    // zero, so the result row is the `add` term alone) instead of an address computed from it
+    const int eid = P.expert_id ? __builtin_amdgcn_readfirstlane(P.expert_id[0]) : 0;
+    const bool bad_expert = P.expert_id && (eid < 0 || eid >= P.n_experts);
+    const uintptr_t w_begin = reinterpret_cast<uintptr_t>(P.w) + (P.expert_id && !bad_expert ? (uintptr_t)((int64_t)eid * P.expert_stride) : 0);
     // one range-checked resource for the whole tensor (host guarantees w_bytes < 2 GiB); the extent is
     // rounded up to whole dwords, which stay inside the last 4-byte word the tensor touches
     const uintptr_t base = w_begin & ~(uintptr_t)3;
     const uint32_t base_delta = (uint32_t)(w_begin & 3);
-    const uint32_t extent = ((uint32_t)P.w_bytes + base_delta + 3u) & ~3u;
+    const uint32_t extent = bad_expert ? 0u : ((uint32_t)P.w_bytes + base_delta + 3u) & ~3u;
     const __amdgpu_buffer_rsrc_t rs =
         __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, (int)extent, 0x00020000);
     const typename F::Lane L = F::lane_setup(sub, l16, row_bytes);
@@ -878,8 +883,8 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         const_cast<float*>(act == kActRmsNorm ? P.norm_w : P.x + K), 0, K * 4, 0x00020000);
     float4 x2[kStageChunk][F::kStageF4];
     // GPT-OSS mode: per-expert bias of the gate and of the up half
-    const bool has_bias = act == kActSwigluOai && P.norm_w != nullptr;
-    const float* bias = has_bias ? P.norm_w + (P.expert_id ? (int64_t)P.expert_id[0] * 2 * K : 0) : P.x;
+    const bool has_bias = act == kActSwigluOai && P.norm_w != nullptr && !bad_expert;
+    const float* bias = has_bias ? P.norm_w + (P.expert_id ? (int64_t)eid * 2 * K : 0) : P.x;
     const __amdgpu_buffer_rsrc_t bgrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bias), 0, K * 4, 0x00020000);
     const __amdgpu_buffer_rsrc_t burs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bias + K), 0, K * 4, 0x00020000);
     float4 bg[kStageChunk][F::kStageF4], bu[kStageChunk][F::kStageF4];
@@ -1216,6 +1221,11 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         g.p[i].K = args[i].K;
         g.p[i].expert_id = args[i].expert_id;
         g.p[i].expert_stride = args[i].expert_stride;
+        g.p[i].n_experts = args[i].n_experts;
+        if (args[i].expert_id && args[i].n_experts <= 0) {
+            set_last_error("gemv: an expert indirection needs the number of experts.");
+            return false;
+        }
         g.wg_begin[i] = begin;
         begin += share;
     }
@@ -1252,7 +1262,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream,
                  const float* add, int act, const float* norm_w, float eps)
 {
-    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, add, act, norm_w, eps};
+    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, 0, add, act, norm_w, eps};
     return launch_gemv_group(type, 1, &a, stream);
 }
 

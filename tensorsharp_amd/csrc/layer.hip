@@ -205,6 +205,16 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
                 }
             }
         }
+        // Slots past the split hold a clamped row (in the last split the row being written by this very launch, or
+        // whatever the cache memory held): their values must not reach the sums, not even multiplied by a zero
+        // weight (0 * NaN), so they are replaced, not scaled.
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                kr[u][j] = live[u] ? kr[u][j] : 0.f;
+                vr[u][j] = live[u] ? vr[u][j] : 0.f;
+            }
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d[kInFlight];
@@ -314,11 +324,11 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_combine_kernel(const flo
             const bool live = s < splits;
             const float* p = base + (int64_t)(live ? s : s0) * kRow;
             ms[u] = live ? p[0] : -INFINITY;
-            ls[u] = p[1];
+            ls[u] = live ? p[1] : 0.f;
 #pragma unroll
             for (int j = 0; j < kPer; ++j) {
                 const int d = lane + 64 * j;
-                v[u][j] = d < head_dim ? p[2 + d] : 0.f;
+                v[u][j] = (live && d < head_dim) ? p[2 + d] : 0.f;
             }
         }
 #pragma unroll

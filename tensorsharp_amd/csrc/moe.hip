@@ -127,6 +127,12 @@ __global__ void __launch_bounds__(1024) moe_group_kernel(const int* __restrict__
     }
     __syncthreads();
     for (int e = tid; e <= E; e += blockDim.x) M.offsets[e] = off[e];
+    // assignments with an id outside the table take no sorted row: the rows past the last expert's stay unused, but
+    // the activation converts walk over all A rows, so those rows name a valid token and expert
+    for (int i = off[E] + tid; i < A; i += blockDim.x) {
+        M.token_of[i] = 0;
+        M.expert_of[i] = 0;
+    }
     for (int j = tbeg[E] + tid; j < max_tiles; j += blockDim.x) {
         M.tile_expert[j] = 0;
         M.tile_row0[j] = 0;
@@ -161,7 +167,7 @@ __global__ void __launch_bounds__(1024) moe_group_kernel(const int* __restrict__
 template <int VEC>
 __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ dn, const float* __restrict__ bias,
                                                           const int* __restrict__ ids, const float* __restrict__ weights,
-                                                          const int* __restrict__ pos_of, int k, int H, int slot_order,
+                                                          const int* __restrict__ pos_of, int k, int E, int H, int slot_order,
                                                           float* __restrict__ out, int64_t ldo)
 {
     const int t = blockIdx.y;
@@ -200,7 +206,7 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restric
         if (j < k) {
             const int64_t a = (int64_t)t * k + slot[j];
             const int pos = pos_of ? pos_of[a] : (int)a;
-            if (pos >= 0) {
+            if (pos >= 0 && id[j] >= 0 && id[j] < E) {     // an id outside the expert table contributes nothing
                 const float w = weights[a];
                 const float* dp = dn + (int64_t)pos * H + h;
                 const float* bp = bias ? bias + (int64_t)id[j] * H + h : nullptr;
@@ -251,7 +257,7 @@ bool launch_moe_group(const int* ids, int A, int k, int E, int bm, int max_tiles
 }
 
 bool launch_moe_combine(const float* dn, const float* bias, const int* ids, const float* weights, const int* pos_of, int T,
-                        int k, int H, bool slot_order, float* out, int64_t ldo, hipStream_t stream)
+                        int k, int E, int H, bool slot_order, float* out, int64_t ldo, hipStream_t stream)
 {
     if (k > kMaxK) {
         set_last_error("moe_combine: k > 16.");
@@ -261,9 +267,9 @@ bool launch_moe_combine(const float* dn, const float* bias, const int* ids, cons
                                                     reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     if (vec)
         hipLaunchKernelGGL(moe_combine_kernel<4>, dim3((H / 4 + 255) / 256, T), dim3(256), 0, stream, dn, bias, ids, weights, pos_of, k,
-                           H, slot_order ? 1 : 0, out, ldo);
+                           E, H, slot_order ? 1 : 0, out, ldo);
     else
-        hipLaunchKernelGGL(moe_combine_kernel<1>, dim3((H + 255) / 256, T), dim3(256), 0, stream, dn, bias, ids, weights, pos_of, k, H,
+        hipLaunchKernelGGL(moe_combine_kernel<1>, dim3((H + 255) / 256, T), dim3(256), 0, stream, dn, bias, ids, weights, pos_of, k, E, H,
                            slot_order ? 1 : 0, out, ldo);
     return hip_ok(hipGetLastError(), "moe_combine launch");
 }

@@ -116,6 +116,7 @@ struct GemvArgs {
     int K;
     const int* expert_id = nullptr;   // optional device pointer (MoE): weight = w + expert_id[0] * expert_stride
     int64_t expert_stride = 0;
+    int n_experts = 0;                // with expert_id: ids outside [0, n_experts) make the problem read zeros
     const float* add = nullptr;       // optional: y = add + W x (add may be y)
     int act = 0;                      // activation mode, see launch_gemv; 3 = GPT-OSS SwiGLU (x is a gate|up row of 2K,
                                       // norm_w the optional [E][2K] bias indexed by expert_id, eps = alpha, limit = clamp)
@@ -154,12 +155,15 @@ struct GemmTiles {
 
 // c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
 // accumulate: c[row] += ... instead of c[row] = ...
-// chunk_ws (device, optional): where the sums of K chunks go; with it the launch allocates nothing (a shape whose
-// chunk sums do not fit runs with whole K per tile, or fails when the kernel cannot do without chunks).  Without it
-// they go to a grow-only buffer of the library.
+// chunk_ws (device): where the sums of K chunks go, gemm_chunk_ws_bytes() of them (a shape whose chunk sums do not fit
+// what is passed runs with whole K per tile, or fails when its kernel cannot do without chunks).  Nothing is allocated.
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc,
                  const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate = false,
                  void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0);
+// bytes of chunk_ws the same launch uses (0 for most shapes); only tiles->bm and tiles->count are read
+size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate);
+// the kernels address one weight (or one launch's converted activations) with 32-bit offsets
+constexpr int64_t kMaxOperandBytes = ((int64_t)1 << 31) - 64;
 
 // ---- fused wrappers around the matmul (RMSNorm prologue, SiLU-gated FFN) ------------------------
 // out[m, 0..K) = x[m] / sqrt(mean(x[m]^2) + eps) * w   (ggml_rms_norm then ggml_mul), contiguous rows
@@ -191,8 +195,9 @@ struct MoeMaps {            // all device pointers, A = T * k assignments
 };
 // counting sort of the assignments by expert (row order inside an expert is unspecified) + m-tile table for the grouped GEMM
 bool launch_moe_group(const int* ids, int A, int k, int E, int bm, int max_tiles, const MoeMaps& maps, hipStream_t stream);
-// out[t][h] = sum_s w[t][s] * (dn[pos_of[t*k+s]][h] + b[e][h]); order: ascending expert (or slot order)
+// out[t][h] = sum_s w[t][s] * (dn[pos_of[t*k+s]][h] + b[e][h]); order: ascending expert (or slot order); assignments whose
+// expert id lies outside [0, E) contribute nothing
 bool launch_moe_combine(const float* dn, const float* bias, const int* ids, const float* weights, const int* pos_of, int T,
-                        int k, int H, bool slot_order, float* out, int64_t ldo, hipStream_t stream);
+                        int k, int E, int H, bool slot_order, float* out, int64_t ldo, hipStream_t stream);
 
 }  // namespace tship

@@ -30,6 +30,9 @@ TYPE_TABLE = {
     16: (256, 66), 17: (256, 74), 18: (256, 98), 19: (256, 50), 20: (32, 18), 21: (256, 110), 22: (256, 82), 23: (256, 136),
     29: (256, 56), 34: (256, 54), 35: (256, 66), 39: (32, 17), 24: (1, 1), 25: (1, 2), 26: (1, 4), 27: (1, 8), 28: (1, 8),
 }
+# block formats the matmul kernels read (tship_internal.h is_quant_type): Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K,
+# IQ4_NL, MXFP4
+MATMUL_TYPES = (2, 3, 6, 7, 8, 12, 13, 14, 20, 39)
 TYPE_NAMES = {0: "F32", 1: "F16", 2: "Q4_0", 3: "Q4_1", 6: "Q5_0", 7: "Q5_1", 8: "Q8_0", 9: "Q8_1", 10: "Q2_K", 11: "Q3_K",
               12: "Q4_K", 13: "Q5_K", 14: "Q6_K", 15: "Q8_K", 20: "IQ4_NL", 30: "BF16", 39: "MXFP4"}
 
@@ -91,6 +94,7 @@ class GgufFile:
         self._bytes = np.frombuffer(self._map, dtype=np.uint8)
         self.Metadata = {}
         self.Tensors = {}
+        self._preloaded = []          # cache keys (mapped addresses) handed to PreloadQuantizedWeight
         try:
             self._parse()
         except Exception:
@@ -119,6 +123,9 @@ class GgufFile:
             offset = c.take("<Q")
             self.Tensors[name] = GgufTensorInfo(name, shape, ggml_type, offset)
         alignment = int(self.Metadata.get("general.alignment", 32))
+        if alignment <= 0 or alignment & (alignment - 1):
+            # the reference divides by it (GgufReader.cs:115-118); the GGUF format requires a power of two
+            raise ValueError(f"GGUF general.alignment must be a positive power of two, not {alignment}.")
         self.DataOffset = c.pos + (alignment - c.pos % alignment) % alignment
 
     def _value(self, c, vt):
@@ -237,18 +244,26 @@ class GgufFile:
         """Upload matrices once through the bridge's preload export, keyed by their mapped address: later host-pointer
         calls with the same weight pointer run from the device copy (ModelBase.cs:660-706).  Returns the weights."""
         from .hip_basic_ops import HipBasicOps
-        from . import hip_native as N
         out = {}
         for name in (names if names is not None else list(self.Tensors)):
             info = self.Tensors[name]
-            if len(info.Shape) != 2 or info.Type not in (N.TYPE_Q8_0, N.TYPE_Q4_K, N.TYPE_Q6_K, N.TYPE_MXFP4):
+            # every block format the matmul kernels read (F32 / F16 / BF16 tensors stay with the host path)
+            if len(info.Shape) != 2 or info.Type not in MATMUL_TYPES:
                 continue
             w = self.quantized_weight(name)
             HipBasicOps.PreloadQuantizedWeight(w.ptr, w.ptr, w.ggml_type, w.ne0, w.ne1, w.raw_bytes)
+            self._preloaded.append(w.ptr)
             out[name] = w
         return out
 
     def close(self):
+        # the device copies are keyed by addresses inside the mapping: once it is gone another file may be mapped at
+        # the same address, and a preload of equal size under the same key would be taken for a repeat
+        if self._preloaded:
+            from .hip_basic_ops import HipBasicOps
+            for key in self._preloaded:
+                HipBasicOps.InvalidateHostBuffer(key)
+            self._preloaded = []
         self._bytes = None
         try:
             self._map.close()

@@ -98,3 +98,14 @@ def test_facade_argument_errors_mirror_the_reference():
         HipBasicOps.AddmmQuant(np.zeros((1, 4), np.float32)[:, ::2], np.zeros((1, 64), np.float32), w.ctypes.data, 8, 64, 2, w.size)
     with pytest.raises(NotImplementedError, match="block size"):
         HipBasicOps.GetRowSizeBytes(N.TYPE_Q4_K, 100)
+
+
+def test_sync_host_buffer_is_a_no_op_for_pointers_that_were_never_cached():
+    # ggml_ops_core.cpp:664-684: null pointer, zero size or an uncached pointer -> success, nothing copied
+    lib = N.lib()
+    a = np.arange(8, dtype=np.float32)
+    assert lib.TSHip_SyncHostBuffer(a.ctypes.data, a.nbytes) == 1
+    assert lib.TSHip_SyncHostBuffer(None, 16) == 1
+    assert lib.TSHip_SyncHostBuffer(a.ctypes.data, 0) == 1
+    assert N.get_last_error() == ""
+    assert np.array_equal(a, np.arange(8, dtype=np.float32))

@@ -91,3 +91,14 @@ def test_rejects_bad_files(tmp_path):
     with GgufFile(str(p)) as g:
         with pytest.raises(ValueError, match="past the end"):
             g.tensor_data("output.weight")
+
+
+@pytest.mark.parametrize("alignment", [0, 24])
+def test_rejects_an_alignment_that_is_not_a_power_of_two(tmp_path, alignment):
+    # header, then one u32 key "general.alignment" (value type 4 = UINT32)
+    key = b"general.alignment"
+    blob = struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + struct.pack("<Q", len(key)) + key + struct.pack("<II", 4, alignment)
+    p = tmp_path / "align.gguf"
+    p.write_bytes(blob)
+    with pytest.raises(ValueError, match="power of two"):
+        GgufFile(str(p))

@@ -10,14 +10,14 @@ from tensorsharp_amd.gguf import GgufFile
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-MATS = ["token_embd.weight", "blk.0.attn_q.weight", "blk.0.ffn_down.weight", "blk.0.ffn_gate_exps.weight"]
+MATS = ["token_embd.weight", "blk.0.attn_q.weight", "blk.0.ffn_down.weight", "blk.0.ffn_gate_exps.weight", "output.weight"]
 
 
 def test_preload_from_the_mapping_then_host_pointer_calls(hip, oracle):
     rng = np.random.default_rng(81)
     with GgufFile(os.path.join(GOLD, "tiny.gguf")) as g:
         ws = g.preload()
-        assert sorted(ws) == sorted(MATS)          # Q8_0, Q4_K, Q6_K, MXFP4 matrices; F32 norm and Q4_0 output are skipped
+        assert sorted(ws) == sorted(MATS)          # Q8_0, Q4_K, Q6_K, MXFP4 and Q4_0 matrices; the F32 norm is skipped
         for name, w in ws.items():
             for M in (1, 5):
                 x = rng.standard_normal((M, w.ne0)).astype(np.float32)
@@ -25,7 +25,8 @@ def test_preload_from_the_mapping_then_host_pointer_calls(hip, oracle):
                 hip.AddmmQuant(y, x, w.ptr, w.ggml_type, w.ne0, w.ne1, w.raw_bytes)
                 ref = oracle.matmul_f64(w.ggml_type, np.array(w.data), w.ne1, w.ne0, x)
                 assert inputs.row_l2_err(y, ref) <= 1e-3, (name, M)
-        hip.ClearHostBufferCache()
+    # close() dropped the device copies: a sync of one of the former keys finds nothing to do, a matmul on the unmapped
+    # address is not attempted here
 
 
 def test_device_copy_and_embedding_rows(hip, oracle):

@@ -251,3 +251,35 @@ def test_host_pointer_model_decode_equals_the_device_form(hip, oracle):
             assert np.array_equal(hl["k_cache"], d["k_cache"].cpu().numpy()) and np.array_equal(hl["v_cache"], d["v_cache"].cpu().numpy())
     finally:
         hip.ClearHostBufferCache()
+
+
+@pytest.mark.parametrize("prefix", [0, 5, 70, 517])
+def test_unwritten_cache_rows_may_hold_nan(hip, oracle, prefix):
+    """Cache rows at and beyond `position` are not part of the attention (ggml_flash_attn_ext skips masked positions): whatever
+    their memory holds - NaN bits from an uninitialised allocation - must not reach the result.  One split (short prefix),
+    a ragged last split and several splits."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(777 + prefix)
+    hidden, heads, kv_heads, head_dim, inter, max_seq = 256, 4, 2, 64, 512, 640
+    layer, dims = make_layer(oracle, rng, hidden, heads, kv_heads, head_dim, inter, (Q8_0, Q8_0, Q8_0, Q8_0), True)
+    dev = to_device_layer(layer, torch, QuantizedWeight, dims)
+    kc = np.zeros((kv_heads, max_seq, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    vc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    kn, vn = kc.copy(), vc.copy()
+    kn[:, prefix:] = np.nan
+    vn[:, prefix:] = np.nan
+    kd, vd = torch.from_numpy(kn).cuda(), torch.from_numpy(vn).cuda()
+    for pos in range(prefix, prefix + 2):
+        h = rng.standard_normal(hidden).astype(np.float32)
+        hd = torch.from_numpy(h.copy()).cuda()
+        oracle.layer_decode(h, layer, kc, vc, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, 2)
+        hip.TransformerLayerDecode(hd, dev["attn_norm"], dev["qkv"], dev["q_norm"], dev["k_norm"], dev["o"], dev["ffn_norm"],
+                                   dev["gate_up"], dev["down"], kd, vd, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, 2)
+        torch.cuda.synchronize()
+        got = hd.cpu().numpy()
+        assert np.all(np.isfinite(got)), pos
+        assert rel(got, h) <= 3e-3, (pos, rel(got, h))
+    assert np.all(np.isnan(kd.cpu().numpy()[:, prefix + 2:]))              # rows past the written ones untouched
