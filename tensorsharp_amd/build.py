@@ -16,11 +16,10 @@ FLAGS = [
 ]
 
 
-def build(verbose=False, jobs=8, defines=(), out=None):
-    """Compile every source and link the shared library.  `defines` / `out` build a tuning variant
-    (extra -D flags, other output path) without touching the default library."""
+def build(verbose=False, jobs=8):
+    """Compile every source and link the shared library."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    lib = out or LIB
+    lib = LIB
     objdir = os.path.join(HERE, "build", os.path.basename(lib))
     os.makedirs(objdir, exist_ok=True)
     procs = []
@@ -28,7 +27,7 @@ def build(verbose=False, jobs=8, defines=(), out=None):
     for src in SOURCES:
         obj = os.path.join(objdir, src + ".o")
         objs.append(obj)
-        cmd = [hipcc] + FLAGS + [f"-D{d}" for d in defines] + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

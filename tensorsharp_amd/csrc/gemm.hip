@@ -525,7 +525,7 @@ struct GLegacy {
             m2 = mbits | (mbits << 16);
         }
         uint32_t qh = 0u;
-        if (kFive) qh = (kHdr & 3) ? __builtin_amdgcn_alignbyte(b[kHdr / 4], b[kHdr / 4 - 1], 2) : b[kHdr / 4 - 1];
+        if constexpr (kFive) qh = (kHdr & 3) ? __builtin_amdgcn_alignbyte(b[kHdr / 4], b[kHdr / 4 - 1], 2) : b[kHdr / 4 - 1];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             // quant bytes 4 w .. 4 w + 3 of the block
@@ -596,11 +596,7 @@ __device__ __forceinline__ void copy16_to_lds(__amdgpu_buffer_rsrc_t rs, uint8_t
 template <int N>
 __device__ __forceinline__ void wait_copies_and_barrier()
 {
-#ifdef TSHIP_GEMM_DEBUG_NOBAR
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory");
-#else
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
-#endif
 }
 
 // Epilogue of one wavefront: D[row = 32 i + 8 (r / 4) + 4 h + r % 4][column my_n] times the row scale.
@@ -746,11 +742,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         const bool any = kt < nkt;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
-#ifdef TSHIP_GEMM_DEBUG_NOX
-            copy16_to_lds(xrs, stage + (wave + NW * i) * 1024, kDeadOffset, (uint32_t)kt * kXRow);
-#else
             copy16_to_lds(xrs, stage + (wave + NW * i) * 1024, any ? x_off[i] : kDeadOffset, (uint32_t)kt * kXRow);
-#endif
         }
     };
     auto issue_w = [&](int s) {
@@ -759,11 +751,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             const int id = wave + NW * i;
-#ifdef TSHIP_GEMM_DEBUG_NOW
-            copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, kDeadOffset, G::sup_offset(s));
-#else
             copy16_to_lds(wrs, id < RIN ? buf + id * 1024 : dump, any ? w_off[i] : kDeadOffset, G::sup_offset(s));
-#endif
         }
     };
 
@@ -813,22 +801,14 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
                 const half8_t b = __builtin_bit_cast(half8_t, bb);
 #pragma unroll
                 for (int i = 0; i < TM; ++i) {
-#ifndef TSHIP_GEMM_DEBUG_NOMMA
                     acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b, acc[i], 0, 0, 0);
-#else
-                    acc[i][0] += (float)a[i][0] * (float)b[0];
-#endif
                     if (ks + 1 < 4) a[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[(ks + 1) & 3]);
                     // matrix and LDS instructions keep this order (each operand is requested TM - 1 MFMAs
                     // before its use); vector and scalar ALU work may move across
                     __builtin_amdgcn_sched_barrier(0x6);
                 }
                 // unpack the next k-tile's operands in the shadow of the matrix pipe
-#ifndef TSHIP_GEMM_DEBUG_NODEQ
                 if (ks == 0) G::dequant(r, jn, h, dn, ((kt + 1) * 2 + h) * 32 < A.K, on);
-#else
-                if (ks == 0) { _Pragma("unroll") for (int q = 0; q < 16; ++q) on[q] = r[q % G::kRegs]; }
-#endif
             }
         }
         // Copies that may stay in flight: the activations requested in the last D - 1 iterations and a
@@ -855,6 +835,379 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         store_tile<TM>(P, acc, m0, m_rows, my_n, h);
     } else {
         store_tile<TM>(A, acc, m0, m_rows, my_n, h);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// gemm_xw_kernel: BM x 256 x 64 tiles, eight wavefronts laid out 2 (rows) x 4 (columns); a wavefront owns BM / 2 rows of
+// 64 output columns, so one A operand read from LDS feeds two matrix instructions and one B operand feeds BM / 64.
+// Every weight of the tile is still unpacked exactly once: wavefront w unpacks columns [32 w, 32 w + 32) of the NEXT
+// k-tile from the raw bytes in LDS and leaves the fp16 operands in an exchange area of LDS ([k-step][k-half][column],
+// 16 bytes each: the layout in which the matrix instruction wants them, so both the write and the read are
+// contiguous 16-byte pieces per lane), double-buffered; the k-tile's one barrier publishes them.
+// Raw weights are copied per k-tile (P: which 16-byte pieces of a row belong to k-tile kt), two stages.
+// ------------------------------------------------------------------------------------------
+struct PQ4K {
+    typedef GQ4K G;
+    static constexpr int kParts = 3;                  // header + the k-tile's 32 quant bytes
+    static constexpr int kRowBytes = 48;
+    static __device__ __forceinline__ uint32_t part_base(int part) { return part == 0 ? 0u : 16u * (uint32_t)part; }
+    static __device__ __forceinline__ uint32_t part_step(int part) { return part == 0 ? 0u : 32u; }   // times kt % 4
+    static __device__ __forceinline__ uint32_t soffset(int kt) { return (uint32_t)(kt >> 2) * 144u; }
+    static __device__ __forceinline__ int phase(int kt) { return kt & 3; }
+    static __device__ __forceinline__ void fetch(const uint8_t* rp, int h, uint32_t (&r)[G::kRegs])
+    {
+        const uint4_t hdr = *reinterpret_cast<const uint4_t*>(rp);
+        const uint4_t q = *reinterpret_cast<const uint4_t*>(rp + 16 + h * 16);
+        r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
+        r[4] = q.x; r[5] = q.y; r[6] = q.z; r[7] = q.w;
+    }
+    // The unpacking of one lane's 32 weights of a k-tile (GQ4K::dequant) cut into kMicro small steps that the kernel
+    // places one by one behind its matrix instructions; step I may use what steps < I left in `st` and `o`.
+    // Quarter q of `o` (o[4 q .. 4 q + 3], the B operand of k-step q) is complete after step kReady[q].
+    static constexpr int kMicro = 17;
+    static constexpr int kFirstHalf = 11;             // steps after which quarters 0 and 2 are complete
+    struct State {
+        uint32_t a, b, c, sc, mn, s1, o1, s2, o2, q8;
+    };
+    // constants kept in registers so that mask-and-merge is one instruction (v_and_or_b32 takes one literal at most)
+    struct Consts {
+        uint32_t magic, lo_mask, hi_mask, neg1024;
+        __device__ __forceinline__ Consts() : magic(0x64006400u), lo_mask(0x000f000fu), hi_mask(0x00f000f0u), neg1024(0xe400e400u)
+        {
+            asm volatile("" : "+v"(magic));
+            asm volatile("" : "+s"(lo_mask), "+s"(hi_mask), "+s"(neg1024));
+        }
+    };
+    static __device__ __forceinline__ int ready_after(int quarter) { return quarter == 0 ? 10 : quarter == 2 ? 10 : 16; }
+    template <int I>
+    static __device__ __forceinline__ void micro(State& st, const uint32_t (&r)[G::kRegs], int j, bool /*live*/, const Consts& K,
+                                                 uint32_t (&o)[16])
+    {
+        if constexpr (I == 0) {
+            const int sh = (j & 1) * 16;
+            st.a = r[1] >> sh;
+            st.b = r[2] >> sh;
+            st.c = r[3] >> sh;
+        } else if constexpr (I == 1) {
+            const uint32_t sc_lo = st.a & 0x3f3fu, sc_hi = (st.c & 0x0f0fu) | ((st.a >> 2) & 0x3030u);
+            st.sc = (j & 2) ? sc_hi : sc_lo;
+        } else if constexpr (I == 2) {
+            const uint32_t m_lo = st.b & 0x3f3fu, m_hi = ((st.c >> 4) & 0x0f0fu) | ((st.b >> 2) & 0x3030u);
+            st.mn = (j & 2) ? m_hi : m_lo;
+        } else if constexpr (I == 3) {
+            H2U dm;
+            dm.u = r[0];
+            const float d = (float)dm.h.x, dmin = (float)dm.h.y;
+            st.s1 = splat(d * (float)(st.sc & 0xffu));
+            st.o1 = splat(-(dmin * (float)(st.mn & 0xffu)));
+        } else if constexpr (I == 4) {
+            H2U dm;
+            dm.u = r[0];
+            const float d = (float)dm.h.x, dmin = (float)dm.h.y;
+            st.s2 = splat(d * (float)(st.sc >> 8) * 0.0625f);
+            st.o2 = splat(-(dmin * (float)(st.mn >> 8)));
+        } else {
+            // raw dword i in three steps: both low nibble pairs; high pair of bytes 0, 2; high pair of bytes 1, 3
+            constexpr int i = (I - 5) / 3, part = (I - 5) % 3;
+            const uint32_t q = r[4 + i];
+            if constexpr (part == 0) {
+                st.q8 = q >> 8;
+                o[2 * i] = pk_fma(pk_add((q & K.lo_mask) | K.magic, K.neg1024), st.s1, st.o1);
+                o[2 * i + 1] = pk_fma(pk_add((st.q8 & K.lo_mask) | K.magic, K.neg1024), st.s1, st.o1);
+            } else if constexpr (part == 1) {
+                o[8 + 2 * i] = pk_fma(pk_add((q & K.hi_mask) | K.magic, K.neg1024), st.s2, st.o2);
+            } else {
+                o[8 + 2 * i + 1] = pk_fma(pk_add((st.q8 & K.hi_mask) | K.magic, K.neg1024), st.s2, st.o2);
+            }
+        }
+    }
+};
+
+template <typename P, int BM, int WN>
+__global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
+{
+    typedef typename P::G G;
+    constexpr int BN = 256;
+    constexpr int NW = 2 * WN;                            // wavefronts: 2 (rows) x WN (columns)
+    constexpr int TMW = BM / 64;                          // 32-row blocks of a wavefront (its BM / 2 rows)
+    constexpr int NB = BN / (32 * WN);                    // 32-column blocks of a wavefront
+    constexpr int DUTY = BN / 32 / NW;                    // 32-column blocks a wavefront unpacks per k-tile
+    constexpr int kXTile = BM * kXRow;
+    constexpr int XI = kXTile / 1024 / NW;                // activation copies per wavefront and k-tile
+    constexpr int kRawTile = BN * P::kRowBytes;
+    constexpr int kRawCopies = kRawTile / 1024;
+    constexpr int RI = (kRawCopies + NW - 1) / NW;        // raw copies per wavefront and k-tile; the surplus goes to a dump area
+    constexpr int kBTile = 4 * 2 * BN * 16;               // exchange area of one k-tile
+    static_assert(kRawCopies * 1024 == kRawTile && XI >= 1 && XI * NW * 1024 == kXTile, "tile pieces must be whole KiB");
+    extern __shared__ uint8_t smem[];
+    uint8_t* const xbuf = smem;                           // 2 x kXTile
+    uint8_t* const rraw = xbuf + 2 * kXTile;              // 2 x kRawTile
+    uint8_t* const bex = rraw + 2 * kRawTile;             // 2 x kBTile
+    uint8_t* const dump = bex + 2 * kBTile;               // 1 KiB
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int col = lane & 31, h = lane >> 5;
+
+    const int tiles = A.m_tiles * A.n_tiles;
+    const int total = tiles * A.k_chunks;
+    int t = blockIdx.x;
+    {
+        const int per = (total + 7) >> 3;
+        const int xcd = t & 7, slot = t >> 3;
+        t = xcd * per + slot;
+        if (slot >= per || t >= total) return;
+    }
+    const int kc = t / tiles;
+    t -= kc * tiles;
+    const int mt = t / A.n_tiles, nt = t - mt * A.n_tiles;
+    int m0, m_rows;
+    const uint8_t* wbase = A.w;
+    if (A.tile_expert) {
+        m0 = A.tile_row0[mt];
+        m_rows = A.tile_rows[mt];
+        if (m_rows <= 0) return;
+        wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+    } else {
+        m0 = mt * BM;
+        m_rows = min(BM, A.M - m0);
+    }
+    const int n0 = nt * BN;
+
+    const __amdgpu_buffer_rsrc_t wrs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(wbase), 0, (int)(((uint32_t)A.w_bytes + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int kt_begin = kc * A.chunk_kt;
+    const int nkt = min(A.Kp / kBK, kt_begin + A.chunk_kt);
+
+    uint32_t x_off[XI], r_off[RI], r_step[RI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+        const int q = (wave + NW * i) * 64 + lane;
+        const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
+        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+    }
+#pragma unroll
+    for (int i = 0; i < RI; ++i) {
+        const int q = (wave + NW * i) * 64 + lane;                // 16-byte piece of the raw tile
+        const int row = q / P::kParts, part = q - row * P::kParts;
+        const bool ok = q < BN * P::kParts && n0 + row < A.N;
+        r_off[i] = ok ? (uint32_t)(n0 + row) * row_bytes + P::part_base(part) : kDeadOffset;
+        r_step[i] = ok ? P::part_step(part) : 0u;
+    }
+    // k-tiles past the end: the offset gets its top bit set (out of range: zeros arrive) by data flow, not by a
+    // branch, so that the loop body stays one scheduling region
+    auto issue_x1 = [&](int kt, int i) {
+        const uint32_t past = kt < nkt ? 0u : kDeadOffset;
+        copy16_to_lds(xrs, xbuf + (kt & 1) * kXTile + (wave + NW * i) * 1024, x_off[i] | past, (uint32_t)kt * kXRow);
+    };
+    auto issue_raw1 = [&](int kt, int i) {
+        const uint32_t past = kt < nkt ? 0u : kDeadOffset;
+        const int id = wave + NW * i;
+        copy16_to_lds(wrs, id < kRawCopies ? rraw + (kt & 1) * kRawTile + id * 1024 : dump,
+                      (r_off[i] + r_step[i] * (uint32_t)P::phase(kt)) | past, P::soffset(kt));
+    };
+
+    float16_t acc[TMW][NB];
+#pragma unroll
+    for (int m = 0; m < TMW; ++m)
+#pragma unroll
+        for (int n = 0; n < NB; ++n)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[m][n][r] = 0.f;
+
+    // LDS addresses of this lane: A operand of k-step ks = 16-byte piece 2 ks + h of row (wm BM/2 + 32 m + col), swizzled;
+    // B operand of k-step ks, column block n = piece ((2 ks + h) 256 + 32 NB wn + 32 n + col) of the exchange area
+    const int sw = (col >> 1) & 7;
+    int a_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) a_off[ks] = (wm * (BM / 2) + col) * kXRow + ((2 * ks + h) ^ sw) * 16;
+    const int b_rd = (h * BN + 32 * NB * wn + col) * 16;
+    const int b_wr = (h * BN + 32 * DUTY * wave + col) * 16;
+    const int my_raw = (32 * DUTY * wave + col) * P::kRowBytes;
+    auto load_ops = [&](int kt, int ks, half8_t (&a)[TMW], half8_t (&b)[NB]) {
+        const uint8_t* xs = xbuf + (kt & 1) * kXTile;
+        const uint8_t* bs = bex + (kt & 1) * kBTile;
+#pragma unroll
+        for (int m = 0; m < TMW; ++m) a[m] = *reinterpret_cast<const half8_t*>(xs + m * 32 * kXRow + a_off[ks]);
+#pragma unroll
+        for (int n = 0; n < NB; ++n) b[n] = *reinterpret_cast<const half8_t*>(bs + b_rd + ks * (2 * BN * 16) + n * 32 * 16);
+    };
+
+    // The loop is rotated around the k-tile's barrier, which sits between k-steps 2 and 3: by then every operand of the
+    // k-tile is in registers, so behind the barrier the stage can take the copy of the k-tile after next, the first
+    // operands of the next k-tile are read and its raw bytes fetched while k-step 3 still feeds the matrix pipe.
+    //   state behind barrier(kt - 1): activations of k-tile kt and raw bytes of kt + 1 have landed, the exchange area of
+    //   kt is complete
+#pragma unroll
+    for (int i = 0; i < RI; ++i) issue_raw1(kt_begin, i);
+#pragma unroll
+    for (int i = 0; i < XI; ++i) issue_x1(kt_begin, i);
+#pragma unroll
+    for (int i = 0; i < RI; ++i) issue_raw1(kt_begin + 1, i);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < DUTY; ++u) {
+        uint32_t r0[G::kRegs], o0[16];
+        P::fetch(rraw + (kt_begin & 1) * kRawTile + my_raw + u * 32 * P::kRowBytes, h, r0);
+        G::dequant(r0, P::phase(kt_begin), h, 0u, (kt_begin * 2 + h) * 32 < A.K, o0);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint4_t v = {o0[4 * ks], o0[4 * ks + 1], o0[4 * ks + 2], o0[4 * ks + 3]};
+            *reinterpret_cast<uint4_t*>(bex + (kt_begin & 1) * kBTile + b_wr + u * 32 * 16 + ks * (2 * BN * 16)) = v;
+        }
+    }
+    __syncthreads();
+    half8_t a0[TMW], b0[NB], a1[TMW], b1[NB];
+    uint32_t r[DUTY][G::kRegs];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) issue_x1(kt_begin + 1, i);
+#pragma unroll
+    for (int i = 0; i < RI; ++i) issue_raw1(kt_begin + 2, i);
+    load_ops(kt_begin, 0, a0, b0);
+#pragma unroll
+    for (int u = 0; u < DUTY; ++u) P::fetch(rraw + ((kt_begin + 1) & 1) * kRawTile + my_raw + u * 32 * P::kRowBytes, h, r[u]);
+
+    // One k-step = NM matrix instructions (column block n, row block m in that order).  The other work of the k-tile is
+    // placed by hand, piece by piece, behind the matrix instructions (one LDS access and a few vector instructions
+    // each) and the scheduler is fenced after every piece, so that it neither clusters the unpacking nor moves an
+    // operand read next to its use.
+    constexpr int NM = TMW * NB;
+    constexpr int kSlots = 3 * NM;                          // matrix instructions of k-steps 0 .. 2
+    constexpr int kWorkOne = P::kMicro + 4;                 // unpack steps and the four exchange writes of 32 columns
+    constexpr int kWork = DUTY * kWorkOne;
+    constexpr int kPer = (kWork + kSlots - 1) / kSlots;
+    static_assert(kPer <= 3, "unpack work must fit the slots");
+    const typename P::Consts KC;
+    for (int kt = kt_begin; kt < nkt; ++kt) {
+        uint32_t o[16];
+        typename P::State st;
+        const int ph = P::phase(kt + 1);
+        const bool live = ((kt + 1) * 2 + h) * 32 < A.K;
+        const uint8_t* const xs = xbuf + (kt & 1) * kXTile;
+        const uint8_t* const bs = bex + (kt & 1) * kBTile + b_rd;
+        uint8_t* const bnext = bex + ((kt + 1) & 1) * kBTile + b_wr;
+        // work item w of the k-tile's unpacking: per 32 columns P::kMicro unpack steps with the four exchange writes
+        // inserted as soon as their quarter is complete (quarters 0 and 2, then 1 and 3)
+        auto work = [&](auto w_tag) {
+            constexpr int wall = decltype(w_tag)::value;
+            if constexpr (wall < kWork) {
+                constexpr int u = wall / kWorkOne, w = wall % kWorkOne;
+                constexpr int first_ready = P::kFirstHalf, second_ready = P::kMicro;
+                uint8_t* const dst = bnext + u * 32 * 16;
+                if constexpr (w < first_ready) {
+                    P::template micro<w>(st, r[u], ph, live, KC, o);
+                } else if constexpr (w == first_ready || w == first_ready + 1) {
+                    constexpr int q = w == first_ready ? 0 : 2;
+                    const uint4_t v = {o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]};
+                    *reinterpret_cast<uint4_t*>(dst + q * (2 * BN * 16)) = v;
+                } else if constexpr (w < second_ready + 2) {
+                    P::template micro<w - 2>(st, r[u], ph, live, KC, o);
+                } else {
+                    constexpr int q = w == second_ready + 2 ? 1 : 3;
+                    const uint4_t v = {o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]};
+                    *reinterpret_cast<uint4_t*>(dst + q * (2 * BN * 16)) = v;
+                }
+            }
+        };
+        auto slot = [&](auto s_tag, const half8_t (&ac)[TMW], const half8_t (&bc)[NB], half8_t (&an)[TMW], half8_t (&bn)[NB], int ks_next) {
+            constexpr int sidx = decltype(s_tag)::value;           // 0 .. kSlots - 1
+            constexpr int i = sidx % NM, n = i / TMW, m = i % TMW;
+            acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ac[m], bc[n], acc[m][n], 0, 0, 0);
+            // operands of the next k-step, one read per matrix instruction
+            if constexpr (i < TMW) an[i] = *reinterpret_cast<const half8_t*>(xs + i * 32 * kXRow + a_off[ks_next]);
+            else if constexpr (i < TMW + NB) bn[i - TMW] = *reinterpret_cast<const half8_t*>(bs + ks_next * (2 * BN * 16) + (i - TMW) * 32 * 16);
+            if constexpr (kPer >= 1) work(std::integral_constant<int, sidx * kPer>{});
+            if constexpr (kPer >= 2) work(std::integral_constant<int, sidx * kPer + 1>{});
+            if constexpr (kPer >= 3) work(std::integral_constant<int, sidx * kPer + 2>{});
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto kstep = [&](auto base_tag, const half8_t (&ac)[TMW], const half8_t (&bc)[NB], half8_t (&an)[TMW], half8_t (&bn)[NB], int ks_next) {
+            constexpr int base = decltype(base_tag)::value;
+            slot(std::integral_constant<int, base + 0>{}, ac, bc, an, bn, ks_next);
+            slot(std::integral_constant<int, base + 1>{}, ac, bc, an, bn, ks_next);
+            slot(std::integral_constant<int, base + 2>{}, ac, bc, an, bn, ks_next);
+            slot(std::integral_constant<int, base + 3>{}, ac, bc, an, bn, ks_next);
+            if constexpr (NM >= 8) {
+                slot(std::integral_constant<int, base + 4>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 5>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 6>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 7>{}, ac, bc, an, bn, ks_next);
+            }
+            if constexpr (NM >= 16) {
+                slot(std::integral_constant<int, base + 8>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 9>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 10>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 11>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 12>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 13>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 14>{}, ac, bc, an, bn, ks_next);
+                slot(std::integral_constant<int, base + 15>{}, ac, bc, an, bn, ks_next);
+            }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        kstep(std::integral_constant<int, 0>{}, a0, b0, a1, b1, 1);
+        kstep(std::integral_constant<int, NM>{}, a1, b1, a0, b0, 2);
+        kstep(std::integral_constant<int, 2 * NM>{}, a0, b0, a1, b1, 3);
+        wait_copies_and_barrier<0>();
+        // behind the barrier: copies two k-tiles ahead, first operands and raw bytes of the next k-tile, k-step 3
+        {
+            const uint8_t* const xn = xbuf + ((kt + 1) & 1) * kXTile;
+            const uint8_t* const bnx = bex + ((kt + 1) & 1) * kBTile + b_rd;
+            const uint8_t* const rawn = rraw + (kt & 1) * kRawTile + my_raw;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < NM; ++i) {
+                const int n = i / TMW, m = i % TMW;
+                acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1[m], b1[n], acc[m][n], 0, 0, 0);
+                if (i < TMW) a0[i] = *reinterpret_cast<const half8_t*>(xn + i * 32 * kXRow + a_off[0]);
+                else if (i < TMW + NB) b0[i - TMW] = *reinterpret_cast<const half8_t*>(bnx + (i - TMW) * 32 * 16);
+                if (i < DUTY) P::fetch(rawn + i * 32 * P::kRowBytes, h, r[i]);
+                if (i < XI) issue_x1(kt + 2, i);
+                else if (i < XI + RI) issue_raw1(kt + 3, i - XI);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+
+    // epilogue: D[row = 32 m + 8 (r / 4) + 4 h + r % 4][column] times the row scale
+    float* cdst = A.c;
+    int64_t ldc = A.ldc;
+    const int* c_rows = A.c_rows;
+    int accumulate = A.accumulate;
+    if (A.partial) {
+        cdst = A.partial + (int64_t)kc * A.M * A.N;
+        ldc = A.N;
+        c_rows = nullptr;
+        accumulate = 0;
+    }
+#pragma unroll
+    for (int m = 0; m < TMW; ++m) {
+        float sc[16];
+        int64_t off[16];
+#pragma unroll
+        for (int r2 = 0; r2 < 16; ++r2) {
+            const int ml = wm * (BM / 2) + m * 32 + 8 * (r2 >> 2) + 4 * h + (r2 & 3);
+            const int mr = m0 + min(ml, m_rows - 1);
+            sc[r2] = A.xscale[mr];
+            off[r2] = (int64_t)(c_rows ? c_rows[mr] : mr) * ldc;
+        }
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const int my_n = n0 + 32 * NB * wn + 32 * n + col;
+            if (my_n >= A.N) continue;
+#pragma unroll
+            for (int r2 = 0; r2 < 16; ++r2) {
+                const int ml = wm * (BM / 2) + m * 32 + 8 * (r2 >> 2) + 4 * h + (r2 & 3);
+                if (ml < m_rows) {
+                    float* p = cdst + off[r2] + my_n;
+                    *p = accumulate ? *p + acc[m][n][r2] * sc[r2] : acc[m][n][r2] * sc[r2];
+                }
+            }
+        }
     }
 }
 
@@ -913,6 +1266,47 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratc
     const int total = a.m_tiles * a.n_tiles * a.k_chunks;
     const int grid = ((total + 7) / 8) * 8;          // whole rounds over the 8 XCDs
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
+    if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
+    if (a.partial) {
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
+                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
+        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+    }
+    return true;
+}
+
+template <typename P, int BM, int WN>
+bool launch_xw(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
+{
+    constexpr int BN = 256;
+    auto kern = gemm_xw_kernel<P, BM, WN>;
+    const size_t lds = (size_t)2 * BM * kXRow + (size_t)2 * BN * P::kRowBytes + (size_t)2 * 4 * 2 * BN * 16 + 1024;
+    static_assert((size_t)2 * BM * kXRow + (size_t)2 * BN * P::kRowBytes + (size_t)2 * 4 * 2 * BN * 16 + 1024 <= 160 * 1024, "LDS");
+    if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + BN - 1) / BN;
+    const int nkt = a.Kp / kBK;
+    a.k_chunks = 1;
+    a.chunk_kt = (nkt + 3) / 4 * 4;
+    a.partial = nullptr;
+    if (!a.tile_expert) {
+        a.k_chunks = pick_k_chunks(a.m_tiles * a.n_tiles, nkt, device_info().num_cus, (int64_t)a.M * a.N, 1.7 * BM * BN / 65536.0);
+        if (a.k_chunks > 1) {
+            a.chunk_kt = ((nkt + a.k_chunks - 1) / a.k_chunks + 3) / 4 * 4;
+            a.k_chunks = (nkt + a.chunk_kt - 1) / a.chunk_kt;
+            const size_t need = (size_t)a.k_chunks * a.M * a.N * sizeof(float);
+            if (cs.need_out) *cs.need_out = need;
+            a.partial = chunk_scratch(cs, need);
+            if (!a.partial) {
+                a.k_chunks = 1;
+                a.chunk_kt = (nkt + 3) / 4 * 4;
+            }
+        }
+    }
+    if (cs.need_out) return true;
+    const int total = a.m_tiles * a.n_tiles * a.k_chunks;
+    const int grid = ((total + 7) / 8) * 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(128 * WN), lds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (a.partial) {
         hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
@@ -1207,12 +1601,17 @@ bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream
 
 // 128-row tiles are 128 x 256 (one workgroup per CU) for these formats, 128 x 128 (two per CU) for the others
 template <typename G>
-constexpr bool kWide128 = G::kSup == 2 || G::kRawRow > 144;
+constexpr bool kWide128 = G::kSup == 2 || G::kRawRow > 144 || std::is_same<G, GQ4K>::value;
 
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
     if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream, cs);
+    // Q4_K: the 2 x 4 wavefront layout with the operand exchange through LDS (gemm_xw_kernel); 128-row tiles are 128 x 256
+    if constexpr (std::is_same<G, GQ4K>::value) {
+        if (bm == 256) return launch_xw<PQ4K, 256, 4>(a, m_tiles, stream, cs);
+        if (bm == 128) return launch_xw<PQ4K, 128, 4>(a, m_tiles, stream, cs);
+    }
     if constexpr (2 * 256 * kXRow + 2 * 256 * G::kRawRow + 1024 <= 160 * 1024) {
         if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream, cs);
     }

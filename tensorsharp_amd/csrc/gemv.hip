@@ -35,14 +35,8 @@ namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-// tuning constants (overridable at build time for experiments)
-#ifndef TSHIP_GEMV_WAVES
-#define TSHIP_GEMV_WAVES 8
-#endif
-#ifndef TSHIP_GEMV_WG_PER_CU
-#define TSHIP_GEMV_WG_PER_CU 2
-#endif
-constexpr int kWaves = TSHIP_GEMV_WAVES;
+constexpr int kWaves = 8;          // wavefronts per workgroup
+constexpr int kWgPerCu = 2;        // persistent workgroups per CU
 constexpr int kThreads = kWaves * 64;
 constexpr int kMaxGroup = 8;
 
@@ -150,11 +144,8 @@ constexpr uint32_t kDeadOffset = 0x80000000u;   // beyond any resource extent us
 //   dword 4j+1 = (x[4j+1], x[4j+3])        low nibbles of bytes 1 and 3
 //   dword 4j+2 = (x[32+4j], x[32+4j+2])    high nibbles
 //   dword 4j+3 = (x[32+4j+1], x[32+4j+3])
-#ifndef TSHIP_GEMV_Q4K_LPR
-#define TSHIP_GEMV_Q4K_LPR 32
-#endif
 struct FmtQ4K {
-    static constexpr int kLPR = TSHIP_GEMV_Q4K_LPR;   // lanes per row: a step covers kLPR consecutive units of 64 / kLPR rows
+    static constexpr int kLPR = 32;   // lanes per row: a step covers kLPR consecutive units of 64 / kLPR rows
     static constexpr int kUnitElems = 64;
     static constexpr int kLdsDwords = 36;
     static constexpr int kRegs = 12;
@@ -346,11 +337,8 @@ struct FmtQ5K : FmtQ4K {
 // ---- MXFP4 -----------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 80 B): 16 dwords (x[j], x[j+16]) as fp16 pairs, then the unit's
 // scale, then 12 B pad.
-#ifndef TSHIP_GEMV_MXFP4_LPR
-#define TSHIP_GEMV_MXFP4_LPR 16
-#endif
 struct FmtMXFP4 {
-    static constexpr int kLPR = TSHIP_GEMV_MXFP4_LPR;
+    static constexpr int kLPR = 16;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 20;
     static constexpr int kRegs = 5;
@@ -569,11 +557,8 @@ struct FmtQ4Legacy {
 
 // ---- Q8_0 ------------------------------------------------------------------------------------
 // LDS unit (one 32-weight block, 144 B): 32 fp32 activations, 16 B pad.  fp32 throughout.
-#ifndef TSHIP_GEMV_Q80_LPR
-#define TSHIP_GEMV_Q80_LPR 16
-#endif
 struct FmtQ80 {
-    static constexpr int kLPR = TSHIP_GEMV_Q80_LPR;
+    static constexpr int kLPR = 16;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 36;
     static constexpr int kRegs = 9;
@@ -657,11 +642,8 @@ struct FmtQ80 {
 // the same of run 2 (t = 4 i); piece B (runs 1, 3) in dwords 16 .. 31; then the four runs' sums of the scaled fp16
 // activations, then the four runs' power-of-two scales, 16 B pad (a 44-dword stride keeps ds_read_b128 conflict-free).
 // A 6-bit value left in the low bits of an fp16 is the subnormal v * 2^-24, exact in v_dot2_f32_f16.
-#ifndef TSHIP_GEMV_Q6K_LPR
-#define TSHIP_GEMV_Q6K_LPR 32
-#endif
 struct FmtQ6K {
-    static constexpr int kLPR = TSHIP_GEMV_Q6K_LPR;
+    static constexpr int kLPR = 32;
     static constexpr int kUnitElems = 64;
     static constexpr int kLdsDwords = 44;
     static constexpr int kRegs = 19;
@@ -1180,7 +1162,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         lds = std::max(lds, lds_bytes_for(type, args[i].K));
         total_bytes += (double)args[i].w_bytes;
     }
-    int per_cu = (int)std::min<size_t>(TSHIP_GEMV_WG_PER_CU, (160 * 1024) / (lds + 256));
+    int per_cu = (int)std::min<size_t>(kWgPerCu, (160 * 1024) / (lds + 256));
     if (per_cu < 1) per_cu = 1;
     const int budget = di.num_cus * per_cu;
     // A single matrix with so few rows that one row group per wavefront would keep at most half of the wavefronts

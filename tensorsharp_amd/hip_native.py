@@ -9,8 +9,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-# TSHIP_LIBRARY selects another build of the same library (tuning variants); default is in-tree.
-LIB_PATH = os.environ.get("TSHIP_LIBRARY") or os.path.join(HERE, "libTsHipOps.so")
+LIB_PATH = os.path.join(HERE, "libTsHipOps.so")
 
 BACKEND_HIP = 4
 TYPE_F32, TYPE_Q8_0, TYPE_Q4_K, TYPE_MXFP4 = 0, 8, 12, 39
