@@ -803,9 +803,7 @@ struct Step {
 
 // ACT: the activation mode of every problem of the launch (compile time: the plain kernel carries none of
 // the other modes' code or registers)
-// KS: wavefronts that share a row group, each taking 1/KS of its steps (few rows, long K: one group per wavefront would
-// leave most wavefronts without work); their sums meet in LDS.  KS = 1 is the plain scheme.
-template <typename F, int ACT, int KS>
+template <typename F, int ACT>
 __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, int mode, uint32_t* lds)
 {
     const int lane = threadIdx.x & 63;
@@ -960,35 +958,15 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // loop the next step is requested before the current one is consumed.
     Step<F> cur, nxt;
     int fgroup = gw, fstep = 0;                // next step to fetch
-    // K-split scheme: rounds of kWaves / KS row groups per workgroup; wavefront (gslot, slice) takes steps
-    // [s_begin, s_end) of its group
-    constexpr int GPW = kWaves / KS;
-    const int wv = (int)(threadIdx.x >> 6), slice = wv % KS, gslot = wv / KS;
-    const int s_begin = slice * nsteps / KS, s_end = (slice + 1) * nsteps / KS;
-    const int rounds = (ngroups + nwg * GPW - 1) / (nwg * GPW);
-    auto group_of = [&](int r) { return r < rounds ? (r * nwg + wg) * GPW + gslot : ngroups; };
-    int fr = 0, fs = s_begin;
-    auto fetch_next = [&](Step<F>& st) {
-        fetch(group_of(fr), fs, st);
-        if (++fs >= s_end) {
-            fs = s_begin;
-            ++fr;
-        }
-    };
     // deep: two steps requested before x is staged and two in flight afterwards.  Only the activation modes use it
     // (their staging takes longer, and they are the short dependent launches of a decode step: fused FFN 33.9 -> 32.2 us,
     // whole layer 66.5 -> 64.0 us in an A/B on one box; plain launches lose, 4096 x 14336 12.7 -> 14.2 us).
     const bool strict = mode == 1, deep = ACT != kActPlain && !strict;
-    if constexpr (KS > 1) {
-        fetch_next(cur);
-        if (deep) fetch_next(nxt);
-    } else {
-        fetch(fgroup, fstep, cur);
+    fetch(fgroup, fstep, cur);
+    advance(fgroup, fstep);
+    if (deep) {
+        fetch(fgroup, fstep, nxt);
         advance(fgroup, fstep);
-        if (deep) {
-            fetch(fgroup, fstep, nxt);
-            advance(fgroup, fstep);
-        }
     }
     stage_issue(0);
     stage_commit(0);
@@ -1000,37 +978,6 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nsteps * LPR * F::kLdsDwords; i += kThreads) lds[i] = 0u;
     __syncthreads();
 
-    if constexpr (KS > 1) {
-        // Every wavefront of the workgroup runs every round (groups past the end read zeros), so the barrier is uniform.
-        float* part = reinterpret_cast<float*>(red + kWaves);        // [2][kWaves][4]
-        bool flip = false;                                            // which buffer holds the step to consume
-        for (int r = 0; r < rounds; ++r) {
-            float acc = 0.f;
-            auto one = [&](Step<F>& a, Step<F>& b) {
-                if (!deep) fetch_next(b);
-                const uint32_t* xu = lds + lds_lane + (uint32_t)a.step * (uint32_t)(LPR * F::kLdsDwords);
-                acc += F::dot(a.w, L, a.aux, xu);
-                if (deep) fetch_next(a);
-            };
-            for (int st = s_begin; st < s_end; ++st) {
-                if (flip) one(nxt, cur);
-                else one(cur, nxt);
-                flip = !flip;
-            }
-            const float t = row_sum<LPR>(acc);
-            float* pr = part + (r & 1) * kWaves * 4;
-            if (l16 == 0) pr[wv * 4 + sub] = t;
-            __syncthreads();
-            const int group = group_of(r), row = group * RPG + sub;
-            if (slice == 0 && l16 == 0 && group < ngroups && row < N) {
-                float sum = 0.f;
-#pragma unroll
-                for (int k = 0; k < KS; ++k) sum += pr[(wv + k) * 4 + sub];
-                P.y[row] = P.add ? P.add[row] + sum : sum;
-            }
-        }
-        return;
-    }
     float acc = 0.f;
     auto consume = [&](const Step<F>& st) {
         // lanes past the end of a row (and steps past the last group) hold zeros, zero scales included
@@ -1069,7 +1016,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     }
 }
 
-template <int TYPE, int ACT, int KS>
+template <int TYPE, int ACT>
 __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
 {
     extern __shared__ uint32_t lds[];
@@ -1079,13 +1026,13 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
         if (j < G.count && (int)blockIdx.x >= G.wg_begin[j]) i = j;
     const int wg = (int)blockIdx.x - G.wg_begin[i];
     const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
-    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
-    else gemv_body<FmtQ80, ACT, KS>(G.p[i], wg, nwg, G.strict, lds);
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    else gemv_body<FmtQ80, ACT>(G.p[i], wg, nwg, G.strict, lds);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
@@ -1100,17 +1047,17 @@ size_t lds_bytes_for(int type, int K)
 {
     const int lpr = lanes_per_row(type);
     const size_t units = (size_t)((K / unit_elems(type) + lpr - 1) / lpr) * lpr;
-    // + the RMSNorm reduction slots + the partial row sums of the K-split scheme
-    return units * unit_lds_bytes(type) + kWaves * sizeof(double) + 2 * kWaves * 4 * sizeof(float);
+    // + the RMSNorm reduction slots
+    return units * unit_lds_bytes(type) + kWaves * sizeof(double);
 }
 
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 constexpr double kStrictBytes = 96.0 * 1024 * 1024;   // launches streaming at least this much run strict (see gemv_body)
 
-template <int TYPE, int ACT, int KS = 1>
+template <int TYPE, int ACT>
 bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    auto kern = gemv_kernel<TYPE, ACT, KS>;
+    auto kern = gemv_kernel<TYPE, ACT>;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g);
     return hip_ok(hipGetLastError(), "gemv launch");
@@ -1165,17 +1112,11 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     int per_cu = (int)std::min<size_t>(kWgPerCu, (160 * 1024) / (lds + 256));
     if (per_cu < 1) per_cu = 1;
     const int budget = di.num_cus * per_cu;
-    // A single matrix with so few rows that one row group per wavefront would keep at most half of the wavefronts
-    // busy, and rows long enough to cut: two or four wavefronts share a row group, each taking a slice of at least two
-    // of its steps.  Only with plain activations: that many more workgroups stage x, and measured with the SiLU /
-    // RMSNorm staging modes that costs more than the extra wavefronts win (4096 x 14336 Q4_K: plain 14.7 -> 12.6 us,
-    // SiLU mode inside the fused FFN 32.7 -> 34.3 us).
+    // (Cutting the K range of a row group over several wavefronts when a matrix has few rows was measured slower on
+    // every shape: 4096 x 14336 Q4_K 13.7 vs 10.9 us, MXFP4 5760 x 2880 7.8 vs 6.7 us.  Requesting more up front - two extra
+    // steps before x is staged, or a ring of four steps per wavefront - was slower too, the 123 MB grouped launch
+    // included: 24.5 vs 24.2 us.)
     const int lpr = lanes_per_row(type), rpg = 64 / lpr;
-    int ksplit = 1;
-    if (count == 1 && args[0].act == kActPlain) {
-        const int ngroups = (args[0].N + rpg - 1) / rpg, nsteps = (args[0].K / unit_elems(type) + lpr - 1) / lpr;
-        while (ksplit < 4 && ngroups * ksplit * 2 <= budget * kWaves && nsteps / (ksplit * 2) >= 2) ksplit *= 2;
-    }
 
     GemvGroup g;
     std::memset(&g, 0, sizeof(g));
@@ -1185,7 +1126,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     for (int i = 0; i < count; ++i) {
         // workgroups in proportion to the bytes each problem streams
         int share = std::max(1, (int)((double)budget * (double)args[i].w_bytes / total_bytes + 0.5));
-        share = std::min(share, ((args[i].N + rpg - 1) / rpg + kWaves / ksplit - 1) / (kWaves / ksplit));
+        share = std::min(share, ((args[i].N + rpg - 1) / rpg + kWaves - 1) / kWaves);
         g.p[i].w = static_cast<const uint8_t*>(args[i].w);
         g.p[i].w_bytes = args[i].w_bytes;
         g.p[i].x = args[i].x;
@@ -1223,9 +1164,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         return false;
     }
 #define TSHIP_GEMV_DISPATCH(T)                                                           \
-    (ksplit == 4          ? launch_type<T, kActPlain, 4>(g, begin, lds, stream)          \
-     : ksplit == 2        ? launch_type<T, kActPlain, 2>(g, begin, lds, stream)          \
-     : act == kActPlain   ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
+    (act == kActPlain     ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
      : act == kActRmsNorm ? launch_type<T, kActRmsNorm>(g, begin, lds, stream)           \
      : act == kActSiluMul ? launch_type<T, kActSiluMul>(g, begin, lds, stream)           \
                           : launch_type<T, kActSwigluOai>(g, begin, lds, stream))
