@@ -283,7 +283,7 @@ def main():
 
             def f(i):
                 gu, dn = sets[i % 2]
-                HipBasicOps.MoEExpertsForward(hidden, idsets[i % 8], wts, gu, None, dn, None, MXFP4, E, H, F)
+                HipBasicOps.MoEExpertsGptOssForward(hidden, idsets[i % 8], wts, gu, None, dn, None, MXFP4, E, H, F)
             for i in range(5):
                 f(i)
             ev, wall = time_region(f, iters, torch)

@@ -152,8 +152,6 @@ TSHIP_EXPORT int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView
                                                 int m2_ggml_type, const int64_t* m2_ne0s, const int64_t* m2_ne1s,
                                                 const int64_t* m2_raw_bytes);
 
-/* ---- MoE (GPT-OSS expert stage), device pointers ------------------------------------------ */
-
 /* ---- fused wrappers around the matmul ------------------------------------------------------ */
 
 /* replaces TSGgml_FusedRmsNormMatMulQuantF32 (ggml_ops_fused.cpp:21-217, :1380-1400; GgmlNative.cs:243-253, :903-912;
@@ -192,6 +190,102 @@ TSHIP_EXPORT int TSHip_FusedFFNSwiGLUQuantF32Device(TSHipTensorView2D residual, 
                                                     int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
                                                     int64_t down_raw_bytes, int half_dim);
 
+/* replaces TSGgml_FusedOutProjFFNQuantF32 (ggml_ops_fused.cpp:1057-1220; GgmlNative.cs:303-309; GgmlBasicOps.cs:449-480):
+ *   residual [M x hidden] += input [M x out_ne0] * W_out^T
+ *   residual += W_down * ( silu(g) * u ),  [g | u] = W_gate_up * (RMSNorm(residual, eps) * ffn_norm)
+ * in place on residual; host pointers, weights cached like TSHip_AddmmQuantF32. */
+TSHIP_EXPORT int TSHip_FusedOutProjFFNQuantF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* out_proj_data,
+                                               int out_proj_type, int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes,
+                                               void* ffn_norm_data, int ffn_norm_count, float eps, void* gu_data, int gu_type,
+                                               int64_t gu_ne0, int64_t gu_ne1, int64_t gu_raw_bytes, void* dn_data, int dn_type,
+                                               int64_t dn_ne0, int64_t dn_ne1, int64_t dn_raw_bytes, int half_dim);
+
+/* replaces TSGgml_FusedOutProjNormRouterQuantF32 (ggml_ops_fused.cpp:1223-1380; GgmlNative.cs:285-292;
+ * GgmlBasicOps.cs:416-447):
+ *   residual += input * W_out^T;  normed_out = RMSNorm(residual, eps) * norm;  router_out = normed_out * W_router^T
+ * three outputs: residual (in place), normed_out [M x hidden], router_out [M x router_ne1].  The router weight is
+ * usually dense: F32, F16 and BF16 weights are accepted beside the block formats. */
+TSHIP_EXPORT int TSHip_FusedOutProjNormRouterQuantF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* out_proj_data,
+                                                      int out_proj_type, int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes,
+                                                      void* norm_data, int norm_count, float eps, TSHipTensorView2D normed_out,
+                                                      void* router_data, int router_type, int64_t router_ne0,
+                                                      int64_t router_ne1, int64_t router_raw_bytes, TSHipTensorView2D router_out);
+
+/* device-pointer forms of the two: asynchronous on the selected stream; normed_out must be contiguous. */
+TSHIP_EXPORT int TSHip_FusedOutProjFFNQuantF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, const void* out_proj_data,
+                                                     int out_proj_type, int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes,
+                                                     const float* ffn_norm_weight, int ffn_norm_count, float eps,
+                                                     const void* gu_data, int gu_type, int64_t gu_ne0, int64_t gu_ne1,
+                                                     int64_t gu_raw_bytes, const void* dn_data, int dn_type, int64_t dn_ne0,
+                                                     int64_t dn_ne1, int64_t dn_raw_bytes, int half_dim);
+TSHIP_EXPORT int TSHip_FusedOutProjNormRouterQuantF32Device(TSHipTensorView2D residual, TSHipTensorView2D input,
+                                                            const void* out_proj_data, int out_proj_type, int64_t out_ne0,
+                                                            int64_t out_ne1, int64_t out_raw_bytes, const float* norm_weight,
+                                                            int norm_count, float eps, TSHipTensorView2D normed_out,
+                                                            const void* router_data, int router_type, int64_t router_ne0,
+                                                            int64_t router_ne1, int64_t router_raw_bytes,
+                                                            TSHipTensorView2D router_out);
+
+/* ---- weighted expert sets: the bridge's per-token MoE calls ---------------------------------- */
+
+/* replaces TSGgml_MoEExpertsForwardF32 (ggml_ops_fused.cpp:1576-1760; GgmlNative.cs:333-347; GgmlBasicOps.cs:586-613;
+ * Nemotron experts): result = sum_e route_weights[e] * W_down[e] * max(W_up[e] * input, 0)^2 over the num_experts
+ * (1..16) selected experts, added in index order.  The pointer arrays and route_weights are host arrays; each expert's
+ * blocks are cached on the device under their host address like any weight.  One token runs as grouped GEMV
+ * launches; more rows run expert by expert through the matmul path. */
+TSHIP_EXPORT int TSHip_MoEExpertsForwardF32(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
+                                            void** up_data_ptrs, void** down_data_ptrs, int up_ggml_type, int64_t up_ne0,
+                                            int64_t up_ne1, int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0,
+                                            int64_t down_ne1, int64_t down_raw_bytes_each, float* route_weights);
+
+/* replaces TSGgml_MoEExpertsSwiGLUForwardF32 (ggml_ops_fused.cpp:1766-1940; GgmlNative.cs:350-369;
+ * GgmlBasicOps.cs:615-645): result = sum_e route_weights[e] * W_down[e] * ( silu(W_gate[e] x) * (W_up[e] x) ),
+ * num_experts 1..16. */
+TSHIP_EXPORT int TSHip_MoEExpertsSwiGLUForwardF32(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
+                                                  void** gate_data_ptrs, void** up_data_ptrs, void** down_data_ptrs,
+                                                  int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1,
+                                                  int64_t gate_raw_bytes_each, int up_ggml_type, int64_t up_ne0, int64_t up_ne1,
+                                                  int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0,
+                                                  int64_t down_ne1, int64_t down_raw_bytes_each, float* route_weights);
+
+/* replaces TSGgml_MoEExpertsSwiGLUResidualF32 (ggml_ops_fused.cpp:1953-2160; GgmlNative.cs:372-408;
+ * GgmlBasicOps.cs:647-700; Qwen3.5 MoE decode): residual += sum_e route_weights[e] * expert_e(input)
+ * [+ shared_scalar * shared_expert(input)], num_experts 1..32.  The shared expert takes part only when use_shared is
+ * non-zero and its three pointers are non-null; it may have its own types and intermediate width. */
+TSHIP_EXPORT int TSHip_MoEExpertsSwiGLUResidualF32(
+    TSHipTensorView2D residual, TSHipTensorView2D input, int num_experts, void** gate_data_ptrs, void** up_data_ptrs,
+    void** down_data_ptrs, int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1, int64_t gate_raw_bytes_each, int up_ggml_type,
+    int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+    int64_t down_raw_bytes_each, float* route_weights, int use_shared, void* shared_gate_data, void* shared_up_data,
+    void* shared_down_data, int shared_gate_ggml_type, int64_t shared_gate_ne0, int64_t shared_gate_ne1,
+    int64_t shared_gate_raw_bytes, int shared_up_ggml_type, int64_t shared_up_ne0, int64_t shared_up_ne1,
+    int64_t shared_up_raw_bytes, int shared_down_ggml_type, int64_t shared_down_ne0, int64_t shared_down_ne1,
+    int64_t shared_down_raw_bytes, float shared_scalar);
+
+/* device-pointer forms of the three: the tensors and every weight pointer are device memory, the pointer arrays and
+ * route_weights stay host arrays (read before the call returns); asynchronous on the selected stream. */
+TSHIP_EXPORT int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
+                                                  void* const* up_data_ptrs, void* const* down_data_ptrs, int up_ggml_type,
+                                                  int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each, int down_ggml_type,
+                                                  int64_t down_ne0, int64_t down_ne1, int64_t down_raw_bytes_each,
+                                                  const float* route_weights);
+TSHIP_EXPORT int TSHip_MoEExpertsSwiGLUForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
+                                                        void* const* gate_data_ptrs, void* const* up_data_ptrs,
+                                                        void* const* down_data_ptrs, int gate_ggml_type, int64_t gate_ne0,
+                                                        int64_t gate_ne1, int64_t gate_raw_bytes_each, int up_ggml_type,
+                                                        int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each,
+                                                        int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                                        int64_t down_raw_bytes_each, const float* route_weights);
+TSHIP_EXPORT int TSHip_MoEExpertsSwiGLUResidualF32Device(
+    TSHipTensorView2D residual, TSHipTensorView2D input, int num_experts, void* const* gate_data_ptrs, void* const* up_data_ptrs,
+    void* const* down_data_ptrs, int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1, int64_t gate_raw_bytes_each,
+    int up_ggml_type, int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0,
+    int64_t down_ne1, int64_t down_raw_bytes_each, const float* route_weights, int use_shared, void* shared_gate_data,
+    void* shared_up_data, void* shared_down_data, int shared_gate_ggml_type, int64_t shared_gate_ne0, int64_t shared_gate_ne1,
+    int64_t shared_gate_raw_bytes, int shared_up_ggml_type, int64_t shared_up_ne0, int64_t shared_up_ne1,
+    int64_t shared_up_raw_bytes, int shared_down_ggml_type, int64_t shared_down_ne0, int64_t shared_down_ne1,
+    int64_t shared_down_raw_bytes, float shared_scalar);
+
 /* replaces TSGgml_GetRowsQuantF32 (ggml_ops_matmul.cpp:519-668, :1339-1368; GgmlNative.cs:324, :1003-1006; caller
  * ModelBase.cs:826-856 embedding lookup): result[i, 0..ne0) = dequantized row indices[i] of the [ne1 x ne0] source
  * (type F32 copies rows).  Host pointers; the source is cached on the device by pointer / preload key like the
@@ -218,7 +312,7 @@ TSHIP_EXPORT int TSHip_MoERouteF32Device(TSHipTensorView2D logits, int k, int32_
  * NULL.  Few assignments (T*k <= 8) run as grouped decode GEMVs with the expert picked on the device; otherwise the
  * assignments are counting-sorted by expert on the device and each linear is ONE grouped MFMA GEMM launch.
  * Accumulation order over experts: ascending expert id for T > 1, selection order for T == 1 (as the reference). */
-TSHIP_EXPORT int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D hidden, const int32_t* ids,
+TSHIP_EXPORT int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D hidden, const int32_t* ids,
                                                   const float* weights, int k, const void* gate_up_w,
                                                   const float* gate_up_bias, const void* down_w, const float* down_bias,
                                                   int ggml_type, int n_experts, int64_t H, int64_t F, float alpha,

@@ -14,12 +14,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 F32, Q8_0, Q4_K, MXFP4 = 0, 8, 12, 39
 F16, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q6_K, IQ4_NL, BF16 = 1, 2, 3, 6, 7, 13, 14, 20, 30
+Q8_1 = 9
 TYPES = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4}
 # formats with a dequantizer only (embedding gather, DequantizeToF32); Q6_K also has matmuls on the GPU
 MORE_TYPES = {"f16": F16, "bf16": BF16, "q4_0": Q4_0, "q4_1": Q4_1, "q5_0": Q5_0, "q5_1": Q5_1, "q5_k": Q5_K,
               "q6_k": Q6_K, "iq4_nl": IQ4_NL}
 BLOCK = {F32: (1, 4), Q8_0: (32, 34), Q4_K: (256, 144), MXFP4: (32, 17), F16: (1, 2), BF16: (1, 2), Q4_0: (32, 18),
-         Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176), Q6_K: (256, 210), IQ4_NL: (32, 18)}
+         Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176), Q6_K: (256, 210), IQ4_NL: (32, 18), Q8_1: (32, 36)}
 
 _f32p = C.POINTER(C.c_float)
 _f64p = C.POINTER(C.c_double)
@@ -245,6 +246,72 @@ class Oracle:
             _ptr(ids, _i32p), _ptr(wts, _f32p), _ptr(out, _f32p))
         assert rc == 0, rc
         return out
+
+    # -- compositions for the bridge's larger fused calls -----------------------------------------
+    # Each chains restatements that are pinned on their own (dequantizers, fp64 product, RMSNorm, SiLU) in the order
+    # of the bridge's ggml graph; intermediate tensors are rounded to fp32 where the graph holds fp32 tensors.
+    def weight_rows(self, t, w, N, K):
+        """[N, K] fp32 values of a weight of any type the matmul entry points take"""
+        if t == F32:
+            return np.ascontiguousarray(w).view(np.float32)[:N * K].reshape(N, K)
+        return self.dequantize(t, w, N * K).reshape(N, K)
+
+    def matmul_any_f64(self, t, w, N, K, x):
+        """x [M, K] times W^T in fp64; dense types (F32 / F16 / BF16) through numpy, block formats through tso_matmul_f64"""
+        if t in (F32, F16, BF16):
+            x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)
+            return x.astype(np.float64) @ self.weight_rows(t, w, N, K).astype(np.float64).T
+        return self.matmul_f64(t, w, N, K, x)
+
+    @staticmethod
+    def relu_sqr(x):
+        """ggml_relu then ggml_sqr on fp32 (ggml_ops_fused.cpp:1700-1710)"""
+        r = np.maximum(np.asarray(x, dtype=np.float32), np.float32(0))
+        return r * r
+
+    def expert_ffn(self, x, expert):
+        """One expert: W_down * act(x) in fp64 from fp32 activations.  expert: dict(up=(t, raw, N, K), down=(...),
+        gate=(...) or None); gate present: silu(W_gate x) * (W_up x) (ggml_ops_fused.cpp:1876-1885), else
+        max(W_up x, 0)^2 (ggml_ops_fused.cpp:1700-1712)."""
+        up = self.matmul_any_f64(*expert["up"], x).astype(np.float32)
+        if expert.get("gate") is not None:
+            gate = self.matmul_any_f64(*expert["gate"], x).astype(np.float32)
+            act = self.silu_mul(np.concatenate([gate, up], axis=1))
+        else:
+            act = self.relu_sqr(up)
+        return self.matmul_any_f64(*expert["down"], act)
+
+    def expert_set(self, x, experts, weights, base=None):
+        """(base +) sum_e weights[e] * expert_e(x), experts added in index order and the base last
+        (ggml_ops_fused.cpp:1716-1722, :2094-2121); returns (result fp64, list of per-expert fp64 down outputs)."""
+        parts = [self.expert_ffn(x, e) for e in experts]
+        acc = None
+        for p, wgt in zip(parts, weights):
+            term = p * float(np.float32(wgt))
+            acc = term if acc is None else acc + term
+        if base is not None:
+            acc = np.asarray(base, dtype=np.float64) + acc
+        return acc, parts
+
+    def outproj_ffn(self, residual, x, out_w, norm_w, eps, gate_up, down, half):
+        """FusedOutProjFFN (ggml_ops_fused.cpp:1164-1190): res = residual + W_out x; res + W_down(silu(g) * u) with
+        [g | u] = W_gate_up (RMSNorm(res) * norm_w).  Weights are (type, raw, N, K) tuples.  Returns (result fp64,
+        fp64 out-projection product, fp64 down product)."""
+        mm1 = self.matmul_any_f64(*out_w, x)
+        res = (np.asarray(residual, dtype=np.float64) + mm1).astype(np.float32)
+        xn = self.rms_norm_mul(res, norm_w, eps)
+        gu = self.matmul_any_f64(*gate_up, xn).astype(np.float32)
+        assert gu.shape[1] == 2 * half
+        mm2 = self.matmul_any_f64(*down, self.silu_mul(gu))
+        return res.astype(np.float64) + mm2, mm1, mm2
+
+    def outproj_norm_router(self, residual, x, out_w, norm_w, eps, router):
+        """FusedOutProjNormRouter (ggml_ops_fused.cpp:1310-1330): returns (residual + W_out x in fp64, its RMSNorm * norm_w
+        in fp32, the router logits in fp64, the fp64 out-projection product)."""
+        mm1 = self.matmul_any_f64(*out_w, x)
+        res = np.asarray(residual, dtype=np.float64) + mm1
+        normed = self.rms_norm_mul(res.astype(np.float32), norm_w, eps)
+        return res, normed, self.matmul_any_f64(*router, normed), mm1
 
 
 class Reference:

@@ -109,7 +109,7 @@ int64_t tso_block_size(int type)
     case TSO_TYPE_Q4_K: return Q4_K_ELEMS;
     case TSO_TYPE_MXFP4: return MXFP4_ELEMS;
     case TSO_TYPE_F16: case TSO_TYPE_BF16: return 1;
-    case TSO_TYPE_Q4_0: case TSO_TYPE_Q4_1: case TSO_TYPE_Q5_0: case TSO_TYPE_Q5_1: case TSO_TYPE_IQ4_NL: return 32;
+    case TSO_TYPE_Q4_0: case TSO_TYPE_Q4_1: case TSO_TYPE_Q5_0: case TSO_TYPE_Q5_1: case TSO_TYPE_IQ4_NL: case TSO_TYPE_Q8_1: return 32;
     case TSO_TYPE_Q5_K: case TSO_TYPE_Q6_K: return 256;
     default: return 0;
     }
@@ -127,6 +127,7 @@ int64_t tso_type_size(int type)
     case TSO_TYPE_Q4_1: return 20;
     case TSO_TYPE_Q5_0: return 22;
     case TSO_TYPE_Q5_1: return 24;
+    case TSO_TYPE_Q8_1: return 36;
     case TSO_TYPE_IQ4_NL: return 18;
     case TSO_TYPE_Q5_K: return 176;
     case TSO_TYPE_Q6_K: return 210;
@@ -420,6 +421,17 @@ static void dequant_q8_0(const uint8_t* src, int64_t n, float* y)
     }
 }
 
+/* Q8_1 block: fp16 d, fp16 s (= d * sum of the quants, not read here), int8 qs[32]; y = q * d.
+ * Reference: ManagedQuantizedOps.cs:429-445, GgufReader.cs:342 (36 bytes). */
+static void dequant_q8_1(const uint8_t* src, int64_t n, float* y)
+{
+    for (int64_t b = 0; b < n / 32; ++b, src += 36, y += 32) {
+        const float d = tso_fp16_to_fp32(rd16(src));
+        const int8_t* q = (const int8_t*)(src + 4);
+        for (int j = 0; j < 32; ++j) y[j] = q[j] * d;
+    }
+}
+
 /* y = (d*sc)*q - (dmin*m); low nibbles are the first 32 of each 64-group.
  * Reference: ManagedQuantizedOps.cs:447-479, ggml-quants.c:1352-1374. */
 static void dequant_q4_K(const uint8_t* src, int64_t n, float* y)
@@ -596,6 +608,7 @@ int tso_dequantize(int type, const void* src, int64_t n, float* dst)
     switch (type) {
     case TSO_TYPE_F32: memcpy(dst, src, (size_t)n * 4); return 0;
     case TSO_TYPE_Q8_0: dequant_q8_0((const uint8_t*)src, n, dst); return 0;
+    case TSO_TYPE_Q8_1: dequant_q8_1((const uint8_t*)src, n, dst); return 0;
     case TSO_TYPE_Q4_K: dequant_q4_K((const uint8_t*)src, n, dst); return 0;
     case TSO_TYPE_MXFP4: dequant_mxfp4((const uint8_t*)src, n, dst); return 0;
     case TSO_TYPE_F16: dequant_f16((const uint8_t*)src, n, dst); return 0;

@@ -22,7 +22,7 @@ extern "C" {
 /* GGUF tensor type ids: TensorSharp.Runtime/GgufReader.cs:26-37 */
 enum {
     TSO_TYPE_F32 = 0, TSO_TYPE_F16 = 1, TSO_TYPE_Q4_0 = 2, TSO_TYPE_Q4_1 = 3, TSO_TYPE_Q5_0 = 6, TSO_TYPE_Q5_1 = 7,
-    TSO_TYPE_Q8_0 = 8, TSO_TYPE_Q4_K = 12, TSO_TYPE_Q5_K = 13, TSO_TYPE_Q6_K = 14, TSO_TYPE_IQ4_NL = 20,
+    TSO_TYPE_Q8_0 = 8, TSO_TYPE_Q8_1 = 9, TSO_TYPE_Q4_K = 12, TSO_TYPE_Q5_K = 13, TSO_TYPE_Q6_K = 14, TSO_TYPE_IQ4_NL = 20,
     TSO_TYPE_BF16 = 30, TSO_TYPE_MXFP4 = 39
 };
 

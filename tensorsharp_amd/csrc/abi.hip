@@ -241,6 +241,10 @@ size_t row_size(int type, int64_t ne)
     return (size_t)(ne / bs * block_bytes(type));
 }
 
+const char* const kUnsupportedTypeMessage =
+    "Unsupported weight type for the HIP backend (supported: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q4_K, Q5_K, Q6_K, IQ4_NL, MXFP4, "
+    "F32, F16, BF16).";
+
 // shape agreement + weight descriptor, messages as in ggml_ops_matmul.cpp:303-329
 bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView2D& m1, const void* m2_data, int type,
                           int64_t ne0, int64_t ne1, int64_t raw_bytes)
@@ -258,8 +262,8 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
         set_last_error("Size mismatch: quantized weight dims don't match in addmm_quant.");
         return false;
     }
-    if (!is_quant_type(type)) {
-        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, MXFP4).");
+    if (!is_matmul_type(type)) {
+        set_last_error(kUnsupportedTypeMessage);
         return false;
     }
     const size_t rs = row_size(type, ne0);
@@ -278,7 +282,8 @@ bool validate_addmm_quant(const TSHipTensorView2D& result, const TSHipTensorView
 bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
 {
     const uintptr_t wa = reinterpret_cast<uintptr_t>(w);
-    const uintptr_t need_align = (type == kTypeQ4_K || type == kTypeQ5_K) ? 16 : (type == kTypeMXFP4) ? 1 : 2;
+    const uintptr_t need_align = is_dense_type(type) ? (uintptr_t)block_bytes(type) : type == kTypeQ8_1 ? 1
+                                 : (type == kTypeQ4_K || type == kTypeQ5_K) ? 16 : (type == kTypeMXFP4) ? 1 : 2;
     if (wa % need_align != 0) {
         set_last_error("Quantized weight pointer is not aligned for its block type.");
         return false;
@@ -294,6 +299,8 @@ bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
 // The kernels address a weight, and the converted activations of a launch, with 32-bit offsets.  Larger operands are
 // cut by rows inside the call, as the bridge does when a buffer passes INT_MAX (ggml_ops_matmul.cpp:331-367): weight
 // rows (output columns) in slices below 2 GiB, activation rows in slices whose fp16 copy stays below 2 GiB.
+constexpr size_t kQ81SliceBytes = (size_t)32 << 20;
+
 struct MatmulPlan {
     bool gemv;            // decode / tiny batch: one bandwidth-bound GEMV per activation row
     int m_step;           // activation rows per launch
@@ -309,6 +316,17 @@ MatmulPlan plan_matmul(int type, int M, int64_t K, int64_t N, bool norm, bool ac
     MatmulPlan p{};
     const size_t rs = row_size(type, K);
     p.n_step = N;
+    if (is_dense_type(type) || type == kTypeQ8_1) {
+        // dense weights: one kernel with 64-bit addressing, no conversion of the activations
+        p.m_step = M;
+        p.conv_bytes = norm ? al((size_t)M * (size_t)K * sizeof(float)) : 0;
+        if (type == kTypeQ8_1) {
+            // fp32 copies of at most kQ81SliceBytes of weight rows at a time
+            p.n_step = std::min<int64_t>(N, std::max<int64_t>(1, (int64_t)(kQ81SliceBytes / ((size_t)K * sizeof(float)))));
+            p.chunk_bytes = al((size_t)p.n_step * (size_t)K * sizeof(float));
+        }
+        return p;
+    }
     if (rs * (size_t)N >= (size_t)kMaxOperandBytes) {
         // slices of whole rows; a multiple of 256 rows keeps every slice's first row as aligned as the tensor itself
         p.n_step = std::max<int64_t>(256, (int64_t)((size_t)(kMaxOperandBytes - 1) / rs) / 256 * 256);
@@ -353,6 +371,27 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
     }
     const uint8_t* wb = static_cast<const uint8_t*>(w);
     float* out = static_cast<float*>(result.data);
+    if (is_dense_type(type) || type == kTypeQ8_1) {
+        const float* xs = static_cast<const float*>(m1.data);
+        int64_t ldx = m1.stride0;
+        if (norm_w) {
+            if (!launch_rms_norm_rows(xs, ldx, norm_w, eps, M, (int)K, static_cast<float*>(ws), stream)) return false;
+            xs = static_cast<const float*>(ws);
+            ldx = K;
+        }
+        if (type != kTypeQ8_1) return launch_dense_matmul(type, w, xs, ldx, out, result.stride0, M, (int)N, (int)K, accumulate, stream);
+        if (plan.total() > ws_bytes) {
+            set_last_error("matmul: the device workspace is too small for the fp32 copy of a Q8_1 weight slice.");
+            return false;
+        }
+        float* rows = reinterpret_cast<float*>(static_cast<char*>(ws) + plan.conv_bytes);
+        for (int64_t n0 = 0; n0 < N; n0 += plan.n_step) {
+            const int64_t n = std::min<int64_t>(plan.n_step, N - n0);
+            if (!launch_dequant(type, wb + (size_t)n0 * rs, n * K, rows, stream)) return false;
+            if (!launch_dense_matmul(kTypeF32, rows, xs, ldx, out + n0, result.stride0, M, (int)n, (int)K, accumulate, stream)) return false;
+        }
+        return true;
+    }
     if (plan.gemv) {
         const float* xs = static_cast<const float*>(m1.data);
         int64_t ldx = m1.stride0;
@@ -465,6 +504,138 @@ bool run_ffn_swiglu_device(const TSHipTensorView2D& residual, const TSHipTensorV
     if (!launch_silu_mul(gu, 2 * half, M, half, act, stream)) return false;
     const TSHipTensorView2D act_view{act, M, half, half, 1, (int64_t)((size_t)M * half * sizeof(float))};
     return run_matmul_device_ws(residual, act_view, down, dn_type, half, hidden, stream, mm_ws, mm_bytes, nullptr, 0.f, true);
+}
+
+// ---- a weighted set of expert FFNs on device operands ------------------------------------------
+// out = (base ? base : 0) + sum_e weight_e * W_down[e] * act_e(x), experts added in index order, with
+//   act_e(x) = silu(W_gate[e] x) * (W_up[e] x)      when the expert has a gate weight   (ggml_ops_fused.cpp:1876-1890)
+//            = max(W_up[e] x, 0)^2                  when it has none                    (ggml_ops_fused.cpp:1700-1722)
+// Every expert maps H -> I -> N.  The routed experts of the bridge calls share their types; a shared expert may differ.
+constexpr int kMaxExpertSet = 33;   // 32 routed experts and one shared expert
+struct ExpertFfn {
+    const void* gate;   // device pointers to raw blocks; gate == nullptr selects the squared-ReLU expert
+    const void* up;
+    const void* down;
+    int gate_type, up_type, down_type;
+    float weight;
+};
+
+struct ExpertSetLayout {
+    size_t act_stride;   // floats between the activation rows of consecutive experts
+    size_t dn_stride;    // floats between their down outputs
+    size_t act_off, dn_off, tmp_off, mm_off, mm_bytes, total;
+};
+
+ExpertSetLayout expert_set_layout(int M, int n, const ExpertFfn* ex, int H, int I, int N)
+{
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    ExpertSetLayout L{};
+    L.act_stride = al((size_t)M * 2 * I * sizeof(float)) / sizeof(float);
+    L.dn_stride = al((size_t)M * N * sizeof(float)) / sizeof(float);
+    L.act_off = 0;
+    L.dn_off = L.act_off + (size_t)n * L.act_stride * sizeof(float);
+    L.tmp_off = L.dn_off + (size_t)n * L.dn_stride * sizeof(float);
+    L.mm_off = L.tmp_off + al((size_t)M * I * sizeof(float));
+    for (int e = 0; e < n; ++e) {
+        if (ex[e].gate) L.mm_bytes = std::max(L.mm_bytes, matmul_ws_bytes(ex[e].gate_type, M, H, I, false, false));
+        L.mm_bytes = std::max(L.mm_bytes, matmul_ws_bytes(ex[e].up_type, M, H, I, false, false));
+        L.mm_bytes = std::max(L.mm_bytes, matmul_ws_bytes(ex[e].down_type, M, I, N, false, false));
+    }
+    L.total = L.mm_off + L.mm_bytes;
+    return L;
+}
+
+// problems of one block type, at most gemv_max_group() per launch
+bool launch_gemv_batches(int type, std::vector<GemvArgs>& list, hipStream_t stream)
+{
+    const int group = gemv_max_group();
+    for (size_t i = 0; i < list.size(); i += (size_t)group)
+        if (!launch_gemv_group(type, (int)std::min<size_t>((size_t)group, list.size() - i), list.data() + i, stream)) return false;
+    return true;
+}
+
+bool run_expert_set_device(const TSHipTensorView2D& out, const float* base, int64_t ldb, const TSHipTensorView2D& x, int n,
+                           const ExpertFfn* ex, int H, int I, int N, hipStream_t stream, char* ws)
+{
+    const int M = x.dim0;
+    const ExpertSetLayout L = expert_set_layout(M, n, ex, H, I, N);
+    float* act = reinterpret_cast<float*>(ws + L.act_off);
+    float* dn = reinterpret_cast<float*>(ws + L.dn_off);
+    float* tmp = reinterpret_cast<float*>(ws + L.tmp_off);
+    void* mm_ws = ws + L.mm_off;
+    WeightedSumCoeffs coeffs{};
+    for (int e = 0; e < n; ++e) coeffs.v[e] = ex[e].weight;
+
+    // single token, every format with a GEMV: the experts' linears run as grouped GEMV launches
+    bool grouped = M == 1;
+    for (int e = 0; e < n && grouped; ++e) {
+        auto fits = [](int type, int64_t rows, int64_t k) {
+            return has_gemv(type) && k <= gemv_max_k(type) && row_size(type, k) * (size_t)rows < (size_t)kMaxOperandBytes;
+        };
+        grouped = fits(ex[e].up_type, I, H) && fits(ex[e].down_type, N, I) && (!ex[e].gate || fits(ex[e].gate_type, I, H));
+    }
+    if (grouped) {
+        const float* xv = static_cast<const float*>(x.data);
+        const int types[] = {kTypeQ8_0, kTypeQ4_K, kTypeMXFP4, kTypeQ6_K, kTypeQ5_K, kTypeQ4_0, kTypeQ4_1};
+        for (int e = 0; e < n; ++e)
+            if (!check_device_operands(x, ex[e].up, ex[e].up_type) || !check_device_operands(x, ex[e].down, ex[e].down_type) ||
+                (ex[e].gate && !check_device_operands(x, ex[e].gate, ex[e].gate_type)))
+                return false;
+        std::vector<GemvArgs> list;
+        for (int t : types) {      // gate and up projections: x -> act[e] = [gate | up] (or [up] alone)
+            list.clear();
+            for (int e = 0; e < n; ++e) {
+                float* row = act + (size_t)e * L.act_stride;
+                if (ex[e].gate && ex[e].gate_type == t) {
+                    GemvArgs a{};
+                    a.w = ex[e].gate, a.w_bytes = (int64_t)(row_size(t, H) * (size_t)I), a.x = xv, a.y = row, a.N = I, a.K = H;
+                    list.push_back(a);
+                }
+                if (ex[e].up_type == t) {
+                    GemvArgs a{};
+                    a.w = ex[e].up, a.w_bytes = (int64_t)(row_size(t, H) * (size_t)I), a.x = xv, a.y = ex[e].gate ? row + I : row, a.N = I, a.K = H;
+                    list.push_back(a);
+                }
+            }
+            if (!launch_gemv_batches(t, list, stream)) return false;
+        }
+        for (int e = 0; e < n; ++e)
+            if (!ex[e].gate && !launch_relu_sqr(act + (size_t)e * L.act_stride, I, stream)) return false;
+        for (int t : types)        // down projections; the gated product is formed while the activation row is staged
+            for (int gated = 0; gated < 2; ++gated) {
+                list.clear();
+                for (int e = 0; e < n; ++e) {
+                    if (ex[e].down_type != t || (ex[e].gate != nullptr) != (gated != 0)) continue;
+                    GemvArgs a{};
+                    a.w = ex[e].down, a.w_bytes = (int64_t)(row_size(t, I) * (size_t)N), a.x = act + (size_t)e * L.act_stride;
+                    a.y = dn + (size_t)e * L.dn_stride, a.N = N, a.K = I, a.act = gated ? 2 : 0;
+                    list.push_back(a);
+                }
+                if (!launch_gemv_batches(t, list, stream)) return false;
+            }
+    } else {
+        for (int e = 0; e < n; ++e) {
+            float* a_e = act + (size_t)e * L.act_stride;
+            float* d_e = dn + (size_t)e * L.dn_stride;
+            const TSHipTensorView2D d_view{d_e, M, N, N, 1, (int64_t)((size_t)M * N * sizeof(float))};
+            if (ex[e].gate) {
+                const int64_t span = (int64_t)(((size_t)(M - 1) * 2 * I + I) * sizeof(float));
+                const TSHipTensorView2D g_view{a_e, M, I, 2 * I, 1, span};
+                const TSHipTensorView2D u_view{a_e + I, M, I, 2 * I, 1, span};
+                if (!run_matmul_device_ws(g_view, x, ex[e].gate, ex[e].gate_type, H, I, stream, mm_ws, L.mm_bytes, nullptr, 0.f, false)) return false;
+                if (!run_matmul_device_ws(u_view, x, ex[e].up, ex[e].up_type, H, I, stream, mm_ws, L.mm_bytes, nullptr, 0.f, false)) return false;
+                if (!launch_silu_mul(a_e, 2 * I, M, I, tmp, stream)) return false;
+                const TSHipTensorView2D t_view{tmp, M, I, I, 1, (int64_t)((size_t)M * I * sizeof(float))};
+                if (!run_matmul_device_ws(d_view, t_view, ex[e].down, ex[e].down_type, I, N, stream, mm_ws, L.mm_bytes, nullptr, 0.f, false)) return false;
+            } else {
+                const TSHipTensorView2D u_view{a_e, M, I, I, 1, (int64_t)((size_t)M * I * sizeof(float))};
+                if (!run_matmul_device_ws(u_view, x, ex[e].up, ex[e].up_type, H, I, stream, mm_ws, L.mm_bytes, nullptr, 0.f, false)) return false;
+                if (!launch_relu_sqr(a_e, (int64_t)M * I, stream)) return false;
+                if (!run_matmul_device_ws(d_view, u_view, ex[e].down, ex[e].down_type, I, N, stream, mm_ws, L.mm_bytes, nullptr, 0.f, false)) return false;
+            }
+        }
+    }
+    return launch_weighted_sum(dn, (int64_t)L.dn_stride, coeffs, n, M, N, base, ldb, static_cast<float*>(out.data), out.stride0, stream);
 }
 
 // Device pointer for m2_data: preloaded key, cached host pointer, or upload now.  The caller holds g_host_call_mutex.
@@ -589,8 +760,8 @@ bool validate_weight(const void* data, int type, int64_t ne0, int64_t ne1, int64
         set_last_error(std::string("Invalid quantized weight descriptor for ") + what + ".");
         return false;
     }
-    if (!is_quant_type(type)) {
-        set_last_error("Unsupported quantized weight type for the HIP backend (supported: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, MXFP4).");
+    if (!is_matmul_type(type)) {
+        set_last_error(kUnsupportedTypeMessage);
         return false;
     }
     const size_t rs = row_size(type, ne0);
@@ -713,6 +884,268 @@ int with_host_tensors(const TSHipTensorView2D& inout, bool upload_inout, const T
     for (int m = 0; m < M; ++m) std::memcpy(io + (size_t)m * inout.stride0, stage_y + (size_t)m * N, N * sizeof(float));
     clear_last_error();
     return 1;
+}
+
+// Several host tensors around a device computation.  Each tensor is packed to [dim0 x dim1] in one pinned region,
+// the region goes up in one copy, body(dev_views, norm_dev, stream) runs, the region comes back in one copy and the
+// tensors marked `down` are written to the caller's views.
+struct HostTensor {
+    const TSHipTensorView2D* view;
+    bool up;
+    bool down;
+};
+
+template <typename Body>
+int with_host_io(const HostTensor* t, int count, const void* norm_w, int norm_count, Body&& body)
+{
+    constexpr int kMaxIo = 6;
+    if (count > kMaxIo) {
+        set_last_error("Too many host tensors in one call.");
+        return 0;
+    }
+    std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    size_t off[kMaxIo + 1], total = 0;
+    for (int i = 0; i < count; ++i) {
+        off[i] = total;
+        total += al((size_t)t[i].view->dim0 * (size_t)t[i].view->dim1 * sizeof(float));
+    }
+    off[count] = total;
+    total += al((size_t)std::max(norm_count, 0) * sizeof(float));
+    if (!ws_reserve(total, total)) return 0;
+    char* dev = static_cast<char*>(g_ws.dev);
+    char* pin = static_cast<char*>(g_ws.pinned);
+    TSHipTensorView2D dv[kMaxIo];
+    for (int i = 0; i < count; ++i) {
+        const TSHipTensorView2D& v = *t[i].view;
+        dv[i] = TSHipTensorView2D{dev + off[i], v.dim0, v.dim1, v.dim1, 1, (int64_t)((size_t)v.dim0 * (size_t)v.dim1 * sizeof(float))};
+        if (!t[i].up) continue;
+        float* stage = reinterpret_cast<float*>(pin + off[i]);
+        const float* src = static_cast<const float*>(v.data);
+        for (int m = 0; m < v.dim0; ++m) {
+            if (v.stride1 == 1) {
+                std::memcpy(stage + (size_t)m * v.dim1, src + (size_t)m * v.stride0, (size_t)v.dim1 * sizeof(float));
+            } else {
+                for (int k = 0; k < v.dim1; ++k) stage[(size_t)m * v.dim1 + k] = src[(size_t)m * v.stride0 + (size_t)k * v.stride1];
+            }
+        }
+    }
+    if (norm_w) std::memcpy(pin + off[count], norm_w, (size_t)norm_count * sizeof(float));
+    hipStream_t stream = nullptr;
+    for (int i = 0; i <= count; ++i) {
+        const bool wanted = i < count ? t[i].up : norm_w != nullptr;
+        const size_t bytes = i < count ? (size_t)dv[i].raw_bytes : (size_t)std::max(norm_count, 0) * sizeof(float);
+        if (wanted && !hip_ok(hipMemcpyAsync(dev + off[i], pin + off[i], bytes, hipMemcpyHostToDevice, stream), "hipMemcpy(inputs)")) return 0;
+    }
+    if (!body(dv, norm_w ? reinterpret_cast<const float*>(dev + off[count]) : nullptr, stream)) return 0;
+    for (int i = 0; i < count; ++i)
+        if (t[i].down && !hip_ok(hipMemcpyAsync(pin + off[i], dev + off[i], (size_t)dv[i].raw_bytes, hipMemcpyDeviceToHost, stream), "hipMemcpy(result)"))
+            return 0;
+    if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+    for (int i = 0; i < count; ++i) {
+        if (!t[i].down) continue;
+        const TSHipTensorView2D& v = *t[i].view;
+        const float* stage = reinterpret_cast<const float*>(pin + off[i]);
+        float* dst = static_cast<float*>(v.data);
+        for (int m = 0; m < v.dim0; ++m) {
+            if (v.stride1 == 1) {
+                std::memcpy(dst + (size_t)m * v.stride0, stage + (size_t)m * v.dim1, (size_t)v.dim1 * sizeof(float));
+            } else {
+                for (int k = 0; k < v.dim1; ++k) dst[(size_t)m * v.stride0 + (size_t)k * v.stride1] = stage[(size_t)m * v.dim1 + k];
+            }
+        }
+    }
+    clear_last_error();
+    return 1;
+}
+
+struct WeightDesc {
+    const void* data;
+    int type;
+    int64_t ne0, ne1, raw_bytes;
+    size_t bytes() const { return row_size(type, ne0) * (size_t)ne1; }
+};
+
+// residual [M x hidden] += input [M x ne0] * W_out^T, then (ffn) the SwiGLU FFN on the new residual
+bool validate_outproj(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const WeightDesc& out_w, const void* norm_w,
+                      int norm_count, const char* what)
+{
+    if (!validate_desc(residual, "residual") || !validate_desc(input, "input")) return false;
+    if (!validate_weight(out_w.data, out_w.type, out_w.ne0, out_w.ne1, out_w.raw_bytes, what)) return false;
+    if (norm_w == nullptr || norm_count <= 0) {
+        set_last_error(std::string(what) + ": invalid norm weight.");
+        return false;
+    }
+    if (residual.dim0 != input.dim0 || out_w.ne0 != input.dim1 || out_w.ne1 != residual.dim1 || norm_count != residual.dim1) {
+        set_last_error(std::string(what) + ": shape mismatch between residual, input, the output projection and the norm weight.");
+        return false;
+    }
+    if (residual.stride1 != 1) {
+        set_last_error(std::string(what) + ": residual must be a standard (stride1 == 1) view.");
+        return false;
+    }
+    return true;
+}
+
+bool validate_outproj_ffn(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const WeightDesc& out_w, const void* norm_w,
+                          int norm_count, const WeightDesc& gu, const WeightDesc& dn, int half_dim)
+{
+    if (!validate_outproj(residual, input, out_w, norm_w, norm_count, "fused_outproj_ffn")) return false;
+    if (!validate_weight(gu.data, gu.type, gu.ne0, gu.ne1, gu.raw_bytes, "fused_outproj_ffn gate_up")) return false;
+    if (!validate_weight(dn.data, dn.type, dn.ne0, dn.ne1, dn.raw_bytes, "fused_outproj_ffn down")) return false;
+    const int hidden = residual.dim1;
+    if (half_dim <= 0 || gu.ne0 != hidden || gu.ne1 != 2 * (int64_t)half_dim || dn.ne0 != half_dim || dn.ne1 != hidden) {
+        set_last_error("fused_outproj_ffn: gate_up / down weight shape mismatch.");
+        return false;
+    }
+    return true;
+}
+
+size_t outproj_ffn_ws_bytes(int M, const WeightDesc& out_w, const WeightDesc& gu, const WeightDesc& dn, int hidden, int half)
+{
+    return std::max(matmul_ws_bytes(out_w.type, M, out_w.ne0, out_w.ne1, false, true), ffn_ws_bytes(M, gu.type, dn.type, hidden, half));
+}
+
+bool run_outproj_ffn_device(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const void* out_w, const WeightDesc& od,
+                            const float* norm_w, float eps, const void* gu, int gu_type, const void* dn, int dn_type, int half,
+                            hipStream_t stream, char* ws, size_t ws_bytes)
+{
+    if (!run_matmul_device_ws(residual, input, out_w, od.type, od.ne0, od.ne1, stream, ws, ws_bytes, nullptr, 0.f, true)) return false;
+    return run_ffn_swiglu_device(residual, residual, norm_w, eps, gu, gu_type, dn, dn_type, residual.dim1, half, stream, ws);
+}
+
+bool validate_outproj_router(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const WeightDesc& out_w, const void* norm_w,
+                             int norm_count, const TSHipTensorView2D& normed_out, const WeightDesc& router, const TSHipTensorView2D& router_out)
+{
+    if (!validate_outproj(residual, input, out_w, norm_w, norm_count, "fused_outproj_norm_router")) return false;
+    if (!validate_desc(normed_out, "normedOut") || !validate_desc(router_out, "routerOut")) return false;
+    if (!validate_weight(router.data, router.type, router.ne0, router.ne1, router.raw_bytes, "fused_outproj_norm_router router")) return false;
+    const int hidden = residual.dim1;
+    if (normed_out.dim0 != residual.dim0 || normed_out.dim1 != hidden || router_out.dim0 != residual.dim0 || router.ne0 != hidden ||
+        router.ne1 != router_out.dim1) {
+        set_last_error("fused_outproj_norm_router: normedOut / router shape mismatch.");
+        return false;
+    }
+    return true;
+}
+
+size_t outproj_router_ws_bytes(int M, const WeightDesc& out_w, const WeightDesc& router)
+{
+    return std::max(matmul_ws_bytes(out_w.type, M, out_w.ne0, out_w.ne1, false, true), matmul_ws_bytes(router.type, M, router.ne0, router.ne1, false, false));
+}
+
+// residual += input * W_out^T; normed_out = RMSNorm(residual) * norm_w; router_out = normed_out * W_router^T
+// (ggml_ops_fused.cpp:1310-1330).  normed_out must be a contiguous [M x hidden] device view.
+bool run_outproj_router_device(const TSHipTensorView2D& residual, const TSHipTensorView2D& input, const void* out_w, const WeightDesc& od,
+                               const float* norm_w, float eps, const TSHipTensorView2D& normed_out, const void* router_w,
+                               const WeightDesc& rd, const TSHipTensorView2D& router_out, hipStream_t stream, char* ws, size_t ws_bytes)
+{
+    if (normed_out.stride1 != 1 || (normed_out.dim0 > 1 && normed_out.stride0 != normed_out.dim1) || router_out.stride1 != 1) {
+        set_last_error("fused_outproj_norm_router: normedOut must be contiguous and routerOut a standard view on the device.");
+        return false;
+    }
+    if (!run_matmul_device_ws(residual, input, out_w, od.type, od.ne0, od.ne1, stream, ws, ws_bytes, nullptr, 0.f, true)) return false;
+    if (!launch_rms_norm_rows(static_cast<const float*>(residual.data), residual.stride0, norm_w, eps, residual.dim0, residual.dim1,
+                              static_cast<float*>(normed_out.data), stream))
+        return false;
+    return run_matmul_device_ws(router_out, normed_out, router_w, rd.type, rd.ne0, rd.ne1, stream, ws, ws_bytes, nullptr, 0.f, false);
+}
+
+// ---- weighted expert sets (the bridge's per-token MoE calls) ------------------------------------
+struct ExpertSetArgs {
+    const char* what;
+    int max_experts;
+    int num_experts;
+    bool gated;            // SwiGLU experts (gate, up, down); otherwise squared-ReLU experts (up, down)
+    void* const* gate;
+    void* const* up;
+    void* const* down;
+    WeightDesc gate_d, up_d, down_d;     // data unused; shapes shared by the routed experts
+    const float* route_weights;
+    bool has_shared;
+    WeightDesc sh_gate, sh_up, sh_down;
+    float shared_scalar;
+};
+
+bool validate_expert_set(const TSHipTensorView2D& out, const TSHipTensorView2D& input, const ExpertSetArgs& a, const char* out_name)
+{
+    if (!validate_desc(out, out_name) || !validate_desc(input, "input")) return false;
+    if (a.num_experts <= 0 || a.num_experts > a.max_experts) {
+        set_last_error(std::string(a.what) + ": num_experts must be 1.." + std::to_string(a.max_experts));
+        return false;
+    }
+    if ((a.gated && a.gate == nullptr) || a.up == nullptr || a.down == nullptr || a.route_weights == nullptr) {
+        set_last_error(std::string(a.what) + ": null expert pointer array or route weights.");
+        return false;
+    }
+    const std::string w = a.what;
+    for (int e = 0; e < a.num_experts; ++e) {
+        if (a.gate && !validate_weight(a.gate[e], a.gate_d.type, a.gate_d.ne0, a.gate_d.ne1, a.gate_d.raw_bytes, (w + " gate").c_str())) return false;
+        if (!validate_weight(a.up[e], a.up_d.type, a.up_d.ne0, a.up_d.ne1, a.up_d.raw_bytes, (w + " up").c_str())) return false;
+        if (!validate_weight(a.down[e], a.down_d.type, a.down_d.ne0, a.down_d.ne1, a.down_d.raw_bytes, (w + " down").c_str())) return false;
+    }
+    const int64_t H = input.dim1, I = a.up_d.ne1, N = out.dim1;
+    bool ok = out.dim0 == input.dim0 && a.up_d.ne0 == H && a.down_d.ne0 == I && a.down_d.ne1 == N &&
+              (!a.gate || (a.gate_d.ne0 == H && a.gate_d.ne1 == I));
+    if (a.has_shared) {
+        if (!validate_weight(a.sh_gate.data, a.sh_gate.type, a.sh_gate.ne0, a.sh_gate.ne1, a.sh_gate.raw_bytes, (w + " shared gate").c_str()) ||
+            !validate_weight(a.sh_up.data, a.sh_up.type, a.sh_up.ne0, a.sh_up.ne1, a.sh_up.raw_bytes, (w + " shared up").c_str()) ||
+            !validate_weight(a.sh_down.data, a.sh_down.type, a.sh_down.ne0, a.sh_down.ne1, a.sh_down.raw_bytes, (w + " shared down").c_str()))
+            return false;
+        // the shared expert may have its own intermediate width
+        ok = ok && a.sh_gate.ne0 == H && a.sh_up.ne0 == H && a.sh_gate.ne1 == a.sh_up.ne1 && a.sh_down.ne0 == a.sh_up.ne1 && a.sh_down.ne1 == N;
+    }
+    if (!ok) {
+        set_last_error(w + ": weight shapes do not match the input / output tensors.");
+        return false;
+    }
+    if (out.stride1 != 1) {
+        set_last_error(w + ": the output must be a standard (stride1 == 1) view.");
+        return false;
+    }
+    return true;
+}
+
+// Runs a validated expert set on device views; `resolve` maps a caller pointer to the device address of its blocks.
+// The shared expert runs as a set of its own (its width may differ) and is added after the routed experts.
+template <typename Resolve>
+bool run_expert_set(const TSHipTensorView2D& out, bool add_to_out, const TSHipTensorView2D& x, const ExpertSetArgs& a, hipStream_t stream,
+                    Resolve&& resolve)
+{
+    ExpertFfn ex[kMaxExpertSet];
+    const int n = a.num_experts;
+    for (int e = 0; e < n; ++e) {
+        ex[e].gate = a.gate ? resolve(a.gate[e], a.gate_d.bytes()) : nullptr;
+        ex[e].up = resolve(a.up[e], a.up_d.bytes());
+        ex[e].down = resolve(a.down[e], a.down_d.bytes());
+        if ((a.gate && !ex[e].gate) || !ex[e].up || !ex[e].down) return false;
+        ex[e].gate_type = a.gate_d.type, ex[e].up_type = a.up_d.type, ex[e].down_type = a.down_d.type;
+        ex[e].weight = a.route_weights[e];
+    }
+    const int M = x.dim0, H = x.dim1, I = (int)a.up_d.ne1, N = out.dim1;
+    const bool same_width = a.has_shared && a.sh_up.ne1 == a.up_d.ne1;
+    ExpertFfn sh{};
+    if (a.has_shared) {
+        sh.gate = resolve(const_cast<void*>(a.sh_gate.data), a.sh_gate.bytes());
+        sh.up = resolve(const_cast<void*>(a.sh_up.data), a.sh_up.bytes());
+        sh.down = resolve(const_cast<void*>(a.sh_down.data), a.sh_down.bytes());
+        if (!sh.gate || !sh.up || !sh.down) return false;
+        sh.gate_type = a.sh_gate.type, sh.up_type = a.sh_up.type, sh.down_type = a.sh_down.type;
+        sh.weight = a.shared_scalar;
+    }
+    int count = n;
+    if (same_width) ex[count++] = sh;     // one weighted sum over routed + shared, in the bridge's order
+    const size_t need = std::max(expert_set_layout(M, count, ex, H, I, N).total,
+                                 a.has_shared && !same_width ? expert_set_layout(M, 1, &sh, H, (int)a.sh_up.ne1, N).total : (size_t)0);
+    WsLease ws(stream, need);
+    if (!ws.ok()) return false;
+    const float* base = add_to_out ? static_cast<const float*>(out.data) : nullptr;
+    if (a.has_shared && !same_width) {
+        // (routed sum) + shared, then + residual: the shared term is added into a copy-free second pass on `out`
+        if (!run_expert_set_device(out, base, out.stride0, x, n, ex, H, I, N, stream, ws.ptr())) return false;
+        return run_expert_set_device(out, static_cast<const float*>(out.data), out.stride0, x, 1, &sh, H, (int)a.sh_up.ne1, N, stream, ws.ptr());
+    }
+    return run_expert_set_device(out, base, out.stride0, x, count, ex, H, I, N, stream, ws.ptr());
 }
 
 }  // namespace
@@ -910,7 +1343,7 @@ int TSHip_MoERouteF32Device(TSHipTensorView2D logits, int k, int32_t* ids, float
     });
 }
 
-int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D hidden, const int32_t* ids,
+int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D hidden, const int32_t* ids,
                                      const float* weights, int k, const void* gate_up_w, const float* gate_up_bias,
                                      const void* down_w, const float* down_bias, int ggml_type, int n_experts, int64_t H,
                                      int64_t F, float alpha, float limit)
@@ -1034,7 +1467,7 @@ int TSHip_AddmmQuantBatchF32(TSHipTensorView2D result, TSHipTensorView2D m1, voi
             return 0;
         }
         const size_t rs = row_size(m2_ggml_type, m2_ne0);
-        if (!is_quant_type(m2_ggml_type) || rs == 0) {
+        if (!is_matmul_type(m2_ggml_type) || rs == 0) {
             set_last_error("Unsupported quantized weight type or row length for addmm_quant_batch.");
             return 0;
         }
@@ -1083,7 +1516,7 @@ int TSHip_PreloadQuantizedWeight(void* cache_key, void* host_data, int ggml_type
             return 0;
         }
         const size_t rs = row_size(ggml_type, ne0);
-        if (!is_quant_type(ggml_type) || rs == 0 || (size_t)raw_bytes < rs * (size_t)ne1) {
+        if (!is_matmul_type(ggml_type) || rs == 0 || (size_t)raw_bytes < rs * (size_t)ne1) {
             set_last_error("Unsupported type or inconsistent size for quantized weight preload.");
             return 0;
         }
@@ -1400,6 +1833,263 @@ int TSHip_FusedFFNSwiGLUQuantF32(TSHipTensorView2D residual, TSHipTensorView2D i
                                      return ws.ok() && run_ffn_swiglu_device(y, x, nw, eps, gu, gate_up_ggml_type, dn, down_ggml_type, x.dim1,
                                                                              half_dim, st, ws.ptr());
                                  });
+    });
+}
+
+int TSHip_FusedOutProjFFNQuantF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, const void* out_proj_data,
+                                        int out_proj_type, int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes,
+                                        const float* ffn_norm_weight, int ffn_norm_count, float eps, const void* gu_data, int gu_type,
+                                        int64_t gu_ne0, int64_t gu_ne1, int64_t gu_raw_bytes, const void* dn_data, int dn_type,
+                                        int64_t dn_ne0, int64_t dn_ne1, int64_t dn_raw_bytes, int half_dim)
+{
+    return guarded(0, "fused_outproj_ffn", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        const WeightDesc od{out_proj_data, out_proj_type, out_ne0, out_ne1, out_raw_bytes};
+        const WeightDesc gd{gu_data, gu_type, gu_ne0, gu_ne1, gu_raw_bytes}, dd{dn_data, dn_type, dn_ne0, dn_ne1, dn_raw_bytes};
+        if (!validate_outproj_ffn(residual, input, od, ffn_norm_weight, ffn_norm_count, gd, dd, half_dim)) return 0;
+        const size_t need = outproj_ffn_ws_bytes(input.dim0, od, gd, dd, residual.dim1, half_dim);
+        WsLease ws(t_stream, need);
+        if (!ws.ok()) return 0;
+        if (!run_outproj_ffn_device(residual, input, out_proj_data, od, ffn_norm_weight, eps, gu_data, gu_type, dn_data, dn_type, half_dim,
+                                    t_stream, ws.ptr(), need))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_FusedOutProjFFNQuantF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* out_proj_data, int out_proj_type,
+                                  int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes, void* ffn_norm_data, int ffn_norm_count,
+                                  float eps, void* gu_data, int gu_type, int64_t gu_ne0, int64_t gu_ne1, int64_t gu_raw_bytes,
+                                  void* dn_data, int dn_type, int64_t dn_ne0, int64_t dn_ne1, int64_t dn_raw_bytes, int half_dim)
+{
+    return guarded(0, "fused_outproj_ffn", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        const WeightDesc od{out_proj_data, out_proj_type, out_ne0, out_ne1, out_raw_bytes};
+        const WeightDesc gd{gu_data, gu_type, gu_ne0, gu_ne1, gu_raw_bytes}, dd{dn_data, dn_type, dn_ne0, dn_ne1, dn_raw_bytes};
+        if (!validate_outproj_ffn(residual, input, od, ffn_norm_data, ffn_norm_count, gd, dd, half_dim)) return 0;
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
+        const void* ow = resolve_weight(out_proj_data, od.bytes());
+        const void* gu = ow ? resolve_weight(gu_data, gd.bytes()) : nullptr;
+        const void* dn = gu ? resolve_weight(dn_data, dd.bytes()) : nullptr;
+        if (!dn) return 0;
+        const HostTensor io[2] = {{&residual, true, true}, {&input, true, false}};
+        return with_host_io(io, 2, ffn_norm_data, ffn_norm_count, [&](const TSHipTensorView2D* dv, const float* nw, hipStream_t st) {
+            const size_t need = outproj_ffn_ws_bytes(dv[1].dim0, od, gd, dd, dv[0].dim1, half_dim);
+            WsLease ws(st, need);
+            return ws.ok() && run_outproj_ffn_device(dv[0], dv[1], ow, od, nw, eps, gu, gu_type, dn, dn_type, half_dim, st, ws.ptr(), need);
+        });
+    });
+}
+
+int TSHip_FusedOutProjNormRouterQuantF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, const void* out_proj_data,
+                                               int out_proj_type, int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes,
+                                               const float* norm_weight, int norm_count, float eps, TSHipTensorView2D normed_out,
+                                               const void* router_data, int router_type, int64_t router_ne0, int64_t router_ne1,
+                                               int64_t router_raw_bytes, TSHipTensorView2D router_out)
+{
+    return guarded(0, "fused_outproj_norm_router", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        const WeightDesc od{out_proj_data, out_proj_type, out_ne0, out_ne1, out_raw_bytes};
+        const WeightDesc rd{router_data, router_type, router_ne0, router_ne1, router_raw_bytes};
+        if (!validate_outproj_router(residual, input, od, norm_weight, norm_count, normed_out, rd, router_out)) return 0;
+        const size_t need = outproj_router_ws_bytes(input.dim0, od, rd);
+        WsLease ws(t_stream, need);
+        if (!ws.ok()) return 0;
+        if (!run_outproj_router_device(residual, input, out_proj_data, od, norm_weight, eps, normed_out, router_data, rd, router_out,
+                                       t_stream, ws.ptr(), need))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_FusedOutProjNormRouterQuantF32(TSHipTensorView2D residual, TSHipTensorView2D input, void* out_proj_data, int out_proj_type,
+                                         int64_t out_ne0, int64_t out_ne1, int64_t out_raw_bytes, void* norm_data, int norm_count,
+                                         float eps, TSHipTensorView2D normed_out, void* router_data, int router_type,
+                                         int64_t router_ne0, int64_t router_ne1, int64_t router_raw_bytes, TSHipTensorView2D router_out)
+{
+    return guarded(0, "fused_outproj_norm_router", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        const WeightDesc od{out_proj_data, out_proj_type, out_ne0, out_ne1, out_raw_bytes};
+        const WeightDesc rd{router_data, router_type, router_ne0, router_ne1, router_raw_bytes};
+        if (!validate_outproj_router(residual, input, od, norm_data, norm_count, normed_out, rd, router_out)) return 0;
+        std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
+        const void* ow = resolve_weight(out_proj_data, od.bytes());
+        const void* rw = ow ? resolve_weight(router_data, rd.bytes()) : nullptr;
+        if (!rw) return 0;
+        const HostTensor io[4] = {{&residual, true, true}, {&input, true, false}, {&normed_out, false, true}, {&router_out, false, true}};
+        return with_host_io(io, 4, norm_data, norm_count, [&](const TSHipTensorView2D* dv, const float* nw, hipStream_t st) {
+            const size_t need = outproj_router_ws_bytes(dv[1].dim0, od, rd);
+            WsLease ws(st, need);
+            return ws.ok() && run_outproj_router_device(dv[0], dv[1], ow, od, nw, eps, dv[2], rw, rd, dv[3], st, ws.ptr(), need);
+        });
+    });
+}
+
+/* ---- weighted expert sets (ggml_ops_fused.cpp:1576-2160) -------------------------------------- */
+namespace {
+
+// the caller's arrays hold device pointers
+int expert_set_device(TSHipTensorView2D out, bool add_to_out, TSHipTensorView2D input, const ExpertSetArgs& a, const char* out_name)
+{
+    if (!ensure_backend()) return 0;
+    if (!validate_expert_set(out, input, a, out_name)) return 0;
+    if (!run_expert_set(out, add_to_out, input, a, t_stream, [](void* p, size_t) -> const void* { return p; })) return 0;
+    clear_last_error();
+    return 1;
+}
+
+// the caller's arrays hold host pointers: each expert's blocks are cached on the device under its host address
+int expert_set_host(TSHipTensorView2D out, bool add_to_out, TSHipTensorView2D input, const ExpertSetArgs& a, const char* out_name)
+{
+    if (!ensure_backend()) return 0;
+    if (!validate_expert_set(out, input, a, out_name)) return 0;
+    std::lock_guard<std::recursive_mutex> call_lock(g_host_call_mutex);
+    const HostTensor io[2] = {{&out, add_to_out, true}, {&input, true, false}};
+    return with_host_io(io, 2, nullptr, 0, [&](const TSHipTensorView2D* dv, const float*, hipStream_t st) {
+        return run_expert_set(dv[0], add_to_out, dv[1], a, st, [](void* p, size_t bytes) { return resolve_weight(p, bytes); });
+    });
+}
+
+ExpertSetArgs relu2_args(int num_experts, void* const* up, void* const* down, int up_type, int64_t up_ne0, int64_t up_ne1,
+                         int64_t up_bytes, int down_type, int64_t down_ne0, int64_t down_ne1, int64_t down_bytes, const float* route_weights)
+{
+    ExpertSetArgs a{};
+    a.what = "MoE", a.max_experts = 16, a.num_experts = num_experts, a.gated = false, a.gate = nullptr, a.up = up, a.down = down;
+    a.up_d = WeightDesc{nullptr, up_type, up_ne0, up_ne1, up_bytes};
+    a.down_d = WeightDesc{nullptr, down_type, down_ne0, down_ne1, down_bytes};
+    a.route_weights = route_weights;
+    return a;
+}
+
+ExpertSetArgs swiglu_args(const char* what, int max_experts, int num_experts, void* const* gate, void* const* up, void* const* down,
+                          int gate_type, int64_t gate_ne0, int64_t gate_ne1, int64_t gate_bytes, int up_type, int64_t up_ne0,
+                          int64_t up_ne1, int64_t up_bytes, int down_type, int64_t down_ne0, int64_t down_ne1, int64_t down_bytes,
+                          const float* route_weights)
+{
+    ExpertSetArgs a{};
+    a.what = what, a.max_experts = max_experts, a.num_experts = num_experts, a.gated = true, a.gate = gate, a.up = up, a.down = down;
+    a.gate_d = WeightDesc{nullptr, gate_type, gate_ne0, gate_ne1, gate_bytes};
+    a.up_d = WeightDesc{nullptr, up_type, up_ne0, up_ne1, up_bytes};
+    a.down_d = WeightDesc{nullptr, down_type, down_ne0, down_ne1, down_bytes};
+    a.route_weights = route_weights;
+    return a;
+}
+
+void set_shared(ExpertSetArgs& a, int use_shared, void* gate, void* up, void* down, int gate_type, int64_t gate_ne0, int64_t gate_ne1,
+                int64_t gate_bytes, int up_type, int64_t up_ne0, int64_t up_ne1, int64_t up_bytes, int down_type, int64_t down_ne0,
+                int64_t down_ne1, int64_t down_bytes, float scalar)
+{
+    // as the bridge: the shared expert takes part only when the flag is set and all three weights are given
+    a.has_shared = use_shared != 0 && gate != nullptr && up != nullptr && down != nullptr;
+    a.sh_gate = WeightDesc{gate, gate_type, gate_ne0, gate_ne1, gate_bytes};
+    a.sh_up = WeightDesc{up, up_type, up_ne0, up_ne1, up_bytes};
+    a.sh_down = WeightDesc{down, down_type, down_ne0, down_ne1, down_bytes};
+    a.shared_scalar = scalar;
+}
+
+}  // namespace
+
+int TSHip_MoEExpertsForwardF32(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts, void** up_data_ptrs,
+                               void** down_data_ptrs, int up_ggml_type, int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each,
+                               int down_ggml_type, int64_t down_ne0, int64_t down_ne1, int64_t down_raw_bytes_each,
+                               float* route_weights)
+{
+    return guarded(0, "MoE experts", [&]() -> int {
+        return expert_set_host(result, false, input,
+                               relu2_args(num_experts, up_data_ptrs, down_data_ptrs, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
+                                          down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights),
+                               "result");
+    });
+}
+
+int TSHip_MoEExpertsForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts, void* const* up_data_ptrs,
+                                     void* const* down_data_ptrs, int up_ggml_type, int64_t up_ne0, int64_t up_ne1,
+                                     int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                     int64_t down_raw_bytes_each, const float* route_weights)
+{
+    return guarded(0, "MoE experts", [&]() -> int {
+        return expert_set_device(result, false, input,
+                                 relu2_args(num_experts, up_data_ptrs, down_data_ptrs, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
+                                            down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights),
+                                 "result");
+    });
+}
+
+int TSHip_MoEExpertsSwiGLUForwardF32(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts, void** gate_data_ptrs,
+                                     void** up_data_ptrs, void** down_data_ptrs, int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1,
+                                     int64_t gate_raw_bytes_each, int up_ggml_type, int64_t up_ne0, int64_t up_ne1,
+                                     int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                     int64_t down_raw_bytes_each, float* route_weights)
+{
+    return guarded(0, "MoE SwiGLU experts", [&]() -> int {
+        return expert_set_host(result, false, input,
+                               swiglu_args("MoE SwiGLU", 16, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
+                                           gate_ne0, gate_ne1, gate_raw_bytes_each, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
+                                           down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights),
+                               "result");
+    });
+}
+
+int TSHip_MoEExpertsSwiGLUForwardF32Device(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
+                                           void* const* gate_data_ptrs, void* const* up_data_ptrs, void* const* down_data_ptrs,
+                                           int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1, int64_t gate_raw_bytes_each,
+                                           int up_ggml_type, int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each,
+                                           int down_ggml_type, int64_t down_ne0, int64_t down_ne1, int64_t down_raw_bytes_each,
+                                           const float* route_weights)
+{
+    return guarded(0, "MoE SwiGLU experts", [&]() -> int {
+        return expert_set_device(result, false, input,
+                                 swiglu_args("MoE SwiGLU", 16, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
+                                             gate_ne0, gate_ne1, gate_raw_bytes_each, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
+                                             down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights),
+                                 "result");
+    });
+}
+
+int TSHip_MoEExpertsSwiGLUResidualF32(TSHipTensorView2D residual, TSHipTensorView2D input, int num_experts, void** gate_data_ptrs,
+                                      void** up_data_ptrs, void** down_data_ptrs, int gate_ggml_type, int64_t gate_ne0,
+                                      int64_t gate_ne1, int64_t gate_raw_bytes_each, int up_ggml_type, int64_t up_ne0, int64_t up_ne1,
+                                      int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0, int64_t down_ne1,
+                                      int64_t down_raw_bytes_each, float* route_weights, int use_shared, void* shared_gate_data,
+                                      void* shared_up_data, void* shared_down_data, int shared_gate_ggml_type, int64_t shared_gate_ne0,
+                                      int64_t shared_gate_ne1, int64_t shared_gate_raw_bytes, int shared_up_ggml_type,
+                                      int64_t shared_up_ne0, int64_t shared_up_ne1, int64_t shared_up_raw_bytes,
+                                      int shared_down_ggml_type, int64_t shared_down_ne0, int64_t shared_down_ne1,
+                                      int64_t shared_down_raw_bytes, float shared_scalar)
+{
+    return guarded(0, "MoE SwiGLU residual", [&]() -> int {
+        ExpertSetArgs a = swiglu_args("MoE SwiGLU residual", 32, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
+                                      gate_ne0, gate_ne1, gate_raw_bytes_each, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
+                                      down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights);
+        set_shared(a, use_shared, shared_gate_data, shared_up_data, shared_down_data, shared_gate_ggml_type, shared_gate_ne0, shared_gate_ne1,
+                   shared_gate_raw_bytes, shared_up_ggml_type, shared_up_ne0, shared_up_ne1, shared_up_raw_bytes, shared_down_ggml_type,
+                   shared_down_ne0, shared_down_ne1, shared_down_raw_bytes, shared_scalar);
+        return expert_set_host(residual, true, input, a, "residual");
+    });
+}
+
+int TSHip_MoEExpertsSwiGLUResidualF32Device(TSHipTensorView2D residual, TSHipTensorView2D input, int num_experts,
+                                            void* const* gate_data_ptrs, void* const* up_data_ptrs, void* const* down_data_ptrs,
+                                            int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1, int64_t gate_raw_bytes_each,
+                                            int up_ggml_type, int64_t up_ne0, int64_t up_ne1, int64_t up_raw_bytes_each,
+                                            int down_ggml_type, int64_t down_ne0, int64_t down_ne1, int64_t down_raw_bytes_each,
+                                            const float* route_weights, int use_shared, void* shared_gate_data, void* shared_up_data,
+                                            void* shared_down_data, int shared_gate_ggml_type, int64_t shared_gate_ne0,
+                                            int64_t shared_gate_ne1, int64_t shared_gate_raw_bytes, int shared_up_ggml_type,
+                                            int64_t shared_up_ne0, int64_t shared_up_ne1, int64_t shared_up_raw_bytes,
+                                            int shared_down_ggml_type, int64_t shared_down_ne0, int64_t shared_down_ne1,
+                                            int64_t shared_down_raw_bytes, float shared_scalar)
+{
+    return guarded(0, "MoE SwiGLU residual", [&]() -> int {
+        ExpertSetArgs a = swiglu_args("MoE SwiGLU residual", 32, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
+                                      gate_ne0, gate_ne1, gate_raw_bytes_each, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
+                                      down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights);
+        set_shared(a, use_shared, shared_gate_data, shared_up_data, shared_down_data, shared_gate_ggml_type, shared_gate_ne0, shared_gate_ne1,
+                   shared_gate_raw_bytes, shared_up_ggml_type, shared_up_ne0, shared_up_ne1, shared_up_raw_bytes, shared_down_ggml_type,
+                   shared_down_ne0, shared_down_ne1, shared_down_raw_bytes, shared_scalar);
+        return expert_set_device(residual, true, input, a, "residual");
     });
 }
 

@@ -1,6 +1,6 @@
 // Bit-exact dequantization of raw GGUF blocks to fp32 on gfx950.
 //
-// The arithmetic is the managed dequantizers' (TensorSharp.Models/ManagedQuantizedOps.cs:411-427 Q8_0,
+// The arithmetic is the managed dequantizers' (TensorSharp.Models/ManagedQuantizedOps.cs:411-427 Q8_0, :429-445 Q8_1,
 // :447-479 Q4_K, :579-598 MXFP4; :268-409 and :481-577 for F16, BF16, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, Q6_K, IQ4_NL):
 // every product is exact in fp32, the subtract of Q4_K / Q5_K and the add of Q4_1 / Q5_1 are the one rounding.
 // Contraction is switched off so the multiply and the subtract stay separately rounded operations.
@@ -47,6 +47,20 @@ __device__ __forceinline__ float mxfp4_value(uint32_t nib)
     const uint64_t neg = 0xf4f8fafcfdfeff00ull;
     const uint64_t tab = (nib & 8u) ? neg : pos;
     return (float)(int)(int8_t)((tab >> ((nib & 7u) * 8)) & 0xffu);
+}
+
+// Q8_1 (ggml-common.h block_q8_1: fp16 d, fp16 s = d * sum(q), int8 qs[32] = 36 bytes): y = q * d, s is not read
+__device__ __forceinline__ float4 dequant4_q8_1(const uint8_t* src, int64_t e0)
+{
+    const uint8_t* blk = src + (e0 >> 5) * 36;
+    const int j = (int)(e0 & 31);
+    const float d = half_bits_to_float((uint32_t)blk[0] | ((uint32_t)blk[1] << 8));
+    float4 o;
+    o.x = (float)(int8_t)blk[4 + j] * d;
+    o.y = (float)(int8_t)blk[5 + j] * d;
+    o.z = (float)(int8_t)blk[6 + j] * d;
+    o.w = (float)(int8_t)blk[7 + j] * d;
+    return o;
 }
 
 // 4 consecutive outputs starting at element e0 (a multiple of 4) of the block sequence at src
@@ -214,6 +228,7 @@ template <int TYPE>
 __device__ __forceinline__ float4 dequant4(const uint8_t* src, int64_t e0)
 {
     if (TYPE == kTypeQ8_0) return dequant4_q8_0(src, e0);
+    if (TYPE == kTypeQ8_1) return dequant4_q8_1(src, e0);
     if (TYPE == kTypeQ4_K) return dequant4_q4_K(src, e0);
     if (TYPE == kTypeMXFP4) return dequant4_mxfp4(src, e0);
     if (TYPE == kTypeF16) return dequant4_f16(src, e0);
@@ -273,7 +288,7 @@ bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_
 #define TSHIP_DEQUANT_CASE(T) case T: hipLaunchKernelGGL(dequant_kernel<T>, grid, block, 0, stream, s, dst, n4); break;
     TSHIP_DEQUANT_CASE(kTypeF16) TSHIP_DEQUANT_CASE(kTypeBF16) TSHIP_DEQUANT_CASE(kTypeQ4_0) TSHIP_DEQUANT_CASE(kTypeQ4_1)
     TSHIP_DEQUANT_CASE(kTypeQ5_0) TSHIP_DEQUANT_CASE(kTypeQ5_1) TSHIP_DEQUANT_CASE(kTypeQ5_K) TSHIP_DEQUANT_CASE(kTypeQ6_K)
-    TSHIP_DEQUANT_CASE(kTypeIQ4_NL)
+    TSHIP_DEQUANT_CASE(kTypeIQ4_NL) TSHIP_DEQUANT_CASE(kTypeQ8_1)
 #undef TSHIP_DEQUANT_CASE
     default: set_last_error("dequantize: unsupported type."); return false;
     }
@@ -301,7 +316,7 @@ bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, 
 #define TSHIP_ROWS_CASE(T) case T: hipLaunchKernelGGL(get_rows_kernel<T>, grid, block, 0, stream, s, row_bytes, ne1, ids, dst, ldd, k4); break;
     TSHIP_ROWS_CASE(kTypeF16) TSHIP_ROWS_CASE(kTypeBF16) TSHIP_ROWS_CASE(kTypeQ4_0) TSHIP_ROWS_CASE(kTypeQ4_1)
     TSHIP_ROWS_CASE(kTypeQ5_0) TSHIP_ROWS_CASE(kTypeQ5_1) TSHIP_ROWS_CASE(kTypeQ5_K) TSHIP_ROWS_CASE(kTypeQ6_K)
-    TSHIP_ROWS_CASE(kTypeIQ4_NL)
+    TSHIP_ROWS_CASE(kTypeIQ4_NL) TSHIP_ROWS_CASE(kTypeQ8_1)
 #undef TSHIP_ROWS_CASE
     default: set_last_error("get_rows: unsupported type."); return false;
     }

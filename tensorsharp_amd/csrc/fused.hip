@@ -2,6 +2,8 @@
 // (TensorSharp.GGML.Native/ggml_ops_fused.cpp:21-640): RMSNorm rows and the SiLU-gated product.
 #include "tship_internal.h"
 
+#include <hip/hip_fp16.h>
+
 namespace tship {
 namespace {
 
@@ -63,6 +65,68 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(const float* __restrict__
     out[(int64_t)blockIdx.y * half + j] = (g / (1.0f + expf(-g))) * u;
 }
 
+// squared ReLU in place (Nemotron experts: ggml_relu then ggml_sqr, ggml_ops_fused.cpp:1700-1710)
+__global__ void __launch_bounds__(256) relu_sqr_kernel(float* __restrict__ x, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = fmaxf(x[i], 0.f);
+    x[i] = v * v;
+}
+
+// out[m][j] = (base ? base[m][j] : 0) + sum_e w.v[e] * rows[e * set_stride + m * N + j], experts added in index order as the
+// bridge's graph chains its ggml_add nodes (ggml_ops_fused.cpp:1716-1722)
+__global__ void __launch_bounds__(256) weighted_sum_kernel(const float* __restrict__ rows, int64_t set_stride, WeightedSumCoeffs w, int count,
+                                                          int N, const float* base, int64_t ldb, float* out, int64_t ldo)
+{
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    const int m = blockIdx.y;
+    if (j >= N) return;
+    float acc = 0.f;
+    for (int e = 0; e < count; ++e) {
+        const float v = rows[(int64_t)e * set_stride + (int64_t)m * N + j] * w.v[e];
+        acc = e == 0 ? v : acc + v;
+    }
+    out[(int64_t)m * ldo + j] = base ? base[(int64_t)m * ldb + j] + acc : acc;
+}
+
+// ---- dense (F32 / F16 / BF16) weights -----------------------------------------------------------
+// The block formats are the hot path; dense weights appear as small matrices beside them (an F32 router, an F16 head).
+// One wavefront per weight row and up to kDenseRows activation rows per workgroup: the weight row is read once per
+// kDenseRows activation rows, fp32 accumulation in k order per lane, then a butterfly over the 64 lanes.
+constexpr int kDenseRows = 4;
+
+__device__ inline float dense_elem(const float* w, int64_t i) { return w[i]; }
+__device__ inline float dense_elem(const __half* w, int64_t i) { return __half2float(w[i]); }
+__device__ inline float dense_elem(const uint16_t* w, int64_t i) { return __uint_as_float((uint32_t)w[i] << 16); }   // bf16
+
+template <typename T>
+__global__ void __launch_bounds__(256) dense_matmul_kernel(const T* __restrict__ w, const float* __restrict__ x, int64_t ldx,
+                                                          float* __restrict__ y, int64_t ldy, int M, int N, int K, int accumulate)
+{
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int m0 = blockIdx.y * kDenseRows;
+    if (n >= N) return;
+    const T* wr = w + (int64_t)n * K;
+    float acc[kDenseRows] = {};
+    for (int k = lane; k < K; k += 64) {
+        const float wv = dense_elem(wr, k);
+#pragma unroll
+        for (int r = 0; r < kDenseRows; ++r)
+            if (m0 + r < M) acc[r] = fmaf(wv, x[(int64_t)(m0 + r) * ldx + k], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < kDenseRows; ++r) {
+        float v = acc[r];
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        if (lane == 0 && m0 + r < M) {
+            float* dst = y + (int64_t)(m0 + r) * ldy + n;
+            *dst = accumulate ? *dst + v : v;
+        }
+    }
+}
+
 }  // namespace
 
 bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps, int M, int K, float* out, hipStream_t stream)
@@ -86,6 +150,52 @@ bool launch_silu_mul(const float* gu, int64_t ldgu, int M, int half, float* out,
     }
     hipLaunchKernelGGL(silu_mul_kernel, dim3((half + 255) / 256, M), dim3(256), 0, stream, gu, ldgu, half, out);
     return hip_ok(hipGetLastError(), "silu_mul launch");
+}
+
+bool launch_relu_sqr(float* x, int64_t n, hipStream_t stream)
+{
+    if (n <= 0) return true;
+    hipLaunchKernelGGL(relu_sqr_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, n);
+    return hip_ok(hipGetLastError(), "relu_sqr launch");
+}
+
+bool launch_weighted_sum(const float* rows, int64_t set_stride, const WeightedSumCoeffs& w, int count, int M, int N, const float* base,
+                         int64_t ldb, float* out, int64_t ldo, hipStream_t stream)
+{
+    if (M <= 0 || N <= 0) return true;
+    if (count < 1 || count > kMaxWeightedRows || M > 65535) {
+        set_last_error("weighted_sum: bad row-set count or more than 65535 rows.");
+        return false;
+    }
+    hipLaunchKernelGGL(weighted_sum_kernel, dim3((N + 255) / 256, M), dim3(256), 0, stream, rows, set_stride, w, count, N, base, ldb, out, ldo);
+    return hip_ok(hipGetLastError(), "weighted_sum launch");
+}
+
+bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, float* y, int64_t ldy, int M, int N, int K,
+                         bool accumulate, hipStream_t stream)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return true;
+    const dim3 grid((N + 3) / 4, (M + kDenseRows - 1) / kDenseRows);
+    if (grid.y > 65535) {
+        set_last_error("dense matmul: too many activation rows per call.");
+        return false;
+    }
+    const int acc = accumulate ? 1 : 0;
+    switch (type) {
+    case kTypeF32:
+        hipLaunchKernelGGL(dense_matmul_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(w), x, ldx, y, ldy, M, N, K, acc);
+        break;
+    case kTypeF16:
+        hipLaunchKernelGGL(dense_matmul_kernel<__half>, grid, dim3(256), 0, stream, static_cast<const __half*>(w), x, ldx, y, ldy, M, N, K, acc);
+        break;
+    case kTypeBF16:
+        hipLaunchKernelGGL(dense_matmul_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(w), x, ldx, y, ldy, M, N, K, acc);
+        break;
+    default:
+        set_last_error("dense matmul: the weight type is not F32, F16 or BF16.");
+        return false;
+    }
+    return hip_ok(hipGetLastError(), "dense matmul launch");
 }
 
 }  // namespace tship

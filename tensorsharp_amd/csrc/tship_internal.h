@@ -17,6 +17,7 @@ constexpr int kTypeQ4_1 = 3;
 constexpr int kTypeQ5_0 = 6;
 constexpr int kTypeQ5_1 = 7;
 constexpr int kTypeQ8_0 = 8;
+constexpr int kTypeQ8_1 = 9;
 constexpr int kTypeQ4_K = 12;
 constexpr int kTypeQ5_K = 13;
 constexpr int kTypeQ6_K = 14;
@@ -34,7 +35,7 @@ inline int64_t block_elems(int type)
     case kTypeQ4_K: return 256;
     case kTypeMXFP4: return 32;
     case kTypeF16: case kTypeBF16: return 1;
-    case kTypeQ4_0: case kTypeQ4_1: case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL: return 32;
+    case kTypeQ4_0: case kTypeQ4_1: case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL: case kTypeQ8_1: return 32;
     case kTypeQ5_K: case kTypeQ6_K: return 256;
     default: return 0;
     }
@@ -52,14 +53,16 @@ inline int64_t block_bytes(int type)
     case kTypeQ4_1: return 20;
     case kTypeQ5_0: return 22;
     case kTypeQ5_1: return 24;
+    case kTypeQ8_1: return 36;
     case kTypeQ5_K: return 176;
     case kTypeQ6_K: return 210;
     default: return 0;
     }
 }
 
-// formats the matmul kernels read: every block format of ManagedQuantizedOps.cs:40-59 except Q8_1; the ones without
-// a GEMV specialisation take the matrix-core kernels for single rows too
+// formats the GEMV / GEMM kernels read: every block format of ManagedQuantizedOps.cs:40-59 except Q8_1 (an activation
+// format that no GGUF file stores weights in; see is_matmul_type); the ones without a GEMV specialisation take the
+// matrix-core kernels for single rows too
 inline bool is_quant_type(int type)
 {
     switch (type) {
@@ -75,7 +78,7 @@ inline bool has_gemv(int type)
            type == kTypeQ4_0 || type == kTypeQ4_1;
 }
 // formats with a dequantizer (DequantizeToF32, embedding gather): every block format the managed code reads
-// (ManagedQuantizedOps.cs:40-59) except Q8_1
+// (ManagedQuantizedOps.cs:40-59)
 inline bool is_dequant_type(int type) { return type != kTypeF32 && block_elems(type) != 0; }
 
 void set_last_error(const std::string& msg);
@@ -170,6 +173,24 @@ constexpr int64_t kMaxOperandBytes = ((int64_t)1 << 31) - 64;
 bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps, int M, int K, float* out, hipStream_t stream);
 // out[m, j] = silu(gu[m, j]) * gu[m, half + j], j < half
 bool launch_silu_mul(const float* gu, int64_t ldgu, int M, int half, float* out, hipStream_t stream);
+
+// x[i] = max(x[i], 0)^2 in place
+bool launch_relu_sqr(float* x, int64_t n, hipStream_t stream);
+// out[m][j] = (base ? base[m][j] : 0) + sum_{e < count} w.v[e] * rows[e * set_stride + m * N + j], added in index order;
+// base may be out
+constexpr int kMaxWeightedRows = 36;
+struct WeightedSumCoeffs {
+    float v[kMaxWeightedRows];
+};
+bool launch_weighted_sum(const float* rows, int64_t set_stride, const WeightedSumCoeffs& w, int count, int M, int N, const float* base,
+                         int64_t ldb, float* out, int64_t ldo, hipStream_t stream);
+// y[m][n] (+)= sum_k W[n][k] x[m][k] for a dense row-major weight of type F32, F16 or BF16
+bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, float* y, int64_t ldy, int M, int N, int K,
+                         bool accumulate, hipStream_t stream);
+inline bool is_dense_type(int type) { return type == kTypeF32 || type == kTypeF16 || type == kTypeBF16; }
+// every weight type the matmul entry points take; Q8_1 weights are dequantized to fp32 in slices of rows and then take
+// the dense kernel
+inline bool is_matmul_type(int type) { return is_quant_type(type) || is_dense_type(type) || type == kTypeQ8_1; }
 
 // ---- single-token attention of the whole-layer decode ---------------------------------------
 // qkv = [q heads | k heads | v heads], head_dim each.  Per head: RMSNorm (weights may be null) + RoPE at `position`; the

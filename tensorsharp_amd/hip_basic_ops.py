@@ -149,6 +149,82 @@ class HipBasicOps:
                 C.c_void_p(down.ptr), down.ggml_type, down.ne0, down.ne1, down.raw_bytes, int(half_dim))
         N.check_result(ok, "fused_ffn_swiglu_quant")
 
+    @staticmethod
+    def _weight_args(w):
+        return (C.c_void_p(w.ptr), w.ggml_type, w.ne0, w.ne1, w.raw_bytes)
+
+    @staticmethod
+    def FusedOutProjFFN(residual, input, out_proj, ffn_norm_weight, eps, gate_up, down, half_dim):
+        """residual += input * W_out^T, then residual += W_down * (silu(g) * u) with [g | u] = W_gate_up * (RMSNorm(residual) *
+        ffn_norm_weight) (GgmlBasicOps.cs:449-480).  All host (numpy) or all device (torch) tensors."""
+        rv, iv, sfx = HipBasicOps._views(residual, input)
+        fn = getattr(N.lib(), "TSHip_FusedOutProjFFNQuantF32" + sfx)
+        ok = fn(rv, iv, *HipBasicOps._weight_args(out_proj), C.c_void_p(HipBasicOps._addr(ffn_norm_weight)),
+                int(ffn_norm_weight.shape[0]), float(eps), *HipBasicOps._weight_args(gate_up), *HipBasicOps._weight_args(down),
+                int(half_dim))
+        N.check_result(ok, "fused_outproj_ffn")
+
+    @staticmethod
+    def FusedOutProjNormRouter(residual, input, out_proj, norm_weight, eps, normed_output, router, router_output):
+        """residual += input * W_out^T; normed_output = RMSNorm(residual) * norm_weight; router_output = normed_output *
+        W_router^T (GgmlBasicOps.cs:416-447).  The router weight may be F32 / F16 / BF16 or a block format."""
+        rv, iv, sfx = HipBasicOps._views(residual, input)
+        view = (lambda a: _host_view(a, standard=True)) if sfx == "" else _device_view
+        fn = getattr(N.lib(), "TSHip_FusedOutProjNormRouterQuantF32" + sfx)
+        ok = fn(rv, iv, *HipBasicOps._weight_args(out_proj), C.c_void_p(HipBasicOps._addr(norm_weight)),
+                int(norm_weight.shape[0]), float(eps), view(normed_output), *HipBasicOps._weight_args(router),
+                view(router_output))
+        N.check_result(ok, "fused_outproj_norm_router")
+
+    @staticmethod
+    def _expert_ptrs(weights):
+        return (C.c_void_p * len(weights))(*[w.ptr for w in weights])
+
+    @staticmethod
+    def _shape_args(w):
+        return (w.ggml_type, w.ne0, w.ne1, w.raw_bytes)
+
+    @staticmethod
+    def MoEExpertsForward(result, input, up, down, route_weights):
+        """result = sum_e route_weights[e] * W_down[e] * relu(W_up[e] * input)^2 for up to 16 selected experts
+        (GgmlBasicOps.cs:586-613; Nemotron).  up / down: lists of QuantizedWeight sharing type and shape."""
+        rv, iv, sfx = HipBasicOps._views(result, input)
+        n = len(up)
+        rw = (C.c_float * n)(*[float(v) for v in route_weights])
+        fn = getattr(N.lib(), "TSHip_MoEExpertsForwardF32" + sfx)
+        ok = fn(rv, iv, n, HipBasicOps._expert_ptrs(up), HipBasicOps._expert_ptrs(down), *HipBasicOps._shape_args(up[0]),
+                *HipBasicOps._shape_args(down[0]), rw)
+        N.check_result(ok, "moe_experts_forward")
+
+    @staticmethod
+    def MoEExpertsSwiGLUForward(result, input, gate, up, down, route_weights):
+        """result = sum_e route_weights[e] * W_down[e] * (silu(W_gate[e] x) * (W_up[e] x)) (GgmlBasicOps.cs:615-645)."""
+        rv, iv, sfx = HipBasicOps._views(result, input)
+        n = len(up)
+        rw = (C.c_float * n)(*[float(v) for v in route_weights])
+        fn = getattr(N.lib(), "TSHip_MoEExpertsSwiGLUForwardF32" + sfx)
+        ok = fn(rv, iv, n, HipBasicOps._expert_ptrs(gate), HipBasicOps._expert_ptrs(up), HipBasicOps._expert_ptrs(down),
+                *HipBasicOps._shape_args(gate[0]), *HipBasicOps._shape_args(up[0]), *HipBasicOps._shape_args(down[0]), rw)
+        N.check_result(ok, "moe_experts_swiglu_forward")
+
+    @staticmethod
+    def MoEExpertsSwiGLUResidual(residual, input, gate, up, down, route_weights, shared=None, shared_scalar=1.0):
+        """residual += sum_e route_weights[e] * expert_e(input) [+ shared_scalar * shared_expert(input)]
+        (GgmlBasicOps.cs:647-700); shared = (gate, up, down) QuantizedWeights or None; up to 32 routed experts."""
+        rv, iv, sfx = HipBasicOps._views(residual, input)
+        n = len(up)
+        rw = (C.c_float * n)(*[float(v) for v in route_weights])
+        if shared is None:
+            sh = (0, None, None, None, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+        else:
+            sh = (1, C.c_void_p(shared[0].ptr), C.c_void_p(shared[1].ptr), C.c_void_p(shared[2].ptr),
+                  *HipBasicOps._shape_args(shared[0]), *HipBasicOps._shape_args(shared[1]), *HipBasicOps._shape_args(shared[2]))
+        fn = getattr(N.lib(), "TSHip_MoEExpertsSwiGLUResidualF32" + sfx)
+        ok = fn(rv, iv, n, HipBasicOps._expert_ptrs(gate), HipBasicOps._expert_ptrs(up), HipBasicOps._expert_ptrs(down),
+                *HipBasicOps._shape_args(gate[0]), *HipBasicOps._shape_args(up[0]), *HipBasicOps._shape_args(down[0]), rw,
+                *sh, float(shared_scalar))
+        N.check_result(ok, "moe_experts_swiglu_residual")
+
     # -- embedding gather ------------------------------------------------------------------
     @staticmethod
     def GetRowsQuant(result, weight_data, ggml_type, ne0, ne1, raw_bytes, indices):
@@ -272,13 +348,13 @@ class HipBasicOps:
         return wts, ids
 
     @staticmethod
-    def MoEExpertsForward(hidden, ids, weights, gate_up_w, gate_up_b, down_w, down_b, ggml_type, n_experts, H, F,
+    def MoEExpertsGptOssForward(hidden, ids, weights, gate_up_w, gate_up_b, down_w, down_b, ggml_type, n_experts, H, F,
                           alpha=1.702, limit=7.0):
         """Expert stage of GptOssModel.MoEForward for routed tokens; all tensors on the device."""
         import torch
         out = torch.empty((hidden.shape[0], H), dtype=torch.float32, device=hidden.device)
         HipBasicOps.UseCurrentStream()
-        ok = N.lib().TSHip_MoEExpertsForwardF32Device(
+        ok = N.lib().TSHip_MoEExpertsGptOssForwardF32Device(
             _device_view(out), _device_view(hidden), ids.data_ptr(), weights.data_ptr(), int(ids.shape[1]),
             gate_up_w.data_ptr(), None if gate_up_b is None else gate_up_b.data_ptr(), down_w.data_ptr(),
             None if down_b is None else down_b.data_ptr(), int(ggml_type), int(n_experts), int(H), int(F), float(alpha),

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(HERE, "libTsHipOps.so")
 
 BACKEND_HIP = 4
 TYPE_F32, TYPE_Q8_0, TYPE_Q4_K, TYPE_MXFP4 = 0, 8, 12, 39
+TYPE_Q8_1 = 9
 TYPE_F16, TYPE_Q4_0, TYPE_Q4_1, TYPE_Q5_0, TYPE_Q5_1, TYPE_Q5_K, TYPE_Q6_K, TYPE_IQ4_NL, TYPE_BF16 = 1, 2, 3, 6, 7, 13, 14, 20, 30
 DTYPE_F32, DTYPE_I32 = 0, 3
 
@@ -74,12 +75,33 @@ SIGNATURES = {
     "TSHip_FusedFFNSwiGLUQuantF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_float,
                                                      C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
                                                      C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
+    "TSHip_FusedOutProjFFNQuantF32": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                C.c_void_p, C.c_int, C.c_float,
+                                                C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
+    "TSHip_FusedOutProjNormRouterQuantF32": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64,
+                                                       C.c_int64, C.c_void_p, C.c_int, C.c_float, TensorView2D,
+                                                       C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, TensorView2D]),
+    "TSHip_MoEExpertsForwardF32": (C.c_int, [TensorView2D, TensorView2D, C.c_int, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                             C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                             C.POINTER(C.c_float)]),
+    "TSHip_MoEExpertsSwiGLUForwardF32": (C.c_int, [TensorView2D, TensorView2D, C.c_int, C.POINTER(C.c_void_p),
+                                                   C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                                   C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                   C.c_int, C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_float)]),
+    "TSHip_MoEExpertsSwiGLUResidualF32": (C.c_int, [TensorView2D, TensorView2D, C.c_int, C.POINTER(C.c_void_p),
+                                                    C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                                    C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                    C.c_int, C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_float),
+                                                    C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                    C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                    C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_float]),
     "TSHip_GetRowsQuantF32": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
                                         ContiguousTensor]),
     "TSHip_GetRowsQuantF32Device": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
                                               C.c_void_p, C.c_int64]),
     "TSHip_MoERouteF32Device": (C.c_int, [TensorView2D, C.c_int, C.c_void_p, C.c_void_p]),
-    "TSHip_MoEExpertsForwardF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+    "TSHip_MoEExpertsGptOssForwardF32Device": (C.c_int, [TensorView2D, TensorView2D, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int64,
                                                    C.c_int64, C.c_float, C.c_float]),
     "TSHip_TransformerLayerDecodeDevice": (C.c_int, [
@@ -100,6 +122,9 @@ SIGNATURES = {
         C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
 }
 # the host-pointer forms take the same argument lists
+for _name in ("TSHip_FusedOutProjFFNQuantF32", "TSHip_FusedOutProjNormRouterQuantF32", "TSHip_MoEExpertsForwardF32",
+              "TSHip_MoEExpertsSwiGLUForwardF32", "TSHip_MoEExpertsSwiGLUResidualF32"):
+    SIGNATURES[_name + "Device"] = SIGNATURES[_name]
 SIGNATURES["TSHip_TransformerLayerDecode"] = SIGNATURES["TSHip_TransformerLayerDecodeDevice"]
 SIGNATURES["TSHip_TransformerModelDecode"] = SIGNATURES["TSHip_TransformerModelDecodeDevice"]
 

@@ -160,7 +160,7 @@ def test_expert_id_outside_the_table_contributes_nothing(hip, oracle, T):
         w0[r, s] = 0.0
     ref = oracle.moe_forward(t, gu, gb, dn, db, E, H, F, hidden, good, w0)
     c = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    out = hip.MoEExpertsForward(c(hidden), c(bad.astype(np.int32)), c(wts), c(gu), c(gb), c(dn), c(db), t, E, H, F)
+    out = hip.MoEExpertsGptOssForward(c(hidden), c(bad.astype(np.int32)), c(wts), c(gu), c(gb), c(dn), c(db), t, E, H, F)
     torch.cuda.synchronize()
     got = out.cpu().numpy()
     assert np.all(np.isfinite(got))

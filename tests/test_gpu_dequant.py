@@ -121,3 +121,36 @@ def test_more_formats_random_bytes_and_row_gather(hip, oracle, name):
     for i, r in enumerate(idx):
         assert bits_equal(res[i], w[r]), (name, i)
     hip.ClearHostBufferCache()
+
+
+def test_q8_1_dequant_gather_and_matmul(hip, oracle):
+    # Q8_1 has no reference-written known answers (ggml has no dequantizer for it); the oracle's restatement is pinned by
+    # its closed form over every scale code.  Here: bit-exact dequantization and row gather, and the matmul (dequantized
+    # slices through the dense kernel) against the fp64 product at the matmul bar 1e-3 * ||row||.
+    import torch
+    from oracle.oracle import Q8_1
+    rng = np.random.default_rng(61)
+    K, rows = 512, 300
+    raw = rng.integers(0, 256, size=rows * (K // 32) * 36, dtype=np.uint8)
+    want = oracle.dequantize(Q8_1, raw)
+    assert bits_equal(hip.DequantizeToFloat32(Q8_1, raw, want.size), want)
+    out = hip.DequantizeToFloat32Device(Q8_1, torch.from_numpy(raw).cuda(), want.size)
+    torch.cuda.synchronize()
+    assert bits_equal(out.cpu().numpy(), want)
+    idx = np.array([299, 0, 17, 150, 17], dtype=np.int32)
+    res = np.full((idx.size, K), 7.0, dtype=np.float32)
+    hip.GetRowsQuant(res, raw.ctypes.data, Q8_1, K, rows, raw.size, idx)
+    for i, r in enumerate(idx):
+        assert bits_equal(res[i], want.reshape(rows, K)[r]), i
+    hip.ClearHostBufferCache()
+    # finite scales for the product
+    blocks = raw.reshape(-1, 36).copy()
+    blocks[:, 0:2] = rng.uniform(1e-3, 4e-3, blocks.shape[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    w = blocks.reshape(-1)
+    for M in (1, 7):
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        ref = oracle.matmul_f64(Q8_1, w, rows, K, x)
+        got = np.full((M, rows), np.nan, np.float32)
+        hip.AddmmQuant(got, x, w.ctypes.data, Q8_1, K, rows, w.size)
+        hip.ClearHostBufferCache()
+        assert np.all(np.abs(got - ref) <= 1e-3 * np.linalg.norm(ref, axis=1, keepdims=True))

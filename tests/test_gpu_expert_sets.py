@@ -1,0 +1,221 @@
+"""GPU parity: the bridge's larger fused calls through the C ABI, host-pointer and device forms.
+
+  FusedOutProjFFN / FusedOutProjNormRouter   (ggml_ops_fused.cpp:1057-1380)
+  MoEExpertsForward (squared-ReLU experts), MoEExpertsSwiGLUForward, MoEExpertsSwiGLUResidual
+                                             (ggml_ops_fused.cpp:1576-2160)
+and dense (F32 / F16 / BF16) weights in the matmul entry points.
+
+Reference value: the oracle's compositions (fp64 products of the bit-exact dequantized weights, fp32 RMSNorm / SiLU
+in ggml order).  Bar per matmul: max_j |y - ref| <= 1e-3 * ||row of the product||_2; chained matmuls (an FFN behind a
+projection, a down projection behind gate/up) pass the first one's error through, so those rows get 2e-3 of the
+last product's norm plus 1e-3 of the first's, written at each assert."""
+import numpy as np
+import pytest
+
+from oracle.oracle import F32, F16, BF16, Q8_0, Q4_K, Q6_K, MXFP4
+
+pytestmark = pytest.mark.gpu
+T_ = {"q8_0": Q8_0, "q4_k": Q4_K, "mxfp4": MXFP4, "f32": F32, "f16": F16, "bf16": BF16}
+EPS = 1e-6
+
+
+def make(oracle, name, N, K, rng, sigma=0.05):
+    """(type, raw bytes, N, K)"""
+    v = (rng.standard_normal(N * K) * sigma).astype(np.float32)
+    t = T_[name]
+    if t == F32:
+        raw = v.view(np.uint8).copy()
+    elif t == F16:
+        raw = v.astype(np.float16).view(np.uint8).copy()
+    elif t == BF16:
+        raw = (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).copy()
+    else:
+        raw = oracle.quantize(t, v)
+    return (t, raw, N, K)
+
+
+def qw(desc, device):
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    t, raw, N, K = desc
+    return QuantizedWeight(torch.from_numpy(raw).cuda() if device else raw, t, K, N)
+
+
+def rownorm(m):
+    return np.linalg.norm(np.asarray(m, dtype=np.float64), axis=1, keepdims=True)
+
+
+def run(hip, device, fn, inout, *tensors_then_rest):
+    """calls fn(inout, ...) with numpy arrays moved to the GPU for the device form; returns inout as numpy"""
+    import torch
+    if not device:
+        fn(inout, *tensors_then_rest)
+        hip.ClearHostBufferCache()
+        return inout
+    moved = [torch.from_numpy(a).cuda() if isinstance(a, np.ndarray) else a for a in (inout,) + tensors_then_rest]
+    fn(*moved)
+    torch.cuda.synchronize()
+    return [m.cpu().numpy() if isinstance(m, torch.Tensor) else m for m in moved]
+
+
+@pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("M", [1, 5, 70])
+@pytest.mark.parametrize("device", [False, True])
+def test_dense_weights_in_addmm_quant(hip, oracle, name, M, device):
+    import torch
+    rng = np.random.default_rng(300 + M)
+    N, K = 131, 520          # K % 64 != 0, N % 4 != 0: tails of the lane loop and the row groups
+    w = make(oracle, name, N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    ref = oracle.matmul_any_f64(*w, x)
+    q = qw(w, device)
+    if device:
+        res = torch.full((M, N), float("nan"), device="cuda")
+        hip.AddmmQuantDevice(res, torch.from_numpy(x).cuda(), q.ptr, q.ggml_type, K, N, q.raw_bytes)
+        torch.cuda.synchronize()
+        got = res.cpu().numpy()
+    else:
+        got = np.full((M, N), np.nan, np.float32)
+        hip.AddmmQuant(got, x, q.ptr, q.ggml_type, K, N, q.raw_bytes)
+        hip.ClearHostBufferCache()
+    # fp32 accumulation of exact products: far inside the matmul bar of 1e-3 * ||row||
+    assert np.all(np.abs(got - ref) <= 1e-5 * rownorm(ref)), float(np.max(np.abs(got - ref) / rownorm(ref)))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
+@pytest.mark.parametrize("M", [1, 3, 40])
+@pytest.mark.parametrize("device", [False, True])
+def test_outproj_ffn(hip, oracle, name, M, device):
+    rng = np.random.default_rng(310 + M)
+    A, H, F = 768, 512, 768        # attention width, hidden, FFN half width
+    out_w = make(oracle, name, H, A, rng)
+    gu = make(oracle, name, 2 * F, H, rng)
+    dn = make(oracle, name, H, F, rng)
+    x = rng.standard_normal((M, A)).astype(np.float32)
+    resid = rng.standard_normal((M, H)).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    ref, mm1, mm2 = oracle.outproj_ffn(resid, x, out_w, nw, EPS, gu, dn, F)
+    fn = lambda r, i, n: hip.FusedOutProjFFN(r, i, qw(out_w, device), n, EPS, qw(gu, device), qw(dn, device), F)
+    got = run(hip, device, fn, resid.copy(), x, nw)
+    got = got[0] if device else got
+    tol = 1e-3 * rownorm(mm1) + 2e-3 * rownorm(mm2)
+    assert np.all(np.abs(got - ref) <= tol), (name, M, device, float(np.max(np.abs(got - ref) / tol)))
+
+
+@pytest.mark.parametrize("name,router", [("q8_0", "f32"), ("q4_k", "f16"), ("mxfp4", "bf16"), ("q4_k", "q8_0")])
+@pytest.mark.parametrize("M", [1, 6])
+@pytest.mark.parametrize("device", [False, True])
+def test_outproj_norm_router(hip, oracle, name, router, M, device):
+    rng = np.random.default_rng(320 + M)
+    A, H, E = 512, 768, 128
+    out_w = make(oracle, name, H, A, rng)
+    rw = make(oracle, router, E, H, rng, 0.2)
+    x = rng.standard_normal((M, A)).astype(np.float32)
+    resid = rng.standard_normal((M, H)).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    res_ref, normed_ref, logits_ref, mm1 = oracle.outproj_norm_router(resid, x, out_w, nw, EPS, rw)
+    normed = np.full((M, H), np.nan, np.float32)
+    logits = np.full((M, E), np.nan, np.float32)
+    fn = lambda r, i, n, no, lo: hip.FusedOutProjNormRouter(r, i, qw(out_w, device), n, EPS, no, qw(rw, device), lo)
+    out = run(hip, device, fn, resid.copy(), x, nw, normed, logits)
+    got_res, got_normed, got_logits = (out[0], out[3], out[4]) if device else (out, normed, logits)
+    tol = 1e-3 * rownorm(mm1)
+    assert np.all(np.abs(got_res - res_ref) <= tol), (name, M, float(np.max(np.abs(got_res - res_ref) / tol)))
+    # the norm divides by the RMS of the row (about 1 here) and scales by norm weights <= 1.5
+    rms = np.sqrt((res_ref ** 2).mean(axis=1, keepdims=True))
+    assert np.all(np.abs(got_normed - normed_ref) <= 2.0 * tol / rms), float(np.max(np.abs(got_normed - normed_ref)))
+    tol_l = 1e-3 * rownorm(logits_ref) + np.abs(oracle.weight_rows(*rw[:2], E, H)).sum(axis=1)[None, :] * np.max(2.0 * tol / rms)
+    assert np.all(np.abs(got_logits - logits_ref) <= tol_l), float(np.max(np.abs(got_logits - logits_ref) / tol_l))
+
+
+def experts(oracle, name, n, H, I, N, rng, gated, down_name=None):
+    return [dict(gate=make(oracle, name, I, H, rng) if gated else None, up=make(oracle, name, I, H, rng),
+                 down=make(oracle, down_name or name, N, I, rng)) for _ in range(n)]
+
+
+def set_tol(oracle, parts, weights):
+    # per expert: 2e-3 of its down product (gate/up errors pass through the activation), scaled by |route weight|
+    return sum(2e-3 * abs(float(w)) * rownorm(p) for p, w in zip(parts, weights))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k"])
+@pytest.mark.parametrize("n,M", [(1, 1), (6, 1), (16, 1), (5, 4)])
+@pytest.mark.parametrize("device", [False, True])
+def test_experts_relu_squared(hip, oracle, name, n, M, device):
+    rng = np.random.default_rng(330 + n + M)
+    H, I = 512, 768 if name == "q4_k" else 352
+    ex = experts(oracle, name, n, H, I, H, rng, gated=False)
+    w = rng.uniform(0.05, 0.6, n).astype(np.float32)
+    x = rng.standard_normal((M, H)).astype(np.float32)
+    ref, parts = oracle.expert_set(x, ex, w)
+    fn = lambda r, i: hip.MoEExpertsForward(r, i, [qw(e["up"], device) for e in ex], [qw(e["down"], device) for e in ex], w)
+    got = run(hip, device, fn, np.full((M, H), np.nan, np.float32), x)
+    got = got[0] if device else got
+    tol = set_tol(oracle, parts, w)
+    assert np.all(np.abs(got - ref) <= tol), (name, n, M, device, float(np.max(np.abs(got - ref) / tol)))
+
+
+@pytest.mark.parametrize("name,down", [("q8_0", None), ("q4_k", None), ("mxfp4", None), ("q4_k", "q8_0")])
+@pytest.mark.parametrize("n,M", [(1, 1), (8, 1), (16, 1), (3, 5)])
+@pytest.mark.parametrize("device", [False, True])
+def test_experts_swiglu_forward(hip, oracle, name, down, n, M, device):
+    rng = np.random.default_rng(340 + n + M)
+    H, I = 512, 256
+    ex = experts(oracle, name, n, H, I, H, rng, gated=True, down_name=down)
+    w = rng.uniform(0.05, 0.6, n).astype(np.float32)
+    x = rng.standard_normal((M, H)).astype(np.float32)
+    ref, parts = oracle.expert_set(x, ex, w)
+    fn = lambda r, i: hip.MoEExpertsSwiGLUForward(r, i, [qw(e["gate"], device) for e in ex], [qw(e["up"], device) for e in ex],
+                                                  [qw(e["down"], device) for e in ex], w)
+    got = run(hip, device, fn, np.full((M, H), np.nan, np.float32), x)
+    got = got[0] if device else got
+    tol = set_tol(oracle, parts, w)
+    assert np.all(np.abs(got - ref) <= tol), (name, n, M, device, float(np.max(np.abs(got - ref) / tol)))
+
+
+@pytest.mark.parametrize("shared", [None, "same", "wider", "other_type"])
+@pytest.mark.parametrize("n,M", [(8, 1), (32, 1), (4, 3)])
+@pytest.mark.parametrize("device", [False, True])
+def test_experts_swiglu_residual_with_shared_expert(hip, oracle, shared, n, M, device):
+    rng = np.random.default_rng(350 + n + M)
+    H, I = 512, 256
+    ex = experts(oracle, "q4_k", n, H, I, H, rng, gated=True)
+    w = rng.uniform(0.02, 0.3, n).astype(np.float32)
+    x = rng.standard_normal((M, H)).astype(np.float32)
+    resid = rng.standard_normal((M, H)).astype(np.float32)
+    all_ex, all_w, sh = list(ex), list(w), None
+    scalar = 0.37
+    if shared is not None:
+        si = 512 if shared == "wider" else I
+        sname = "q8_0" if shared == "other_type" else "q4_k"
+        s = experts(oracle, sname, 1, H, si, H, rng, gated=True)[0]
+        all_ex.append(s)
+        all_w.append(scalar)
+        sh = (qw(s["gate"], device), qw(s["up"], device), qw(s["down"], device))
+    ref, parts = oracle.expert_set(x, all_ex, all_w, base=resid)
+    fn = lambda r, i: hip.MoEExpertsSwiGLUResidual(r, i, [qw(e["gate"], device) for e in ex], [qw(e["up"], device) for e in ex],
+                                                   [qw(e["down"], device) for e in ex], w, shared=sh, shared_scalar=scalar)
+    got = run(hip, device, fn, resid.copy(), x)
+    got = got[0] if device else got
+    tol = set_tol(oracle, parts, all_w)
+    assert np.all(np.abs(got - ref) <= tol), (shared, n, M, device, float(np.max(np.abs(got - ref) / tol)))
+
+
+def test_expert_set_argument_errors(hip, oracle):
+    rng = np.random.default_rng(360)
+    H, I = 64, 64
+    ex = experts(oracle, "q8_0", 1, H, I, H, rng, gated=True)
+    x = np.zeros((1, H), np.float32)
+    out = np.zeros((1, H), np.float32)
+    g, u, d = qw(ex[0]["gate"], False), qw(ex[0]["up"], False), qw(ex[0]["down"], False)
+    with pytest.raises(RuntimeError, match="num_experts must be 1..16"):
+        hip.MoEExpertsForward(out, x, [u] * 17, [d] * 17, [0.1] * 17)
+    with pytest.raises(RuntimeError, match="num_experts must be 1..16"):
+        hip.MoEExpertsSwiGLUForward(out, x, [g] * 17, [u] * 17, [d] * 17, [0.1] * 17)
+    with pytest.raises(RuntimeError, match="num_experts must be 1..32"):
+        hip.MoEExpertsSwiGLUResidual(out, x, [g] * 33, [u] * 33, [d] * 33, [0.1] * 33)
+    with pytest.raises(RuntimeError, match="weight shapes do not match"):
+        hip.MoEExpertsSwiGLUForward(np.zeros((1, H + 32), np.float32), x, [g], [u], [d], [1.0])
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        hip.FusedOutProjFFN(np.zeros((2, H), np.float32), x, u, np.ones(H, np.float32), EPS, g, d, 32)
+    hip.ClearHostBufferCache()

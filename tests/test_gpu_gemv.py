@@ -168,7 +168,7 @@ def test_error_paths(hip, oracle):
     assert "m1.dim0 != result.dim0" in call(y[:1], x, wq.ctypes.data, Q4_K, K, Nn, wq.size)
     assert "quantized weight dims don't match" in call(y, x, wq.ctypes.data, Q4_K, K, Nn + 1, wq.size)
     assert "quantized weight dims don't match" in call(y, x[:, :128], wq.ctypes.data, Q4_K, K, Nn, wq.size)
-    assert "Unsupported quantized weight type" in call(y, x, wq.ctypes.data, 10, K, Nn, wq.size)      # Q2_K
+    assert "Unsupported weight type" in call(y, x, wq.ctypes.data, 10, K, Nn, wq.size)      # Q2_K
     assert "too small" in call(y, x, wq.ctypes.data, Q4_K, K, Nn, wq.size - 144)
     x32 = np.zeros((2, 32), np.float32)
     assert "multiple of the block size" in call(y, x32, wq.ctypes.data, Q4_K, 32, Nn, wq.size)

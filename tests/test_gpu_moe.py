@@ -41,7 +41,7 @@ def make_experts(oracle, t, E, H, F, rng, sigma=0.05):
 def run_gpu(hip, t, gu, gb, dn, db, E, H, F, hidden, ids, wts):
     import torch
     c = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    out = hip.MoEExpertsForward(c(hidden), c(ids.astype(np.int32)), c(wts), c(gu), c(gb), c(dn), c(db), t, E, H, F)
+    out = hip.MoEExpertsGptOssForward(c(hidden), c(ids.astype(np.int32)), c(wts), c(gu), c(gb), c(dn), c(db), t, E, H, F)
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -94,7 +94,7 @@ def test_config4_mxfp4_moe(hip, oracle, T):
     wts = np.exp(lg - lg.max(1, keepdims=True))
     wts = (wts / wts.sum(1, keepdims=True)).astype(np.float32)
     c = lambda a: torch.from_numpy(a).cuda()
-    out = hip.MoEExpertsForward(c(hidden), c(ids), c(wts), gu_d, None, dn_d, None, MXFP4, E, H, F)
+    out = hip.MoEExpertsGptOssForward(c(hidden), c(ids), c(wts), gu_d, None, dn_d, None, MXFP4, E, H, F)
     torch.cuda.synchronize()
     got = out.cpu().numpy()
     gu, dn = gu_d.cpu().numpy(), dn_d.cpu().numpy()

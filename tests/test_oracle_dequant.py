@@ -230,3 +230,24 @@ def test_iq4_nl_f16_bf16_closed_form(oracle):
     assert np.array_equal(y.view(np.uint32)[ok], want.view(np.uint32)[ok])
     y = oracle.dequantize(BF16, codes.view(np.uint8))
     assert np.array_equal(y.view(np.uint32), codes.astype(np.uint32) << 16)
+
+
+def test_q8_1_closed_form_all_scales(oracle):
+    # Q8_1 (ManagedQuantizedOps.cs:429-445): fp16 d at byte 0, the fp16 sum term at byte 2 is skipped, 32 int8 at byte 4.
+    # ggml has no dequantizer for this activation format, so the pin is the closed form y = q * float(d) over every
+    # scale code; filling the skipped bytes with a value that would change the result catches a wrong offset.
+    from oracle.oracle import Q8_1
+    codes = np.arange(65536, dtype=np.uint16)
+    raw = np.zeros((65536, 36), dtype=np.uint8)
+    raw[:, 0] = codes & 0xFF
+    raw[:, 1] = codes >> 8
+    raw[:, 2] = 0x55
+    raw[:, 3] = 0x7B          # a large finite fp16 in the sum slot
+    q = ((np.arange(32)[None, :] * 29 + codes[:, None] * 7) % 256).astype(np.uint8)
+    raw[:, 4:] = q
+    y = oracle.dequantize(Q8_1, raw.reshape(-1)).reshape(65536, 32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = q.view(np.int8).astype(np.float32) * codes.view(np.float16).astype(np.float32)[:, None]
+    ok = ~np.isnan(want)
+    assert np.array_equal(y.view(np.uint32)[ok], want.view(np.uint32)[ok])
+    assert oracle.row_size(Q8_1, 64) == 72
