@@ -55,6 +55,18 @@ typedef struct TSHipTensorView2D {
     int64_t raw_bytes;
 } TSHipTensorView2D;
 
+/* ggml_ops_internal.h TensorView3DDesc == GgmlNative.cs:49-71 (GgmlTensorView3D): strides in elements. */
+typedef struct TSHipTensorView3D {
+    void* data;
+    int dim0;
+    int dim1;
+    int dim2;
+    int stride0;
+    int stride1;
+    int stride2;
+    int64_t raw_bytes;
+} TSHipTensorView3D;
+
 /* ggml_ops_internal.h:104-109 == GgmlNative.cs:100-113 (GgmlContiguousTensor). element_type: 0 = F32, 3 = I32. */
 typedef struct TSHipContiguousTensor {
     void* data;
@@ -285,6 +297,20 @@ TSHIP_EXPORT int TSHip_MoEExpertsSwiGLUResidualF32Device(
     int64_t shared_gate_raw_bytes, int shared_up_ggml_type, int64_t shared_up_ne0, int64_t shared_up_ne1,
     int64_t shared_up_raw_bytes, int shared_down_ggml_type, int64_t shared_down_ne0, int64_t shared_down_ne1,
     int64_t shared_down_raw_bytes, float shared_scalar);
+
+/* replaces TSGgml_MulMatIdF32 (ggml_ops_matmul.cpp:958-1121, :1427-1449; GgmlNative.cs:433-439, :1076-1079): ggml_mul_mat_id
+ * with F32 expert weights, not a quantized path.  expert_weights [E x rows x K], input [T x slots x K], ids [ids_rows x
+ * ids_cols] (I32, or F32 truncated) with ids_rows == T and ids_cols a multiple of slots;
+ *   result[t][s][r] = sum_k expert_weights[ids[t][s]][r][k] * input[t][s % slots][k],  result [T x ids_cols x rows].
+ * Host pointers, standard views (innermost stride 1, no overlap); like the bridge the weights travel on every call
+ * (nothing is cached).  An id outside [0, E) is an error (the bridge's ggml asserts). */
+TSHIP_EXPORT int TSHip_MulMatIdF32(TSHipTensorView3D result, TSHipTensorView3D expert_weights, TSHipTensorView3D input,
+                                   TSHipContiguousTensor ids, int ids_rows, int ids_cols);
+
+/* device-pointer form: ids is a device array of ids_rows x ids_cols int32; rows of an out-of-range id are zero;
+ * ids_rows * ids_cols <= 65535.  Asynchronous on the selected stream. */
+TSHIP_EXPORT int TSHip_MulMatIdF32Device(TSHipTensorView3D result, TSHipTensorView3D expert_weights, TSHipTensorView3D input,
+                                         const int32_t* ids, int ids_rows, int ids_cols);
 
 /* replaces TSGgml_GetRowsQuantF32 (ggml_ops_matmul.cpp:519-668, :1339-1368; GgmlNative.cs:324, :1003-1006; caller
  * ModelBase.cs:826-856 embedding lookup): result[i, 0..ne0) = dequantized row indices[i] of the [ne1 x ne0] source

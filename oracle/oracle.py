@@ -313,6 +313,20 @@ class Oracle:
         normed = self.rms_norm_mul(res.astype(np.float32), norm_w, eps)
         return res, normed, self.matmul_any_f64(*router, normed), mm1
 
+    @staticmethod
+    def mul_mat_id(experts, x, ids):
+        """ggml_mul_mat_id with F32 experts (include/ggml.h:1409-1413; bridge call ggml_ops_matmul.cpp:958-1121):
+        out[t, s, :] = experts[ids[t, s]] @ x[t, s % slots], accumulated in fp64.  experts [E, rows, K], x [T, slots, K]."""
+        experts = np.asarray(experts, dtype=np.float64)
+        x = np.asarray(x, dtype=np.float64)
+        ids = np.asarray(ids).astype(np.int64)
+        T, cols = ids.shape
+        out = np.empty((T, cols, experts.shape[1]), dtype=np.float64)
+        for t in range(T):
+            for s in range(cols):
+                out[t, s] = experts[ids[t, s]] @ x[t, s % x.shape[1]]
+        return out
+
 
 class Reference:
     """The reference's own ggml code, compiled from its sources by `make ref`.

@@ -7,5 +7,5 @@ gguf            GGUF file reader (memory-mapped) and weight upload from the mapp
 build           hipcc build of the shared library
 """
 from . import hip_native  # noqa: F401
-from .hip_basic_ops import HipBasicOps, QuantizedWeight  # noqa: F401
+from .hip_basic_ops import HipBasicOps, QuantizedWeight, FuseGateUpWeights, FuseQKVWeights  # noqa: F401
 from .gguf import GgufFile  # noqa: F401

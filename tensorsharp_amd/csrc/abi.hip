@@ -2093,6 +2093,171 @@ int TSHip_MoEExpertsSwiGLUResidualF32Device(TSHipTensorView2D residual, TSHipTen
     });
 }
 
+/* ---- ggml_mul_mat_id with F32 experts (ggml_ops_matmul.cpp:958-1121) --------------------------- */
+namespace {
+
+bool validate_desc3(const TSHipTensorView3D& d, const char* name)
+{
+    if (d.data == nullptr) {
+        set_last_error(std::string("Null pointer passed for ") + name + '.');
+        return false;
+    }
+    if (d.dim0 <= 0 || d.dim1 <= 0 || d.dim2 <= 0) {
+        set_last_error(std::string("Invalid tensor shape passed for ") + name + '.');
+        return false;
+    }
+    if (d.stride0 < 0 || d.stride1 < 0 || d.stride2 < 0) {
+        set_last_error(std::string("Negative tensor strides are not supported for ") + name + '.');
+        return false;
+    }
+    const int64_t max_off = ((int64_t)d.dim0 - 1) * d.stride0 + ((int64_t)d.dim1 - 1) * d.stride1 + ((int64_t)d.dim2 - 1) * d.stride2;
+    if (d.raw_bytes <= 0 || (d.raw_bytes % (int64_t)sizeof(float)) != 0 || d.raw_bytes < (max_off + 1) * (int64_t)sizeof(float)) {
+        set_last_error(std::string("Invalid raw byte size passed for ") + name + '.');
+        return false;
+    }
+    return true;
+}
+
+// innermost stride 1, rows and planes do not overlap (ggml_ops_core.cpp can_map_standard_view, 3-D form)
+bool is_standard_view3(const TSHipTensorView3D& d)
+{
+    return d.stride2 == 1 && (d.dim1 == 1 || d.stride1 >= d.dim2) && (d.dim0 == 1 || (int64_t)d.stride0 >= (int64_t)d.stride1 * (d.dim1 - 1) + d.dim2);
+}
+
+bool validate_mul_mat_id(const TSHipTensorView3D& result, const TSHipTensorView3D& experts, const TSHipTensorView3D& input, const void* ids,
+                         int ids_rows, int ids_cols)
+{
+    if (!validate_desc3(result, "result") || !validate_desc3(experts, "expertWeights") || !validate_desc3(input, "input")) return false;
+    if (ids == nullptr) {
+        set_last_error("Null pointer passed for ids.");
+        return false;
+    }
+    if (ids_rows <= 0 || ids_cols <= 0) {
+        set_last_error("mulmatid requires positive id matrix dimensions.");
+        return false;
+    }
+    if (experts.dim2 != input.dim2) {
+        set_last_error("mulmatid expects expert weights and input to share the inner dimension.");
+        return false;
+    }
+    if (input.dim0 != ids_rows || (ids_cols % input.dim1) != 0) {
+        set_last_error("mulmatid expects ids rows to match input tokens and ids cols to broadcast over input expert slots.");
+        return false;
+    }
+    if (result.dim0 != input.dim0 || result.dim1 != ids_cols || result.dim2 != experts.dim1) {
+        set_last_error("mulmatid expects result shape [tokens, expert_used, rows].");
+        return false;
+    }
+    if (!is_standard_view3(result) || !is_standard_view3(experts) || !is_standard_view3(input)) {
+        set_last_error("Tensor layout is not supported by the mulmatid path.");
+        return false;
+    }
+    return true;
+}
+
+bool run_mul_mat_id(const TSHipTensorView3D& result, const TSHipTensorView3D& experts, const TSHipTensorView3D& input, const int32_t* ids_dev,
+                    int ids_cols, hipStream_t stream)
+{
+    return launch_mul_mat_id_f32(static_cast<const float*>(experts.data), experts.stride0, experts.stride1, experts.dim0, experts.dim1,
+                                 experts.dim2, static_cast<const float*>(input.data), input.stride0, input.stride1, input.dim1, ids_dev,
+                                 input.dim0, ids_cols, static_cast<float*>(result.data), result.stride0, result.stride1, stream);
+}
+
+}  // namespace
+
+int TSHip_MulMatIdF32Device(TSHipTensorView3D result, TSHipTensorView3D expert_weights, TSHipTensorView3D input, const int32_t* ids,
+                            int ids_rows, int ids_cols)
+{
+    return guarded(0, "mulmatid", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_mul_mat_id(result, expert_weights, input, ids, ids_rows, ids_cols)) return 0;
+        if (!run_mul_mat_id(result, expert_weights, input, ids, ids_cols, t_stream)) return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_MulMatIdF32(TSHipTensorView3D result, TSHipTensorView3D expert_weights, TSHipTensorView3D input, TSHipContiguousTensor ids,
+                      int ids_rows, int ids_cols)
+{
+    return guarded(0, "mulmatid", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_mul_mat_id(result, expert_weights, input, ids.data, ids_rows, ids_cols)) return 0;
+        const int64_t n_ids = (int64_t)ids_rows * ids_cols;
+        if (ids.element_count != n_ids || (ids.element_type != 0 && ids.element_type != 3)) {
+            set_last_error("mulmatid: ids must hold ids_rows x ids_cols I32 (or F32) values.");
+            return 0;
+        }
+        std::vector<int32_t> id_host((size_t)n_ids);
+        if (ids.element_type == 3) {
+            std::memcpy(id_host.data(), ids.data, (size_t)n_ids * sizeof(int32_t));
+        } else {
+            for (int64_t i = 0; i < n_ids; ++i) id_host[(size_t)i] = (int32_t)static_cast<const float*>(ids.data)[i];
+        }
+        for (int32_t e : id_host)
+            if (e < 0 || e >= expert_weights.dim0) {
+                set_last_error("mulmatid: expert id out of range.");
+                return 0;
+            }
+        // contiguous device copies: [ids][input T x slots x K][weights E x rows x K][result T x cols x rows]
+        auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+        const int T = input.dim0, slots = input.dim1, K = input.dim2, E = expert_weights.dim0, rows = expert_weights.dim1;
+        const size_t id_bytes = al((size_t)n_ids * sizeof(int32_t)), x_bytes = al((size_t)T * slots * K * sizeof(float));
+        const size_t w_bytes = al((size_t)E * rows * K * sizeof(float)), y_bytes = al((size_t)T * ids_cols * rows * sizeof(float));
+        std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
+        if (!ws_reserve(id_bytes + x_bytes + w_bytes + y_bytes, std::max(id_bytes + x_bytes, y_bytes))) return 0;
+        char* dev = static_cast<char*>(g_ws.dev);
+        char* pin = static_cast<char*>(g_ws.pinned);
+        std::memcpy(pin, id_host.data(), (size_t)n_ids * sizeof(int32_t));
+        float* xs = reinterpret_cast<float*>(pin + id_bytes);
+        for (int t = 0; t < T; ++t)
+            for (int s = 0; s < slots; ++s)
+                std::memcpy(xs + ((size_t)t * slots + s) * K,
+                            static_cast<const float*>(input.data) + (size_t)t * input.stride0 + (size_t)s * input.stride1, (size_t)K * sizeof(float));
+        hipStream_t stream = nullptr;
+        if (!hip_ok(hipMemcpyAsync(dev, pin, id_bytes + x_bytes, hipMemcpyHostToDevice, stream), "hipMemcpy(inputs)")) return 0;
+        // the weights go up from the caller's (pageable) memory plane by plane, row by row when rows are padded
+        float* w_dev = reinterpret_cast<float*>(dev + id_bytes + x_bytes);
+        const float* w_host = static_cast<const float*>(expert_weights.data);
+        if (expert_weights.stride1 == K && (E == 1 || expert_weights.stride0 == (int64_t)rows * K)) {
+            if (!hip_ok(hipMemcpy(w_dev, w_host, (size_t)E * rows * K * sizeof(float), hipMemcpyHostToDevice), "hipMemcpy(expert weights)")) return 0;
+        } else {
+            for (int e = 0; e < E; ++e)
+                if (!hip_ok(hipMemcpy2D(w_dev + (size_t)e * rows * K, (size_t)K * sizeof(float), w_host + (size_t)e * expert_weights.stride0,
+                                        (size_t)expert_weights.stride1 * sizeof(float), (size_t)K * sizeof(float), (size_t)rows,
+                                        hipMemcpyHostToDevice),
+                            "hipMemcpy2D(expert weights)"))
+                    return 0;
+        }
+        float* y_dev = reinterpret_cast<float*>(dev + id_bytes + x_bytes + w_bytes);
+        const TSHipTensorView3D xd{dev + id_bytes, T, slots, K, slots * K, K, 1, (int64_t)((size_t)T * slots * K * sizeof(float))};
+        const TSHipTensorView3D wd{w_dev, E, rows, K, rows * K, K, 1, (int64_t)((size_t)E * rows * K * sizeof(float))};
+        const TSHipTensorView3D yd{y_dev, T, ids_cols, rows, ids_cols * rows, rows, 1, (int64_t)((size_t)T * ids_cols * rows * sizeof(float))};
+        // (token, slot) pairs in launches of at most 65535
+        const int t_step = std::max(1, 65535 / ids_cols);
+        if (ids_cols > 65535) {
+            set_last_error("mulmatid: more than 65535 id columns.");
+            return 0;
+        }
+        for (int t0 = 0; t0 < T; t0 += t_step) {
+            const int tn = std::min(t_step, T - t0);
+            TSHipTensorView3D xs_v = xd, ys_v = yd;
+            xs_v.data = static_cast<float*>(xd.data) + (size_t)t0 * xd.stride0, xs_v.dim0 = tn;
+            ys_v.data = static_cast<float*>(yd.data) + (size_t)t0 * yd.stride0, ys_v.dim0 = tn;
+            if (!run_mul_mat_id(ys_v, wd, xs_v, reinterpret_cast<const int32_t*>(dev) + (size_t)t0 * ids_cols, ids_cols, stream)) return 0;
+        }
+        if (!hip_ok(hipMemcpyAsync(pin, y_dev, (size_t)T * ids_cols * rows * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpy(result)")) return 0;
+        if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+        const float* ys = reinterpret_cast<const float*>(pin);
+        for (int t = 0; t < T; ++t)
+            for (int s = 0; s < ids_cols; ++s)
+                std::memcpy(static_cast<float*>(result.data) + (size_t)t * result.stride0 + (size_t)s * result.stride1,
+                            ys + ((size_t)t * ids_cols + s) * rows, (size_t)rows * sizeof(float));
+        clear_last_error();
+        return 1;
+    });
+}
+
 }  // extern "C"
 
 namespace {

@@ -127,6 +127,28 @@ __global__ void __launch_bounds__(256) dense_matmul_kernel(const T* __restrict__
     }
 }
 
+// ggml_mul_mat_id with F32 experts (include/ggml.h:1409-1413): out[t][s][r] = sum_k W[ids[t][s]][r][k] * x[t][s % slots][k].
+// One wavefront per output row r of one (t, s) pair; rows of an id outside [0, E) are zero.
+__global__ void __launch_bounds__(256) mul_mat_id_f32_kernel(const float* __restrict__ w, int64_t w_s0, int64_t w_s1, int E, int rows,
+                                                            int K, const float* __restrict__ x, int64_t x_s0, int64_t x_s1, int slots,
+                                                            const int32_t* __restrict__ ids, int cols, float* __restrict__ out,
+                                                            int64_t o_s0, int64_t o_s1)
+{
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int t = blockIdx.y / cols, s = blockIdx.y % cols;
+    if (r >= rows) return;
+    const int e = ids[(int64_t)t * cols + s];
+    float acc = 0.f;
+    if (e >= 0 && e < E) {
+        const float* wr = w + (int64_t)e * w_s0 + (int64_t)r * w_s1;
+        const float* xr = x + (int64_t)t * x_s0 + (int64_t)(s % slots) * x_s1;
+        for (int k = lane; k < K; k += 64) acc = fmaf(wr[k], xr[k], acc);
+    }
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+    if (lane == 0) out[(int64_t)t * o_s0 + (int64_t)s * o_s1 + r] = acc;
+}
+
 }  // namespace
 
 bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps, int M, int K, float* out, hipStream_t stream)
@@ -196,6 +218,19 @@ bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, f
         return false;
     }
     return hip_ok(hipGetLastError(), "dense matmul launch");
+}
+
+bool launch_mul_mat_id_f32(const float* w, int64_t w_s0, int64_t w_s1, int E, int rows, int K, const float* x, int64_t x_s0, int64_t x_s1,
+                           int slots, const int32_t* ids, int T, int cols, float* out, int64_t o_s0, int64_t o_s1, hipStream_t stream)
+{
+    if (T <= 0 || cols <= 0 || rows <= 0) return true;
+    if ((int64_t)T * cols > 65535 || slots <= 0) {
+        set_last_error("mulmatid: more than 65535 (token, slot) pairs per call.");
+        return false;
+    }
+    hipLaunchKernelGGL(mul_mat_id_f32_kernel, dim3((rows + 3) / 4, T * cols), dim3(256), 0, stream, w, w_s0, w_s1, E, rows, K, x, x_s0, x_s1,
+                       slots, ids, cols, out, o_s0, o_s1);
+    return hip_ok(hipGetLastError(), "mulmatid launch");
 }
 
 }  // namespace tship

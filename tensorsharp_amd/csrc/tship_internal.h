@@ -187,6 +187,10 @@ bool launch_weighted_sum(const float* rows, int64_t set_stride, const WeightedSu
 // y[m][n] (+)= sum_k W[n][k] x[m][k] for a dense row-major weight of type F32, F16 or BF16
 bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, float* y, int64_t ldy, int M, int N, int K,
                          bool accumulate, hipStream_t stream);
+// out[t][s][0..rows) = W[ids[t][s]] (rows x K, fp32) * x[t][s % slots]; strides in elements, innermost stride 1;
+// T * cols <= 65535; rows of an id outside [0, E) are zero
+bool launch_mul_mat_id_f32(const float* w, int64_t w_s0, int64_t w_s1, int E, int rows, int K, const float* x, int64_t x_s0, int64_t x_s1,
+                           int slots, const int32_t* ids, int T, int cols, float* out, int64_t o_s0, int64_t o_s1, hipStream_t stream);
 inline bool is_dense_type(int type) { return type == kTypeF32 || type == kTypeF16 || type == kTypeBF16; }
 // every weight type the matmul entry points take; Q8_1 weights are dequantized to fp32 in slices of rows and then take
 // the dense kernel

@@ -237,8 +237,9 @@ class GgufFile:
                 warnings.simplefilter("ignore", UserWarning)      # read-only mapping: it is only ever read
                 src = torch.frombuffer(self._map, dtype=torch.uint8, count=data.size, offset=self.DataOffset + info.Offset)
             t.copy_(src)
-            data = t
-        return QuantizedWeight(data, info.Type, info.Shape[0], info.Shape[1])
+            return QuantizedWeight(t, info.Type, info.Shape[0], info.Shape[1])
+        # a view of the mapping, kept alive by this file object: adjacent tensors concatenate without a copy
+        return QuantizedWeight.CreateExternalView(data, info.Type, info.Shape[0], info.Shape[1], self)
 
     def preload(self, names=None):
         """Upload matrices once through the bridge's preload export, keyed by their mapped address: later host-pointer

@@ -17,26 +17,171 @@ from . import hip_native as N
 
 
 class QuantizedWeight:
-    """Raw GGUF blocks of one 2-D weight: the fields of ModelBase.QuantizedWeight
-    (TensorSharp.Models/ModelBase.cs:24-202) that the matmul boundary consumes."""
+    """Raw GGUF blocks of one 2-D weight: twin of ModelBase.QuantizedWeight (TensorSharp.Models/ModelBase.cs:24-202).
 
-    def __init__(self, data, ggml_type, ne0, ne1):
+    data        numpy uint8 array (host) or torch uint8 CUDA tensor (device) holding ne1 rows of row_size(type, ne0) bytes
+    cache_key   the pointer the matmul entry points take as m2_data: the host address, or - after
+                EnsureDeviceCacheKey() - an opaque key that stays valid once the host bytes are released
+    An instance either owns its bytes (built from an array, or a concatenated copy) or is an external view of a larger
+    buffer kept alive by `owner_token` (the GGUF mapping); adjacent external views of one owner concatenate without
+    a copy."""
+
+    def __init__(self, data, ggml_type, ne0, ne1, owner_token=None):
         self.ggml_type = int(ggml_type)
         self.ne0 = int(ne0)   # K, in features
         self.ne1 = int(ne1)   # N, out features
-        self.data = data      # numpy uint8 (host) or torch uint8 CUDA tensor (device)
+        self.data = data
         self.raw_bytes = int(data.numel() if hasattr(data, "numel") else data.size)
+        self._owner_token = owner_token
+        self._owns_buffer = owner_token is None
+        self._key = None      # opaque device cache key (EnsureDeviceCacheKey)
         expect = HipBasicOps.GetRowSizeBytes(self.ggml_type, self.ne0) * self.ne1
         if self.raw_bytes < expect:
             raise ValueError(f"weight bytes {self.raw_bytes} < {expect} for {ne1}x{ne0} type {ggml_type}")
 
+    # -- storage -----------------------------------------------------------------------------
     @property
     def is_device(self):
         return hasattr(self.data, "data_ptr")
 
     @property
+    def HasHostData(self):
+        return self.data is not None and not self.is_device
+
+    @property
+    def HasExternalHostView(self):
+        return self.HasHostData and not self._owns_buffer and self._owner_token is not None
+
+    @property
     def ptr(self):
+        """what the matmul entry points receive: the cache key when the bytes were released, else the data address"""
+        if self.data is None:
+            if self._key is None:
+                raise RuntimeError("Quantized weight has neither host data nor a device cache key.")
+            return self._key
         return self.data.data_ptr() if self.is_device else self.data.ctypes.data
+
+    @property
+    def CacheKey(self):
+        return self._key if self._key is not None else (0 if self.data is None else self.ptr)
+
+    @staticmethod
+    def AllocateBuffer(size):
+        """64-byte aligned host bytes (ModelBase.cs:189-195)"""
+        raw = np.empty(int(size) + 64, dtype=np.uint8)
+        off = (-raw.ctypes.data) % 64
+        return raw[off:off + int(size)]
+
+    @staticmethod
+    def CreateExternalView(data, ggml_type, ne0, ne1, owner_token):
+        """A view of bytes owned by `owner_token` (ModelBase.cs:82-90)."""
+        if data is None or (hasattr(data, "size") and data.size == 0):
+            raise ValueError("External quantized weight view requires a non-empty data view.")
+        if owner_token is None:
+            raise ValueError("ownerToken must not be None.")
+        return QuantizedWeight(data, ggml_type, ne0, ne1, owner_token=owner_token)
+
+    @staticmethod
+    def TryCreateConcatenatedView(*weights):
+        """One weight of ne1 = sum(ne1) over byte-adjacent external views of the same owner, type and row length; None when
+        the views do not qualify (ModelBase.cs:92-126)."""
+        if len(weights) < 2 or weights[0] is None:
+            return None
+        first = weights[0]
+        if not first.HasHostData or first._owns_buffer or first._owner_token is None:
+            return None
+        total_bytes = total_ne1 = 0
+        expected = first.ptr
+        for w in weights:
+            if (w is None or not w.HasHostData or w._owns_buffer or w._owner_token is not first._owner_token or
+                    w.ggml_type != first.ggml_type or w.ne0 != first.ne0 or w.ptr != expected):
+                return None
+            total_bytes += w.raw_bytes
+            total_ne1 += w.ne1
+            expected += w.raw_bytes
+        span = (C.c_uint8 * total_bytes).from_address(first.ptr)
+        data = np.frombuffer(span, dtype=np.uint8)
+        fused = QuantizedWeight(data, first.ggml_type, first.ne0, total_ne1, owner_token=first._owner_token)
+        fused._keepalive = [w.data for w in weights]     # the span borrows these views' memory
+        return fused
+
+    @staticmethod
+    def ConcatOrCreateCopy(*weights):
+        """Rows of the weights stacked in order: a view when they are adjacent in one mapping, else a copy into a fresh
+        aligned buffer (ModelBase.cs:128-159)."""
+        if len(weights) == 0 or weights[0] is None:
+            raise ValueError("At least one quantized weight is required.")
+        fused = QuantizedWeight.TryCreateConcatenatedView(*weights)
+        if fused is not None:
+            return fused
+        first = weights[0]
+        total = 0
+        for w in weights:
+            if w is None:
+                raise ValueError("Quantized weight list cannot contain null entries.")
+            if not w.HasHostData:
+                raise RuntimeError("Cannot concatenate quantized weights after their host storage has been released.")
+            total += w.raw_bytes
+        buf = QuantizedWeight.AllocateBuffer(total)
+        off = 0
+        for w in weights:
+            buf[off:off + w.raw_bytes] = w.data.reshape(-1)
+            off += w.raw_bytes
+        return QuantizedWeight(buf, first.ggml_type, first.ne0, sum(w.ne1 for w in weights))
+
+    def EnsureDeviceCacheKey(self):
+        """An opaque key for PreloadQuantizedWeight that outlives the host bytes (ModelBase.cs:161-170: a GCHandle there,
+        the address of a small pinned-by-reference buffer here)."""
+        if self._key is None:
+            self._key_anchor = np.zeros(1, dtype=np.uint8)
+            self._key = self._key_anchor.ctypes.data
+        return self._key
+
+    def ReleaseHostData(self):
+        """Drop the host bytes (ModelBase.cs:172-187); the weight stays usable through its device cache key."""
+        self.data = None
+        self._owns_buffer = False
+        self._owner_token = None
+        self._keepalive = None
+
+    def Dispose(self):
+        self.ReleaseHostData()
+        self._key = None
+
+
+def FuseGateUpWeights(quant_weights, num_layers):
+    """Twin of ModelBase.FuseGateUpWeights (ModelBase.cs:768-802) for the quantized branch: blk.L.ffn_gate.weight and
+    blk.L.ffn_up.weight of equal type and row length become blk.L.ffn_gate_up.weight (gate rows, then up rows); the two
+    originals are removed and disposed.  Returns the number of layers fused."""
+    fused = 0
+    for layer in range(int(num_layers)):
+        gate_name, up_name = f"blk.{layer}.ffn_gate.weight", f"blk.{layer}.ffn_up.weight"
+        gw, uw = quant_weights.get(gate_name), quant_weights.get(up_name)
+        if gw is None or uw is None or gw.ggml_type != uw.ggml_type or gw.ne0 != uw.ne0:
+            continue
+        quant_weights[f"blk.{layer}.ffn_gate_up.weight"] = QuantizedWeight.ConcatOrCreateCopy(gw, uw)
+        del quant_weights[gate_name], quant_weights[up_name]
+        gw.Dispose()
+        uw.Dispose()
+        fused += 1
+    return fused
+
+
+def FuseQKVWeights(quant_weights, num_layers):
+    """Twin of the models' FuseQKVWeights (Qwen3Model.cs:57-85): attn_q / attn_k / attn_v of equal type and row length
+    become blk.L.attn_qkv.weight."""
+    fused = 0
+    for layer in range(int(num_layers)):
+        names = [f"blk.{layer}.attn_{p}.weight" for p in "qkv"]
+        ws = [quant_weights.get(n) for n in names]
+        if any(w is None for w in ws) or any(w.ggml_type != ws[0].ggml_type or w.ne0 != ws[0].ne0 for w in ws):
+            continue
+        quant_weights[f"blk.{layer}.attn_qkv.weight"] = QuantizedWeight.ConcatOrCreateCopy(*ws)
+        for n, w in zip(names, ws):
+            del quant_weights[n]
+            w.Dispose()
+        fused += 1
+    return fused
 
 
 def _host_view(a, standard):
@@ -224,6 +369,36 @@ class HipBasicOps:
                 *HipBasicOps._shape_args(gate[0]), *HipBasicOps._shape_args(up[0]), *HipBasicOps._shape_args(down[0]), rw,
                 *sh, float(shared_scalar))
         N.check_result(ok, "moe_experts_swiglu_residual")
+
+    @staticmethod
+    def _view3(a):
+        """3-D fp32 view of a numpy array or a torch CUDA tensor (strides in elements)"""
+        host = isinstance(a, np.ndarray)
+        if (a.ndim if host else a.dim()) != 3 or str(a.dtype).split(".")[-1] != "float32":
+            raise ValueError("MulMatId requires 3D Float32 tensors.")
+        st = [v // 4 for v in a.strides] if host else list(a.stride())
+        span = (sum((d - 1) * s for d, s in zip(a.shape, st)) + 1) * 4
+        return N.TensorView3D(HipBasicOps._addr(a), a.shape[0], a.shape[1], a.shape[2], st[0], st[1], st[2], span)
+
+    @staticmethod
+    def MulMatId(result, expert_weights, input, ids):
+        """result[t, s, :] = expert_weights[ids[t, s]] @ input[t, s % slots] with F32 experts [E, rows, K]
+        (GgmlNative.MulMatId, GgmlNative.cs:1076-1079).  All host (numpy; ids int32 or float32) or all device (torch; ids
+        int32) tensors."""
+        host = isinstance(result, np.ndarray)
+        rows, cols = int(ids.shape[0]), int(ids.shape[1])
+        if host:
+            idc = np.ascontiguousarray(ids)
+            if idc.dtype not in (np.int32, np.float32):
+                raise ValueError("MulMatId ids must be Int32 or Float32.")
+            desc = N.ContiguousTensor(idc.ctypes.data, int(idc.size), 3 if idc.dtype == np.int32 else 0)
+            ok = N.lib().TSHip_MulMatIdF32(HipBasicOps._view3(result), HipBasicOps._view3(expert_weights),
+                                           HipBasicOps._view3(input), desc, rows, cols)
+        else:
+            HipBasicOps.UseCurrentStream()
+            ok = N.lib().TSHip_MulMatIdF32Device(HipBasicOps._view3(result), HipBasicOps._view3(expert_weights),
+                                                 HipBasicOps._view3(input), C.c_void_p(ids.contiguous().data_ptr()), rows, cols)
+        N.check_result(ok, "mulmatid")
 
     # -- embedding gather ------------------------------------------------------------------
     @staticmethod

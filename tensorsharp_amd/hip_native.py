@@ -24,6 +24,12 @@ class TensorView2D(C.Structure):
                 ("stride1", C.c_int), ("raw_bytes", C.c_int64)]
 
 
+class TensorView3D(C.Structure):
+    """GgmlTensorView3D (GgmlNative.cs:49-71): strides in elements, raw_bytes = span in bytes."""
+    _fields_ = [("data", C.c_void_p), ("dim0", C.c_int), ("dim1", C.c_int), ("dim2", C.c_int), ("stride0", C.c_int),
+                ("stride1", C.c_int), ("stride2", C.c_int), ("raw_bytes", C.c_int64)]
+
+
 class ContiguousTensor(C.Structure):
     """GgmlContiguousTensor (GgmlNative.cs:100-113)."""
     _fields_ = [("data", C.c_void_p), ("element_count", C.c_int64), ("element_type", C.c_int)]
@@ -96,6 +102,8 @@ SIGNATURES = {
                                                     C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
                                                     C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int64, C.c_int64,
                                                     C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_float]),
+    "TSHip_MulMatIdF32": (C.c_int, [TensorView3D, TensorView3D, TensorView3D, ContiguousTensor, C.c_int, C.c_int]),
+    "TSHip_MulMatIdF32Device": (C.c_int, [TensorView3D, TensorView3D, TensorView3D, C.c_void_p, C.c_int, C.c_int]),
     "TSHip_GetRowsQuantF32": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
                                         ContiguousTensor]),
     "TSHip_GetRowsQuantF32Device": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,

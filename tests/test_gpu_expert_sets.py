@@ -219,3 +219,35 @@ def test_expert_set_argument_errors(hip, oracle):
     with pytest.raises(RuntimeError, match="shape mismatch"):
         hip.FusedOutProjFFN(np.zeros((2, H), np.float32), x, u, np.ones(H, np.float32), EPS, g, d, 32)
     hip.ClearHostBufferCache()
+
+
+@pytest.mark.parametrize("slots", [1, 4])
+@pytest.mark.parametrize("device", [False, True])
+def test_mul_mat_id_f32_experts(hip, oracle, slots, device):
+    import torch
+    rng = np.random.default_rng(370 + slots)
+    E, rows, K, T, k = 6, 130, 200, 5, 4
+    w = (rng.standard_normal((E, rows, K)) * 0.1).astype(np.float32)
+    x = rng.standard_normal((T, slots, K)).astype(np.float32)
+    ids = rng.integers(0, E, (T, k)).astype(np.int32)
+    ref = oracle.mul_mat_id(w, x, ids)
+    if device:
+        out = torch.full((T, k, rows), float("nan"), device="cuda")
+        hip.MulMatId(out, torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda(), torch.from_numpy(ids).cuda())
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+    else:
+        got = np.full((T, k, rows), np.nan, np.float32)
+        hip.MulMatId(got, w, x, ids)
+        # F32 ids are truncated like the bridge's read_i32_values; a padded (strided) weight stack is packed on upload
+        got_f = np.full((T, k, rows), np.nan, np.float32)
+        wide = np.zeros((E, rows + 3, K + 5), np.float32)
+        wide[:, :rows, :K] = w
+        hip.MulMatId(got_f, wide[:, :rows, :K], x, ids.astype(np.float32) + 0.4)
+        assert np.array_equal(got_f, got)
+        with pytest.raises(RuntimeError, match="expert id out of range"):
+            hip.MulMatId(got_f, w, x, np.full((T, k), E, np.int32))
+        with pytest.raises(RuntimeError, match="share the inner dimension"):
+            hip.MulMatId(got_f, w, x[:, :, :K - 8], ids)
+    # fp32 accumulation of exact fp32 products
+    assert np.all(np.abs(got - ref) <= 1e-5 * np.linalg.norm(ref, axis=2, keepdims=True))

@@ -176,3 +176,34 @@ def test_ffn_swiglu_q4_k_gate_up_q6_k_down(hip, oracle, M):
     tol = 2e-3 * np.linalg.norm(mm, axis=1, keepdims=True)
     got = r.cpu().numpy()
     assert np.all(np.abs(got - ref) <= tol), (M, float(np.max(np.abs(got - ref) / tol)))
+
+
+@pytest.mark.parametrize("adjacent", [True, False])
+def test_gate_up_fused_at_load_feeds_the_ffn(hip, oracle, adjacent):
+    # ModelBase.FuseGateUpWeights (ModelBase.cs:768-802): gate and up become one [2F x H] weight - a view when the two
+    # tensors are adjacent in the mapping, a copy otherwise - and the fused FFN on it equals the FFN of the two halves
+    from tensorsharp_amd import QuantizedWeight, FuseGateUpWeights
+    rng = np.random.default_rng(101)
+    H, F, M = 512, 768, 3
+    gate = make(oracle, "q4_k", F, H, rng, 0.05)
+    up = make(oracle, "q4_k", F, H, rng, 0.05)
+    dn = make(oracle, "q4_k", H, F, rng, 0.05)
+    owner = object()
+    mapping = np.concatenate([gate, np.zeros(0 if adjacent else 144, np.uint8), up])
+    weights = {"blk.0.ffn_gate.weight": QuantizedWeight.CreateExternalView(mapping[:gate.size], Q4_K, H, F, owner),
+               "blk.0.ffn_up.weight": QuantizedWeight.CreateExternalView(mapping[mapping.size - up.size:], Q4_K, H, F, owner)}
+    assert FuseGateUpWeights(weights, 1) == 1
+    gu = weights["blk.0.ffn_gate_up.weight"]
+    assert (gu.ptr == mapping.ctypes.data) == adjacent and gu.ne1 == 2 * F
+    x = (rng.standard_normal((M, H)) * 2).astype(np.float32)
+    resid = rng.standard_normal((M, H)).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    xn = oracle.rms_norm_mul(x, nw, EPS)
+    g = oracle.matmul_f64(Q4_K, gate, F, H, xn).astype(np.float32)
+    u = oracle.matmul_f64(Q4_K, up, F, H, xn).astype(np.float32)
+    mm = oracle.matmul_f64(Q4_K, dn, H, F, oracle.silu_mul(np.concatenate([g, u], axis=1)))
+    got = resid.copy()
+    hip.FusedFFNSwiGLUQuant(got, x, nw, EPS, gu, QuantizedWeight(dn, Q4_K, F, H), F)
+    hip.ClearHostBufferCache()
+    tol = 2e-3 * np.linalg.norm(mm, axis=1, keepdims=True)
+    assert np.all(np.abs(got - (resid + mm)) <= tol)

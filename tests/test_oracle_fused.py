@@ -130,3 +130,23 @@ def test_dense_weight_rows(oracle):
     assert np.array_equal(oracle.weight_rows(BF16, b.view(np.uint8).reshape(-1), 4, 8), want)
     x = rng.standard_normal((3, 8)).astype(np.float32)
     assert np.allclose(oracle.matmul_any_f64(F16, h.view(np.uint8).reshape(-1), 4, 8, x), x.astype(np.float64) @ h.astype(np.float64).T)
+
+
+def test_mul_mat_id_brute_force_and_broadcast(oracle):
+    rng = np.random.default_rng(89)
+    E, rows, K, T, k = 5, 3, 4, 2, 4
+    w = rng.standard_normal((E, rows, K)).astype(np.float32)
+    ids = rng.integers(0, E, (T, k))
+    # one input slot broadcast over the k selected experts, then one slot per selected expert
+    for slots in (1, k, 2):
+        x = rng.standard_normal((T, slots, K)).astype(np.float32)
+        got = oracle.mul_mat_id(w, x, ids)
+        for t in range(T):
+            for s in range(k):
+                for r in range(rows):
+                    want = sum(float(w[ids[t, s], r, j]) * float(x[t, s % slots, j]) for j in range(K))
+                    assert abs(got[t, s, r] - want) < 1e-12
+    # the id picks the expert: a one-hot expert stack returns the selected expert's marker
+    mark = np.zeros((E, 1, 1), np.float32)
+    mark[:, 0, 0] = np.arange(E) + 1
+    assert np.array_equal(oracle.mul_mat_id(mark, np.ones((T, 1, 1), np.float32), ids)[:, :, 0], ids + 1)
