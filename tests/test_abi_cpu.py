@@ -109,3 +109,53 @@ def test_sync_host_buffer_is_a_no_op_for_pointers_that_were_never_cached():
     assert lib.TSHip_SyncHostBuffer(a.ctypes.data, 0) == 1
     assert N.get_last_error() == ""
     assert np.array_equal(a, np.arange(8, dtype=np.float32))
+
+
+# ---- the managed P/Invoke file declares the same argument lists as the header ----------------------------------
+def _c_params(decl):
+    """argument kinds of one C declaration: 'ptr', 'i32', 'i64', 'f32', 'size', or a struct name"""
+    out = []
+    for p in decl.split(","):
+        p = " ".join(p.split())
+        if not p or p == "void":
+            continue
+        if "*" in p:
+            out.append("ptr")
+            continue
+        ty = " ".join(p.split(" ")[:-1]).replace("const ", "")
+        out.append({"int": "i32", "int64_t": "i64", "float": "f32", "size_t": "size", "TSHipTensorView2D": "view2",
+                    "TSHipTensorView3D": "view3", "TSHipContiguousTensor": "contig"}[ty])
+    return out
+
+
+def _cs_params(decl):
+    out = []
+    for p in decl.split(","):
+        p = " ".join(p.split())
+        if not p:
+            continue
+        ty = p.split(" ")[0]
+        out.append({"IntPtr": "ptr", "IntPtr[]": "ptr", "long[]": "ptr", "float[]": "ptr", "int": "i32", "long": "i64",
+                    "float": "f32", "UIntPtr": "size", "HipTensorView2D": "view2", "HipTensorView3D": "view3",
+                    "HipContiguousTensor": "contig"}[ty])
+    return out
+
+
+def test_managed_pinvoke_declarations_match_the_header():
+    header = open(os.path.join(ROOT, "include", "tship_ops.h")).read()
+    cs = open(os.path.join(ROOT, "managed", "TensorSharp.Backends.HIP", "HipNative.cs")).read()
+    c_decls = {m.group(1): _c_params(m.group(2))
+               for m in re.finditer(r"TSHIP_EXPORT[^;(]*?\b(TSHip_\w+)\s*\(([^;]*?)\)\s*;", header, re.S)}
+    cs_decls = {m.group(1): _cs_params(m.group(2))
+                for m in re.finditer(r"static extern \S+ (TSHip_\w+)\s*\(([^;]*?)\)\s*;", cs, re.S)}
+    assert len(cs_decls) >= 25
+    for name, params in cs_decls.items():
+        assert name in c_decls, f"{name} bound in HipNative.cs but not declared in tship_ops.h"
+        assert params == c_decls[name], f"{name}: managed {params} != header {c_decls[name]}"
+    # every host-pointer export is bound (the *Device family and SetStream serve native callers that own device memory)
+    unbound = [n for n in c_decls if n not in cs_decls and not n.endswith("Device") and "NoAlloc" not in n and n != "TSHip_SetStream"]
+    assert unbound == [], unbound
+
+
+def test_struct_layout_3d_view():
+    assert C.sizeof(N.TensorView3D) == 40 and N.TensorView3D.raw_bytes.offset == 32
