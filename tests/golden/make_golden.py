@@ -98,7 +98,8 @@ def main():
     out["q8k_q"] = ref.quantize_q8_K(xa)
 
     # digests of the seeded BASELINE weights, quantized by the reference
-    for cfg_name, cfg in (("cfg1", inputs.CFG1), ("cfg2", inputs.CFG2), ("cfg4", inputs.CFG4)):
+    for cfg_name, cfg in (("cfg1", inputs.CFG1), ("cfg2", inputs.CFG2), ("cfg3", inputs.CFG3), ("cfg4", inputs.CFG4),
+                          ("cfg5", inputs.CFG5)):
         for tname, (fmt, N, K) in cfg.items():
             tag = f"{cfg_name}.{tname}"
             w = inputs.weights(tag, N * K)

@@ -83,9 +83,14 @@ def test_matches_reference_build(oracle, reference):
     assert np.array_equal(oracle.quantize_q8_K(xa), reference.quantize_q8_K(xa))
 
 
-@pytest.mark.parametrize("cfg_name,tname", [("cfg1", "ffn_up"), ("cfg2", "wk"), ("cfg2", "wq"), ("cfg4", "down")])
+ALL_BASELINE_WEIGHTS = [(c, t) for c in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5") for t in getattr(inputs, c.upper())]
+
+
+@pytest.mark.parametrize("cfg_name,tname", ALL_BASELINE_WEIGHTS)
 def test_baseline_weight_digests(oracle, golden, cfg_name, tname):
-    """SHA-256 of the reference-quantized bytes of the seeded BASELINE weights (full shapes)."""
+    """SHA-256 of the reference-quantized bytes of the seeded BASELINE weights, every config at its full shape (the
+    digests were written from the reference's own quantizers by tests/golden/make_golden.py): the oracle's quantizers
+    produce the same bytes, so the GPU tests below them run on reference-quantized weights."""
     fmt, N, K = getattr(inputs, cfg_name.upper())[tname]
     tag = f"{cfg_name}.{tname}"
     q = oracle.quantize(T[fmt], inputs.weights(tag, N * K))
