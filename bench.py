@@ -22,9 +22,12 @@ sys.path.insert(0, ROOT)
 
 Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 8, 12, 13, 14, 39
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the grouped Q4_K GEMV from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by the
-# reading of a 1 GiB copy (profiles/gemv_q4k_layer_hbm_traffic.txt); not measured by this script.
-MEASURED_TRAFFIC_BYTES = 124240000
+MFMA_FP16_PEAK_TFLOPS = 2516.6
+# HBM bytes per launch of the grouped Q4_K GEMV come from rocprofv3 FETCH_SIZE + WRITE_SIZE runs, not from this script.
+# The summary of those runs records the figure together with the SHA-256 of the kernel source it was measured on; the
+# figure is reported only while the source still has that digest.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemv_q4k_layer_hbm_traffic.txt")
+GEMV_SOURCE = os.path.join(ROOT, "tensorsharp_amd", "csrc", "gemv.hip")
 
 LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
     ("wq", 4096, 4096), ("wk", 1024, 4096), ("wv", 1024, 4096), ("wo", 4096, 4096),
@@ -84,6 +87,22 @@ def cpu_reference_ggml(layer_host, xs_host, n_threads):
             "seconds_per_layer": round(best, 4)}
 
 
+def measured_traffic_bytes():
+    """HBM bytes per launch from the committed counter summary, or None when the kernel source changed since."""
+    import hashlib
+    import re
+    try:
+        text = open(TRAFFIC_SUMMARY).read()
+        digest = hashlib.sha256(open(GEMV_SOURCE, "rb").read()).hexdigest()
+    except OSError:
+        return None
+    m_bytes = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    m_sha = re.search(r"^gemv_source_sha256:\s*([0-9a-f]{64})", text, re.M)
+    if not m_bytes or not m_sha or m_sha.group(1) != digest:
+        return None
+    return int(m_bytes.group(1))
+
+
 def time_region(fn, steps, torch):
     """fn(i) launches step i on the current stream. Returns (event_ms, wall_ms)."""
     e0 = torch.cuda.Event(enable_timing=True)
@@ -110,6 +129,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy (20 times): the known-size kernel against "
                          "which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
+    ap.add_argument("--aux", metavar="OP,TYPE,ROWS,K",
+                    help="time only the dequantizer (OP = dequant: ROWS x K weights to fp32) or the embedding gather "
+                         "(OP = get_rows: ROWS random rows of a 131072 x K table); for profiling a single kernel")
     ap.add_argument("--matmul", metavar="TYPE,M,N,K",
                     help="time only one matmul shape (GGUF type id, rows, out features, in features) through "
                          "TSHip_AddmmQuantF32Device, --steps calls after --warmup; for profiling a single kernel")
@@ -141,6 +163,35 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes_read": src.numel() * 4, "calibrate_copy_bytes_written": src.numel() * 4,
                           "launches": 20}))
+        return
+
+    def aux_case(op, t, rows, k, iters, warm):
+        """dequantizer / embedding gather through the device entry points; HBM bytes = blocks read + fp32 written"""
+        table_rows = rows if op == "dequant" else 131072
+        w = QuantizedWeight(synth.random_weight(t, table_rows, k, dev, seed=31), t, k, table_rows)
+        out_t = torch.empty((rows, k), device=dev, dtype=torch.float32)
+        gi = torch.Generator(device="cpu")
+        gi.manual_seed(5)
+        idx = [torch.randint(0, table_rows, (rows,), generator=gi, dtype=torch.int32).to(dev) for _ in range(8)]
+
+        def f(i):
+            if op == "dequant":
+                HipBasicOps.DequantizeToFloat32Device(t, w.data, rows * k, out_t.view(-1))
+            else:
+                HipBasicOps.GetRowsQuantDevice(out_t, w, idx[i % 8])
+        for i in range(warm):
+            f(i)
+        ev, wall = time_region(f, iters, torch)
+        us = ev * 1e3 / iters
+        b = rows * row_bytes(t, k) + rows * k * 4
+        return {"us_per_call_events": round(us, 2), "bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)}
+
+    if args.aux:
+        op, t, rows, k = args.aux.split(",")
+        r = aux_case(op, int(t), int(rows), int(k), args.steps, args.warmup)
+        r["aux"] = {"op": op, "type": int(t), "rows": int(rows), "K": int(k)}
+        print(json.dumps(r))
         return
 
     if args.matmul:
@@ -182,19 +233,27 @@ def main():
 
     for i in range(args.warmup):
         step(i)
-    ev_ms, wall_ms = time_region(step, args.steps, torch)
+    # exactly --steps steps between two synchronisations ...
+    k_ev_ms, k_wall_ms = time_region(step, args.steps, torch)
+    # ... and, because a region of a few steps of 25 us each is mostly the cost of the two synchronisations, a region of
+    # at least 200 steps from which `value` is taken; both are reported
+    timed_steps = max(args.steps, 200)
+    ev_ms, wall_ms = (k_ev_ms, k_wall_ms) if timed_steps == args.steps else time_region(step, timed_steps, torch)
     assert all(bool(torch.isfinite(y).all()) for y in ys)
-    ms_per_step = wall_ms / args.steps
+    ms_per_step = wall_ms / timed_steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    kern_us = ev_ms * 1e3 / args.steps          # one launch per step: HIP-event time per launch
+    kern_us = ev_ms * 1e3 / timed_steps         # one launch per step: HIP-event time per launch
     achieved = step_bytes / (kern_us * 1e-6) / 1e9
 
-    traffic = MEASURED_TRAFFIC_BYTES
+    traffic = measured_traffic_bytes()
 
     out = {
         "metric": "Q4_K/Q8_0/MXFP4 matmul: decode GB/s (% HBM peak), prefill TFLOP/s (% MFMA)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 5), "timed_steps": timed_steps,
+        "exact_steps_region": {"steps": args.steps, "ms_per_step_wall": round(k_wall_ms / args.steps, 5),
+                               "ms_per_step_events": round(k_ev_ms / args.steps, 5),
+                               "GBps_wall": round(step_bytes / (k_wall_ms / args.steps * 1e-3) / 1e9, 1)}, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "q4_k weights x f32 activations (fp16 operands, f32 accumulate)",
         "data": "synthetic: W ~ N(0,0.02) in Q4_K blocks (min/max-fit quantizer), x ~ N(0,1) f32, "
                 f"{args.copies} distinct layer copies cycled",
@@ -203,9 +262,35 @@ def main():
                    "bytes_per_step": step_bytes, "launches_per_step": 1, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "tship::gemv_kernel<12, 0, 1> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
+                     "kernel": "tship::gemv_kernel<12, 0> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
                      "bytes_per_launch": step_bytes},
     }
+
+    # ---- the prefill half of the metric: configs[4] Q4_K, M = 2048, N = 21504, K = 5376 -------------------------
+    # One call = the activation convert kernel + the MFMA GEMM; the HIP events bracket whole calls, so `achieved` prices
+    # both launches against the fp16 matrix peak (the GEMM kernel alone is in the rocprofv3 summary).
+    def prefill(t, m, n, k, iters=20):
+        w = QuantizedWeight(synth.random_weight(t, n, k, dev, seed=91), t, k, n)
+        x = torch.randn((m, k), device=dev, dtype=torch.float32)
+        y = torch.empty((m, n), device=dev, dtype=torch.float32)
+
+        def f(i):
+            HipBasicOps.AddmmQuantDevice(y, x, w.ptr, t, k, n, w.raw_bytes)
+        for i in range(3):
+            f(i)
+        ev, wall = time_region(f, iters, torch)
+        us = ev * 1e3 / iters
+        tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
+        return {"us_per_call_events": round(us, 1), "TFLOPs": round(tf, 1), "pct_mfma_fp16_peak": round(100 * tf / MFMA_FP16_PEAK_TFLOPS, 1)}
+
+    pm, pn, pk = 2048, 21504, 5376
+    pre = prefill(Q4_K, pm, pn, pk, 20)
+    out["roofline_prefill"] = {
+        "bound": "mfma", "achieved": pre["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(pre["TFLOPs"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+        "workload": "configs[4]: Q4_K prefill GEMM M=2048 N=21504 K=5376, fp16 operands, f32 accumulate",
+        "kernel": "tship::gemm_xw_kernel<tship::PQ4K, 256, 4> (+ tship::convert_x_kernel on the activations, inside the timed call)",
+        "avg_call_us": pre["us_per_call_events"], "flops_per_call": 2 * pm * pn * pk, "calls_timed": 20}
 
     # ---- secondary workloads (reported, not the headline) ---------------------------------------
     if not args.no_extra:
@@ -242,22 +327,8 @@ def main():
 
         # prefill GEMMs (configs[2] and configs[4]): TFLOP/s = 2*M*N*K / time of the whole call
         # (activation convert kernel + MFMA GEMM), fp16 operands -> priced against 2516.6 TFLOP/s
-        def prefill(t, m, n, k, iters=20):
-            w = QuantizedWeight(synth.random_weight(t, n, k, dev, seed=91), t, k, n)
-            x = torch.randn((m, k), device=dev, dtype=torch.float32)
-            y = torch.empty((m, n), device=dev, dtype=torch.float32)
-
-            def f(i):
-                HipBasicOps.AddmmQuantDevice(y, x, w.ptr, t, k, n, w.raw_bytes)
-            for i in range(3):
-                f(i)
-            ev, wall = time_region(f, iters, torch)
-            us = ev * 1e3 / iters
-            tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
-            return {"us_per_call_events": round(us, 1), "TFLOPs": round(tf, 1), "pct_mfma_fp16_peak": round(100 * tf / 2516.6, 1)}
-
         extra["cfg3_q4_k_gemm_512x14336x4096"] = prefill(Q4_K, 512, 14336, 4096)
-        extra["cfg5_q4_k_gemm_2048x21504x5376"] = prefill(Q4_K, 2048, 21504, 5376, 10)
+        extra["cfg5_q4_k_gemm_2048x21504x5376"] = pre
         extra["cfg5_q8_0_gemm_2048x21504x5376"] = prefill(Q8_0, 2048, 21504, 5376, 10)
         extra["cfg5_q4_k_gemm_2048x5376x21504"] = prefill(Q4_K, 2048, 5376, 21504, 10)
         extra["cfg5_q8_0_gemm_2048x5376x21504"] = prefill(Q8_0, 2048, 5376, 21504, 10)
@@ -301,7 +372,7 @@ def main():
                 res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
                             "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1),
                             "TFLOPs": round(fl / (us * 1e-6) / 1e12, 1),
-                            "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / 2516.6, 1)})
+                            "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / MFMA_FP16_PEAK_TFLOPS, 1)})
             return res
 
         extra["cfg4_mxfp4_moe_experts_T1"] = moe(1, n_it)
@@ -364,6 +435,10 @@ def main():
                     "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)}
 
         extra["cfg2_q4_k_fused_ffn_decode_4096x14336"] = fused_ffn()
+        # dequantizer and embedding gather (HBM-bound: blocks read + fp32 written)
+        extra["dequant_q4_k_14336x4096"] = aux_case("dequant", Q4_K, 14336, 4096, 50, 5)
+        extra["dequant_q8_0_9728x2560"] = aux_case("dequant", Q8_0, 9728, 2560, 50, 5)
+        extra["get_rows_q8_0_512_of_131072x4096"] = aux_case("get_rows", Q8_0, 512, 4096, 50, 5)
         out["extra"] = extra
 
     if not args.no_cpu:
