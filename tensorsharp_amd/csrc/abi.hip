@@ -488,19 +488,32 @@ bool run_ffn_swiglu_device(const TSHipTensorView2D& residual, const TSHipTensorV
     float* gu = reinterpret_cast<float*>(ws);
     float* act = reinterpret_cast<float*>(ws + gu_bytes);
     void* mm_ws = ws + gu_bytes + act_bytes;
-    const TSHipTensorView2D gu_view{gu, M, 2 * half, 2 * half, 1, (int64_t)((size_t)M * 2 * half * sizeof(float))};
-    if (!run_matmul_device_ws(gu_view, input, gate_up, gu_type, hidden, 2 * half, stream, mm_ws, mm_bytes, norm_w, eps, false)) return false;
-    if (M <= 3 && half <= gemv_max_k(dn_type) && row_size(dn_type, half) * (size_t)hidden < (size_t)kMaxOperandBytes) {
-        // decode: the down GEMV forms silu(gate) * up while it stages its activations and adds the residual in its store
-        if (!check_device_operands(gu_view, down, dn_type)) return false;
-        const size_t dn_bytes = row_size(dn_type, half) * (size_t)hidden;
+    auto streams = [](int type, int64_t rows, int64_t k) {
+        return has_gemv(type) && k <= gemv_max_k(type) && row_size(type, k) * (size_t)rows < (size_t)kMaxOperandBytes;
+    };
+    if (M <= 3 && streams(gu_type, 2 * (int64_t)half, hidden) && streams(dn_type, hidden, half)) {
+        // decode, two launches per row: the gate_up GEMV stages RMSNorm(x) * w, computes gate row j and up row j in one
+        // wavefront and stores silu(gate_j) * up_j; the down GEMV adds the residual in its store
+        if (!check_device_operands(input, gate_up, gu_type) || !check_device_operands(input, down, dn_type)) return false;
+        if ((reinterpret_cast<uintptr_t>(norm_w) & 15) != 0) {
+            set_last_error("The norm weight must be 16-byte aligned on the device.");
+            return false;
+        }
+        const size_t gu_w_bytes = row_size(gu_type, hidden) * (size_t)(2 * half), dn_w_bytes = row_size(dn_type, half) * (size_t)hidden;
+        for (int m = 0; m < M; ++m) {
+            GemvArgs a{};
+            a.w = gate_up, a.w_bytes = (int64_t)gu_w_bytes, a.x = static_cast<const float*>(input.data) + (int64_t)m * input.stride0;
+            a.y = gu + (size_t)m * half, a.N = 2 * half, a.K = hidden, a.act = 1, a.norm_w = norm_w, a.eps = eps, a.pair_rows = half;
+            if (!launch_gemv_group(gu_type, 1, &a, stream)) return false;
+        }
         for (int m = 0; m < M; ++m) {
             float* y = static_cast<float*>(residual.data) + (int64_t)m * residual.stride0;
-            if (!launch_gemv(dn_type, down, (int64_t)dn_bytes, gu + (size_t)m * 2 * half, y, hidden, half, stream, y, 2, nullptr, 0.f))
-                return false;
+            if (!launch_gemv(dn_type, down, (int64_t)dn_w_bytes, gu + (size_t)m * half, y, hidden, half, stream, y, 0, nullptr, 0.f)) return false;
         }
         return true;
     }
+    const TSHipTensorView2D gu_view{gu, M, 2 * half, 2 * half, 1, (int64_t)((size_t)M * 2 * half * sizeof(float))};
+    if (!run_matmul_device_ws(gu_view, input, gate_up, gu_type, hidden, 2 * half, stream, mm_ws, mm_bytes, norm_w, eps, false)) return false;
     if (!launch_silu_mul(gu, 2 * half, M, half, act, stream)) return false;
     const TSHipTensorView2D act_view{act, M, half, half, 1, (int64_t)((size_t)M * half * sizeof(float))};
     return run_matmul_device_ws(residual, act_view, down, dn_type, half, hidden, stream, mm_ws, mm_bytes, nullptr, 0.f, true);

@@ -19,7 +19,12 @@
 //     pairs -> fp16 with v_cvt_scalef32_pk_f16_fp4 feeding v_dot2_f32_f16; block scales (fp16 d, 6-bit K-quant
 //     scales / mins, int8 Q6_K scales, E8M0) are applied once per unit in fp32;
 //   * the per-lane sums of a row are reduced with four DPP adds inside 16 lanes (and a lane-swap add for 32-lane
-//     rows); the results of a group leave as one store instruction.
+//     rows); the results of a group leave as one store instruction;
+//   * the fused decode paths hang on the two ends of the same kernel.  Staging modes: x * norm_weight with the RMSNorm
+//     scale applied to the row sums at the store (a scalar commutes with the product, so no reduction precedes the
+//     staging), silu(gate) * up of a [gate | up] row, and the GPT-OSS clamped SwiGLU with per-expert bias.  Store modes:
+//     y = add + W x (residual), and the paired mode in which a wavefront computes gate row j and up row j of a stacked
+//     [gate; up] weight side by side and stores silu(gate_j) * up_j.
 //
 // Arithmetic restated from TensorSharp.Models/ManagedQuantizedOps.cs:156-200 (dot of a dequantised row with the
 // activation row); except for Q8_0 the activations of each unit are rounded to fp16 after a power-of-two scale of
@@ -61,6 +66,7 @@ struct GemvProblem {
     const int* expert_id;     // optional (MoE): the weight is w + expert_id[0] * expert_stride
     int64_t expert_stride;
     int n_experts;            // ids outside [0, n_experts) select no weight: the problem reads zeros
+    int pair_rows;            // F > 0: the weight holds F gate rows then F up rows and y[j] = silu(gate_j) * up_j, j < F
     int N;
     int K;
 };
@@ -809,10 +815,19 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const int lane = threadIdx.x & 63;
     constexpr int LPR = F::kLPR, RPG = 64 / LPR;     // lanes per row, rows per group
     const int sub = lane / LPR, l16 = lane % LPR;    // row of the group, lane inside the row
-    const int N = P.N, K = P.K;
+    const int K = P.K;
     const int upr = K / F::kUnitElems;          // units per row
     const int nsteps = (upr + LPR - 1) / LPR;   // steps per row group
-    const int ngroups = (N + RPG - 1) / RPG;
+    // Plain: a group is RPG consecutive rows.  Paired (gate | up stacks of pair_rows rows each): a group is RPG / 2
+    // consecutive gate rows in the lower half of the wavefront and the matching up rows in the upper half, so that gate j
+    // and up j finish in lanes 32 apart and meet at the store.
+    const int pair = P.pair_rows;                      // uniform
+    constexpr int HALF = RPG / 2;
+    const int gstep = pair ? HALF : RPG;               // output rows per group
+    const int N = pair ? pair : P.N;                   // output rows
+    const int ngroups = (N + gstep - 1) / gstep;
+    const int osub = pair ? sub % (HALF > 0 ? HALF : 1) : sub;          // the lane's output row inside the group
+    const int lane_row = pair ? osub + (sub / (HALF > 0 ? HALF : 1)) * pair : sub;   // its weight row relative to the group's first
     const uint32_t row_bytes = (uint32_t)F::row_bytes(K);
     const int wave_stride = nwg * kWaves;
     const int gw = __builtin_amdgcn_readfirstlane(wg * kWaves + (int)(threadIdx.x >> 6));
@@ -828,16 +843,16 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const uint32_t extent = bad_expert ? 0u : ((uint32_t)P.w_bytes + base_delta + 3u) & ~3u;
     const __amdgpu_buffer_rsrc_t rs =
         __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, (int)extent, 0x00020000);
-    const typename F::Lane L = F::lane_setup(sub, l16, row_bytes);
+    const typename F::Lane L = F::lane_setup(lane_row, l16, row_bytes);
     const uint32_t lds_lane = (uint32_t)l16 * F::kLdsDwords;
 
     // issue the loads of step (group, step); no waiting, no branches
     auto fetch = [&](int group, int step, Step<F>& st) {
         const bool group_ok = group < ngroups;                         // uniform
-        const int row0 = group_ok ? group * RPG : 0;
+        const int row0 = group_ok ? group * gstep : 0;
         const uint32_t start = base_delta + (uint32_t)row0 * row_bytes + (uint32_t)step * F::kSlotBytes;
         const uint32_t soff = start & ~3u;                             // scalar part of the address
-        const bool live = group_ok && (row0 + sub < N) && (l16 + step * LPR < upr);
+        const bool live = group_ok && (row0 + osub < N) && (l16 + step * LPR < upr);
         st.step = step;
         st.group = group;
         st.aux = F::load(rs, L, soff, start & 3u, step, live, st.w);
@@ -893,31 +908,23 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             }
         }
     };
-    // kActRmsNorm: the whole row is in the registers of the workgroup after ONE pass (the host guarantees it);
-    // sum of squares in double over the workgroup, then (x * scale) * w in place
+    // kActRmsNorm: RMSNorm(x) * w = (x * w) * scale with the scalar scale = 1 / sqrt(mean(x^2) + eps), and a scalar
+    // commutes with the matrix product.  So x * w is staged at once, each thread adds the squares of the values it
+    // holds, and the scale meets the row sums at the store: no reduction and no barrier stands between the loads of x
+    // and the staging.  (Sum of squares in double over fp32 squares, as ggml_rms_norm.)
     double* red = reinterpret_cast<double*>(lds + nsteps * LPR * F::kLdsDwords);      // [kWaves], after the x area
+    double ss = 0.0;
     auto apply_act = [&]() {
         if (act == kActRmsNorm) {
-            double ss = 0.0;
 #pragma unroll
             for (int c = 0; c < kStageChunk; ++c)
 #pragma unroll
-                for (int q = 0; q < F::kStageF4; ++q)
+                for (int q = 0; q < F::kStageF4; ++q) {
                     ss += (double)(xv[c][q].x * xv[c][q].x) + (double)(xv[c][q].y * xv[c][q].y) +
                           (double)(xv[c][q].z * xv[c][q].z) + (double)(xv[c][q].w * xv[c][q].w);
-            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-            if (lane == 0) red[threadIdx.x >> 6] = ss;
-            __syncthreads();
-            double tot = 0.0;
-#pragma unroll
-            for (int i = 0; i < kWaves; ++i) tot += red[i];
-            const float scale = 1.0f / sqrtf((float)(tot / (double)K) + P.eps);
-#pragma unroll
-            for (int c = 0; c < kStageChunk; ++c)
-#pragma unroll
-                for (int q = 0; q < F::kStageF4; ++q)
-                    xv[c][q] = float4{(xv[c][q].x * scale) * x2[c][q].x, (xv[c][q].y * scale) * x2[c][q].y,
-                                      (xv[c][q].z * scale) * x2[c][q].z, (xv[c][q].w * scale) * x2[c][q].w};
+                    xv[c][q] = float4{xv[c][q].x * x2[c][q].x, xv[c][q].y * x2[c][q].y, xv[c][q].z * x2[c][q].z,
+                                      xv[c][q].w * x2[c][q].w};
+                }
         } else if (act == kActSiluMul) {
             // hardware exp2 / reciprocal: relative error below 1e-5, far under the fp16 rounding the staged value gets
             // next (every workgroup evaluates the whole row, so the exact expf and division cost microseconds)
@@ -958,10 +965,11 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // loop the next step is requested before the current one is consumed.
     Step<F> cur, nxt;
     int fgroup = gw, fstep = 0;                // next step to fetch
-    // deep: two steps requested before x is staged and two in flight afterwards.  Only the activation modes use it
-    // (their staging takes longer, and they are the short dependent launches of a decode step: fused FFN 33.9 -> 32.2 us,
-    // whole layer 66.5 -> 64.0 us in an A/B on one box; plain launches lose, 4096 x 14336 12.7 -> 14.2 us).
-    const bool strict = mode == 1, deep = ACT != kActPlain && !strict;
+    // deep: two steps requested before x is staged and two in flight afterwards.  Only the modes that evaluate a
+    // function of two operands while staging use it (their staging takes longer, and they are the short dependent
+    // launches of a decode step: fused FFN 33.9 -> 32.2 us in an A/B on one box); plain launches lose (4096 x 14336
+    // 12.7 -> 14.2 us) and so does the RMSNorm mode, whose staging is as short as the plain one (28672 x 4096 17.2 vs 16.0 us).
+    const bool strict = mode == 1, deep = (ACT == kActSiluMul || ACT == kActSwigluOai) && !strict;
     fetch(fgroup, fstep, cur);
     advance(fgroup, fstep);
     if (deep) {
@@ -976,7 +984,18 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     }
     // lanes past the end of a row read their activations from the zero-filled tail of the last step
     for (int i = upr * F::kLdsDwords + (int)threadIdx.x; i < nsteps * LPR * F::kLdsDwords; i += kThreads) lds[i] = 0u;
+    if (act == kActRmsNorm) {
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if (lane == 0) red[threadIdx.x >> 6] = ss;
+    }
     __syncthreads();
+    float out_scale = 1.0f;      // factor on every row sum
+    if (act == kActRmsNorm) {
+        double tot = 0.0;
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) tot += red[i];
+        out_scale = 1.0f / sqrtf((float)(tot / (double)K) + P.eps);
+    }
 
     float acc = 0.f;
     auto consume = [&](const Step<F>& st) {
@@ -984,9 +1003,16 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         const uint32_t* xu = lds + lds_lane + (uint32_t)st.step * (uint32_t)(LPR * F::kLdsDwords);
         acc += F::dot(st.w, L, st.aux, xu);
         if (st.step == nsteps - 1) {   // uniform: the 4 rows of the group are complete
-            const float t = row_sum<LPR>(acc);
-            const int row = st.group * RPG + sub;
-            if (l16 == 0 && st.group < ngroups && row < N) P.y[row] = P.add ? P.add[row] + t : t;
+            float t = act == kActRmsNorm ? row_sum<LPR>(acc) * out_scale : row_sum<LPR>(acc);
+            const int row = st.group * gstep + osub;
+            bool writer = l16 == 0 && st.group < ngroups && row < N;
+            if (pair) {
+                // ggml_silu then ggml_mul (ggml-cpu/vec.h:958-960) on the fp32 sums; the up value sits 32 lanes above
+                const float up = __shfl_xor(t, 32);
+                t = (t / (1.0f + expf(-t))) * up;
+                writer = writer && lane < 32;
+            }
+            if (writer) P.y[row] = P.add ? P.add[row] + t : t;
             acc = 0.f;
         }
     };
@@ -1082,7 +1108,8 @@ int gemv_max_k(int type)
 int gemv_max_group() { return kMaxGroup; }
 
 // one staging pass covers 8 float4 per thread
-int gemv_rms_max_k() { return kThreads * 8 * 4; }
+// the RMSNorm mode stages rows of any length the kernel can hold (its scale is applied at the store)
+int gemv_rms_max_k() { return 1 << 30; }
 
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream)
 {
@@ -1126,7 +1153,12 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     for (int i = 0; i < count; ++i) {
         // workgroups in proportion to the bytes each problem streams
         int share = std::max(1, (int)((double)budget * (double)args[i].w_bytes / total_bytes + 0.5));
-        share = std::min(share, ((args[i].N + rpg - 1) / rpg + kWaves - 1) / kWaves);
+        const int out_rows = args[i].pair_rows ? args[i].pair_rows : args[i].N, out_rpg = args[i].pair_rows ? rpg / 2 : rpg;
+        if (args[i].pair_rows && (args[i].N != 2 * args[i].pair_rows || rpg < 2)) {
+            set_last_error("gemv: the paired gate | up mode needs N = 2 * pair_rows.");
+            return false;
+        }
+        share = std::min(share, ((out_rows + out_rpg - 1) / out_rpg + kWaves - 1) / kWaves);
         g.p[i].w = static_cast<const uint8_t*>(args[i].w);
         g.p[i].w_bytes = args[i].w_bytes;
         g.p[i].x = args[i].x;
@@ -1145,6 +1177,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         g.p[i].expert_id = args[i].expert_id;
         g.p[i].expert_stride = args[i].expert_stride;
         g.p[i].n_experts = args[i].n_experts;
+        g.p[i].pair_rows = args[i].pair_rows;
         if (args[i].expert_id && args[i].n_experts <= 0) {
             set_last_error("gemv: an expert indirection needs the number of experts.");
             return false;
@@ -1183,7 +1216,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream,
                  const float* add, int act, const float* norm_w, float eps)
 {
-    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, 0, add, act, norm_w, eps};
+    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, 0, 0, add, act, norm_w, eps};
     return launch_gemv_group(type, 1, &a, stream);
 }
 
