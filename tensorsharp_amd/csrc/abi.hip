@@ -1414,21 +1414,21 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
         float* dn = reinterpret_cast<float*>(ws + o_dn);
         const float* hid = static_cast<const float*>(hidden.data);
         if (small) {
-            // decode: one GEMV per (token, slot), expert chosen on the device through ids
+            // decode: one GEMV per (token, slot), expert chosen on the device through ids.  The gate_up launch computes
+            // gate row j and up row j side by side and stores bias + SwiGLU-OAI of the pair: gu holds [A][F] activations.
             GemvArgs args[16];
             for (int a = 0; a < A; ++a) {
-                args[a] = GemvArgs{gate_up_w, gu_bytes, hid + (int64_t)(a / k) * hidden.stride0, gu + (int64_t)a * 2 * F,
+                args[a] = GemvArgs{gate_up_w, gu_bytes, hid + (int64_t)(a / k) * hidden.stride0, gu + (int64_t)a * F,
                                    (int)(2 * F), (int)H, ids + a, gu_bytes, E};
-            }
-            if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
-            // the down GEMVs form bias + SwiGLU-OAI from the gate|up rows while they stage their activations
-            for (int a = 0; a < A; ++a) {
-                args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * 2 * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes, E};
-                args[a].act = 3;
+                args[a].pair_rows = (int)F;
+                args[a].pair_kind = 1;
                 args[a].norm_w = gate_up_bias;
                 args[a].eps = alpha;
                 args[a].limit = limit;
             }
+            if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
+            for (int a = 0; a < A; ++a)
+                args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes, E};
             if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
             if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, E, (int)H, T == 1, static_cast<float*>(result.data),
                                     result.stride0, stream))

@@ -66,7 +66,9 @@ struct GemvProblem {
     const int* expert_id;     // optional (MoE): the weight is w + expert_id[0] * expert_stride
     int64_t expert_stride;
     int n_experts;            // ids outside [0, n_experts) select no weight: the problem reads zeros
-    int pair_rows;            // F > 0: the weight holds F gate rows then F up rows and y[j] = silu(gate_j) * up_j, j < F
+    int pair_rows;            // F > 0: the weight holds F gate rows then F up rows and y[j] = glu(gate_j, up_j), j < F
+    int pair_kind;            // glu of the paired mode: 0 silu(g) * u; 1 GPT-OSS (norm_w: optional [E][2F] bias indexed by
+                              // expert_id, eps: alpha, limit: clamp), with plain activation staging only
     int N;
     int K;
 };
@@ -1007,9 +1009,18 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             const int row = st.group * gstep + osub;
             bool writer = l16 == 0 && st.group < ngroups && row < N;
             if (pair) {
-                // ggml_silu then ggml_mul (ggml-cpu/vec.h:958-960) on the fp32 sums; the up value sits 32 lanes above
-                const float up = __shfl_xor(t, 32);
-                t = (t / (1.0f + expf(-t))) * up;
+                const float up = __shfl_xor(t, 32);       // the up value sits 32 lanes above its gate value
+                if (P.pair_kind == 0) {
+                    // ggml_silu then ggml_mul (ggml-cpu/vec.h:958-960) on the fp32 sums
+                    t = (t / (1.0f + expf(-t))) * up;
+                } else {
+                    // GptOssModel.cs:901-934: x = min(g + b_g, limit), y = clamp(u + b_u), x * sigmoid(alpha x) * (y + 1)
+                    const bool biased = P.norm_w != nullptr && !bad_expert && writer;
+                    const float* pb = P.norm_w + (int64_t)(P.expert_id ? eid : 0) * 2 * pair;
+                    const float x = fminf(t + (biased ? pb[row] : 0.f), P.limit);
+                    const float y = fminf(fmaxf(up + (biased ? pb[pair + row] : 0.f), -P.limit), P.limit);
+                    t = (x / (1.0f + expf(P.eps * (-x)))) * (y + 1.0f);
+                }
                 writer = writer && lane < 32;
             }
             if (writer) P.y[row] = P.add ? P.add[row] + t : t;
@@ -1138,12 +1149,34 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     }
     int per_cu = (int)std::min<size_t>(kWgPerCu, (160 * 1024) / (lds + 256));
     if (per_cu < 1) per_cu = 1;
+    const int lpr = lanes_per_row(type), rpg = 64 / lpr;
+    // row groups per wavefront of the busiest problem when every CU holds `wgs` workgroups
+    auto rounds = [&](int wgs) {
+        int worst = 0;
+        for (int i = 0; i < count; ++i) {
+            const int out_rows = args[i].pair_rows ? args[i].pair_rows : args[i].N, out_rpg = args[i].pair_rows ? rpg / 2 : rpg;
+            const int groups = (out_rows + std::max(out_rpg, 1) - 1) / std::max(out_rpg, 1);
+            const int share = std::max(1, (int)((double)(di.num_cus * wgs) * (double)args[i].w_bytes / total_bytes + 0.5));
+            worst = std::max(worst, (groups + share * kWaves - 1) / (share * kWaves));
+        }
+        return worst;
+    };
+    // Two workgroups per CU stream best (four: the 123 MB grouped launch 28 instead of 24 us, since twice as many
+    // workgroups stage x).  The exception is a launch whose busiest problem has between one and two row groups per
+    // wavefront AND long rows: half of the wavefronts then work twice as long as the rest, and four workgroups per CU
+    // give every row group a wavefront of its own.  Measured: the four expert matrices of a GPT-OSS token (1440 groups
+    // of 6 steps each) 13.8 -> 12.7 us; a 14336 x 4096 Q4_K matrix (7168 groups of 2 steps) loses, 9.7 -> 12.0 us, so
+    // the rule asks for at least 8 steps per wavefront.
+    int max_steps = 0;
+    for (int i = 0; i < count; ++i) max_steps = std::max(max_steps, (args[i].K / unit_elems(type) + lpr - 1) / lpr);
+    const int dense_cu = (int)std::min<size_t>(2 * kWgPerCu, (160 * 1024) / (lds + 256));
+    if (per_cu == kWgPerCu && dense_cu == 2 * kWgPerCu && rounds(per_cu) == 2 && rounds(dense_cu) == 1 && 2 * max_steps >= 8)
+        per_cu = dense_cu;
     const int budget = di.num_cus * per_cu;
     // (Cutting the K range of a row group over several wavefronts when a matrix has few rows was measured slower on
     // every shape: 4096 x 14336 Q4_K 13.7 vs 10.9 us, MXFP4 5760 x 2880 7.8 vs 6.7 us.  Requesting more up front - two extra
     // steps before x is staged, or a ring of four steps per wavefront - was slower too, the 123 MB grouped launch
     // included: 24.5 vs 24.2 us.)
-    const int lpr = lanes_per_row(type), rpg = 64 / lpr;
 
     GemvGroup g;
     std::memset(&g, 0, sizeof(g));
@@ -1178,6 +1211,11 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         g.p[i].expert_stride = args[i].expert_stride;
         g.p[i].n_experts = args[i].n_experts;
         g.p[i].pair_rows = args[i].pair_rows;
+        g.p[i].pair_kind = args[i].pair_kind;
+        if (args[i].pair_kind != 0 && (args[i].pair_rows == 0 || args[i].act != kActPlain)) {
+            set_last_error("gemv: the GPT-OSS paired store needs pair_rows and plain activation staging.");
+            return false;
+        }
         if (args[i].expert_id && args[i].n_experts <= 0) {
             set_last_error("gemv: an expert indirection needs the number of experts.");
             return false;
@@ -1216,7 +1254,8 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K, hipStream_t stream,
                  const float* add, int act, const float* norm_w, float eps)
 {
-    GemvArgs a{w, w_bytes, x, y, N, K, nullptr, 0, 0, 0, add, act, norm_w, eps};
+    GemvArgs a{};
+    a.w = w, a.w_bytes = w_bytes, a.x = x, a.y = y, a.N = N, a.K = K, a.add = add, a.act = act, a.norm_w = norm_w, a.eps = eps;
     return launch_gemv_group(type, 1, &a, stream);
 }
 

@@ -120,7 +120,9 @@ struct GemvArgs {
     const int* expert_id = nullptr;   // optional device pointer (MoE): weight = w + expert_id[0] * expert_stride
     int64_t expert_stride = 0;
     int n_experts = 0;                // with expert_id: ids outside [0, n_experts) make the problem read zeros
-    int pair_rows = 0;                // F > 0: W is F gate rows then F up rows (N = 2F) and y[j] = silu(gate_j) * up_j, j < F
+    int pair_rows = 0;                // F > 0: W is F gate rows then F up rows (N = 2F) and y[j] = glu(gate_j, up_j), j < F
+    int pair_kind = 0;                // 0: glu = silu(g) * u; 1: GPT-OSS SwiGLU at the store (act must be 0; norm_w the optional
+                                      // [E][2F] bias indexed by expert_id, eps = alpha, limit = clamp)
     const float* add = nullptr;       // optional: y = add + W x (add may be y)
     int act = 0;                      // activation mode, see launch_gemv; 3 = GPT-OSS SwiGLU (x is a gate|up row of 2K,
                                       // norm_w the optional [E][2K] bias indexed by expert_id, eps = alpha, limit = clamp)
