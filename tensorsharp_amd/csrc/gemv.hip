@@ -50,8 +50,6 @@ constexpr int kMaxGroup = 8;
 constexpr int kActPlain = 0;      // x[k]
 constexpr int kActRmsNorm = 1;    // (x[k] / sqrt(mean(x^2) + eps)) * norm_w[k]        (ggml_rms_norm, ggml_mul)
 constexpr int kActSiluMul = 2;    // silu(x[k]) * x[K + k]: x is a [2K] gate|up row    (ggml_silu, ggml_mul)
-constexpr int kActSwigluOai = 3;  // GPT-OSS: g = x[k] + b[k], u = x[K + k] + b[K + k] (b = norm_w + expert * 2K, optional),
-                                  // min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1); alpha = eps
 
 struct GemvProblem {
     const uint8_t* w;
@@ -871,20 +869,14 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const int items = F::stage_items(K);
     const __amdgpu_buffer_rsrc_t xrs =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(P.x), 0, K * 4, 0x00020000);
-    // work items per thread per pass (the GPT-OSS mode keeps four operands per item, so it takes smaller passes)
-    constexpr int kStageChunk = (ACT == kActSwigluOai ? 2 : 8) / F::kStageF4;
+    // work items per thread per pass
+    constexpr int kStageChunk = 8 / F::kStageF4;
     float4 xv[kStageChunk][F::kStageF4];
     // second operand of the activation modes: the norm weight (same offsets) or the "up" half (offsets + 4 K)
     constexpr int act = ACT;
     const __amdgpu_buffer_rsrc_t x2rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(act == kActRmsNorm ? P.norm_w : P.x + K), 0, K * 4, 0x00020000);
     float4 x2[kStageChunk][F::kStageF4];
-    // GPT-OSS mode: per-expert bias of the gate and of the up half
-    const bool has_bias = act == kActSwigluOai && P.norm_w != nullptr && !bad_expert;
-    const float* bias = has_bias ? P.norm_w + (P.expert_id ? (int64_t)eid * 2 * K : 0) : P.x;
-    const __amdgpu_buffer_rsrc_t bgrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bias), 0, K * 4, 0x00020000);
-    const __amdgpu_buffer_rsrc_t burs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bias + K), 0, K * 4, 0x00020000);
-    float4 bg[kStageChunk][F::kStageF4], bu[kStageChunk][F::kStageF4];
     auto stage_issue = [&](int base) {
 #pragma unroll
         for (int c = 0; c < kStageChunk; ++c) {
@@ -899,13 +891,6 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
                 if (act != kActPlain) {
                     const uint4_t u = __builtin_amdgcn_raw_buffer_load_b128(x2rs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
                     x2[c][q] = float4{__uint_as_float(u.x), __uint_as_float(u.y), __uint_as_float(u.z), __uint_as_float(u.w)};
-                }
-                if (act == kActSwigluOai) {
-                    const int o = (int)(it < items && has_bias ? off[q] : kDeadOffset);
-                    const uint4_t a = __builtin_amdgcn_raw_buffer_load_b128(bgrs, o, 0, 0);
-                    const uint4_t b = __builtin_amdgcn_raw_buffer_load_b128(burs, o, 0, 0);
-                    bg[c][q] = float4{__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z), __uint_as_float(a.w)};
-                    bu[c][q] = float4{__uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w)};
                 }
             }
         }
@@ -937,19 +922,6 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
                 for (int q = 0; q < F::kStageF4; ++q)
                     xv[c][q] = float4{silu(xv[c][q].x) * x2[c][q].x, silu(xv[c][q].y) * x2[c][q].y,
                                       silu(xv[c][q].z) * x2[c][q].z, silu(xv[c][q].w) * x2[c][q].w};
-        } else if (act == kActSwigluOai) {
-            const float alpha = P.eps, limit = P.limit;
-            auto glu = [&](float g, float u, float b0, float b1) {      // GptOssModel.cs:901-934
-                const float x = fminf(g + b0, limit);
-                const float y = fminf(fmaxf(u + b1, -limit), limit);
-                return (x * __builtin_amdgcn_rcpf(1.0f + __expf(alpha * (-x)))) * (y + 1.0f);
-            };
-#pragma unroll
-            for (int c = 0; c < kStageChunk; ++c)
-#pragma unroll
-                for (int q = 0; q < F::kStageF4; ++q)
-                    xv[c][q] = float4{glu(xv[c][q].x, x2[c][q].x, bg[c][q].x, bu[c][q].x), glu(xv[c][q].y, x2[c][q].y, bg[c][q].y, bu[c][q].y),
-                                      glu(xv[c][q].z, x2[c][q].z, bg[c][q].z, bu[c][q].z), glu(xv[c][q].w, x2[c][q].w, bg[c][q].w, bu[c][q].w)};
         }
     };
     auto stage_commit = [&](int base) {
@@ -967,11 +939,11 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // loop the next step is requested before the current one is consumed.
     Step<F> cur, nxt;
     int fgroup = gw, fstep = 0;                // next step to fetch
-    // deep: two steps requested before x is staged and two in flight afterwards.  Only the modes that evaluate a
-    // function of two operands while staging use it (their staging takes longer, and they are the short dependent
+    // deep: two steps requested before x is staged and two in flight afterwards.  Only the mode that evaluates a
+    // function of two operands while staging uses it (their staging takes longer, and they are the short dependent
     // launches of a decode step: fused FFN 33.9 -> 32.2 us in an A/B on one box); plain launches lose (4096 x 14336
     // 12.7 -> 14.2 us) and so does the RMSNorm mode, whose staging is as short as the plain one (28672 x 4096 17.2 vs 16.0 us).
-    const bool strict = mode == 1, deep = (ACT == kActSiluMul || ACT == kActSwigluOai) && !strict;
+    const bool strict = mode == 1, deep = ACT == kActSiluMul && !strict;
     fetch(fgroup, fstep, cur);
     advance(fgroup, fstep);
     if (deep) {
@@ -1230,15 +1202,14 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
             set_last_error("gemv: the problems of one launch must share the activation mode.");
             return false;
         }
-    if (act < kActPlain || act > kActSwigluOai) {
+    if (act < kActPlain || act > kActSiluMul) {
         set_last_error("gemv: unknown activation mode.");
         return false;
     }
 #define TSHIP_GEMV_DISPATCH(T)                                                           \
     (act == kActPlain     ? launch_type<T, kActPlain>(g, begin, lds, stream)             \
      : act == kActRmsNorm ? launch_type<T, kActRmsNorm>(g, begin, lds, stream)           \
-     : act == kActSiluMul ? launch_type<T, kActSiluMul>(g, begin, lds, stream)           \
-                          : launch_type<T, kActSwigluOai>(g, begin, lds, stream))
+                          : launch_type<T, kActSiluMul>(g, begin, lds, stream))
     switch (type) {
     case kTypeQ4_K: return TSHIP_GEMV_DISPATCH(kTypeQ4_K);
     case kTypeMXFP4: return TSHIP_GEMV_DISPATCH(kTypeMXFP4);

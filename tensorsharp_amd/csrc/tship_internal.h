@@ -101,8 +101,8 @@ bool launch_get_rows(int type, const void* src, int64_t row_bytes, int64_t ne1, 
                      float* dst, int64_t ldd, hipStream_t stream);
 
 // y[N] = W[N x K] * x[K] (+ add[N] when given; add may be y); W raw GGUF blocks, row-major; w_bytes = N * row_size.
-// act: 0 plain x; 1 RMSNorm(x, eps) * norm_w formed while x is staged (K <= gemv_rms_max_k()); 2 x is a [2K] row
-// gate|up and the staged activation is silu(gate) * up.
+// act: 0 plain x; 1 RMSNorm(x, eps) * norm_w (x * norm_w is staged, the scale applied to the row sums); 2 x is a [2K]
+// row gate|up and the staged activation is silu(gate) * up.
 bool launch_gemv(int type, const void* w, int64_t w_bytes, const float* x, float* y, int N, int K,
                  hipStream_t stream, const float* add = nullptr, int act = 0, const float* norm_w = nullptr, float eps = 0.f);
 int gemv_rms_max_k();
@@ -124,8 +124,7 @@ struct GemvArgs {
     int pair_kind = 0;                // 0: glu = silu(g) * u; 1: GPT-OSS SwiGLU at the store (act must be 0; norm_w the optional
                                       // [E][2F] bias indexed by expert_id, eps = alpha, limit = clamp)
     const float* add = nullptr;       // optional: y = add + W x (add may be y)
-    int act = 0;                      // activation mode, see launch_gemv; 3 = GPT-OSS SwiGLU (x is a gate|up row of 2K,
-                                      // norm_w the optional [E][2K] bias indexed by expert_id, eps = alpha, limit = clamp)
+    int act = 0;                      // activation mode, see launch_gemv
     const float* norm_w = nullptr;
     float eps = 0.f;
     float limit = 0.f;
