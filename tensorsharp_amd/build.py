@@ -14,6 +14,9 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
+# per-source additions.  gemv.hip: the first 11 dwords of kernel arguments (the workgroup -> problem table of
+# gemv_kernel) arrive preloaded in SGPRs; the code object keeps a loading prologue for firmware without the feature.
+EXTRA_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=11"]}
 
 
 def build(verbose=False, jobs=8):
@@ -27,7 +30,7 @@ def build(verbose=False, jobs=8):
     for src in SOURCES:
         obj = os.path.join(objdir, src + ".o")
         objs.append(obj)
-        cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

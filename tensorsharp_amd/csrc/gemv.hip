@@ -1025,23 +1025,35 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     }
 }
 
+// The workgroup -> problem table and the flags travel as the kernel's first scalar arguments: built with
+// -amdgpu-kernarg-preload-count the hardware delivers them in SGPRs at wave launch, so a workgroup knows its problem
+// without a memory round trip and the one scalar load left (the problem's fields) is issued at once.
+struct GemvProblems {
+    GemvProblem p[kMaxGroup];
+};
 template <int TYPE, int ACT>
-__global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvGroup G)
+__global__ void __launch_bounds__(kThreads) gemv_kernel(int b0, int b1, int b2, int b3, int b4, int b5, int b6, int b7, int b8, int count,
+                                                        int strict, const GemvProblems G)
 {
+    static_assert(kMaxGroup == 8, "one scalar argument per table entry");
     extern __shared__ uint32_t lds[];
-    int i = 0;
-#pragma unroll
-    for (int j = 1; j < kMaxGroup; ++j)
-        if (j < G.count && (int)blockIdx.x >= G.wg_begin[j]) i = j;
-    const int wg = (int)blockIdx.x - G.wg_begin[i];
-    const int nwg = G.wg_begin[i + 1] - G.wg_begin[i];
-    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT>(G.p[i], wg, nwg, G.strict, lds);
-    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT>(G.p[i], wg, nwg, G.strict, lds);
-    else gemv_body<FmtQ80, ACT>(G.p[i], wg, nwg, G.strict, lds);
+    const int bx = (int)blockIdx.x;
+    int i = 0, lo = b0, hi = b1;
+    if (1 < count && bx >= b1) { i = 1; lo = b1; hi = b2; }
+    if (2 < count && bx >= b2) { i = 2; lo = b2; hi = b3; }
+    if (3 < count && bx >= b3) { i = 3; lo = b3; hi = b4; }
+    if (4 < count && bx >= b4) { i = 4; lo = b4; hi = b5; }
+    if (5 < count && bx >= b5) { i = 5; lo = b5; hi = b6; }
+    if (6 < count && bx >= b6) { i = 6; lo = b6; hi = b7; }
+    if (7 < count && bx >= b7) { i = 7; lo = b7; hi = b8; }
+    const int wg = bx - lo, nwg = hi - lo;
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT>(G.p[i], wg, nwg, strict, lds);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT>(G.p[i], wg, nwg, strict, lds);
+    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT>(G.p[i], wg, nwg, strict, lds);
+    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT>(G.p[i], wg, nwg, strict, lds);
+    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT>(G.p[i], wg, nwg, strict, lds);
+    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT>(G.p[i], wg, nwg, strict, lds);
+    else gemv_body<FmtQ80, ACT>(G.p[i], wg, nwg, strict, lds);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
@@ -1068,7 +1080,10 @@ bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
     auto kern = gemv_kernel<TYPE, ACT>;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g);
+    GemvProblems gp;
+    std::memcpy(gp.p, g.p, sizeof(gp.p));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g.wg_begin[0], g.wg_begin[1], g.wg_begin[2], g.wg_begin[3],
+                       g.wg_begin[4], g.wg_begin[5], g.wg_begin[6], g.wg_begin[7], g.wg_begin[8], g.count, g.strict, gp);
     return hip_ok(hipGetLastError(), "gemv launch");
 }
 
