@@ -283,3 +283,48 @@ def test_unwritten_cache_rows_may_hold_nan(hip, oracle, prefix):
         assert np.all(np.isfinite(got)), pos
         assert rel(got, h) <= 3e-3, (pos, rel(got, h))
     assert np.all(np.isnan(kd.cpu().numpy()[:, prefix + 2:]))              # rows past the written ones untouched
+
+
+def test_layer_decode_replayed_from_a_hip_graph(hip, oracle):
+    # After one call on a stream the layer call allocates nothing (its scratch is the stream's grow-only buffer) and
+    # records no memset, so its six launches can be captured on that stream and replayed.  Every replay is checked
+    # against the eager result, with eager work and synchronisations of the program's own between the replays.
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(131)
+    hidden, heads, kv_heads, head_dim, inter, max_seq = 512, 8, 2, 64, 1024, 256
+    layer, dims = make_layer(oracle, rng, hidden, heads, kv_heads, head_dim, inter, (Q4_K, Q4_K, Q4_K, Q4_K))
+    dev = to_device_layer(layer, torch, QuantizedWeight, dims)
+    pos = 140
+    k0 = torch.randn((kv_heads, max_seq, head_dim), device="cuda")
+    v0 = torch.randn((kv_heads, max_seq, head_dim), device="cuda")
+    h0 = torch.randn(hidden, device="cuda")
+    hd, kd, vd = h0.clone(), k0.clone(), v0.clone()
+
+    def call():
+        hip.TransformerLayerDecode(hd, dev["attn_norm"], dev["qkv"], dev["q_norm"], dev["k_norm"], dev["o"], dev["ffn_norm"],
+                                   dev["gate_up"], dev["down"], kd, vd, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, 2)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                                   # eager: sizes this stream's scratch, gives the expected result
+    side.synchronize()
+    want_h, want_k, want_v = hd.clone(), kd[:, pos].clone(), vd[:, pos].clone()
+    graph = torch.cuda.CUDAGraph()
+    hd.copy_(h0)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        call()
+    for rep in range(4):
+        hd.copy_(h0)
+        kd.copy_(k0)
+        vd.copy_(v0)
+        # unrelated eager work of the same library on the default stream between replays
+        y = torch.empty((1, hidden), device="cuda")
+        hip.AddmmQuantDevice(y, h0.view(1, -1) * float(rep + 1), dev["o"].ptr, Q4_K, hidden, hidden, dev["o"].raw_bytes)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(hd, want_h), rep
+        assert torch.equal(kd[:, pos], want_k) and torch.equal(vd[:, pos], want_v), rep
