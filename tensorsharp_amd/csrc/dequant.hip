@@ -250,6 +250,155 @@ __global__ void __launch_bounds__(256) dequant_kernel(const uint8_t* __restrict_
     reinterpret_cast<float4*>(dst)[t] = dequant4<TYPE>(src, t * 4);
 }
 
+constexpr int kWideItems = 1;      // items of 8 weights per thread in the wide dequantization kernels (2 and 4 measured slower)
+
+// A little-endian dword / word at any byte address (global memory takes unaligned addresses; where the compiler may
+// not assume that, it falls back to byte loads by itself).
+__device__ __forceinline__ uint32_t load_u32(const uint8_t* p)
+{
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
+__device__ __forceinline__ uint32_t load_u16(const uint8_t* p)
+{
+    uint16_t v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+
+// Q8_0: one thread takes a quarter of a block: the scale and eight quants (two dwords) -> 32 contiguous output bytes.
+// y = q * d (ManagedQuantizedOps.cs:411-427).
+__global__ void __launch_bounds__(256) dequant_q8_0_wide_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst, int64_t n8)
+{
+    // kWideItems quarter blocks per thread, 256 apart, all loads issued before the first store
+    const int64_t t0 = (int64_t)blockIdx.x * (256 * kWideItems) + threadIdx.x;
+    uint32_t dh[kWideItems], q0[kWideItems], q1[kWideItems];
+#pragma unroll
+    for (int u = 0; u < kWideItems; ++u) {
+        const int64_t t = t0 + 256 * u;
+        if (t < n8) {
+            const uint8_t* blk = src + (t >> 2) * 34;
+            const int part = (int)(t & 3);
+            dh[u] = load_u16(blk);
+            q0[u] = load_u32(blk + 2 + 8 * part);
+            q1[u] = load_u32(blk + 6 + 8 * part);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kWideItems; ++u) {
+        const int64_t t = t0 + 256 * u;
+        if (t < n8) {
+            const float d = half_bits_to_float(dh[u]);
+            float4 a, b;
+            a.x = (float)(int8_t)(q0[u] & 0xffu) * d;
+            a.y = (float)(int8_t)((q0[u] >> 8) & 0xffu) * d;
+            a.z = (float)(int8_t)((q0[u] >> 16) & 0xffu) * d;
+            a.w = (float)(int8_t)(q0[u] >> 24) * d;
+            b.x = (float)(int8_t)(q1[u] & 0xffu) * d;
+            b.y = (float)(int8_t)((q1[u] >> 8) & 0xffu) * d;
+            b.z = (float)(int8_t)((q1[u] >> 16) & 0xffu) * d;
+            b.w = (float)(int8_t)(q1[u] >> 24) * d;
+            float4* o = reinterpret_cast<float4*>(dst + t * 8);
+            o[0] = a;
+            o[1] = b;
+        }
+    }
+}
+
+// MXFP4: one thread takes the scale byte and one dword of a block's quants: four weights in the low nibbles
+// (elements 4 part ..) and four in the high nibbles (elements 16 + 4 part ..).  value = table[nibble] * 2^(e - 128)
+// (ManagedQuantizedOps.cs:579-598).
+__global__ void __launch_bounds__(256) dequant_mxfp4_wide_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst, int64_t n8)
+{
+    const int64_t t0 = (int64_t)blockIdx.x * (256 * kWideItems) + threadIdx.x;
+    uint32_t e[kWideItems], q[kWideItems];
+#pragma unroll
+    for (int u = 0; u < kWideItems; ++u) {
+        const int64_t t = t0 + 256 * u;
+        if (t < n8) {
+            const uint8_t* blk = src + (t >> 2) * 17;
+            e[u] = blk[0];
+            q[u] = load_u32(blk + 1 + 4 * (int)(t & 3));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kWideItems; ++u) {
+        const int64_t t = t0 + 256 * u;
+        if (t < n8) {
+            const float d = e8m0_half_scale(e[u]);
+            const uint32_t v = q[u];
+            float4 lo, hi;
+            lo.x = d * mxfp4_value(v & 0x0fu);
+            lo.y = d * mxfp4_value((v >> 8) & 0x0fu);
+            lo.z = d * mxfp4_value((v >> 16) & 0x0fu);
+            lo.w = d * mxfp4_value((v >> 24) & 0x0fu);
+            hi.x = d * mxfp4_value((v >> 4) & 0x0fu);
+            hi.y = d * mxfp4_value((v >> 12) & 0x0fu);
+            hi.z = d * mxfp4_value((v >> 20) & 0x0fu);
+            hi.w = d * mxfp4_value(v >> 28);
+            float* o = dst + (t >> 2) * 32 + 4 * (int)(t & 3);
+            *reinterpret_cast<float4*>(o) = lo;
+            *reinterpret_cast<float4*>(o + 16) = hi;
+        }
+    }
+}
+
+// Q4_K with 16-byte aligned blocks: one thread takes one dword of a block's quants (four bytes = four weights of an even
+// sub-block in the low nibbles and four of the odd sub-block after it in the high nibbles) and the block's 16-byte
+// header: two loads, two 16-byte stores.  Eight neighbouring threads write 128 contiguous bytes of each sub-block.
+// Same arithmetic as dequant4_q4_K (ManagedQuantizedOps.cs:447-479): (d * sc) * q - dmin * m.
+__global__ void __launch_bounds__(256) dequant_q4k_wide_kernel(const uint8_t* __restrict__ src, float* __restrict__ dst, int64_t n8)
+{
+    const int64_t t0 = (int64_t)blockIdx.x * (256 * kWideItems) + threadIdx.x;
+    uint4 hd[kWideItems];
+    uint32_t qd[kWideItems];
+#pragma unroll
+    for (int u = 0; u < kWideItems; ++u) {
+        const int64_t t = t0 + 256 * u;
+        if (t < n8) {
+            const uint8_t* blk = src + (t >> 5) * 144;
+            hd[u] = *reinterpret_cast<const uint4*>(blk);
+            qd[u] = *reinterpret_cast<const uint32_t*>(blk + 16 + 4 * (int)(t & 31));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kWideItems; ++u) {
+        const int64_t t = t0 + 256 * u;
+        if (t >= n8) continue;
+        const int64_t b = t >> 5;
+        const int i = (int)(t & 31), g = i >> 3, l = (i & 7) * 4;
+        const uint4 hdr = hd[u];
+        const uint32_t q = qd[u];
+        const float d = half_bits_to_float(hdr.x & 0xffffu), dmin = half_bits_to_float(hdr.x >> 16);
+        // scales[12] = hdr.y, hdr.z, hdr.w; sub-blocks j = 2 g and 2 g + 1 (get_scale_min_k4, ggml-quants.c:703-710)
+        uint32_t sc[2], mn[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int j = 2 * g + k;
+            const uint32_t pj = ((j < 4 ? hdr.y : hdr.z) >> (8 * (j & 3))) & 0xffu;      // scales[j]
+            const uint32_t pj4 = ((j < 4 ? hdr.z : hdr.w) >> (8 * (j & 3))) & 0xffu;     // scales[j + 4]
+            const uint32_t pjm4 = (hdr.y >> (8 * (j & 3))) & 0xffu;                      // scales[j - 4], used for j >= 4
+            sc[k] = j < 4 ? (pj & 63u) : ((pj4 & 0x0fu) | ((pjm4 >> 6) << 4));
+            mn[k] = j < 4 ? (pj4 & 63u) : ((pj4 >> 4) | ((pj >> 6) << 4));
+        }
+        const float d1 = d * (float)sc[0], m1 = dmin * (float)mn[0];
+        const float d2 = d * (float)sc[1], m2 = dmin * (float)mn[1];
+        float4 lo, hi;
+        lo.x = d1 * (float)(q & 0x0fu) - m1;
+        lo.y = d1 * (float)((q >> 8) & 0x0fu) - m1;
+        lo.z = d1 * (float)((q >> 16) & 0x0fu) - m1;
+        lo.w = d1 * (float)((q >> 24) & 0x0fu) - m1;
+        hi.x = d2 * (float)((q >> 4) & 0x0fu) - m2;
+        hi.y = d2 * (float)((q >> 12) & 0x0fu) - m2;
+        hi.z = d2 * (float)((q >> 20) & 0x0fu) - m2;
+        hi.w = d2 * (float)(q >> 28) - m2;
+        float* o = dst + b * 256 + 64 * g + l;
+        *reinterpret_cast<float4*>(o) = lo;
+        *reinterpret_cast<float4*>(o + 32) = hi;
+    }
+}
+
 // dst[i, :] = dequantized row ids[i] of the weight; rows with an index outside [0, ne1) become zeros
 template <int TYPE>
 __global__ void __launch_bounds__(256) get_rows_kernel(const uint8_t* __restrict__ src, int64_t row_bytes, int64_t ne1,
@@ -282,9 +431,27 @@ bool launch_dequant(int type, const void* src, int64_t n, float* dst, hipStream_
     const dim3 grid((unsigned)blocks), block(256);
     const uint8_t* s = static_cast<const uint8_t*>(src);
     switch (type) {
-    case kTypeQ8_0: hipLaunchKernelGGL(dequant_kernel<kTypeQ8_0>, grid, block, 0, stream, s, dst, n4); break;
-    case kTypeQ4_K: hipLaunchKernelGGL(dequant_kernel<kTypeQ4_K>, grid, block, 0, stream, s, dst, n4); break;
-    case kTypeMXFP4: hipLaunchKernelGGL(dequant_kernel<kTypeMXFP4>, grid, block, 0, stream, s, dst, n4); break;
+    case kTypeQ8_0:
+    case kTypeMXFP4:
+        if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+            const int64_t n8 = n / 8;
+            const dim3 wide((unsigned)((n8 + 256 * kWideItems - 1) / (256 * kWideItems)));
+            if (type == kTypeQ8_0) hipLaunchKernelGGL(dequant_q8_0_wide_kernel, wide, block, 0, stream, s, dst, n8);
+            else hipLaunchKernelGGL(dequant_mxfp4_wide_kernel, wide, block, 0, stream, s, dst, n8);
+        } else if (type == kTypeQ8_0) {
+            hipLaunchKernelGGL(dequant_kernel<kTypeQ8_0>, grid, block, 0, stream, s, dst, n4);
+        } else {
+            hipLaunchKernelGGL(dequant_kernel<kTypeMXFP4>, grid, block, 0, stream, s, dst, n4);
+        }
+        break;
+    case kTypeQ4_K:
+        if ((reinterpret_cast<uintptr_t>(s) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+            const int64_t n8 = n / 8;
+            hipLaunchKernelGGL(dequant_q4k_wide_kernel, dim3((unsigned)((n8 + 256 * kWideItems - 1) / (256 * kWideItems))), block, 0, stream, s, dst, n8);
+        } else {
+            hipLaunchKernelGGL(dequant_kernel<kTypeQ4_K>, grid, block, 0, stream, s, dst, n4);
+        }
+        break;
 #define TSHIP_DEQUANT_CASE(T) case T: hipLaunchKernelGGL(dequant_kernel<T>, grid, block, 0, stream, s, dst, n4); break;
     TSHIP_DEQUANT_CASE(kTypeF16) TSHIP_DEQUANT_CASE(kTypeBF16) TSHIP_DEQUANT_CASE(kTypeQ4_0) TSHIP_DEQUANT_CASE(kTypeQ4_1)
     TSHIP_DEQUANT_CASE(kTypeQ5_0) TSHIP_DEQUANT_CASE(kTypeQ5_1) TSHIP_DEQUANT_CASE(kTypeQ5_K) TSHIP_DEQUANT_CASE(kTypeQ6_K)

@@ -60,6 +60,38 @@ def test_random_bytes_host_and_device_entry(hip, oracle, name):
     assert bits_equal(out.cpu().numpy(), want)
 
 
+def test_q4_k_every_scale_code_and_unaligned_blocks(hip, oracle):
+    # every 6-bit scale / min code in every sub-block position and every nibble; then the same blocks at a device
+    # address that is not 16-byte aligned (the dequantizer has a kernel for aligned blocks and one for the rest)
+    import torch
+    rng = np.random.default_rng(77)
+    raw = rng.integers(0, 256, size=(4096, 144), dtype=np.uint8)
+    codes = np.arange(4096)
+    raw[:, 0:2] = np.array([0x00, 0x3C], dtype=np.uint8)            # d = 1.0
+    raw[:, 2:4] = np.array([0x00, 0x38], dtype=np.uint8)            # dmin = 0.5
+    for j in range(8):                                              # sub-block j: scale = code % 64, min = code // 64 (rotated per j)
+        sc, mn = (codes + 7 * j) % 64, ((codes // 64) + 5 * j) % 64
+        if j < 4:
+            raw[:, 4 + j] = (raw[:, 4 + j] & 0xC0) | sc
+            raw[:, 8 + j] = (raw[:, 8 + j] & 0xC0) | mn
+        else:
+            raw[:, 8 + j] = (sc & 15) | ((mn & 15) << 4)
+            raw[:, j] = (raw[:, j] & 0x3F) | ((sc >> 4) << 6)
+            raw[:, 4 + j] = (raw[:, 4 + j] & 0x3F) | ((mn >> 4) << 6)
+    raw = raw.reshape(-1)
+    want = oracle.dequantize(Q4_K, raw)
+    dev = torch.from_numpy(raw).cuda()
+    out = hip.DequantizeToFloat32Device(Q4_K, dev, want.size)
+    torch.cuda.synchronize()
+    assert bits_equal(out.cpu().numpy(), want)
+    shifted = torch.empty(raw.size + 16, dtype=torch.uint8, device="cuda")
+    for off in (2, 4, 9):
+        shifted[off:off + raw.size] = dev
+        out = hip.DequantizeToFloat32Device(Q4_K, shifted[off:off + raw.size], want.size)
+        torch.cuda.synchronize()
+        assert bits_equal(out.cpu().numpy(), want), off
+
+
 def test_full_size_weight(hip, oracle):
     # cfg 2 gate projection, 58.7 M weights, reference-quantized
     fmt, N, K = inputs.CFG2["gate"]
