@@ -167,6 +167,35 @@ def test_head_shapes_groupings_and_split_counts(hip, oracle, heads, kv_heads, he
         assert rel(kd.cpu().numpy()[:, pos], kc[:, pos]) <= 1e-5 and rel(vd.cpu().numpy()[:, pos], vc[:, pos]) <= 1e-5
 
 
+@pytest.mark.parametrize("head_dim", [64, 80, 96, 128, 192, 256])
+@pytest.mark.parametrize("group,kv_heads,prefix", [(1, 4, 70), (4, 8, 2100), (8, 8, 2100)])
+def test_every_attention_instantiation(hip, oracle, head_dim, group, kv_heads, prefix):
+    # the attention kernel is compiled per head width and per number of query heads a workgroup serves (1, 2, 4, 8); the
+    # launcher serves 4 or 8 only when that still leaves 128 workgroups, i.e. with many KV heads and splits - shapes the
+    # tests above do not reach
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    heads = group * kv_heads
+    rng = np.random.default_rng(head_dim * 10 + group)
+    hidden, inter, max_seq = 256, 256, prefix + 2
+    layer, dims = make_layer(oracle, rng, hidden, heads, kv_heads, head_dim, inter, (Q8_0, Q8_0, Q8_0, Q8_0), True)
+    dev = to_device_layer(layer, torch, QuantizedWeight, dims)
+    kc = np.zeros((kv_heads, max_seq, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    vc[:, :prefix] = rng.standard_normal((kv_heads, prefix, head_dim)).astype(np.float32)
+    kd, vd = torch.from_numpy(kc.copy()).cuda(), torch.from_numpy(vc.copy()).cuda()
+    for pos in range(prefix, prefix + 2):
+        h = rng.standard_normal(hidden).astype(np.float32)
+        hd = torch.from_numpy(h.copy()).cuda()
+        oracle.layer_decode(h, layer, kc, vc, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, 2)
+        hip.TransformerLayerDecode(hd, dev["attn_norm"], dev["qkv"], dev["q_norm"], dev["k_norm"], dev["o"], dev["ffn_norm"],
+                                   dev["gate_up"], dev["down"], kd, vd, heads, kv_heads, head_dim, pos, 1e-6, 10000.0, 1.0, 2)
+        torch.cuda.synchronize()
+        assert rel(hd.cpu().numpy(), h) <= 3e-3, (pos, rel(hd.cpu().numpy(), h))
+        assert rel(kd.cpu().numpy()[:, pos], kc[:, pos]) <= 1e-5 and rel(vd.cpu().numpy()[:, pos], vc[:, pos]) <= 1e-5
+
+
 def to_host_layer(layer, QuantizedWeight, dims):
     d = {k: (None if layer[k] is None else np.ascontiguousarray(layer[k])) for k in ("attn_norm", "q_norm", "k_norm", "ffn_norm")}
     for k, (ne0, ne1) in dims.items():
