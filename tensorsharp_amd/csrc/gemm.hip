@@ -1692,24 +1692,25 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
 {
     if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream, cs);
     // Q4_K and MXFP4: the 2 x 4 wavefront layout with the operand exchange through LDS (gemm_xw_kernel); 128-row tiles are
-    // 128 x 256
+    // 128 x 256.  Q4_K takes it for every launch, MXFP4 for plain ones: the MXFP4 expert tiles of a MoE prefill (128
+    // rows) stay on two 128 x 128 workgroups per CU (926 vs 968 us at 2048 tokens).
     if constexpr (std::is_same<G, GQ4K>::value) {
         if (bm == 256) return launch_xw<PQ4K, 256, 4>(a, m_tiles, stream, cs);
         if (bm == 128) return launch_xw<PQ4K, 128, 4>(a, m_tiles, stream, cs);
-    }
-    // (MXFP4 expert tiles of a MoE prefill stay on two 128 x 128 workgroups per CU: 926 vs 968 us at 2048 tokens)
-    if constexpr (std::is_same<G, GMXFP4>::value) {
+    } else if constexpr (std::is_same<G, GMXFP4>::value) {
         if (bm == 256 && !a.tile_expert) return launch_xw<PMXFP4, 256, 4>(a, m_tiles, stream, cs);
         if (bm == 128 && !a.tile_expert) return launch_xw<PMXFP4, 128, 4>(a, m_tiles, stream, cs);
+        if (bm == 128) return launch_tiles<G, 128, 2, 4>(a, m_tiles, stream, cs);
+    } else {
+        if constexpr (2 * 256 * kXRow + 2 * 256 * G::kRawRow + 1024 <= 160 * 1024) {
+            if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream, cs);
+        }
+        // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
+        // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 and Q6_K the other way round
+        if (bm == 128)
+            return kWide128<G> ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream, cs)
+                               : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream, cs);
     }
-    if constexpr (2 * 256 * kXRow + 2 * 256 * G::kRawRow + 1024 <= 160 * 1024) {
-        if (bm == 256) return launch_tiles<G, 256, 2, 8>(a, m_tiles, stream, cs);
-    }
-    // 128-row tiles: for the 4-bit formats two independent 128 x 128 workgroups per CU (their copy, LDS and
-    // matrix phases overlap) measured faster than one 128 x 256 workgroup; Q8_0 and Q6_K the other way round
-    if (bm == 128)
-        return kWide128<G> ? launch_tiles<G, 128, 2, 8>(a, m_tiles, stream, cs)
-                                                   : launch_tiles<G, 128, 2, 4>(a, m_tiles, stream, cs);
     set_last_error("gemm: unsupported tile height.");
     return false;
 }

@@ -92,6 +92,19 @@ def test_q4_k_every_scale_code_and_unaligned_blocks(hip, oracle):
         assert bits_equal(out.cpu().numpy(), want), off
 
 
+@pytest.mark.parametrize("name", ["q8_0", "mxfp4", "q4_k"])
+def test_destination_not_16_byte_aligned(hip, oracle, name):
+    import torch
+    rng = np.random.default_rng(79)
+    raw = rng.integers(0, 256, size=BB[name] * 3000, dtype=np.uint8)
+    want = oracle.dequantize(T[name], raw)
+    buf = torch.zeros(want.size + 8, dtype=torch.float32, device="cuda")
+    for off in (1, 3):
+        hip.DequantizeToFloat32Device(T[name], torch.from_numpy(raw).cuda(), want.size, dst=buf[off:off + want.size])
+        torch.cuda.synchronize()
+        assert bits_equal(buf[off:off + want.size].cpu().numpy(), want), (name, off)
+
+
 def test_full_size_weight(hip, oracle):
     # cfg 2 gate projection, 58.7 M weights, reference-quantized
     fmt, N, K = inputs.CFG2["gate"]

@@ -12,6 +12,8 @@ last product's norm plus 1e-3 of the first's, written at each assert."""
 import numpy as np
 import pytest
 
+import inputs
+
 from oracle.oracle import F32, F16, BF16, Q8_0, Q4_K, Q6_K, MXFP4
 
 pytestmark = pytest.mark.gpu
@@ -171,6 +173,36 @@ def test_experts_swiglu_forward(hip, oracle, name, down, n, M, device):
     got = got[0] if device else got
     tol = set_tol(oracle, parts, w)
     assert np.all(np.abs(got - ref) <= tol), (name, n, M, device, float(np.max(np.abs(got - ref) / tol)))
+
+
+def make_blocks(name, N, K, rng):
+    """(type, raw bytes, N, K) of valid random blocks for the formats whose quantizer the oracle does not restate"""
+    import torch
+    from oracle.oracle import MORE_TYPES
+    from tensorsharp_amd import synth
+    if name == "q6_k":
+        g = torch.Generator()
+        g.manual_seed(int(rng.integers(1 << 30)))
+        return (Q6_K, synth.quantize_q6_k_simple(torch.randn((N, K), generator=g) * 0.05).numpy().reshape(-1), N, K)
+    return (MORE_TYPES[name], inputs.random_blocks(name, N, K, rng), N, K)
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_k", "q6_k"])
+@pytest.mark.parametrize("n", [1, 6])
+def test_experts_swiglu_single_row_other_gemv_formats(hip, oracle, name, n):
+    # one row: the down projection of each expert is a GEMV that forms silu(gate) * up while it stages its activations,
+    # compiled per format
+    rng = np.random.default_rng(350 + n)
+    H, I = 512, 256
+    ex = [dict(gate=make_blocks(name, I, H, rng), up=make_blocks(name, I, H, rng), down=make_blocks(name, H, I, rng)) for _ in range(n)]
+    w = rng.uniform(0.05, 0.6, n).astype(np.float32)
+    x = rng.standard_normal((1, H)).astype(np.float32)
+    ref, parts = oracle.expert_set(x, ex, w)
+    fn = lambda r, i: hip.MoEExpertsSwiGLUForward(r, i, [qw(e["gate"], True) for e in ex], [qw(e["up"], True) for e in ex],
+                                                  [qw(e["down"], True) for e in ex], w)
+    got = run(hip, True, fn, np.full((1, H), np.nan, np.float32), x)[0]
+    tol = set_tol(oracle, parts, w)
+    assert np.all(np.abs(got - ref) <= tol), (name, n, float(np.max(np.abs(got - ref) / tol)))
 
 
 @pytest.mark.parametrize("shared", [None, "same", "wider", "other_type"])

@@ -248,6 +248,33 @@ def test_more_formats_matmul(hip, oracle, name, M, N, K):
     check(y, oracle.matmul_f64(t, wq, N, K, x), (name, M, N, K))
 
 
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "q5_k", "mxfp4"])
+def test_256_row_tiles_of_the_other_formats(hip, oracle, name):
+    # 1024 x 8448: more 128-row tiles than one round of workgroups, so the launcher takes 256-row tiles
+    from oracle.oracle import MORE_TYPES
+    M, N, K = 1024, 8448, 512
+    t = MORE_TYPES[name] if name in MORE_TYPES else T[name]
+    rng = np.random.default_rng(N + t)
+    wq = inputs.random_blocks(name, N, K, rng) if name in MORE_TYPES else oracle.quantize(t, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, t, wq, N, K, x)
+    rows = np.unique(np.concatenate([np.arange(0, M, 37), [255, 256, 511, 767, 1023]]))
+    check(y[rows], oracle.matmul_f64(t, wq, N, K, x[rows]), (name, M, N, K))
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl"])
+def test_small_batch_k_range_of_four_tiles(hip, oracle, name):
+    # K = 1536: 24 k-tiles over eight wavefronts -> the register-resident kernel built for four k-tiles per wavefront
+    from oracle.oracle import MORE_TYPES
+    M, N, K = 16, 300, 1536
+    t = MORE_TYPES[name]
+    rng = np.random.default_rng(K + t)
+    wq = inputs.random_blocks(name, N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, t, wq, N, K, x)
+    check(y, oracle.matmul_f64(t, wq, N, K, x), (name, M, N, K))
+
+
 @pytest.mark.parametrize("name,row_bytes", [("q4_0", 18 * 3), ("q5_0", 22 * 3), ("q5_1", 24 * 5)])
 def test_more_formats_rows_two_bytes_off(hip, oracle, name, row_bytes):
     import torch

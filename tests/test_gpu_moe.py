@@ -64,6 +64,51 @@ def test_expert_stage_small_dims(hip, oracle, name, T, k):
     assert inputs.row_l2_err(got2, ref2) <= 1e-3
 
 
+@pytest.mark.parametrize("name", ["mxfp4", "q4_k"])
+def test_expert_tiles_of_128_rows(hip, oracle, name):
+    # more than 160 rows per expert on average: the grouped GEMM runs 128-row tiles instead of 32-row ones
+    rng = np.random.default_rng(71)
+    E, H, F, T, k = 4, 256, 256, 400, 2
+    t = T_[name]
+    gu, gb, dn, db = make_experts(oracle, t, E, H, F, rng)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    ref = oracle.moe_forward(t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    got = run_gpu(hip, t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got, ref) <= 1e-3, (name, inputs.row_l2_err(got, ref))
+
+
+@pytest.mark.parametrize("T", [1, 2])
+def test_top_1_routing(hip, oracle, T):
+    rng = np.random.default_rng(73)
+    E, H, F = 8, 512, 768
+    gu, gb, dn, db = make_experts(oracle, MXFP4, E, H, F, rng)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), 1)
+    ref = oracle.moe_forward(MXFP4, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    got = run_gpu(hip, MXFP4, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got, ref) <= 1e-3, inputs.row_l2_err(got, ref)
+
+
+@pytest.mark.parametrize("T", [1, 40])
+def test_down_bias_at_an_address_that_is_not_16_byte_aligned(hip, oracle, T):
+    # the weighted sum over a token's experts reads rows, bias and output as 16-byte vectors only when all are aligned
+    import torch
+    rng = np.random.default_rng(75)
+    E, H, F, k = 8, 512, 768, 4
+    gu, gb, dn, db = make_experts(oracle, MXFP4, E, H, F, rng)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    ref = oracle.moe_forward(MXFP4, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    c = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    buf = torch.zeros(E * H + 4, dtype=torch.float32, device="cuda")
+    buf[1:1 + E * H] = c(db).reshape(-1)
+    out = hip.MoEExpertsGptOssForward(c(hidden), c(ids.astype(np.int32)), c(wts), c(gu), c(gb), c(dn), buf[1:1 + E * H].view(E, H),
+                                      MXFP4, E, H, F)
+    torch.cuda.synchronize()
+    assert inputs.row_l2_err(out.cpu().numpy(), ref) <= 1e-3
+
+
 def test_unbalanced_and_empty_experts(hip, oracle):
     rng = np.random.default_rng(65)
     E, H, F, T, k = 16, 256, 256, 200, 2
