@@ -235,10 +235,16 @@ def main():
         step(i)
     # exactly --steps steps between two synchronisations ...
     k_ev_ms, k_wall_ms = time_region(step, args.steps, torch)
-    # ... and, because a region of a few steps of 25 us each is mostly the cost of the two synchronisations, a region of
-    # at least 200 steps from which `value` is taken; both are reported
-    timed_steps = max(args.steps, 200)
-    ev_ms, wall_ms = (k_ev_ms, k_wall_ms) if timed_steps == args.steps else time_region(step, timed_steps, torch)
+    # ... and, because a region of a few steps of 25 us each is mostly the cost of the two synchronisations and the first
+    # ~10 ms of launches after an idle period run slower (500 steps average 24.9 us per launch where 2000 average 24.15),
+    # a region of at least 1000 steps, entered after at least 800 launches, from which `value` is taken; both are reported
+    timed_steps = max(args.steps, 1000)
+    if timed_steps == args.steps:
+        ev_ms, wall_ms = k_ev_ms, k_wall_ms
+    else:
+        for i in range(max(0, 800 - args.warmup - args.steps)):
+            step(i)
+        ev_ms, wall_ms = time_region(step, timed_steps, torch)
     assert all(bool(torch.isfinite(y).all()) for y in ys)
     ms_per_step = wall_ms / timed_steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
