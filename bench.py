@@ -118,6 +118,20 @@ def time_region(fn, steps, torch):
     return e0.elapsed_time(e1), wall
 
 
+def library_fp16_gemm_us(torch, dev, m, n, k, iters=20):
+    """Reference point only, never part of `value` or of the product: the vendor library's GEMM (torch.matmul) on DENSE fp16
+    operands of the same shape - no dequantization, half-precision inputs and output - timed like the calls beside it."""
+    x = torch.randn((m, k), device=dev, dtype=torch.float16)
+    w = (torch.randn((n, k), device=dev, dtype=torch.float32) * 0.02).to(torch.float16)
+
+    def f(i):
+        torch.matmul(x, w.t())
+    for i in range(3):
+        f(i)
+    ev, wall = time_region(f, iters, torch)
+    return ev * 1e3 / iters
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -211,8 +225,11 @@ def main():
         ev, wall = time_region(one, args.steps, torch)
         us = ev * 1e3 / args.steps
         b = algorithmic_bytes(t, n, k, m)
-        print(json.dumps({"matmul": {"type": t, "M": m, "N": n, "K": k, "weight_copies": copies}, "us_per_call_events": round(us, 2), "bytes": b,
-                          "GBps": round(b / (us * 1e-6) / 1e9, 1), "TFLOPs": round(2.0 * m * n * k / (us * 1e-6) / 1e12, 2)}))
+        res = {"matmul": {"type": t, "M": m, "N": n, "K": k, "weight_copies": copies}, "us_per_call_events": round(us, 2), "bytes": b,
+               "GBps": round(b / (us * 1e-6) / 1e9, 1), "TFLOPs": round(2.0 * m * n * k / (us * 1e-6) / 1e12, 2)}
+        if m >= 128:
+            res["library_dense_fp16_gemm_us"] = round(library_fp16_gemm_us(torch, dev, m, n, k, min(args.steps, 20)), 1)
+        print(json.dumps(res))
         return
 
     # ---- workload: `copies` layers of seven Q4_K matrices, device resident -------------------
@@ -287,7 +304,13 @@ def main():
         ev, wall = time_region(f, iters, torch)
         us = ev * 1e3 / iters
         tf = 2.0 * m * n * k / (us * 1e-6) / 1e12
-        return {"us_per_call_events": round(us, 1), "TFLOPs": round(tf, 1), "pct_mfma_fp16_peak": round(100 * tf / MFMA_FP16_PEAK_TFLOPS, 1)}
+        res = {"us_per_call_events": round(us, 1), "TFLOPs": round(tf, 1), "pct_mfma_fp16_peak": round(100 * tf / MFMA_FP16_PEAK_TFLOPS, 1)}
+        if m >= 512 and t in (Q4_K, Q8_0) and not args.no_extra:
+            del w, y
+            lib = library_fp16_gemm_us(torch, dev, m, n, k)
+            res["library_dense_fp16_gemm"] = {"us_per_call_events": round(lib, 1),
+                                              "pct_mfma_fp16_peak": round(100 * 2.0 * m * n * k / (lib * 1e-6) / 1e12 / MFMA_FP16_PEAK_TFLOPS, 1)}
+        return res
 
     pm, pn, pk = 2048, 21504, 5376
     pre = prefill(Q4_K, pm, pn, pk, 20)
