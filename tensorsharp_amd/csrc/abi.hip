@@ -418,11 +418,16 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
     for (int m0 = 0; m0 < M; m0 += plan.m_step) {
         const int m = std::min(plan.m_step, M - m0);
         const float* x = static_cast<const float*>(m1.data) + (int64_t)m0 * m1.stride0;
-        if (!launch_convert_x(type, x, m1.stride0, nullptr, m, (int)K, ws, stream, norm_w, eps)) return false;
+        int converted = -1;         // activation layout in the workspace (row slices of an over-large weight may differ)
         for (int64_t n0 = 0; n0 < N; n0 += plan.n_step) {
             const int64_t n = std::min<int64_t>(plan.n_step, N - n0);
+            const int layout = gemm_x_layout(type, m, (int)n, (int)K);
+            if (layout != converted) {
+                if (!launch_convert_x(type, x, m1.stride0, nullptr, m, (int)K, ws, stream, norm_w, eps, layout)) return false;
+                converted = layout;
+            }
             if (!launch_gemm(type, wb + (size_t)n0 * rs, (int64_t)(rs * (size_t)n), ws, out + (int64_t)m0 * result.stride0 + n0,
-                             result.stride0, nullptr, m, (int)n, (int)K, nullptr, stream, accumulate, chunk_ws, chunk_bytes))
+                             result.stride0, nullptr, m, (int)n, (int)K, nullptr, stream, accumulate, chunk_ws, chunk_bytes, layout))
                 return false;
         }
     }

@@ -24,6 +24,7 @@
 #include "tship_internal.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -37,6 +38,8 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kBK = 64;                 // k-tile
 constexpr uint32_t kDeadOffset = 0x80000000u;
+// activation layout tag of convert_x_kernel for gemm_mx_kernel: two block-scaled fp6 (E2M3) terms per activation
+constexpr int kXMx = 1000;
 
 union H2U {
     uint32_t u;
@@ -126,7 +129,7 @@ __device__ __forceinline__ float swiglu_oai(float gate, float up, float alpha, f
 }
 
 template <int TYPE, int THREADS, int SRC>
-__global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, int K, int Kp, _Float16* __restrict__ out,
+__global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, int K, int Kp, int ldo, _Float16* __restrict__ out,
                                                             float* __restrict__ scales)
 {
     const int m = blockIdx.x;
@@ -207,7 +210,128 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
     const int se = e - 13;
     const float inv = __uint_as_float((uint32_t)(254 - se) << 23);
     if (tid == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
-    _Float16* dst = out + (int64_t)m * Kp;
+    _Float16* dst = out + (int64_t)m * ldo;
+    if constexpr (TYPE == kXMx) {
+        // gemm_mx_kernel: every 32 activations are two MX blocks of fp6 (E2M3) values, x = hi * 2^Eh + lo * 2^El with
+        // lo the same encoding of the rest x - hi * 2^Eh: what is left is below 2^-9 of the block's largest magnitude.
+        // The exponents are absolute (E8M0), so the row scale is one.  A k-tile of a row is 128 bytes = 8 pieces of 16:
+        // term p (hi, lo) of block g keeps the first 16 bytes of its 24-byte field stream in piece 3 p + 2 g and the last
+        // 8 in half g of piece 3 p + 1; piece 6 holds the scale bytes (hi, lo) of block g in the low bytes of dword g.
+        // Field f of a stream pairs with nibble f of the weight block: element f / 2 (f even) or 16 + f / 2 (f odd).
+        uint8_t* const d8 = reinterpret_cast<uint8_t*>(dst);
+        if (tid == 0) scales[m] = 1.0f;
+        // biased exponent E + 127 that brings amax into (3.75, 7.5]; 127 for an empty block, 255 (NaN) for inf / NaN
+        auto block_exp = [](float amax) -> int {
+            const uint32_t u = __float_as_uint(amax);
+            const int ex = (int)(u >> 23) & 0xff;
+            if (ex == 255) return 255;
+            if (amax == 0.f) return 127;
+            const int eb = ex - ((u & 0x7fffffu) > 0x700000u ? 1 : 2);      // mantissa above 1.875 would round up to 8
+            return eb < 1 ? 1 : eb;                                            // at most 253: 2^(254 - eb) is a normal float
+        };
+        auto pow2 = [](int biased) { return __uint_as_float((uint32_t)biased << 23); };      // biased 1..254
+        // E2M3 code of v (|v| <= 7.75): codes 0..16 step 1/8, 16..24 step 1/4, 24..31 step 1/2; sign in bit 5
+        auto enc = [](float v) -> uint32_t {
+            const float mag = fabsf(v);
+            const float c = mag < 2.f ? mag * 8.f : mag < 4.f ? 16.f + (mag - 2.f) * 4.f : 24.f + (mag - 4.f) * 2.f;
+            uint32_t code = (uint32_t)__builtin_rintf(c);
+            code = code > 31u ? 31u : code;
+            return code | (v < 0.f ? 32u : 0u);
+        };
+        auto dec = [](uint32_t code) -> float {
+            const uint32_t c = code & 31u;
+            const float mag = c < 16u ? (float)c * 0.125f : c < 24u ? 2.f + (float)(c - 16u) * 0.25f : 4.f + (float)(c - 24u) * 0.5f;
+            return (code & 32u) ? -mag : mag;
+        };
+        // where byte b (0..23) of the stream of term p, block g lives inside the row's k-tile
+        auto stream_off = [](int p, int g, int b) { return b < 16 ? (3 * p + 2 * g) * 16 + b : (3 * p + 1) * 16 + 8 * g + (b - 16); };
+        constexpr int kIters = kCvtHold;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+            if (i * THREADS >= k4) break;                          // uniform: whole passes beyond the row
+            const int q = tid + i * THREADS;                       // lanes past the row hold zeros and take part
+            const float4 v = hold[i];
+            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            amax = fmaxf(amax, __shfl_xor(amax, 1));
+            amax = fmaxf(amax, __shfl_xor(amax, 2));
+            amax = fmaxf(amax, __shfl_xor(amax, 4));
+            if (!(amax == amax)) amax = __uint_as_float(0x7f800000u);
+            {
+                // a NaN anywhere in the block must reach the maximum (fmaxf drops NaNs)
+                const bool nan = (v.x != v.x) || (v.y != v.y) || (v.z != v.z) || (v.w != v.w);
+                const unsigned long long any = __ballot(nan);
+                if ((any >> ((threadIdx.x & 63) & ~7)) & 0xffull) amax = __uint_as_float(0x7f800000u);
+            }
+            const int eh = block_exp(amax);
+            const bool finite = eh != 255;
+            const float inv_h = finite ? pow2(254 - eh) : 0.f, sc_h = finite ? pow2(eh) : 0.f;
+            const uint32_t h0 = enc(v.x * inv_h), h1 = enc(v.y * inv_h), h2 = enc(v.z * inv_h), h3 = enc(v.w * inv_h);
+            const float r0 = finite ? v.x - dec(h0) * sc_h : 0.f, r1 = finite ? v.y - dec(h1) * sc_h : 0.f;
+            const float r2 = finite ? v.z - dec(h2) * sc_h : 0.f, r3 = finite ? v.w - dec(h3) * sc_h : 0.f;
+            float rmax = fmaxf(fmaxf(fabsf(r0), fabsf(r1)), fmaxf(fabsf(r2), fabsf(r3)));
+            rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
+            rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
+            rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
+            const int el = block_exp(rmax);
+            const float inv_l = pow2(254 - el);
+            const uint32_t l0 = enc(r0 * inv_l), l1 = enc(r1 * inv_l), l2 = enc(r2 * inv_l), l3 = enc(r3 * inv_l);
+            // the lane four to the right (left) holds the elements 16 further on (back): together they own fields
+            // 8 t .. 8 t + 7 of the stream (t = lane % 4), six bytes; each lane packs all eight codes
+            const uint32_t mine_h = h0 | (h1 << 6) | (h2 << 12) | (h3 << 18), mine_l = l0 | (l1 << 6) | (l2 << 12) | (l3 << 18);
+            const uint32_t other_h = __shfl_xor(mine_h, 4), other_l = __shfl_xor(mine_l, 4);
+            const bool upper = (q & 4) != 0;
+            const uint32_t even_h = upper ? other_h : mine_h, odd_h = upper ? mine_h : other_h;
+            const uint32_t even_l = upper ? other_l : mine_l, odd_l = upper ? mine_l : other_l;
+            auto weave = [](uint32_t ev, uint32_t od) -> unsigned long long {      // fields e0 o0 e1 o1 e2 o2 e3 o3
+                unsigned long long w = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    w |= (unsigned long long)((ev >> (6 * j)) & 63u) << (12 * j) | (unsigned long long)((od >> (6 * j)) & 63u) << (12 * j + 6);
+                return w;
+            };
+            const unsigned long long wh = weave(even_h, odd_h), wl = weave(even_l, odd_l);
+            const int k0 = 4 * (q & ~4);                           // first element of the lower lane of the pair
+            const int g = (k0 >> 5) & 1, t4 = (k0 & 15) >> 2;      // block of the k-tile, quarter of the stream
+            uint8_t* const row = d8 + (k0 >> 6) * 128;
+            // the four lower lanes of a block assemble the hi stream, the four upper lanes the lo stream: lane t4 holds
+            // bytes 6 t4 .. 6 t4 + 5 and fetches the lane after it for the dwords that straddle two lanes
+            const unsigned long long w = upper ? wl : wh;
+            const uint32_t w_lo = (uint32_t)w, w_hi = (uint32_t)(w >> 32);
+            const uint32_t nb_lo = __shfl_down(w_lo, 1);
+            const int p = upper ? 1 : 0;
+            if (q < k4) {
+                uint8_t* const main_piece = row + (3 * p + 2 * g) * 16;
+                uint8_t* const rest_piece = row + (3 * p + 1) * 16 + 8 * g;
+                const uint32_t straddle = (w_hi & 0xffffu) | (nb_lo << 16);       // bytes 4, 5 of this lane, 0, 1 of the next
+                const uint32_t upper4 = (w_lo >> 16) | (w_hi << 16);              // bytes 2 .. 5 of this lane
+                if (t4 == 0) {
+                    uint2 v2;
+                    v2.x = w_lo;
+                    v2.y = straddle;
+                    *reinterpret_cast<uint2*>(main_piece) = v2;
+                    if (!upper) *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = (uint32_t)eh | ((uint32_t)el << 8);
+                } else if (t4 == 1) {
+                    *reinterpret_cast<uint32_t*>(main_piece + 8) = upper4;
+                } else if (t4 == 2) {
+                    *reinterpret_cast<uint32_t*>(main_piece + 12) = w_lo;
+                    *reinterpret_cast<uint32_t*>(rest_piece) = straddle;
+                } else {
+                    *reinterpret_cast<uint32_t*>(rest_piece + 4) = upper4;
+                }
+            }
+        }
+        // blocks past K inside the last k-tile: zero streams under a scale of one
+        for (int blk = (K >> 5) + tid; blk < (Kp >> 5); blk += THREADS) {
+            uint8_t* const row = d8 + (blk >> 1) * 128;
+            const int g = blk & 1;
+            for (int bb = 0; bb < 24; bb += 2) {
+                *reinterpret_cast<uint16_t*>(row + stream_off(0, g, bb)) = 0;
+                *reinterpret_cast<uint16_t*>(row + stream_off(1, g, bb)) = 0;
+            }
+            *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = 127u | (127u << 8);
+        }
+        return;
+    }
     auto put = [&](int k, float v) { dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)(v * inv); };
     // Four consecutive activations land in one aligned 8-byte piece of the k-tile: in the K-quant order as
     // (x0, x2, x1, x3), in the natural order as they are, and in the split-nibble order interleaved with the four
@@ -569,6 +693,7 @@ struct GemmArgs {
     int64_t ldc;
     const int* c_rows;       // optional: result row index per activation row (scatter)
     int M, N, K, Kp;
+    int xld;                 // halfs between activation rows of x16 (x_row_halfs)
     int m_tiles, n_tiles;
     // grouped (MoE) launches: m-tiles enumerated through this table
     const int* tile_expert;  // [m_tiles] expert id
@@ -581,6 +706,7 @@ struct GemmArgs {
     float* partial;          // null: one chunk, results go straight to c
     int k_chunks;
     int chunk_kt;            // k-tiles per chunk (8 wavefronts x KTW)
+    int x_mx;                // the activations are MX fp6 pairs in gemm_mx_kernel's layout (convert_x_kernel<kXMx>)
 };
 
 constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
@@ -722,7 +848,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
     for (int i = 0; i < XI; ++i) {
         const int q = (wave + NW * i) * 64 + lane;           // LDS chunk slot: row q / 8, position q % 8
         const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
-        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.xld * 2) + (uint32_t)chunk * 16u : kDeadOffset;
     }
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
@@ -1051,7 +1177,7 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
     for (int i = 0; i < XI; ++i) {
         const int q = (wave + NW * i) * 64 + lane;
         const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
-        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.Kp * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.xld * 2) + (uint32_t)chunk * 16u : kDeadOffset;
     }
 #pragma unroll
     for (int i = 0; i < RI; ++i) {
@@ -1401,6 +1527,316 @@ bool launch_xw(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
 }
 
 // ------------------------------------------------------------------------------------------
+// MXFP4 on the block-scaled matrix instruction (v_mfma_scale_f32_32x32x64_f8f6f4): the weight operand is the RAW block -
+// 16 bytes of E2M1 pairs plus its E8M0 scale byte, exactly what the instruction's fp4 operand and block scale are -
+// so nothing is unpacked at all.  The activations are two MX terms of fp6 (E2M3) per 32-element block, x = hi 2^Eh +
+// lo 2^El (convert_x_kernel<kXMx>), every product takes two instructions, and fp6 x fp4 runs at twice the rate of the
+// fp16 instruction, so the pair costs half of what the fp16 k-tile costs.  Same tiles as gemm_xw_kernel (BM x 256 x 64,
+// 2 x 4 wavefronts of BM / 2 x 64) and the same LDS-direct copies; no exchange area, so ST copy stages fit.  Operand
+// layout of the instruction (probed on the device): output as the fp16 instructions; lane = column + 32 g holds block g
+// of the k-tile's weights, 32 nibbles low nibble first, and lane = row + 32 g block g of the activations as a stream
+// of 32 six-bit fields, field f pairing with nibble f; each lane's scale byte (selected by op_sel from its scale
+// register) applies to its own block.
+// A scale byte of 255 is NaN to the instruction (ggml's table gives 2^127 there; no quantizer writes it).
+typedef int int8v_t __attribute__((ext_vector_type(8)));
+
+template <int BM, int ST>
+__global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
+{
+    typedef PMXFP4 P;
+    typedef GMXFP4 G;
+    constexpr int BN = 256, WN = 4, NW = 8;
+    constexpr int TMW = BM / 64;                          // 32-row blocks of a wavefront
+    constexpr int NB = 2;                                 // 32-column blocks of a wavefront
+    constexpr int kXTile = BM * kXRow;
+    constexpr int XI = kXTile / 1024 / NW;
+    constexpr int kRawTile = BN * P::kRowBytes;
+    constexpr int kRawCopies = kRawTile / 1024;
+    constexpr int RI = (kRawCopies + NW - 1) / NW;
+    static_assert(TMW == 2 || TMW == 4, "128- or 256-row tiles");
+    static_assert(kRawCopies * 1024 == kRawTile && XI >= 1 && XI * NW * 1024 == kXTile && ST >= 2, "tile pieces must be whole KiB");
+    extern __shared__ uint8_t smem[];
+    uint8_t* const xbuf = smem;                           // ST x kXTile
+    uint8_t* const rraw = xbuf + ST * kXTile;             // ST x kRawTile
+    uint8_t* const dump = rraw + ST * kRawTile;           // 1 KiB
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int col = lane & 31, h = lane >> 5;
+
+    const int tiles = A.m_tiles * A.n_tiles;
+    const int total = tiles * A.k_chunks;
+    int t = blockIdx.x;
+    {
+        const int per = (total + 7) >> 3;
+        const int xcd = t & 7, slot = t >> 3;
+        t = xcd * per + slot;
+        if (slot >= per || t >= total) return;
+    }
+    const int kc = t / tiles;
+    t -= kc * tiles;
+    const int mt = t / A.n_tiles, nt = t - mt * A.n_tiles;
+    const int m0 = mt * BM, m_rows = min(BM, A.M - m0), n0 = nt * BN;
+
+    const uintptr_t wa = reinterpret_cast<uintptr_t>(A.w);
+    const uint32_t base_delta = (uint32_t)(wa & 3);
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<void*>(wa - base_delta), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int kt_begin = kc * A.chunk_kt;
+    const int nkt = min(A.Kp / kBK, kt_begin + A.chunk_kt);
+
+    uint32_t x_off[XI], r_off[RI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+        const int q = (wave + NW * i) * 64 + lane;
+        const int row = q >> 3, chunk = (q & 7) ^ ((row >> 1) & 7);
+        x_off[i] = row < m_rows ? (uint32_t)(m0 + row) * (uint32_t)(A.xld * 2) + (uint32_t)chunk * 16u : kDeadOffset;
+    }
+#pragma unroll
+    for (int i = 0; i < RI; ++i) {
+        const int q = (wave + NW * i) * 64 + lane;                // 16-byte piece of the raw tile
+        const int row = q / P::kParts, part = q - row * P::kParts;
+        const bool ok = q < BN * P::kParts && n0 + row < A.N;
+        r_off[i] = ok ? P::row_window(base_delta + (uint32_t)(n0 + row) * row_bytes) + P::part_base(part) : kDeadOffset;
+    }
+    // every wavefront issues XI + RI copies per k-tile (surplus raw copies go to the dump area, k-tiles past the end
+    // read out of range), so the wait before a barrier is a count
+    // copy c (0 .. RI + XI - 1) of k-tile kt into a stage
+    auto issue_one = [&](int kt, int stage, int c) {
+        const uint32_t past = kt < nkt ? 0u : kDeadOffset;
+        if (c < RI) {
+            const int id = wave + NW * c;
+            copy16_to_lds(wrs, id < kRawCopies ? rraw + stage * kRawTile + id * 1024 : dump, r_off[c] | past, P::soffset(kt));
+        } else {
+            const int i = c - RI;
+            copy16_to_lds(xrs, xbuf + stage * kXTile + (wave + NW * i) * 1024, x_off[i] | past, (uint32_t)kt * kXRow);
+        }
+    };
+    auto issue = [&](int kt, int stage) {
+#pragma unroll
+        for (int c = 0; c < RI + XI; ++c) issue_one(kt, stage, c);
+    };
+    // The copies of a k-tile are spread over the TMW groups of matrix instructions that follow the barrier which freed
+    // their stage (copy c goes behind group c % TMW): a copy occupies the wavefront and the CU's address path for tens
+    // of cycles, and behind a group the matrix pipe has work queued for that long.
+    auto issue_slot = [&](int kt, int stage, int slot) {
+#pragma unroll
+        for (int c = 0; c < RI + XI; ++c)
+            if (c % TMW == slot) issue_one(kt, stage, c);
+    };
+
+    float16_t acc[TMW][NB];
+#pragma unroll
+    for (int m = 0; m < TMW; ++m)
+#pragma unroll
+        for (int n = 0; n < NB; ++n)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[m][n][r] = 0.f;
+
+    // this lane's pieces of an activation row (block h of the k-tile): term p keeps the first 16 bytes of its stream in
+    // piece 3 p + 2 h and the last 8 in half h of piece 3 p + 1; the two scale bytes are dword h of piece 6; pieces sit
+    // where the copy's swizzle placed them
+    const int sw = (col >> 1) & 7;
+    const int a_row = (wm * (BM / 2) + col) * kXRow;
+    int a_main[2], a_rest[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        a_main[p] = a_row + ((3 * p + 2 * h) ^ sw) * 16;
+        a_rest[p] = a_row + ((3 * p + 1) ^ sw) * 16 + 8 * h;
+    }
+    const int a_scale = a_row + (6 ^ sw) * 16 + 4 * h;
+    const int my_raw = (32 * NB * wn + col) * P::kRowBytes;
+    uint32_t my_d0[NB];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) my_d0[n] = P::row_delta(base_delta + (uint32_t)(n0 + 32 * NB * wn + 32 * n + col) * row_bytes);
+
+    // B operands of k-tile kt from its stage: the lane's raw block, re-aligned, and its scale byte
+    auto load_b = [&](int kt, int st, int8v_t (&b)[NB], int (&sb)[NB]) {
+        const uint8_t* const rws = rraw + st * kRawTile + my_raw;
+        const bool live = (kt * 2 + h) * 32 < A.K;
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            uint32_t r[G::kRegs];
+            const uint32_t dl = P::delta(my_d0[n], kt);
+            P::fetch(rws + n * 32 * P::kRowBytes, h, dl, r);
+            const uint32_t sft = (dl + (uint32_t)h * 17u) & 3u;
+            const uint32_t e = (r[0] >> (8 * sft)) & 0xffu;
+            const bool wrap = sft == 3;
+            const uint32_t b0 = wrap ? r[1] : r[0], b1 = wrap ? r[2] : r[1], b2 = wrap ? r[3] : r[2];
+            const uint32_t b3 = wrap ? r[4] : r[3], b4 = r[4];
+            const uint32_t shb = (sft + 1) & 3;
+            // a block past the end of K: zeros under a scale of one (its bytes belong to the next row)
+            b[n][0] = live ? (int)__builtin_amdgcn_alignbyte(b1, b0, shb) : 0;
+            b[n][1] = live ? (int)__builtin_amdgcn_alignbyte(b2, b1, shb) : 0;
+            b[n][2] = live ? (int)__builtin_amdgcn_alignbyte(b3, b2, shb) : 0;
+            b[n][3] = live ? (int)__builtin_amdgcn_alignbyte(b4, b3, shb) : 0;
+            b[n][4] = b[n][5] = b[n][6] = b[n][7] = 0;
+            sb[n] = live ? (int)e : 127;
+        }
+    };
+    // A operands of 32-row block m: the two streams of the lane's block (24 bytes each) and its two scale bytes, kept in
+    // plain registers (an aggregate would live in scratch memory, whose loads share the counter of the copies)
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+#define TSHIP_MX_AOP(V) uint4_t V##_h0, V##_l0; uint2_t V##_h1, V##_l1; uint32_t V##_sa
+#define TSHIP_MX_LOAD_A(st, m, V)                                                              \
+    do {                                                                                       \
+        const uint8_t* const xr_ = xbuf + (st) * kXTile + (m) * 32 * kXRow;                     \
+        V##_h0 = *reinterpret_cast<const uint4_t*>(xr_ + a_main[0]);                           \
+        V##_h1 = *reinterpret_cast<const uint2_t*>(xr_ + a_rest[0]);                           \
+        V##_l0 = *reinterpret_cast<const uint4_t*>(xr_ + a_main[1]);                           \
+        V##_l1 = *reinterpret_cast<const uint2_t*>(xr_ + a_rest[1]);                           \
+        V##_sa = *reinterpret_cast<const uint32_t*>(xr_ + a_scale); /* byte 0: scale of hi, byte 1: of lo */ \
+    } while (0)
+#define TSHIP_MX_MULTIPLY(V, m, B, SB)                                                                                   \
+    do {                                                                                                                 \
+        const int8v_t ahi_ = {(int)V##_h0.x, (int)V##_h0.y, (int)V##_h0.z, (int)V##_h0.w, (int)V##_h1.x, (int)V##_h1.y, 0, 0}; \
+        const int8v_t alo_ = {(int)V##_l0.x, (int)V##_l0.y, (int)V##_l0.z, (int)V##_l0.w, (int)V##_l1.x, (int)V##_l1.y, 0, 0}; \
+        _Pragma("unroll") for (int n = 0; n < NB; ++n) {                                                                 \
+            acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ahi_, B[n], acc[m][n], 2, 4, 0, (int)V##_sa, 0, SB[n]); \
+            acc[m][n] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(alo_, B[n], acc[m][n], 2, 4, 1, (int)V##_sa, 0, SB[n]); \
+        }                                                                                                                \
+    } while (0)
+
+    // The operands of a row block are read while the block before it is multiplied, and the k-tile's barrier sits in
+    // front of its LAST row block: by then every operand of the k-tile is in registers, so behind the barrier the stage
+    // takes the copy ST k-tiles on and the first operands of the next k-tile are read under that last block's matrix
+    // instructions.  The LDS latency then never stands between two groups of matrix instructions.
+    int stage = 0;                                         // stage of k-tile kt
+#pragma unroll
+    for (int j = 0; j < ST - 1; ++j) issue(kt_begin + j, j);
+    wait_copies_and_barrier<(ST - 2) * (XI + RI)>();
+    issue_slot(kt_begin + ST - 1, ST - 1, 0);              // its other copies follow in the first k-tile of the loop
+    int8v_t b[NB], bn[NB];
+    int sb[NB], sbn[NB];
+    TSHIP_MX_AOP(a0);                                      // row blocks alternate between the two (TMW is even)
+    TSHIP_MX_AOP(a1);
+    load_b(kt_begin, 0, b, sb);
+    TSHIP_MX_LOAD_A(0, 0, a0);
+#define TSHIP_MX_KTILE(KT, B, SB, BNX, SBNX)                                                                              \
+    do {                                                                                                                 \
+        const int prev_ = stage == 0 ? ST - 1 : stage - 1;     /* the stage freed by the barrier of k-tile KT - 1 */     \
+        TSHIP_MX_LOAD_A(stage, 1, a1);                                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                               \
+        TSHIP_MX_MULTIPLY(a0, 0, B, SB);                                                                                 \
+        issue_slot((KT) - 1 + ST, prev_, 1);                                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                               \
+        if constexpr (TMW == 4) {                                                                                        \
+            TSHIP_MX_LOAD_A(stage, 2, a0);                                                                               \
+            __builtin_amdgcn_sched_barrier(0);                                                                           \
+            TSHIP_MX_MULTIPLY(a1, 1, B, SB);                                                                             \
+            issue_slot((KT) - 1 + ST, prev_, 2);                                                                         \
+            __builtin_amdgcn_sched_barrier(0);                                                                           \
+            TSHIP_MX_LOAD_A(stage, 3, a1);                                                                               \
+            __builtin_amdgcn_sched_barrier(0);                                                                           \
+            TSHIP_MX_MULTIPLY(a0, 2, B, SB);                                                                             \
+            issue_slot((KT) - 1 + ST, prev_, 3);                                                                         \
+            __builtin_amdgcn_sched_barrier(0);                                                                           \
+        }                                                                                                                \
+        const int next_ = stage == ST - 1 ? 0 : stage + 1;                                                               \
+        /* k-tile KT + 1 has landed once at most the copies of the ST - 2 k-tiles after it are in flight */              \
+        wait_copies_and_barrier<(ST - 2) * (XI + RI)>();                                                                 \
+        load_b((KT) + 1, next_, BNX, SBNX);                                                                              \
+        TSHIP_MX_LOAD_A(next_, 0, a0);                                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                               \
+        TSHIP_MX_MULTIPLY(a1, TMW - 1, B, SB);                                                                           \
+        issue_slot((KT) + ST, stage, 0);                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                               \
+        stage = next_;                                                                                                   \
+    } while (0)
+    for (int kt = kt_begin; kt < nkt; ++kt) {
+        TSHIP_MX_KTILE(kt, b, sb, bn, sbn);
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            b[n] = bn[n];
+            sb[n] = sbn[n];
+        }
+    }
+#undef TSHIP_MX_KTILE
+#undef TSHIP_MX_AOP
+#undef TSHIP_MX_LOAD_A
+#undef TSHIP_MX_MULTIPLY
+
+    // epilogue: D[row = 32 m + 8 (r / 4) + 4 h + r % 4][column] times the row scale
+    float* cdst = A.c;
+    int64_t ldc = A.ldc;
+    const int* c_rows = A.c_rows;
+    int accumulate = A.accumulate;
+    if (A.partial) {
+        cdst = A.partial + (int64_t)kc * A.M * A.N;
+        ldc = A.N;
+        c_rows = nullptr;
+        accumulate = 0;
+    }
+#pragma unroll
+    for (int m = 0; m < TMW; ++m) {
+        float sc[16];
+        int64_t off[16];
+#pragma unroll
+        for (int r2 = 0; r2 < 16; ++r2) {
+            const int ml = wm * (BM / 2) + m * 32 + 8 * (r2 >> 2) + 4 * h + (r2 & 3);
+            const int mr = m0 + min(ml, m_rows - 1);
+            sc[r2] = A.xscale[mr];
+            off[r2] = (int64_t)(c_rows ? c_rows[mr] : mr) * ldc;
+        }
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const int my_n = n0 + 32 * NB * wn + 32 * n + col;
+            if (my_n >= A.N) continue;
+#pragma unroll
+            for (int r2 = 0; r2 < 16; ++r2) {
+                const int ml = wm * (BM / 2) + m * 32 + 8 * (r2 >> 2) + 4 * h + (r2 & 3);
+                if (ml < m_rows) {
+                    float* pc = cdst + off[r2] + my_n;
+                    *pc = accumulate ? *pc + acc[m][n][r2] * sc[r2] : acc[m][n][r2] * sc[r2];
+                }
+            }
+        }
+    }
+}
+
+template <int BM>
+bool launch_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
+{
+    constexpr int BN = 256, ST = BM == 128 ? 5 : 3;
+    auto kern = gemm_mx_kernel<BM, ST>;
+    constexpr size_t kLds = (size_t)ST * BM * kXRow + (size_t)ST * BN * PMXFP4::kRowBytes + 1024;
+    static_assert(kLds <= 160 * 1024, "LDS");
+    if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), kLds)) return false;
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + BN - 1) / BN;
+    const int nkt = a.Kp / kBK;
+    a.k_chunks = 1;
+    a.chunk_kt = (nkt + 3) / 4 * 4;
+    a.partial = nullptr;
+    a.k_chunks = pick_k_chunks(a.m_tiles * a.n_tiles, nkt, device_info().num_cus, (int64_t)a.M * a.N, 1.7 * BM * BN / 65536.0);
+    if (a.k_chunks > 1) {
+        a.chunk_kt = ((nkt + a.k_chunks - 1) / a.k_chunks + 3) / 4 * 4;
+        a.k_chunks = (nkt + a.chunk_kt - 1) / a.chunk_kt;
+        const size_t need = (size_t)a.k_chunks * a.M * a.N * sizeof(float);
+        if (cs.need_out) *cs.need_out = need;
+        a.partial = chunk_scratch(cs, need);
+        if (!a.partial) {
+            a.k_chunks = 1;
+            a.chunk_kt = (nkt + 3) / 4 * 4;
+        }
+    }
+    if (cs.need_out) return true;
+    const int total = a.m_tiles * a.n_tiles * a.k_chunks;
+    const int grid = ((total + 7) / 8) * 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, a);
+    if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
+    if (a.partial) {
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
+                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
+        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+    }
+    return true;
+}
+
+// ------------------------------------------------------------------------------------------
 // At most 32 activation rows per tile (small batches, MoE experts with few tokens; also single rows of formats
 // without a GEMV kernel).  The activations stay in REGISTERS: the eight wavefronts of a workgroup split K between
 // them (KTW k-tiles each), every wavefront keeps the MFMA A operands of its K range for all 32 rows, and the
@@ -1486,7 +1922,7 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
         // MFMA A operands of this wavefront's K range: row `col`, k-half h of every k-step
         half8_t a[KTW][4];
         {
-            const _Float16* xr = A.x16 + (int64_t)(m0 + min(col, m_rows - 1)) * A.Kp + h * 8;
+            const _Float16* xr = A.x16 + (int64_t)(m0 + min(col, m_rows - 1)) * A.xld + h * 8;
             const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int t = 0; t < KTW; ++t) {
@@ -1698,6 +2134,12 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
         if (bm == 256) return launch_xw<PQ4K, 256, 4>(a, m_tiles, stream, cs);
         if (bm == 128) return launch_xw<PQ4K, 128, 4>(a, m_tiles, stream, cs);
     } else if constexpr (std::is_same<G, GMXFP4>::value) {
+        if (a.x_mx) {
+            if (bm == 256 && !a.tile_expert) return launch_mx<256>(a, m_tiles, stream, cs);
+            if (bm == 128 && !a.tile_expert) return launch_mx<128>(a, m_tiles, stream, cs);
+            set_last_error("gemm: the MX activation layout serves plain launches of 128- and 256-row tiles only.");
+            return false;
+        }
         if (bm == 256 && !a.tile_expert) return launch_xw<PMXFP4, 256, 4>(a, m_tiles, stream, cs);
         if (bm == 128 && !a.tile_expert) return launch_xw<PMXFP4, 128, 4>(a, m_tiles, stream, cs);
         if (bm == 128) return launch_tiles<G, 128, 2, 4>(a, m_tiles, stream, cs);
@@ -1717,10 +2159,20 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
 
 }  // namespace
 
+namespace {
+// Halfs between two rows of converted activations: the padded row length, plus one cache line when that length is an
+// even number of lines - rows at a stride of an even number of 128-byte lines fall on few of the L2's channels, and
+// the 32 CUs of an XCD read the same activation k-tile at the same time.
+int x_row_halfs(int K)
+{
+    const int kp = (K + kBK - 1) / kBK * kBK;
+    return kp;
+}
+}  // namespace
+
 size_t gemm_workspace_bytes(int M, int K)
 {
-    const size_t kp = (size_t)((K + kBK - 1) / kBK) * kBK;
-    return (size_t)M * kp * sizeof(_Float16) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255) + 256;
+    return (size_t)M * x_row_halfs(K) * sizeof(_Float16) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255) + 256;
 }
 
 // Rows of activations per tile for a plain (ungrouped) launch.  The 32-row register-resident kernel streams the
@@ -1771,19 +2223,28 @@ namespace {
 template <int TYPE, int SRC>
 void launch_convert_typed(const ConvertSrc& src, int M, int K, int kp, _Float16* x16, float* scales, hipStream_t stream)
 {
+    const int ldo = x_row_halfs(K);
     // short rows: 256 threads hold the whole row and eight workgroups share a CU
     if (K <= 256 * kCvtHold * 4)
-        hipLaunchKernelGGL((convert_x_kernel<TYPE, 256, SRC>), dim3(M), dim3(256), 0, stream, src, K, kp, x16, scales);
+        hipLaunchKernelGGL((convert_x_kernel<TYPE, 256, SRC>), dim3(M), dim3(256), 0, stream, src, K, kp, ldo, x16, scales);
     else
-        hipLaunchKernelGGL((convert_x_kernel<TYPE, 1024, SRC>), dim3(M), dim3(1024), 0, stream, src, K, kp, x16, scales);
+        hipLaunchKernelGGL((convert_x_kernel<TYPE, 1024, SRC>), dim3(M), dim3(1024), 0, stream, src, K, kp, ldo, x16, scales);
 }
 
 template <int SRC>
-bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspace, hipStream_t stream)
+bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspace, hipStream_t stream, int layout = 0)
 {
     const int kp = (K + kBK - 1) / kBK * kBK;
     float* scales = static_cast<float*>(workspace);
     _Float16* x16 = reinterpret_cast<_Float16*>(static_cast<char*>(workspace) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
+    if (layout == 1) {
+        if (type != kTypeMXFP4) {
+            set_last_error("gemm: the MX activation layout is for MXFP4 weights.");
+            return false;
+        }
+        launch_convert_typed<kXMx, SRC>(src, M, K, kp, x16, scales, stream);
+        return hip_ok(hipGetLastError(), "activation convert launch");
+    }
     // three activation orders: the K-quant nibble order, the split-nibble order of the 32-weight blocks, natural
     switch (type) {
     case kTypeQ4_K: case kTypeQ5_K: launch_convert_typed<kTypeQ4_K, SRC>(src, M, K, kp, x16, scales, stream); break;
@@ -1798,8 +2259,16 @@ bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspa
 
 }  // namespace
 
+// Which activation layout the GEMM of this shape reads: 0 fp16 in the format's unpack order; 1 two MX fp6 terms for
+// gemm_mx_kernel (plain MXFP4 launches on 128- or 256-row tiles).
+// (rows longer than the convert kernel holds in registers stay on the fp16 path)
+int gemm_x_layout(int type, int M, int N, int K)
+{
+    return type == kTypeMXFP4 && K <= 1024 * kCvtHold * 4 && gemm_tile_m(type, M, N) >= 128 ? 1 : 0;
+}
+
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
-                      hipStream_t stream, const float* norm_w, float eps)
+                      hipStream_t stream, const float* norm_w, float eps, int layout)
 {
     ConvertSrc src{};
     src.x = x;
@@ -1807,7 +2276,7 @@ bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map,
     src.row_map = row_map;
     src.norm_w = norm_w;
     src.eps = eps;
-    return launch_convert<kSrcPlain>(type, src, M, K, workspace, stream);
+    return launch_convert<kSrcPlain>(type, src, M, K, workspace, stream, layout);
 }
 
 bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, const int* expert_of, float alpha, float limit,
@@ -1825,7 +2294,8 @@ bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, 
 
 namespace {
 bool gemm_dispatch(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
-                   int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, const ChunkScratch& cs)
+                   int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, const ChunkScratch& cs,
+                   int x_layout)
 {
     if (w_bytes >= kMaxOperandBytes && !tiles) {
         set_last_error("gemm: a single weight of 2 GiB or more must be split by rows.");
@@ -1840,11 +2310,13 @@ bool gemm_dispatch(int type, const void* w, int64_t w_bytes, const void* workspa
     a.ldc = ldc;
     a.c_rows = c_rows;
     a.accumulate = accumulate ? 1 : 0;
+    a.x_mx = x_layout == 1 ? 1 : 0;
     a.M = M;
     a.N = N;
     a.K = K;
     a.Kp = (K + kBK - 1) / kBK * kBK;
-    a.x16_bytes = (int64_t)M * a.Kp * (int64_t)sizeof(_Float16);
+    a.xld = x_row_halfs(K);
+    a.x16_bytes = (int64_t)M * a.xld * (int64_t)sizeof(_Float16);
     if (a.x16_bytes >= kMaxOperandBytes) {
         set_last_error("gemm: the converted activations of one call must stay below 2 GiB; split the rows.");
         return false;
@@ -1881,10 +2353,10 @@ bool gemm_dispatch(int type, const void* w, int64_t w_bytes, const void* workspa
 
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc, const int* c_rows,
                  int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate, void* chunk_ws,
-                 size_t chunk_ws_bytes)
+                 size_t chunk_ws_bytes, int x_layout)
 {
     const ChunkScratch cs{static_cast<float*>(chunk_ws), chunk_ws ? chunk_ws_bytes : 0, nullptr};
-    return gemm_dispatch(type, w, w_bytes, workspace, c, ldc, c_rows, M, N, K, tiles, stream, accumulate, cs);
+    return gemm_dispatch(type, w, w_bytes, workspace, c, ldc, c_rows, M, N, K, tiles, stream, accumulate, cs, x_layout);
 }
 
 size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate)
@@ -1893,7 +2365,9 @@ size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles
     // a buffer "large enough" so that the launchers make the choices they would make with the reported bytes at hand
     const ChunkScratch cs{nullptr, ~(size_t)0, &need};
     const int64_t w_bytes = tiles ? 0 : (int64_t)(block_bytes(type) * (K / block_elems(type))) * N;
-    if (!gemm_dispatch(type, nullptr, w_bytes, nullptr, nullptr, N, nullptr, M, N, K, tiles, nullptr, accumulate, cs)) return 0;
+    if (!gemm_dispatch(type, nullptr, w_bytes, nullptr, nullptr, N, nullptr, M, N, K, tiles, nullptr, accumulate, cs,
+                       tiles ? 0 : gemm_x_layout(type, M, N, K)))
+        return 0;
     return need;
 }
 

@@ -141,7 +141,10 @@ int gemm_tile_m(int type, int M, int N);   // rows of activations per tile for a
 // row_map (device, optional) gathers source rows.
 // norm_w (device, optional) applies RMSNorm first: x <- x / sqrt(mean(x^2) + eps) * norm_w.
 bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map, int M, int K, void* workspace,
-                      hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f);
+                      hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f, int layout = 0);
+// layout of the converted activations the GEMM of this shape reads (plain launches): 0 fp16, 1 MX fp6 pairs (MXFP4 on the
+// block-scaled matrix instruction); pass it to launch_convert_x and to launch_gemm
+int gemm_x_layout(int type, int M, int N, int K);
 // The same for the activations of an expert's down projection: row m is SwiGLU-OAI of (gate | up)[m] (+ the bias
 // row of expert_of[m]), formed while it is read.
 bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, const int* expert_of, float alpha, float limit,
@@ -164,7 +167,7 @@ struct GemmTiles {
 // what is passed runs with whole K per tile, or fails when its kernel cannot do without chunks).  Nothing is allocated.
 bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace, float* c, int64_t ldc,
                  const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate = false,
-                 void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0);
+                 void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0, int x_layout = 0);
 // bytes of chunk_ws the same launch uses (0 for most shapes); only tiles->bm and tiles->count are read
 size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate);
 // the kernels address one weight (or one launch's converted activations) with 32-bit offsets
