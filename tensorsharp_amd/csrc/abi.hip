@@ -1397,6 +1397,10 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
         // rows per tile of the grouped GEMMs: up to about 160 tokens per expert the 32-row register-resident kernel
         // is fastest (measured at 32 experts of 2880 x 2880: T = 256 ... 1024), beyond that 128-row tiles
         const int per_expert = A / E;
+        // MXFP4 experts with few tokens run on the block-scaled matrix instruction (activations converted to MX fp6
+        // pairs, gemm_slim_mx_kernel)
+        const bool mx = ggml_type == kTypeMXFP4 && per_expert <= 160 && H <= 32768 && F <= 32768;
+        const int x_layout = mx ? 1 : 0;
         const int bm = per_expert > 160 ? 128 : 32;
         const int max_tiles = A / bm + E;
         // carve the workspace
@@ -1409,8 +1413,8 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
         const size_t o_gu = take((size_t)A * 2 * F * 4), o_dn = take((size_t)A * H * 4);
         const GemmTiles plan_tiles{nullptr, nullptr, nullptr, max_tiles, bm, 0};
         const size_t chunk_bytes = small ? 0
-                                         : std::max(gemm_chunk_ws_bytes(ggml_type, A, (int)(2 * F), (int)H, &plan_tiles, false),
-                                                    gemm_chunk_ws_bytes(ggml_type, A, (int)H, (int)F, &plan_tiles, false));
+                                         : std::max(gemm_chunk_ws_bytes(ggml_type, A, (int)(2 * F), (int)H, &plan_tiles, false, x_layout),
+                                                    gemm_chunk_ws_bytes(ggml_type, A, (int)H, (int)F, &plan_tiles, false, x_layout));
         const size_t o_chunk = take(chunk_bytes);
         WsLease lease(stream, off);
         if (!lease.ok()) return 0;
@@ -1445,16 +1449,17 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
                          reinterpret_cast<int*>(ws + o_trn)};
             if (!launch_moe_group(ids, A, k, E, bm, max_tiles, maps, stream)) return 0;
             GemmTiles tiles{maps.tile_expert, maps.tile_row0, maps.tile_rows, max_tiles, bm, gu_bytes};
-            if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream)) return 0;
+            if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream, nullptr, 0.f, x_layout))
+                return 0;
             if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream, false,
-                             ws + o_chunk, chunk_bytes))
+                             ws + o_chunk, chunk_bytes, x_layout))
                 return 0;
             // bias + SwiGLU-OAI are formed while the down projection's activations are converted
-            if (!launch_convert_x_swiglu(ggml_type, gu, gate_up_bias, maps.expert_of, alpha, limit, A, (int)F, ws + o_ws2, stream))
+            if (!launch_convert_x_swiglu(ggml_type, gu, gate_up_bias, maps.expert_of, alpha, limit, A, (int)F, ws + o_ws2, stream, x_layout))
                 return 0;
             tiles.expert_stride = dn_bytes;
             if (!launch_gemm(ggml_type, down_w, dn_bytes, ws + o_ws2, dn, H, nullptr, A, (int)H, (int)F, &tiles, stream, false,
-                             ws + o_chunk, chunk_bytes))
+                             ws + o_chunk, chunk_bytes, x_layout))
                 return 0;
             if (!launch_moe_combine(dn, down_bias, ids, weights, maps.pos_of, T, k, E, (int)H, false,
                                     static_cast<float*>(result.data), result.stride0, stream))

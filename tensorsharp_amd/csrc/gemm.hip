@@ -159,10 +159,19 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
         if (SRC == kSrcSwiglu) return swiglu_oai(src[k] + (bias ? bias[k] : 0.f), src[K + k] + (bias ? bias[K + k] : 0.f), S.alpha, S.limit);
         return src[k];
     };
+    // which float4 of the row register i holds: thread after thread, except for the MX layout, where a thread owns
+    // the pair (elements 4 t .. 4 t + 3 and the four 16 further on) of a 32-element block in registers 2 j, 2 j + 1
+    auto held = [&](int i) -> int {
+        if constexpr (TYPE == kXMx) {
+            const int pair = tid + (i >> 1) * THREADS;
+            return ((pair >> 2) << 3) + (pair & 3) + ((i & 1) << 2);
+        }
+        return tid + i * THREADS;
+    };
     float4 hold[kCvtHold];
 #pragma unroll
     for (int i = 0; i < kCvtHold; ++i) {
-        const int q = tid + i * THREADS;
+        const int q = held(i);
         hold[i] = q < k4 ? raw4(q) : float4{0.f, 0.f, 0.f, 0.f};
     }
     // optional RMSNorm prologue (ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1/sqrtf(mean + eps),
@@ -184,7 +193,7 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
         rms = 1.0f / sqrtf((float)(tot / (double)K) + S.eps);
 #pragma unroll
         for (int i = 0; i < kCvtHold; ++i) {
-            const int q = tid + i * THREADS;
+            const int q = held(i);
             if (q < k4) {
                 const float4 wv = reinterpret_cast<const float4*>(norm_w)[q];
                 hold[i] = float4{(hold[i].x * rms) * wv.x, (hold[i].y * rms) * wv.y, (hold[i].z * rms) * wv.z, (hold[i].w * rms) * wv.w};
@@ -230,103 +239,110 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
             return eb < 1 ? 1 : eb;                                            // at most 253: 2^(254 - eb) is a normal float
         };
         auto pow2 = [](int biased) { return __uint_as_float((uint32_t)biased << 23); };      // biased 1..254
-        // E2M3 code of v (|v| <= 7.75): codes 0..16 step 1/8, 16..24 step 1/4, 24..31 step 1/2; sign in bit 5
+        // E2M3 code of v (|v| < 7.75).  From 1.0 up the code is the float's exponent and top three mantissa bits (rounded
+        // by the add, the carry running into the exponent); below 1.0 it counts eighths.  Sign in bit 5.
         auto enc = [](float v) -> uint32_t {
-            const float mag = fabsf(v);
-            const float c = mag < 2.f ? mag * 8.f : mag < 4.f ? 16.f + (mag - 2.f) * 4.f : 24.f + (mag - 4.f) * 2.f;
-            uint32_t code = (uint32_t)__builtin_rintf(c);
+            const uint32_t u = __float_as_uint(v), mag = u & 0x7fffffffu;
+            const uint32_t normal = ((mag + 0x80000u) >> 20) - (126u << 3);
+            const uint32_t small = (uint32_t)(__uint_as_float(mag) * 8.f + 0.5f);
+            uint32_t code = mag >= 0x3f800000u ? normal : small;
             code = code > 31u ? 31u : code;
-            return code | (v < 0.f ? 32u : 0u);
+            return code | ((u >> 26) & 32u);
         };
         auto dec = [](uint32_t code) -> float {
             const uint32_t c = code & 31u;
-            const float mag = c < 16u ? (float)c * 0.125f : c < 24u ? 2.f + (float)(c - 16u) * 0.25f : 4.f + (float)(c - 24u) * 0.5f;
+            const float mag = c >= 8u ? __uint_as_float((c + (126u << 3)) << 20) : (float)c * 0.125f;
             return (code & 32u) ? -mag : mag;
         };
-        // where byte b (0..23) of the stream of term p, block g lives inside the row's k-tile
-        auto stream_off = [](int p, int g, int b) { return b < 16 ? (3 * p + 2 * g) * 16 + b : (3 * p + 1) * 16 + 8 * g + (b - 16); };
-        constexpr int kIters = kCvtHold;
+        auto max4 = [](const float4& v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); };
+        // eight fields e0 o0 e1 o1 e2 o2 e3 o3 -> the low four bytes and the last two of the thread's six
+        auto weave = [](const uint32_t (&e)[4], const uint32_t (&o)[4], uint32_t& low, uint32_t& high) {
+            low = e[0] | (o[0] << 6) | (e[1] << 12) | (o[1] << 18) | (e[2] << 24) | (o[2] << 30);
+            high = (o[2] >> 2) | (e[3] << 4) | (o[3] << 10);
+        };
 #pragma unroll
-        for (int i = 0; i < kIters; ++i) {
-            if (i * THREADS >= k4) break;                          // uniform: whole passes beyond the row
-            const int q = tid + i * THREADS;                       // lanes past the row hold zeros and take part
-            const float4 v = hold[i];
-            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        for (int i = 0; i < kCvtHold; i += 2) {
+            if ((i >> 1) * THREADS * 2 >= k4) break;               // uniform: whole passes beyond the row
+            const int pair = tid + (i >> 1) * THREADS;             // threads past the row hold zeros and take part
+            const float4 va = hold[i], vb = hold[i + 1];           // fields 8 t .. 8 t + 7 of the block: va even, vb odd
+            float amax = fmaxf(max4(va), max4(vb));
             amax = fmaxf(amax, __shfl_xor(amax, 1));
             amax = fmaxf(amax, __shfl_xor(amax, 2));
-            amax = fmaxf(amax, __shfl_xor(amax, 4));
-            if (!(amax == amax)) amax = __uint_as_float(0x7f800000u);
             {
                 // a NaN anywhere in the block must reach the maximum (fmaxf drops NaNs)
-                const bool nan = (v.x != v.x) || (v.y != v.y) || (v.z != v.z) || (v.w != v.w);
+                const bool nan = (va.x != va.x) || (va.y != va.y) || (va.z != va.z) || (va.w != va.w) || (vb.x != vb.x) ||
+                                 (vb.y != vb.y) || (vb.z != vb.z) || (vb.w != vb.w);
                 const unsigned long long any = __ballot(nan);
-                if ((any >> ((threadIdx.x & 63) & ~7)) & 0xffull) amax = __uint_as_float(0x7f800000u);
+                if ((any >> ((threadIdx.x & 63) & ~3)) & 0xfull) amax = __uint_as_float(0x7f800000u);
             }
             const int eh = block_exp(amax);
             const bool finite = eh != 255;
             const float inv_h = finite ? pow2(254 - eh) : 0.f, sc_h = finite ? pow2(eh) : 0.f;
-            const uint32_t h0 = enc(v.x * inv_h), h1 = enc(v.y * inv_h), h2 = enc(v.z * inv_h), h3 = enc(v.w * inv_h);
-            const float r0 = finite ? v.x - dec(h0) * sc_h : 0.f, r1 = finite ? v.y - dec(h1) * sc_h : 0.f;
-            const float r2 = finite ? v.z - dec(h2) * sc_h : 0.f, r3 = finite ? v.w - dec(h3) * sc_h : 0.f;
-            float rmax = fmaxf(fmaxf(fabsf(r0), fabsf(r1)), fmaxf(fabsf(r2), fabsf(r3)));
+            const float xa[4] = {va.x, va.y, va.z, va.w}, xb[4] = {vb.x, vb.y, vb.z, vb.w};
+            uint32_t ha[4], hb[4], la[4], lb[4];
+            float ra[4], rb[4];
+            float rmax = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                ha[j] = enc(xa[j] * inv_h);
+                hb[j] = enc(xb[j] * inv_h);
+                ra[j] = finite ? xa[j] - dec(ha[j]) * sc_h : 0.f;
+                rb[j] = finite ? xb[j] - dec(hb[j]) * sc_h : 0.f;
+                rmax = fmaxf(rmax, fmaxf(fabsf(ra[j]), fabsf(rb[j])));
+            }
             rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
             rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
-            rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
             const int el = block_exp(rmax);
             const float inv_l = pow2(254 - el);
-            const uint32_t l0 = enc(r0 * inv_l), l1 = enc(r1 * inv_l), l2 = enc(r2 * inv_l), l3 = enc(r3 * inv_l);
-            // the lane four to the right (left) holds the elements 16 further on (back): together they own fields
-            // 8 t .. 8 t + 7 of the stream (t = lane % 4), six bytes; each lane packs all eight codes
-            const uint32_t mine_h = h0 | (h1 << 6) | (h2 << 12) | (h3 << 18), mine_l = l0 | (l1 << 6) | (l2 << 12) | (l3 << 18);
-            const uint32_t other_h = __shfl_xor(mine_h, 4), other_l = __shfl_xor(mine_l, 4);
-            const bool upper = (q & 4) != 0;
-            const uint32_t even_h = upper ? other_h : mine_h, odd_h = upper ? mine_h : other_h;
-            const uint32_t even_l = upper ? other_l : mine_l, odd_l = upper ? mine_l : other_l;
-            auto weave = [](uint32_t ev, uint32_t od) -> unsigned long long {      // fields e0 o0 e1 o1 e2 o2 e3 o3
-                unsigned long long w = 0;
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    w |= (unsigned long long)((ev >> (6 * j)) & 63u) << (12 * j) | (unsigned long long)((od >> (6 * j)) & 63u) << (12 * j + 6);
-                return w;
-            };
-            const unsigned long long wh = weave(even_h, odd_h), wl = weave(even_l, odd_l);
-            const int k0 = 4 * (q & ~4);                           // first element of the lower lane of the pair
-            const int g = (k0 >> 5) & 1, t4 = (k0 & 15) >> 2;      // block of the k-tile, quarter of the stream
-            uint8_t* const row = d8 + (k0 >> 6) * 128;
-            // the four lower lanes of a block assemble the hi stream, the four upper lanes the lo stream: lane t4 holds
-            // bytes 6 t4 .. 6 t4 + 5 and fetches the lane after it for the dwords that straddle two lanes
-            const unsigned long long w = upper ? wl : wh;
-            const uint32_t w_lo = (uint32_t)w, w_hi = (uint32_t)(w >> 32);
-            const uint32_t nb_lo = __shfl_down(w_lo, 1);
-            const int p = upper ? 1 : 0;
-            if (q < k4) {
+            for (int j = 0; j < 4; ++j) {
+                la[j] = enc(ra[j] * inv_l);
+                lb[j] = enc(rb[j] * inv_l);
+            }
+            uint32_t w_lo[2], w_hi[2];
+            weave(ha, hb, w_lo[0], w_hi[0]);
+            weave(la, lb, w_lo[1], w_hi[1]);
+            const int t4 = pair & 3, blk = pair >> 2;              // quarter of the stream, block of the row
+            const int g = blk & 1;
+            uint8_t* const row = d8 + (blk >> 1) * 128;
+            const bool inside = 2 * pair < k4;                     // the pair's block lies inside the row
+            // thread t4 holds bytes 6 t4 .. 6 t4 + 5 of either stream and fetches the thread after it for the dwords
+            // that straddle two threads
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const uint32_t nb_lo = __shfl_down(w_lo[p], 1);
                 uint8_t* const main_piece = row + (3 * p + 2 * g) * 16;
                 uint8_t* const rest_piece = row + (3 * p + 1) * 16 + 8 * g;
-                const uint32_t straddle = (w_hi & 0xffffu) | (nb_lo << 16);       // bytes 4, 5 of this lane, 0, 1 of the next
-                const uint32_t upper4 = (w_lo >> 16) | (w_hi << 16);              // bytes 2 .. 5 of this lane
-                if (t4 == 0) {
-                    uint2 v2;
-                    v2.x = w_lo;
-                    v2.y = straddle;
-                    *reinterpret_cast<uint2*>(main_piece) = v2;
-                    if (!upper) *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = (uint32_t)eh | ((uint32_t)el << 8);
-                } else if (t4 == 1) {
-                    *reinterpret_cast<uint32_t*>(main_piece + 8) = upper4;
-                } else if (t4 == 2) {
-                    *reinterpret_cast<uint32_t*>(main_piece + 12) = w_lo;
-                    *reinterpret_cast<uint32_t*>(rest_piece) = straddle;
-                } else {
-                    *reinterpret_cast<uint32_t*>(rest_piece + 4) = upper4;
+                const uint32_t straddle = (w_hi[p] & 0xffffu) | (nb_lo << 16);    // bytes 4, 5 of this thread, 0, 1 of the next
+                const uint32_t upper4 = (w_lo[p] >> 16) | (w_hi[p] << 16);        // bytes 2 .. 5 of this thread
+                if (inside) {
+                    if (t4 == 0) {
+                        uint2 v2;
+                        v2.x = w_lo[p];
+                        v2.y = straddle;
+                        *reinterpret_cast<uint2*>(main_piece) = v2;
+                    } else if (t4 == 1) {
+                        *reinterpret_cast<uint32_t*>(main_piece + 8) = upper4;
+                    } else if (t4 == 2) {
+                        *reinterpret_cast<uint32_t*>(main_piece + 12) = w_lo[p];
+                        *reinterpret_cast<uint32_t*>(rest_piece) = straddle;
+                    } else {
+                        *reinterpret_cast<uint32_t*>(rest_piece + 4) = upper4;
+                    }
                 }
             }
+            if (inside && t4 == 0) *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = (uint32_t)eh | ((uint32_t)el << 8);
         }
         // blocks past K inside the last k-tile: zero streams under a scale of one
         for (int blk = (K >> 5) + tid; blk < (Kp >> 5); blk += THREADS) {
             uint8_t* const row = d8 + (blk >> 1) * 128;
             const int g = blk & 1;
-            for (int bb = 0; bb < 24; bb += 2) {
-                *reinterpret_cast<uint16_t*>(row + stream_off(0, g, bb)) = 0;
-                *reinterpret_cast<uint16_t*>(row + stream_off(1, g, bb)) = 0;
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                uint32_t* const main_piece = reinterpret_cast<uint32_t*>(row + (3 * p + 2 * g) * 16);
+                uint32_t* const rest_piece = reinterpret_cast<uint32_t*>(row + (3 * p + 1) * 16 + 8 * g);
+                main_piece[0] = main_piece[1] = main_piece[2] = main_piece[3] = 0u;
+                rest_piece[0] = rest_piece[1] = 0u;
             }
             *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = 127u | (127u << 8);
         }
@@ -2087,6 +2103,293 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch
     return true;
 }
 
+// ------------------------------------------------------------------------------------------
+// The register-resident kernel for MXFP4 on the block-scaled matrix instruction (see gemm_mx_kernel): the activations
+// of the wavefront's K range stay in registers as MX fp6 pairs (12.5 registers per k-tile and 32-row block, where fp16
+// operands take 16), the raw weight blocks of the ring buffers are the B operands as they are, and the pair of
+// instructions per k-tile costs half of the four fp16 ones.  RB row blocks per unit: 1 is what the launcher uses.
+// (RB = 2, 64-row units for the matrix time of one 32-row fp16 unit, so that an expert with 33 .. 64 tokens streams its
+// weights once, is correct but no faster: its 8 KB of partial sums per wavefront leave room for a ring of two buffers
+// only, and a unit's time is the wavefronts' LDS-direct copies and the two barriers, not the matrix instructions -
+// 200.8 vs 200.6 us for the 256-token GPT-OSS expert stage.)
+// ------------------------------------------------------------------------------------------
+template <int KTW, int RB>
+struct SlimMxLayout {
+    static constexpr int kNeed = (GMXFP4::window_bytes(KTW) + 15) / 16;
+    static constexpr int CH = kNeed | 1;                                 // odd: the dword reads of the 32 rows spread over the banks
+    static constexpr int DI = (32 * CH + 63) / 64;
+    static constexpr int RAW = 32 * CH * 16;
+    static constexpr int BUF = RAW > RB * 4096 ? RAW : RB * 4096;        // raw rows, later RB x 32 x 32 fp32 partial sums
+    static constexpr int RING = 8 * 3 * BUF + 1024 <= 160 * 1024 ? 3 : 2;
+};
+
+template <int KTW, int RB>
+__global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
+{
+    typedef GMXFP4 G;
+    using L = SlimMxLayout<KTW, RB>;
+    constexpr int CH = L::CH, DI = L::DI, BUF = L::BUF, RING = L::RING;
+    constexpr int NQ = 2 * RB;                                          // results per thread in the reduction
+    static_assert(KTW % G::kTileStep == 0, "a wavefront's K range must start at a block");
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+    extern __shared__ uint8_t smem[];                                   // 8 wavefronts x RING x BUF
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, h = lane >> 5;
+    uint8_t* const my_buf = smem + wave * RING * BUF;
+
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int nkt = A.Kp / kBK;
+    const int n32 = (A.N + 31) >> 5;
+    const int per_tile = A.k_chunks * n32;                              // units of one row tile
+
+    int live_tiles = A.m_tiles;
+    if (A.tile_expert) {
+        int c = 0;
+        for (int i = lane; i < A.m_tiles; i += 64) c += A.tile_rows[i] > 0 ? 1 : 0;
+        for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+        live_tiles = __builtin_amdgcn_readfirstlane(c);
+    }
+    const int64_t units = (int64_t)live_tiles * per_tile;
+    int u = (int)(units * blockIdx.x / gridDim.x);
+    const int u_end = (int)(units * (blockIdx.x + 1) / gridDim.x);
+
+    while (u < u_end) {
+        const int mt = u / per_tile, rem = u - mt * per_tile;
+        const int kc = rem / n32, nt0 = rem - kc * n32, cnt = min(n32 - nt0, u_end - u);
+        u += cnt;
+        const int kt0 = kc * A.chunk_kt + wave * KTW;
+        const int kcnt = max(0, min(KTW, nkt - kt0));                  // k-tiles of this wavefront in this chunk
+        int m0, m_rows;
+        const uint8_t* wbase = A.w;
+        if (A.tile_expert) {
+            m0 = A.tile_row0[mt];
+            m_rows = min(32 * RB, A.tile_rows[mt]);
+            wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+        } else {
+            m0 = mt * 32 * RB;
+            m_rows = min(32 * RB, A.M - m0);
+        }
+        const int rbs = RB > 1 && m_rows > 32 ? RB : 1;                // row blocks with rows in them (uniform)
+        const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
+        const uint32_t base_delta = (uint32_t)(wa & 3);
+        const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+            reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
+
+        // A operands of this wavefront's K range: row col + 32 rb, block h of every k-tile - the two 24-byte streams
+        // and the scale dword (layout of convert_x_kernel<kXMx>)
+        uint4_t ah0[KTW][RB], al0[KTW][RB];
+        uint2_t ah1[KTW][RB], al1[KTW][RB];
+        uint32_t asa[KTW / 2][RB];                 // scale bytes (hi, lo) of k-tile 2 j in bytes 0, 1 and of 2 j + 1 in bytes 2, 3
+        // (range-checked loads: rows past the tile and k-tiles past the wavefront's range read zeros - zero fields
+        // under the smallest scale - without a select per register)
+        const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int ml = col + 32 * rb;
+            const uint32_t xrow = (uint32_t)(m0 + min(ml, m_rows - 1)) * (uint32_t)(A.xld * 2);
+#pragma unroll
+            for (int t = 0; t < KTW; ++t) {
+                const bool on = ml < m_rows && t < kcnt;
+                const uint32_t xt = on ? xrow + (uint32_t)(kt0 + t) * 128u : kDeadOffset;
+                const uint4_t vh0 = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (uint32_t)(2 * h) * 16u), 0, 0);
+                const uint4_t vl0 = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (uint32_t)(3 + 2 * h) * 16u), 0, 0);
+                ah0[t][rb] = vh0;
+                al0[t][rb] = vl0;
+                ah1[t][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 16u + 8u * (uint32_t)h), 0, 0);
+                al1[t][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 64u + 8u * (uint32_t)h), 0, 0);
+                const uint32_t two = __builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(xt + 96u + 4u * (uint32_t)h), 0, 0) & 0xffffu;
+                if (t & 1) asa[t >> 1][rb] |= two << 16;
+                else asa[t >> 1][rb] = two;
+            }
+        }
+        const uint32_t koff = G::tile_offset(kt0);
+        uint32_t w_off[DI];
+#pragma unroll
+        for (int i = 0; i < DI; ++i) {
+            const int q = i * 64 + lane;
+            const int row = q / CH, chunk = q - row * CH;
+            w_off[i] = (row < 32 && kcnt > 0) ? ((base_delta + (uint32_t)row * row_bytes + koff) & ~3u) + (uint32_t)chunk * 16u : kDeadOffset;
+        }
+        const uint32_t my_delta = (base_delta + (uint32_t)col * row_bytes + koff) & 3u;
+        // copy q of column tile nt0 + i -> buffer b
+        auto issue_one = [&](int i, int b, int q) {
+            const bool any = i < cnt;
+            const uint32_t so = any ? (uint32_t)(nt0 + i) * 32u * row_bytes : 0u;
+            if (q * 64 + 32 < 32 * CH || lane < 32) copy16_to_lds(wrs, my_buf + b * BUF + q * 1024, any ? w_off[q] : kDeadOffset, so);
+        };
+        auto issue = [&](int i, int b) {
+#pragma unroll
+            for (int q = 0; q < DI; ++q) issue_one(i, b, q);
+        };
+        // With three buffers the refill of a buffer waits for the NEXT unit and goes out copy by copy behind the matrix
+        // instructions of its k-tiles (copy q behind k-tile q % KTW): a copy keeps the wavefront busy for tens of
+        // cycles, and there the matrix pipe has work queued for that long.
+        constexpr bool kDefer = RING >= 3;
+        // results of this thread in the reduction: accumulator registers wave + 8 q of the RB x 16
+        int64_t coff[NQ];
+        bool ok[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int rr = wave + 8 * q, r = rr & 15;
+            const int ml = 32 * (rr >> 4) + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int m = m0 + min(ml, m_rows - 1);
+            coff[q] = A.partial ? ((int64_t)kc * A.M + m) * A.N : (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
+            ok[q] = ml < m_rows;
+        }
+
+#pragma unroll
+        for (int b = 0; b < RING; ++b) issue(b, b);
+        int b = 0;                                      // buffer of column tile i
+        float pend[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) pend[q] = 0.f;
+        int pend_n = -1;
+        float* const dst = A.partial ? A.partial : A.c;
+        auto flush = [&]() {
+            if (pend_n >= 0 && pend_n < A.N) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q)
+                    if (ok[q]) dst[coff[q] + pend_n] = pend[q];
+            }
+        };
+        for (int i = 0; i < cnt; ++i) {
+            // the copies of tile i have landed; those of the tiles after it stay in flight (deferred refills: the tile
+            // RING - 1 on is only issued during this unit)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kDefer ? RING - 2 : RING - 1) * DI) : "memory");
+            flush();
+            const int b_prev = b == 0 ? RING - 1 : b - 1;      // the buffer of tile i - 1
+            float16_t acc[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
+            const uint8_t* raw = my_buf + b * BUF + col * (CH * 16);
+            // the raw block of k-tile t + 1 is fetched from LDS while k-tile t is multiplied; the fences keep the compiler
+            // from fetching every k-tile up front (the A operands leave few registers)
+            auto k_tiles = [&](auto full_tag) {
+                constexpr bool kFull = decltype(full_tag)::value;
+                uint32_t r[KTW + 1][G::kRegs];
+                G::fetch(raw, 0, h, my_delta, r[0]);
+#pragma unroll
+                for (int t = 0; t < KTW; ++t) {
+                    if (t + 1 < KTW) G::fetch(raw, t + 1, h, my_delta, r[t + 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (kFull || t < kcnt) {
+                        // the lane's raw block of k-tile t: sixteen bytes of nibbles re-aligned, and its scale byte
+                        const uint32_t sft = (my_delta + (uint32_t)(2 * t + h) * 17u) & 3u;
+                        const uint32_t e = (r[t][0] >> (8 * sft)) & 0xffu;
+                        const bool wrap = sft == 3;
+                        const uint32_t b0 = wrap ? r[t][1] : r[t][0], b1 = wrap ? r[t][2] : r[t][1], b2 = wrap ? r[t][3] : r[t][2];
+                        const uint32_t b3 = wrap ? r[t][4] : r[t][3], b4 = r[t][4];
+                        const uint32_t shb = (sft + 1) & 3;
+                        const bool live = ((kt0 + t) * 2 + h) * 32 < A.K;
+                        const int8v_t bq = {live ? (int)__builtin_amdgcn_alignbyte(b1, b0, shb) : 0, live ? (int)__builtin_amdgcn_alignbyte(b2, b1, shb) : 0,
+                                            live ? (int)__builtin_amdgcn_alignbyte(b3, b2, shb) : 0, live ? (int)__builtin_amdgcn_alignbyte(b4, b3, shb) : 0,
+                                            0, 0, 0, 0};
+                        const int sbq = live ? (int)e : 127;
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb) {
+                            if (rb < rbs) {
+                                const int8v_t ahi = {(int)ah0[t][rb].x, (int)ah0[t][rb].y, (int)ah0[t][rb].z, (int)ah0[t][rb].w,
+                                                     (int)ah1[t][rb].x, (int)ah1[t][rb].y, 0, 0};
+                                const int8v_t alo = {(int)al0[t][rb].x, (int)al0[t][rb].y, (int)al0[t][rb].z, (int)al0[t][rb].w,
+                                                     (int)al1[t][rb].x, (int)al1[t][rb].y, 0, 0};
+                                const int sa2 = (int)asa[t >> 1][rb];
+                                if (t & 1) {
+                                    acc[rb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ahi, bq, acc[rb], 2, 4, 2, sa2, 0, sbq);
+                                    acc[rb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(alo, bq, acc[rb], 2, 4, 3, sa2, 0, sbq);
+                                } else {
+                                    acc[rb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ahi, bq, acc[rb], 2, 4, 0, sa2, 0, sbq);
+                                    acc[rb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(alo, bq, acc[rb], 2, 4, 1, sa2, 0, sbq);
+                                }
+                            }
+                        }
+                    }
+                    if (kDefer && i > 0) {
+#pragma unroll
+                        for (int q = t; q < DI; q += KTW) issue_one(i - 1 + RING, b_prev, q);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            if (kcnt == KTW) k_tiles(std::true_type{});
+            else k_tiles(std::false_type{});
+            // partial sums of this wavefront's K range -> the buffer it has just consumed
+            float* part = reinterpret_cast<float*>(my_buf + b * BUF);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part[(rb * 16 + r) * 64 + lane] = acc[rb][r];
+            lds_barrier();
+            float s[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) s[q] = 0.f;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float* pv = reinterpret_cast<const float*>(smem + (v * RING + b) * BUF);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) s[q] += pv[(wave + 8 * q) * 64 + lane];
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) pend[q] = s[q];      // the row scale of this activation layout is one
+            pend_n = (nt0 + i) * 32 + col;
+            lds_barrier();                              // every partial sum has been read: the buffers may be refilled
+            if (!kDefer) issue(i + RING, b);
+            b = b + 1 == RING ? 0 : b + 1;
+        }
+        flush();
+    }
+}
+
+template <int KTW, int RB>
+bool launch_slim_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
+{
+    using L = SlimMxLayout<KTW, RB>;
+    auto kern = gemm_slim_mx_kernel<KTW, RB>;
+    constexpr size_t lds = (size_t)8 * L::RING * L::BUF + 64;
+    static_assert(lds <= 160 * 1024, "raw buffers must fit LDS");
+    if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + 31) / 32;
+    a.chunk_kt = 8 * KTW;
+    a.k_chunks = (a.Kp / kBK + a.chunk_kt - 1) / a.chunk_kt;
+    a.partial = nullptr;
+    const bool two_pass = a.k_chunks > 1 || a.accumulate;
+    if (two_pass) {
+        const size_t need = (size_t)a.k_chunks * a.M * a.N * sizeof(float);
+        if (cs.need_out) *cs.need_out = need;
+        a.partial = chunk_scratch(cs, need);
+        if (!a.partial && !cs.need_out) {
+            set_last_error("gemm: the K-chunk sums of this shape do not fit the scratch buffer.");
+            return false;
+        }
+    }
+    if (cs.need_out) return true;
+    const int64_t units = (int64_t)m_tiles * a.k_chunks * a.n_tiles;
+    const int grid = (int)std::min<int64_t>(units, device_info().num_cus);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
+    if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
+    if (two_pass) {
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial, a.k_chunks, a.M, a.N,
+                           a.c_rows, a.c, a.ldc, a.accumulate);
+        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+    }
+    return true;
+}
+
+// k-tiles per wavefront of the MX register-resident kernel: 2, 4 or 6 (75 registers of A operands at 6), a longer K in
+// chunks
+template <int RB>
+bool launch_slim_mx_for(const GemmArgs& a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
+{
+    const int need = (a.Kp / kBK + 7) / 8;
+    if (need <= 2) return launch_slim_mx<2, RB>(a, m_tiles, stream, cs);
+    if (need <= 4) return launch_slim_mx<4, RB>(a, m_tiles, stream, cs);
+    return launch_slim_mx<6, RB>(a, m_tiles, stream, cs);
+}
+
 // k-tiles per wavefront of the register-resident kernel: a multiple of the format's block step, at most what two
 // raw buffers per wavefront fit into LDS; a longer K is cut into chunks of 8 x that many k-tiles
 template <typename G, int KTW>
@@ -2126,7 +2429,7 @@ constexpr bool kWide128 = G::kSup == 2 || G::kRawRow > 144 || std::is_same<G, GQ
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
-    if (bm == 32) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream, cs);
+    if (bm == 32 && !a.x_mx) return launch_slim_for<G>(a, slim_ktw<G>(a.Kp / kBK), m_tiles, stream, cs);
     // Q4_K and MXFP4: the 2 x 4 wavefront layout with the operand exchange through LDS (gemm_xw_kernel); 128-row tiles are
     // 128 x 256.  Q4_K takes it for every launch, MXFP4 for plain ones: the MXFP4 expert tiles of a MoE prefill (128
     // rows) stay on two 128 x 128 workgroups per CU (926 vs 968 us at 2048 tokens).
@@ -2137,7 +2440,8 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
         if (a.x_mx) {
             if (bm == 256 && !a.tile_expert) return launch_mx<256>(a, m_tiles, stream, cs);
             if (bm == 128 && !a.tile_expert) return launch_mx<128>(a, m_tiles, stream, cs);
-            set_last_error("gemm: the MX activation layout serves plain launches of 128- and 256-row tiles only.");
+            if (bm == 32) return launch_slim_mx_for<1>(a, m_tiles, stream, cs);
+            set_last_error("gemm: the MX activation layout serves 32-row units and plain launches of 128- and 256-row tiles.");
             return false;
         }
         if (bm == 256 && !a.tile_expert) return launch_xw<PMXFP4, 256, 4>(a, m_tiles, stream, cs);
@@ -2280,7 +2584,7 @@ bool launch_convert_x(int type, const float* x, int64_t ldx, const int* row_map,
 }
 
 bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, const int* expert_of, float alpha, float limit,
-                             int M, int F, void* workspace, hipStream_t stream)
+                             int M, int F, void* workspace, hipStream_t stream, int layout)
 {
     ConvertSrc src{};
     src.x = gate_up;
@@ -2289,7 +2593,7 @@ bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, 
     src.expert_of = expert_of;
     src.alpha = alpha;
     src.limit = limit;
-    return launch_convert<kSrcSwiglu>(type, src, M, F, workspace, stream);
+    return launch_convert<kSrcSwiglu>(type, src, M, F, workspace, stream, layout);
 }
 
 namespace {
@@ -2359,14 +2663,14 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
     return gemm_dispatch(type, w, w_bytes, workspace, c, ldc, c_rows, M, N, K, tiles, stream, accumulate, cs, x_layout);
 }
 
-size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate)
+size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate, int x_layout)
 {
     size_t need = 0;
     // a buffer "large enough" so that the launchers make the choices they would make with the reported bytes at hand
     const ChunkScratch cs{nullptr, ~(size_t)0, &need};
     const int64_t w_bytes = tiles ? 0 : (int64_t)(block_bytes(type) * (K / block_elems(type))) * N;
     if (!gemm_dispatch(type, nullptr, w_bytes, nullptr, nullptr, N, nullptr, M, N, K, tiles, nullptr, accumulate, cs,
-                       tiles ? 0 : gemm_x_layout(type, M, N, K)))
+                       x_layout >= 0 ? x_layout : tiles ? 0 : gemm_x_layout(type, M, N, K)))
         return 0;
     return need;
 }

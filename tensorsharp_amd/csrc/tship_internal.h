@@ -148,7 +148,7 @@ int gemm_x_layout(int type, int M, int N, int K);
 // The same for the activations of an expert's down projection: row m is SwiGLU-OAI of (gate | up)[m] (+ the bias
 // row of expert_of[m]), formed while it is read.
 bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, const int* expert_of, float alpha, float limit,
-                             int M, int F, void* workspace, hipStream_t stream);
+                             int M, int F, void* workspace, hipStream_t stream, int layout = 0);
 
 // Grouped launches (MoE): m-tiles enumerated by device tables; weights of expert e start at
 // w + e * expert_stride and span w_bytes each.
@@ -169,7 +169,7 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
                  const int* c_rows, int M, int N, int K, const GemmTiles* tiles, hipStream_t stream, bool accumulate = false,
                  void* chunk_ws = nullptr, size_t chunk_ws_bytes = 0, int x_layout = 0);
 // bytes of chunk_ws the same launch uses (0 for most shapes); only tiles->bm and tiles->count are read
-size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate);
+size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate, int x_layout = -1);
 // the kernels address one weight (or one launch's converted activations) with 32-bit offsets
 constexpr int64_t kMaxOperandBytes = ((int64_t)1 << 31) - 64;
 

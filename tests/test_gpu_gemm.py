@@ -225,6 +225,53 @@ def test_128_row_tiles(hip, oracle, name, M, N, K):
     check(y, oracle.matmul_f64(T[name], wq, N, K, x), (name, M, N, K))
 
 
+# ---- plain MXFP4 launches of 128- / 256-row tiles: the block-scaled matrix instruction, activations as two MX fp6 terms ----
+@pytest.mark.parametrize("M,N,K", [(300, 520, 32 * 33),      # odd block count: half of the last k-tile is past K
+                                   (700, 1500, 2880),        # 256-row tiles, ragged last tile in both directions
+                                   (257, 300, 64),           # a single k-tile
+                                   (1030, 264, 4096 + 32)])
+def test_mxfp4_block_scaled_tiles(hip, oracle, M, N, K):
+    rng = np.random.default_rng(M + 3 * N + K)
+    wq = oracle.quantize(MXFP4, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    check(run_device(hip, MXFP4, wq, N, K, x), oracle.matmul_f64(MXFP4, wq, N, K, x), ("mx", M, N, K))
+
+
+def test_mxfp4_block_scaled_dynamic_range(hip, oracle):
+    """Every 32-element block of the activations has its own magnitude (2^-40 .. 2^40), some blocks and rows are zero,
+    single outliers sit in otherwise small blocks: the block exponents are absolute, so nothing saturates or vanishes."""
+    rng = np.random.default_rng(5)
+    M, N, K = 300, 260, 1024
+    wq = oracle.quantize(MXFP4, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    mag = np.exp2(rng.integers(-40, 41, size=(M, K // 32))).astype(np.float32)
+    x = (x.reshape(M, K // 32, 32) * mag[:, :, None]).reshape(M, K)
+    x[:, 64:96] = 0.0
+    x[7, :] = 0.0
+    x[np.arange(M), rng.integers(0, K, size=M)] *= 1000.0
+    y = run_device(hip, MXFP4, wq, N, K, x)
+    assert np.isfinite(y).all()
+    assert (y[7] == 0).all()
+    check(y, oracle.matmul_f64(MXFP4, wq, N, K, x), "mx dynamic range")
+
+
+def test_mxfp4_block_scaled_non_finite_rows(hip, oracle):
+    """An inf or a NaN in a row makes that row of the result non-finite (its block's scale byte becomes NaN) and
+    leaves the other rows alone."""
+    rng = np.random.default_rng(6)
+    M, N, K = 260, 256, 512
+    wq = oracle.quantize(MXFP4, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    ref = oracle.matmul_f64(MXFP4, wq, N, K, x)
+    x[3, 100] = np.inf
+    x[200, 5] = np.nan
+    y = run_device(hip, MXFP4, wq, N, K, x)
+    assert not np.isfinite(y[3]).any() and not np.isfinite(y[200]).any()
+    keep = np.ones(M, bool)
+    keep[[3, 200]] = False
+    check(y[keep], ref[keep], "mx rows beside non-finite ones")
+
+
 def test_q6_k_128_row_tiles(hip, oracle):
     from oracle.oracle import Q6_K
     rng = np.random.default_rng(77)
