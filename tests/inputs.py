@@ -69,6 +69,11 @@ def random_blocks(name, rows, k, rng):
         if name in ("q4_1", "q5_1"):
             raw[:, 2:4] = f16(-0.06, 0.0, nb)
         return raw.reshape(-1)
+    if name == "mxfp4":
+        nb = rows * (k // 32)
+        raw = rng.integers(0, 256, size=(nb, 17), dtype=np.uint8)
+        raw[:, 0] = rng.integers(112, 124, nb)          # E8M0 scales of 2^-15 .. 2^-4
+        return raw.reshape(-1)
     if name == "q5_k":
         nb = rows * (k // 256)
         raw = rng.integers(0, 256, size=(nb, 176), dtype=np.uint8)

@@ -272,6 +272,27 @@ def test_mxfp4_block_scaled_non_finite_rows(hip, oracle):
     check(y[keep], ref[keep], "mx rows beside non-finite ones")
 
 
+@pytest.mark.parametrize("M", [9, 40])
+def test_mxfp4_block_scaled_small_batch_large_weight(hip, oracle, M):
+    """A small batch over a weight of 64 M elements or more takes the register-resident kernel on the block-scaled
+    instruction (32-row units); two K chunks at this K.  Random valid blocks; the oracle checks 300 sampled columns."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(M)
+    N, K = 21000, 3200
+    wq = inputs.random_blocks("mxfp4", N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(torch.from_numpy(wq).cuda(), MXFP4, K, N))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+    cols = np.unique(np.concatenate([[0, 31, 32, N - 1], rng.integers(0, N, 300)]))
+    rb = K // 32 * 17
+    sub = np.concatenate([wq[c * rb:(c + 1) * rb] for c in cols])
+    ref = oracle.matmul_f64(MXFP4, sub, len(cols), K, x)
+    # the row norm of the full result scales the bound: a column subset has a smaller norm, which only tightens it
+    check(y[:, cols], ref, ("mx small batch", M))
+
+
 def test_q6_k_128_row_tiles(hip, oracle):
     from oracle.oracle import Q6_K
     rng = np.random.default_rng(77)
