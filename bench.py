@@ -23,6 +23,7 @@ sys.path.insert(0, ROOT)
 Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 8, 12, 13, 14, 39
 HBM_PEAK_GBS = 8000.0
 MFMA_FP16_PEAK_TFLOPS = 2516.6
+MFMA_FP6_FP4_PEAK_TFLOPS = 10066.0   # dense fp6 / fp4 operands (two instructions per k-tile count 4 M N K operations)
 # HBM bytes per launch of the grouped Q4_K GEMV come from rocprofv3 FETCH_SIZE + WRITE_SIZE runs, not from this script.
 # The summary of those runs records the figure together with the SHA-256 of the kernel source it was measured on; the
 # figure is reported only while the source still has that digest.
@@ -321,6 +322,20 @@ def main():
         "kernel": "tship::gemm_xw_kernel<tship::PQ4K, 256, 4> (+ tship::convert_x_kernel on the activations, inside the timed call)",
         "avg_call_us": pre["us_per_call_events"], "flops_per_call": 2 * pm * pn * pk, "calls_timed": 20}
 
+    # The same shape with MXFP4 weights (the third format of the metric; BASELINE names MXFP4 for the MoE stage only, so
+    # this is beside the metric's own prefill figure, not in place of it): the weight blocks go to the block-scaled
+    # matrix instruction as they are and every activation is two MX fp6 terms, so a k-tile is two fp6 x fp4 instructions
+    # where fp16 operands take four of half the rate.  `frac` stays against the fp16 peak of the other formats.
+    if not args.no_extra:
+        mx = prefill(MXFP4, pm, pn, pk, 20)
+        out["roofline_prefill_mxfp4"] = {
+            "bound": "mfma", "achieved": mx["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(mx["TFLOPs"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+            "workload": "MXFP4 prefill GEMM M=2048 N=21504 K=5376: raw fp4 blocks x two MX fp6 (E2M3) activation terms, f32 accumulate",
+            "kernel": "tship::gemm_mx_kernel<256, 3> (+ tship::convert_x_kernel<1000, ...> on the activations, inside the timed call)",
+            "avg_call_us": mx["us_per_call_events"], "flops_per_call": 2 * pm * pn * pk, "calls_timed": 20,
+            "instruction_ops_over_fp6_fp4_peak": round(2 * mx["TFLOPs"] / MFMA_FP6_FP4_PEAK_TFLOPS, 4)}
+
     # ---- secondary workloads (reported, not the headline) ---------------------------------------
     if not args.no_extra:
         extra = {}
@@ -361,6 +376,9 @@ def main():
         extra["cfg5_q8_0_gemm_2048x21504x5376"] = prefill(Q8_0, 2048, 21504, 5376, 10)
         extra["cfg5_q4_k_gemm_2048x5376x21504"] = prefill(Q4_K, 2048, 5376, 21504, 10)
         extra["cfg5_q8_0_gemm_2048x5376x21504"] = prefill(Q8_0, 2048, 5376, 21504, 10)
+        extra["mxfp4_gemm_2048x21504x5376"] = mx
+        extra["mxfp4_gemm_2048x5376x21504"] = prefill(MXFP4, 2048, 5376, 21504, 10)
+        extra["mxfp4_gemm_1024x5760x2880"] = prefill(MXFP4, 1024, 5760, 2880)
         # small batches (speculative decoding / few concurrent sequences): weight streaming, GB/s is the figure of merit
         for m in (8, 32, 128):
             r = prefill(Q4_K, m, 14336, 4096)
