@@ -1669,20 +1669,23 @@ __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
 #pragma unroll
     for (int n = 0; n < NB; ++n) my_d0[n] = P::row_delta(base_delta + (uint32_t)(n0 + 32 * NB * wn + 32 * n + col) * row_bytes);
 
-    // B operands of k-tile kt from its stage: the lane's raw block, re-aligned, and its scale byte
-    auto load_b = [&](int kt, int st, int8v_t (&b)[NB], int (&sb)[NB]) {
+    // B operands of k-tile kt from its stage: the lane's raw block as five dwords (fetch_b), then re-aligned and with
+    // its scale byte (finish_b) - two steps, so that the matrix instructions between them cover the LDS latency
+    auto fetch_b = [&](int kt, int st, uint32_t (&r)[NB][G::kRegs]) {
         const uint8_t* const rws = rraw + st * kRawTile + my_raw;
+#pragma unroll
+        for (int n = 0; n < NB; ++n) P::fetch(rws + n * 32 * P::kRowBytes, h, P::delta(my_d0[n], kt), r[n]);
+    };
+    auto finish_b = [&](int kt, const uint32_t (&r)[NB][G::kRegs], int8v_t (&b)[NB], int (&sb)[NB]) {
         const bool live = (kt * 2 + h) * 32 < A.K;
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
-            uint32_t r[G::kRegs];
             const uint32_t dl = P::delta(my_d0[n], kt);
-            P::fetch(rws + n * 32 * P::kRowBytes, h, dl, r);
             const uint32_t sft = (dl + (uint32_t)h * 17u) & 3u;
-            const uint32_t e = (r[0] >> (8 * sft)) & 0xffu;
+            const uint32_t e = (r[n][0] >> (8 * sft)) & 0xffu;
             const bool wrap = sft == 3;
-            const uint32_t b0 = wrap ? r[1] : r[0], b1 = wrap ? r[2] : r[1], b2 = wrap ? r[3] : r[2];
-            const uint32_t b3 = wrap ? r[4] : r[3], b4 = r[4];
+            const uint32_t b0 = wrap ? r[n][1] : r[n][0], b1 = wrap ? r[n][2] : r[n][1], b2 = wrap ? r[n][3] : r[n][2];
+            const uint32_t b3 = wrap ? r[n][4] : r[n][3], b4 = r[n][4];
             const uint32_t shb = (sft + 1) & 3;
             // a block past the end of K: zeros under a scale of one (its bytes belong to the next row)
             b[n][0] = live ? (int)__builtin_amdgcn_alignbyte(b1, b0, shb) : 0;
@@ -1725,13 +1728,15 @@ __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
     for (int j = 0; j < ST - 1; ++j) issue(kt_begin + j, j);
     wait_copies_and_barrier<(ST - 2) * (XI + RI)>();
     issue_slot(kt_begin + ST - 1, ST - 1, 0);              // its other copies follow in the first k-tile of the loop
-    int8v_t b[NB], bn[NB];
-    int sb[NB], sbn[NB];
+    int8v_t b[NB];
+    int sb[NB];
+    uint32_t braw[NB][G::kRegs];
     TSHIP_MX_AOP(a0);                                      // row blocks alternate between the two (TMW is even)
     TSHIP_MX_AOP(a1);
-    load_b(kt_begin, 0, b, sb);
+    fetch_b(kt_begin, 0, braw);
     TSHIP_MX_LOAD_A(0, 0, a0);
-#define TSHIP_MX_KTILE(KT, B, SB, BNX, SBNX)                                                                              \
+    finish_b(kt_begin, braw, b, sb);
+#define TSHIP_MX_KTILE(KT, B, SB)                                                                                          \
     do {                                                                                                                 \
         const int prev_ = stage == 0 ? ST - 1 : stage - 1;     /* the stage freed by the barrier of k-tile KT - 1 */     \
         TSHIP_MX_LOAD_A(stage, 1, a1);                                                                                   \
@@ -1754,22 +1759,16 @@ __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
         const int next_ = stage == ST - 1 ? 0 : stage + 1;                                                               \
         /* k-tile KT + 1 has landed once at most the copies of the ST - 2 k-tiles after it are in flight */              \
         wait_copies_and_barrier<(ST - 2) * (XI + RI)>();                                                                 \
-        load_b((KT) + 1, next_, BNX, SBNX);                                                                              \
+        fetch_b((KT) + 1, next_, braw);                                                                                  \
         TSHIP_MX_LOAD_A(next_, 0, a0);                                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                               \
         TSHIP_MX_MULTIPLY(a1, TMW - 1, B, SB);                                                                           \
         issue_slot((KT) + ST, stage, 0);                                                                                 \
         __builtin_amdgcn_sched_barrier(0);                                                                               \
+        finish_b((KT) + 1, braw, B, SB);      /* the last multiply has read B: the next k-tile's operands take its place */ \
         stage = next_;                                                                                                   \
     } while (0)
-    for (int kt = kt_begin; kt < nkt; ++kt) {
-        TSHIP_MX_KTILE(kt, b, sb, bn, sbn);
-#pragma unroll
-        for (int n = 0; n < NB; ++n) {
-            b[n] = bn[n];
-            sb[n] = sbn[n];
-        }
-    }
+    for (int kt = kt_begin; kt < nkt; ++kt) TSHIP_MX_KTILE(kt, b, sb);
 #undef TSHIP_MX_KTILE
 #undef TSHIP_MX_AOP
 #undef TSHIP_MX_LOAD_A
