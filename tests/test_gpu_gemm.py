@@ -227,14 +227,46 @@ def test_128_row_tiles(hip, oracle, name, M, N, K):
 
 # ---- plain MXFP4 launches of 128- / 256-row tiles: the block-scaled matrix instruction, activations as two MX fp6 terms ----
 @pytest.mark.parametrize("M,N,K", [(300, 520, 32 * 33),      # odd block count: half of the last k-tile is past K
-                                   (700, 1500, 2880),        # 256-row tiles, ragged last tile in both directions
+                                   (700, 1500, 2880),        # ragged last tile in both directions, 45 k-tiles
                                    (257, 300, 64),           # a single k-tile
-                                   (1030, 264, 4096 + 32)])
+                                   (1030, 264, 4096 + 32),
+                                   (300, 264, 8192 + 64)])   # rows beyond 8192: the 1024-thread conversion
 def test_mxfp4_block_scaled_tiles(hip, oracle, M, N, K):
     rng = np.random.default_rng(M + 3 * N + K)
     wq = oracle.quantize(MXFP4, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
     x = rng.standard_normal((M, K)).astype(np.float32)
     check(run_device(hip, MXFP4, wq, N, K, x), oracle.matmul_f64(MXFP4, wq, N, K, x), ("mx", M, N, K))
+
+
+def test_mxfp4_block_scaled_256_row_tiles(hip, oracle):
+    # more 128-row tiles than one round of workgroups: 256-row tiles; an odd block count and a ragged last column tile
+    rng = np.random.default_rng(8)
+    M, N, K = 1024, 8500, 32 * 35
+    wq = inputs.random_blocks("mxfp4", N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, MXFP4, wq, N, K, x)
+    rows = np.unique(np.concatenate([np.arange(0, M, 41), [127, 128, 255, 256, 511, 767, 1023]]))
+    check(y[rows], oracle.matmul_f64(MXFP4, wq, N, K, x[rows]), "mx 256-row tiles")
+
+
+@pytest.mark.parametrize("K", [256, 1024, 2048])
+def test_mxfp4_block_scaled_register_resident_k_ranges(hip, oracle, K):
+    """Small batch over a large weight with a short K: two and four k-tiles per wavefront of the register-resident
+    kernel (K = 256 leaves most wavefronts without a k-tile)."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(K)
+    M = 24
+    N = (64 << 20) // K + 40
+    wq = inputs.random_blocks("mxfp4", N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(torch.from_numpy(wq).cuda(), MXFP4, K, N))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+    cols = np.unique(np.concatenate([[0, 31, 32, N - 1], rng.integers(0, N, 300)]))
+    rb = K // 32 * 17
+    sub = np.concatenate([wq[c * rb:(c + 1) * rb] for c in cols])
+    check(y[:, cols], oracle.matmul_f64(MXFP4, sub, len(cols), K, x), ("mx register-resident", K))
 
 
 def test_mxfp4_block_scaled_dynamic_range(hip, oracle):
