@@ -24,7 +24,6 @@
 #include "tship_internal.h"
 
 #include <algorithm>
-#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -2463,14 +2462,10 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
 }  // namespace
 
 namespace {
-// Halfs between two rows of converted activations: the padded row length, plus one cache line when that length is an
-// even number of lines - rows at a stride of an even number of 128-byte lines fall on few of the L2's channels, and
-// the 32 CUs of an XCD read the same activation k-tile at the same time.
-int x_row_halfs(int K)
-{
-    const int kp = (K + kBK - 1) / kBK * kBK;
-    return kp;
-}
+// Halfs between two rows of converted activations: the row length padded to whole k-tiles.  (Padding the stride by a
+// cache line or more, so that rows at an even number of 128-byte lines apart would not share L2 channels, changed no
+// GEMM time: 0, 128, 256, 384 and 2176 bytes measured alike.)
+int x_row_halfs(int K) { return (K + kBK - 1) / kBK * kBK; }
 }  // namespace
 
 size_t gemm_workspace_bytes(int M, int K)
