@@ -1559,7 +1559,6 @@ template <int BM, int ST>
 __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
 {
     typedef PMXFP4 P;
-    typedef GMXFP4 G;
     constexpr int BN = 256, WN = 4, NW = 8;
     constexpr int TMW = BM / 64;                          // 32-row blocks of a wavefront
     constexpr int NB = 2;                                 // 32-column blocks of a wavefront
@@ -1668,29 +1667,34 @@ __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
 #pragma unroll
     for (int n = 0; n < NB; ++n) my_d0[n] = P::row_delta(base_delta + (uint32_t)(n0 + 32 * NB * wn + 32 * n + col) * row_bytes);
 
-    // B operands of k-tile kt from its stage: the lane's raw block as five dwords (fetch_b), then re-aligned and with
-    // its scale byte (finish_b) - two steps, so that the matrix instructions between them cover the LDS latency
-    auto fetch_b = [&](int kt, int st, uint32_t (&r)[NB][G::kRegs]) {
-        const uint8_t* const rws = rraw + st * kRawTile + my_raw;
+    // B operands of k-tile kt from its stage: the lane's raw block (fetch_b), then re-aligned and with its scale byte
+    // (finish_b) - two steps, so that the matrix instructions between them cover the LDS latency.  Block h of the
+    // k-tile starts delta + 17 h bytes into the row's 48-byte window, i.e. delta + h (0 .. 6) bytes into the window's
+    // 16-byte piece h: the 17 bytes lie in pieces h and h + 1, read as two aligned 16-byte pieces (at the 48-byte row
+    // stride sixteen lanes cover all 64 banks once; dword reads at that stride collide four ways).
+    auto fetch_b = [&](int /*kt*/, int st, uint4_t (&r)[NB][2]) {
+        const uint8_t* const rws = rraw + st * kRawTile + my_raw + 16 * h;
 #pragma unroll
-        for (int n = 0; n < NB; ++n) P::fetch(rws + n * 32 * P::kRowBytes, h, P::delta(my_d0[n], kt), r[n]);
+        for (int n = 0; n < NB; ++n) {
+            r[n][0] = *reinterpret_cast<const uint4_t*>(rws + n * 32 * P::kRowBytes);
+            r[n][1] = *reinterpret_cast<const uint4_t*>(rws + n * 32 * P::kRowBytes + 16);
+        }
     };
-    auto finish_b = [&](int kt, const uint32_t (&r)[NB][G::kRegs], int8v_t (&b)[NB], int (&sb)[NB]) {
+    auto finish_b = [&](int kt, const uint4_t (&r)[NB][2], int8v_t (&b)[NB], int (&sb)[NB]) {
         const bool live = (kt * 2 + h) * 32 < A.K;
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
-            const uint32_t dl = P::delta(my_d0[n], kt);
-            const uint32_t sft = (dl + (uint32_t)h * 17u) & 3u;
-            const uint32_t e = (r[n][0] >> (8 * sft)) & 0xffu;
-            const bool wrap = sft == 3;
-            const uint32_t b0 = wrap ? r[n][1] : r[n][0], b1 = wrap ? r[n][2] : r[n][1], b2 = wrap ? r[n][3] : r[n][2];
-            const uint32_t b3 = wrap ? r[n][4] : r[n][3], b4 = r[n][4];
-            const uint32_t shb = (sft + 1) & 3;
+            const uint32_t sh = P::delta(my_d0[n], kt) + (uint32_t)h;          // scale byte at sh, nibbles behind it
+            const uint32_t e = ((sh >> 2 ? r[n][0].y : r[n][0].x) >> (8 * (sh & 3))) & 0xffu;
+            const bool up = ((sh + 1) >> 2) != 0;                              // the nibbles start in dword 1
+            const uint32_t shb = (sh + 1) & 3;
+            const uint32_t v0 = up ? r[n][0].y : r[n][0].x, v1 = up ? r[n][0].z : r[n][0].y, v2 = up ? r[n][0].w : r[n][0].z;
+            const uint32_t v3 = up ? r[n][1].x : r[n][0].w, v4 = up ? r[n][1].y : r[n][1].x;
             // a block past the end of K: zeros under a scale of one (its bytes belong to the next row)
-            b[n][0] = live ? (int)__builtin_amdgcn_alignbyte(b1, b0, shb) : 0;
-            b[n][1] = live ? (int)__builtin_amdgcn_alignbyte(b2, b1, shb) : 0;
-            b[n][2] = live ? (int)__builtin_amdgcn_alignbyte(b3, b2, shb) : 0;
-            b[n][3] = live ? (int)__builtin_amdgcn_alignbyte(b4, b3, shb) : 0;
+            b[n][0] = live ? (int)__builtin_amdgcn_alignbyte(v1, v0, shb) : 0;
+            b[n][1] = live ? (int)__builtin_amdgcn_alignbyte(v2, v1, shb) : 0;
+            b[n][2] = live ? (int)__builtin_amdgcn_alignbyte(v3, v2, shb) : 0;
+            b[n][3] = live ? (int)__builtin_amdgcn_alignbyte(v4, v3, shb) : 0;
             b[n][4] = b[n][5] = b[n][6] = b[n][7] = 0;
             sb[n] = live ? (int)e : 127;
         }
@@ -1729,7 +1733,7 @@ __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
     issue_slot(kt_begin + ST - 1, ST - 1, 0);              // its other copies follow in the first k-tile of the loop
     int8v_t b[NB];
     int sb[NB];
-    uint32_t braw[NB][G::kRegs];
+    uint4_t braw[NB][2];
     TSHIP_MX_AOP(a0);                                      // row blocks alternate between the two (TMW is even)
     TSHIP_MX_AOP(a1);
     fetch_b(kt_begin, 0, braw);
