@@ -2272,19 +2272,29 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
             // from fetching every k-tile up front (the A operands leave few registers)
             auto k_tiles = [&](auto full_tag) {
                 constexpr bool kFull = decltype(full_tag)::value;
-                uint32_t r[KTW + 1][G::kRegs];
-                G::fetch(raw, 0, h, my_delta, r[0]);
+                // Block h of k-tile t starts my_delta + 17 (2 t + h) bytes into the row, i.e. s = my_delta + h + 2 t (< 16)
+                // bytes into its 16-byte piece h + 2 t: two aligned 16-byte reads hold it (at the odd row stride sixteen
+                // lanes cover all 64 banks once, where dword reads collide four ways).
+                uint4_t r[KTW + 1][2];
+                const uint8_t* const rawh = raw + 16 * h;
+                auto fetch = [&](int t) {
+                    r[t][0] = *reinterpret_cast<const uint4_t*>(rawh + 32 * t);
+                    r[t][1] = *reinterpret_cast<const uint4_t*>(rawh + 32 * t + 16);
+                };
+                fetch(0);
 #pragma unroll
                 for (int t = 0; t < KTW; ++t) {
-                    if (t + 1 < KTW) G::fetch(raw, t + 1, h, my_delta, r[t + 1]);
+                    if (t + 1 < KTW) fetch(t + 1);
                     __builtin_amdgcn_sched_barrier(0);
                     if (kFull || t < kcnt) {
                         // the lane's raw block of k-tile t: sixteen bytes of nibbles re-aligned, and its scale byte
-                        const uint32_t sft = (my_delta + (uint32_t)(2 * t + h) * 17u) & 3u;
-                        const uint32_t e = (r[t][0] >> (8 * sft)) & 0xffu;
-                        const bool wrap = sft == 3;
-                        const uint32_t b0 = wrap ? r[t][1] : r[t][0], b1 = wrap ? r[t][2] : r[t][1], b2 = wrap ? r[t][3] : r[t][2];
-                        const uint32_t b3 = wrap ? r[t][4] : r[t][3], b4 = r[t][4];
+                        const uint32_t v[8] = {r[t][0].x, r[t][0].y, r[t][0].z, r[t][0].w, r[t][1].x, r[t][1].y, r[t][1].z, r[t][1].w};
+                        const uint32_t sft = my_delta + (uint32_t)h + 2u * t;          // scale byte at sft, nibbles behind it
+                        const int e0 = (2 * t) >> 2, d0 = (2 * t + 1) >> 2;            // the dwords they start in at the least
+                        const uint32_t e = (((int)(sft >> 2) != e0 ? v[e0 + 1] : v[e0]) >> (8 * (sft & 3))) & 0xffu;
+                        const bool up = (int)((sft + 1) >> 2) != d0;
+                        const uint32_t b0 = up ? v[d0 + 1] : v[d0], b1 = up ? v[d0 + 2] : v[d0 + 1], b2 = up ? v[d0 + 3] : v[d0 + 2];
+                        const uint32_t b3 = up ? v[d0 + 4] : v[d0 + 3], b4 = up ? v[d0 + 5 < 8 ? d0 + 5 : 7] : v[d0 + 4];
                         const uint32_t shb = (sft + 1) & 3;
                         const bool live = ((kt0 + t) * 2 + h) * 32 < A.K;
                         const int8v_t bq = {live ? (int)__builtin_amdgcn_alignbyte(b1, b0, shb) : 0, live ? (int)__builtin_amdgcn_alignbyte(b2, b1, shb) : 0,
