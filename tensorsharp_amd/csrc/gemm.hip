@@ -37,8 +37,6 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kBK = 64;                 // k-tile
 constexpr uint32_t kDeadOffset = 0x80000000u;
-// activation layout tag of convert_x_kernel for gemm_mx_kernel: two block-scaled fp6 (E2M3) terms per activation
-constexpr int kXMx = 1000;
 
 union H2U {
     uint32_t u;
@@ -158,15 +156,7 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
         if (SRC == kSrcSwiglu) return swiglu_oai(src[k] + (bias ? bias[k] : 0.f), src[K + k] + (bias ? bias[K + k] : 0.f), S.alpha, S.limit);
         return src[k];
     };
-    // which float4 of the row register i holds: thread after thread, except for the MX layout, where a thread owns
-    // the pair (elements 4 t .. 4 t + 3 and the four 16 further on) of a 32-element block in registers 2 j, 2 j + 1
-    auto held = [&](int i) -> int {
-        if constexpr (TYPE == kXMx) {
-            const int pair = tid + (i >> 1) * THREADS;
-            return ((pair >> 2) << 3) + (pair & 3) + ((i & 1) << 2);
-        }
-        return tid + i * THREADS;
-    };
+    auto held = [&](int i) -> int { return tid + i * THREADS; };      // which float4 of the row register i holds
     float4 hold[kCvtHold];
 #pragma unroll
     for (int i = 0; i < kCvtHold; ++i) {
@@ -219,134 +209,6 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
     const float inv = __uint_as_float((uint32_t)(254 - se) << 23);
     if (tid == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
     _Float16* dst = out + (int64_t)m * ldo;
-    if constexpr (TYPE == kXMx) {
-        // gemm_mx_kernel: every 32 activations are two MX blocks of fp6 (E2M3) values, x = hi * 2^Eh + lo * 2^El with
-        // lo the same encoding of the rest x - hi * 2^Eh: what is left is below 2^-9 of the block's largest magnitude.
-        // The exponents are absolute (E8M0), so the row scale is one.  A k-tile of a row is 128 bytes = 8 pieces of 16:
-        // term p (hi, lo) of block g keeps the first 16 bytes of its 24-byte field stream in piece 3 p + 2 g and the last
-        // 8 in half g of piece 3 p + 1; piece 6 holds the scale bytes (hi, lo) of block g in the low bytes of dword g.
-        // Field f of a stream pairs with nibble f of the weight block: element f / 2 (f even) or 16 + f / 2 (f odd).
-        uint8_t* const d8 = reinterpret_cast<uint8_t*>(dst);
-        if (tid == 0) scales[m] = 1.0f;
-        // biased exponent E + 127 that brings amax into (3.75, 7.5]; 127 for an empty block, 255 (NaN) for inf / NaN
-        auto block_exp = [](float amax) -> int {
-            const uint32_t u = __float_as_uint(amax);
-            const int ex = (int)(u >> 23) & 0xff;
-            if (ex == 255) return 255;
-            if (amax == 0.f) return 127;
-            const int eb = ex - ((u & 0x7fffffu) > 0x700000u ? 1 : 2);      // mantissa above 1.875 would round up to 8
-            return eb < 1 ? 1 : eb;                                            // at most 253: 2^(254 - eb) is a normal float
-        };
-        auto pow2 = [](int biased) { return __uint_as_float((uint32_t)biased << 23); };      // biased 1..254
-        // E2M3 code of v (|v| < 7.75).  From 1.0 up the code is the float's exponent and top three mantissa bits (rounded
-        // by the add, the carry running into the exponent); below 1.0 it counts eighths.  Sign in bit 5.
-        auto enc = [](float v) -> uint32_t {
-            const uint32_t u = __float_as_uint(v), mag = u & 0x7fffffffu;
-            const uint32_t normal = ((mag + 0x80000u) >> 20) - (126u << 3);
-            const uint32_t small = (uint32_t)(__uint_as_float(mag) * 8.f + 0.5f);
-            uint32_t code = mag >= 0x3f800000u ? normal : small;
-            code = code > 31u ? 31u : code;
-            return code | ((u >> 26) & 32u);
-        };
-        auto dec = [](uint32_t code) -> float {
-            const uint32_t c = code & 31u;
-            const float mag = c >= 8u ? __uint_as_float((c + (126u << 3)) << 20) : (float)c * 0.125f;
-            return (code & 32u) ? -mag : mag;
-        };
-        auto max4 = [](const float4& v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); };
-        // eight fields e0 o0 e1 o1 e2 o2 e3 o3 -> the low four bytes and the last two of the thread's six
-        auto weave = [](const uint32_t (&e)[4], const uint32_t (&o)[4], uint32_t& low, uint32_t& high) {
-            low = e[0] | (o[0] << 6) | (e[1] << 12) | (o[1] << 18) | (e[2] << 24) | (o[2] << 30);
-            high = (o[2] >> 2) | (e[3] << 4) | (o[3] << 10);
-        };
-#pragma unroll
-        for (int i = 0; i < kCvtHold; i += 2) {
-            if ((i >> 1) * THREADS * 2 >= k4) break;               // uniform: whole passes beyond the row
-            const int pair = tid + (i >> 1) * THREADS;             // threads past the row hold zeros and take part
-            const float4 va = hold[i], vb = hold[i + 1];           // fields 8 t .. 8 t + 7 of the block: va even, vb odd
-            float amax = fmaxf(max4(va), max4(vb));
-            amax = fmaxf(amax, __shfl_xor(amax, 1));
-            amax = fmaxf(amax, __shfl_xor(amax, 2));
-            {
-                // a NaN anywhere in the block must reach the maximum (fmaxf drops NaNs)
-                const bool nan = (va.x != va.x) || (va.y != va.y) || (va.z != va.z) || (va.w != va.w) || (vb.x != vb.x) ||
-                                 (vb.y != vb.y) || (vb.z != vb.z) || (vb.w != vb.w);
-                const unsigned long long any = __ballot(nan);
-                if ((any >> ((threadIdx.x & 63) & ~3)) & 0xfull) amax = __uint_as_float(0x7f800000u);
-            }
-            const int eh = block_exp(amax);
-            const bool finite = eh != 255;
-            const float inv_h = finite ? pow2(254 - eh) : 0.f, sc_h = finite ? pow2(eh) : 0.f;
-            const float xa[4] = {va.x, va.y, va.z, va.w}, xb[4] = {vb.x, vb.y, vb.z, vb.w};
-            uint32_t ha[4], hb[4], la[4], lb[4];
-            float ra[4], rb[4];
-            float rmax = 0.f;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                ha[j] = enc(xa[j] * inv_h);
-                hb[j] = enc(xb[j] * inv_h);
-                ra[j] = finite ? xa[j] - dec(ha[j]) * sc_h : 0.f;
-                rb[j] = finite ? xb[j] - dec(hb[j]) * sc_h : 0.f;
-                rmax = fmaxf(rmax, fmaxf(fabsf(ra[j]), fabsf(rb[j])));
-            }
-            rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
-            rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
-            const int el = block_exp(rmax);
-            const float inv_l = pow2(254 - el);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                la[j] = enc(ra[j] * inv_l);
-                lb[j] = enc(rb[j] * inv_l);
-            }
-            uint32_t w_lo[2], w_hi[2];
-            weave(ha, hb, w_lo[0], w_hi[0]);
-            weave(la, lb, w_lo[1], w_hi[1]);
-            const int t4 = pair & 3, blk = pair >> 2;              // quarter of the stream, block of the row
-            const int g = blk & 1;
-            uint8_t* const row = d8 + (blk >> 1) * 128;
-            const bool inside = 2 * pair < k4;                     // the pair's block lies inside the row
-            // thread t4 holds bytes 6 t4 .. 6 t4 + 5 of either stream and fetches the thread after it for the dwords
-            // that straddle two threads
-#pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                const uint32_t nb_lo = __shfl_down(w_lo[p], 1);
-                uint8_t* const main_piece = row + (3 * p + 2 * g) * 16;
-                uint8_t* const rest_piece = row + (3 * p + 1) * 16 + 8 * g;
-                const uint32_t straddle = (w_hi[p] & 0xffffu) | (nb_lo << 16);    // bytes 4, 5 of this thread, 0, 1 of the next
-                const uint32_t upper4 = (w_lo[p] >> 16) | (w_hi[p] << 16);        // bytes 2 .. 5 of this thread
-                if (inside) {
-                    if (t4 == 0) {
-                        uint2 v2;
-                        v2.x = w_lo[p];
-                        v2.y = straddle;
-                        *reinterpret_cast<uint2*>(main_piece) = v2;
-                    } else if (t4 == 1) {
-                        *reinterpret_cast<uint32_t*>(main_piece + 8) = upper4;
-                    } else if (t4 == 2) {
-                        *reinterpret_cast<uint32_t*>(main_piece + 12) = w_lo[p];
-                        *reinterpret_cast<uint32_t*>(rest_piece) = straddle;
-                    } else {
-                        *reinterpret_cast<uint32_t*>(rest_piece + 4) = upper4;
-                    }
-                }
-            }
-            if (inside && t4 == 0) *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = (uint32_t)eh | ((uint32_t)el << 8);
-        }
-        // blocks past K inside the last k-tile: zero streams under a scale of one
-        for (int blk = (K >> 5) + tid; blk < (Kp >> 5); blk += THREADS) {
-            uint8_t* const row = d8 + (blk >> 1) * 128;
-            const int g = blk & 1;
-#pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                uint32_t* const main_piece = reinterpret_cast<uint32_t*>(row + (3 * p + 2 * g) * 16);
-                uint32_t* const rest_piece = reinterpret_cast<uint32_t*>(row + (3 * p + 1) * 16 + 8 * g);
-                main_piece[0] = main_piece[1] = main_piece[2] = main_piece[3] = 0u;
-                rest_piece[0] = rest_piece[1] = 0u;
-            }
-            *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = 127u | (127u << 8);
-        }
-        return;
-    }
     auto put = [&](int k, float v) { dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)(v * inv); };
     // Four consecutive activations land in one aligned 8-byte piece of the k-tile: in the K-quant order as
     // (x0, x2, x1, x3), in the natural order as they are, and in the split-nibble order interleaved with the four
@@ -378,6 +240,133 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
     }
     for (int k = kHeld + tid; k < K; k += THREADS) put(k, tail_value(k));
     for (int k = K + tid; k < Kp; k += THREADS) dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)0.f;
+}
+
+// ------------------------------------------------------------------------------------------
+// activations for gemm_mx_kernel / gemm_slim_mx_kernel: fp32 [M x K] -> two block-scaled fp6 (E2M3) terms per
+// activation, x = hi * 2^Eh + lo * 2^El with lo the same encoding of the rest x - hi * 2^Eh: what is left is below 2^-9
+// of the block's largest magnitude.  The exponents are absolute (E8M0), so the row scale is one.
+// A k-tile of a row is 128 bytes = 8 pieces of 16: term p (hi, lo) of block g keeps the first 16 bytes of its 24-byte
+// stream of 32 six-bit fields in piece 3 p + 2 g and the last 8 in half g of piece 3 p + 1; piece 6 holds the scale
+// bytes (hi, lo) of block g in the low bytes of dword g.  Field f of a stream pairs with nibble f of the weight block:
+// element f / 2 (f even) or 16 + f / 2 (f odd) - the order in which v_cvt_scalef32_2xpk16_fp6_f32 packs its two
+// sixteen-float sources, so a thread converts a whole block with one instruction per term (round to nearest even)
+// and one more (v_cvt_scalef32_pk32_f32_fp6) for the values of the hi term that the rest is taken against.
+// A workgroup takes kMxCvtBlocks consecutive blocks of one row: its threads read them float4 by float4 (coalesced),
+// pass them through LDS (144 bytes per block: the 16-byte reads of sixteen threads cover the banks once) and each
+// thread converts one block.
+// ------------------------------------------------------------------------------------------
+constexpr int kMxCvtBlocks = 128;
+typedef float float16v_t __attribute__((ext_vector_type(16)));
+typedef float float32v_t __attribute__((ext_vector_type(32)));
+typedef uint32_t uint6_t __attribute__((ext_vector_type(6)));
+
+template <int SRC>
+__global__ void __launch_bounds__(kMxCvtBlocks) convert_x_mx_kernel(const ConvertSrc S, int K, int Kp, int ldo, int chunks,
+                                                                     _Float16* __restrict__ out, float* __restrict__ scales)
+{
+    constexpr int T = kMxCvtBlocks;
+    __shared__ float4 stage[T * 9];
+    __shared__ double redd[T / 64];
+    const int m = blockIdx.x / chunks, chunk = blockIdx.x - m * chunks;
+    const int tid = threadIdx.x;
+    const float* src = S.x + (int64_t)(S.row_map ? S.row_map[m] : m) * S.ldx;
+    const float* norm_w = SRC == kSrcPlain ? S.norm_w : nullptr;
+    const float* bias = (SRC == kSrcSwiglu && S.bias) ? S.bias + (int64_t)S.expert_of[m] * 2 * K : nullptr;
+    const int k4 = K >> 2;                       // K is a multiple of 32
+    if (chunk == 0 && tid == 0) scales[m] = 1.0f;
+    // optional RMSNorm prologue (ggml-cpu/ops.cpp:3646-3695: sum of squares in double, scale = 1/sqrtf(mean + eps),
+    // then the multiply by the norm weight: (x * scale) * w); every workgroup of the row sums the whole row
+    float rms = 1.f;
+    if (norm_w) {
+        double ss = 0.0;
+        for (int q = tid; q < k4; q += T) {
+            const float4 v = reinterpret_cast<const float4*>(src)[q];
+            ss += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+        }
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        if ((tid & 63) == 0) redd[tid >> 6] = ss;
+        __syncthreads();
+        double tot = 0.0;
+#pragma unroll
+        for (int i = 0; i < T / 64; ++i) tot += redd[i];
+        rms = 1.0f / sqrtf((float)(tot / (double)K) + S.eps);
+    }
+    const int q0 = chunk * T * 8;                // first float4 of the chunk
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int ql = tid + j * T, q = q0 + ql;
+        float4 v = float4{0.f, 0.f, 0.f, 0.f};
+        if (q < k4) {
+            if (SRC == kSrcSwiglu) {
+                float4 g = reinterpret_cast<const float4*>(src)[q], u = reinterpret_cast<const float4*>(src + K)[q];
+                if (bias) {
+                    const float4 bg = reinterpret_cast<const float4*>(bias)[q], bu = reinterpret_cast<const float4*>(bias + K)[q];
+                    g = float4{g.x + bg.x, g.y + bg.y, g.z + bg.z, g.w + bg.w};
+                    u = float4{u.x + bu.x, u.y + bu.y, u.z + bu.z, u.w + bu.w};
+                }
+                v = float4{swiglu_oai(g.x, u.x, S.alpha, S.limit), swiglu_oai(g.y, u.y, S.alpha, S.limit),
+                           swiglu_oai(g.z, u.z, S.alpha, S.limit), swiglu_oai(g.w, u.w, S.alpha, S.limit)};
+            } else {
+                v = reinterpret_cast<const float4*>(src)[q];
+                if (norm_w) {
+                    const float4 wv = reinterpret_cast<const float4*>(norm_w)[q];
+                    v = float4{(v.x * rms) * wv.x, (v.y * rms) * wv.y, (v.z * rms) * wv.z, (v.w * rms) * wv.w};
+                }
+            }
+        }
+        stage[(ql >> 3) * 9 + (ql & 7)] = v;
+    }
+    __syncthreads();
+    const int blk = chunk * T + tid;             // this thread's block of the row
+    if (blk >= (Kp >> 5)) return;
+    uint8_t* const row = reinterpret_cast<uint8_t*>(out + (int64_t)m * ldo) + (blk >> 1) * 128;
+    const int g = blk & 1;
+    float16v_t a, b;                             // elements 0 .. 15 and 16 .. 31 of the block
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float4 va = stage[tid * 9 + j], vb = stage[tid * 9 + 4 + j];
+        a[4 * j] = va.x, a[4 * j + 1] = va.y, a[4 * j + 2] = va.z, a[4 * j + 3] = va.w;
+        b[4 * j] = vb.x, b[4 * j + 1] = vb.y, b[4 * j + 2] = vb.z, b[4 * j + 3] = vb.w;
+    }
+    // Largest magnitude as an integer maximum of the bit patterns: an infinity or a NaN anywhere in the block comes out
+    // on top.  Biased exponent E + 127 that brings it into (3.75, 7.5]; 127 for an empty block, 255 (NaN) for inf / NaN.
+    auto top = [](const float16v_t& x, const float16v_t& y) -> uint32_t {
+        uint32_t t = 0u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t = max(t, max(__float_as_uint(x[i]) & 0x7fffffffu, __float_as_uint(y[i]) & 0x7fffffffu));
+        return t;
+    };
+    auto block_exp = [](uint32_t u) -> int {
+        const int ex = (int)(u >> 23);
+        if (ex == 255) return 255;
+        if (u == 0u) return 127;
+        const int eb = ex - ((u & 0x7fffffu) > 0x700000u ? 1 : 2);      // a mantissa above 1.875 would round up to 8
+        return eb < 1 ? 1 : eb;                                            // at most 253
+    };
+    auto pow2 = [](int biased) { return __uint_as_float((uint32_t)biased << 23); };      // biased 1 .. 254
+    int eh = 127, el = 127;
+    uint6_t hi = {0u, 0u, 0u, 0u, 0u, 0u}, lo = {0u, 0u, 0u, 0u, 0u, 0u};
+    if (blk < (K >> 5)) {                        // blocks past K inside the last k-tile: zero streams under a scale of one
+        eh = block_exp(top(a, b));
+        if (eh != 255) {
+            const float sc_h = pow2(eh);
+            hi = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(a, b, sc_h);
+            const float32v_t back = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(hi, sc_h);      // in field order
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                a[i] -= back[2 * i];
+                b[i] -= back[2 * i + 1];
+            }
+            el = block_exp(top(a, b));
+            lo = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(a, b, pow2(el));
+        }
+    }
+    *reinterpret_cast<uint4_t*>(row + (2 * g) * 16) = uint4_t{hi[0], hi[1], hi[2], hi[3]};
+    *reinterpret_cast<uint2*>(row + 16 + 8 * g) = uint2{hi[4], hi[5]};
+    *reinterpret_cast<uint4_t*>(row + (3 + 2 * g) * 16) = uint4_t{lo[0], lo[1], lo[2], lo[3]};
+    *reinterpret_cast<uint2*>(row + 64 + 8 * g) = uint2{lo[4], lo[5]};
+    *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = (uint32_t)eh | ((uint32_t)el << 8);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -721,7 +710,7 @@ struct GemmArgs {
     float* partial;          // null: one chunk, results go straight to c
     int k_chunks;
     int chunk_kt;            // k-tiles per chunk (8 wavefronts x KTW)
-    int x_mx;                // the activations are MX fp6 pairs in gemm_mx_kernel's layout (convert_x_kernel<kXMx>)
+    int x_mx;                // the activations are MX fp6 pairs in gemm_mx_kernel's layout (convert_x_mx_kernel)
 };
 
 constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
@@ -1545,7 +1534,7 @@ bool launch_xw(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
 // MXFP4 on the block-scaled matrix instruction (v_mfma_scale_f32_32x32x64_f8f6f4): the weight operand is the RAW block -
 // 16 bytes of E2M1 pairs plus its E8M0 scale byte, exactly what the instruction's fp4 operand and block scale are -
 // so nothing is unpacked at all.  The activations are two MX terms of fp6 (E2M3) per 32-element block, x = hi 2^Eh +
-// lo 2^El (convert_x_kernel<kXMx>), every product takes two instructions, and fp6 x fp4 runs at twice the rate of the
+// lo 2^El (convert_x_mx_kernel), every product takes two instructions, and fp6 x fp4 runs at twice the rate of the
 // fp16 instruction, so the pair costs half of what the fp16 k-tile costs.  Same tiles as gemm_xw_kernel (BM x 256 x 64,
 // 2 x 4 wavefronts of BM / 2 x 64) and the same LDS-direct copies; no exchange area, so ST copy stages fit.  Operand
 // layout of the instruction (probed on the device): output as the fp16 instructions; lane = column + 32 g holds block g
@@ -2180,7 +2169,7 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
             reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
 
         // A operands of this wavefront's K range: row col + 32 rb, block h of every k-tile - the two 24-byte streams
-        // and the scale dword (layout of convert_x_kernel<kXMx>)
+        // and the scale dword (layout of convert_x_mx_kernel)
         uint4_t ah0[KTW][RB], al0[KTW][RB];
         uint2_t ah1[KTW][RB], al1[KTW][RB];
         uint32_t asa[KTW / 2][RB];                 // scale bytes (hi, lo) of k-tile 2 j in bytes 0, 1 and of 2 j + 1 in bytes 2, 3
@@ -2554,7 +2543,9 @@ bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspa
             set_last_error("gemm: the MX activation layout is for MXFP4 weights.");
             return false;
         }
-        launch_convert_typed<kXMx, SRC>(src, M, K, kp, x16, scales, stream);
+        const int chunks = (kp / 32 + kMxCvtBlocks - 1) / kMxCvtBlocks;
+        hipLaunchKernelGGL((convert_x_mx_kernel<SRC>), dim3((unsigned)((int64_t)M * chunks)), dim3(kMxCvtBlocks), 0, stream, src, K, kp,
+                           x_row_halfs(K), chunks, x16, scales);
         return hip_ok(hipGetLastError(), "activation convert launch");
     }
     // three activation orders: the K-quant nibble order, the split-nibble order of the 32-weight blocks, natural
