@@ -1451,12 +1451,19 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
             GemmTiles tiles{maps.tile_expert, maps.tile_row0, maps.tile_rows, max_tiles, bm, gu_bytes};
             if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream, nullptr, 0.f, x_layout))
                 return 0;
-            if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream, false,
-                             ws + o_chunk, chunk_bytes, x_layout))
-                return 0;
-            // bias + SwiGLU-OAI are formed while the down projection's activations are converted
-            if (!launch_convert_x_swiglu(ggml_type, gu, gate_up_bias, maps.expert_of, alpha, limit, A, (int)F, ws + o_ws2, stream, x_layout))
-                return 0;
+            if (mx && bm == 32 && gemm_swiglu_mx_fits((int)F, (int)H)) {
+                // bias + SwiGLU-OAI and the conversion of the down projection's activations happen in the GEMM's epilogue
+                if (!launch_gemm_swiglu_mx(gate_up_w, ws + o_ws1, ws + o_ws2, gate_up_bias, alpha, limit, A, (int)F, (int)H, &tiles, stream))
+                    return 0;
+            } else {
+                if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream,
+                                 false, ws + o_chunk, chunk_bytes, x_layout))
+                    return 0;
+                // bias + SwiGLU-OAI are formed while the down projection's activations are converted
+                if (!launch_convert_x_swiglu(ggml_type, gu, gate_up_bias, maps.expert_of, alpha, limit, A, (int)F, ws + o_ws2, stream,
+                                             x_layout))
+                    return 0;
+            }
             tiles.expert_stride = dn_bytes;
             if (!launch_gemm(ggml_type, down_w, dn_bytes, ws + o_ws2, dn, H, nullptr, A, (int)H, (int)F, &tiles, stream, false,
                              ws + o_chunk, chunk_bytes, x_layout))

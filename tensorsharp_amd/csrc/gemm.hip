@@ -261,6 +261,60 @@ typedef float float16v_t __attribute__((ext_vector_type(16)));
 typedef float float32v_t __attribute__((ext_vector_type(32)));
 typedef uint32_t uint6_t __attribute__((ext_vector_type(6)));
 
+// One block of 32 activations (a: elements 0 .. 15, b: 16 .. 31) as its two fp6 streams and their biased exponents.
+// A block that is not live (past K inside the last k-tile) gives zero streams under a scale of one.
+struct MxBlock {
+    uint6_t hi, lo;
+    int eh, el;
+};
+__device__ __forceinline__ MxBlock mx_encode_block(float16v_t a, float16v_t b, bool live)
+{
+    // Largest magnitude as an integer maximum of the bit patterns: an infinity or a NaN anywhere in the block comes out
+    // on top.  Biased exponent E + 127 that brings it into (3.75, 7.5]; 127 for an empty block, 255 (NaN) for inf / NaN.
+    auto top = [](const float16v_t& x, const float16v_t& y) -> uint32_t {
+        uint32_t t = 0u;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t = max(t, max(__float_as_uint(x[i]) & 0x7fffffffu, __float_as_uint(y[i]) & 0x7fffffffu));
+        return t;
+    };
+    auto block_exp = [](uint32_t u) -> int {
+        const int ex = (int)(u >> 23);
+        if (ex == 255) return 255;
+        if (u == 0u) return 127;
+        const int eb = ex - ((u & 0x7fffffu) > 0x700000u ? 1 : 2);      // a mantissa above 1.875 would round up to 8
+        return eb < 1 ? 1 : eb;                                            // at most 253
+    };
+    auto pow2 = [](int biased) { return __uint_as_float((uint32_t)biased << 23); };      // biased 1 .. 254
+    MxBlock r;
+    r.eh = r.el = 127;
+    r.hi = r.lo = uint6_t{0u, 0u, 0u, 0u, 0u, 0u};
+    if (live) {
+        r.eh = block_exp(top(a, b));
+        if (r.eh != 255) {
+            const float sc_h = pow2(r.eh);
+            r.hi = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(a, b, sc_h);
+            const float32v_t back = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(r.hi, sc_h);      // in field order
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                a[i] -= back[2 * i];
+                b[i] -= back[2 * i + 1];
+            }
+            r.el = block_exp(top(a, b));
+            r.lo = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(a, b, pow2(r.el));
+        }
+    }
+    return r;
+}
+// block g (0, 1) of the k-tile whose 128 bytes start at `tile`
+__device__ __forceinline__ void mx_store_block(uint8_t* tile, int g, const MxBlock& r)
+{
+    *reinterpret_cast<uint4_t*>(tile + (2 * g) * 16) = uint4_t{r.hi[0], r.hi[1], r.hi[2], r.hi[3]};
+    *reinterpret_cast<uint2*>(tile + 16 + 8 * g) = uint2{r.hi[4], r.hi[5]};
+    *reinterpret_cast<uint4_t*>(tile + (3 + 2 * g) * 16) = uint4_t{r.lo[0], r.lo[1], r.lo[2], r.lo[3]};
+    *reinterpret_cast<uint2*>(tile + 64 + 8 * g) = uint2{r.lo[4], r.lo[5]};
+    *reinterpret_cast<uint32_t*>(tile + 96 + 4 * g) = (uint32_t)r.eh | ((uint32_t)r.el << 8);
+}
+
 template <int SRC>
 __global__ void __launch_bounds__(kMxCvtBlocks) convert_x_mx_kernel(const ConvertSrc S, int K, int Kp, int ldo, int chunks,
                                                                      _Float16* __restrict__ out, float* __restrict__ scales)
@@ -329,44 +383,7 @@ __global__ void __launch_bounds__(kMxCvtBlocks) convert_x_mx_kernel(const Conver
         a[4 * j] = va.x, a[4 * j + 1] = va.y, a[4 * j + 2] = va.z, a[4 * j + 3] = va.w;
         b[4 * j] = vb.x, b[4 * j + 1] = vb.y, b[4 * j + 2] = vb.z, b[4 * j + 3] = vb.w;
     }
-    // Largest magnitude as an integer maximum of the bit patterns: an infinity or a NaN anywhere in the block comes out
-    // on top.  Biased exponent E + 127 that brings it into (3.75, 7.5]; 127 for an empty block, 255 (NaN) for inf / NaN.
-    auto top = [](const float16v_t& x, const float16v_t& y) -> uint32_t {
-        uint32_t t = 0u;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) t = max(t, max(__float_as_uint(x[i]) & 0x7fffffffu, __float_as_uint(y[i]) & 0x7fffffffu));
-        return t;
-    };
-    auto block_exp = [](uint32_t u) -> int {
-        const int ex = (int)(u >> 23);
-        if (ex == 255) return 255;
-        if (u == 0u) return 127;
-        const int eb = ex - ((u & 0x7fffffu) > 0x700000u ? 1 : 2);      // a mantissa above 1.875 would round up to 8
-        return eb < 1 ? 1 : eb;                                            // at most 253
-    };
-    auto pow2 = [](int biased) { return __uint_as_float((uint32_t)biased << 23); };      // biased 1 .. 254
-    int eh = 127, el = 127;
-    uint6_t hi = {0u, 0u, 0u, 0u, 0u, 0u}, lo = {0u, 0u, 0u, 0u, 0u, 0u};
-    if (blk < (K >> 5)) {                        // blocks past K inside the last k-tile: zero streams under a scale of one
-        eh = block_exp(top(a, b));
-        if (eh != 255) {
-            const float sc_h = pow2(eh);
-            hi = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(a, b, sc_h);
-            const float32v_t back = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(hi, sc_h);      // in field order
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                a[i] -= back[2 * i];
-                b[i] -= back[2 * i + 1];
-            }
-            el = block_exp(top(a, b));
-            lo = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(a, b, pow2(el));
-        }
-    }
-    *reinterpret_cast<uint4_t*>(row + (2 * g) * 16) = uint4_t{hi[0], hi[1], hi[2], hi[3]};
-    *reinterpret_cast<uint2*>(row + 16 + 8 * g) = uint2{hi[4], hi[5]};
-    *reinterpret_cast<uint4_t*>(row + (3 + 2 * g) * 16) = uint4_t{lo[0], lo[1], lo[2], lo[3]};
-    *reinterpret_cast<uint2*>(row + 64 + 8 * g) = uint2{lo[4], lo[5]};
-    *reinterpret_cast<uint32_t*>(row + 96 + 4 * g) = (uint32_t)eh | ((uint32_t)el << 8);
+    mx_store_block(row, g, mx_encode_block(a, b, blk < (K >> 5)));      // blocks past K inside the last k-tile: zeros
 }
 
 // ------------------------------------------------------------------------------------------
@@ -711,6 +728,11 @@ struct GemmArgs {
     int k_chunks;
     int chunk_kt;            // k-tiles per chunk (8 wavefronts x KTW)
     int x_mx;                // the activations are MX fp6 pairs in gemm_mx_kernel's layout (convert_x_mx_kernel)
+    // gemm_slim_mx_kernel<.., .., 1>: bias + SwiGLU-OAI of (gate, up) column pairs, written as MX activation rows
+    const float* epi_bias;   // optional [experts x 2 F]
+    float epi_alpha, epi_limit;
+    uint8_t* epi_out;        // activation rows of the down projection (layout of convert_x_mx_kernel)
+    int64_t epi_ld;          // bytes between them
 };
 
 constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
@@ -1853,6 +1875,12 @@ bool launch_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
 // the raw buffer the wavefront has just consumed), are added in a fixed order and stored.  A K longer than
 // 8 * KTW k-tiles is cut into chunks whose sums a second kernel adds.
 // ------------------------------------------------------------------------------------------
+// an address that is the same in every lane, for the compiler to keep in scalar registers
+__device__ __forceinline__ uintptr_t uniform_address(uintptr_t a)
+{
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    return ((uintptr_t)hi << 32) | lo;
+}
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // LDS layout of one wavefront of the register-resident kernel: RING raw buffers of 32 rows x CH 16-byte chunks
@@ -1921,7 +1949,9 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
             m0 = mt * 32;
             m_rows = min(32, A.M - m0);
         }
-        const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
+        // (the expert id comes from memory the kernel also writes to, so the compiler loads it per lane: without the
+        // hint every copy would run in a loop over the distinct descriptors of the wavefront)
+        const uintptr_t wa = uniform_address(reinterpret_cast<uintptr_t>(wbase));
         const uint32_t base_delta = (uint32_t)(wa & 3);
         const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
             reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
@@ -2114,12 +2144,14 @@ struct SlimMxLayout {
     static constexpr int RING = 8 * 3 * BUF + 1024 <= 160 * 1024 ? 3 : 2;
 };
 
-template <int KTW, int RB>
+template <int KTW, int RB, int EPI>
 __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
 {
+    static_assert(EPI == 0 || RB == 1, "the fused epilogue takes 32-row units");
     typedef GMXFP4 G;
     using L = SlimMxLayout<KTW, RB>;
     constexpr int CH = L::CH, DI = L::DI, BUF = L::BUF, RING = L::RING;
+    constexpr int DIE = DI + (EPI ? 1 : 0);                              // copies per tile: EPI adds the tile's 32 bias values
     constexpr int NQ = 2 * RB;                                          // results per thread in the reduction
     static_assert(KTW % G::kTileStep == 0, "a wavefront's K range must start at a block");
     typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
@@ -2129,6 +2161,7 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, h = lane >> 5;
     uint8_t* const my_buf = smem + wave * RING * BUF;
+    float* const my_bias = reinterpret_cast<float*>(smem + 8 * RING * BUF) + wave * RING * 32;      // EPI: 32 floats per buffer
 
     const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
     const int nkt = A.Kp / kBK;
@@ -2144,7 +2177,15 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
     }
     const int64_t units = (int64_t)live_tiles * per_tile;
     int u = (int)(units * blockIdx.x / gridDim.x);
-    const int u_end = (int)(units * (blockIdx.x + 1) / gridDim.x);
+    int u_end = (int)(units * (blockIdx.x + 1) / gridDim.x);
+    // EPI = 1, gate_up of the gpt-oss experts (N = 2 F, one K chunk, F / 32 whole column tiles): the units of a row tile
+    // walk the column tiles as gate tile 0, up tile 0, gate tile 1, ... so that a workgroup holds both halves of a pair;
+    // ranges start at pairs.  Unit j of the walk is column tile phys(j).
+    if (EPI) {
+        u &= ~1;
+        u_end &= ~1;                                                   // units is even: every row tile has 2 x F / 32
+    }
+    auto phys = [&](int j) { return EPI ? (j >> 1) + (j & 1) * (n32 >> 1) : j; };
 
     while (u < u_end) {
         const int mt = u / per_tile, rem = u - mt * per_tile;
@@ -2163,7 +2204,9 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
             m_rows = min(32 * RB, A.M - m0);
         }
         const int rbs = RB > 1 && m_rows > 32 ? RB : 1;                // row blocks with rows in them (uniform)
-        const uintptr_t wa = reinterpret_cast<uintptr_t>(wbase);
+        // (the expert id comes from memory the kernel also writes to, so the compiler loads it per lane: without the
+        // hint every copy would run in a loop over the distinct descriptors of the wavefront)
+        const uintptr_t wa = uniform_address(reinterpret_cast<uintptr_t>(wbase));
         const uint32_t base_delta = (uint32_t)(wa & 3);
         const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
             reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
@@ -2204,20 +2247,32 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
             w_off[i] = (row < 32 && kcnt > 0) ? ((base_delta + (uint32_t)row * row_bytes + koff) & ~3u) + (uint32_t)chunk * 16u : kDeadOffset;
         }
         const uint32_t my_delta = (base_delta + (uint32_t)col * row_bytes + koff) & 3u;
+        // EPI: the expert's [2 F] bias row (an empty range without a bias: the copies deliver zeros)
+        const float* const eb = EPI && A.epi_bias ? A.epi_bias + (int64_t)(A.tile_expert ? A.tile_expert[mt] : 0) * A.N : nullptr;
+        const uintptr_t ba = uniform_address(reinterpret_cast<uintptr_t>(eb));
+        const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(ba & ~(uintptr_t)3), 0, ba ? A.N * 4 : 0, 0x00020000);
+        const uint32_t bias_off = (uint32_t)lane * 16u;
         // copy q of column tile nt0 + i -> buffer b
         auto issue_one = [&](int i, int b, int q) {
             const bool any = i < cnt;
-            const uint32_t so = any ? (uint32_t)(nt0 + i) * 32u * row_bytes : 0u;
+            const uint32_t so = any ? (uint32_t)phys(nt0 + i) * 32u * row_bytes : 0u;
+            if (EPI && q == DI) {
+                // the bias of the tile's 32 columns (zeros without one) comes the same way: a plain load would make the
+                // compiler wait for every copy in flight before its value is used
+                if (lane < 8) copy16_to_lds(brs, reinterpret_cast<uint8_t*>(my_bias + b * 32), any ? bias_off + (uint32_t)phys(nt0 + i) * 128u : kDeadOffset, 0u);
+                return;
+            }
             if (q * 64 + 32 < 32 * CH || lane < 32) copy16_to_lds(wrs, my_buf + b * BUF + q * 1024, any ? w_off[q] : kDeadOffset, so);
         };
         auto issue = [&](int i, int b) {
 #pragma unroll
-            for (int q = 0; q < DI; ++q) issue_one(i, b, q);
+            for (int q = 0; q < DIE; ++q) issue_one(i, b, q);
         };
         // With three buffers the refill of a buffer waits for the NEXT unit and goes out copy by copy behind the matrix
         // instructions of its k-tiles (copy q behind k-tile q % KTW): a copy keeps the wavefront busy for tens of
         // cycles, and there the matrix pipe has work queued for that long.
         constexpr bool kDefer = RING >= 3;
+        static_assert(EPI == 0 || (kDefer && BUF >= 32 * 144), "the fused epilogue stages a 32 x 32 tile in a buffer that is refilled a unit later");
         // results of this thread in the reduction: accumulator registers wave + 8 q of the RB x 16
         int64_t coff[NQ];
         bool ok[NQ];
@@ -2238,17 +2293,40 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
         for (int q = 0; q < NQ; ++q) pend[q] = 0.f;
         int pend_n = -1;
         float* const dst = A.partial ? A.partial : A.c;
+        float gate[NQ];                                 // EPI: the gate sums of the pair whose up tile is next
+        int epi_blk = -1, epi_buf = 0;                  // EPI: the staged activation block that waits for its conversion
         auto flush = [&]() {
-            if (pend_n >= 0 && pend_n < A.N) {
+            if constexpr (EPI == 0) {
+                if (pend_n >= 0 && pend_n < A.N) {
 #pragma unroll
-                for (int q = 0; q < NQ; ++q)
-                    if (ok[q]) dst[coff[q] + pend_n] = pend[q];
+                    for (int q = 0; q < NQ; ++q)
+                        if (ok[q]) dst[coff[q] + pend_n] = pend[q];
+                }
+            } else {
+                // lane r of the last wavefront (whose K range is the one that may be short) converts row r of the staged
+                // 32 x 32 activations into block epi_blk of the down projection's activation rows
+                if (epi_blk >= 0 && wave == 7 && lane < m_rows && lane < 32) {
+                    const float* const stage = reinterpret_cast<const float*>(smem + (7 * RING + epi_buf) * BUF) + lane * 36;
+                    float16v_t va, vb;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        // (vector-typed reads: for reads through a struct type the compiler waits for every copy in flight)
+                        const uint4_t fa = reinterpret_cast<const uint4_t*>(stage)[t], fb = reinterpret_cast<const uint4_t*>(stage)[4 + t];
+                        va[4 * t] = __uint_as_float(fa.x), va[4 * t + 1] = __uint_as_float(fa.y), va[4 * t + 2] = __uint_as_float(fa.z), va[4 * t + 3] = __uint_as_float(fa.w);
+                        vb[4 * t] = __uint_as_float(fb.x), vb[4 * t + 1] = __uint_as_float(fb.y), vb[4 * t + 2] = __uint_as_float(fb.z), vb[4 * t + 3] = __uint_as_float(fb.w);
+                    }
+                    uint8_t* const tile = A.epi_out + (int64_t)(m0 + lane) * A.epi_ld + (epi_blk >> 1) * 128;
+                    mx_store_block(tile, epi_blk & 1, mx_encode_block(va, vb, true));
+                    // the last block of an odd count: the other half of its k-tile lies past F
+                    if (epi_blk + 1 == (n32 >> 1) && !(epi_blk & 1)) mx_store_block(tile, 1, mx_encode_block(va, vb, false));
+                }
+                epi_blk = -1;
             }
         };
         for (int i = 0; i < cnt; ++i) {
             // the copies of tile i have landed; those of the tiles after it stay in flight (deferred refills: the tile
             // RING - 1 on is only issued during this unit)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kDefer ? RING - 2 : RING - 1) * DI) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kDefer ? RING - 2 : RING - 1) * DIE) : "memory");
             flush();
             const int b_prev = b == 0 ? RING - 1 : b - 1;      // the buffer of tile i - 1
             float16_t acc[RB];
@@ -2310,7 +2388,7 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
                     }
                     if (kDefer && i > 0) {
 #pragma unroll
-                        for (int q = t; q < DI; q += KTW) issue_one(i - 1 + RING, b_prev, q);
+                        for (int q = t; q < DIE; q += KTW) issue_one(i - 1 + RING, b_prev, q);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -2336,7 +2414,37 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
 #pragma unroll
             for (int q = 0; q < NQ; ++q) pend[q] = s[q];      // the row scale of this activation layout is one
             pend_n = (nt0 + i) * 32 + col;
+            if constexpr (EPI == 1) {
+                const int j = nt0 + i;
+                if (j & 1) {
+                    // bias + SwiGLU-OAI of this thread's (gate, up) sums: columns (j / 2) 32 + col of the F activations
+                    const float bu = my_bias[b * 32 + col];
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) pend[q] = ok[q] ? swiglu_oai(gate[q], s[q] + bu, A.epi_alpha, A.epi_limit) : 0.f;
+                } else {
+                    const float bg = my_bias[b * 32 + col];
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) gate[q] = s[q] + bg;
+                }
+            }
             lds_barrier();                              // every partial sum has been read: the buffers may be refilled
+            if constexpr (EPI == 1) {
+                const int j = nt0 + i;
+                if (j & 1) {
+                    // The 32 x 32 activations are one MX block per row: they meet in the last wavefront's buffer of this
+                    // tile (free until that wavefront refills it during the next unit), 144 bytes per row; flush() converts
+                    // them at the top of the next unit, where its stores lie behind the wait for the copies.
+                    float* const stage = reinterpret_cast<float*>(smem + (7 * RING + b) * BUF);
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) {
+                        const int rr = wave + 8 * q, r = rr & 15;
+                        stage[(8 * (r >> 2) + 4 * h + (r & 3)) * 36 + col] = pend[q];
+                    }
+                    lds_barrier();
+                    epi_blk = j >> 1;
+                    epi_buf = b;
+                }
+            }
             if (!kDefer) issue(i + RING, b);
             b = b + 1 == RING ? 0 : b + 1;
         }
@@ -2344,12 +2452,12 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
     }
 }
 
-template <int KTW, int RB>
+template <int KTW, int RB, int EPI = 0>
 bool launch_slim_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
     using L = SlimMxLayout<KTW, RB>;
-    auto kern = gemm_slim_mx_kernel<KTW, RB>;
-    constexpr size_t lds = (size_t)8 * L::RING * L::BUF + 64;
+    auto kern = gemm_slim_mx_kernel<KTW, RB, EPI>;
+    constexpr size_t lds = (size_t)8 * L::RING * L::BUF + (EPI ? 8 * L::RING * 128 : 64);      // EPI: 32 bias values per buffer
     static_assert(lds <= 160 * 1024, "raw buffers must fit LDS");
     if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
@@ -2358,6 +2466,10 @@ bool launch_slim_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScra
     a.k_chunks = (a.Kp / kBK + a.chunk_kt - 1) / a.chunk_kt;
     a.partial = nullptr;
     const bool two_pass = a.k_chunks > 1 || a.accumulate;
+    if (EPI && (two_pass || (a.N & 63) || a.M <= 0)) {
+        set_last_error("gemm: the fused SwiGLU epilogue takes one K chunk and whole 32-column tiles of gate and of up.");
+        return false;
+    }
     if (two_pass) {
         const size_t need = (size_t)a.k_chunks * a.M * a.N * sizeof(float);
         if (cs.need_out) *cs.need_out = need;
@@ -2663,6 +2775,49 @@ bool launch_gemm(int type, const void* w, int64_t w_bytes, const void* workspace
 {
     const ChunkScratch cs{static_cast<float*>(chunk_ws), chunk_ws ? chunk_ws_bytes : 0, nullptr};
     return gemm_dispatch(type, w, w_bytes, workspace, c, ldc, c_rows, M, N, K, tiles, stream, accumulate, cs, x_layout);
+}
+
+bool gemm_swiglu_mx_fits(int F, int K)
+{
+    const int kt = (K + kBK - 1) / kBK;
+    return F > 0 && F % 32 == 0 && kt > 16 && kt <= 48 && F <= 32768;
+}
+
+bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace_out, const float* bias, float alpha, float limit,
+                           int M, int F, int K, const GemmTiles* tiles, hipStream_t stream)
+{
+    if (!tiles || tiles->bm != 32 || !gemm_swiglu_mx_fits(F, K)) {
+        set_last_error("gemm: the fused SwiGLU epilogue takes 32-row expert tiles, F a multiple of 32 and 1025 .. 3072 columns of K.");
+        return false;
+    }
+    GemmArgs a{};
+    a.w = static_cast<const uint8_t*>(w);
+    a.w_bytes = tiles->expert_stride;
+    a.xscale = static_cast<const float*>(workspace);
+    a.x16 = reinterpret_cast<const _Float16*>(static_cast<const char*>(workspace) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
+    a.x_mx = 1;
+    a.M = M;
+    a.N = 2 * F;
+    a.K = K;
+    a.Kp = (K + kBK - 1) / kBK * kBK;
+    a.xld = x_row_halfs(K);
+    a.x16_bytes = (int64_t)M * a.xld * (int64_t)sizeof(_Float16);
+    a.epi_bias = bias;
+    a.epi_alpha = alpha;
+    a.epi_limit = limit;
+    a.epi_out = reinterpret_cast<uint8_t*>(static_cast<char*>(workspace_out) + (((size_t)M * sizeof(float) + 255) & ~(size_t)255));
+    a.epi_ld = (int64_t)x_row_halfs(F) * (int64_t)sizeof(_Float16);
+    if (a.x16_bytes >= kMaxOperandBytes || (int64_t)M * a.epi_ld >= kMaxOperandBytes) {
+        set_last_error("gemm: the converted activations of one call must stay below 2 GiB; split the rows.");
+        return false;
+    }
+    a.tile_expert = tiles->expert;
+    a.tile_row0 = tiles->row0;
+    a.tile_rows = tiles->rows;
+    a.expert_stride = tiles->expert_stride;
+    if (tiles->count == 0) return true;
+    const ChunkScratch cs{nullptr, 0, nullptr};
+    return a.Kp / kBK <= 32 ? launch_slim_mx<4, 1, 1>(a, tiles->count, stream, cs) : launch_slim_mx<6, 1, 1>(a, tiles->count, stream, cs);
 }
 
 size_t gemm_chunk_ws_bytes(int type, int M, int N, int K, const GemmTiles* tiles, bool accumulate, int x_layout)

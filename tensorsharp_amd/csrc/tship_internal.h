@@ -161,6 +161,14 @@ struct GemmTiles {
     int64_t expert_stride;
 };
 
+// The gate_up GEMM of MXFP4 gpt-oss experts on 32-row tiles with the down projection's activations as its result:
+// bias + SwiGLU-OAI of every (gate, up) column pair, converted to the MX activation layout in workspace_out (a
+// gemm_workspace_bytes(M, F) buffer), without the [M x 2 F] matrix in between.  workspace holds the MX activations of
+// the M rows x K (launch_convert_x with layout 1).  gemm_swiglu_mx_fits: whether the shape can take this path.
+bool gemm_swiglu_mx_fits(int F, int K);
+bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace_out, const float* bias, float alpha, float limit,
+                           int M, int F, int K, const GemmTiles* tiles, hipStream_t stream);
+
 // c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
 // accumulate: c[row] += ... instead of c[row] = ...
 // chunk_ws (device): where the sums of K chunks go, gemm_chunk_ws_bytes() of them (a shape whose chunk sums do not fit

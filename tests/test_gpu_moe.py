@@ -123,6 +123,28 @@ def test_unbalanced_and_empty_experts(hip, oracle):
     assert inputs.row_l2_err(got, ref) <= 1e-3
 
 
+# MXFP4 experts whose gate_up rows are 1025 .. 3072 long form bias + SwiGLU in the gate_up GEMM's epilogue and write the
+# down projection's block-scaled activations from there: row lengths at both ends of that range and of both k-tile
+# counts per wavefront, F / 32 even and odd (an odd count leaves half a k-tile of padding), experts with more than 32
+# tokens (two row tiles), partly filled tiles and empty experts, with and without biases.
+@pytest.mark.parametrize("E,H,F,T,k", [(4, 1088, 160, 70, 2), (4, 2048, 256, 130, 2), (8, 2880, 96, 40, 4),
+                                       (4, 3072, 512, 9, 2), (4, 1536, 2880, 40, 2)])
+def test_gate_up_epilogue_writes_down_activations(hip, oracle, E, H, F, T, k):
+    rng = np.random.default_rng(1000 + H + F)
+    gu, gb, dn, db = make_experts(oracle, MXFP4, E, H, F, rng, sigma=0.03)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 1] += 2.0                 # expert 1 takes most tokens
+    logits[:, E - 1] -= 50.0            # the last expert takes none
+    ids, wts = oracle.moe_route(logits, k)
+    ref = oracle.moe_forward(MXFP4, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    got = run_gpu(hip, MXFP4, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got, ref) <= 1e-3, inputs.row_l2_err(got, ref)
+    ref2 = oracle.moe_forward(MXFP4, gu, None, dn, None, E, H, F, hidden, ids, wts)
+    got2 = run_gpu(hip, MXFP4, gu, None, dn, None, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got2, ref2) <= 1e-3, inputs.row_l2_err(got2, ref2)
+
+
 @pytest.fixture(scope="module")
 def cfg4_weights(oracle):
     E, H, F = 32, 2880, 2880
