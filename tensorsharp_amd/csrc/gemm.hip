@@ -373,17 +373,35 @@ __global__ void __launch_bounds__(kMxCvtBlocks) convert_x_mx_kernel(const Conver
     }
     __syncthreads();
     const int blk = chunk * T + tid;             // this thread's block of the row
-    if (blk >= (Kp >> 5)) return;
-    uint8_t* const row = reinterpret_cast<uint8_t*>(out + (int64_t)m * ldo) + (blk >> 1) * 128;
-    const int g = blk & 1;
-    float16v_t a, b;                             // elements 0 .. 15 and 16 .. 31 of the block
+    const bool in_row = blk < (Kp >> 5);
+    MxBlock r;
+    if (in_row) {
+        float16v_t a, b;                         // elements 0 .. 15 and 16 .. 31 of the block
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float4 va = stage[tid * 9 + j], vb = stage[tid * 9 + 4 + j];
-        a[4 * j] = va.x, a[4 * j + 1] = va.y, a[4 * j + 2] = va.z, a[4 * j + 3] = va.w;
-        b[4 * j] = vb.x, b[4 * j + 1] = vb.y, b[4 * j + 2] = vb.z, b[4 * j + 3] = vb.w;
+        for (int j = 0; j < 4; ++j) {
+            const float4 va = stage[tid * 9 + j], vb = stage[tid * 9 + 4 + j];
+            a[4 * j] = va.x, a[4 * j + 1] = va.y, a[4 * j + 2] = va.z, a[4 * j + 3] = va.w;
+            b[4 * j] = vb.x, b[4 * j + 1] = vb.y, b[4 * j + 2] = vb.z, b[4 * j + 3] = vb.w;
+        }
+        r = mx_encode_block(a, b, blk < (K >> 5));      // blocks past K inside the last k-tile: zeros
     }
-    mx_store_block(row, g, mx_encode_block(a, b, blk < (K >> 5)));      // blocks past K inside the last k-tile: zeros
+    // The k-tiles of the chunk are put together in LDS and leave as whole 16-byte pieces, thread after thread: stored
+    // from the threads' own registers (4 .. 16 bytes each, 64 bytes apart) the same bytes took five times as long.
+    __syncthreads();                             // every block has been read: the staging area takes the k-tiles
+    uint8_t* const tiles = reinterpret_cast<uint8_t*>(stage);
+    if (in_row) {
+        mx_store_block(tiles + (tid >> 1) * 128, tid & 1, r);
+        if (tid & 1) {                           // the bytes no kernel reads, as zeros
+            *reinterpret_cast<uint2*>(tiles + (tid >> 1) * 128 + 104) = uint2{0u, 0u};
+            *reinterpret_cast<uint4_t*>(tiles + (tid >> 1) * 128 + 112) = uint4_t{0u, 0u, 0u, 0u};
+        }
+    }
+    __syncthreads();
+    const int pieces = min(T / 2, (Kp >> 6) - chunk * (T / 2)) * 8;      // 16-byte pieces of this chunk's k-tiles
+    uint4_t* const dst = reinterpret_cast<uint4_t*>(reinterpret_cast<uint8_t*>(out + (int64_t)m * ldo) + (int64_t)chunk * (T / 2) * 128);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (tid + j * T < pieces) dst[tid + j * T] = reinterpret_cast<const uint4_t*>(tiles)[tid + j * T];
 }
 
 // ------------------------------------------------------------------------------------------
