@@ -1401,7 +1401,10 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
         // pairs, gemm_slim_mx_kernel)
         const bool mx = ggml_type == kTypeMXFP4 && per_expert <= 160 && H <= 32768 && F <= 32768;
         const int x_layout = mx ? 1 : 0;
-        const int bm = per_expert > 160 ? 128 : 32;
+        // 48-row units of that kernel (K <= 3072 on both matmuls) once an expert's tokens often pass 32: nearly every expert
+        // then streams its weights once
+        const bool rows48 = mx && per_expert > 20 && H <= 3072 && F <= 3072;
+        const int bm = per_expert > 160 ? 128 : rows48 ? 48 : 32;
         const int max_tiles = A / bm + E;
         // carve the workspace
         size_t off = 0;
@@ -1451,9 +1454,9 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
             GemmTiles tiles{maps.tile_expert, maps.tile_row0, maps.tile_rows, max_tiles, bm, gu_bytes};
             if (!launch_convert_x(ggml_type, hid, hidden.stride0, maps.token_of, A, (int)H, ws + o_ws1, stream, nullptr, 0.f, x_layout))
                 return 0;
-            if (mx && bm == 32 && gemm_swiglu_mx_fits((int)F, (int)H)) {
+            if (mx && bm <= 48 && gemm_swiglu_mx_fits((int)F, (int)H)) {
                 // bias + SwiGLU-OAI and the conversion of the down projection's activations happen in the GEMM's epilogue
-                if (!launch_gemm_swiglu_mx(gate_up_w, ws + o_ws1, ws + o_ws2, gate_up_bias, alpha, limit, A, (int)F, (int)H, &tiles, stream))
+                if (!launch_gemm_swiglu_mx(gate_up_w, ws + o_ws1, ws + o_ws2, gu, gate_up_bias, alpha, limit, A, (int)F, (int)H, &tiles, stream))
                     return 0;
             } else {
                 if (!launch_gemm(ggml_type, gate_up_w, gu_bytes, ws + o_ws1, gu, 2 * F, nullptr, A, (int)(2 * F), (int)H, &tiles, stream,

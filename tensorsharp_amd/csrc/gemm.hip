@@ -2470,6 +2470,264 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// 48-row units of the register-resident MX kernel, on v_mfma_scale_f32_16x16x128_f8f6f4 (lane = index + 16 g holds the
+// 32 values of K block g of the 128; results: column = lane & 15, rows 4 (lane >> 4) + 0 .. 3 - probed on the device
+// like the 32 x 32 x 64 form).  Three row blocks and two column blocks of 16 per unit: the A operands of 48 rows over a
+// wavefront's six k-tiles take 114 registers where 64 rows of the 32 x 32 form would take 150, and 24 accumulators
+// make 6 KB of partial sums per wavefront, which fit the raw buffer they replace.  With 32 experts and four of them
+// per token, 256 tokens give an expert 32 rows on average and more than 48 almost never: nearly every expert streams
+// its weights once, where 32-row units stream those of every second expert twice.
+// One K chunk (K <= 3072); tiles, copies, ring and reduction as in gemm_slim_mx_kernel.  EPI = 1 (gate_up of the
+// gpt-oss experts, column tiles walked in (gate, up) pairs): the result is bias + SwiGLU-OAI of each pair, an
+// [M x F] fp32 matrix - half the bytes of the [M x 2 F] sums - which convert_x_mx_kernel then turns into the down
+// projection's activations (the conversion inside the epilogue, as the 32-row kernel has it, does not fit the
+// registers beside the A operands of 48 rows).
+// ------------------------------------------------------------------------------------------
+template <int EPI>
+__global__ void __launch_bounds__(512) gemm_slim_mx48_kernel(const GemmArgs A)
+{
+    typedef GMXFP4 G;
+    constexpr int KTW = 6, KG = 3;                                      // k-tiles and 128-wide K groups per wavefront
+    using L = SlimMxLayout<KTW, 1>;
+    constexpr int CH = L::CH, DI = L::DI, BUF = L::BUF, RING = L::RING;
+    constexpr int DIE = DI + (EPI ? 1 : 0);
+    constexpr int NQ = 3;                                               // results per thread in the reduction
+    static_assert(RING == 3 && BUF >= 24 * 256, "the partial sums replace a raw buffer");
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+    typedef float float4v_t __attribute__((ext_vector_type(4)));
+    extern __shared__ uint8_t smem[];                                   // 8 wavefronts x RING x BUF (+ EPI: bias values)
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int idx = lane & 15, g = lane >> 4;
+    uint8_t* const my_buf = smem + wave * RING * BUF;
+    float* const my_bias = reinterpret_cast<float*>(smem + 8 * RING * BUF) + wave * RING * 32;
+
+    const uint32_t row_bytes = (uint32_t)((int64_t)A.w_bytes / A.N);
+    const int nkt = A.Kp / kBK;
+    const int n32 = (A.N + 31) >> 5;
+
+    int live_tiles = A.m_tiles;
+    if (A.tile_expert) {
+        int c = 0;
+        for (int i = lane; i < A.m_tiles; i += 64) c += A.tile_rows[i] > 0 ? 1 : 0;
+        for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+        live_tiles = __builtin_amdgcn_readfirstlane(c);
+    }
+    const int64_t units = (int64_t)live_tiles * n32;
+    int u = (int)(units * blockIdx.x / gridDim.x);
+    int u_end = (int)(units * (blockIdx.x + 1) / gridDim.x);
+    if (EPI) {                                                          // pairs of (gate, up) column tiles, see gemm_slim_mx_kernel
+        u &= ~1;
+        u_end &= ~1;
+    }
+    auto phys = [&](int j) { return EPI ? (j >> 1) + (j & 1) * (n32 >> 1) : j; };
+
+    while (u < u_end) {
+        const int mt = u / n32, nt0 = u - mt * n32, cnt = min(n32 - nt0, u_end - u);
+        u += cnt;
+        const int kt0 = wave * KTW;
+        const int kcnt = max(0, min(KTW, nkt - kt0));                  // k-tiles of this wavefront
+        int m0, m_rows;
+        const uint8_t* wbase = A.w;
+        if (A.tile_expert) {
+            m0 = A.tile_row0[mt];
+            m_rows = min(48, A.tile_rows[mt]);
+            wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+        } else {
+            m0 = mt * 48;
+            m_rows = min(48, A.M - m0);
+        }
+        const uintptr_t wa = uniform_address(reinterpret_cast<uintptr_t>(wbase));
+        const uint32_t base_delta = (uint32_t)(wa & 3);
+        const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+            reinterpret_cast<void*>(wa & ~(uintptr_t)3), 0, (int)(((uint32_t)A.w_bytes + base_delta + 3u) & ~3u), 0x00020000);
+
+        // A operands: row idx + 16 rb, K block 4 T + g of the wavefront's range = half g & 1 of its k-tile 2 T + g / 2
+        uint4_t ah0[KG][3], al0[KG][3];
+        uint2_t ah1[KG][3], al1[KG][3];
+        uint32_t asa[2][3];                        // scale bytes (hi, lo): group 0 in bytes 0, 1 and group 1 in bytes 2, 3 of [0], group 2 in [1]
+        const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+        const uint32_t hh = (uint32_t)(g & 1);
+#pragma unroll
+        for (int rb = 0; rb < 3; ++rb) {
+            const int ml = idx + 16 * rb;
+            const uint32_t xrow = (uint32_t)(m0 + min(ml, m_rows - 1)) * (uint32_t)(A.xld * 2);
+#pragma unroll
+            for (int T = 0; T < KG; ++T) {
+                const int t = 2 * T + (g >> 1);
+                const bool on = ml < m_rows && t < kcnt;
+                const uint32_t xt = on ? xrow + (uint32_t)(kt0 + t) * 128u : kDeadOffset;
+                ah0[T][rb] = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + 2u * hh * 16u), 0, 0);
+                al0[T][rb] = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (3u + 2u * hh) * 16u), 0, 0);
+                ah1[T][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 16u + 8u * hh), 0, 0);
+                al1[T][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 64u + 8u * hh), 0, 0);
+                const uint32_t two = __builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(xt + 96u + 4u * hh), 0, 0) & 0xffffu;
+                if (T == 0) asa[0][rb] = two;
+                else if (T == 1) asa[0][rb] |= two << 16;
+                else asa[1][rb] = two;
+            }
+        }
+        const uint32_t koff = G::tile_offset(kt0);
+        uint32_t w_off[DI];
+#pragma unroll
+        for (int i = 0; i < DI; ++i) {
+            const int q = i * 64 + lane;
+            const int row = q / CH, chunk = q - row * CH;
+            w_off[i] = (row < 32 && kcnt > 0) ? ((base_delta + (uint32_t)row * row_bytes + koff) & ~3u) + (uint32_t)chunk * 16u : kDeadOffset;
+        }
+        // where the raw rows of this lane's two columns (idx, 16 + idx) start inside their windows
+        uint32_t my_delta[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) my_delta[cb] = (base_delta + (uint32_t)(16 * cb + idx) * row_bytes + koff) & 3u;
+        const float* const eb = EPI && A.epi_bias ? A.epi_bias + (int64_t)(A.tile_expert ? A.tile_expert[mt] : 0) * A.N : nullptr;
+        const uintptr_t ba = uniform_address(reinterpret_cast<uintptr_t>(eb));
+        const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(ba & ~(uintptr_t)3), 0, ba ? A.N * 4 : 0, 0x00020000);
+        const uint32_t bias_off = (uint32_t)lane * 16u;
+        auto issue_one = [&](int i, int b, int q) {
+            const bool any = i < cnt;
+            const uint32_t so = any ? (uint32_t)phys(nt0 + i) * 32u * row_bytes : 0u;
+            if (EPI && q == DI) {
+                if (lane < 8) copy16_to_lds(brs, reinterpret_cast<uint8_t*>(my_bias + b * 32), any ? bias_off + (uint32_t)phys(nt0 + i) * 128u : kDeadOffset, 0u);
+                return;
+            }
+            if (q * 64 + 32 < 32 * CH || lane < 32) copy16_to_lds(wrs, my_buf + b * BUF + q * 1024, any ? w_off[q] : kDeadOffset, so);
+        };
+        auto issue = [&](int i, int b) {
+#pragma unroll
+            for (int q = 0; q < DIE; ++q) issue_one(i, b, q);
+        };
+        // results of this thread in the reduction: accumulator registers a = wave + 8 q of the 24 -
+        // a = (4 (2 rb + cb) + r): row 16 rb + 4 g + r, column 16 cb + idx
+        int64_t coff[NQ];
+        int ncol[NQ], mloc[NQ];
+        bool ok[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int a = wave + 8 * q;
+            mloc[q] = 16 * (a >> 3) + 4 * g + (a & 3);
+            ncol[q] = 16 * ((a >> 2) & 1) + idx;
+            const int m = m0 + min(mloc[q], m_rows - 1);
+            coff[q] = (int64_t)(A.c_rows ? A.c_rows[m] : m) * A.ldc;
+            ok[q] = mloc[q] < m_rows;
+        }
+
+#pragma unroll
+        for (int b = 0; b < RING; ++b) issue(b, b);
+        int b = 0;                                      // buffer of column tile i
+        float pend[NQ], gate[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) pend[q] = gate[q] = 0.f;
+        int pend_n0 = -1;
+        const int width = EPI ? A.N >> 1 : A.N;         // columns of the result
+        auto flush = [&]() {
+            if (pend_n0 >= 0) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q)
+                    if (ok[q] && pend_n0 + ncol[q] < width) A.c[coff[q] + pend_n0 + ncol[q]] = pend[q];
+            }
+        };
+        for (int i = 0; i < cnt; ++i) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RING - 2) * DIE) : "memory");
+            flush();
+            const int b_prev = b == 0 ? RING - 1 : b - 1;      // the buffer of tile i - 1
+            float4v_t acc[3][2];
+#pragma unroll
+            for (int rb = 0; rb < 3; ++rb)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) acc[rb][cb] = float4v_t{0.f, 0.f, 0.f, 0.f};
+            const uint8_t* const raw = my_buf + b * BUF + idx * (CH * 16) + 16 * g;
+#pragma unroll
+            for (int T = 0; T < KG; ++T) {
+                if (2 * T < kcnt) {
+                    // Block 4 T + g of raw row 16 cb + idx starts s = my_delta + 4 T + g (< 16) bytes into its 16-byte
+                    // piece 4 T + g: two aligned 16-byte reads hold it.
+                    int8v_t bq[2];
+                    int sbq[2];
+#pragma unroll
+                    for (int cb = 0; cb < 2; ++cb) {
+                        const uint8_t* const rp = raw + cb * 16 * (CH * 16) + 64 * T;
+                        const uint4_t r0 = *reinterpret_cast<const uint4_t*>(rp), r1 = *reinterpret_cast<const uint4_t*>(rp + 16);
+                        const uint32_t v[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+                        const uint32_t sft = my_delta[cb] + (uint32_t)g + 4u * T;       // scale byte at sft, nibbles behind it
+                        const uint32_t e = (((int)(sft >> 2) != T ? v[T + 1] : v[T]) >> (8 * (sft & 3))) & 0xffu;
+                        const bool up = (int)((sft + 1) >> 2) != T;
+                        const uint32_t b0 = up ? v[T + 1] : v[T], b1 = up ? v[T + 2] : v[T + 1], b2 = up ? v[T + 3] : v[T + 2];
+                        const uint32_t b3 = up ? v[T + 4] : v[T + 3], b4 = up ? v[T + 5] : v[T + 4];
+                        const uint32_t shb = (sft + 1) & 3;
+                        // a block of a k-tile past the wavefront's range or past K: zeros under a scale of one
+                        const bool live = 2 * T + (g >> 1) < kcnt && ((kt0 * 2 + 4 * T + g) * 32 < A.K);
+                        bq[cb] = int8v_t{live ? (int)__builtin_amdgcn_alignbyte(b1, b0, shb) : 0, live ? (int)__builtin_amdgcn_alignbyte(b2, b1, shb) : 0,
+                                         live ? (int)__builtin_amdgcn_alignbyte(b3, b2, shb) : 0, live ? (int)__builtin_amdgcn_alignbyte(b4, b3, shb) : 0,
+                                         0, 0, 0, 0};
+                        sbq[cb] = live ? (int)e : 127;
+                    }
+#pragma unroll
+                    for (int rb = 0; rb < 3; ++rb) {
+                        const int8v_t ahi = {(int)ah0[T][rb].x, (int)ah0[T][rb].y, (int)ah0[T][rb].z, (int)ah0[T][rb].w,
+                                             (int)ah1[T][rb].x, (int)ah1[T][rb].y, 0, 0};
+                        const int8v_t alo = {(int)al0[T][rb].x, (int)al0[T][rb].y, (int)al0[T][rb].z, (int)al0[T][rb].w,
+                                             (int)al1[T][rb].x, (int)al1[T][rb].y, 0, 0};
+                        const int sa2 = (int)asa[T >> 1][rb];
+#pragma unroll
+                        for (int cb = 0; cb < 2; ++cb) {
+                            if (T == 1) {
+                                acc[rb][cb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ahi, bq[cb], acc[rb][cb], 2, 4, 2, sa2, 0, sbq[cb]);
+                                acc[rb][cb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(alo, bq[cb], acc[rb][cb], 2, 4, 3, sa2, 0, sbq[cb]);
+                            } else {
+                                acc[rb][cb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ahi, bq[cb], acc[rb][cb], 2, 4, 0, sa2, 0, sbq[cb]);
+                                acc[rb][cb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(alo, bq[cb], acc[rb][cb], 2, 4, 1, sa2, 0, sbq[cb]);
+                            }
+                        }
+                    }
+                }
+                // the refill of the buffer of tile i - 1, copy by copy behind the groups (see gemm_slim_mx_kernel)
+                if (i > 0) {
+#pragma unroll
+                    for (int q = T; q < DIE; q += KG) issue_one(i - 1 + RING, b_prev, q);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // partial sums of this wavefront's K range -> the buffer it has just consumed
+            float* part = reinterpret_cast<float*>(my_buf + b * BUF);
+#pragma unroll
+            for (int rb = 0; rb < 3; ++rb)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) part[(4 * (2 * rb + cb) + r) * 64 + lane] = acc[rb][cb][r];
+            lds_barrier();
+            float s[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) s[q] = 0.f;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float* pv = reinterpret_cast<const float*>(smem + (v * RING + b) * BUF);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) s[q] += pv[(wave + 8 * q) * 64 + lane];
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) pend[q] = s[q];      // the row scale of this activation layout is one
+            pend_n0 = EPI ? ((nt0 + i) & 1 ? ((nt0 + i) >> 1) * 32 : -1) : (nt0 + i) * 32;      // EPI: a pair's activations after its up tile
+            if constexpr (EPI == 1) {
+                const int j = nt0 + i;
+                if (j & 1) {
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q)
+                        pend[q] = ok[q] ? swiglu_oai(gate[q], s[q] + my_bias[b * 32 + ncol[q]], A.epi_alpha, A.epi_limit) : 0.f;
+                } else {
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) gate[q] = s[q] + my_bias[b * 32 + ncol[q]];
+                }
+            }
+            lds_barrier();                              // every partial sum has been read: the buffers may be refilled
+            b = b + 1 == RING ? 0 : b + 1;
+        }
+        flush();
+    }
+}
+
 template <int KTW, int RB, int EPI = 0>
 bool launch_slim_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
@@ -2557,6 +2815,34 @@ bool launch_slim_for(const GemmArgs& a, int ktw, int m_tiles, hipStream_t stream
 template <typename G>
 constexpr bool kWide128 = G::kSup == 2 || G::kRawRow > 144 || std::is_same<G, GQ4K>::value;
 
+// 48-row units (gemm_slim_mx48_kernel): one K chunk
+template <int EPI>
+bool launch_slim_mx48(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
+{
+    using L = SlimMxLayout<6, 1>;
+    auto kern = gemm_slim_mx48_kernel<EPI>;
+    constexpr size_t lds = (size_t)8 * L::RING * L::BUF + (EPI ? 8 * L::RING * 128 : 64);
+    static_assert(lds <= 160 * 1024, "raw buffers must fit LDS");
+    if (a.Kp / kBK > 48 || a.accumulate || (EPI && (a.N & 63))) {
+        set_last_error("gemm: 48-row units take K <= 3072, no accumulation and, with the fused epilogue, whole column tiles.");
+        return false;
+    }
+    if (cs.need_out) {
+        *cs.need_out = 0;
+        return true;
+    }
+    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    a.m_tiles = m_tiles;
+    a.n_tiles = (a.N + 31) / 32;
+    a.chunk_kt = 48;
+    a.k_chunks = 1;
+    a.partial = nullptr;
+    const int64_t units = (int64_t)m_tiles * a.n_tiles;
+    const int grid = (int)std::min<int64_t>(units, device_info().num_cus);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
+    return hip_ok(hipGetLastError(), "gemm launch");
+}
+
 template <typename G>
 bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
@@ -2572,7 +2858,8 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
             if (bm == 256 && !a.tile_expert) return launch_mx<256>(a, m_tiles, stream, cs);
             if (bm == 128 && !a.tile_expert) return launch_mx<128>(a, m_tiles, stream, cs);
             if (bm == 32) return launch_slim_mx_for<1>(a, m_tiles, stream, cs);
-            set_last_error("gemm: the MX activation layout serves 32-row units and plain launches of 128- and 256-row tiles.");
+            if (bm == 48) return launch_slim_mx48<0>(a, m_tiles, stream, cs);
+            set_last_error("gemm: the MX activation layout serves 32- and 48-row units and plain launches of 128- and 256-row tiles.");
             return false;
         }
         if (bm == 256 && !a.tile_expert) return launch_xw<PMXFP4, 256, 4>(a, m_tiles, stream, cs);
@@ -2801,11 +3088,11 @@ bool gemm_swiglu_mx_fits(int F, int K)
     return F > 0 && F % 32 == 0 && kt > 16 && kt <= 48 && F <= 32768;
 }
 
-bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace_out, const float* bias, float alpha, float limit,
-                           int M, int F, int K, const GemmTiles* tiles, hipStream_t stream)
+bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace_out, float* act, const float* bias, float alpha,
+                           float limit, int M, int F, int K, const GemmTiles* tiles, hipStream_t stream)
 {
-    if (!tiles || tiles->bm != 32 || !gemm_swiglu_mx_fits(F, K)) {
-        set_last_error("gemm: the fused SwiGLU epilogue takes 32-row expert tiles, F a multiple of 32 and 1025 .. 3072 columns of K.");
+    if (!tiles || (tiles->bm != 32 && tiles->bm != 48) || !gemm_swiglu_mx_fits(F, K)) {
+        set_last_error("gemm: the fused SwiGLU epilogue takes 32- or 48-row expert tiles, F a multiple of 32 and 1025 .. 3072 columns of K.");
         return false;
     }
     GemmArgs a{};
@@ -2835,6 +3122,13 @@ bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace
     a.expert_stride = tiles->expert_stride;
     if (tiles->count == 0) return true;
     const ChunkScratch cs{nullptr, 0, nullptr};
+    if (tiles->bm == 48) {
+        // 48-row units leave the activations as fp32 [M x F] in act; the conversion is a launch of its own
+        a.c = act;
+        a.ldc = F;
+        return launch_slim_mx48<1>(a, tiles->count, stream, cs) &&
+               launch_convert_x(kTypeMXFP4, act, F, nullptr, M, F, workspace_out, stream, nullptr, 0.f, 1);
+    }
     return a.Kp / kBK <= 32 ? launch_slim_mx<4, 1, 1>(a, tiles->count, stream, cs) : launch_slim_mx<6, 1, 1>(a, tiles->count, stream, cs);
 }
 

@@ -97,13 +97,12 @@ __global__ void __launch_bounds__(1024) moe_group_kernel(const int* __restrict__
     }
     __syncthreads();
     // exclusive scans of the row counts and of the tile counts: one wavefront, 64 experts per step
-    const int bm_shift = __ffs(bm) - 1;          // bm is a power of two
     if (wave == 0) {
         int carry_o = 0, carry_t = 0;
         for (int e0 = 0; e0 < E; e0 += 64) {
             const int e = e0 + lane;
             const int c = e < E ? cnt[e] : 0;
-            const int nt = (c + bm - 1) >> bm_shift;
+            const int nt = (c + bm - 1) / bm;
             int so = c, st = nt;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
@@ -154,7 +153,7 @@ __global__ void __launch_bounds__(1024) moe_group_kernel(const int* __restrict__
     }
     for (int e = wave; e < E; e += nw) {
         const int rows = off[e + 1] - off[e];
-        const int nt = (rows + bm - 1) >> bm_shift;
+        const int nt = (rows + bm - 1) / bm;
         for (int j = lane; j < nt; j += 64) {
             M.tile_expert[tbeg[e] + j] = e;
             M.tile_row0[tbeg[e] + j] = off[e] + j * bm;

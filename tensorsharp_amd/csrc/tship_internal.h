@@ -163,11 +163,12 @@ struct GemmTiles {
 
 // The gate_up GEMM of MXFP4 gpt-oss experts on 32-row tiles with the down projection's activations as its result:
 // bias + SwiGLU-OAI of every (gate, up) column pair, converted to the MX activation layout in workspace_out (a
-// gemm_workspace_bytes(M, F) buffer), without the [M x 2 F] matrix in between.  workspace holds the MX activations of
+// gemm_workspace_bytes(M, F) buffer), without the [M x 2 F] matrix in between (48-row tiles pass through act, an
+// [M x F] fp32 scratch matrix, on the way).  workspace holds the MX activations of
 // the M rows x K (launch_convert_x with layout 1).  gemm_swiglu_mx_fits: whether the shape can take this path.
 bool gemm_swiglu_mx_fits(int F, int K);
-bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace_out, const float* bias, float alpha, float limit,
-                           int M, int F, int K, const GemmTiles* tiles, hipStream_t stream);
+bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace_out, float* act, const float* bias, float alpha,
+                           float limit, int M, int F, int K, const GemmTiles* tiles, hipStream_t stream);
 
 // c[row] (row = c_rows ? c_rows[m] : m) [N] = x16[m] . W^T * scale[m], m < M
 // accumulate: c[row] += ... instead of c[row] = ...
