@@ -126,9 +126,10 @@ def test_unbalanced_and_empty_experts(hip, oracle):
 # MXFP4 experts whose gate_up rows are 1025 .. 3072 long form bias + SwiGLU in the gate_up GEMM's epilogue and write the
 # down projection's block-scaled activations from there: row lengths at both ends of that range and of both k-tile
 # counts per wavefront, F / 32 even and odd (an odd count leaves half a k-tile of padding), experts with more than 32
-# tokens (two row tiles), partly filled tiles and empty experts, with and without biases.
+# tokens (two row tiles), partly filled tiles and empty experts, with and without biases.  More than 20 tokens per expert
+# on average (the first two cases and the last) run in 48-row units, the others in 32-row units.
 @pytest.mark.parametrize("E,H,F,T,k", [(4, 1088, 160, 70, 2), (4, 2048, 256, 130, 2), (8, 2880, 96, 40, 4),
-                                       (4, 3072, 512, 9, 2), (4, 1536, 2880, 40, 2)])
+                                       (4, 3072, 512, 9, 2), (4, 1536, 2880, 40, 2), (2, 3072, 1024, 60, 2)])
 def test_gate_up_epilogue_writes_down_activations(hip, oracle, E, H, F, T, k):
     rng = np.random.default_rng(1000 + H + F)
     gu, gb, dn, db = make_experts(oracle, MXFP4, E, H, F, rng, sigma=0.03)
