@@ -150,6 +150,9 @@ def main():
     ap.add_argument("--matmul", metavar="TYPE,M,N,K",
                     help="time only one matmul shape (GGUF type id, rows, out features, in features) through "
                          "TSHip_AddmmQuantF32Device, --steps calls after --warmup; for profiling a single kernel")
+    ap.add_argument("--moe", metavar="T", type=int,
+                    help="time only the configs[3] MoE expert stage (32 MXFP4 experts, top-4, 2880) at T tokens, --steps calls; "
+                         "for profiling its kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU kernel path only: this build has no multi-GPU code; run with --gpus 1.",
@@ -202,10 +205,53 @@ def main():
         return {"us_per_call_events": round(us, 2), "bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
                 "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)}
 
+    # MoE expert stage (configs[3]): 32 MXFP4 experts, top-4, hidden 2880; T = 1 (decode, HBM-bound:
+    # bytes of the 4 selected experts' gate_up + down blocks) and T = 256 (prefill, grouped GEMM)
+    def moe(T, iters):
+        E, H, F, k = 32, 2880, 2880, 4
+        sets = [(synth.random_weight(MXFP4, E * 2 * F, H, dev, seed=500 + c),
+                 synth.random_weight(MXFP4, E * H, F, dev, seed=600 + c)) for c in range(2)]
+        hidden = torch.randn((T, H), device=dev, dtype=torch.float32)
+        gi = torch.Generator(device="cpu")
+        gi.manual_seed(11)
+        idsets = [torch.stack([torch.randperm(E, generator=gi)[:k] for _ in range(T)]).to(torch.int32).to(dev)
+                  for _ in range(8)]
+        wts = torch.softmax(torch.randn((T, k), device=dev), dim=1).contiguous()
+
+        def f(i):
+            gu, dn = sets[i % 2]
+            HipBasicOps.MoEExpertsGptOssForward(hidden, idsets[i % 8], wts, gu, None, dn, None, MXFP4, E, H, F)
+        for i in range(5):
+            f(i)
+        ev, wall = time_region(f, iters, torch)
+        us = ev * 1e3 / iters
+        res = {"us_per_call_events": round(us, 1)}
+        if T == 1:
+            b = k * (2 * F + H) * row_bytes(MXFP4, H)
+            res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                        "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)})
+        else:
+            # weight-streaming bound (about 120 FLOP per weight byte): bytes of all 32 experts are the figure
+            # of merit, TFLOP/s beside it
+            b = E * (2 * F + H) * row_bytes(MXFP4, H)
+            fl = 2.0 * T * k * (2 * F * H + H * F)
+            res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
+                        "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1),
+                        "TFLOPs": round(fl / (us * 1e-6) / 1e12, 1),
+                        "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / MFMA_FP16_PEAK_TFLOPS, 1)})
+        return res
+
+
     if args.aux:
         op, t, rows, k = args.aux.split(",")
         r = aux_case(op, int(t), int(rows), int(k), args.steps, args.warmup)
         r["aux"] = {"op": op, "type": int(t), "rows": int(rows), "K": int(k)}
+        print(json.dumps(r))
+        return
+
+    if args.moe:
+        r = moe(args.moe, args.steps)
+        r["moe"] = {"tokens": args.moe}
         print(json.dumps(r))
         return
 
@@ -332,7 +378,7 @@ def main():
             "bound": "mfma", "achieved": mx["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(mx["TFLOPs"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
             "workload": "MXFP4 prefill GEMM M=2048 N=21504 K=5376: raw fp4 blocks x two MX fp6 (E2M3) activation terms, f32 accumulate",
-            "kernel": "tship::gemm_mx_kernel<256, 3> (+ tship::convert_x_kernel<1000, ...> on the activations, inside the timed call)",
+            "kernel": "tship::gemm_mx_kernel<256, 3> (+ tship::convert_x_mx_kernel on the activations, inside the timed call)",
             "avg_call_us": mx["us_per_call_events"], "flops_per_call": 2 * pm * pn * pk, "calls_timed": 20,
             "instruction_ops_over_fp6_fp4_peak": round(2 * mx["TFLOPs"] / MFMA_FP6_FP4_PEAK_TFLOPS, 4)}
 
@@ -386,42 +432,6 @@ def main():
             r.update({"bytes": b, "GBps": round(b / (r["us_per_call_events"] * 1e-6) / 1e9, 1)})
             extra[f"q4_k_gemm_{m}x14336x4096"] = r
         extra["q6_k_gemm_512x14336x4096"] = prefill(Q6_K, 512, 14336, 4096)
-        # MoE expert stage (configs[3]): 32 MXFP4 experts, top-4, hidden 2880; T = 1 (decode, HBM-bound:
-        # bytes of the 4 selected experts' gate_up + down blocks) and T = 256 (prefill, grouped GEMM)
-        def moe(T, iters):
-            E, H, F, k = 32, 2880, 2880, 4
-            sets = [(synth.random_weight(MXFP4, E * 2 * F, H, dev, seed=500 + c),
-                     synth.random_weight(MXFP4, E * H, F, dev, seed=600 + c)) for c in range(2)]
-            hidden = torch.randn((T, H), device=dev, dtype=torch.float32)
-            gi = torch.Generator(device="cpu")
-            gi.manual_seed(11)
-            idsets = [torch.stack([torch.randperm(E, generator=gi)[:k] for _ in range(T)]).to(torch.int32).to(dev)
-                      for _ in range(8)]
-            wts = torch.softmax(torch.randn((T, k), device=dev), dim=1).contiguous()
-
-            def f(i):
-                gu, dn = sets[i % 2]
-                HipBasicOps.MoEExpertsGptOssForward(hidden, idsets[i % 8], wts, gu, None, dn, None, MXFP4, E, H, F)
-            for i in range(5):
-                f(i)
-            ev, wall = time_region(f, iters, torch)
-            us = ev * 1e3 / iters
-            res = {"us_per_call_events": round(us, 1)}
-            if T == 1:
-                b = k * (2 * F + H) * row_bytes(MXFP4, H)
-                res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
-                            "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1)})
-            else:
-                # weight-streaming bound (about 120 FLOP per weight byte): bytes of all 32 experts are the figure
-                # of merit, TFLOP/s beside it
-                b = E * (2 * F + H) * row_bytes(MXFP4, H)
-                fl = 2.0 * T * k * (2 * F * H + H * F)
-                res.update({"bytes": b, "GBps": round(b / (us * 1e-6) / 1e9, 1),
-                            "pct_hbm_peak": round(100 * b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 1),
-                            "TFLOPs": round(fl / (us * 1e-6) / 1e12, 1),
-                            "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / MFMA_FP16_PEAK_TFLOPS, 1)})
-            return res
-
         extra["cfg4_mxfp4_moe_experts_T1"] = moe(1, n_it)
         extra["cfg4_mxfp4_moe_experts_T256"] = moe(256, 30)
         # whole-layer decode (TransformerLayerDecode) at configs[1] shapes: hidden 4096, 32 heads / 8 KV heads of 128,
