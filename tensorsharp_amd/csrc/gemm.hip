@@ -2665,6 +2665,7 @@ __global__ void __launch_bounds__(512) gemm_slim_mx48_kernel(const GemmArgs A)
                     }
 #pragma unroll
                     for (int rb = 0; rb < 3; ++rb) {
+                        if (16 * rb >= m_rows) continue;              // a row block without rows (uniform)
                         const int8v_t ahi = {(int)ah0[T][rb].x, (int)ah0[T][rb].y, (int)ah0[T][rb].z, (int)ah0[T][rb].w,
                                              (int)ah1[T][rb].x, (int)ah1[T][rb].y, 0, 0};
                         const int8v_t alo = {(int)al0[T][rb].x, (int)al0[T][rb].y, (int)al0[T][rb].z, (int)al0[T][rb].w,
