@@ -347,29 +347,40 @@ __global__ void __launch_bounds__(kMxCvtBlocks) convert_x_mx_kernel(const Conver
         rms = 1.0f / sqrtf((float)(tot / (double)K) + S.eps);
     }
     const int q0 = chunk * T * 8;                // first float4 of the chunk
+    // every load of the thread is issued before the first value is used: no branch between them (float4s past the row
+    // read its last one and become zeros afterwards)
+    float4 v[8], w[8];
+    int qs[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int ql = tid + j * T, q = q0 + ql;
-        float4 v = float4{0.f, 0.f, 0.f, 0.f};
-        if (q < k4) {
-            if (SRC == kSrcSwiglu) {
-                float4 g = reinterpret_cast<const float4*>(src)[q], u = reinterpret_cast<const float4*>(src + K)[q];
-                if (bias) {
-                    const float4 bg = reinterpret_cast<const float4*>(bias)[q], bu = reinterpret_cast<const float4*>(bias + K)[q];
-                    g = float4{g.x + bg.x, g.y + bg.y, g.z + bg.z, g.w + bg.w};
-                    u = float4{u.x + bu.x, u.y + bu.y, u.z + bu.z, u.w + bu.w};
-                }
-                v = float4{swiglu_oai(g.x, u.x, S.alpha, S.limit), swiglu_oai(g.y, u.y, S.alpha, S.limit),
-                           swiglu_oai(g.z, u.z, S.alpha, S.limit), swiglu_oai(g.w, u.w, S.alpha, S.limit)};
-            } else {
-                v = reinterpret_cast<const float4*>(src)[q];
-                if (norm_w) {
-                    const float4 wv = reinterpret_cast<const float4*>(norm_w)[q];
-                    v = float4{(v.x * rms) * wv.x, (v.y * rms) * wv.y, (v.z * rms) * wv.z, (v.w * rms) * wv.w};
-                }
+    for (int j = 0; j < 8; ++j) qs[j] = min(q0 + tid + j * T, k4 - 1);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = reinterpret_cast<const float4*>(src)[qs[j]];
+    if (SRC == kSrcSwiglu) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = reinterpret_cast<const float4*>(src + K)[qs[j]];
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float4 bg = reinterpret_cast<const float4*>(bias)[qs[j]], bu = reinterpret_cast<const float4*>(bias + K)[qs[j]];
+                v[j] = float4{v[j].x + bg.x, v[j].y + bg.y, v[j].z + bg.z, v[j].w + bg.w};
+                w[j] = float4{w[j].x + bu.x, w[j].y + bu.y, w[j].z + bu.z, w[j].w + bu.w};
             }
         }
-        stage[(ql >> 3) * 9 + (ql & 7)] = v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            v[j] = float4{swiglu_oai(v[j].x, w[j].x, S.alpha, S.limit), swiglu_oai(v[j].y, w[j].y, S.alpha, S.limit),
+                          swiglu_oai(v[j].z, w[j].z, S.alpha, S.limit), swiglu_oai(v[j].w, w[j].w, S.alpha, S.limit)};
+    } else if (norm_w) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = reinterpret_cast<const float4*>(norm_w)[qs[j]];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            v[j] = float4{(v[j].x * rms) * w[j].x, (v[j].y * rms) * w[j].y, (v[j].z * rms) * w[j].z, (v[j].w * rms) * w[j].w};
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int ql = tid + j * T;
+        stage[(ql >> 3) * 9 + (ql & 7)] = q0 + ql < k4 ? v[j] : float4{0.f, 0.f, 0.f, 0.f};
     }
     __syncthreads();
     const int blk = chunk * T + tid;             // this thread's block of the row
