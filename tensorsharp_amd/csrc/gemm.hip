@@ -2869,6 +2869,12 @@ bool launch_for_type(const GemmArgs& a, int bm, int m_tiles, hipStream_t stream,
         if (a.x_mx) {
             if (bm == 256 && !a.tile_expert) return launch_mx<256>(a, m_tiles, stream, cs);
             if (bm == 128 && !a.tile_expert) return launch_mx<128>(a, m_tiles, stream, cs);
+            // a plain small batch whose K fits one chunk, in 48-row units where those are at most two thirds as many as
+            // 32-row units (33 .. 48, 65 .. 96, 129 .. 144 rows): a unit less is a pass less over the weights, and a 48-row
+            // pass costs a little more than a 32-row one (32 x 184320 x 2880 65 us; 48 rows 77 instead of 97, 96 rows 132
+            // instead of 164, but 128 rows 208 instead of 186)
+            if (bm == 32 && !a.tile_expert && !a.accumulate && a.Kp / kBK <= 48 && 3 * ((a.M + 47) / 48) <= 2 * ((a.M + 31) / 32))
+                return launch_slim_mx48<0>(a, (a.M + 47) / 48, stream, cs);
             if (bm == 32) return launch_slim_mx_for<1>(a, m_tiles, stream, cs);
             if (bm == 48) return launch_slim_mx48<0>(a, m_tiles, stream, cs);
             set_last_error("gemm: the MX activation layout serves 32- and 48-row units and plain launches of 128- and 256-row tiles.");

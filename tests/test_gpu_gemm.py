@@ -325,6 +325,27 @@ def test_mxfp4_block_scaled_small_batch_large_weight(hip, oracle, M):
     check(y[:, cols], ref, ("mx small batch", M))
 
 
+@pytest.mark.parametrize("M", [40, 48, 90, 130])
+def test_mxfp4_block_scaled_small_batch_48_row_units(hip, oracle, M):
+    """With K in one chunk (K <= 3072) a small batch over a large weight runs in 48-row units where they are at most two
+    thirds as many as 32-row units (40, 48, 90 and 130 rows: 1, 1, 2 and 3 units instead of 2, 2, 3 and 5; the last unit
+    of 130 holds 34 rows).  N is not a multiple of 32 and K not of 64."""
+    import torch
+    from tensorsharp_amd import QuantizedWeight
+    rng = np.random.default_rng(100 + M)
+    N, K = 24010, 2848
+    wq = inputs.random_blocks("mxfp4", N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(torch.from_numpy(wq).cuda(), MXFP4, K, N))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+    cols = np.unique(np.concatenate([[0, 15, 16, 31, 32, N - 1, N - 10], rng.integers(0, N, 300)]))
+    rb = K // 32 * 17
+    sub = np.concatenate([wq[c * rb:(c + 1) * rb] for c in cols])
+    ref = oracle.matmul_f64(MXFP4, sub, len(cols), K, x)
+    check(y[:, cols], ref, ("mx 48-row units", M))
+
+
 def test_q6_k_128_row_tiles(hip, oracle):
     from oracle.oracle import Q6_K
     rng = np.random.default_rng(77)
