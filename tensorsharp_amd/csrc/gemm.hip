@@ -819,6 +819,7 @@ struct ChunkScratch {
 inline float* chunk_scratch(const ChunkScratch& cs, size_t bytes) { return bytes <= cs.bytes ? cs.ptr : nullptr; }
 __global__ void gemm_chunk_sum_kernel(const float* __restrict__ partial, int k_chunks, int M, int N, const int* __restrict__ c_rows,
                                       float* __restrict__ c, int64_t ldc, int accumulate);
+bool launch_chunk_sum(const GemmArgs& a, hipStream_t stream);
 
 // BM x 256 x 64 tiles, eight wavefronts, each owning all BM rows of 32 output columns.
 //   * Activation k-tiles (fp16) and raw weight super-tiles go from global memory straight into LDS
@@ -1532,9 +1533,7 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratc
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (a.partial) {
-        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
-                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
-        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+        return launch_chunk_sum(a, stream);
     }
     return true;
 }
@@ -1574,9 +1573,7 @@ bool launch_xw(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
     hipLaunchKernelGGL(kern, dim3(grid), dim3(128 * WN), lds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (a.partial) {
-        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
-                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
-        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+        return launch_chunk_sum(a, stream);
     }
     return true;
 }
@@ -1887,9 +1884,7 @@ bool launch_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kLds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (a.partial) {
-        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
-                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
-        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+        return launch_chunk_sum(a, stream);
     }
     return true;
 }
@@ -2117,6 +2112,38 @@ __global__ void __launch_bounds__(256) gemm_chunk_sum_kernel(const float* __rest
     }
 }
 
+// the same, four columns per thread (N, ldc multiples of 4, c 16-byte aligned)
+__global__ void __launch_bounds__(256) gemm_chunk_sum4_kernel(const float* __restrict__ partial, int k_chunks, int M, int N,
+                                                              const int* __restrict__ c_rows, float* __restrict__ c, int64_t ldc,
+                                                              int accumulate)
+{
+    const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (n >= N) return;
+    for (int m = blockIdx.y; m < M; m += gridDim.y) {
+        float4* out = reinterpret_cast<float4*>(c + (int64_t)(c_rows ? c_rows[m] : m) * ldc + n);
+        float4 s = accumulate ? *out : float4{0.f, 0.f, 0.f, 0.f};
+        for (int kc = 0; kc < k_chunks; ++kc) {
+            const float4 v = *reinterpret_cast<const float4*>(partial + ((int64_t)kc * M + m) * N + n);
+            s = float4{s.x + v.x, s.y + v.y, s.z + v.z, s.w + v.w};
+        }
+        *out = s;
+    }
+}
+
+// c[row] (+)= the chunk sums of a launch whose K was cut into chunks
+bool launch_chunk_sum(const GemmArgs& a, hipStream_t stream)
+{
+    const bool vec = (a.N & 3) == 0 && (a.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(a.c) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.partial) & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL(gemm_chunk_sum4_kernel, dim3((a.N / 4 + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
+                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
+    else
+        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial,
+                           a.k_chunks, a.M, a.N, a.c_rows, a.c, a.ldc, a.accumulate);
+    return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+}
+
 template <typename G, int KTW>
 bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& cs)
 {
@@ -2146,9 +2173,7 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (two_pass) {
-        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial, a.k_chunks, a.M, a.N,
-                           a.c_rows, a.c, a.ldc, a.accumulate);
-        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+        return launch_chunk_sum(a, stream);
     }
     return true;
 }
@@ -2773,9 +2798,7 @@ bool launch_slim_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScra
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, a);
     if (!hip_ok(hipGetLastError(), "gemm launch")) return false;
     if (two_pass) {
-        hipLaunchKernelGGL(gemm_chunk_sum_kernel, dim3((a.N + 255) / 256, std::min(a.M, 65535)), dim3(256), 0, stream, a.partial, a.k_chunks, a.M, a.N,
-                           a.c_rows, a.c, a.ldc, a.accumulate);
-        return hip_ok(hipGetLastError(), "gemm chunk sum launch");
+        return launch_chunk_sum(a, stream);
     }
     return true;
 }
