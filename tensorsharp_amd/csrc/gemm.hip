@@ -783,6 +783,32 @@ __device__ __forceinline__ void wait_copies_and_barrier()
 // Epilogue of one wavefront: D[row = 32 i + 8 (r / 4) + 4 h + r % 4][column my_n] times the row scale.
 // The scales (and scatter indices) of a 32-row block are loaded before its stores: the result may
 // alias them as far as the compiler knows, so a load placed after a store would wait for it.
+// Plain stores of a wavefront's TMW x NB blocks of 32 x 32 (no scatter, no accumulation).  Loads and stores share one
+// counter that retires in order, so row scales loaded from global memory behind a block's stores would wait until those
+// stores have been acknowledged, once per row block: the scales come from LDS (tile_scales[row of the tile], put there
+// in the kernel's prologue) or are one (kUnitScale), and nothing stands between the stores.
+template <int TMW, int NB, bool kUnitScale>
+__device__ __forceinline__ void store_wave_tile(const float* tile_scales, const float16_t (&acc)[TMW][NB], float* cdst, int64_t ldc, int N,
+                                                int m0, int m_rows, int row_first, int n_first, int h)
+{
+#pragma unroll
+    for (int m = 0; m < TMW; ++m) {
+        float sc[16];
+#pragma unroll
+        for (int r2 = 0; r2 < 16; ++r2) sc[r2] = kUnitScale ? 1.0f : tile_scales[row_first + m * 32 + 8 * (r2 >> 2) + 4 * h + (r2 & 3)];
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const int my_n = n_first + 32 * n;
+            if (my_n >= N) continue;
+#pragma unroll
+            for (int r2 = 0; r2 < 16; ++r2) {
+                const int ml = row_first + m * 32 + 8 * (r2 >> 2) + 4 * h + (r2 & 3);
+                if (ml < m_rows) cdst[(int64_t)(m0 + ml) * ldc + my_n] = kUnitScale ? acc[m][n][r2] : acc[m][n][r2] * sc[r2];
+            }
+        }
+    }
+}
+
 template <int TM>
 __device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&acc)[TM], int m0, int m_rows, int my_n, int h)
 {
@@ -1187,6 +1213,7 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
     uint8_t* const rraw = xbuf + ST * kXTile;             // ST x kRawTile
     uint8_t* const bex = rraw + ST * kRawTile;            // 2 x kBTile
     uint8_t* const dump = bex + 2 * kBTile;               // 1 KiB
+    float* const tile_scales = reinterpret_cast<float*>(dump + 1024);      // BM row scales for the epilogue
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1296,6 +1323,7 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
     for (int i = 0; i < XI; ++i) issue_x1(kt_begin, i);
 #pragma unroll
     for (int i = 0; i < RI; ++i) issue_raw1(kt_begin + 1, i);
+    if (tid < BM) tile_scales[tid] = A.xscale[m0 + min(tid, m_rows - 1)];
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < DUTY; ++u) {
@@ -1449,6 +1477,10 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
         c_rows = nullptr;
         accumulate = 0;
     }
+    if (!c_rows && !accumulate) {
+        store_wave_tile<TMW, NB, false>(tile_scales, acc, cdst, ldc, A.N, m0, m_rows, wm * (BM / 2), n0 + 32 * NB * wn + col, h);
+        return;
+    }
 #pragma unroll
     for (int m = 0; m < TMW; ++m) {
         float sc[16];
@@ -1543,7 +1575,7 @@ bool launch_xw(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
 {
     constexpr int BN = 256;
     auto kern = gemm_xw_kernel<P, BM, WN>;
-    constexpr size_t kLds = (size_t)2 * BM * kXRow + (size_t)2 * BN * P::kRowBytes + (size_t)2 * 4 * 2 * BN * 16 + 1024;
+    constexpr size_t kLds = (size_t)2 * BM * kXRow + (size_t)2 * BN * P::kRowBytes + (size_t)2 * 4 * 2 * BN * 16 + 1024 + BM * 4;
     static_assert(kLds <= 160 * 1024, "LDS");
     const size_t lds = kLds;
     if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
@@ -1824,6 +1856,10 @@ __global__ void __launch_bounds__(512) gemm_mx_kernel(const GemmArgs A)
         ldc = A.N;
         c_rows = nullptr;
         accumulate = 0;
+    }
+    if (!c_rows && !accumulate) {
+        store_wave_tile<TMW, NB, true>(nullptr, acc, cdst, ldc, A.N, m0, m_rows, wm * (BM / 2), n0 + 32 * NB * wn + col, h);
+        return;
     }
 #pragma unroll
     for (int m = 0; m < TMW; ++m) {
