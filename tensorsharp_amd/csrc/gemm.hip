@@ -810,9 +810,26 @@ __device__ __forceinline__ void store_wave_tile(const float* tile_scales, const 
 }
 
 template <int TM>
-__device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&acc)[TM], int m0, int m_rows, int my_n, int h)
+__device__ __forceinline__ void store_tile(const GemmArgs& A, const float16_t (&acc)[TM], int m0, int m_rows, int my_n, int h,
+                                           const float* tile_scales)
 {
     if (my_n >= A.N) return;
+    if (!A.c_rows && !A.accumulate) {
+        // plain stores with the row scales from LDS (tile_scales[row of the tile]): a scale loaded from global memory
+        // behind a row block's stores would wait until they have been acknowledged (one counter tracks both)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            float sc[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[r] = tile_scales[i * 32 + 8 * (r >> 2) + 4 * h + (r & 3)];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ml = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (ml < m_rows) A.c[(int64_t)(m0 + ml) * A.ldc + my_n] = acc[i][r] * sc[r];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         float sc[16], old[16];
@@ -881,6 +898,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
     uint8_t* const xbuf = smem;                          // XST x kXTile
     uint8_t* const rbuf = smem + XST * kXTile;           // RB x RT
     uint8_t* const dump = rbuf + RB * RT;          // 1 KiB
+    float* const tile_scales = reinterpret_cast<float*>(dump + 1024);      // BM row scales for the epilogue
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -981,6 +999,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
     for (int i = 0; i < RL; ++i) issue_w(s + i);
 #pragma unroll
     for (int i = 0; i < D; ++i) issue_x(kt_begin + i);
+    for (int i = threadIdx.x; i < BM; i += NW * 64) tile_scales[i] = A.xscale[m0 + min(i, m_rows - 1)];
     __syncthreads();
     uint32_t oc[16], on[16];
     {
@@ -1040,9 +1059,9 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         P.ldc = A.N;
         P.c_rows = nullptr;
         P.accumulate = 0;
-        store_tile<TM>(P, acc, m0, m_rows, my_n, h);
+        store_tile<TM>(P, acc, m0, m_rows, my_n, h, tile_scales);
     } else {
-        store_tile<TM>(A, acc, m0, m_rows, my_n, h);
+        store_tile<TM>(A, acc, m0, m_rows, my_n, h, tile_scales);
     }
 }
 
@@ -1532,7 +1551,7 @@ bool launch_tiles(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratc
     constexpr int BN = NW * 32, RT = BN * G::kRawRow;
     auto kern = gemm_kernel<G, BM, XST, NW>;
     constexpr int RB = (XST > 2 && G::kSup == 2) ? 3 : 2;
-    const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * RT + 1024;
+    const size_t lds = (size_t)XST * BM * kXRow + (size_t)RB * RT + 1024 + BM * 4;
     if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     a.m_tiles = m_tiles;
     a.n_tiles = (a.N + BN - 1) / BN;
