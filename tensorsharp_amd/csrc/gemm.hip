@@ -2246,7 +2246,7 @@ bool launch_slim(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch
 template <int KTW, int RB>
 struct SlimMxLayout {
     static constexpr int kNeed = (GMXFP4::window_bytes(KTW) + 15) / 16;
-    static constexpr int CH = kNeed | 1;                                 // odd: the dword reads of the 32 rows spread over the banks
+    static constexpr int CH = kNeed | 1;                                 // odd: the 16-byte reads of 16 rows cover the banks once
     static constexpr int DI = (32 * CH + 63) / 64;
     static constexpr int RAW = 32 * CH * 16;
     static constexpr int BUF = RAW > RB * 4096 ? RAW : RB * 4096;        // raw rows, later RB x 32 x 32 fp32 partial sums
@@ -3077,9 +3077,9 @@ bool launch_convert(int type, const ConvertSrc& src, int M, int K, void* workspa
 
 // Which activation layout the GEMM of this shape reads: 0 fp16 in the format's unpack order; 1 two MX fp6 terms for
 // gemm_mx_kernel (plain MXFP4 launches on 128- or 256-row tiles).
-// (rows longer than the convert kernel holds in registers stay on the fp16 path, and so do small batches over small
-// weights, where the costlier conversion outweighs the kernel's gain: 64 x 5760 x 2880 20.2 vs 17.6 us, but
-// 32 x 184320 x 2880 73.6 vs 83.8 us)
+// (rows longer than 32768 stay on the fp16 path, whose tile kernels cut such a K into chunks, and so do small batches
+// over small weights, which gain nothing: 64 x 5760 x 2880 18.2 vs 17.7 us, 16 x 4096 x 14336 26.9 vs 23.0 us, but
+// 32 x 184320 x 2880 61-67 vs 74-84 us)
 int gemm_x_layout(int type, int M, int N, int K)
 {
     if (type != kTypeMXFP4 || K > 1024 * kCvtHold * 4) return 0;
