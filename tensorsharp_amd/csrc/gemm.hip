@@ -2641,23 +2641,39 @@ __global__ void __launch_bounds__(512) gemm_slim_mx48_kernel(const GemmArgs A)
         uint32_t asa[2][3];                        // scale bytes (hi, lo): group 0 in bytes 0, 1 and group 1 in bytes 2, 3 of [0], group 2 in [1]
         const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
         const uint32_t hh = (uint32_t)(g & 1);
+        // They reach the registers through the wavefront's (still empty) raw buffers: LDS-direct copies of whole row
+        // pieces - 768 contiguous bytes per row, one row block of 16 rows per pass - and 16-byte LDS reads from there.
+        // Loading them straight from memory (a lane per row and K block, 45 instructions of scattered 16-byte pieces
+        // per wavefront) took 10 us of a launch: every CU asked the L2 for five pieces of each 128-byte line separately.
+        {
+            constexpr int kRowPieces = KTW * 8 + 1;                     // 49: one piece of padding spreads the rows over the banks
+            constexpr int kPassCopies = (16 * kRowPieces + 63) / 64;    // 13
+            static_assert(kPassCopies * 1024 <= RING * BUF, "a pass of 16 rows fits the ring");
+            const uint32_t a_row = (uint32_t)(A.xld * 2);
 #pragma unroll
-        for (int rb = 0; rb < 3; ++rb) {
-            const int ml = idx + 16 * rb;
-            const uint32_t xrow = (uint32_t)(m0 + min(ml, m_rows - 1)) * (uint32_t)(A.xld * 2);
+            for (int rb = 0; rb < 3; ++rb) {
+#pragma unroll 1
+                for (int c = 0; c < kPassCopies; ++c) {             // a loop: unrolled, its 39 offsets would all be live at once
+                    const int q = c * 64 + lane;
+                    const int row = q / kRowPieces, piece = q - row * kRowPieces;
+                    const int rl = 16 * rb + row;
+                    const bool valid = row < 16 && piece < KTW * 8 && rl < m_rows && (piece >> 3) < kcnt;
+                    copy16_to_lds(xrs, my_buf + c * 1024, valid ? (uint32_t)(m0 + rl) * a_row + (uint32_t)(kt0 * 128 + piece * 16) : kDeadOffset, 0u);
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-            for (int T = 0; T < KG; ++T) {
-                const int t = 2 * T + (g >> 1);
-                const bool on = ml < m_rows && t < kcnt;
-                const uint32_t xt = on ? xrow + (uint32_t)(kt0 + t) * 128u : kDeadOffset;
-                ah0[T][rb] = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + 2u * hh * 16u), 0, 0);
-                al0[T][rb] = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (3u + 2u * hh) * 16u), 0, 0);
-                ah1[T][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 16u + 8u * hh), 0, 0);
-                al1[T][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 64u + 8u * hh), 0, 0);
-                const uint32_t two = __builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(xt + 96u + 4u * hh), 0, 0) & 0xffffu;
-                if (T == 0) asa[0][rb] = two;
-                else if (T == 1) asa[0][rb] |= two << 16;
-                else asa[1][rb] = two;
+                for (int T = 0; T < KG; ++T) {
+                    const uint8_t* const kp = my_buf + idx * (kRowPieces * 16) + (2 * T + (g >> 1)) * 128;
+                    ah0[T][rb] = *reinterpret_cast<const uint4_t*>(kp + 2u * hh * 16u);
+                    al0[T][rb] = *reinterpret_cast<const uint4_t*>(kp + (3u + 2u * hh) * 16u);
+                    ah1[T][rb] = *reinterpret_cast<const uint2_t*>(kp + 16u + 8u * hh);
+                    al1[T][rb] = *reinterpret_cast<const uint2_t*>(kp + 64u + 8u * hh);
+                    const uint32_t two = *reinterpret_cast<const uint32_t*>(kp + 96u + 4u * hh) & 0xffffu;
+                    if (T == 0) asa[0][rb] = two;
+                    else if (T == 1) asa[0][rb] |= two << 16;
+                    else asa[1][rb] = two;
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the reads are done: the buffers may be written again
             }
         }
         const uint32_t koff = G::tile_offset(kt0);
