@@ -2328,23 +2328,65 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
         // (range-checked loads: rows past the tile and k-tiles past the wavefront's range read zeros - zero fields
         // under the smallest scale - without a select per register)
         const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(A.x16), 0, (int)A.x16_bytes, 0x00020000);
+        if (RB == 1 && m_rows > 16) {
+            // (units of a few rows load them directly, further down: for them the pass through LDS is only a second latency)
+            // Through the wavefront's (still empty) raw buffers: LDS-direct copies of whole row pieces (128 KTW contiguous
+            // bytes per row, 16 rows per pass) and 16-byte LDS reads from there; loaded straight from memory, a lane per
+            // row and K block, every 128-byte line was asked for in five separate pieces (see gemm_slim_mx48_kernel).
+            constexpr int kRowPieces = KTW * 8 + 1;                     // one piece of padding spreads the rows over the banks
+            constexpr int kPassCopies = (16 * kRowPieces + 63) / 64;
+            static_assert(kPassCopies * 1024 <= RING * BUF, "a pass of 16 rows fits the ring");
+            const uint32_t a_row = (uint32_t)(A.xld * 2);
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const int ml = col + 32 * rb;
-            const uint32_t xrow = (uint32_t)(m0 + min(ml, m_rows - 1)) * (uint32_t)(A.xld * 2);
+            for (int pass = 0; pass < 2; ++pass) {
+                // only the rows the unit has: an expert with two tokens copies two rows, and none in the second pass
+                const int pass_rows = __builtin_amdgcn_readfirstlane(min(16, m_rows - 16 * pass));
+                if (pass_rows <= 0) break;
+                const int pass_copies = (pass_rows * kRowPieces + 63) >> 6;
+#pragma unroll 1
+                for (int c = 0; c < pass_copies; ++c) {
+                    const int q = c * 64 + lane;
+                    const int row = q / kRowPieces, piece = q - row * kRowPieces;
+                    const int rl = 16 * pass + row;
+                    const bool valid = row < pass_rows && piece < KTW * 8 && (piece >> 3) < kcnt;
+                    copy16_to_lds(xrs, my_buf + c * 1024, valid ? (uint32_t)(m0 + rl) * a_row + (uint32_t)(kt0 * 128 + piece * 16) : kDeadOffset, 0u);
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                // rows 0 .. 15 in the first pass (the upper lanes read along and are overwritten), 16 .. 31 in the second
+                if (pass == 0 || col >= 16) {
 #pragma unroll
-            for (int t = 0; t < KTW; ++t) {
-                const bool on = ml < m_rows && t < kcnt;
-                const uint32_t xt = on ? xrow + (uint32_t)(kt0 + t) * 128u : kDeadOffset;
-                const uint4_t vh0 = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (uint32_t)(2 * h) * 16u), 0, 0);
-                const uint4_t vl0 = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (uint32_t)(3 + 2 * h) * 16u), 0, 0);
-                ah0[t][rb] = vh0;
-                al0[t][rb] = vl0;
-                ah1[t][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 16u + 8u * (uint32_t)h), 0, 0);
-                al1[t][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 64u + 8u * (uint32_t)h), 0, 0);
-                const uint32_t two = __builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(xt + 96u + 4u * (uint32_t)h), 0, 0) & 0xffffu;
-                if (t & 1) asa[t >> 1][rb] |= two << 16;
-                else asa[t >> 1][rb] = two;
+                    for (int t = 0; t < KTW; ++t) {
+                        const uint8_t* const kp = my_buf + (col & 15) * (kRowPieces * 16) + t * 128;
+                        ah0[t][0] = *reinterpret_cast<const uint4_t*>(kp + (uint32_t)(2 * h) * 16u);
+                        al0[t][0] = *reinterpret_cast<const uint4_t*>(kp + (uint32_t)(3 + 2 * h) * 16u);
+                        ah1[t][0] = *reinterpret_cast<const uint2_t*>(kp + 16u + 8u * (uint32_t)h);
+                        al1[t][0] = *reinterpret_cast<const uint2_t*>(kp + 64u + 8u * (uint32_t)h);
+                        const uint32_t two = *reinterpret_cast<const uint32_t*>(kp + 96u + 4u * (uint32_t)h) & 0xffffu;
+                        if (t & 1) asa[t >> 1][0] = (asa[t >> 1][0] & 0xffffu) | (two << 16);
+                        else asa[t >> 1][0] = two;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the reads are done: the buffers may be written again
+            }
+        } else {
+    #pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int ml = col + 32 * rb;
+                const uint32_t xrow = (uint32_t)(m0 + min(ml, m_rows - 1)) * (uint32_t)(A.xld * 2);
+    #pragma unroll
+                for (int t = 0; t < KTW; ++t) {
+                    const bool on = ml < m_rows && t < kcnt;
+                    const uint32_t xt = on ? xrow + (uint32_t)(kt0 + t) * 128u : kDeadOffset;
+                    const uint4_t vh0 = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (uint32_t)(2 * h) * 16u), 0, 0);
+                    const uint4_t vl0 = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(xt + (uint32_t)(3 + 2 * h) * 16u), 0, 0);
+                    ah0[t][rb] = vh0;
+                    al0[t][rb] = vl0;
+                    ah1[t][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 16u + 8u * (uint32_t)h), 0, 0);
+                    al1[t][rb] = __builtin_amdgcn_raw_buffer_load_b64(xrs, (int)(xt + 64u + 8u * (uint32_t)h), 0, 0);
+                    const uint32_t two = __builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(xt + 96u + 4u * (uint32_t)h), 0, 0) & 0xffffu;
+                    if (t & 1) asa[t >> 1][rb] |= two << 16;
+                    else asa[t >> 1][rb] = two;
+                }
             }
         }
         const uint32_t koff = G::tile_offset(kt0);
