@@ -249,14 +249,15 @@ def test_mxfp4_block_scaled_256_row_tiles(hip, oracle):
     check(y[rows], oracle.matmul_f64(MXFP4, wq, N, K, x[rows]), "mx 256-row tiles")
 
 
-@pytest.mark.parametrize("K", [256, 1024, 2048])
-def test_mxfp4_block_scaled_register_resident_k_ranges(hip, oracle, K):
-    """Small batch over a large weight with a short K: two and four k-tiles per wavefront of the register-resident
-    kernel (K = 256 leaves most wavefronts without a k-tile)."""
+@pytest.mark.parametrize("K,M", [(256, 24), (1024, 24), (2048, 24), (2848, 17), (1024, 32), (3008, 31), (2880, 16)])
+def test_mxfp4_block_scaled_register_resident_k_ranges(hip, oracle, K, M):
+    """Small batch over a large weight with a short K: two, four and six k-tiles per wavefront of the register-resident
+    kernel (K = 256 leaves most wavefronts without a k-tile; 2848 and 3008 end in half a k-tile).  Units of more than
+    16 rows fetch their activations through LDS in two passes of 16 rows (17: a single row in the second pass),
+    smaller ones load them directly."""
     import torch
     from tensorsharp_amd import QuantizedWeight
-    rng = np.random.default_rng(K)
-    M = 24
+    rng = np.random.default_rng(K + M)
     N = (64 << 20) // K + 40
     wq = inputs.random_blocks("mxfp4", N, K, rng)
     x = rng.standard_normal((M, K)).astype(np.float32)
