@@ -230,7 +230,9 @@ def test_128_row_tiles(hip, oracle, name, M, N, K):
                                    (700, 1500, 2880),        # ragged last tile in both directions, 45 k-tiles
                                    (257, 300, 64),           # a single k-tile
                                    (1030, 264, 4096 + 32),
-                                   (300, 264, 8192 + 64)])   # rows beyond 8192: the 1024-thread conversion
+                                   (300, 264, 8192 + 64),    # rows beyond 8192: the 1024-thread conversion
+                                   (384, 1500, 2880),        # few tiles: K chunks of 12 k-tiles, the last one of 9
+                                   (640, 1100, 2880 - 32)])  # the same with half a k-tile at the end
 def test_mxfp4_block_scaled_tiles(hip, oracle, M, N, K):
     rng = np.random.default_rng(M + 3 * N + K)
     wq = oracle.quantize(MXFP4, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
