@@ -1529,13 +1529,16 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
 
 // Number of K chunks for a plain launch: with few tiles and a long K, chunks of K fill the CUs that a whole-K launch
 // leaves idle.  Model: rounds of workgroups x k-tiles per chunk, plus writing and re-reading the chunk sums.
-inline int pick_k_chunks(int tiles, int nkt, int slots, int64_t out_elems, double us_per_ktile, int min_chunk = 32)
+inline int pick_k_chunks(int tiles, int nkt, int slots, int64_t out_elems, double us_per_ktile)
 {
     int best = 1;
     double best_t = (double)((tiles + slots - 1) / slots) * nkt * us_per_ktile;
     for (int sc = 2; sc <= 4; ++sc) {
         const int chunk = ((nkt + sc - 1) / sc + 3) / 4 * 4;
-        if (chunk < min_chunk) break;
+        // chunks down to 12 k-tiles (a floor of 32 was slower on every launch of few tiles that was measured: Q4_K
+        // 1024 x 4096 x 3072 62.7 -> 53.9 us, Q8_0 512 x 4096 x 2048 45.8 -> 35.8, Q6_K 1024 x 4096 x 3072 87.1 -> 65.6,
+        // MXFP4 640 x 2880 x 2880 42.1 -> 32.6)
+        if (chunk < 12) break;
         const double t = (double)((tiles * sc + slots - 1) / slots) * chunk * us_per_ktile + 2.0 * sc * out_elems * 4 / 4.5e6;
         if (t < 0.9 * best_t) {
             best = sc;
@@ -1921,9 +1924,7 @@ bool launch_mx(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
     a.k_chunks = 1;
     a.chunk_kt = (nkt + 3) / 4 * 4;
     a.partial = nullptr;
-    // chunks down to 12 k-tiles (the fp16 tile kernels stop at 32): measured 512 x 5760 x 2880 43.2 -> 39.3 us, 384 rows
-    // 41.7 -> 34.2, 640 x 2880 x 2880 42.1 -> 32.6, 1024 x 2880 x 2880 44.1 -> 40.0; shapes with enough tiles are unchanged
-    a.k_chunks = pick_k_chunks(a.m_tiles * a.n_tiles, nkt, device_info().num_cus, (int64_t)a.M * a.N, 1.7 * BM * BN / 65536.0, 12);
+    a.k_chunks = pick_k_chunks(a.m_tiles * a.n_tiles, nkt, device_info().num_cus, (int64_t)a.M * a.N, 1.7 * BM * BN / 65536.0);
     if (a.k_chunks > 1) {
         a.chunk_kt = ((nkt + a.k_chunks - 1) / a.k_chunks + 3) / 4 * 4;
         a.k_chunks = (nkt + a.chunk_kt - 1) / a.chunk_kt;

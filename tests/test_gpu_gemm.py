@@ -215,7 +215,9 @@ def test_q6_k_rows_two_bytes_off(hip, oracle, M):
 @pytest.mark.parametrize("name,M,N,K", [("mxfp4", 600, 300, 768), ("q4_k", 520, 1000, 1024), ("q8_0", 70, 500, 1088),
                                        ("mxfp4", 300, 17000, 512),
                                        # few tiles and a long K: K is cut into chunks whose sums a second kernel adds
-                                       ("q8_0", 200, 300, 8192), ("q4_k", 600, 260, 8192), ("mxfp4", 1100, 300, 6144 + 64)])
+                                       ("q8_0", 200, 300, 8192), ("q4_k", 600, 260, 8192), ("mxfp4", 1100, 300, 6144 + 64),
+                                       # chunks of 12 and 16 k-tiles
+                                       ("q4_k", 1024, 520, 2048), ("q8_0", 520, 600, 3072), ("q4_k", 700, 520, 3072)])
 def test_128_row_tiles(hip, oracle, name, M, N, K):
     # row counts past the register-resident kernel's range: 128-row tiles, ragged last tile
     rng = np.random.default_rng(M + N + K)
