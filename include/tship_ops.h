@@ -252,7 +252,7 @@ TSHIP_EXPORT int TSHip_MoEExpertsForwardF32(TSHipTensorView2D result, TSHipTenso
 
 /* replaces TSGgml_MoEExpertsSwiGLUForwardF32 (ggml_ops_fused.cpp:1766-1940; GgmlNative.cs:350-369;
  * GgmlBasicOps.cs:615-645): result = sum_e route_weights[e] * W_down[e] * ( silu(W_gate[e] x) * (W_up[e] x) ),
- * num_experts 1..16. */
+ * num_experts 1..32 as in the bridge (ggml_ops_fused.cpp:1795-1799; only the squared-ReLU form above stops at 16). */
 TSHIP_EXPORT int TSHip_MoEExpertsSwiGLUForwardF32(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
                                                   void** gate_data_ptrs, void** up_data_ptrs, void** down_data_ptrs,
                                                   int gate_ggml_type, int64_t gate_ne0, int64_t gate_ne1,

@@ -234,6 +234,17 @@ bool is_standard_view(const TSHipTensorView2D& d)
     return d.stride1 == 1 && (d.dim0 == 1 || d.stride0 >= d.dim1);
 }
 
+// The *Device entry points index their operands in place: an output whose rows overlap or an input with a
+// non-unit inner stride would silently give wrong numbers, so both are refused (the host forms pack such views).
+bool check_device_views(const TSHipTensorView2D& out, const TSHipTensorView2D& input)
+{
+    if (!is_standard_view(out) || input.stride1 != 1) {
+        set_last_error("Device addmm_quant needs stride1 == 1 views.");
+        return false;
+    }
+    return true;
+}
+
 size_t row_size(int type, int64_t ne)
 {
     const int64_t bs = block_elems(type);
@@ -1262,10 +1273,7 @@ int TSHip_AddmmQuantF32Device(TSHipTensorView2D result, TSHipTensorView2D m1, co
     return guarded(0, "addmm_quant", [&]() -> int {
         if (!ensure_backend()) return 0;
         if (!validate_addmm_quant(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes)) return 0;
-        if (!is_standard_view(result) || m1.stride1 != 1) {
-            set_last_error("Device addmm_quant needs stride1 == 1 views.");
-            return 0;
-        }
+        if (!check_device_views(result, m1)) return 0;
         if (!run_matmul_device(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, t_stream)) return 0;
         clear_last_error();
         return 1;
@@ -1278,10 +1286,7 @@ int TSHip_AddmmQuantF32DeviceNoAlloc(TSHipTensorView2D result, TSHipTensorView2D
     return guarded(0, "addmm_quant", [&]() -> int {
         if (!ensure_backend()) return 0;
         if (!validate_addmm_quant(result, m1, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes)) return 0;
-        if (!is_standard_view(result) || m1.stride1 != 1) {
-            set_last_error("Device addmm_quant needs stride1 == 1 views.");
-            return 0;
-        }
+        if (!check_device_views(result, m1)) return 0;
         // [converted activations + row scales][sums of K chunks]: both live in the static array
         const size_t need = plan_matmul(m2_ggml_type, m1.dim0, m2_ne0, m2_ne1, false, false).conv_bytes;
         if (need > kScratchBytes) {
@@ -1315,10 +1320,7 @@ int TSHip_AddmmQuantGroupF32Device(int count, const TSHipTensorView2D* results, 
             if (!validate_addmm_quant(results[i], m1s[i], m2_datas[i], m2_ggml_type, m2_ne0s[i], m2_ne1s[i],
                                       m2_raw_bytes[i]))
                 return 0;
-            if (!is_standard_view(results[i]) || m1s[i].stride1 != 1) {
-                set_last_error("Device addmm_quant needs stride1 == 1 views.");
-                return 0;
-            }
+            if (!check_device_views(results[i], m1s[i])) return 0;
             if (!check_device_operands(m1s[i], m2_datas[i], m2_ggml_type)) return 0;
             decode = decode && m1s[i].dim0 == 1 && m2_ne0s[i] <= gemv_max_k(m2_ggml_type);
         }
@@ -1756,6 +1758,7 @@ int TSHip_FusedRmsNormMatMulQuantF32Device(TSHipTensorView2D result, TSHipTensor
         if (!validate_fused_matmul(result, input, norm_weight, norm_weight_count, true, m2_data, m2_ggml_type, m2_ne0, m2_ne1,
                                    m2_raw_bytes, "fused rms_norm_matmul", "result"))
             return 0;
+        if (!check_device_views(result, input)) return 0;
         const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, m2_ne1, true, false);
         WsLease ws(t_stream, need);
         if (!ws.ok()) return 0;
@@ -1774,6 +1777,7 @@ int TSHip_FusedMatMulQuantAddF32Device(TSHipTensorView2D residual, TSHipTensorVi
         if (!validate_fused_matmul(residual, input, nullptr, 0, false, m2_data, m2_ggml_type, m2_ne0, m2_ne1, m2_raw_bytes,
                                    "fused matmul_add", "residual"))
             return 0;
+        if (!check_device_views(residual, input)) return 0;
         const size_t need = matmul_ws_bytes(m2_ggml_type, input.dim0, m2_ne0, m2_ne1, false, true);
         WsLease ws(t_stream, need);
         if (!ws.ok()) return 0;
@@ -1795,6 +1799,7 @@ int TSHip_FusedFFNSwiGLUQuantF32Device(TSHipTensorView2D residual, TSHipTensorVi
         if (!validate_ffn(residual, input, norm_weight, norm_weight_count, gate_up_data, gate_up_ggml_type, gate_up_ne0,
                           gate_up_ne1, gate_up_raw_bytes, down_data, down_ggml_type, down_ne0, down_ne1, down_raw_bytes, half_dim))
             return 0;
+        if (!check_device_views(residual, input)) return 0;
         WsLease ws(t_stream, ffn_ws_bytes(input.dim0, gate_up_ggml_type, down_ggml_type, input.dim1, half_dim));
         if (!ws.ok()) return 0;
         if (!run_ffn_swiglu_device(residual, input, norm_weight, eps, gate_up_data, gate_up_ggml_type, down_data, down_ggml_type,
@@ -1881,6 +1886,7 @@ int TSHip_FusedOutProjFFNQuantF32Device(TSHipTensorView2D residual, TSHipTensorV
         const WeightDesc od{out_proj_data, out_proj_type, out_ne0, out_ne1, out_raw_bytes};
         const WeightDesc gd{gu_data, gu_type, gu_ne0, gu_ne1, gu_raw_bytes}, dd{dn_data, dn_type, dn_ne0, dn_ne1, dn_raw_bytes};
         if (!validate_outproj_ffn(residual, input, od, ffn_norm_weight, ffn_norm_count, gd, dd, half_dim)) return 0;
+        if (!check_device_views(residual, input)) return 0;
         const size_t need = outproj_ffn_ws_bytes(input.dim0, od, gd, dd, residual.dim1, half_dim);
         WsLease ws(t_stream, need);
         if (!ws.ok()) return 0;
@@ -1927,6 +1933,10 @@ int TSHip_FusedOutProjNormRouterQuantF32Device(TSHipTensorView2D residual, TSHip
         const WeightDesc od{out_proj_data, out_proj_type, out_ne0, out_ne1, out_raw_bytes};
         const WeightDesc rd{router_data, router_type, router_ne0, router_ne1, router_raw_bytes};
         if (!validate_outproj_router(residual, input, od, norm_weight, norm_count, normed_out, rd, router_out)) return 0;
+        if (!check_device_views(residual, input) || !is_standard_view(router_out)) {
+            set_last_error("Device addmm_quant needs stride1 == 1 views.");
+            return 0;
+        }
         const size_t need = outproj_router_ws_bytes(input.dim0, od, rd);
         WsLease ws(t_stream, need);
         if (!ws.ok()) return 0;
@@ -1969,6 +1979,7 @@ int expert_set_device(TSHipTensorView2D out, bool add_to_out, TSHipTensorView2D 
 {
     if (!ensure_backend()) return 0;
     if (!validate_expert_set(out, input, a, out_name)) return 0;
+    if (!check_device_views(out, input)) return 0;
     if (!run_expert_set(out, add_to_out, input, a, t_stream, [](void* p, size_t) -> const void* { return p; })) return 0;
     clear_last_error();
     return 1;
@@ -2059,7 +2070,7 @@ int TSHip_MoEExpertsSwiGLUForwardF32(TSHipTensorView2D result, TSHipTensorView2D
 {
     return guarded(0, "MoE SwiGLU experts", [&]() -> int {
         return expert_set_host(result, false, input,
-                               swiglu_args("MoE SwiGLU", 16, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
+                               swiglu_args("MoE SwiGLU", 32, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
                                            gate_ne0, gate_ne1, gate_raw_bytes_each, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
                                            down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights),
                                "result");
@@ -2075,7 +2086,7 @@ int TSHip_MoEExpertsSwiGLUForwardF32Device(TSHipTensorView2D result, TSHipTensor
 {
     return guarded(0, "MoE SwiGLU experts", [&]() -> int {
         return expert_set_device(result, false, input,
-                                 swiglu_args("MoE SwiGLU", 16, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
+                                 swiglu_args("MoE SwiGLU", 32, num_experts, gate_data_ptrs, up_data_ptrs, down_data_ptrs, gate_ggml_type,
                                              gate_ne0, gate_ne1, gate_raw_bytes_each, up_ggml_type, up_ne0, up_ne1, up_raw_bytes_each,
                                              down_ggml_type, down_ne0, down_ne1, down_raw_bytes_each, route_weights),
                                  "result");
@@ -2189,12 +2200,25 @@ bool validate_mul_mat_id(const TSHipTensorView3D& result, const TSHipTensorView3
     return true;
 }
 
+// (token, slot) pairs go out in launches of at most 65535, the limit of the launch's second grid dimension.
 bool run_mul_mat_id(const TSHipTensorView3D& result, const TSHipTensorView3D& experts, const TSHipTensorView3D& input, const int32_t* ids_dev,
                     int ids_cols, hipStream_t stream)
 {
-    return launch_mul_mat_id_f32(static_cast<const float*>(experts.data), experts.stride0, experts.stride1, experts.dim0, experts.dim1,
-                                 experts.dim2, static_cast<const float*>(input.data), input.stride0, input.stride1, input.dim1, ids_dev,
-                                 input.dim0, ids_cols, static_cast<float*>(result.data), result.stride0, result.stride1, stream);
+    if (ids_cols > 65535) {
+        set_last_error("mulmatid: more than 65535 id columns.");
+        return false;
+    }
+    const int T = input.dim0, t_step = std::max(1, 65535 / ids_cols);
+    for (int t0 = 0; t0 < T; t0 += t_step) {
+        const int tn = std::min(t_step, T - t0);
+        const float* x = static_cast<const float*>(input.data) + (size_t)t0 * input.stride0;
+        float* y = static_cast<float*>(result.data) + (size_t)t0 * result.stride0;
+        if (!launch_mul_mat_id_f32(static_cast<const float*>(experts.data), experts.stride0, experts.stride1, experts.dim0, experts.dim1,
+                                   experts.dim2, x, input.stride0, input.stride1, input.dim1, ids_dev + (size_t)t0 * ids_cols, tn, ids_cols, y,
+                                   result.stride0, result.stride1, stream))
+            return false;
+    }
+    return true;
 }
 
 }  // namespace
@@ -2267,19 +2291,7 @@ int TSHip_MulMatIdF32(TSHipTensorView3D result, TSHipTensorView3D expert_weights
         const TSHipTensorView3D xd{dev + id_bytes, T, slots, K, slots * K, K, 1, (int64_t)((size_t)T * slots * K * sizeof(float))};
         const TSHipTensorView3D wd{w_dev, E, rows, K, rows * K, K, 1, (int64_t)((size_t)E * rows * K * sizeof(float))};
         const TSHipTensorView3D yd{y_dev, T, ids_cols, rows, ids_cols * rows, rows, 1, (int64_t)((size_t)T * ids_cols * rows * sizeof(float))};
-        // (token, slot) pairs in launches of at most 65535
-        const int t_step = std::max(1, 65535 / ids_cols);
-        if (ids_cols > 65535) {
-            set_last_error("mulmatid: more than 65535 id columns.");
-            return 0;
-        }
-        for (int t0 = 0; t0 < T; t0 += t_step) {
-            const int tn = std::min(t_step, T - t0);
-            TSHipTensorView3D xs_v = xd, ys_v = yd;
-            xs_v.data = static_cast<float*>(xd.data) + (size_t)t0 * xd.stride0, xs_v.dim0 = tn;
-            ys_v.data = static_cast<float*>(yd.data) + (size_t)t0 * yd.stride0, ys_v.dim0 = tn;
-            if (!run_mul_mat_id(ys_v, wd, xs_v, reinterpret_cast<const int32_t*>(dev) + (size_t)t0 * ids_cols, ids_cols, stream)) return 0;
-        }
+        if (!run_mul_mat_id(yd, wd, xd, reinterpret_cast<const int32_t*>(dev), ids_cols, stream)) return 0;
         if (!hip_ok(hipMemcpyAsync(pin, y_dev, (size_t)T * ids_cols * rows * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpy(result)")) return 0;
         if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
         const float* ys = reinterpret_cast<const float*>(pin);

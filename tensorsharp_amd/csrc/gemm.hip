@@ -75,6 +75,30 @@ __device__ __forceinline__ uint32_t pack2(float a, float b)
 }
 __device__ __forceinline__ uint32_t splat(float a) { return pack2(a, a); }
 
+// Range of the fp16 weight operands.  A dequantised weight enters the matrix cores as an fp16 number, so a block scale
+// near the ends of its own range would overflow fp16 or lose bits as an fp16 subnormal, where the reference
+// (ManagedQuantizedOps.cs:411-598) is exact in fp32 for every scale.  Weights of trained models are far below one, so
+// the operands carry the weight times 2^kWShift (the activations' row scale carries 2^-kWShift, see convert_x_kernel):
+// the smallest fp16 scale (2^-24) then gives a normal fp16 operand, and only scales ABOVE a per-format limit
+// (weights of magnitude about 32 and more; MXFP4: block exponents outside 94 .. 130) cannot be represented.  The
+// unpackers keep a high-water mark of the scales they met in `bad` (out_of_range() reads it), and the kernels then
+// store NaN in the columns such a block belongs to instead of a wrong number.
+constexpr int kWShift = 10;
+constexpr float kWUp = 1024.f;                   // 2^kWShift
+constexpr uint32_t kWUp2 = 0x64006400u;          // the same as two fp16
+constexpr uint32_t kNaNBits = 0x7fc00000u;
+typedef uint16_t ushort2_t __attribute__((ext_vector_type(2)));
+// high-water mark of the magnitude bits of two fp16 numbers (the order of the bits is the order of the magnitudes)
+__device__ __forceinline__ void mark2(uint32_t& mark, uint32_t two_halfs)
+{
+    mark = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ushort2_t, mark),
+                                                                  __builtin_bit_cast(ushort2_t, two_halfs & 0x7fff7fffu)));
+}
+__device__ __forceinline__ bool over2(uint32_t mark, uint32_t limit_lo, uint32_t limit_hi)
+{
+    return (mark & 0xffffu) > limit_lo || (mark >> 16) > limit_hi;
+}
+
 // Position inside a k-tile at which activation k (0..63) is stored, per weight format.  MFMA k-step ks
 // (0..3) takes positions [16 ks, 16 ks + 16): the first eight from the lanes with k-half h = 0, the
 // next eight from h = 1, and element e of those eight pairs with element e of the lane's B operand,
@@ -207,7 +231,8 @@ __global__ void __launch_bounds__(THREADS) convert_x_kernel(const ConvertSrc S, 
     if (e < 14) e = 14;
     const int se = e - 13;
     const float inv = __uint_as_float((uint32_t)(254 - se) << 23);
-    if (tid == 0) scales[m] = __uint_as_float((uint32_t)se << 23);
+    // the weight operands carry 2^kWShift (see kWShift), the row scale takes it back
+    if (tid == 0) scales[m] = __uint_as_float((uint32_t)se << 23) * (1.0f / kWUp);
     _Float16* dst = out + (int64_t)m * ldo;
     auto put = [&](int k, float v) { dst[(k & ~(kBK - 1)) | k_slot<TYPE>(k & (kBK - 1))] = (_Float16)(v * inv); };
     // Four consecutive activations land in one aligned 8-byte piece of the k-tile: in the K-quant order as
@@ -445,8 +470,11 @@ struct GQ4K {
         r[4] = q.x; r[5] = q.y; r[6] = q.z; r[7] = q.w;
     }
     // o[0..7]: low nibbles (sub-block 2j, elements 16h..16h+15), o[8..15]: high nibbles (sub-block 2j+1)
+    static constexpr uint32_t kLimit = 0x2c00u;      // |d|, |dmin| <= 2^-4: 15 * 63 * d * 2^kWShift stays finite in fp16
+    static __device__ __forceinline__ bool out_of_range(uint32_t mark) { return over2(mark, kLimit, kLimit); }
+    // (blocks past the end of K or N arrive as zeros, whose scale is in range: `live` is not needed)
     static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int /*h*/, uint32_t /*delta*/, bool /*live*/,
-                                                   uint32_t (&o)[16])
+                                                   uint32_t (&o)[16], uint32_t& bad)
     {
         const int sh = (j & 1) * 16;
         const uint32_t a = r[1] >> sh, b = r[2] >> sh, c = r[3] >> sh;
@@ -456,9 +484,10 @@ struct GQ4K {
         const uint32_t sc = (j & 2) ? sc_hi : sc_lo, mn = (j & 2) ? m_hi : m_lo;
         H2U dm;
         dm.u = r[0];
-        const float d = (float)dm.h.x, dmin = (float)dm.h.y;
-        const uint32_t s1 = splat(d * (float)(sc & 0xffu)), o1 = splat(-(dmin * (float)(mn & 0xffu)));
-        const uint32_t s2 = splat(d * (float)(sc >> 8) * 0.0625f), o2 = splat(-(dmin * (float)(mn >> 8)));
+        mark2(bad, r[0]);
+        const float d = (float)dm.h.x, dmin = (float)dm.h.y * kWUp;
+        const uint32_t s1 = splat(d * kWUp * (float)(sc & 0xffu)), o1 = splat(-(dmin * (float)(mn & 0xffu)));
+        const uint32_t s2 = splat(d * (float)(sc >> 8) * (0.0625f * kWUp)), o2 = splat(-(dmin * (float)(mn >> 8)));
         const uint32_t magic = 0x64006400u, neg1024 = 0xe400e400u;   // 1024.0, -1024.0
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -496,7 +525,17 @@ struct GMXFP4 {
         return c.u;
     }
     // quant byte i of the block -> (element i, element i + 16); o[4 w + s] holds byte 4 w + s
-    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int h, uint32_t delta, bool live, uint32_t (&o)[16])
+    // block exponents the fp16 operand holds exactly: 0.5 * 2^(e - 127 + kWShift) >= 2^-24 and 6 * 2^(e - 127 + kWShift) < 2^16
+    static constexpr uint32_t kMinE = 104 - kWShift, kMaxE = 140 - kWShift;
+    // E2M1 * 2^(e - 127) (the doubled table of ggml-common.h:1094-1096 times 2^(e - 128)) times 2^kWShift as a scale operand
+    static __device__ __forceinline__ float block_scale(uint32_t e, bool live, uint32_t& bad)
+    {
+        bad = max(bad, live ? e - kMinE : 0u);          // codes below the window wrap to large numbers
+        return live ? __uint_as_float((e + kWShift) << 23) : 0.f;
+    }
+    static __device__ __forceinline__ bool out_of_range(uint32_t mark) { return mark > kMaxE - kMinE; }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int h, uint32_t delta, bool live, uint32_t (&o)[16],
+                                                   uint32_t& bad)
     {
         const uint32_t sft = (delta + (uint32_t)(2 * j + h) * 17u) & 3u;
         const uint32_t e = (r[0] >> (8 * sft)) & 0xffu;
@@ -506,8 +545,8 @@ struct GMXFP4 {
         const uint32_t shb = (sft + 1) & 3;
         const uint32_t q[4] = {__builtin_amdgcn_alignbyte(b1, b0, shb), __builtin_amdgcn_alignbyte(b2, b1, shb),
                                __builtin_amdgcn_alignbyte(b3, b2, shb), __builtin_amdgcn_alignbyte(b4, b3, shb)};
-        // doubled E2M1 * 2^(e-128) = E2M1 * 2^(e-127); a block past the end of K contributes zeros
-        const float scale = live ? __uint_as_float(e == 0 ? 0x00400000u : (e << 23)) : 0.f;
+        // a block past the end of K contributes zeros
+        const float scale = block_scale(e, live, bad);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             o[4 * w] = cvt<0>(q[w], scale);
@@ -534,11 +573,15 @@ struct GQ80 {
 #pragma unroll
         for (int i = 0; i < kRegs; ++i) r[i] = p[i];
     }
-    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int h, uint32_t delta, bool live, uint32_t (&o)[16])
+    static constexpr uint32_t kLimit = 0x37ffu;      // |d| < 0.5: 128 * d * 2^kWShift stays finite in fp16
+    static __device__ __forceinline__ bool out_of_range(uint32_t mark) { return over2(mark, kLimit, 0xffffu); }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int j, int h, uint32_t delta, bool live, uint32_t (&o)[16],
+                                                   uint32_t& bad)
     {
         const bool odd = ((delta + (uint32_t)(2 * j + h) * 34u) & 2u) != 0;
-        const uint32_t dbits = odd ? (r[0] >> 16) : (r[0] & 0xffffu);
-        const uint32_t d2 = live ? (dbits | (dbits << 16)) : 0u;      // fp16 d in both halves
+        const uint32_t dbits = live ? (odd ? (r[0] >> 16) : (r[0] & 0xffffu)) : 0u;
+        mark2(bad, dbits);
+        const uint32_t d2 = pk_mul(dbits | (dbits << 16), kWUp2);     // fp16 d * 2^kWShift in both halves
         const uint32_t bias = 0xe480e480u;                              // -1152.0 = -(1024 + 128)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -580,7 +623,10 @@ struct GQ6K {
         r[18] = *reinterpret_cast<const uint32_t*>(rp + ((blk + 192u + 8u * nh + 2u * (2 * (j & 1) + h)) & ~3u));
         r[19] = *reinterpret_cast<const uint32_t*>(rp + ((blk + 208u) & ~3u));
     }
-    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int h, uint32_t delta, bool live, uint32_t (&o)[16])
+    static constexpr uint32_t kLimit = 0x23ffu;      // |d| < 2^-6: 32 * 128 * d * 2^kWShift stays finite in fp16
+    static __device__ __forceinline__ bool out_of_range(uint32_t mark) { return over2(mark, kLimit, 0xffffu); }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int h, uint32_t delta, bool live, uint32_t (&o)[16],
+                                                   uint32_t& bad)
     {
         const uint32_t blk = delta + (uint32_t)(t >> 2) * 210u;
         const int j = t & 3, g4 = 2 * (j & 1) + h;
@@ -589,8 +635,9 @@ struct GQ6K {
         const uint32_t scw = r[18] >> ((ps & 2u) * 8u);
         const float sc0 = (float)(int)(int8_t)(scw & 0xffu), sc1 = (float)(int)(int8_t)((scw >> 8) & 0xffu);
         H2U dd;
-        dd.u = (r[19] >> ((blk & 2u) * 8u)) & 0xffffu;
-        const float d = live ? (float)dd.h.x : 0.f;
+        dd.u = live ? (r[19] >> ((blk & 2u) * 8u)) & 0xffffu : 0u;
+        mark2(bad, dd.u);
+        const float d = (float)dd.h.x * kWUp;
         const uint32_t s0 = splat(d * sc0), s1 = splat(d * sc1);
         const uint32_t bias = 0xe420e420u;                              // -(1024 + 32)
 #pragma unroll
@@ -631,8 +678,10 @@ struct GQ5K {
         r[4] = q.x; r[5] = q.y; r[6] = q.z; r[7] = q.w;
         r[8] = qh.x; r[9] = qh.y; r[10] = qh.z; r[11] = qh.w;
     }
+    static constexpr uint32_t kLimit = 0x2800u;      // |d|, |dmin| <= 2^-5: 31 * 63 * d * 2^kWShift stays finite in fp16
+    static __device__ __forceinline__ bool out_of_range(uint32_t mark) { return over2(mark, kLimit, kLimit); }
     static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int /*h*/, uint32_t /*delta*/, bool /*live*/,
-                                                   uint32_t (&o)[16])
+                                                   uint32_t (&o)[16], uint32_t& bad)
     {
         const int j = t & 3;
         const int sh = (j & 1) * 16;
@@ -643,7 +692,8 @@ struct GQ5K {
         const uint32_t sc = (j & 2) ? sc_hi : sc_lo, mn = (j & 2) ? m_hi : m_lo;
         H2U dm;
         dm.u = r[0];
-        const float d = (float)dm.h.x, dmin = (float)dm.h.y;
+        mark2(bad, r[0]);
+        const float d = (float)dm.h.x * kWUp, dmin = (float)dm.h.y * kWUp;
         const uint32_t s1 = splat(d * (float)(sc & 0xffu)), o1 = splat(-(dmin * (float)(mn & 0xffu)));
         const uint32_t s2 = splat(d * (float)(sc >> 8) * 0.0625f), o2 = splat(-(dmin * (float)(mn >> 8)));
         const uint32_t magic = 0x64006400u, neg1024 = 0xe400e400u;
@@ -685,18 +735,27 @@ struct GLegacy {
 #pragma unroll
         for (int i = 0; i < kRegs; ++i) r[i] = p[i];
     }
-    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int h, uint32_t delta, bool live, uint32_t (&o)[16])
+    // |d| <= 4 (Q4_0: 8 d), 2 (Q4_1: 15 d + m; Q5_0: 16 d), 1 (Q5_1: 31 d + m), < 0.5 (IQ4_NL: 127 d) and |m| <= 32: the
+    // value times 2^kWShift stays finite in fp16
+    static constexpr uint32_t kLimitD = TYPE == kTypeQ4_0 ? 0x4400u : TYPE == kTypeQ5_1 ? 0x3c00u : TYPE == kTypeIQ4_NL ? 0x37ffu : 0x4000u;
+    static constexpr uint32_t kLimitM = 0x5000u;
+    static __device__ __forceinline__ bool out_of_range(uint32_t mark) { return over2(mark, kLimitD, kMin ? kLimitM : 0xffffu); }
+    static __device__ __forceinline__ void dequant(const uint32_t (&r)[kRegs], int t, int h, uint32_t delta, bool live, uint32_t (&o)[16],
+                                                   uint32_t& bad)
     {
         const uint32_t sft = (delta + (uint32_t)(2 * t + h) * kBlock) & 3u;
         uint32_t b[kWords];                                  // the block from its first byte
 #pragma unroll
         for (int i = 0; i < kWords; ++i) b[i] = __builtin_amdgcn_alignbyte(r[i + 1], r[i], sft);
         const uint32_t dbits = live ? b[0] & 0xffffu : 0u;
-        const uint32_t d2 = dbits | (dbits << 16);
+        const uint32_t d2 = pk_mul(dbits | (dbits << 16), kWUp2);
         uint32_t m2 = 0u;
         if (kMin) {
             const uint32_t mbits = live ? b[0] >> 16 : 0u;
-            m2 = mbits | (mbits << 16);
+            mark2(bad, dbits | (mbits << 16));
+            m2 = pk_mul(mbits | (mbits << 16), kWUp2);
+        } else {
+            mark2(bad, dbits);
         }
         uint32_t qh = 0u;
         if constexpr (kFive) qh = (kHdr & 3) ? __builtin_amdgcn_alignbyte(b[kHdr / 4], b[kHdr / 4 - 1], 2) : b[kHdr / 4 - 1];
@@ -806,6 +865,21 @@ __device__ __forceinline__ void store_wave_tile(const float* tile_scales, const 
                 if (ml < m_rows) cdst[(int64_t)(m0 + ml) * ldc + my_n] = kUnitScale ? acc[m][n][r2] : acc[m][n][r2] * sc[r2];
             }
         }
+    }
+}
+
+// A column whose weights held a scale outside the fp16 operand range (kWShift) is stored as NaN.
+template <int TM>
+__device__ __forceinline__ void poison_column(float16_t (&acc)[TM], bool flagged)
+{
+    // the two lanes of a column (k-halves) saw different blocks and hold different rows of it
+    if (__builtin_amdgcn_ballot_w64(flagged) == 0) return;
+    const int bad = (flagged ? 1 : 0) | __shfl_xor(flagged ? 1 : 0, 32);
+    if (bad) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][r] = __uint_as_float(kNaNBits);
     }
 }
 
@@ -1002,10 +1076,11 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
     for (int i = threadIdx.x; i < BM; i += NW * 64) tile_scales[i] = A.xscale[m0 + min(i, m_rows - 1)];
     __syncthreads();
     uint32_t oc[16], on[16];
+    uint32_t bad = 0u;                               // a scale of this lane's column does not fit the fp16 operands
     {
         uint32_t r[G::kRegs];
         G::fetch(rbuf + rb * RT + my_raw, 0, h, G::sup_delta(my_delta, s), r);
-        G::dequant(r, 0, h, G::sup_delta(my_delta, s), (kt_begin * 2 + h) * 32 < A.K, oc);
+        G::dequant(r, 0, h, G::sup_delta(my_delta, s), (kt_begin * 2 + h) * 32 < A.K && my_n < A.N, oc, bad);
     }
     for (int kt = kt_begin; kt < nkt; ++kt) {
         if (j == 0) issue_w(s + RL);
@@ -1035,7 +1110,8 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
                     __builtin_amdgcn_sched_barrier(0x6);
                 }
                 // unpack the next k-tile's operands in the shadow of the matrix pipe
-                if (ks == 0) G::dequant(r, jn, h, dn, ((kt + 1) * 2 + h) * 32 < A.K, on);
+                // (past the unit's last k-tile the raw bytes are stale: nothing of them is used)
+                if (ks == 0) G::dequant(r, jn, h, dn, kt + 1 < nkt && ((kt + 1) * 2 + h) * 32 < A.K && my_n < A.N, on, bad);
             }
         }
         // Copies that may stay in flight: the activations requested in the last D - 1 iterations and a
@@ -1052,6 +1128,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         xst = xst + 1 == XST ? 0 : xst + 1;
     }
 
+    poison_column<TM>(acc, G::out_of_range(bad));
     if (A.partial) {
         // chunk sums: [kc][activation row][column], already scaled; a second kernel adds the chunks
         GemmArgs P = A;
@@ -1101,6 +1178,7 @@ struct PQ4K {
     static constexpr int kFirstHalf = 11;             // steps after which quarters 0 and 2 are complete
     struct State {
         uint32_t a, b, c, sc, mn, s1, o1, s2, o2, q8;
+        float dmin;                                   // times 2^kWShift
     };
     // constants kept in registers so that mask-and-merge is one instruction (v_and_or_b32 takes one literal at most)
     struct Consts {
@@ -1114,13 +1192,14 @@ struct PQ4K {
     static __device__ __forceinline__ int ready_after(int quarter) { return quarter == 0 ? 10 : quarter == 2 ? 10 : 16; }
     template <int I>
     static __device__ __forceinline__ void micro(State& st, const uint32_t (&r)[G::kRegs], int j, int /*h*/, uint32_t /*delta*/, bool /*live*/,
-                                                 const Consts& K, uint32_t (&o)[16])
+                                                 const Consts& K, uint32_t (&o)[16], uint32_t& bad)
     {
         if constexpr (I == 0) {
             const int sh = (j & 1) * 16;
             st.a = r[1] >> sh;
             st.b = r[2] >> sh;
             st.c = r[3] >> sh;
+            mark2(bad, r[0]);
         } else if constexpr (I == 1) {
             const uint32_t sc_lo = st.a & 0x3f3fu, sc_hi = (st.c & 0x0f0fu) | ((st.a >> 2) & 0x3030u);
             st.sc = (j & 2) ? sc_hi : sc_lo;
@@ -1130,15 +1209,16 @@ struct PQ4K {
         } else if constexpr (I == 3) {
             H2U dm;
             dm.u = r[0];
-            const float d = (float)dm.h.x, dmin = (float)dm.h.y;
+            const float d = (float)dm.h.x * kWUp, dmin = (float)dm.h.y * kWUp;
             st.s1 = splat(d * (float)(st.sc & 0xffu));
             st.o1 = splat(-(dmin * (float)(st.mn & 0xffu)));
+            st.dmin = dmin;
         } else if constexpr (I == 4) {
             H2U dm;
             dm.u = r[0];
-            const float d = (float)dm.h.x, dmin = (float)dm.h.y;
-            st.s2 = splat(d * (float)(st.sc >> 8) * 0.0625f);
-            st.o2 = splat(-(dmin * (float)(st.mn >> 8)));
+            const float d = (float)dm.h.x;
+            st.s2 = splat(d * (float)(st.sc >> 8) * (0.0625f * kWUp));
+            st.o2 = splat(-(st.dmin * (float)(st.mn >> 8)));
         } else {
             // raw dword i in three steps: both low nibble pairs; high pair of bytes 0, 2; high pair of bytes 1, 3
             constexpr int i = (I - 5) / 3, part = (I - 5) % 3;
@@ -1185,7 +1265,7 @@ struct PMXFP4 {
     struct Consts {};
     template <int I>
     static __device__ __forceinline__ void micro(State& st, const uint32_t (&r)[G::kRegs], int /*j*/, int h, uint32_t delta, bool live,
-                                                 const Consts&, uint32_t (&o)[16])
+                                                 const Consts&, uint32_t (&o)[16], uint32_t& bad)
     {
         if constexpr (I == 0) {
             // the re-alignment of GMXFP4::dequant for block h of the window
@@ -1199,7 +1279,7 @@ struct PMXFP4 {
             st.q[1] = __builtin_amdgcn_alignbyte(b2, b1, shb);
             st.q[2] = __builtin_amdgcn_alignbyte(b3, b2, shb);
             st.q[3] = __builtin_amdgcn_alignbyte(b4, b3, shb);
-            st.scale = live ? __uint_as_float(e == 0 ? 0x00400000u : (e << 23)) : 0.f;
+            st.scale = G::block_scale(e, live, bad);
         } else {
             constexpr int w = I == 1 ? 0 : I == 2 ? 2 : I == 3 ? 1 : 3;
             o[4 * w] = G::template cvt<0>(st.q[w], st.scale);
@@ -1233,6 +1313,7 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
     uint8_t* const bex = rraw + ST * kRawTile;            // 2 x kBTile
     uint8_t* const dump = bex + 2 * kBTile;               // 1 KiB
     float* const tile_scales = reinterpret_cast<float*>(dump + 1024);      // BM row scales for the epilogue
+    uint32_t* const col_bad = reinterpret_cast<uint32_t*>(tile_scales + BM);   // BN flags: a scale of the column left the operand range
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1344,11 +1425,18 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
     for (int i = 0; i < RI; ++i) issue_raw1(kt_begin + 1, i);
     if (tid < BM) tile_scales[tid] = A.xscale[m0 + min(tid, m_rows - 1)];
     __syncthreads();
+    uint32_t bad[DUTY];                                   // per 32-column block this lane unpacks
+    bool in_n[DUTY];
+#pragma unroll
+    for (int u = 0; u < DUTY; ++u) {
+        bad[u] = 0u;
+        in_n[u] = n0 + 32 * DUTY * wave + 32 * u + col < A.N;
+    }
 #pragma unroll
     for (int u = 0; u < DUTY; ++u) {
         uint32_t r0[G::kRegs], o0[16];
         P::fetch(rraw + (kt_begin & (ST - 1)) * kRawTile + my_raw + u * 32 * P::kRowBytes, h, P::delta(my_d0[u], kt_begin), r0);
-        G::dequant(r0, P::phase(kt_begin), h, P::delta(my_d0[u], kt_begin), (kt_begin * 2 + h) * 32 < A.K, o0);
+        G::dequant(r0, P::phase(kt_begin), h, P::delta(my_d0[u], kt_begin), (kt_begin * 2 + h) * 32 < A.K && in_n[u], o0, bad[u]);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const uint4_t v = {o0[4 * ks], o0[4 * ks + 1], o0[4 * ks + 2], o0[4 * ks + 3]};
@@ -1385,7 +1473,7 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
         uint32_t o[16];
         typename P::State st;
         const int ph = P::phase(kt + 1);
-        const bool live = ((kt + 1) * 2 + h) * 32 < A.K;
+        const bool live_k = kt + 1 < nkt && ((kt + 1) * 2 + h) * 32 < A.K;      // past the unit's end the raw bytes are zeros or stale
         const uint8_t* const xs = xbuf + (kt & (ST - 1)) * kXTile;
         const uint8_t* const bs = bex + (kt & 1) * kBTile + b_rd;
         uint8_t* const bnext = bex + ((kt + 1) & 1) * kBTile + b_wr;
@@ -1398,14 +1486,15 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
                 constexpr int first_ready = P::kFirstHalf, second_ready = P::kMicro;
                 uint8_t* const dst = bnext + u * 32 * 16;
                 const uint32_t dl = P::delta(my_d0[u], kt + 1);
+                const bool live = live_k && in_n[u];
                 if constexpr (w < first_ready) {
-                    P::template micro<w>(st, r[u], ph, h, dl, live, KC, o);
+                    P::template micro<w>(st, r[u], ph, h, dl, live, KC, o, bad[u]);
                 } else if constexpr (w == first_ready || w == first_ready + 1) {
                     constexpr int q = w == first_ready ? 0 : 2;
                     const uint4_t v = {o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]};
                     *reinterpret_cast<uint4_t*>(dst + q * (2 * BN * 16)) = v;
                 } else if constexpr (w < second_ready + 2) {
-                    P::template micro<w - 2>(st, r[u], ph, h, dl, live, KC, o);
+                    P::template micro<w - 2>(st, r[u], ph, h, dl, live, KC, o, bad[u]);
                 } else {
                     constexpr int q = w == second_ready + 2 ? 1 : 3;
                     const uint4_t v = {o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]};
@@ -1482,6 +1571,24 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
                 else if (i < XI + RI) issue_raw1(kt + ST + 1, i - XI);
                 __builtin_amdgcn_sched_barrier(0);
             }
+        }
+    }
+
+    // columns with a scale outside the operand range: the unpacking lanes publish their flags, the owners store NaN
+#pragma unroll
+    for (int u = 0; u < DUTY; ++u) {
+        const int mine = G::out_of_range(bad[u]) ? 1 : 0;
+        const int both = mine | __shfl_xor(mine, 32);                             // the column's two k-halves
+        if (h == 0) col_bad[32 * DUTY * wave + 32 * u + col] = (uint32_t)both;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int n = 0; n < NB; ++n) {
+        if (col_bad[32 * NB * wn + 32 * n + col]) {
+#pragma unroll
+            for (int m = 0; m < TMW; ++m)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[m][n][r] = __uint_as_float(kNaNBits);
         }
     }
 
@@ -1597,7 +1704,7 @@ bool launch_xw(GemmArgs a, int m_tiles, hipStream_t stream, const ChunkScratch& 
 {
     constexpr int BN = 256;
     auto kern = gemm_xw_kernel<P, BM, WN>;
-    constexpr size_t kLds = (size_t)2 * BM * kXRow + (size_t)2 * BN * P::kRowBytes + (size_t)2 * 4 * 2 * BN * 16 + 1024 + BM * 4;
+    constexpr size_t kLds = (size_t)2 * BM * kXRow + (size_t)2 * BN * P::kRowBytes + (size_t)2 * 4 * 2 * BN * 16 + 1024 + BM * 4 + BN * 4;
     static_assert(kLds <= 160 * 1024, "LDS");
     const size_t lds = kLds;
     if (!cs.need_out && !raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
@@ -2111,6 +2218,8 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
             float16_t acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            uint32_t bad = 0u;                          // a scale of this lane's column does not fit the fp16 operands
+            const bool in_n = (nt0 + i) * 32 + col < A.N;
             const uint8_t* raw = my_buf + b * BUF + col * (CH * 16);
             // a wavefront with a full K range runs the k-tiles as one branch-free block, so the unpacking of one
             // k-tile is scheduled into the matrix instructions of the previous one
@@ -2121,7 +2230,7 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
                     if (kFull || t < kcnt) {
                         uint32_t r[G::kRegs], o[16];
                         G::fetch(raw, t, h, my_delta, r);
-                        G::dequant(r, t, h, my_delta, ((kt0 + t) * 2 + h) * 32 < A.K, o);
+                        G::dequant(r, t, h, my_delta, ((kt0 + t) * 2 + h) * 32 < A.K && in_n, o, bad);
 #pragma unroll
                         for (int ks = 0; ks < 4; ++ks) {
                             const uint4_t bb = {o[4 * ks], o[4 * ks + 1], o[4 * ks + 2], o[4 * ks + 3]};
@@ -2132,6 +2241,11 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
             };
             if (kcnt == KTW) k_tiles(std::true_type{});
             else k_tiles(std::false_type{});
+            {
+                float16_t one[1] = {acc};
+                poison_column<1>(one, G::out_of_range(bad));
+                acc = one[0];
+            }
             // partial sums of this wavefront's K range -> the buffer it has just consumed
             float* part = reinterpret_cast<float*>(my_buf + b * BUF);
 #pragma unroll

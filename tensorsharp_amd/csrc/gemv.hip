@@ -442,9 +442,11 @@ struct FmtMXFP4 {
         s = dot2(fp4_pair<2>(q2), x2.z, s); t = dot2(fp4_pair<3>(q2), x2.w, t);
         s = dot2(fp4_pair<0>(q3), x3.x, s); t = dot2(fp4_pair<1>(q3), x3.y, t);
         s = dot2(fp4_pair<2>(q3), x3.z, s); t = dot2(fp4_pair<3>(q3), x3.w, t);
-        // table value = 2 * E2M1, block scale = 2^(e-128)  ->  E2M1 * 2^(e-127)
-        const float bscale = __uint_as_float(e == 0 ? 0x00400000u : (e << 23));
-        return (s + t) * bscale * xscale;
+        // table value = 2 * E2M1, block scale = 2^(e-128) with the subnormal patterns of ggml_e8m0_to_fp32_half
+        // (ggml-impl.h:471-489) for e < 2: exact for every code, 255 included
+        const float bscale = __uint_as_float(e < 2 ? (0x00200000u << e) : ((e - 1u) << 23));
+        // the activations' own scale first: the sums are of staged magnitude (up to 2^19), the block scale may be 2^127
+        return ((s + t) * xscale) * 2.0f * bscale;
     }
 };
 

@@ -158,7 +158,7 @@ def test_experts_relu_squared(hip, oracle, name, n, M, device):
 
 
 @pytest.mark.parametrize("name,down", [("q8_0", None), ("q4_k", None), ("mxfp4", None), ("q4_k", "q8_0")])
-@pytest.mark.parametrize("n,M", [(1, 1), (8, 1), (16, 1), (3, 5)])
+@pytest.mark.parametrize("n,M", [(1, 1), (8, 1), (16, 1), (17, 1), (32, 1), (3, 5), (17, 3), (32, 2)])
 @pytest.mark.parametrize("device", [False, True])
 def test_experts_swiglu_forward(hip, oracle, name, down, n, M, device):
     rng = np.random.default_rng(340 + n + M)
@@ -242,8 +242,9 @@ def test_expert_set_argument_errors(hip, oracle):
     g, u, d = qw(ex[0]["gate"], False), qw(ex[0]["up"], False), qw(ex[0]["down"], False)
     with pytest.raises(RuntimeError, match="num_experts must be 1..16"):
         hip.MoEExpertsForward(out, x, [u] * 17, [d] * 17, [0.1] * 17)
-    with pytest.raises(RuntimeError, match="num_experts must be 1..16"):
-        hip.MoEExpertsSwiGLUForward(out, x, [g] * 17, [u] * 17, [d] * 17, [0.1] * 17)
+    # the gated forward takes up to 32 experts like the bridge (ggml_ops_fused.cpp:1795-1799); only the squared-ReLU form stops at 16
+    with pytest.raises(RuntimeError, match="num_experts must be 1..32"):
+        hip.MoEExpertsSwiGLUForward(out, x, [g] * 33, [u] * 33, [d] * 33, [0.1] * 33)
     with pytest.raises(RuntimeError, match="num_experts must be 1..32"):
         hip.MoEExpertsSwiGLUResidual(out, x, [g] * 33, [u] * 33, [d] * 33, [0.1] * 33)
     with pytest.raises(RuntimeError, match="weight shapes do not match"):
@@ -283,3 +284,58 @@ def test_mul_mat_id_f32_experts(hip, oracle, slots, device):
             hip.MulMatId(got_f, w, x[:, :, :K - 8], ids)
     # fp32 accumulation of exact fp32 products
     assert np.all(np.abs(got - ref) <= 1e-5 * np.linalg.norm(ref, axis=2, keepdims=True))
+
+
+def test_mul_mat_id_device_more_than_65535_pairs(hip, oracle):
+    """The device form cuts (token, slot) pairs into launches like the host form: a prefill of 16 500 tokens x 4 slots."""
+    import torch
+    rng = np.random.default_rng(380)
+    E, rows, K, T, k = 5, 12, 24, 16_500, 4
+    assert T * k > 65535
+    w = (rng.standard_normal((E, rows, K)) * 0.1).astype(np.float32)
+    x = rng.standard_normal((T, 1, K)).astype(np.float32)
+    ids = rng.integers(0, E, (T, k)).astype(np.int32)
+    out = torch.full((T, k, rows), float("nan"), device="cuda")
+    hip.MulMatId(out, torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda(), torch.from_numpy(ids).cuda())
+    torch.cuda.synchronize()
+    ref = np.einsum("tsrk,tk->tsr", w.astype(np.float64)[ids], x[:, 0].astype(np.float64))
+    assert np.all(np.abs(out.cpu().numpy() - ref) <= 1e-5 * np.linalg.norm(ref, axis=2, keepdims=True))
+
+
+def test_device_forms_refuse_strided_views(hip, oracle):
+    """The device entry points index operands in place, so an input whose inner stride is not 1 and an output whose rows
+    overlap are refused with the message of the plain device matmul (the host forms pack such views instead)."""
+    import ctypes as C
+    import torch
+    from tensorsharp_amd import hip_native as N
+    rng = np.random.default_rng(390)
+    H, I, M = 64, 64, 3
+    ex = experts(oracle, "q8_0", 1, H, I, H, rng, gated=True)[0]
+    g, u, d = (qw(ex[n], True) for n in ("gate", "up", "down"))
+    x = torch.zeros((M, 2 * H), device="cuda")
+    out = torch.zeros((M, H), device="cuda")
+    nw = torch.ones(H, device="cuda")
+    strided_x = N.TensorView2D(x.data_ptr(), M, H, 2 * H, 2, x.numel() * 4)            # every second element
+    good_x = N.TensorView2D(x.data_ptr(), M, H, 2 * H, 1, x.numel() * 4)
+    good_out = N.TensorView2D(out.data_ptr(), M, H, H, 1, out.numel() * 4)
+    overlap_out = N.TensorView2D(out.data_ptr(), M, H, H // 2, 1, out.numel() * 4)     # rows overlap
+    lib = N.lib()
+    wa = lambda q: (C.c_void_p(q.ptr), q.ggml_type, q.ne0, q.ne1, q.raw_bytes)
+    ptrs = lambda q: (C.c_void_p * 1)(q.ptr)
+    rw = (C.c_float * 1)(1.0)
+    shape = lambda q: (q.ggml_type, q.ne0, q.ne1, q.raw_bytes)
+    nwp = C.c_void_p(nw.data_ptr())
+    calls = {
+        "AddmmQuant": lambda o, i: lib.TSHip_AddmmQuantF32Device(o, i, *wa(u)),
+        "FusedRmsNormMatMul": lambda o, i: lib.TSHip_FusedRmsNormMatMulQuantF32Device(o, i, nwp, H, 1e-6, *wa(u)),
+        "FusedMatMulAdd": lambda o, i: lib.TSHip_FusedMatMulQuantAddF32Device(o, i, *wa(u)),
+        "MoEExpertsForward": lambda o, i: lib.TSHip_MoEExpertsForwardF32Device(o, i, 1, ptrs(u), ptrs(d), *shape(u), *shape(d), rw),
+        "MoEExpertsSwiGLUForward": lambda o, i: lib.TSHip_MoEExpertsSwiGLUForwardF32Device(o, i, 1, ptrs(g), ptrs(u), ptrs(d), *shape(g),
+                                                                                     *shape(u), *shape(d), rw),
+    }
+    for name, call in calls.items():
+        for o, i in ((good_out, strided_x), (overlap_out, good_x)):
+            assert call(o, i) == 0, name
+            assert "stride1 == 1" in N.get_last_error(), (name, N.get_last_error())
+        assert call(good_out, good_x) == 1, (name, N.get_last_error())
+    torch.cuda.synchronize()
