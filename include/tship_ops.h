@@ -308,9 +308,22 @@ TSHIP_EXPORT int TSHip_MulMatIdF32(TSHipTensorView3D result, TSHipTensorView3D e
                                    TSHipContiguousTensor ids, int ids_rows, int ids_cols);
 
 /* device-pointer form: ids is a device array of ids_rows x ids_cols int32; rows of an out-of-range id are zero;
- * ids_rows * ids_cols <= 65535.  Asynchronous on the selected stream. */
+ * any number of (token, slot) pairs (cut into launches of 65535).  Asynchronous on the selected stream. */
 TSHIP_EXPORT int TSHip_MulMatIdF32Device(TSHipTensorView3D result, TSHipTensorView3D expert_weights, TSHipTensorView3D input,
                                          const int32_t* ids, int ids_rows, int ids_cols);
+
+/* replaces TSGgml_AddIdF32 (ggml_ops_matmul.cpp:1123-1290, :1451-1473; GgmlNative.cs:442-448, :1081-1084; managed
+ * GgmlBasicOps.AddID :1092-1108): ggml_add_id, the per-expert bias that goes with a mul_mat_id,
+ *   result[t][s][r] = src[t][s][r] + bias[ids[t][s]][r],  src / result [T x ids_cols x rows], bias [E x rows],
+ * ids [ids_rows x ids_cols] (I32, or F32 truncated) with ids_rows == T.  Host pointers, standard views.  An id outside
+ * [0, E) is an error (the bridge's ggml asserts). */
+TSHIP_EXPORT int TSHip_AddIdF32(TSHipTensorView3D result, TSHipTensorView3D src, TSHipTensorView2D bias, TSHipContiguousTensor ids,
+                                int ids_rows, int ids_cols);
+
+/* device-pointer form: ids is a device array of ids_rows x ids_cols int32 (a pair with an id outside [0, E) gets no
+ * bias); result may be src (in place).  Asynchronous on the selected stream. */
+TSHIP_EXPORT int TSHip_AddIdF32Device(TSHipTensorView3D result, TSHipTensorView3D src, TSHipTensorView2D bias, const int32_t* ids,
+                                      int ids_rows, int ids_cols);
 
 /* replaces TSGgml_GetRowsQuantF32 (ggml_ops_matmul.cpp:519-668, :1339-1368; GgmlNative.cs:324, :1003-1006; caller
  * ModelBase.cs:826-856 embedding lookup): result[i, 0..ne0) = dequantized row indices[i] of the [ne1 x ne0] source

@@ -244,6 +244,23 @@ namespace TensorSharp.HIP
             HipNative.MulMatId(r, w, x, Indices("MulMatId", ids), (int)ids.Sizes[0], (int)ids.Sizes[1]);
         }
 
+        /// <summary>result[t, s, :] = src[t, s, :] + bias[ids[t, s], :]: the per-expert bias of a MulMatId (GgmlBasicOps.AddID).</summary>
+        [RegisterOpStorageType("addid", typeof(HipStorage))]
+        public static Tensor AddID(Tensor result, Tensor src, Tensor bias, Tensor ids)
+        {
+            if (src.DimensionCount != 3)
+                throw new NotSupportedException("addid expects a 3D source tensor.");
+            if (bias.DimensionCount != 2 || ids.DimensionCount != 2)
+                throw new NotSupportedException("addid expects 2D bias and id tensors.");
+            if (src.Sizes[2] != bias.Sizes[1] || src.Sizes[0] != ids.Sizes[0] || src.Sizes[1] != ids.Sizes[1])
+                throw new InvalidOperationException("addid expects src shape [tokens, expert_used, rows], bias shape [experts, rows], and ids shape [tokens, expert_used].");
+            Tensor writeTarget = TensorResultBuilder.GetWriteTarget(result, src, false, src.Sizes);
+            if (!Standard3(writeTarget, out var r) | !Standard3(src, out var s) | !Standard(bias, out var b))
+                throw new NotSupportedException("HIP addid requires Float32 standard-layout source/result tensors and a standard-layout 2D bias matrix.");
+            HipNative.AddId(r, s, b, Indices("AddID", ids), (int)ids.Sizes[0], (int)ids.Sizes[1]);
+            return writeTarget;
+        }
+
         // ---- weighted expert sets -----------------------------------------------------------------------------------------
         public static void MoEExpertsForward(Tensor result, Tensor input, int numExperts, IntPtr[] upDataPtrs, IntPtr[] downDataPtrs,
             int upGgmlType, long upNe0, long upNe1, long upRawBytesEach,

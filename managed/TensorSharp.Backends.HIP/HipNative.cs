@@ -91,6 +91,10 @@ namespace TensorSharp.HIP
         private static extern int TSHip_MulMatIdF32(HipTensorView3D result, HipTensorView3D expertWeights, HipTensorView3D input,
             HipContiguousTensor ids, int idsRows, int idsCols);
 
+        [DllImport(Dll, CallingConvention = CC)]
+        private static extern int TSHip_AddIdF32(HipTensorView3D result, HipTensorView3D src, HipTensorView2D bias,
+            HipContiguousTensor ids, int idsRows, int idsCols);
+
         // ---- fused wrappers ------------------------------------------------------------------------------------
         [DllImport(Dll, CallingConvention = CC)]
         private static extern int TSHip_FusedRmsNormMatMulQuantF32(HipTensorView2D result, HipTensorView2D input, IntPtr normWeightData,
@@ -223,6 +227,9 @@ namespace TensorSharp.HIP
 
         internal static void MulMatId(HipTensorView3D result, HipTensorView3D experts, HipTensorView3D input, HipContiguousTensor ids, int rows, int cols)
             => Check(TSHip_MulMatIdF32(result, experts, input, ids, rows, cols), "mulmatid");
+
+        internal static void AddId(HipTensorView3D result, HipTensorView3D src, HipTensorView2D bias, HipContiguousTensor ids, int rows, int cols)
+            => Check(TSHip_AddIdF32(result, src, bias, ids, rows, cols), "addid");
 
         internal static void FusedRmsNormMatMulQuant(HipTensorView2D result, HipTensorView2D input, IntPtr norm, int normCount, float eps,
             IntPtr w, int type, long ne0, long ne1, long rawBytes)

@@ -328,6 +328,17 @@ class Oracle:
         return out
 
 
+def add_id(src, bias, ids):
+    """ggml_add_id (include/ggml.h:886-891; bridge call ggml_ops_matmul.cpp:1123-1290): out[t, s, :] = src[t, s, :] +
+    bias[ids[t, s], :] in fp32.  The definition itself, element by element."""
+    src = np.asarray(src, dtype=np.float32)
+    out = np.empty_like(src)
+    for t in range(src.shape[0]):
+        for s in range(src.shape[1]):
+            out[t, s] = src[t, s] + np.asarray(bias, dtype=np.float32)[int(ids[t, s])]
+    return out
+
+
 class Reference:
     """The reference's own ggml code, compiled from its sources by `make ref`.
     Exists only where the reference checkout was available at build time."""
@@ -405,6 +416,17 @@ class Reference:
                      rope_freq_scale=1.0, rope_mode=2):
         _layer_call(self.lib.ref_layer_decode, hidden, layer, k_cache, v_cache, heads, kv_heads, head_dim, position, eps,
                     rope_base, rope_freq_scale, rope_mode)
+
+    def add_id(self, src, bias, ids):
+        """ggml_add_id on the reference's CPU backend"""
+        src = np.ascontiguousarray(src, dtype=np.float32)
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        out = np.empty_like(src)
+        T, cols, rows = src.shape
+        self.lib.ref_add_id.restype = C.c_int
+        assert self.lib.ref_add_id(_ptr(src, _f32p), _ptr(bias, _f32p), _vp(ids), T, cols, rows, bias.shape[0], _ptr(out, _f32p)) == 0
+        return out
 
     def mul_mat(self, t, w, N, K, x, threads=4):
         x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, K)

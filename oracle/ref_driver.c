@@ -8,6 +8,7 @@
 #include "ggml-cpu.h"
 
 #include <stdint.h>
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 #include <math.h>
@@ -55,23 +56,34 @@ int ref_mul_mat(int type, const void* w, int64_t N, int64_t K, const float* x, i
     return st == GGML_STATUS_SUCCESS ? 0 : -3;
 }
 
-/* A small GGUF file written by the reference's own writer (gguf.cpp): fixed metadata of every value kind the
- * managed reader handles, plus the given 2-D tensors (raw block bytes, ne0 = row length).  Pins the GGUF reader. */
+/* Small GGUF files written by the reference's own writer (gguf.cpp): fixed metadata of every value kind the
+ * managed reader handles, plus the given tensors (raw block bytes, ne0 = row length; ne2 > 1 makes a 3-D tensor such as
+ * the stacked experts of a MoE layer; ne1 = 1 with ne2 = 1 stays 2-D as ggml writes it).  Pins the GGUF reader. */
 #include "gguf.h"
 
-int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** names, const int* types,
-                   const int64_t* ne0, const int64_t* ne1, const void** data)
+static int write_gguf(const char* path, int alignment, const char* arch, int expert_count, int expert_used, int n_tensors,
+                      const char** names, const int* types, const int64_t* ne0, const int64_t* ne1, const int64_t* ne2,
+                      const void** data)
 {
     size_t total = 1u << 20;
-    for (int i = 0; i < n_tensors; ++i) total += ggml_row_size((enum ggml_type)types[i], ne0[i]) * (size_t)ne1[i] + 4096;
+    for (int i = 0; i < n_tensors; ++i)
+        total += ggml_row_size((enum ggml_type)types[i], ne0[i]) * (size_t)ne1[i] * (size_t)(ne2 ? ne2[i] : 1) + 4096;
     struct ggml_init_params ip = { total, NULL, false };
     struct ggml_context* ctx = ggml_init(ip);
     if (!ctx) return -1;
     struct gguf_context* g = gguf_init_empty();
-    gguf_set_val_str(g, "general.architecture", "llama");
+    char key[128];
+    gguf_set_val_str(g, "general.architecture", arch);
     gguf_set_val_str(g, "general.name", "tiny \xe2\x9c\x93 model");          /* non-ASCII UTF-8 */
     if (alignment != 32) gguf_set_val_u32(g, "general.alignment", (uint32_t)alignment);
-    gguf_set_val_u32(g, "llama.block_count", 2);
+    snprintf(key, sizeof key, "%s.block_count", arch);
+    gguf_set_val_u32(g, key, 2);
+    if (expert_count > 0) {
+        snprintf(key, sizeof key, "%s.expert_count", arch);
+        gguf_set_val_u32(g, key, (uint32_t)expert_count);
+        snprintf(key, sizeof key, "%s.expert_used_count", arch);
+        gguf_set_val_u32(g, key, (uint32_t)expert_used);
+    }
     gguf_set_val_i32(g, "test.i32", -7);
     gguf_set_val_u8(g, "test.u8", 200);
     gguf_set_val_i8(g, "test.i8", -100);
@@ -79,7 +91,8 @@ int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** 
     gguf_set_val_i16(g, "test.i16", -30000);
     gguf_set_val_u64(g, "test.u64", 1ull << 40);
     gguf_set_val_i64(g, "test.i64", -(1ll << 41));
-    gguf_set_val_f32(g, "llama.attention.layer_norm_rms_epsilon", 1e-5f);
+    snprintf(key, sizeof key, "%s.attention.layer_norm_rms_epsilon", arch);
+    gguf_set_val_f32(g, key, 1e-5f);
     gguf_set_val_f64(g, "test.f64", 0.1);
     gguf_set_val_bool(g, "test.flag", true);
     const char* toks[4] = { "<s>", "</s>", "hello", "w\xc3\xb6rld" };
@@ -91,7 +104,8 @@ int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** 
     const uint32_t u32s[3] = { 1, 2, 4000000000u };
     gguf_set_arr_data(g, "test.u32s", GGUF_TYPE_UINT32, u32s, 3);
     for (int i = 0; i < n_tensors; ++i) {
-        struct ggml_tensor* t = ggml_new_tensor_2d(ctx, (enum ggml_type)types[i], ne0[i], ne1[i]);
+        struct ggml_tensor* t = (ne2 && ne2[i] > 1) ? ggml_new_tensor_3d(ctx, (enum ggml_type)types[i], ne0[i], ne1[i], ne2[i])
+                                                    : ggml_new_tensor_2d(ctx, (enum ggml_type)types[i], ne0[i], ne1[i]);
         ggml_set_name(t, names[i]);
         memcpy(t->data, data[i], ggml_nbytes(t));
         gguf_add_tensor(g, t);
@@ -102,6 +116,19 @@ int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** 
     return ok;
 }
 
+int ref_write_gguf(const char* path, int alignment, int n_tensors, const char** names, const int* types,
+                   const int64_t* ne0, const int64_t* ne1, const void** data)
+{
+    return write_gguf(path, alignment, "llama", 0, 0, n_tensors, names, types, ne0, ne1, NULL, data);
+}
+
+/* A MoE layer as llama.cpp's converter stores it: the experts of a projection stacked in one 3-D tensor [ne0, ne1, experts]. */
+int ref_write_gguf_moe(const char* path, const char* arch, int expert_count, int expert_used, int n_tensors, const char** names,
+                       const int* types, const int64_t* ne0, const int64_t* ne1, const int64_t* ne2, const void** data)
+{
+    return write_gguf(path, 32, arch, expert_count, expert_used, n_tensors, names, types, ne0, ne1, ne2, data);
+}
+
 /* ---- known answers for the whole-layer decode, computed by the reference's ggml CPU ops ---------------- */
 
 static int run_graph(struct ggml_context* ctx, struct ggml_tensor* out)
@@ -109,6 +136,25 @@ static int run_graph(struct ggml_context* ctx, struct ggml_tensor* out)
     struct ggml_cgraph* g = ggml_new_graph(ctx);
     ggml_build_forward_expand(g, out);
     return ggml_graph_compute_with_ctx(ctx, g, 1) == GGML_STATUS_SUCCESS ? 0 : -3;
+}
+
+/* ggml_add_id as the bridge builds it (ggml_ops_matmul.cpp:1218): src [rows, cols, T], bias [rows, E], ids [cols, T] */
+int ref_add_id(const float* src, const float* bias, const int32_t* ids, int T, int cols, int rows, int E, float* out)
+{
+    struct ggml_init_params ip = { 16u << 20, NULL, false };
+    struct ggml_context* ctx = ggml_init(ip);
+    if (!ctx) return -1;
+    struct ggml_tensor* a = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, rows, cols, T);
+    struct ggml_tensor* b = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, rows, E);
+    struct ggml_tensor* i = ggml_new_tensor_2d(ctx, GGML_TYPE_I32, cols, T);
+    memcpy(a->data, src, (size_t)T * cols * rows * sizeof(float));
+    memcpy(b->data, bias, (size_t)E * rows * sizeof(float));
+    memcpy(i->data, ids, (size_t)T * cols * sizeof(int32_t));
+    struct ggml_tensor* y = ggml_add_id(ctx, a, b, i);
+    const int rc = run_graph(ctx, y);
+    if (rc == 0) memcpy(out, y->data, (size_t)T * cols * rows * sizeof(float));
+    ggml_free(ctx);
+    return rc;
 }
 
 /* ggml_rope_ext as the bridge calls it (ggml_ops_transformer.cpp:403-406): n_dims = head_dim, n_ctx_orig 0,

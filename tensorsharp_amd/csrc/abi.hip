@@ -2304,6 +2304,107 @@ int TSHip_MulMatIdF32(TSHipTensorView3D result, TSHipTensorView3D expert_weights
     });
 }
 
+/* ---- ggml_add_id: per-expert bias rows added to the rows of a mul_mat_id (ggml_ops_matmul.cpp:1123-1290) ---- */
+namespace {
+
+bool validate_add_id(const TSHipTensorView3D& result, const TSHipTensorView3D& src, const TSHipTensorView2D& bias, const void* ids,
+                     int ids_rows, int ids_cols)
+{
+    if (!validate_desc3(result, "result") || !validate_desc3(src, "src") || !validate_desc(bias, "bias")) return false;
+    if (ids == nullptr) {
+        set_last_error("Null pointer passed for ids.");
+        return false;
+    }
+    if (ids_rows <= 0 || ids_cols <= 0) {
+        set_last_error("addid requires positive id matrix dimensions.");
+        return false;
+    }
+    if (result.dim0 != src.dim0 || result.dim1 != src.dim1 || result.dim2 != src.dim2) {
+        set_last_error("addid expects result and src to have the same shape.");
+        return false;
+    }
+    if (src.dim0 != ids_rows || src.dim1 != ids_cols || src.dim2 != bias.dim1) {
+        set_last_error("addid expects src shape [tokens, expert_used, rows], bias shape [experts, rows], and ids shape [tokens, expert_used].");
+        return false;
+    }
+    if (!is_standard_view3(result) || !is_standard_view3(src) || !is_standard_view(bias)) {
+        set_last_error("Tensor layout is not supported by the addid path.");
+        return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+int TSHip_AddIdF32Device(TSHipTensorView3D result, TSHipTensorView3D src, TSHipTensorView2D bias, const int32_t* ids, int ids_rows,
+                         int ids_cols)
+{
+    return guarded(0, "addid", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_add_id(result, src, bias, ids, ids_rows, ids_cols)) return 0;
+        if (!launch_add_id_f32(static_cast<const float*>(src.data), src.stride0, src.stride1, static_cast<const float*>(bias.data), bias.stride0,
+                               bias.dim0, ids, ids_rows, ids_cols, src.dim2, static_cast<float*>(result.data), result.stride0, result.stride1,
+                               t_stream))
+            return 0;
+        clear_last_error();
+        return 1;
+    });
+}
+
+int TSHip_AddIdF32(TSHipTensorView3D result, TSHipTensorView3D src, TSHipTensorView2D bias, TSHipContiguousTensor ids, int ids_rows,
+                   int ids_cols)
+{
+    return guarded(0, "addid", [&]() -> int {
+        if (!ensure_backend()) return 0;
+        if (!validate_add_id(result, src, bias, ids.data, ids_rows, ids_cols)) return 0;
+        const int64_t n_ids = (int64_t)ids_rows * ids_cols;
+        if (ids.element_count != n_ids || (ids.element_type != 0 && ids.element_type != 3)) {
+            set_last_error("addid: ids must hold ids_rows x ids_cols I32 (or F32) values.");
+            return 0;
+        }
+        const int T = src.dim0, cols = src.dim1, rows = src.dim2, E = bias.dim0;
+        auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+        const size_t id_bytes = al((size_t)n_ids * sizeof(int32_t)), x_bytes = al((size_t)n_ids * rows * sizeof(float));
+        const size_t b_bytes = al((size_t)E * rows * sizeof(float));
+        std::lock_guard<std::recursive_mutex> lock(g_host_call_mutex);
+        if (!ws_reserve(id_bytes + x_bytes + b_bytes, id_bytes + x_bytes + b_bytes)) return 0;
+        char* dev = static_cast<char*>(g_ws.dev);
+        char* pin = static_cast<char*>(g_ws.pinned);
+        int32_t* id_host = reinterpret_cast<int32_t*>(pin);
+        for (int64_t i = 0; i < n_ids; ++i) {
+            const int32_t e = ids.element_type == 3 ? static_cast<const int32_t*>(ids.data)[i] : (int32_t)static_cast<const float*>(ids.data)[i];
+            if (e < 0 || e >= E) {
+                set_last_error("addid: expert id out of range.");
+                return 0;
+            }
+            id_host[i] = e;
+        }
+        float* xs = reinterpret_cast<float*>(pin + id_bytes);
+        for (int t = 0; t < T; ++t)
+            for (int sl = 0; sl < cols; ++sl)
+                std::memcpy(xs + ((size_t)t * cols + sl) * rows, static_cast<const float*>(src.data) + (size_t)t * src.stride0 + (size_t)sl * src.stride1,
+                            (size_t)rows * sizeof(float));
+        float* bs = reinterpret_cast<float*>(pin + id_bytes + x_bytes);
+        for (int e = 0; e < E; ++e)
+            std::memcpy(bs + (size_t)e * rows, static_cast<const float*>(bias.data) + (size_t)e * bias.stride0, (size_t)rows * sizeof(float));
+        hipStream_t stream = nullptr;
+        if (!hip_ok(hipMemcpyAsync(dev, pin, id_bytes + x_bytes + b_bytes, hipMemcpyHostToDevice, stream), "hipMemcpy(inputs)")) return 0;
+        float* x_dev = reinterpret_cast<float*>(dev + id_bytes);
+        // in place on the packed copy of src
+        if (!launch_add_id_f32(x_dev, (int64_t)cols * rows, rows, reinterpret_cast<const float*>(dev + id_bytes + x_bytes), rows, E,
+                               reinterpret_cast<const int32_t*>(dev), T, cols, rows, x_dev, (int64_t)cols * rows, rows, stream))
+            return 0;
+        if (!hip_ok(hipMemcpyAsync(xs, x_dev, (size_t)n_ids * rows * sizeof(float), hipMemcpyDeviceToHost, stream), "hipMemcpy(result)")) return 0;
+        if (!hip_ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return 0;
+        for (int t = 0; t < T; ++t)
+            for (int sl = 0; sl < cols; ++sl)
+                std::memcpy(static_cast<float*>(result.data) + (size_t)t * result.stride0 + (size_t)sl * result.stride1,
+                            xs + ((size_t)t * cols + sl) * rows, (size_t)rows * sizeof(float));
+        clear_last_error();
+        return 1;
+    });
+}
+
 }  // extern "C"
 
 namespace {

@@ -2,6 +2,8 @@
 // (TensorSharp.GGML.Native/ggml_ops_fused.cpp:21-640): RMSNorm rows and the SiLU-gated product.
 #include "tship_internal.h"
 
+#include <algorithm>
+
 #include <hip/hip_fp16.h>
 
 namespace tship {
@@ -218,6 +220,32 @@ bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, f
         return false;
     }
     return hip_ok(hipGetLastError(), "dense matmul launch");
+}
+
+// out[t][s][r] = src[t][s][r] + bias[ids[t][s]][r] (ggml_add_id: ggml.h:886-891); a pair with an id outside the table
+// gets no bias (the host entry point refuses such ids before anything is launched)
+__global__ void __launch_bounds__(256) add_id_f32_kernel(const float* __restrict__ src, int64_t s_s0, int64_t s_s1, const float* __restrict__ bias,
+                                                         int64_t b_s0, int E, const int32_t* __restrict__ ids, int cols, int rows,
+                                                         float* __restrict__ out, int64_t o_s0, int64_t o_s1, int64_t pairs)
+{
+    for (int64_t p = blockIdx.y; p < pairs; p += gridDim.y) {
+        const int t = (int)(p / cols), sl = (int)(p - (int64_t)t * cols);
+        const int e = ids[p];
+        const float* sp = src + t * s_s0 + sl * s_s1;
+        const float* bp = (e >= 0 && e < E) ? bias + e * b_s0 : nullptr;
+        float* op = out + t * o_s0 + sl * o_s1;
+        for (int r = blockIdx.x * 256 + threadIdx.x; r < rows; r += gridDim.x * 256) op[r] = sp[r] + (bp ? bp[r] : 0.f);
+    }
+}
+
+bool launch_add_id_f32(const float* src, int64_t s_s0, int64_t s_s1, const float* bias, int64_t b_s0, int E, const int32_t* ids, int T,
+                       int cols, int rows, float* out, int64_t o_s0, int64_t o_s1, hipStream_t stream)
+{
+    if (T <= 0 || cols <= 0 || rows <= 0) return true;
+    const int64_t pairs = (int64_t)T * cols;
+    hipLaunchKernelGGL(add_id_f32_kernel, dim3(std::min((rows + 255) / 256, 64), (unsigned)std::min<int64_t>(pairs, 65535)), dim3(256), 0, stream,
+                       src, s_s0, s_s1, bias, b_s0, E, ids, cols, rows, out, o_s0, o_s1, pairs);
+    return hip_ok(hipGetLastError(), "addid launch");
 }
 
 bool launch_mul_mat_id_f32(const float* w, int64_t w_s0, int64_t w_s1, int E, int rows, int K, const float* x, int64_t x_s0, int64_t x_s1,

@@ -203,6 +203,8 @@ bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, f
                          bool accumulate, hipStream_t stream);
 // out[t][s][0..rows) = W[ids[t][s]] (rows x K, fp32) * x[t][s % slots]; strides in elements, innermost stride 1;
 // T * cols <= 65535; rows of an id outside [0, E) are zero
+bool launch_add_id_f32(const float* src, int64_t s_s0, int64_t s_s1, const float* bias, int64_t b_s0, int E, const int32_t* ids, int T,
+                       int cols, int rows, float* out, int64_t o_s0, int64_t o_s1, hipStream_t stream);
 bool launch_mul_mat_id_f32(const float* w, int64_t w_s0, int64_t w_s1, int E, int rows, int K, const float* x, int64_t x_s0, int64_t x_s1,
                            int slots, const int32_t* ids, int T, int cols, float* out, int64_t o_s0, int64_t o_s1, hipStream_t stream);
 inline bool is_dense_type(int type) { return type == kTypeF32 || type == kTypeF16 || type == kTypeBF16; }

@@ -221,40 +221,114 @@ class GgufFile:
             raise ValueError(f"tensor {name!r} extends past the end of the file.")
         return self._bytes[begin:end]
 
+    def _device_bytes(self, offset, count, device):
+        """`count` bytes of the mapping from `offset` as a new torch uint8 tensor on `device`: one host-to-device copy
+        straight from the page cache"""
+        import torch
+        import warnings
+        t = torch.empty(count, dtype=torch.uint8, device=device)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", UserWarning)      # read-only mapping: it is only ever read
+            src = torch.frombuffer(self._map, dtype=torch.uint8, count=count, offset=offset)
+        t.copy_(src)
+        return t
+
+    @staticmethod
+    def is_expert_stack(info):
+        """A 3-D tensor holding the experts of one projection, [ne0, ne1, experts] (ModelBase.cs:507-510, :554)."""
+        return len(info.Shape) == 3 and "_exps." in info.Name
+
+    @classmethod
+    def should_store_quantized(cls, info):
+        """BackendExecutionPlan.ShouldStoreWeightQuantized (ModelBase.cs:499-511) for a backend that reads raw blocks:
+        everything but F32 that is a matrix or a stack of expert matrices."""
+        return info.Type != 0 and (len(info.Shape) == 2 or cls.is_expert_stack(info))
+
     def quantized_weight(self, name, device=None):
         """A 2-D tensor as a QuantizedWeight: over the mapping (host form), or copied to `device` (torch device)."""
         from .hip_basic_ops import QuantizedWeight
         info = self.Tensors[name]
         if len(info.Shape) != 2:
-            raise ValueError(f"tensor {name!r} is not a matrix: shape {info.Shape}")
+            raise ValueError(f"tensor {name!r} is not a matrix: shape {info.Shape}" +
+                             (" (a stack of experts: use expert_weights)" if self.is_expert_stack(info) else ""))
         data = self.tensor_data(name)
         if device is not None:
-            import torch
-            # one host-to-device copy straight from the page cache
-            import warnings
-            t = torch.empty(data.size, dtype=torch.uint8, device=device)
-            with warnings.catch_warnings():
-                warnings.simplefilter("ignore", UserWarning)      # read-only mapping: it is only ever read
-                src = torch.frombuffer(self._map, dtype=torch.uint8, count=data.size, offset=self.DataOffset + info.Offset)
-            t.copy_(src)
+            t = self._device_bytes(self.DataOffset + info.Offset, data.size, device)
             return QuantizedWeight(t, info.Type, info.Shape[0], info.Shape[1])
         # a view of the mapping, kept alive by this file object: adjacent tensors concatenate without a copy
         return QuantizedWeight.CreateExternalView(data, info.Type, info.Shape[0], info.Shape[1], self)
 
+    @staticmethod
+    def expert_weight_names(name, num_experts):
+        """Names of the per-expert weights a stack is split into: `blk.L.ffn_up_exps.weight` -> `blk.L.ffn_up_exps.<e>.weight`
+        (ModelBase.cs:559-569)."""
+        base = name[:-len(".weight")] if name.endswith(".weight") else name
+        return [f"{base}.{e}.weight" for e in range(int(num_experts))]
+
+    def expert_weights(self, name, device=None):
+        """The experts of a 3-D `*_exps.` tensor [ne0, ne1, E] as E QuantizedWeights of ne1 rows: expert e is the bytes at
+        e * (bytes / E) of the tensor (ModelBase.cs:554-595).  Host form: external views of the mapping, adjacent to
+        each other, so the whole stack concatenates back into one view without a copy; device form: one upload of
+        the whole tensor, the experts are slices of it."""
+        from .hip_basic_ops import QuantizedWeight
+        info = self.Tensors[name]
+        if not self.is_expert_stack(info):
+            raise ValueError(f"tensor {name!r} is not a stack of expert matrices: shape {info.Shape}")
+        ne0, ne1, count = info.Shape
+        data = self.tensor_data(name)
+        per_expert = data.size // count
+        if device is not None:
+            whole = self._device_bytes(self.DataOffset + info.Offset, data.size, device)
+            return [QuantizedWeight(whole[e * per_expert:(e + 1) * per_expert], info.Type, ne0, ne1) for e in range(count)]
+        return [QuantizedWeight.CreateExternalView(data[e * per_expert:(e + 1) * per_expert], info.Type, ne0, ne1, self)
+                for e in range(count)]
+
+    def float_tensor(self, name):
+        """An F32 / F16 / BF16 tensor as a float32 numpy array shaped [.., ne1, ne0] (the managed side's `_weights`)."""
+        info = self.Tensors[name]
+        raw = self.tensor_data(name)
+        shape = tuple(reversed(info.Shape))
+        if info.Type == 0:
+            return np.array(raw.view(np.float32)).reshape(shape)
+        if info.Type == 1:
+            return raw.view(np.float16).astype(np.float32).reshape(shape)
+        if info.Type == 30:
+            return (raw.view(np.uint16).astype(np.uint32) << 16).view(np.float32).reshape(shape)
+        raise ValueError(f"tensor {name!r} has a block format; use quantized_weight / expert_weights")
+
+    def load_quantized_weights(self, device=None):
+        """name -> QuantizedWeight for every tensor the reference keeps as raw blocks: matrices under their own name,
+        expert stacks split into `<base>.<e>.weight` (the `_quantWeights` dictionary of ModelBase.LoadWeights,
+        ModelBase.cs:540-625)."""
+        out = {}
+        for name, info in self.Tensors.items():
+            if not self.should_store_quantized(info):
+                continue
+            if self.is_expert_stack(info):
+                out.update(zip(self.expert_weight_names(name, info.Shape[2]), self.expert_weights(name, device)))
+            else:
+                out[name] = self.quantized_weight(name, device)
+        return out
+
     def preload(self, names=None):
-        """Upload matrices once through the bridge's preload export, keyed by their mapped address: later host-pointer
-        calls with the same weight pointer run from the device copy (ModelBase.cs:660-706).  Returns the weights."""
+        """Upload weights once through the bridge's preload export, keyed by their mapped address: later host-pointer
+        calls with the same weight pointer run from the device copy (ModelBase.cs:660-706).  Expert stacks go up expert
+        by expert under `<base>.<e>.weight`, which is what the per-expert calls pass.  Returns the weights."""
         from .hip_basic_ops import HipBasicOps
         out = {}
         for name in (names if names is not None else list(self.Tensors)):
             info = self.Tensors[name]
             # every block format the matmul kernels read (F32 / F16 / BF16 tensors stay with the host path)
-            if len(info.Shape) != 2 or info.Type not in MATMUL_TYPES:
+            if info.Type not in MATMUL_TYPES or not self.should_store_quantized(info):
                 continue
-            w = self.quantized_weight(name)
-            HipBasicOps.PreloadQuantizedWeight(w.ptr, w.ptr, w.ggml_type, w.ne0, w.ne1, w.raw_bytes)
-            self._preloaded.append(w.ptr)
-            out[name] = w
+            if self.is_expert_stack(info):
+                ws = dict(zip(self.expert_weight_names(name, info.Shape[2]), self.expert_weights(name)))
+            else:
+                ws = {name: self.quantized_weight(name)}
+            for n, w in ws.items():
+                HipBasicOps.PreloadQuantizedWeight(w.ptr, w.ptr, w.ggml_type, w.ne0, w.ne1, w.raw_bytes)
+                self._preloaded.append(w.ptr)
+                out[n] = w
         return out
 
     def close(self):

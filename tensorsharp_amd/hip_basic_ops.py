@@ -167,6 +167,56 @@ def FuseGateUpWeights(quant_weights, num_layers):
     return fused
 
 
+def FuseExpertGateUpWeights(quant_weights, num_layers, num_experts, biases=None):
+    """Twin of GptOssModel.FuseExpertGateUpWeights (GptOssModel.cs:126-180): per layer and expert,
+    blk.L.ffn_gate_exps.E.weight and blk.L.ffn_up_exps.E.weight of equal type and row length become
+    blk.L.ffn_gate_up_exps.E.weight (gate rows, then up rows; a copy, since gate and up live in different tensors of the
+    file).  `biases` (name -> float32 array [1, n], the split biases of GptOssModel.cs:95-121) are fused the same way.
+    Returns the number of experts fused."""
+    fused = 0
+    for layer in range(int(num_layers)):
+        for e in range(int(num_experts)):
+            gate_name, up_name = f"blk.{layer}.ffn_gate_exps.{e}.weight", f"blk.{layer}.ffn_up_exps.{e}.weight"
+            gw, uw = quant_weights.get(gate_name), quant_weights.get(up_name)
+            if gw is not None and uw is not None and gw.ggml_type == uw.ggml_type and gw.ne0 == uw.ne0:
+                quant_weights[f"blk.{layer}.ffn_gate_up_exps.{e}.weight"] = QuantizedWeight.ConcatOrCreateCopy(gw, uw)
+                del quant_weights[gate_name], quant_weights[up_name]
+                gw.Dispose()
+                uw.Dispose()
+                fused += 1
+            if biases is not None:
+                gb_name, ub_name = f"blk.{layer}.ffn_gate_exps.{e}.bias", f"blk.{layer}.ffn_up_exps.{e}.bias"
+                if gb_name in biases and ub_name in biases:
+                    biases[f"blk.{layer}.ffn_gate_up_exps.{e}.bias"] = np.concatenate(
+                        [biases.pop(gb_name).reshape(1, -1), biases.pop(ub_name).reshape(1, -1)], axis=1)
+    return fused
+
+
+def SplitExpertBiases(float_weights, num_layers):
+    """Twin of GptOssModel.SplitExpertBiases (GptOssModel.cs:93-124): blk.L.ffn_{gate,up,down}_exps.bias [E, n] become
+    blk.L.ffn_*_exps.E.bias [1, n].  Returns the number of tensors split."""
+    split = 0
+    for layer in range(int(num_layers)):
+        for kind in ("ffn_gate_exps", "ffn_up_exps", "ffn_down_exps"):
+            name = f"blk.{layer}.{kind}.bias"
+            if name not in float_weights:
+                continue
+            b = float_weights.pop(name)
+            for e in range(b.shape[0]):
+                float_weights[f"blk.{layer}.{kind}.{e}.bias"] = np.ascontiguousarray(b[e]).reshape(1, -1)
+            split += 1
+    return split
+
+
+def StackExpertWeights(weights):
+    """One weight holding the rows of all experts in order ([E * ne1] rows), the operand of
+    HipBasicOps.MoEExpertsGptOssForward: a view when the experts are byte-adjacent views of one mapping (a `*_exps.` tensor
+    split by GgufFile.expert_weights), else a copy into one aligned buffer (experts fused from two tensors)."""
+    if len(weights) == 1:
+        return weights[0]
+    return QuantizedWeight.ConcatOrCreateCopy(*weights)
+
+
 def FuseQKVWeights(quant_weights, num_layers):
     """Twin of the models' FuseQKVWeights (Qwen3Model.cs:57-85): attn_q / attn_k / attn_v of equal type and row length
     become blk.L.attn_qkv.weight."""
@@ -399,6 +449,26 @@ class HipBasicOps:
             ok = N.lib().TSHip_MulMatIdF32Device(HipBasicOps._view3(result), HipBasicOps._view3(expert_weights),
                                                  HipBasicOps._view3(input), C.c_void_p(ids.contiguous().data_ptr()), rows, cols)
         N.check_result(ok, "mulmatid")
+
+    @staticmethod
+    def AddId(result, src, bias, ids):
+        """result[t, s, :] = src[t, s, :] + bias[ids[t, s], :] (GgmlBasicOps.AddID, GgmlBasicOps.cs:1092-1108; the bias of
+        a MulMatId).  All host (numpy; ids int32 or float32) or all device (torch; ids int32) tensors; result may be src."""
+        host = isinstance(result, np.ndarray)
+        if (ids.ndim if host else ids.dim()) != 2 or (bias.ndim if host else bias.dim()) != 2:
+            raise NotImplementedError("addid expects 2D bias and id tensors.")
+        rows, cols = int(ids.shape[0]), int(ids.shape[1])
+        if host:
+            idc = np.ascontiguousarray(ids)
+            if idc.dtype not in (np.int32, np.float32):
+                raise ValueError("AddId ids must be Int32 or Float32.")
+            desc = N.ContiguousTensor(idc.ctypes.data, int(idc.size), 3 if idc.dtype == np.int32 else 0)
+            ok = N.lib().TSHip_AddIdF32(HipBasicOps._view3(result), HipBasicOps._view3(src), _host_view(bias, standard=True), desc, rows, cols)
+        else:
+            HipBasicOps.UseCurrentStream()
+            ok = N.lib().TSHip_AddIdF32Device(HipBasicOps._view3(result), HipBasicOps._view3(src), _device_view(bias),
+                                              C.c_void_p(ids.contiguous().data_ptr()), rows, cols)
+        N.check_result(ok, "addid")
 
     # -- embedding gather ------------------------------------------------------------------
     @staticmethod

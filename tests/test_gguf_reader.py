@@ -102,3 +102,78 @@ def test_rejects_an_alignment_that_is_not_a_power_of_two(tmp_path, alignment):
     p.write_bytes(blob)
     with pytest.raises(ValueError, match="power of two"):
         GgufFile(str(p))
+
+
+# ---- a MoE file: expert stacks as 3-D tensors (written by the reference's writer, tests/golden/make_golden_gguf.py) ----
+MOE_E, MOE_H, MOE_F = 4, 64, 32
+
+
+@pytest.fixture(scope="module")
+def moe_expect():
+    z = np.load(os.path.join(GOLD, "tiny_moe_gguf_expect.npz"))
+    return {k.replace("__", "."): z[k] for k in z.files}
+
+
+def test_expert_stacks_split_per_expert_like_the_reference(moe_expect):
+    """ModelBase.cs:554-595: expert e of a 3-D `*_exps.` tensor is the view at e * (bytes / experts) of the mapping,
+    stored under `<base>.<e>.weight`."""
+    from tensorsharp_amd.hip_basic_ops import QuantizedWeight
+    with GgufFile(os.path.join(GOLD, "tiny_moe.gguf")) as g:
+        assert g.GetString("general.architecture") == "gpt-oss"
+        assert g.GetUint32("gpt-oss.expert_count") == MOE_E and g.GetUint32("gpt-oss.expert_used_count") == 2
+        info = g.Tensors["blk.0.ffn_gate_exps.weight"]
+        assert info.Shape == (MOE_H, MOE_F, MOE_E) and info.Type == 39
+        assert g.GetTensorByteCount(info) == MOE_E * MOE_F * 34 == moe_expect["blk.0.ffn_gate_exps.weight"].size
+        assert g.Tensors["blk.0.ffn_gate_inp.bias"].Shape == (MOE_E,)
+        with pytest.raises(ValueError, match="stack of experts"):
+            g.quantized_weight("blk.0.ffn_gate_exps.weight")
+        with pytest.raises(ValueError, match="not a stack"):
+            g.expert_weights("blk.0.ffn_gate_inp.weight")
+        for name in ("blk.0.ffn_gate_exps.weight", "blk.0.ffn_down_exps.weight", "blk.1.ffn_up_exps.weight", "blk.1.ffn_down_exps.weight"):
+            info = g.Tensors[name]
+            ex = g.expert_weights(name)
+            whole = moe_expect[name]
+            per = whole.size // MOE_E
+            assert len(ex) == MOE_E
+            for e, w in enumerate(ex):
+                assert (w.ggml_type, w.ne0, w.ne1, w.raw_bytes) == (info.Type, info.Shape[0], info.Shape[1], per)
+                assert w.HasExternalHostView
+                np.testing.assert_array_equal(np.array(w.data), whole[e * per:(e + 1) * per])
+            # adjacent views of one mapping: the stack is one view again, no copy
+            stacked = QuantizedWeight.TryCreateConcatenatedView(*ex)
+            assert stacked is not None and stacked.ptr == ex[0].ptr and stacked.ne1 == MOE_E * info.Shape[1]
+            np.testing.assert_array_equal(np.array(stacked.data), whole)
+        ws = g.load_quantized_weights()
+        want = {f"blk.{l}.ffn_{p}_exps.{e}.weight" for l in (0, 1) for p in ("gate", "up", "down") for e in range(MOE_E)}
+        assert set(ws) == want          # the F32 router and biases are not stored as blocks
+        b = g.float_tensor("blk.0.ffn_down_exps.bias")
+        assert b.shape == (MOE_E, MOE_H)
+        np.testing.assert_array_equal(b.reshape(-1), moe_expect["blk.0.ffn_down_exps.bias"].view(np.float32))
+
+
+def test_gate_up_fusion_per_expert_and_bias_split(moe_expect):
+    """GptOssModel.cs:93-180: biases [E, n] are split per expert, gate and up of an expert are stacked (a copy: they live
+    in different tensors), and the per-expert stacks put together are the operand of the grouped expert stage."""
+    from tensorsharp_amd.hip_basic_ops import FuseExpertGateUpWeights, SplitExpertBiases, StackExpertWeights
+    with GgufFile(os.path.join(GOLD, "tiny_moe.gguf")) as g:
+        ws = g.load_quantized_weights()
+        fl = {n: g.float_tensor(n) for n in g.Tensors if n.endswith(".bias") and "_exps" in n}
+        assert SplitExpertBiases(fl, 2) == 3
+        assert fl["blk.0.ffn_up_exps.2.bias"].shape == (1, MOE_F)
+        assert FuseExpertGateUpWeights(ws, 2, MOE_E, fl) == 2 * MOE_E
+        assert "blk.0.ffn_gate_exps.0.weight" not in ws and "blk.0.ffn_up_exps.0.bias" not in fl
+        gate, up = moe_expect["blk.0.ffn_gate_exps.weight"], moe_expect["blk.0.ffn_up_exps.weight"]
+        per = gate.size // MOE_E
+        for e in range(MOE_E):
+            w = ws[f"blk.0.ffn_gate_up_exps.{e}.weight"]
+            assert (w.ne0, w.ne1, w.raw_bytes) == (MOE_H, 2 * MOE_F, 2 * per) and w.ptr % 64 == 0 and not w.HasExternalHostView
+            np.testing.assert_array_equal(w.data[:per], gate[e * per:(e + 1) * per])
+            np.testing.assert_array_equal(w.data[per:], up[e * per:(e + 1) * per])
+            fb = fl[f"blk.0.ffn_gate_up_exps.{e}.bias"]
+            assert fb.shape == (1, 2 * MOE_F)
+            np.testing.assert_array_equal(fb[0, :MOE_F], moe_expect["blk.0.ffn_gate_exps.bias"].view(np.float32)[e * MOE_F:(e + 1) * MOE_F])
+        gu = StackExpertWeights([ws[f"blk.0.ffn_gate_up_exps.{e}.weight"] for e in range(MOE_E)])
+        assert gu.ne1 == MOE_E * 2 * MOE_F and gu.raw_bytes == 2 * gate.size
+        dn = StackExpertWeights([ws[f"blk.0.ffn_down_exps.{e}.weight"] for e in range(MOE_E)])
+        assert dn.HasExternalHostView                           # still a view of the mapping
+        np.testing.assert_array_equal(np.array(dn.data), moe_expect["blk.0.ffn_down_exps.weight"])

@@ -339,3 +339,40 @@ def test_device_forms_refuse_strided_views(hip, oracle):
             assert "stride1 == 1" in N.get_last_error(), (name, N.get_last_error())
         assert call(good_out, good_x) == 1, (name, N.get_last_error())
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("device", [False, True])
+def test_add_id_bias_rows_by_expert(hip, oracle, device):
+    """TSHip_AddIdF32: result[t, s, :] = src[t, s, :] + bias[ids[t, s], :], bit-equal to the definition (one fp32 add)."""
+    import torch
+    from oracle.oracle import add_id
+    rng = np.random.default_rng(395)
+    T, cols, rows, E = 7, 4, 300, 9
+    src = rng.standard_normal((T, cols, rows)).astype(np.float32)
+    bias = rng.standard_normal((E, rows)).astype(np.float32)
+    ids = rng.integers(0, E, (T, cols)).astype(np.int32)
+    want = add_id(src, bias, ids)
+    if device:
+        s = torch.from_numpy(src).cuda()
+        out = torch.full_like(s, float("nan"))
+        hip.AddId(out, s, torch.from_numpy(bias).cuda(), torch.from_numpy(ids).cuda())
+        hip.AddId(s, s, torch.from_numpy(bias).cuda(), torch.from_numpy(ids).cuda())       # in place
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(s.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        out = np.full_like(src, np.nan)
+        hip.AddId(out, src, bias, ids)
+        assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+        # F32 ids are truncated like the bridge's read_i32_values; padded (strided) views are packed
+        wide = np.zeros((T, cols + 1, rows + 5), np.float32)
+        wide[:, :cols, :rows] = src
+        out2 = np.full_like(src, np.nan)
+        hip.AddId(out2, wide[:, :cols, :rows], bias, ids.astype(np.float32) + 0.3)
+        assert np.array_equal(out2.view(np.uint32), want.view(np.uint32))
+        with pytest.raises(RuntimeError, match="expert id out of range"):
+            hip.AddId(out2, src, bias, np.full((T, cols), E, np.int32))
+        with pytest.raises(RuntimeError, match="same shape"):
+            hip.AddId(out2[:, :, :rows - 4], src, bias, ids)
+        with pytest.raises(RuntimeError, match="bias shape"):
+            hip.AddId(out2, src, bias[:, :rows - 4], ids)

@@ -150,3 +150,17 @@ def test_mul_mat_id_brute_force_and_broadcast(oracle):
     mark = np.zeros((E, 1, 1), np.float32)
     mark[:, 0, 0] = np.arange(E) + 1
     assert np.array_equal(oracle.mul_mat_id(mark, np.ones((T, 1, 1), np.float32), ids)[:, :, 0], ids + 1)
+
+
+def test_add_id_definition_and_reference(reference):
+    """ggml_add_id (the per-expert bias of a mul_mat_id): the oracle is the definition written out; the reference's own
+    CPU op must agree bit for bit."""
+    from oracle.oracle import add_id
+    rng = np.random.default_rng(2710)
+    T, cols, rows, E = 5, 3, 37, 6
+    src = rng.standard_normal((T, cols, rows)).astype(np.float32)
+    bias = rng.standard_normal((E, rows)).astype(np.float32)
+    ids = rng.integers(0, E, (T, cols)).astype(np.int32)
+    want = add_id(src, bias, ids)
+    assert np.array_equal(want, src + bias[ids])                      # the same thing through numpy's gather
+    assert np.array_equal(reference.add_id(src, bias, ids).view(np.uint32), want.view(np.uint32))
