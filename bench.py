@@ -133,6 +133,81 @@ def library_fp16_gemm_us(torch, dev, m, n, k, iters=20):
     return ev * 1e3 / iters
 
 
+def timeline(args, torch, dev, HipBasicOps, QuantizedWeight, synth):
+    """Where the time of one decode launch goes: TSHip_SetGemvTimeline makes every wavefront of the GEMV kernel stamp the
+    100 MHz constant clock at entry, after the activations are staged and at exit.  The launch is repeated (cycling weight
+    copies larger than the memory-side cache) and every repetition is read back; times are relative to the launch's
+    first entry, medians over the repetitions."""
+    import ctypes as C
+    import numpy as np
+    from tensorsharp_amd import hip_native as N
+    if args.timeline == "layer":
+        shapes, t = [(n, k) for _, n, k in LAYER], Q4_K
+    else:
+        t, n, k = (int(v) for v in args.timeline.split(","))
+        shapes = [(n, k)]
+    wbytes = sum(n * row_bytes(t, k) for n, k in shapes)
+    copies = max(2, min(48, int(700e6 // wbytes) + 1))
+    xs = [torch.randn((1, k), device=dev, dtype=torch.float32) for _, k in shapes]
+    ys = [torch.empty((1, n), device=dev, dtype=torch.float32) for n, _ in shapes]
+    # (the packs hold raw addresses: the weights must stay alive beside them)
+    keep = [[QuantizedWeight(synth.random_weight(t, n, k, dev, seed=77 * c + i), t, k, n) for i, (n, k) in enumerate(shapes)]
+            for c in range(copies)]
+    packs = [HipBasicOps.PrepareGroup(ys, xs, ws) for ws in keep]
+    cap_waves = 1 << 13
+    reps = max(8, min(args.steps, 64))
+    buf = torch.zeros((reps, cap_waves * 8), dtype=torch.int64, device=dev)
+    set_region = lambda r: N.check_result(N.lib().TSHip_SetGemvTimeline(C.c_void_p(buf[r].data_ptr()), cap_waves * 64), "timeline")
+    # a decode stream: launches back to back, every one of the last `reps` stamping a region of its own
+    set_region(0)
+    for i in range(300):
+        HipBasicOps.AddmmQuantGroupDevice(packs[i % copies])
+    buf.zero_()
+    for r in range(reps):
+        set_region(r)
+        HipBasicOps.AddmmQuantGroupDevice(packs[r % copies])
+    torch.cuda.synchronize()
+    # the same stream timed with HIP events, with the stamping build and with the normal one
+    step = lambda i: HipBasicOps.AddmmQuantGroupDevice(packs[i % copies])
+    set_region(0)
+    ev_tl = time_region(step, 1000, torch)[0]
+    N.lib().TSHip_SetGemvTimeline(None, 0)
+    for i in range(200):
+        step(i)
+    ev_plain = time_region(step, 1000, torch)[0]
+    runs = []
+    for r in range(reps):
+        a = buf[r].cpu().numpy().reshape(-1, 8)
+        runs.append(a[a[:, 4] != 0].copy())
+    first = np.array([r[:, 0].min() for r in runs], dtype=np.int64)
+    last = np.array([r[:, 4].max() for r in runs], dtype=np.int64)
+    stream = {"period_us_p50": round(float(np.median(np.diff(first))) * 0.01, 2),
+              "span_us_p50": round(float(np.median(last - first)) * 0.01, 2),
+              "gap_last_exit_to_next_entry_us_p50": round(float(np.median(first[1:] - last[:-1])) * 0.01, 2),
+              "events_us_per_launch_stamping_build": round(ev_tl, 2), "events_us_per_launch_normal_build": round(ev_plain, 2)}  # ms over 1000 launches = us per launch
+    waves = runs[0].shape[0]
+    rel = lambda col: np.median(np.stack([(r[:, col] - r[:, 0].min()) * 0.01 for r in runs]), axis=0)       # us
+    e, xa, s_, f1, x = rel(0), rel(1), rel(2), rel(3), rel(4)
+    xcc = (runs[0][:, 5] & 0xff).astype(int)
+    prob = ((runs[0][:, 5] >> 8) & 0xff).astype(int)
+    q = lambda v: [round(float(np.percentile(v, p)), 2) for p in (0, 10, 50, 90, 100)]
+    per_xcc = {}
+    for c in sorted(set(xcc.tolist())):
+        m = xcc == c
+        per_xcc[str(c)] = {"waves": int(m.sum()), "entry_min_p50_max": [round(float(f(e[m])), 2) for f in (np.min, np.median, np.max)],
+                           "exit_p0_p10_p50_p90_p100": q(x[m]), "life_p50": round(float(np.median(x[m] - e[m])), 2)}
+    per_prob = {str(pi): {"waves": int((prob == pi).sum()), "entry_p50": round(float(np.median(e[prob == pi])), 2),
+                          "activations_arrived_p50": round(float(np.median(xa[prob == pi])), 2),
+                          "staged_p50": round(float(np.median(s_[prob == pi])), 2),
+                          "first_step_done_p50": round(float(np.median(f1[prob == pi])), 2),
+                          "exit_p0_p10_p50_p90_p100": q(x[prob == pi])} for pi in sorted(set(prob.tolist()))}
+    return {"timeline": args.timeline, "type": t, "shapes": shapes, "weight_bytes": wbytes, "weight_copies": copies, "repetitions": reps,
+            "wavefronts": int(waves), "clock": "s_memrealtime, 10 ns", "stream": stream,
+            "entry_p0_p10_p50_p90_p100": q(e), "activations_arrived_p0_p10_p50_p90_p100": q(xa),
+            "staged_p0_p10_p50_p90_p100": q(s_), "first_step_done_p0_p10_p50_p90_p100": q(f1), "exit_p0_p10_p50_p90_p100": q(x),
+            "stage_time_p50": round(float(np.median(s_ - e)), 2), "per_xcc": per_xcc, "per_problem": per_prob}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,6 +225,9 @@ def main():
     ap.add_argument("--matmul", metavar="TYPE,M,N,K",
                     help="time only one matmul shape (GGUF type id, rows, out features, in features) through "
                          "TSHip_AddmmQuantF32Device, --steps calls after --warmup; for profiling a single kernel")
+    ap.add_argument("--timeline", metavar="layer|TYPE,N,K",
+                    help="per-wavefront entry / staged / exit times of one decode launch (the headline grouped launch, or a "
+                         "single matrix) from the library's timeline build of the GEMV kernel; prints a JSON summary")
     ap.add_argument("--moe", metavar="T", type=int,
                     help="time only the configs[3] MoE expert stage (32 MXFP4 experts, top-4, 2880) at T tokens, --steps calls; "
                          "for profiling its kernels")
@@ -241,6 +319,10 @@ def main():
                         "pct_mfma_fp16_peak": round(100 * fl / (us * 1e-6) / 1e12 / MFMA_FP16_PEAK_TFLOPS, 1)})
         return res
 
+
+    if args.timeline:
+        print(json.dumps(timeline(args, torch, dev, HipBasicOps, QuantizedWeight, synth)))
+        return
 
     if args.aux:
         op, t, rows, k = args.aux.split(",")

@@ -312,6 +312,14 @@ TSHIP_EXPORT int TSHip_MulMatIdF32(TSHipTensorView3D result, TSHipTensorView3D e
 TSHIP_EXPORT int TSHip_MulMatIdF32Device(TSHipTensorView3D result, TSHipTensorView3D expert_weights, TSHipTensorView3D input,
                                          const int32_t* ids, int ids_rows, int ids_cols);
 
+/* Diagnostics, no counterpart in the reference: while a device buffer is set, the single-row (GEMV) launches of the plain
+ * activation mode run a build of the kernel in which every wavefront writes 64-bit words at byte offset
+ * 64 * (workgroup * 8 + wavefront) of the buffer: the 100 MHz constant-clock times of [0] its entry, [1] the arrival of its
+ * activations, [2] the barrier behind the staging, [3] the end of its first weight step, [4] its exit, and [5] (XCC id |
+ * problem index << 8 | wavefront index << 16).  Launches with more wavefronts than capacity_bytes / 64 run the normal kernel.  Pass a null buffer to switch it off.  For profiling runs only
+ * (bench.py --timeline); not thread-safe. */
+TSHIP_EXPORT int TSHip_SetGemvTimeline(void* device_buffer, int64_t capacity_bytes);
+
 /* replaces TSGgml_AddIdF32 (ggml_ops_matmul.cpp:1123-1290, :1451-1473; GgmlNative.cs:442-448, :1081-1084; managed
  * GgmlBasicOps.AddID :1092-1108): ggml_add_id, the per-expert bias that goes with a mul_mat_id,
  *   result[t][s][r] = src[t][s][r] + bias[ids[t][s]][r],  src / result [T x ids_cols x rows], bias [E x rows],

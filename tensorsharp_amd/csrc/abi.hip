@@ -1225,6 +1225,18 @@ int TSHip_SetStream(void* hip_stream)
     return 1;
 }
 
+int TSHip_SetGemvTimeline(void* device_buffer, int64_t capacity_bytes)
+{
+    const int64_t per_wave = (int64_t)gemv_timeline_slots() * (int64_t)sizeof(uint64_t);
+    if (device_buffer != nullptr && (capacity_bytes < per_wave || (reinterpret_cast<uintptr_t>(device_buffer) & 7) != 0)) {
+        set_last_error("gemv timeline: the buffer must be 8-byte aligned device memory of at least 64 bytes per wavefront.");
+        return 0;
+    }
+    set_gemv_timeline(static_cast<uint64_t*>(device_buffer), device_buffer ? capacity_bytes / per_wave : 0);
+    clear_last_error();
+    return 1;
+}
+
 int TSHip_DequantizeToF32Device(int ggml_type, const void* src, int64_t num_elements, float* dst)
 {
     return guarded(-1, "dequantize", [&]() -> int {

@@ -811,10 +811,24 @@ struct Step {
 
 // ACT: the activation mode of every problem of the launch (compile time: the plain kernel carries none of
 // the other modes' code or registers)
-template <typename F, int ACT>
-__device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, int mode, uint32_t* lds)
+// TL: the timeline build of the kernel (diagnostics, see set_gemv_timeline): every wavefront leaves the 100 MHz
+// constant-clock time of its entry, of the moment x is staged and of its exit in tl[]; the plain build has none of it.
+// u64 per wavefront: entry, activations arrived, activations staged (behind the barrier), first weight step consumed, exit,
+// (XCC id | problem << 8 | wavefront-in-launch << 16); the stamps stay in scalar registers until the exit, so that no store
+// of theirs stands between the loads being timed
+constexpr int kTimelineSlots = 8;
+// EAGER > 0: the build for launches in which no wavefront has more than one row group and a group has at most EAGER
+// steps.  Such a launch is all latency: with one step requested ahead a wavefront waits for memory once per step.
+// Here the activations are requested first (so that their staging waits for nothing else: memory answers a wavefront
+// in order), then every step of the wavefront's group at once, and the steps are consumed as they arrive.  Measured on
+// one box against the streaming build: MXFP4 5760 x 2880 7.0 -> 6.0 us, 2880 x 2880 5.7 -> 5.0 us, Q4_K 4096 x 4096
+// 5.9 -> 5.5 us; Q8_0 9728 x 2560 loses (9.9 -> 10.8 us) and has no eager build.
+template <typename F, int ACT, bool TL, int EAGER>
+__device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg, int mode, uint32_t* lds, uint64_t* tl, int prob)
 {
     const int lane = threadIdx.x & 63;
+    uint64_t t_entry = 0, t_x = 0, t_staged = 0, t_first = 0;
+    if (TL) t_entry = __builtin_amdgcn_s_memrealtime();
     constexpr int LPR = F::kLPR, RPG = 64 / LPR;     // lanes per row, rows per group
     const int sub = lane / LPR, l16 = lane % LPR;    // row of the group, lane inside the row
     const int K = P.K;
@@ -946,13 +960,27 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // launches of a decode step: fused FFN 33.9 -> 32.2 us in an A/B on one box); plain launches lose (4096 x 14336
     // 12.7 -> 14.2 us) and so does the RMSNorm mode, whose staging is as short as the plain one (28672 x 4096 17.2 vs 16.0 us).
     const bool strict = mode == 1, deep = ACT == kActSiluMul && !strict;
-    fetch(fgroup, fstep, cur);
-    advance(fgroup, fstep);
-    if (deep) {
-        fetch(fgroup, fstep, nxt);
+    Step<F> eager[EAGER > 0 ? EAGER : 1];
+    if constexpr (EAGER > 0) {
+        stage_issue(0);
+        __builtin_amdgcn_sched_barrier(0);       // the activations' loads stay ahead of the weights'
+#pragma unroll
+        for (int s = 0; s < EAGER; ++s) fetch(s < nsteps ? gw : ngroups, s, eager[s]);
+    } else {
+        fetch(fgroup, fstep, cur);
         advance(fgroup, fstep);
+        if (deep) {
+            fetch(fgroup, fstep, nxt);
+            advance(fgroup, fstep);
+        }
+        stage_issue(0);
     }
-    stage_issue(0);
+    if (TL && EAGER == 0) {
+        // the first chunk of activations is in registers (the weight step requested before them has arrived too: memory
+        // answers a wavefront in order)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        t_x = __builtin_amdgcn_s_memrealtime();
+    }
     stage_commit(0);
     for (int base = kThreads * kStageChunk; base < items; base += kThreads * kStageChunk) {
         stage_issue(base);
@@ -965,6 +993,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         if (lane == 0) red[threadIdx.x >> 6] = ss;
     }
     __syncthreads();
+    if (TL) t_staged = __builtin_amdgcn_s_memrealtime();
     float out_scale = 1.0f;      // factor on every row sum
     if (act == kActRmsNorm) {
         double tot = 0.0;
@@ -1019,11 +1048,31 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
             advance(fgroup, fstep);
         }
     };
-    for (;;) {
-        if (cur.group >= ngroups) break;
-        one(cur, nxt);
-        if (nxt.group >= ngroups) break;
-        one(nxt, cur);
+    if constexpr (EAGER > 0) {
+#pragma unroll
+        for (int s = 0; s < EAGER; ++s) {
+            if (s < nsteps) consume(eager[s]);       // uniform
+            if (TL && s == 0) t_first = __builtin_amdgcn_s_memrealtime();
+        }
+    } else {
+        for (;;) {
+            if (cur.group >= ngroups) break;
+            one(cur, nxt);
+            if (TL && t_first == 0) t_first = __builtin_amdgcn_s_memrealtime();
+            if (nxt.group >= ngroups) break;
+            one(nxt, cur);
+        }
+    }
+    if (TL) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the last stores have been acknowledged
+        const uint64_t t_exit = __builtin_amdgcn_s_memrealtime();
+        if (lane == 0) {
+            const int wave_in_launch = (int)blockIdx.x * kWaves + (int)(threadIdx.x >> 6);
+            uint64_t* my_tl = tl + (size_t)wave_in_launch * kTimelineSlots;
+            my_tl[0] = t_entry, my_tl[1] = t_x, my_tl[2] = t_staged, my_tl[3] = t_first, my_tl[4] = t_exit;
+            // hardware register 20 (XCC_ID), 4 bits from bit 0
+            my_tl[5] = (uint64_t)(__builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xfu) | ((uint64_t)prob << 8) | ((uint64_t)wave_in_launch << 16);
+        }
     }
 }
 
@@ -1033,9 +1082,9 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
 struct GemvProblems {
     GemvProblem p[kMaxGroup];
 };
-template <int TYPE, int ACT>
+template <int TYPE, int ACT, bool TL, int EAGER>
 __global__ void __launch_bounds__(kThreads) gemv_kernel(int b0, int b1, int b2, int b3, int b4, int b5, int b6, int b7, int b8, int count,
-                                                        int strict, const GemvProblems G)
+                                                        int strict, const GemvProblems G, uint64_t* tl)
 {
     static_assert(kMaxGroup == 8, "one scalar argument per table entry");
     extern __shared__ uint32_t lds[];
@@ -1049,13 +1098,29 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(int b0, int b1, int b2, 
     if (6 < count && bx >= b6) { i = 6; lo = b6; hi = b7; }
     if (7 < count && bx >= b7) { i = 7; lo = b7; hi = b8; }
     const int wg = bx - lo, nwg = hi - lo;
-    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT>(G.p[i], wg, nwg, strict, lds);
-    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT>(G.p[i], wg, nwg, strict, lds);
-    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT>(G.p[i], wg, nwg, strict, lds);
-    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT>(G.p[i], wg, nwg, strict, lds);
-    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT>(G.p[i], wg, nwg, strict, lds);
-    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT>(G.p[i], wg, nwg, strict, lds);
-    else gemv_body<FmtQ80, ACT>(G.p[i], wg, nwg, strict, lds);
+    // Eager build: the problem's fields arrive with one round trip.  Read lazily, where the code first needs them, they
+    // cost one dependent scalar load after the other (seven before the first weight request, about 1 us), which a launch of
+    // a few microseconds feels (MXFP4 5760 x 2880: 6.3 -> 6.0 us).  The streaming build keeps the lazy reads: with them
+    // the wavefronts of a long launch start a little apart and it measured faster that way (123 MB grouped launch 24.0
+    // against 25.1 us, Q8_0 4096 x 4096 8.2 against 8.9 us on one box).
+    GemvProblem Pv;
+    if constexpr (EAGER > 0) {
+        Pv = G.p[i];
+        uint64_t w = reinterpret_cast<uint64_t>(Pv.w), x = reinterpret_cast<uint64_t>(Pv.x), y = reinterpret_cast<uint64_t>(Pv.y);
+        uint64_t add = reinterpret_cast<uint64_t>(Pv.add), nw = reinterpret_cast<uint64_t>(Pv.norm_w), eid = reinterpret_cast<uint64_t>(Pv.expert_id);
+        asm volatile("" : "+s"(w), "+s"(x), "+s"(y), "+s"(add), "+s"(nw), "+s"(eid), "+s"(Pv.w_bytes), "+s"(Pv.expert_stride));
+        asm volatile("" : "+s"(Pv.N), "+s"(Pv.K), "+s"(Pv.pair_rows), "+s"(Pv.pair_kind), "+s"(Pv.n_experts), "+s"(Pv.eps), "+s"(Pv.limit));
+        Pv.w = reinterpret_cast<const uint8_t*>(w), Pv.x = reinterpret_cast<const float*>(x), Pv.y = reinterpret_cast<float*>(y);
+        Pv.add = reinterpret_cast<const float*>(add), Pv.norm_w = reinterpret_cast<const float*>(nw), Pv.expert_id = reinterpret_cast<const int*>(eid);
+    }
+    const GemvProblem& P = EAGER > 0 ? Pv : G.p[i];
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else gemv_body<FmtQ80, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
@@ -1077,16 +1142,43 @@ size_t lds_bytes_for(int type, int K)
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 constexpr double kStrictBytes = 96.0 * 1024 * 1024;   // launches streaming at least this much run strict (see gemv_body)
 
-template <int TYPE, int ACT>
-bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
+// Diagnostics: while a buffer is set, plain-activation launches run the timeline build of the kernel and leave
+// kTimelineSlots stamps per wavefront in it (the last launch wins).  Not thread-safe; meant for a profiling run.
+uint64_t* g_timeline = nullptr;
+int64_t g_timeline_waves = 0;
+
+template <int TYPE, int ACT, bool TL, int EAGER>
+bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    auto kern = gemv_kernel<TYPE, ACT>;
+    auto kern = gemv_kernel<TYPE, ACT, TL, EAGER>;
     if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
     GemvProblems gp;
     std::memcpy(gp.p, g.p, sizeof(gp.p));
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g.wg_begin[0], g.wg_begin[1], g.wg_begin[2], g.wg_begin[3],
-                       g.wg_begin[4], g.wg_begin[5], g.wg_begin[6], g.wg_begin[7], g.wg_begin[8], g.count, g.strict, gp);
+                       g.wg_begin[4], g.wg_begin[5], g.wg_begin[6], g.wg_begin[7], g.wg_begin[8], g.count, g.strict, gp,
+                       TL ? g_timeline : nullptr);
     return hip_ok(hipGetLastError(), "gemv launch");
+}
+
+// steps the eager build of a format holds in registers (0: the format has no eager build)
+template <int TYPE>
+constexpr int kEagerSteps = TYPE == kTypeQ4_K ? 4 : TYPE == kTypeMXFP4 ? 6 : 0;
+int eager_steps(int type)
+{
+    return type == kTypeQ4_K ? kEagerSteps<kTypeQ4_K> : type == kTypeMXFP4 ? kEagerSteps<kTypeMXFP4> : 0;
+}
+
+template <int TYPE, int ACT>
+bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
+{
+    const bool tl = ACT == kActPlain && g_timeline != nullptr && (int64_t)grid * kWaves <= g_timeline_waves;
+    if constexpr (ACT == kActPlain && kEagerSteps<TYPE> > 0) {
+        if (g.strict == 2)
+            return tl ? launch_type_tl<TYPE, kActPlain, true, kEagerSteps<TYPE>>(g, grid, lds, stream)
+                      : launch_type_tl<TYPE, kActPlain, false, kEagerSteps<TYPE>>(g, grid, lds, stream);
+    }
+    if (tl) return launch_type_tl<TYPE, kActPlain, true, 0>(g, grid, lds, stream);
+    return launch_type_tl<TYPE, ACT, false, 0>(g, grid, lds, stream);
 }
 
 }  // namespace
@@ -1106,6 +1198,13 @@ int gemv_max_k(int type)
 }
 
 int gemv_max_group() { return kMaxGroup; }
+
+int gemv_timeline_slots() { return kTimelineSlots; }
+void set_gemv_timeline(uint64_t* device_buffer, int64_t wavefronts)
+{
+    g_timeline = device_buffer;
+    g_timeline_waves = device_buffer ? wavefronts : 0;
+}
 
 // one staging pass covers 8 float4 per thread
 // the RMSNorm mode stages rows of any length the kernel can hold (its scale is applied at the store)
@@ -1214,6 +1313,17 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     }
     for (int i = count; i <= kMaxGroup; ++i) g.wg_begin[i] = begin;
     const int act = args[0].act;
+    // eager build: every problem has at most one row group per wavefront and few enough steps per group
+    if (act == kActPlain && eager_steps(type) > 0) {
+        bool ok = true;
+        for (int i = 0; i < count; ++i) {
+            const int out_rows = args[i].pair_rows ? args[i].pair_rows : args[i].N, out_rpg = args[i].pair_rows ? rpg / 2 : rpg;
+            const int groups = (out_rows + out_rpg - 1) / out_rpg, waves = (g.wg_begin[i + 1] - g.wg_begin[i]) * kWaves;
+            const int steps = (args[i].K / unit_elems(type) + lpr - 1) / lpr;
+            ok = ok && groups <= waves && steps <= eager_steps(type);
+        }
+        if (ok) g.strict = 2;
+    }
     for (int i = 1; i < count; ++i)
         if (args[i].act != act) {
             set_last_error("gemv: the problems of one launch must share the activation mode.");

@@ -130,6 +130,9 @@ struct GemvArgs {
     float limit = 0.f;
 };
 int gemv_max_group();
+// diagnostics: per-wavefront time stamps of the GEMV launches (see TSHip_SetGemvTimeline)
+int gemv_timeline_slots();
+void set_gemv_timeline(uint64_t* device_buffer, int64_t wavefronts);
 bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t stream);
 
 // ---- prefill GEMM ---------------------------------------------------------------------------

@@ -104,6 +104,7 @@ SIGNATURES = {
                                                     C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_float]),
     "TSHip_MulMatIdF32": (C.c_int, [TensorView3D, TensorView3D, TensorView3D, ContiguousTensor, C.c_int, C.c_int]),
     "TSHip_MulMatIdF32Device": (C.c_int, [TensorView3D, TensorView3D, TensorView3D, C.c_void_p, C.c_int, C.c_int]),
+    "TSHip_SetGemvTimeline": (C.c_int, [C.c_void_p, C.c_int64]),
     "TSHip_AddIdF32": (C.c_int, [TensorView3D, TensorView3D, TensorView2D, ContiguousTensor, C.c_int, C.c_int]),
     "TSHip_AddIdF32Device": (C.c_int, [TensorView3D, TensorView3D, TensorView2D, C.c_void_p, C.c_int, C.c_int]),
     "TSHip_GetRowsQuantF32": (C.c_int, [TensorView2D, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int64,
