@@ -1454,12 +1454,31 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
                 args[a].limit = limit;
             }
             if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
-            for (int a = 0; a < A; ++a)
-                args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes, E};
-            if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
-            if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, E, (int)H, T == 1, static_cast<float*>(result.data),
-                                    result.stride0, stream))
-                return 0;
+            // The down projections and the weighted sum over a token's experts.  Where the format's row groups hold as
+            // many rows as a token has experts (k = 4 for the 16-lane formats) one launch does both: a wavefront takes
+            // row h of the token's k experts side by side and stores sum_s w_s (row . act_s + bias), in slot order: the
+            // order of the reference's single-token path (GptOssModel.cs:718-735; a batch adds in expert order, :737-812).
+            const bool routed = T == 1 && k == gemv_routed_slots(ggml_type) && (dn_bytes & 3) == 0 &&
+                                (int64_t)E * dn_bytes < kMaxOperandBytes && (int64_t)k * F <= gemv_max_k(ggml_type);
+            if (routed) {
+                for (int t = 0; t < T; ++t) {
+                    args[t] = GemvArgs{down_w, (int64_t)E * dn_bytes, gu + (int64_t)t * k * F,
+                                       static_cast<float*>(result.data) + (int64_t)t * result.stride0, (int)H, (int)F};
+                    args[t].expert_stride = dn_bytes;
+                    args[t].n_experts = E;
+                    args[t].slot_ids = ids + (int64_t)t * k;
+                    args[t].slot_w = weights + (int64_t)t * k;
+                    args[t].slot_bias = down_bias;
+                }
+                if (!launch_gemv_group(ggml_type, T, args, stream)) return 0;
+            } else {
+                for (int a = 0; a < A; ++a)
+                    args[a] = GemvArgs{down_w, dn_bytes, gu + (int64_t)a * F, dn + (int64_t)a * H, (int)H, (int)F, ids + a, dn_bytes, E};
+                if (!launch_gemv_group(ggml_type, A, args, stream)) return 0;
+                if (!launch_moe_combine(dn, down_bias, ids, weights, nullptr, T, k, E, (int)H, T == 1, static_cast<float*>(result.data),
+                                        result.stride0, stream))
+                    return 0;
+            }
         } else {
             MoeMaps maps{reinterpret_cast<int*>(ws + o_offsets), reinterpret_cast<int*>(ws + o_token),
                          reinterpret_cast<int*>(ws + o_expert), reinterpret_cast<int*>(ws + o_pos),

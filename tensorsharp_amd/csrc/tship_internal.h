@@ -123,6 +123,13 @@ struct GemvArgs {
     int pair_rows = 0;                // F > 0: W is F gate rows then F up rows (N = 2F) and y[j] = glu(gate_j, up_j), j < F
     int pair_kind = 0;                // 0: glu = silu(g) * u; 1: GPT-OSS SwiGLU at the store (act must be 0; norm_w the optional
                                       // [E][2F] bias indexed by expert_id, eps = alpha, limit = clamp)
+    // routed sum (MoE down projection of one token): w is the stack of n_experts matrices expert_stride bytes apart
+    // (w_bytes spans the stack), x holds gemv_routed_slots(type) activation vectors of K floats back to back, and
+    // y[h] = sum_slot slot_w[slot] * (W[slot_ids[slot]][h] . x[slot] + slot_bias[slot_ids[slot]][h]) in slot order; slots
+    // whose id lies outside [0, n_experts) add nothing.  Excludes expert_id, pair_rows, add and the activation modes.
+    const int* slot_ids = nullptr;    // device [slots]
+    const float* slot_w = nullptr;    // device [slots]
+    const float* slot_bias = nullptr; // device [n_experts][N], optional
     const float* add = nullptr;       // optional: y = add + W x (add may be y)
     int act = 0;                      // activation mode, see launch_gemv
     const float* norm_w = nullptr;
@@ -130,6 +137,8 @@ struct GemvArgs {
     float limit = 0.f;
 };
 int gemv_max_group();
+// slots (experts per token) the routed-sum mode of a format combines: 64 / lanes per row, 0 where the format has none
+int gemv_routed_slots(int type);
 // diagnostics: per-wavefront time stamps of the GEMV launches (see TSHip_SetGemvTimeline)
 int gemv_timeline_slots();
 void set_gemv_timeline(uint64_t* device_buffer, int64_t wavefronts);
