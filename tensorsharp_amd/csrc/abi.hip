@@ -605,7 +605,7 @@ bool run_expert_set_device(const TSHipTensorView2D& out, const float* base, int6
     }
     if (grouped) {
         const float* xv = static_cast<const float*>(x.data);
-        const int types[] = {kTypeQ8_0, kTypeQ4_K, kTypeMXFP4, kTypeQ6_K, kTypeQ5_K, kTypeQ4_0, kTypeQ4_1};
+        const int types[] = {kTypeQ8_0, kTypeQ4_K, kTypeMXFP4, kTypeQ6_K, kTypeQ5_K, kTypeQ4_0, kTypeQ4_1, kTypeQ5_0, kTypeQ5_1, kTypeIQ4_NL};
         for (int e = 0; e < n; ++e)
             if (!check_device_operands(x, ex[e].up, ex[e].up_type) || !check_device_operands(x, ex[e].down, ex[e].down_type) ||
                 (ex[e].gate && !check_device_operands(x, ex[e].gate, ex[e].gate_type)))

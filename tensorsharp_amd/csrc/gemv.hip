@@ -457,18 +457,25 @@ struct FmtMXFP4 {
 };
 
 // ---- Q4_0 / Q4_1 -----------------------------------------------------------------------------
-// Blocks of 32 weights: fp16 d (Q4_1: also fp16 m), then 16 bytes whose low nibble is weight j and high nibble weight
-// j + 16; value d * (q - 8) (Q4_1: d * q + m) (ggml-quants.c dequantize_row_q4_0 / q4_1; ManagedQuantizedOps.cs:268-330).
+// Blocks of 32 weights behind a small header: fp16 d (Q4_1 / Q5_1: also fp16 m; Q5_0 / Q5_1: also 32 fifth bits), then 16
+// bytes whose low nibble is weight j and high nibble weight j + 16.  Values d * (q - 8), d * q + m, d * (q5 - 16),
+// d * q5 + m, d * table[q] (ggml-quants.c dequantize_row_q4_0 / q4_1 / q5_0 / q5_1 / iq4_nl; ManagedQuantizedOps.cs:268-409,
+// :559-577).
 // LDS unit (80 B): for quant dword i, dwords 4i .. 4i+3 = (x[4i], x[4i+2]), (x[4i+1], x[4i+3]), then the same of
 // x[16 + ..]; then the sum of the scaled fp16 activations and the unit's power-of-two scale.  Nibbles masked in place
-// are fp16 subnormals (q * 2^-24, high nibbles 16 q * 2^-24) for v_dot2_f32_f16; the -8 / + m term leaves through the sum.
-template <bool HAS_MIN>
-struct FmtQ4Legacy {
+// are fp16 subnormals (q * 2^-24, high nibbles 16 q * 2^-24) for v_dot2_f32_f16, a fifth bit joins them one bit above
+// (bit 4 / bit 8), IQ4_NL's table values enter as bytes value + 128; the -8 / -16 / -128 / + m term leaves through the sum.
+template <int TYPE>
+struct FmtLegacy {
+    static constexpr bool kMin = TYPE == kTypeQ4_1 || TYPE == kTypeQ5_1;
+    static constexpr bool kFive = TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1;
+    static constexpr bool kTable = TYPE == kTypeIQ4_NL;
+    static constexpr int kHdr = 2 + (kMin ? 2 : 0) + (kFive ? 4 : 0);      // bytes before the 16 quant bytes
     static constexpr int kLPR = 16;
     static constexpr int kUnitElems = 32;
     static constexpr int kLdsDwords = 20;
-    static constexpr int kRegs = 6;
-    static constexpr int kBlock = HAS_MIN ? 20 : 18;
+    static constexpr int kBlock = kHdr + 16;
+    static constexpr int kRegs = (kBlock + 2 + 3) / 4;     // dwords of the window: the block at byte 0 or 2 of it
 
     static __device__ __forceinline__ int64_t row_bytes(int K) { return (int64_t)(K >> 5) * kBlock; }
 
@@ -528,44 +535,78 @@ struct FmtQ4Legacy {
         return L;
     }
 
-    // the block sits at byte 0 or 2 of a 24-byte dword-aligned window.  Returns p & 3.
+    // the block sits at byte 0 or 2 of a dword-aligned window of kRegs dwords.  Returns p & 3.
     static __device__ __forceinline__ uint32_t load(__amdgpu_buffer_rsrc_t rs, const Lane& L, uint32_t soff,
                                                     uint32_t row_delta, int /*slot*/, bool live, uint32_t (&w)[kRegs])
     {
         const uint32_t p = L.voff + row_delta;
         const uint32_t al = live ? (p & ~3u) : kDeadOffset;
         buf_load4(rs, al, soff, &w[0]);
-        w[4] = buf_load1(rs, al + 16, soff);
-        w[5] = HAS_MIN ? buf_load1(rs, al + 20, soff) : 0u;
+#pragma unroll
+        for (int i = 4; i < kRegs; ++i) w[i] = buf_load1(rs, al + 4u * i, soff);
         return p & 3u;
+    }
+
+    // the aligned dword at byte `off` (a multiple of 2) of the block, which starts 0 (odd == false) or 2 bytes into w
+    static __device__ __forceinline__ uint32_t at(const uint32_t (&w)[kRegs], bool odd, int off)
+    {
+        // even block: byte off of w; odd block: byte off + 2 of w
+        const int e = off, o = off + 2;
+        const uint32_t ve = (e & 3) ? __builtin_amdgcn_alignbyte(w[(e >> 2) + 1 < kRegs ? (e >> 2) + 1 : kRegs - 1], w[e >> 2], 2) : w[e >> 2];
+        const uint32_t vo = (o & 3) ? __builtin_amdgcn_alignbyte(w[(o >> 2) + 1 < kRegs ? (o >> 2) + 1 : kRegs - 1], w[o >> 2], 2) : w[o >> 2];
+        return odd ? vo : ve;
     }
 
     static __device__ __forceinline__ float dot(const uint32_t (&w)[kRegs], const Lane& /*L*/, uint32_t o, const uint32_t* xu_dw)
     {
         const bool odd = (o & 2u) != 0;
+        const uint32_t hdr = at(w, odd, 0);                   // d | (m or the next two bytes) << 16
         H2U dh, mh;
-        dh.u = odd ? (w[0] >> 16) : (w[0] & 0xffffu);
-        mh.u = HAS_MIN ? (odd ? (w[1] & 0xffffu) : (w[0] >> 16)) : 0u;
+        dh.u = hdr & 0xffffu;
+        mh.u = kMin ? hdr >> 16 : 0u;
         const float d = (float)dh.h.x, m = (float)mh.h.x;
+        const uint32_t qh = kFive ? at(w, odd, kMin ? 4 : 2) : 0u;
         const uint4* xu = reinterpret_cast<const uint4*>(xu_dw);
         float lo = 0.f, hi = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            // quant bytes start 2 (Q4_1: 4) bytes into the block
-            uint32_t q;
-            if (HAS_MIN) q = odd ? __builtin_amdgcn_alignbyte(w[i + 2], w[i + 1], 2) : w[i + 1];
-            else q = odd ? w[i + 1] : __builtin_amdgcn_alignbyte(w[i + 1], w[i], 2);
-            const uint32_t q8 = q >> 8;
+            const uint32_t q = at(w, odd, kHdr + 4 * i);      // quant bytes 4i .. 4i + 3
             const uint4 xv = xu[i];
-            lo = dot2(q & 0x000f000fu, xv.x, lo);
-            lo = dot2(q8 & 0x000f000fu, xv.y, lo);
-            hi = dot2(q & 0x00f000f0u, xv.z, hi);
-            hi = dot2(q8 & 0x00f000f0u, xv.w, hi);
+            if constexpr (kTable) {
+                // {-127,-104,-83,-65,-49,-35,-22,-10, 1,13,25,38,53,69,89,113} + 128 as bytes, looked up with v_perm
+                const uint32_t t0 = 0x3f2d1801u, t1 = 0x766a5d4fu, t2 = 0xa6998d81u, t3 = 0xf1d9c5b5u;
+                uint32_t nl = q & 0x0f0f0f0fu, nh = (q >> 4) & 0x0f0f0f0fu;
+                const uint32_t ml = ((nl >> 3) & 0x01010101u) * 0xffu, mh2 = ((nh >> 3) & 0x01010101u) * 0xffu;
+                const uint32_t sl = nl & 0x07070707u, sh = nh & 0x07070707u;
+                nl = (__builtin_amdgcn_perm(t3, t2, sl) & ml) | (__builtin_amdgcn_perm(t1, t0, sl) & ~ml);
+                nh = (__builtin_amdgcn_perm(t3, t2, sh) & mh2) | (__builtin_amdgcn_perm(t1, t0, sh) & ~mh2);
+                // bytes (0, 2) and (1, 3) into the low bytes of the two halves: subnormals (value + 128) * 2^-24
+                lo = dot2(__builtin_amdgcn_perm(0u, nl, 0x0c020c00u), xv.x, lo);
+                lo = dot2(__builtin_amdgcn_perm(0u, nl, 0x0c030c01u), xv.y, lo);
+                hi = dot2(__builtin_amdgcn_perm(0u, nh, 0x0c020c00u), xv.z, hi);
+                hi = dot2(__builtin_amdgcn_perm(0u, nh, 0x0c030c01u), xv.w, hi);
+            } else {
+                const uint32_t q8 = q >> 8;
+                uint32_t a = q & 0x000f000fu, b = q8 & 0x000f000fu, c = q & 0x00f000f0u, e = q8 & 0x00f000f0u;
+                if constexpr (kFive) {
+                    // fifth bits of elements 4i .. 4i + 3 (bit 4 above a low nibble) and 16 + 4i .. (bit 8 above a high nibble)
+                    const uint32_t t = qh >> (4 * i), u = qh >> (16 + 4 * i);
+                    a |= ((t & 1u) << 4) | ((t & 4u) << 18);
+                    b |= ((t & 2u) << 3) | ((t & 8u) << 17);
+                    c |= ((u & 1u) << 8) | ((u & 4u) << 22);
+                    e |= ((u & 2u) << 7) | ((u & 8u) << 21);
+                }
+                lo = dot2(a, xv.x, lo);
+                lo = dot2(b, xv.y, lo);
+                hi = dot2(c, xv.z, hi);
+                hi = dot2(e, xv.w, hi);
+            }
         }
         const uint4 tail = xu[4];
         const float sum = __uint_as_float(tail.x), xscale = __uint_as_float(tail.y);
+        if constexpr (kTable) return d * ((lo + hi) * 16777216.f - 128.f * sum) * xscale;
         const float qx = lo * 16777216.f + hi * 1048576.f;
-        return (HAS_MIN ? d * qx + m * sum : d * (qx - 8.f * sum)) * xscale;
+        return (kMin ? d * qx + m * sum : d * (qx - (kFive ? 16.f : 8.f) * sum)) * xscale;
     }
 };
 
@@ -1170,13 +1211,14 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(int b0, int b1, int b2, 
     else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
-    else if (TYPE == kTypeQ4_0) gemv_body<FmtQ4Legacy<false>, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
-    else if (TYPE == kTypeQ4_1) gemv_body<FmtQ4Legacy<true>, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+    else if (TYPE == kTypeQ4_0 || TYPE == kTypeQ4_1 || TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1 || TYPE == kTypeIQ4_NL)
+        gemv_body<FmtLegacy<TYPE>, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else gemv_body<FmtQ80, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
-int unit_lds_bytes(int type) { return type == kTypeMXFP4 || type == kTypeQ4_0 || type == kTypeQ4_1 ? 80 : type == kTypeQ6_K ? 176 : 144; }
+bool legacy_type(int type) { return type == kTypeQ4_0 || type == kTypeQ4_1 || type == kTypeQ5_0 || type == kTypeQ5_1 || type == kTypeIQ4_NL; }
+int unit_lds_bytes(int type) { return type == kTypeMXFP4 || legacy_type(type) ? 80 : type == kTypeQ6_K ? 176 : 144; }
 int lanes_per_row(int type)
 {
     return type == kTypeQ4_K || type == kTypeQ5_K ? FmtQ4K::kLPR : type == kTypeMXFP4 ? FmtMXFP4::kLPR : type == kTypeQ6_K ? FmtQ6K::kLPR : FmtQ80::kLPR;
@@ -1243,8 +1285,7 @@ int gemv_max_k(int type)
     case kTypeMXFP4: return (int)(kMaxLds / 80 / FmtMXFP4::kLPR) * FmtMXFP4::kLPR * 32;
     case kTypeQ6_K: return (int)(kMaxLds / 176 / FmtQ6K::kLPR) * FmtQ6K::kLPR * 64;
     case kTypeQ5_K: return (int)(kMaxLds / 144 / FmtQ4K::kLPR) * FmtQ4K::kLPR * 64;
-    case kTypeQ4_0:
-    case kTypeQ4_1: return (int)(kMaxLds / 80 / 16) * 16 * 32;
+    case kTypeQ4_0: case kTypeQ4_1: case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL: return (int)(kMaxLds / 80 / 16) * 16 * 32;
     default: return 0;
     }
 }
@@ -1270,7 +1311,7 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
         set_last_error("gemv: group size out of range.");
         return false;
     }
-    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K && type != kTypeQ5_K && type != kTypeQ4_0 && type != kTypeQ4_1) {
+    if (type != kTypeQ8_0 && type != kTypeQ4_K && type != kTypeMXFP4 && type != kTypeQ6_K && type != kTypeQ5_K && !legacy_type(type)) {
         set_last_error("gemv: unsupported type.");
         return false;
     }
@@ -1422,6 +1463,9 @@ bool launch_gemv_group(int type, int count, const GemvArgs* args, hipStream_t st
     case kTypeQ5_K: return TSHIP_GEMV_DISPATCH(kTypeQ5_K);
     case kTypeQ4_0: return TSHIP_GEMV_DISPATCH(kTypeQ4_0);
     case kTypeQ4_1: return TSHIP_GEMV_DISPATCH(kTypeQ4_1);
+    case kTypeQ5_0: return TSHIP_GEMV_DISPATCH(kTypeQ5_0);
+    case kTypeQ5_1: return TSHIP_GEMV_DISPATCH(kTypeQ5_1);
+    case kTypeIQ4_NL: return TSHIP_GEMV_DISPATCH(kTypeIQ4_NL);
     default: return TSHIP_GEMV_DISPATCH(kTypeQ8_0);
     }
 #undef TSHIP_GEMV_DISPATCH

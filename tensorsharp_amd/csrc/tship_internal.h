@@ -61,8 +61,7 @@ inline int64_t block_bytes(int type)
 }
 
 // formats the GEMV / GEMM kernels read: every block format of ManagedQuantizedOps.cs:40-59 except Q8_1 (an activation
-// format that no GGUF file stores weights in; see is_matmul_type); the ones without a GEMV specialisation take the
-// matrix-core kernels for single rows too
+// format that no GGUF file stores weights in; see is_matmul_type)
 inline bool is_quant_type(int type)
 {
     switch (type) {
@@ -75,7 +74,7 @@ inline bool is_quant_type(int type)
 inline bool has_gemv(int type)
 {
     return type == kTypeQ8_0 || type == kTypeQ4_K || type == kTypeMXFP4 || type == kTypeQ6_K || type == kTypeQ5_K ||
-           type == kTypeQ4_0 || type == kTypeQ4_1;
+           type == kTypeQ4_0 || type == kTypeQ4_1 || type == kTypeQ5_0 || type == kTypeQ5_1 || type == kTypeIQ4_NL;
 }
 // formats with a dequantizer (DequantizeToF32, embedding gather): every block format the managed code reads
 // (ManagedQuantizedOps.cs:40-59)

@@ -187,7 +187,7 @@ def make_blocks(name, N, K, rng):
     return (MORE_TYPES[name], inputs.random_blocks(name, N, K, rng), N, K)
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "q5_k", "q6_k"])
 @pytest.mark.parametrize("n", [1, 6])
 def test_experts_swiglu_single_row_other_gemv_formats(hip, oracle, name, n):
     # one row: the down projection of each expert is a GEMV that forms silu(gate) * up while it stages its activations,

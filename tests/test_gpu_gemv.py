@@ -101,15 +101,15 @@ def test_unaligned_sub_weight_views(hip, oracle, name):
 
 def host_case_weight(oracle, name, N, K, rng):
     """(ggml type, raw blocks) of a random weight in any format with a GEMV kernel."""
-    from oracle.oracle import Q6_K, Q5_K, Q4_0, Q4_1
+    from oracle.oracle import Q6_K, MORE_TYPES
     if name in T:
         return T[name], oracle.quantize(T[name], (rng.standard_normal(N * K) * 0.02).astype(np.float32))
     if name == "q6_k":
         return Q6_K, q6k_weight(N, K, 35)
-    return {"q5_k": Q5_K, "q4_0": Q4_0, "q4_1": Q4_1}[name], inputs.random_blocks(name, N, K, rng)
+    return MORE_TYPES[name], inputs.random_blocks(name, N, K, rng)
 
 
-@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4", "q6_k", "q5_k", "q4_0", "q4_1"])
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4", "q6_k", "q5_k", "q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl"])
 def test_host_entry_points(hip, oracle, name):
     """Drop-in path: host pointers, strided activation view, preload key, batch form."""
     rng = np.random.default_rng(35)
@@ -323,12 +323,15 @@ def test_q5_k_shapes(hip, oracle, N, K):
     assert np.all(run_device(hip, Q5_K, wq, N, K, np.zeros((1, K), np.float32)) == 0)
 
 
-# ---- Q4_0 / Q4_1: 18- and 20-byte blocks of 32 weights ----
-@pytest.mark.parametrize("name", ["q4_0", "q4_1"])
+# ---- Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL: 18- to 24-byte blocks of 32 weights ----
+LEGACY = ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl"]
+
+
+@pytest.mark.parametrize("name", LEGACY)
 @pytest.mark.parametrize("N,K", [(1, 32), (3, 96), (7, 1056), (130, 2560), (257, 4096), (1001, 2880), (4096, 14336)])
 def test_q4_legacy_shapes(hip, oracle, name, N, K):
-    from oracle.oracle import Q4_0, Q4_1
-    t = {"q4_0": Q4_0, "q4_1": Q4_1}[name]
+    from oracle.oracle import MORE_TYPES
+    t = MORE_TYPES[name]
     rng = np.random.default_rng(N * 17 + K)
     wq = inputs.random_blocks(name, N, K, rng)
     x = rng.standard_normal((1, K)).astype(np.float32)
@@ -338,13 +341,14 @@ def test_q4_legacy_shapes(hip, oracle, name, N, K):
     assert np.all(run_device(hip, t, wq, N, K, np.zeros((1, K), np.float32)) == 0)
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1"])
+@pytest.mark.parametrize("name", LEGACY)
 def test_q4_legacy_views_at_odd_rows(hip, oracle, name):
-    # 35 blocks per row: Q4_0 rows alternate between byte 0 and byte 2 of a dword; views that start rows into a tensor
+    # 35 blocks per row: rows of the 18- and 22-byte blocks alternate between byte 0 and byte 2 of a dword; views that
+    # start rows into a tensor
     import torch
     from tensorsharp_amd import QuantizedWeight
-    from oracle.oracle import Q4_0, Q4_1
-    t = {"q4_0": Q4_0, "q4_1": Q4_1}[name]
+    from oracle.oracle import MORE_TYPES
+    t = MORE_TYPES[name]
     rng = np.random.default_rng(44)
     N, K = 64, 1120
     wq = inputs.random_blocks(name, N + 3, K, rng)
@@ -356,3 +360,28 @@ def test_q4_legacy_views_at_odd_rows(hip, oracle, name):
         y = hip.LinearForward(xd, QuantizedWeight(dev[rb * rs:(rb + N) * rs], t, K, N))
         torch.cuda.synchronize()
         check("q4_k", y.cpu().numpy(), oracle.matmul_f64(t, wq[rb * rs:(rb + N) * rs], N, K, x))
+
+
+@pytest.mark.parametrize("name", LEGACY)
+def test_legacy_formats_element_by_element(hip, oracle, name):
+    """A one-hot activation picks one weight: every element position of a block (nibble halves, fifth bits, table entries)
+    must come out as the dequantizer gives it, blocks with all-zero and all-one quant bits included."""
+    from oracle.oracle import MORE_TYPES
+    t = MORE_TYPES[name]
+    rng = np.random.default_rng(4400)
+    N, K = 6, 64
+    wq = inputs.random_blocks(name, N, K, rng).reshape(N * 2, -1)
+    hdr = wq.shape[1] - 16
+    wq[0, hdr:] = 0xff                       # every nibble 15
+    wq[1, hdr:] = 0x00
+    if name in ("q5_0", "q5_1"):
+        wq[0, hdr - 4:hdr] = 0xff            # every fifth bit set
+        wq[1, hdr - 4:hdr] = 0x00
+        wq[2, hdr - 4:hdr] = [0x01, 0x80, 0x00, 0x10]     # single bits: elements 0, 15, 28
+    wq = wq.reshape(-1)
+    w = oracle.dequantize(t, wq, N * K).reshape(N, K)
+    for k in range(K):
+        x = np.zeros((1, K), np.float32)
+        x[0, k] = 1.5
+        y = run_device(hip, t, wq, N, K, x)
+        assert np.allclose(y[0], 1.5 * w[:, k], rtol=2e-6, atol=1e-9), (name, k, y[0], 1.5 * w[:, k])
