@@ -37,7 +37,7 @@ LAYER = [  # name, N (out), K (in) — BASELINE.json configs[1]
 
 
 def row_bytes(t, k):
-    return {2: 18 * (k // 32), 3: 20 * (k // 32), Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), Q5_K: 176 * (k // 256), Q6_K: 210 * (k // 256), MXFP4: 17 * (k // 32)}[t]
+    return {2: 18 * (k // 32), 3: 20 * (k // 32), 6: 22 * (k // 32), 7: 24 * (k // 32), 20: 18 * (k // 32), Q8_0: 34 * (k // 32), Q4_K: 144 * (k // 256), Q5_K: 176 * (k // 256), Q6_K: 210 * (k // 256), MXFP4: 17 * (k // 32)}[t]
 
 
 def algorithmic_bytes(t, n, k, m=1):

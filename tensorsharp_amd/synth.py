@@ -161,7 +161,24 @@ def quantize_q4_1_simple(w):
     return out.reshape(-1)
 
 
-QUANTIZERS = {2: quantize_q4_0_simple, 3: quantize_q4_1_simple, 8: quantize_q8_0, 12: quantize_q4_k_simple, 13: quantize_q5_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
+def _random_legacy_blocks(header_bytes, with_min):
+    """Blocks of 32 weights whose quant bits are random and whose fp16 scale (and minimum) suit weights ~ N(0, 0.02): for
+    the formats that only the throughput measurements use (Q5_0, Q5_1, IQ4_NL); values do not follow `w`."""
+    def make(w):
+        nb = w.numel() // 32
+        g = torch.Generator(device=w.device)
+        g.manual_seed(int(w.numel()) + header_bytes)
+        out = torch.randint(0, 256, (nb, header_bytes + 16), dtype=torch.uint8, device=w.device, generator=g)
+        d = torch.full((nb,), 2.5e-3 if header_bytes != 2 else 4e-4, device=w.device)
+        out[:, 0:2] = _half_bytes(d)
+        if with_min:
+            out[:, 2:4] = _half_bytes(torch.full((nb,), -0.04, device=w.device))
+        return out.reshape(-1)
+    return make
+
+
+QUANTIZERS = {6: _random_legacy_blocks(6, False), 7: _random_legacy_blocks(8, True), 20: _random_legacy_blocks(2, False),
+              2: quantize_q4_0_simple, 3: quantize_q4_1_simple, 8: quantize_q8_0, 12: quantize_q4_k_simple, 13: quantize_q5_k_simple, 14: quantize_q6_k_simple, 39: quantize_mxfp4}
 
 
 def random_weight(ggml_type, n_rows, n_cols, device, seed, sigma=0.02, chunk_rows=4096):
