@@ -414,7 +414,7 @@ def main():
                    "bytes_per_step": step_bytes, "launches_per_step": 1, "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "tship::gemv_kernel<12, 0> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
+                     "kernel": "tship::gemv_kernel<12, 0, false, 0> (grouped Q4_K GEMV)", "avg_launch_us": round(kern_us, 3),
                      "bytes_per_launch": step_bytes},
     }
 
@@ -453,12 +453,15 @@ def main():
     # The same shape with MXFP4 weights (the third format of the metric; BASELINE names MXFP4 for the MoE stage only, so
     # this is beside the metric's own prefill figure, not in place of it): the weight blocks go to the block-scaled
     # matrix instruction as they are and every activation is two MX fp6 terms, so a k-tile is two fp6 x fp4 instructions
-    # where fp16 operands take four of half the rate.  `frac` stays against the fp16 peak of the other formats.
+    # where fp16 operands take four of half the rate.  The kernel's operand type is fp6 x fp4, so `frac` prices the
+    # algorithmic flops against that instruction's peak; the figure against the fp16 peak of the other formats, and the
+    # instruction rate (two terms per activation: twice the algorithmic flops), stand beside it.
     if not args.no_extra:
         mx = prefill(MXFP4, pm, pn, pk, 20)
         out["roofline_prefill_mxfp4"] = {
-            "bound": "mfma", "achieved": mx["TFLOPs"], "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(mx["TFLOPs"] / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+            "bound": "mfma", "achieved": mx["TFLOPs"], "peak": MFMA_FP6_FP4_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(mx["TFLOPs"] / MFMA_FP6_FP4_PEAK_TFLOPS, 4), "traffic": None,
+            "frac_of_fp16_peak": round(mx["TFLOPs"] / MFMA_FP16_PEAK_TFLOPS, 4),
             "workload": "MXFP4 prefill GEMM M=2048 N=21504 K=5376: raw fp4 blocks x two MX fp6 (E2M3) activation terms, f32 accumulate",
             "kernel": "tship::gemm_mx_kernel<256, 3> (+ tship::convert_x_mx_kernel on the activations, inside the timed call)",
             "avg_call_us": mx["us_per_call_events"], "flops_per_call": 2 * pm * pn * pk, "calls_timed": 20,
@@ -551,6 +554,16 @@ def main():
 
         extra["cfg2_q4_k_layer_decode_ctx512"] = layer_decode(512, 200)
         extra["cfg2_q4_k_layer_decode_ctx4096"] = layer_decode(4096, 200)
+        # the same seven matrices as the headline, but as the dependent chain a decode step really runs (RMSNorm + QKV,
+        # attention over 512 cached tokens, Wo + residual, RMSNorm + gate | up + SiLU, down + residual: six launches):
+        # every launch pays its start, its tail and the gap to the next one, which the grouped launch pays once
+        chain = extra["cfg2_q4_k_layer_decode_ctx512"]
+        out["roofline_decode_chain"] = {
+            "bound": "hbm", "achieved": chain["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(chain["GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
+            "workload": "configs[1] shapes as one dependent decode layer at context 512 (TSHip_TransformerLayerDecodeDevice)",
+            "kernel": "six launches: tship::gemv_kernel<12, ...> x 4, tship::attn_decode_kernel, tship::attn_combine_kernel",
+            "avg_call_us": chain["us_per_layer_events"], "bytes_per_call": chain["bytes"]}
         # fused SwiGLU FFN at decode (configs[1] shapes: hidden 4096, intermediate 14336, Q4_K, one token):
         # RMSNorm -> gate_up GEMV -> SiLU*up -> down GEMV + residual, one ABI call (4 launches)
         def fused_ffn(copies=3):
