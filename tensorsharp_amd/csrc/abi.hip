@@ -553,7 +553,27 @@ struct ExpertSetLayout {
     size_t act_stride;   // floats between the activation rows of consecutive experts
     size_t dn_stride;    // floats between their down outputs
     size_t act_off, dn_off, tmp_off, mm_off, mm_bytes, total;
+    // more than one row, block formats only: every linear of the set is one tile-table GEMM per block type over the experts'
+    // pointers (rows e * M .. of the packed [n * M] activation / result matrices belong to expert e)
+    bool tiled;
+    int bm;              // rows per m-tile
+    size_t x1_off, x2_off;        // converted activations of the [n M x H] gathered input and of the [n M x I] gated rows
+    size_t tbl_off, tbl_bytes;    // tile tables, offset table, row map
+    size_t chunk_off, chunk_bytes;
 };
+
+// block formats with a tile-table GEMM
+bool has_tile_gemm(int type)
+{
+    switch (type) {
+    case kTypeQ8_0: case kTypeQ4_K: case kTypeMXFP4: case kTypeQ6_K: case kTypeQ5_K:
+    case kTypeQ4_0: case kTypeQ4_1: case kTypeQ5_0: case kTypeQ5_1: case kTypeIQ4_NL: return true;
+    default: return false;
+    }
+}
+
+// activation layout of a tile-table launch over expert pointers: MXFP4 on 32-row units reads MX fp6 pairs
+int expert_tiles_x_layout(int type, int bm, int K) { return type == kTypeMXFP4 && bm == 32 && K <= 32768 ? 1 : 0; }
 
 ExpertSetLayout expert_set_layout(int M, int n, const ExpertFfn* ex, int H, int I, int N)
 {
@@ -571,7 +591,93 @@ ExpertSetLayout expert_set_layout(int M, int n, const ExpertFfn* ex, int H, int 
         L.mm_bytes = std::max(L.mm_bytes, matmul_ws_bytes(ex[e].down_type, M, I, N, false, false));
     }
     L.total = L.mm_off + L.mm_bytes;
+    // the tiled form
+    const int64_t rows = (int64_t)n * M;
+    bool tiled = M > 1 && rows <= 65535;
+    for (int e = 0; e < n && tiled; ++e) {
+        auto fits = [](int type, int64_t wrows, int64_t k) {
+            return has_tile_gemm(type) && row_size(type, k) * (size_t)wrows < (size_t)kMaxOperandBytes;
+        };
+        tiled = (ex[e].gate != nullptr) == (ex[0].gate != nullptr) && fits(ex[e].up_type, I, H) && fits(ex[e].down_type, N, I) &&
+                (!ex[e].gate || fits(ex[e].gate_type, I, H));
+    }
+    tiled = tiled && gemm_workspace_bytes((int)rows, std::max(H, I)) < (size_t)kMaxOperandBytes;
+    if (!tiled) return L;
+    L.tiled = true;
+    L.bm = M > 160 ? 128 : 32;
+    const int ld = ex[0].gate ? 2 * I : I;
+    L.act_stride = (size_t)M * ld;
+    L.dn_stride = (size_t)M * N;
+    const int max_tiles = n * ((M + L.bm - 1) / L.bm);
+    size_t off = 0;
+    auto take = [&](size_t b) { const size_t o = off; off += al(b); return o; };
+    L.act_off = take((size_t)rows * ld * sizeof(float));
+    L.dn_off = take((size_t)rows * N * sizeof(float));
+    L.tmp_off = take((size_t)rows * I * sizeof(float));
+    L.x1_off = take(gemm_workspace_bytes((int)rows, H));
+    L.x2_off = take(gemm_workspace_bytes((int)rows, I));
+    L.tbl_bytes = al((size_t)max_tiles * 4) * 3 + al((size_t)n * 8) + al((size_t)rows * 4);
+    L.tbl_off = take(L.tbl_bytes);
+    const GemmTiles plan_tiles{nullptr, nullptr, nullptr, max_tiles, L.bm, 0};
+    for (int e = 0; e < n; ++e) {
+        auto need = [&](int type, int nn, int kk) {
+            return gemm_chunk_ws_bytes(type, (int)rows, nn, kk, &plan_tiles, false, expert_tiles_x_layout(type, L.bm, kk));
+        };
+        if (ex[e].gate) L.chunk_bytes = std::max(L.chunk_bytes, need(ex[e].gate_type, I, H));
+        L.chunk_bytes = std::max(L.chunk_bytes, need(ex[e].up_type, I, H));
+        L.chunk_bytes = std::max(L.chunk_bytes, need(ex[e].down_type, N, I));
+    }
+    L.chunk_off = take(L.chunk_bytes);
+    L.mm_off = off, L.mm_bytes = 0;
+    L.total = off;
     return L;
+}
+
+// One linear of a tiled expert set: per block type one tile-table GEMM over the members whose weight has that type.
+// x: fp32 source rows (ldx), gathered through row_map when given; the members' results go to rows slot * M .. of c.
+struct ExpertLinear {
+    const void* w[kMaxExpertSet];
+    int type[kMaxExpertSet];
+};
+
+bool run_expert_linear_tiled(const ExpertSetLayout& L, char* ws, int n, int M, const ExpertLinear& lin, const float* x, int64_t ldx,
+                             bool gather, size_t x_off, float* c, int64_t ldc, int out_features, int K, hipStream_t stream)
+{
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const int per = (M + L.bm - 1) / L.bm;
+    const size_t tile_bytes = al((size_t)n * per * 4);
+    int* t_expert = reinterpret_cast<int*>(ws + L.tbl_off);
+    int* t_row0 = reinterpret_cast<int*>(ws + L.tbl_off + tile_bytes);
+    int* t_rows = reinterpret_cast<int*>(ws + L.tbl_off + 2 * tile_bytes);
+    int64_t* offs = reinterpret_cast<int64_t*>(ws + L.tbl_off + 3 * tile_bytes);
+    int* row_map = reinterpret_cast<int*>(ws + L.tbl_off + 3 * tile_bytes + al((size_t)n * 8));
+    const int rows = n * M;
+    bool handled[kMaxExpertSet] = {};
+    for (int first = 0; first < n; ++first) {
+        if (handled[first]) continue;
+        const int t = lin.type[first];
+        // base pointer: the lowest address among the type's members, so that every offset is >= 0
+        uintptr_t base = reinterpret_cast<uintptr_t>(lin.w[first]);
+        for (int e = first; e < n; ++e)
+            if (lin.type[e] == t) base = std::min(base, reinterpret_cast<uintptr_t>(lin.w[e]));
+        ExpertTileSpec spec{};
+        for (int e = first; e < n; ++e) {
+            if (lin.type[e] != t) continue;
+            handled[e] = true;
+            spec.off[spec.count] = (int64_t)(reinterpret_cast<uintptr_t>(lin.w[e]) - base);
+            spec.slot[spec.count] = e;
+            ++spec.count;
+        }
+        const int layout = expert_tiles_x_layout(t, L.bm, K);
+        if (!launch_expert_tiles(spec, M, L.bm, t_expert, t_row0, t_rows, offs, gather ? row_map : nullptr, rows, stream)) return false;
+        if (!launch_convert_x(t, x, ldx, gather ? row_map : nullptr, rows, K, ws + x_off, stream, nullptr, 0.f, layout)) return false;
+        GemmTiles tiles{t_expert, t_row0, t_rows, spec.count * per, L.bm, (int64_t)(row_size(t, K) * (size_t)out_features)};
+        tiles.expert_off = offs;
+        if (!launch_gemm(t, reinterpret_cast<const void*>(base), tiles.expert_stride, ws + x_off, c, ldc, nullptr, rows, out_features, K, &tiles,
+                         stream, false, L.chunk_bytes ? ws + L.chunk_off : nullptr, L.chunk_bytes, layout))
+            return false;
+    }
+    return true;
 }
 
 // problems of one block type, at most gemv_max_group() per launch
@@ -642,6 +748,32 @@ bool run_expert_set_device(const TSHipTensorView2D& out, const float* base, int6
                 }
                 if (!launch_gemv_batches(t, list, stream)) return false;
             }
+    } else if (L.tiled) {
+        // several rows, block formats: gate, up and down are one tile-table GEMM each (per block type) over the experts'
+        // pointers; the M input rows are gathered once per expert into the [n M x H] activations
+        for (int e = 0; e < n; ++e)
+            if (!check_device_operands(x, ex[e].up, ex[e].up_type) || !check_device_operands(x, ex[e].down, ex[e].down_type) ||
+                (ex[e].gate && !check_device_operands(x, ex[e].gate, ex[e].gate_type)))
+                return false;
+        const bool gated = ex[0].gate != nullptr;
+        const int ld = gated ? 2 * I : I;
+        const float* xv = static_cast<const float*>(x.data);
+        ExpertLinear lin{};
+        if (gated) {
+            for (int e = 0; e < n; ++e) lin.w[e] = ex[e].gate, lin.type[e] = ex[e].gate_type;
+            if (!run_expert_linear_tiled(L, ws, n, M, lin, xv, x.stride0, true, L.x1_off, act, ld, I, H, stream)) return false;
+        }
+        for (int e = 0; e < n; ++e) lin.w[e] = ex[e].up, lin.type[e] = ex[e].up_type;
+        if (!run_expert_linear_tiled(L, ws, n, M, lin, xv, x.stride0, true, L.x1_off, gated ? act + I : act, ld, I, H, stream)) return false;
+        const float* rows_in = act;
+        if (gated) {
+            if (!launch_silu_mul(act, ld, n * M, I, tmp, stream)) return false;
+            rows_in = tmp;
+        } else if (!launch_relu_sqr(act, (int64_t)n * M * I, stream)) {
+            return false;
+        }
+        for (int e = 0; e < n; ++e) lin.w[e] = ex[e].down, lin.type[e] = ex[e].down_type;
+        if (!run_expert_linear_tiled(L, ws, n, M, lin, rows_in, I, false, L.x2_off, dn, N, N, I, stream)) return false;
     } else {
         for (int e = 0; e < n; ++e) {
             float* a_e = act + (size_t)e * L.act_stride;

@@ -165,6 +165,25 @@ bool launch_rms_norm_rows(const float* x, int64_t ldx, const float* w, float eps
     return hip_ok(hipGetLastError(), "rms_norm launch");
 }
 
+// Tables of a tile-table GEMM launch over experts held by pointer (every expert sees the same M rows): m-tiles of bm rows
+// per expert, the experts' byte offsets from the launch's base pointer, and the row map that repeats the M source rows
+// once per member of the set.
+__global__ void __launch_bounds__(256) expert_tiles_kernel(ExpertTileSpec s, int M, int bm, int* tile_expert, int* tile_row0, int* tile_rows,
+                                                          int64_t* off_table, int* row_map, int map_rows)
+{
+    const int per = (M + bm - 1) / bm;
+    const int i0 = blockIdx.x * 256 + threadIdx.x, step = gridDim.x * 256;
+    for (int i = i0; i < s.count * per; i += step) {
+        const int e = i / per, j = i - e * per;
+        tile_expert[i] = e;
+        tile_row0[i] = s.slot[e] * M + j * bm;
+        tile_rows[i] = min(bm, M - j * bm);
+    }
+    for (int i = i0; i < s.count; i += step) off_table[i] = s.off[i];
+    if (row_map)
+        for (int i = i0; i < map_rows; i += step) row_map[i] = i % M;
+}
+
 bool launch_silu_mul(const float* gu, int64_t ldgu, int M, int half, float* out, hipStream_t stream)
 {
     if (M <= 0 || half <= 0) return true;
@@ -181,6 +200,19 @@ bool launch_relu_sqr(float* x, int64_t n, hipStream_t stream)
     if (n <= 0) return true;
     hipLaunchKernelGGL(relu_sqr_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, n);
     return hip_ok(hipGetLastError(), "relu_sqr launch");
+}
+
+bool launch_expert_tiles(const ExpertTileSpec& spec, int M, int bm, int* tile_expert, int* tile_row0, int* tile_rows, int64_t* off_table,
+                         int* row_map, int map_rows, hipStream_t stream)
+{
+    if (spec.count < 1 || spec.count > kMaxWeightedRows || M < 1 || bm < 1) {
+        set_last_error("expert_tiles: bad expert count or tile height.");
+        return false;
+    }
+    const int items = std::max(spec.count * ((M + bm - 1) / bm), row_map ? map_rows : 0);
+    hipLaunchKernelGGL(expert_tiles_kernel, dim3((unsigned)std::min(64, (items + 255) / 256)), dim3(256), 0, stream, spec, M, bm, tile_expert,
+                       tile_row0, tile_rows, off_table, row_map, map_rows);
+    return hip_ok(hipGetLastError(), "expert_tiles launch");
 }
 
 bool launch_weighted_sum(const float* rows, int64_t set_stride, const WeightedSumCoeffs& w, int count, int M, int N, const float* base,

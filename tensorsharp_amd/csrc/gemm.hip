@@ -809,6 +809,7 @@ struct GemmArgs {
     const int* tile_row0;    // [m_tiles] first activation row
     const int* tile_rows;    // [m_tiles] rows in the tile (<= BM)
     int64_t expert_stride;   // bytes between experts
+    const int64_t* expert_off;  // optional [experts]: byte offset of each expert from w instead (experts held by pointer)
     int accumulate;          // c += ... instead of c = ...
     // register-resident kernel with K cut into chunks: chunk kc of a row tile writes its sums (already scaled) to
     // partial[kc][activation row][column]; a second kernel adds the chunks in order into c
@@ -822,6 +823,13 @@ struct GemmArgs {
     uint8_t* epi_out;        // activation rows of the down projection (layout of convert_x_mx_kernel)
     int64_t epi_ld;          // bytes between them
 };
+
+// where the weights of m-tile mt's expert start, relative to A.w
+__device__ __forceinline__ int64_t expert_offset(const GemmArgs& A, int mt)
+{
+    const int e = A.tile_expert[mt];
+    return A.expert_off ? A.expert_off[e] : (int64_t)e * A.expert_stride;
+}
 
 constexpr int kXRow = kBK * 2;               // bytes of one activation row of a k-tile in LDS (no padding, swizzled)
 
@@ -1000,7 +1008,7 @@ __global__ void __launch_bounds__(NW * 64) gemm_kernel(const GemmArgs A)
         m0 = A.tile_row0[mt];
         m_rows = A.tile_rows[mt];
         if (m_rows <= 0) return;          // table entries past the last tile
-        wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+        wbase += expert_offset(A, mt);
     } else {
         m0 = mt * BM;
         m_rows = min(BM, A.M - m0);
@@ -1338,7 +1346,7 @@ __global__ void __launch_bounds__(128 * WN) gemm_xw_kernel(const GemmArgs A)
         m0 = A.tile_row0[mt];
         m_rows = A.tile_rows[mt];
         if (m_rows <= 0) return;
-        wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+        wbase += expert_offset(A, mt);
     } else {
         m0 = mt * BM;
         m_rows = min(BM, A.M - m0);
@@ -2133,7 +2141,7 @@ __global__ void __launch_bounds__(512) gemm_slim_kernel(const GemmArgs A)
         if (A.tile_expert) {
             m0 = A.tile_row0[mt];
             m_rows = min(32, A.tile_rows[mt]);
-            wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+            wbase += expert_offset(A, mt);
         } else {
             m0 = mt * 32;
             m_rows = min(32, A.M - m0);
@@ -2424,7 +2432,7 @@ __global__ void __launch_bounds__(512) gemm_slim_mx_kernel(const GemmArgs A)
         if (A.tile_expert) {
             m0 = A.tile_row0[mt];
             m_rows = min(32 * RB, A.tile_rows[mt]);
-            wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+            wbase += expert_offset(A, mt);
         } else {
             m0 = mt * 32 * RB;
             m_rows = min(32 * RB, A.M - m0);
@@ -2784,7 +2792,7 @@ __global__ void __launch_bounds__(512) gemm_slim_mx48_kernel(const GemmArgs A)
         if (A.tile_expert) {
             m0 = A.tile_row0[mt];
             m_rows = min(48, A.tile_rows[mt]);
-            wbase += (int64_t)A.tile_expert[mt] * A.expert_stride;
+            wbase += expert_offset(A, mt);
         } else {
             m0 = mt * 48;
             m_rows = min(48, A.M - m0);
@@ -3321,6 +3329,7 @@ bool gemm_dispatch(int type, const void* w, int64_t w_bytes, const void* workspa
         a.tile_row0 = tiles->row0;
         a.tile_rows = tiles->rows;
         a.expert_stride = tiles->expert_stride;
+        a.expert_off = tiles->expert_off;
         bm = tiles->bm;
         m_tiles = tiles->count;
     } else {
@@ -3391,6 +3400,7 @@ bool launch_gemm_swiglu_mx(const void* w, const void* workspace, void* workspace
     a.tile_row0 = tiles->row0;
     a.tile_rows = tiles->rows;
     a.expert_stride = tiles->expert_stride;
+    a.expert_off = tiles->expert_off;
     if (tiles->count == 0) return true;
     const ChunkScratch cs{nullptr, 0, nullptr};
     if (tiles->bm == 48) {

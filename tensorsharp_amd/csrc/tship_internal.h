@@ -162,7 +162,7 @@ bool launch_convert_x_swiglu(int type, const float* gate_up, const float* bias, 
                              int M, int F, void* workspace, hipStream_t stream, int layout = 0);
 
 // Grouped launches (MoE): m-tiles enumerated by device tables; weights of expert e start at
-// w + e * expert_stride and span w_bytes each.
+// w + e * expert_stride (or, for experts held by pointer, at w + expert_off[e]) and span expert_stride bytes each.
 struct GemmTiles {
     const int* expert;
     const int* row0;
@@ -170,6 +170,7 @@ struct GemmTiles {
     int count;
     int bm;
     int64_t expert_stride;
+    const int64_t* expert_off = nullptr;   // device table, optional
 };
 
 // The gate_up GEMM of MXFP4 gpt-oss experts on 32-row tiles with the down projection's activations as its result:
@@ -209,6 +210,16 @@ struct WeightedSumCoeffs {
 };
 bool launch_weighted_sum(const float* rows, int64_t set_stride, const WeightedSumCoeffs& w, int count, int M, int N, const float* base,
                          int64_t ldb, float* out, int64_t ldo, hipStream_t stream);
+// Tables of a tile-table GEMM launch (GemmTiles with expert_off) over experts held by pointer, all on the same M rows:
+// member e of the launch has its weight at base + off[e] and its activation / result rows at slot[e] * M; row_map
+// (optional, map_rows entries) becomes i -> i % M, the gather that repeats the M source rows per member of the set.
+struct ExpertTileSpec {
+    int64_t off[kMaxWeightedRows];
+    int slot[kMaxWeightedRows];
+    int count;
+};
+bool launch_expert_tiles(const ExpertTileSpec& spec, int M, int bm, int* tile_expert, int* tile_row0, int* tile_rows, int64_t* off_table,
+                         int* row_map, int map_rows, hipStream_t stream);
 // y[m][n] (+)= sum_k W[n][k] x[m][k] for a dense row-major weight of type F32, F16 or BF16
 bool launch_dense_matmul(int type, const void* w, const float* x, int64_t ldx, float* y, int64_t ldy, int M, int N, int K,
                          bool accumulate, hipStream_t stream);

@@ -205,6 +205,31 @@ def test_experts_swiglu_single_row_other_gemv_formats(hip, oracle, name, n):
     assert np.all(np.abs(got - ref) <= tol), (name, n, float(np.max(np.abs(got - ref) / tol)))
 
 
+@pytest.mark.parametrize("up,down,n,M", [("q4_k", "q4_k", 3, 40), ("mxfp4", "mxfp4", 5, 33), ("q8_0", "q8_0", 2, 170),
+                                         ("q4_k", "q8_0", 2, 200), ("q8_0", "mxfp4", 6, 7), ("q5_1", "q6_k", 4, 36)])
+@pytest.mark.parametrize("gated", [True, False])
+def test_expert_sets_of_many_rows_run_as_tile_table_launches(hip, oracle, up, down, n, M, gated):
+    """More than one row with block-format weights: every linear of the set is one tile-table GEMM over the experts'
+    pointers (32-row tiles up to 160 rows, then 128-row tiles; M = 40 / 170 / 200 need two tiles per expert, the last one
+    partial).  A shared expert of another type in the same set (two launches for that linear) is covered by
+    test_experts_swiglu_residual_with_shared_expert."""
+    rng = np.random.default_rng(360 + n + M)
+    H, I = 512, 256
+    mk = lambda nm, N, K: make(oracle, nm, N, K, rng) if nm in T_ else make_blocks(nm, N, K, rng)
+    ex = [dict(gate=mk(up, I, H) if gated else None, up=mk(up, I, H), down=mk(down, H, I)) for e in range(n)]
+    w = rng.uniform(0.05, 0.6, n).astype(np.float32)
+    x = rng.standard_normal((M, H)).astype(np.float32)
+    ref, parts = oracle.expert_set(x, ex, w)
+    if gated:
+        fn = lambda r, i: hip.MoEExpertsSwiGLUForward(r, i, [qw(e["gate"], True) for e in ex], [qw(e["up"], True) for e in ex],
+                                                      [qw(e["down"], True) for e in ex], w)
+    else:
+        fn = lambda r, i: hip.MoEExpertsForward(r, i, [qw(e["up"], True) for e in ex], [qw(e["down"], True) for e in ex], w)
+    got = run(hip, True, fn, np.full((M, H), np.nan, np.float32), x)[0]
+    tol = set_tol(oracle, parts, w)
+    assert np.all(np.abs(got - ref) <= tol), (up, down, n, M, gated, float(np.max(np.abs(got - ref) / tol)))
+
+
 @pytest.mark.parametrize("shared", [None, "same", "wider", "other_type"])
 @pytest.mark.parametrize("n,M", [(8, 1), (32, 1), (4, 3)])
 @pytest.mark.parametrize("device", [False, True])
