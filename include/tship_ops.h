@@ -244,7 +244,8 @@ TSHIP_EXPORT int TSHip_FusedOutProjNormRouterQuantF32Device(TSHipTensorView2D re
  * Nemotron experts): result = sum_e route_weights[e] * W_down[e] * max(W_up[e] * input, 0)^2 over the num_experts
  * (1..16) selected experts, added in index order.  The pointer arrays and route_weights are host arrays; each expert's
  * blocks are cached on the device under their host address like any weight.  One token runs as grouped GEMV
- * launches; more rows run expert by expert through the matmul path. */
+ * launches; more rows of block-format experts run every linear as one tile-table GEMM over the experts' pointers (dense
+ * or Q8_1 experts: expert by expert through the matmul path). */
 TSHIP_EXPORT int TSHip_MoEExpertsForwardF32(TSHipTensorView2D result, TSHipTensorView2D input, int num_experts,
                                             void** up_data_ptrs, void** down_data_ptrs, int up_ggml_type, int64_t up_ne0,
                                             int64_t up_ne1, int64_t up_raw_bytes_each, int down_ggml_type, int64_t down_ne0,
