@@ -572,8 +572,12 @@ bool has_tile_gemm(int type)
     }
 }
 
-// activation layout of a tile-table launch over expert pointers: MXFP4 on 32-row units reads MX fp6 pairs
-int expert_tiles_x_layout(int type, int bm, int K) { return type == kTypeMXFP4 && bm == 32 && K <= 32768 ? 1 : 0; }
+// activation layout of a tile-table launch over expert pointers: MXFP4 on 32-row units reads MX fp6 pairs (rows of at least
+// 256 outputs: the error of fp6 pairs against a short row's norm is too close to the 1e-3 bound)
+int expert_tiles_x_layout(int type, int bm, int K, int out_features)
+{
+    return type == kTypeMXFP4 && bm == 32 && K <= 32768 && out_features >= 256 ? 1 : 0;
+}
 
 ExpertSetLayout expert_set_layout(int M, int n, const ExpertFfn* ex, int H, int I, int N)
 {
@@ -621,7 +625,7 @@ ExpertSetLayout expert_set_layout(int M, int n, const ExpertFfn* ex, int H, int 
     const GemmTiles plan_tiles{nullptr, nullptr, nullptr, max_tiles, L.bm, 0};
     for (int e = 0; e < n; ++e) {
         auto need = [&](int type, int nn, int kk) {
-            return gemm_chunk_ws_bytes(type, (int)rows, nn, kk, &plan_tiles, false, expert_tiles_x_layout(type, L.bm, kk));
+            return gemm_chunk_ws_bytes(type, (int)rows, nn, kk, &plan_tiles, false, expert_tiles_x_layout(type, L.bm, kk, nn));
         };
         if (ex[e].gate) L.chunk_bytes = std::max(L.chunk_bytes, need(ex[e].gate_type, I, H));
         L.chunk_bytes = std::max(L.chunk_bytes, need(ex[e].up_type, I, H));
@@ -668,7 +672,7 @@ bool run_expert_linear_tiled(const ExpertSetLayout& L, char* ws, int n, int M, c
             spec.slot[spec.count] = e;
             ++spec.count;
         }
-        const int layout = expert_tiles_x_layout(t, L.bm, K);
+        const int layout = expert_tiles_x_layout(t, L.bm, K, out_features);
         if (!launch_expert_tiles(spec, M, L.bm, t_expert, t_row0, t_rows, offs, gather ? row_map : nullptr, rows, stream)) return false;
         if (!launch_convert_x(t, x, ldx, gather ? row_map : nullptr, rows, K, ws + x_off, stream, nullptr, 0.f, layout)) return false;
         GemmTiles tiles{t_expert, t_row0, t_rows, spec.count * per, L.bm, (int64_t)(row_size(t, K) * (size_t)out_features)};
@@ -1547,7 +1551,10 @@ int TSHip_MoEExpertsGptOssForwardF32Device(TSHipTensorView2D result, TSHipTensor
         // on both matmuls in 48-row units of the register-resident kernel once an expert's tokens often pass 32 (nearly
         // every expert of a 256-token batch then streams its weights once; measured faster than the 128-row tiles up to
         // 2048 tokens per expert: 16384 tokens 4.17 vs 4.96 ms), else in its 32-row units up to 160 tokens per expert
-        const bool mx_type = ggml_type == kTypeMXFP4 && H <= 32768 && F <= 32768;
+        // MX fp6 pairs leave each activation with an error of up to 2^-10 of its BLOCK's largest magnitude (fp16: 2^-11 of
+        // the value itself).  Against the norm of a result row that is a few 1e-5 for rows of thousands of outputs but
+        // approaches 1e-3 for rows of 32: narrow stages stay on fp16 operands.
+        const bool mx_type = ggml_type == kTypeMXFP4 && H <= 32768 && F <= 32768 && H >= 256 && F >= 128;
         const bool rows48 = mx_type && per_expert > 20 && H <= 3072 && F <= 3072;
         const bool mx = mx_type && (rows48 || per_expert <= 160);
         const int x_layout = mx ? 1 : 0;

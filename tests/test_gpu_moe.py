@@ -146,6 +146,22 @@ def test_gate_up_epilogue_writes_down_activations(hip, oracle, E, H, F, T, k):
     assert inputs.row_l2_err(got2, ref2) <= 1e-3, inputs.row_l2_err(got2, ref2)
 
 
+@pytest.mark.parametrize("H,F", [(32, 672), (64, 96), (224, 64)])
+def test_narrow_mxfp4_stages_stay_on_fp16_operands(hip, oracle, H, F):
+    """Rows of a few dozen outputs: the MX fp6 pairs of the block-scaled path leave every activation with an error of up to
+    2^-10 of its block's largest magnitude, which against the norm of a 32-wide result row comes to 1e-3 (a sweep case
+    measured 1.24e-3 at H = 32); stages narrower than 256 (H) / 128 (F) therefore run on fp16 operands.  Same bar as every
+    matmul: row-L2 <= 1e-3."""
+    rng = np.random.default_rng(2000 + H)
+    E, T, k = 4, 200, 2
+    gu, _, dn, _ = make_experts(oracle, MXFP4, E, H, F, rng)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    ref = oracle.moe_forward(MXFP4, gu, None, dn, None, E, H, F, hidden, ids, wts)
+    got = run_gpu(hip, MXFP4, gu, None, dn, None, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got, ref) <= 5e-4, inputs.row_l2_err(got, ref)
+
+
 @pytest.fixture(scope="module")
 def cfg4_weights(oracle):
     E, H, F = 32, 2880, 2880
