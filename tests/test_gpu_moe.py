@@ -159,7 +159,7 @@ def test_narrow_mxfp4_stages_stay_on_fp16_operands(hip, oracle, H, F):
     ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
     ref = oracle.moe_forward(MXFP4, gu, None, dn, None, E, H, F, hidden, ids, wts)
     got = run_gpu(hip, MXFP4, gu, None, dn, None, E, H, F, hidden, ids, wts)
-    assert inputs.row_l2_err(got, ref) <= 5e-4, inputs.row_l2_err(got, ref)
+    assert inputs.row_l2_err(got, ref) <= 1e-3, inputs.row_l2_err(got, ref)
 
 
 @pytest.fixture(scope="module")
