@@ -844,6 +844,30 @@ __device__ __forceinline__ float row_sum(float v)
     return t;
 }
 
+// Sum of a double over the 64 lanes of a wavefront (every lane gets it): the permutations of row_sum on both halves of
+// the value (register moves; a shuffle would make twelve trips through the LDS crossbar).
+__device__ __forceinline__ double wave_sum_f64(double v)
+{
+    typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+    auto moved = [](double d, auto perm) { return __hiloint2double(perm(__double2hiint(d)), perm(__double2loint(d))); };
+    double t = v;
+    t += moved(t, [](int x) { return __builtin_amdgcn_update_dpp(0, x, kDppXor1, 0xf, 0xf, true); });
+    t += moved(t, [](int x) { return __builtin_amdgcn_update_dpp(0, x, kDppXor2, 0xf, 0xf, true); });
+    t += moved(t, [](int x) { return __builtin_amdgcn_update_dpp(0, x, kDppHalfMirror, 0xf, 0xf, true); });
+    t += moved(t, [](int x) { return __builtin_amdgcn_update_dpp(0, x, kDppMirror, 0xf, 0xf, true); });
+    {
+        const u2_t hi = __builtin_amdgcn_permlane16_swap((uint32_t)__double2hiint(t), (uint32_t)__double2hiint(t), false, false);
+        const u2_t lo = __builtin_amdgcn_permlane16_swap((uint32_t)__double2loint(t), (uint32_t)__double2loint(t), false, false);
+        t = __hiloint2double((int)hi.x, (int)lo.x) + __hiloint2double((int)hi.y, (int)lo.y);
+    }
+    {
+        const u2_t hi = __builtin_amdgcn_permlane32_swap((uint32_t)__double2hiint(t), (uint32_t)__double2hiint(t), false, false);
+        const u2_t lo = __builtin_amdgcn_permlane32_swap((uint32_t)__double2loint(t), (uint32_t)__double2loint(t), false, false);
+        t = __hiloint2double((int)hi.x, (int)lo.x) + __hiloint2double((int)hi.y, (int)lo.y);
+    }
+    return t;
+}
+
 // A wavefront works on a group of 64 / LPR consecutive rows at a time, one row per LPR lanes (LPR = 16 unless the
 // format says otherwise).
 // One step = LPR consecutive units of each row of the group.  Steps of a wavefront are numbered group-major over
@@ -992,18 +1016,23 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // and the staging.  (Sum of squares in double over fp32 squares, as ggml_rms_norm.)
     const int lds_units = (routed ? (RPG - 1) * upr : 0) + nsteps * LPR;               // unit slots the lanes may read
     double* red = reinterpret_cast<double*>(lds + lds_units * F::kLdsDwords);         // [kWaves], after the x area
-    double ss = 0.0;
-    auto apply_act = [&]() {
+    // four partial sums per thread, so that the double additions of a pass do not form one dependent chain
+    double ss4[4] = {0.0, 0.0, 0.0, 0.0};
+    auto apply_act = [&](int base) {
         if (act == kActRmsNorm) {
 #pragma unroll
-            for (int c = 0; c < kStageChunk; ++c)
+            for (int c = 0; c < kStageChunk; ++c) {
+                if (base + c * kThreads >= items) continue;      // uniform: nothing was loaded for this chunk
 #pragma unroll
                 for (int q = 0; q < F::kStageF4; ++q) {
-                    ss += (double)(xv[c][q].x * xv[c][q].x) + (double)(xv[c][q].y * xv[c][q].y) +
-                          (double)(xv[c][q].z * xv[c][q].z) + (double)(xv[c][q].w * xv[c][q].w);
+                    ss4[0] += (double)(xv[c][q].x * xv[c][q].x);
+                    ss4[1] += (double)(xv[c][q].y * xv[c][q].y);
+                    ss4[2] += (double)(xv[c][q].z * xv[c][q].z);
+                    ss4[3] += (double)(xv[c][q].w * xv[c][q].w);
                     xv[c][q] = float4{xv[c][q].x * x2[c][q].x, xv[c][q].y * x2[c][q].y, xv[c][q].z * x2[c][q].z,
                                       xv[c][q].w * x2[c][q].w};
                 }
+            }
         } else if (act == kActSiluMul) {
             // hardware exp2 / reciprocal: relative error below 1e-5, far under the fp16 rounding the staged value gets
             // next (every workgroup evaluates the whole row, so the exact expf and division cost microseconds)
@@ -1017,7 +1046,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         }
     };
     auto stage_commit = [&](int base) {
-        if (act != kActPlain) apply_act();
+        if (act != kActPlain) apply_act(base);
 #pragma unroll
         for (int c = 0; c < kStageChunk; ++c) {
             if (base + c * kThreads < items) {   // uniform
@@ -1065,7 +1094,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     // lanes past the end of a row read their activations from the zero-filled tail of the last step
     for (int i = (kx / F::kUnitElems) * F::kLdsDwords + (int)threadIdx.x; i < lds_units * F::kLdsDwords; i += kThreads) lds[i] = 0u;
     if (act == kActRmsNorm) {
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        const double ss = wave_sum_f64((ss4[0] + ss4[1]) + (ss4[2] + ss4[3]));
         if (lane == 0) red[threadIdx.x >> 6] = ss;
     }
     __syncthreads();
