@@ -169,38 +169,43 @@ struct FmtQ4K {
     // work item `it` = activations [4*it, 4*it+4): byte offset of its float4
     static __device__ __forceinline__ void stage_offsets(int it, uint32_t (&off)[kStageF4]) { off[0] = (uint32_t)it * 16u; }
 
-    // one work item = one float4; the 16 lanes of a DPP row share a unit
+    // one work item = one float4; the 16 lanes of a DPP row share a unit.  Every workgroup converts the whole vector, so
+    // the instruction count of this routine is launch time (K = 14336: 7 items per thread, 16 wavefronts per CU): the
+    // largest magnitude is an integer maximum of the bit patterns (one DPP instruction per level, NaN / inf on top), the
+    // sub-block sums come from two dot products with (1, 1).
     static __device__ __forceinline__ void stage_store(const float4 (&vv)[kStageF4], int it, bool live, uint32_t* lds)
     {
         const float4 v = vv[0];
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor1));
-        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppXor2));
-        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppHalfMirror));
-        amax = fmaxf(amax, TSHIP_DPP_F(amax, kDppMirror));
+        constexpr uint32_t kAbs = 0x7fffffffu;
+        uint32_t m = max(max(__float_as_uint(v.x) & kAbs, __float_as_uint(v.y) & kAbs),
+                         max(__float_as_uint(v.z) & kAbs, __float_as_uint(v.w) & kAbs));
+        m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, kDppXor1, 0xf, 0xf, true));
+        m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, kDppXor2, 0xf, 0xf, true));
+        m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, kDppHalfMirror, 0xf, 0xf, true));
+        m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, kDppMirror, 0xf, 0xf, true));
         float inv, scale;
-        pow2_scale(amax, &inv, &scale);
+        pow2_scale(__uint_as_float(m), &inv, &scale);
         const _Float16 h0 = (_Float16)(v.x * inv), h1 = (_Float16)(v.y * inv);
         const _Float16 h2 = (_Float16)(v.z * inv), h3 = (_Float16)(v.w * inv);
-        float s = ((float)h0 + (float)h1) + ((float)h2 + (float)h3);
+        H2U a, b;
+        a.h = half2_t{h0, h2};
+        b.h = half2_t{h1, h3};
+        // sum of the four fp16 values in fp32
+        float s = dot2(b.u, 0x3c003c00u, dot2(a.u, 0x3c003c00u, 0.f));
         // sum over the 8 lanes of one 32-weight sub-block
         s += TSHIP_DPP_F(s, kDppXor1);
         s += TSHIP_DPP_F(s, kDppXor2);
         s += TSHIP_DPP_F(s, kDppHalfMirror);
         if (live) {
-            const int e = it << 2;
-            const int g = e >> 6, r = e & 63;
-            const int sub = r >> 5, j = (r & 31) >> 2;
+            // item it = floats [4 it, 4 it + 4): unit it / 16, sub-block (it / 8) % 2, quant dword it % 8
+            const int g = it >> 4, sub = (it >> 3) & 1, j = it & 7;
             uint32_t* unit = lds + g * kLdsDwords;
-            H2U a, b;
-            a.h = half2_t{h0, h2};
-            b.h = half2_t{h1, h3};
             uint2 w2;
             w2.x = a.u;
             w2.y = b.u;
             *reinterpret_cast<uint2*>(unit + 4 * j + 2 * sub) = w2;
-            if ((threadIdx.x & 7) == 0) reinterpret_cast<float*>(unit)[32 + sub] = s;
-            if ((threadIdx.x & 15) == 0) reinterpret_cast<float*>(unit)[34] = scale;
+            if ((it & 7) == 0) reinterpret_cast<float*>(unit)[32 + sub] = s;
+            if ((it & 15) == 0) reinterpret_cast<float*>(unit)[34] = scale;
         }
     }
     static __device__ __forceinline__ int stage_items(int K) { return K >> 2; }
@@ -1202,7 +1207,7 @@ struct GemvProblems {
     GemvProblem p[kMaxGroup];
 };
 template <int TYPE, int ACT, bool TL, int EAGER>
-__global__ void __launch_bounds__(kThreads) gemv_kernel(int b0, int b1, int b2, int b3, int b4, int b5, int b6, int b7, int b8, int count,
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) gemv_kernel(int b0, int b1, int b2, int b3, int b4, int b5, int b6, int b7, int b8, int count,
                                                         int strict, const GemvProblems G, uint64_t* tl)
 {
     static_assert(kMaxGroup == 8, "one scalar argument per table entry");
