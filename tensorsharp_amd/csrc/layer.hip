@@ -31,10 +31,25 @@ __device__ __forceinline__ float wave_sum(float v)
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     return v;
 }
+// (register permutations on both halves of the value; a shuffle of a double is two trips through the LDS crossbar)
 __device__ __forceinline__ double wave_sum(double v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+    auto moved = [](double d, auto perm) { return __hiloint2double(perm(__double2hiint(d)), perm(__double2loint(d))); };
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0xb1, 0xf, 0xf, true); });
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0x4e, 0xf, 0xf, true); });
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, true); });
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0x140, 0xf, 0xf, true); });
+    {
+        const u2_t hi = __builtin_amdgcn_permlane16_swap((uint32_t)__double2hiint(v), (uint32_t)__double2hiint(v), false, false);
+        const u2_t lo = __builtin_amdgcn_permlane16_swap((uint32_t)__double2loint(v), (uint32_t)__double2loint(v), false, false);
+        v = __hiloint2double((int)hi.x, (int)lo.x) + __hiloint2double((int)hi.y, (int)lo.y);
+    }
+    {
+        const u2_t hi = __builtin_amdgcn_permlane32_swap((uint32_t)__double2hiint(v), (uint32_t)__double2hiint(v), false, false);
+        const u2_t lo = __builtin_amdgcn_permlane32_swap((uint32_t)__double2loint(v), (uint32_t)__double2loint(v), false, false);
+        v = __hiloint2double((int)hi.x, (int)lo.x) + __hiloint2double((int)hi.y, (int)lo.y);
+    }
     return v;
 }
 
@@ -62,6 +77,18 @@ __device__ __forceinline__ void softmax_merge(float& m, float& l, float (&acc)[N
 #pragma unroll
     for (int j = 0; j < N; ++j) acc[j] = acc[j] * f1 + acc2[j] * f2;
     m = mm;
+}
+
+// Sum over the 16 lanes of a group, every lane gets it: four register permutations (pairs inside a quad, quads, mirrored
+// eights, mirrored sixteen) instead of four trips through the LDS crossbar.
+__device__ __forceinline__ float sum16(float v)
+{
+    auto moved = [](float x, auto perm) { return __int_as_float(perm(__float_as_int(x))); };
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0xb1, 0xf, 0xf, true); });     // quad_perm [1,0,3,2]
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0x4e, 0xf, 0xf, true); });     // quad_perm [2,3,0,1]
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, true); });    // lane i <-> 7 - i of each 8
+    v += moved(v, [](int x) { return __builtin_amdgcn_update_dpp(0, x, 0x140, 0xf, 0xf, true); });    // lane i <-> 15 - i of each 16
+    return v;
 }
 
 // grid (num_kv_heads, splits, q-head chunks): one workgroup serves G query heads that share a KV head, so every K / V
@@ -109,27 +136,45 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
     {
         constexpr int kPer = (HD + 63) / 64, kPairs = (HD / 2 + 63) / 64;
         constexpr int half = HD / 2;
-        float cs[kPairs], sn[kPairs];
-#pragma unroll
-        for (int j = 0; j < kPairs; ++j) {
-            const int p = lane + 64 * j;
-            // the reference builds theta by repeated multiplication; the same float products in the same order
-            float theta = (float)position;
-            for (int i = 0; i < p && p < half; ++i) theta *= F.theta_scale;
-            const float ang = F.freq_scale * theta;
-            cs[j] = cosf(ang);
-            sn[j] = sinf(ang);
-        }
         const int nprep = G + (last ? 1 : 0);
+        auto head_src = [&](int hh) { return F.qkv + (int64_t)(hh < G ? h0 + hh : F.num_heads + kvh) * HD; };
+        // the wavefront's first head is requested before the angles are worked out
+        float xv[kPer];
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+            const int d = lane + 64 * j;
+            xv[j] = (wave < nprep && d < HD) ? head_src(wave)[d] : 0.f;
+        }
+        float cs[kPairs], sn[kPairs];
+        {
+            // the reference builds theta by repeated multiplication; the same float products in the same order.  One
+            // uniform chain of half - 1 products, every lane keeping the value of its own pair (a loop of lane-dependent
+            // length costs several times as many instructions per product).
+            float chain = (float)position;
+#pragma unroll
+            for (int j = 0; j < kPairs; ++j) cs[j] = chain;       // pair 0
+            for (int i = 1; i < half; ++i) {
+                chain *= F.theta_scale;
+#pragma unroll
+                for (int j = 0; j < kPairs; ++j) cs[j] = (lane + 64 * j == i) ? chain : cs[j];
+            }
+#pragma unroll
+            for (int j = 0; j < kPairs; ++j) {
+                const float ang = F.freq_scale * cs[j];
+                cs[j] = cosf(ang);
+                sn[j] = sinf(ang);
+            }
+        }
         for (int hh = wave; hh < nprep; hh += kAttnWaves) {          // uniform per wavefront
             const bool is_q = hh < G;
-            const float* src = F.qkv + (int64_t)(is_q ? h0 + hh : F.num_heads + kvh) * HD;
+            const float* src = head_src(hh);
             const float* nw = is_q ? F.q_norm_w : F.k_norm_w;
-            float xv[kPer];
+            if (hh != wave) {
 #pragma unroll
-            for (int j = 0; j < kPer; ++j) {
-                const int d = lane + 64 * j;
-                xv[j] = d < HD ? src[d] : 0.f;
+                for (int j = 0; j < kPer; ++j) {
+                    const int d = lane + 64 * j;
+                    xv[j] = d < HD ? src[d] : 0.f;
+                }
             }
             float rs = 1.f;
             if (nw) {
@@ -225,9 +270,7 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
                 for (int j = 0; j < PER; ++j) d[u] += qr[g][j] * kr[u][j];
             }
 #pragma unroll
-            for (int o = 8; o > 0; o >>= 1)
-#pragma unroll
-                for (int u = 0; u < kInFlight; ++u) d[u] += __shfl_xor(d[u], o);
+            for (int u = 0; u < kInFlight; ++u) d[u] = sum16(d[u]);
             float mn = m[g];
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u) {
@@ -256,13 +299,27 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
     // the four groups of a wavefront
 #pragma unroll
     for (int g = 0; g < G; ++g) {
+        // rows 0 | 1 and 2 | 3 of the wavefront, then the two halves: a lane gets the state of the even and of the odd
+        // member of its pair (register swaps between rows) and merges them, so every lane ends with the same result
 #pragma unroll
-        for (int o = 16; o <= 32; o <<= 1) {
-            const float m2 = __shfl_xor(m[g], o), l2 = __shfl_xor(l[g], o);
-            float a2[PER];
+        for (int level = 0; level < 2; ++level) {
+            typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+            auto both = [&](float x, float& even, float& odd) {
+                const u2_t r = level == 0 ? __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false)
+                                          : __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+                even = __uint_as_float(r.x);
+                odd = __uint_as_float(r.y);
+            };
+            float m1, m2, l1, l2, a1[PER], a2[PER];
+            both(m[g], m1, m2);
+            both(l[g], l1, l2);
 #pragma unroll
-            for (int j = 0; j < PER; ++j) a2[j] = __shfl_xor(acc[g][j], o);
-            softmax_merge<PER>(m[g], l[g], acc[g], m2, l2, a2);
+            for (int j = 0; j < PER; ++j) both(acc[g][j], a1[j], a2[j]);
+            softmax_merge<PER>(m1, l1, a1, m2, l2, a2);
+            m[g] = m1;
+            l[g] = l1;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) acc[g][j] = a1[j];
         }
         if (lane < 16) {
             if (lane == 0) {
