@@ -365,16 +365,8 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_combine_kernel(const flo
     __shared__ float sacc[kAttnWaves][kMaxHeadDim], sl[kAttnWaves];
     const int h = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* base = partial + (int64_t)h * splits * kRow;
-    // the maximum over all splits: every wavefront computes it (independent loads, one pass)
-    float mm = -INFINITY;
-    for (int s = lane; s < splits; s += 64) mm = fmaxf(mm, base[(int64_t)s * kRow]);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
-    float acc[kPer], ll = 0.f;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) acc[j] = 0.f;
-    for (int s0 = wave; s0 < splits; s0 += 4 * kAttnWaves) {
-        float ms[4], ls[4], v[4][kPer];
+    float ms[4], ls[4], v[4][kPer];
+    auto load_rows = [&](int s0) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int s = s0 + u * kAttnWaves;
@@ -388,6 +380,22 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_combine_kernel(const flo
                 v[u][j] = (live && d < head_dim) ? p[2 + d] : 0.f;
             }
         }
+    };
+    // When one batch of rows per wavefront covers the splits (up to 1024 positions), it is requested before the maximum
+    // over all splits is worked out (every wavefront computes it: independent loads, one pass), so that the two round
+    // trips overlap: 0.35 us per layer.  (With more batches the early request measured 0.3 us slower.)
+    constexpr int kBatch = 4 * kAttnWaves;
+    const bool early = splits <= kBatch;
+    if (early && wave < splits) load_rows(wave);
+    float mm = -INFINITY;
+    for (int s = lane; s < splits; s += 64) mm = fmaxf(mm, base[(int64_t)s * kRow]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
+    float acc[kPer], ll = 0.f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) acc[j] = 0.f;
+    for (int s0 = wave; s0 < splits; s0 += kBatch) {
+        if (!early) load_rows(s0);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const float f = ms[u] == -INFINITY ? 0.f : expf(ms[u] - mm);
