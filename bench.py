@@ -478,9 +478,13 @@ def main():
             x = torch.randn((1, k), device=dev, dtype=torch.float32)
             y = torch.empty((1, n), device=dev, dtype=torch.float32)
 
+            # arguments marshalled once per weight copy (TSHip_AddmmQuantGroupF32Device with one problem, as a decode loop
+            # would hold them): building the views of TSHip_AddmmQuantF32Device in Python on every call costs about
+            # 6.5 us, more than the shortest launches last, and would be what the events measure
+            packs = [HipBasicOps.PrepareGroup([y], [x], [w]) for w in ws]
+
             def f(i):
-                w = ws[i % copies]
-                HipBasicOps.AddmmQuantDevice(y, x, w.ptr, t, k, n, w.raw_bytes)
+                HipBasicOps.AddmmQuantGroupDevice(packs[i % copies])
             for i in range(50):
                 f(i)
             ev, wall = time_region(f, n_it, torch)
