@@ -559,6 +559,41 @@ def main():
 
         extra["cfg2_q4_k_layer_decode_ctx512"] = layer_decode(512, 200)
         extra["cfg2_q4_k_layer_decode_ctx4096"] = layer_decode(4096, 200)
+        # One decode step of a whole model of these layers (llama-3-8B shapes: 32 layers, 128256-entry vocabulary): the
+        # 32 layer calls as one TSHip_TransformerModelDecodeDevice call, then the final RMSNorm + LM head (Q6_K, as Q4_K_M
+        # files store it) as one TSHip_FusedRmsNormMatMulQuantF32Device call.  32 distinct layers (3.9 GB of weights).
+        # Embedding lookup and sampling are not included.
+        def model_decode(context, n_layers=32, iters=30):
+            hidden, heads, kvh, hd, inter, max_seq, vocab = 4096, 32, 8, 128, 14336, 1024, 128256
+            q_dim, k_dim = heads * hd, kvh * hd
+            mk = lambda t, n, k, sd: QuantizedWeight(synth.random_weight(t, n, k, dev, seed=sd), t, k, n)
+            layers = []
+            for c in range(n_layers):
+                layers.append({"qkv": mk(Q4_K, q_dim + 2 * k_dim, hidden, 5000 + 10 * c), "o": mk(Q4_K, hidden, q_dim, 5001 + 10 * c),
+                               "gate_up": mk(Q4_K, 2 * inter, hidden, 5002 + 10 * c), "down": mk(Q4_K, hidden, inter, 5003 + 10 * c),
+                               "attn_norm": torch.ones(hidden, device=dev), "ffn_norm": torch.ones(hidden, device=dev),
+                               "q_norm": None, "k_norm": None,
+                               "k_cache": torch.randn((kvh, max_seq, hd), device=dev), "v_cache": torch.randn((kvh, max_seq, hd), device=dev)})
+            head = mk(Q6_K, vocab, hidden, 5999)
+            out_norm = torch.ones(hidden, device=dev)
+            logits = torch.empty((1, vocab), device=dev)
+            h = torch.randn(hidden, device=dev)
+
+            def f(i):
+                HipBasicOps.TransformerModelDecode(h, layers, heads, kvh, hd, context - 1, 1e-6, 500000.0, 1.0, 2)
+                HipBasicOps.FusedRmsNormMatMulQuant(logits, h.view(1, hidden), out_norm, 1e-6, head)
+                h.normal_()
+            for i in range(3):
+                f(i)
+            ev, wall = time_region(f, iters, torch)
+            ms = ev / iters
+            wbytes = n_layers * sum(layers[0][k].raw_bytes for k in ("qkv", "o", "gate_up", "down")) + head.raw_bytes
+            b = wbytes + n_layers * 2 * kvh * context * hd * 4
+            return {"ms_per_token_events": round(ms, 3), "tokens_per_s": round(1e3 / ms, 1), "bytes": b,
+                    "GBps": round(b / (ms * 1e-3) / 1e9, 1), "pct_hbm_peak": round(100 * b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 1),
+                    "layers": n_layers, "context": context, "launches_per_token": 6 * n_layers + 1}
+
+        extra["llama8b_shape_q4_k_model_decode_ctx512"] = model_decode(512)
         # the same seven matrices as the headline, but as the dependent chain a decode step really runs (RMSNorm + QKV,
         # attention over 512 cached tokens, Wo + residual, RMSNorm + gate | up + SiLU, down + residual: six launches):
         # every launch pays its start, its tail and the gap to the next one, which the grouped launch pays once
