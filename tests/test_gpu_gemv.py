@@ -385,3 +385,47 @@ def test_legacy_formats_element_by_element(hip, oracle, name):
         x[0, k] = 1.5
         y = run_device(hip, t, wq, N, K, x)
         assert np.allclose(y[0], 1.5 * w[:, k], rtol=2e-6, atol=1e-9), (name, k, y[0], 1.5 * w[:, k])
+
+
+@pytest.mark.parametrize("name,N,K", [("q4_k", 4096, 4096), ("q4_k", 9000, 1024), ("mxfp4", 2880, 2880), ("mxfp4", 6000, 512),
+                                      ("q8_0", 1000, 2560), ("q6_k", 700, 1024), ("q5_k", 700, 1024), ("q4_0", 900, 1024),
+                                      ("q4_1", 900, 1024), ("q5_0", 900, 1024), ("q5_1", 900, 1024), ("iq4_nl", 900, 1024)])
+def test_timeline_build_same_results_and_ordered_stamps(hip, oracle, name, N, K):
+    """TSHip_SetGemvTimeline selects a build of the kernel that stamps s_memrealtime per wavefront (the eager build for the
+    first and third case, which fit one row group per wavefront, the streaming build otherwise).  Its results are the
+    normal build's bit for bit, and every wavefront left entry <= staged <= exit (first step done in between where it had a
+    row group)."""
+    import ctypes as C
+    import torch
+    from tensorsharp_amd import QuantizedWeight, hip_native as Nat, synth
+    from oracle.oracle import MORE_TYPES, Q6_K
+    t = {"q4_k": Q4_K, "mxfp4": MXFP4, "q8_0": Q8_0, "q6_k": Q6_K}.get(name) or MORE_TYPES[name]
+    dev = torch.device("cuda:0")
+    w = synth.random_weight(t, N, K, dev, seed=91)
+    qw = QuantizedWeight(w, t, K, N)
+    x = torch.randn((1, K), device=dev, generator=torch.Generator(device=dev).manual_seed(5))
+    want = hip.LinearForward(x, qw)
+    torch.cuda.synchronize()
+    waves = 8 * 4 * 256 + 64                       # at most four workgroups of eight wavefronts per CU
+    buf = torch.zeros((waves, 8), dtype=torch.int64, device=dev)
+    Nat.check_result(Nat.lib().TSHip_SetGemvTimeline(C.c_void_p(buf.data_ptr()), waves * 64), "timeline")
+    try:
+        got = hip.LinearForward(x, qw)
+        torch.cuda.synchronize()
+    finally:
+        Nat.check_result(Nat.lib().TSHip_SetGemvTimeline(None, 0), "timeline")
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    a = buf.cpu().numpy()
+    ran = a[a[:, 4] != 0]
+    assert ran.shape[0] >= 8 and ran.shape[0] % 8 == 0, ran.shape
+    entry, staged, first, exit_ = ran[:, 0], ran[:, 2], ran[:, 3], ran[:, 4]
+    worked = first != 0                            # wavefronts without a row group never finish a step
+    assert worked.any()
+    assert np.all(entry <= staged) and np.all(staged <= exit_)
+    assert np.all(staged[worked] <= first[worked]) and np.all(first[worked] <= exit_[worked])
+    assert (exit_.max() - entry.min()) * 10 < 5_000_000        # 10 ns ticks: the launch took less than 5 ms
+    # and a later launch without the buffer leaves nothing behind
+    buf.zero_()
+    hip.LinearForward(x, qw)
+    torch.cuda.synchronize()
+    assert int(buf.abs().sum().item()) == 0
