@@ -206,7 +206,8 @@ def test_experts_swiglu_single_row_other_gemv_formats(hip, oracle, name, n):
 
 
 @pytest.mark.parametrize("up,down,n,M", [("q4_k", "q4_k", 3, 40), ("mxfp4", "mxfp4", 5, 33), ("q8_0", "q8_0", 2, 170),
-                                         ("q4_k", "q8_0", 2, 200), ("q8_0", "mxfp4", 6, 7), ("q5_1", "q6_k", 4, 36)])
+                                         ("q4_k", "q8_0", 2, 200), ("q8_0", "mxfp4", 6, 7), ("q5_1", "q6_k", 4, 36),
+                                         ("mxfp4", "mxfp4", 2, 170)])
 @pytest.mark.parametrize("gated", [True, False])
 def test_expert_sets_of_many_rows_run_as_tile_table_launches(hip, oracle, up, down, n, M, gated):
     """More than one row with block-format weights: every linear of the set is one tile-table GEMM over the experts'

@@ -209,19 +209,19 @@ def test_gate_up_fused_at_load_feeds_the_ffn(hip, oracle, adjacent):
     assert np.all(np.abs(got - (resid + mm)) <= tol)
 
 
-@pytest.mark.parametrize("gu_type", ["q4_0", "q4_1", "q5_k", "q6_k", "q8_0", "mxfp4"])
+@pytest.mark.parametrize("gu_type", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "q5_k", "q6_k", "q8_0", "mxfp4"])
 @pytest.mark.parametrize("M", [1, 2])
 def test_ffn_decode_paired_store_every_gemv_format(hip, oracle, gu_type, M):
     # decode FFN: the gate_up launch computes gate row j and up row j in one wavefront (rows F apart in the stacked
     # weight) and stores silu(gate) * up; every format with a GEMV kernel has its own row-group geometry
     # (2 rows x 32 lanes or 4 rows x 16 lanes), so each is run once, with a Q8_0 down projection
     import torch
-    from oracle.oracle import Q4_0, Q4_1, Q5_K, Q6_K
+    from oracle.oracle import Q4_0, Q4_1, Q5_K, Q6_K, MORE_TYPES
     from tensorsharp_amd import QuantizedWeight, synth
     types = {"q4_0": Q4_0, "q4_1": Q4_1, "q5_k": Q5_K, "q6_k": Q6_K, "q8_0": Q8_0, "mxfp4": MXFP4}
-    t = types[gu_type]
+    t = types.get(gu_type) or MORE_TYPES[gu_type]
     rng = np.random.default_rng(103 + M)
-    H, F = 512, 1056 if t in (Q8_0, MXFP4, Q4_0, Q4_1) else 1024      # 1056 = 33 blocks: an odd number of row groups
+    H, F = 512, 1024 if t in (Q5_K, Q6_K) else 1056      # 1056 = 33 blocks: an odd number of row groups
     dev = torch.device("cuda")
     gu_d = synth.random_weight(t, 2 * F, H, dev, seed=11, sigma=0.05)
     gu = gu_d.cpu().numpy()

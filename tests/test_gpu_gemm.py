@@ -242,6 +242,19 @@ def test_mxfp4_block_scaled_tiles(hip, oracle, M, N, K):
     check(run_device(hip, MXFP4, wq, N, K, x), oracle.matmul_f64(MXFP4, wq, N, K, x), ("mx", M, N, K))
 
 
+@pytest.mark.parametrize("M,N", [(600, 2100), (1024, 8448)])
+def test_mxfp4_rows_longer_than_the_block_scaled_kernels_take(hip, oracle, M, N):
+    # K > 32768: the activations stay fp16 and the launch runs the exchange-layout kernel (128-row tiles for the first
+    # shape, 256-row tiles for the second), K cut into chunks
+    rng = np.random.default_rng(900 + M)
+    K = 32768 + 32 * 9
+    wq = inputs.random_blocks("mxfp4", N, K, rng)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = run_device(hip, MXFP4, wq, N, K, x)
+    rows = np.unique(np.concatenate([np.arange(0, M, 149), [M - 1]]))
+    check(y[rows], oracle.matmul_f64(MXFP4, wq, N, K, x[rows]), ("mx long rows", M, N))
+
+
 def test_mxfp4_block_scaled_256_row_tiles(hip, oracle):
     # more 128-row tiles than one round of workgroups: 256-row tiles; an odd block count and a ragged last column tile
     rng = np.random.default_rng(8)

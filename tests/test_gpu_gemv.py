@@ -387,12 +387,12 @@ def test_legacy_formats_element_by_element(hip, oracle, name):
         assert np.allclose(y[0], 1.5 * w[:, k], rtol=2e-6, atol=1e-9), (name, k, y[0], 1.5 * w[:, k])
 
 
-@pytest.mark.parametrize("name,N,K", [("q4_k", 4096, 4096), ("q4_k", 9000, 1024), ("mxfp4", 2880, 2880), ("mxfp4", 6000, 512),
+@pytest.mark.parametrize("name,N,K", [("q4_k", 4096, 4096), ("q4_k", 9000, 1024), ("mxfp4", 2880, 2880), ("mxfp4", 20000, 512),
                                       ("q8_0", 1000, 2560), ("q6_k", 700, 1024), ("q5_k", 700, 1024), ("q4_0", 900, 1024),
                                       ("q4_1", 900, 1024), ("q5_0", 900, 1024), ("q5_1", 900, 1024), ("iq4_nl", 900, 1024)])
 def test_timeline_build_same_results_and_ordered_stamps(hip, oracle, name, N, K):
     """TSHip_SetGemvTimeline selects a build of the kernel that stamps s_memrealtime per wavefront (the eager build for the
-    first and third case, which fit one row group per wavefront, the streaming build otherwise).  Its results are the
+    first and third case, which fit one row group per wavefront; the streaming build otherwise).  Its results are the
     normal build's bit for bit, and every wavefront left entry <= staged <= exit (first step done in between where it had a
     row group)."""
     import ctypes as C

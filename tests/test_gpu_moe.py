@@ -66,11 +66,27 @@ def test_expert_stage_small_dims(hip, oracle, name, T, k):
 
 @pytest.mark.parametrize("name", ["mxfp4", "q4_k"])
 def test_expert_tiles_of_128_rows(hip, oracle, name):
-    # more than 160 rows per expert on average: the grouped GEMM runs 128-row tiles instead of 32-row ones
+    # more than 160 rows per expert on average: the grouped GEMM runs 128-row tiles instead of 32-row ones (MXFP4: with a
+    # hidden size past the 3072 that the 48-row block-scaled units take)
     rng = np.random.default_rng(71)
-    E, H, F, T, k = 4, 256, 256, 400, 2
+    E, H, F, T, k = 4, 3328 if name == "mxfp4" else 256, 256, 400, 2
     t = T_[name]
     gu, gb, dn, db = make_experts(oracle, t, E, H, F, rng)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    ref = oracle.moe_forward(t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    got = run_gpu(hip, t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got, ref) <= 1e-3, (name, inputs.row_l2_err(got, ref))
+
+
+@pytest.mark.parametrize("name", ["mxfp4", "q4_k", "q8_0"])
+def test_intermediate_rows_longer_than_one_conversion_pass(hip, oracle, name):
+    # F > 8192: the SwiGLU-forming conversion of the down projection's activations runs its 1024-thread form; more than
+    # 160 tokens per expert, so MXFP4 too stays on fp16 operands (128-row tiles)
+    rng = np.random.default_rng(77)
+    E, H, F, T, k = 2, 256, 8448, 330, 1
+    t = T_[name]
+    gu, gb, dn, db = make_experts(oracle, t, E, H, F, rng, sigma=0.03)
     hidden = rng.standard_normal((T, H)).astype(np.float32)
     ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
     ref = oracle.moe_forward(t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
