@@ -16,7 +16,7 @@ FLAGS = [
 ]
 # per-source additions.  gemv.hip: the first 11 dwords of kernel arguments (the workgroup -> problem table of
 # gemv_kernel) arrive preloaded in SGPRs; the code object keeps a loading prologue for firmware without the feature.
-EXTRA_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=11"]}
+EXTRA_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
 
 
 def build(verbose=False, jobs=8):

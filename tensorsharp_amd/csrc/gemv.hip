@@ -1203,10 +1203,22 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
 // The workgroup -> problem table and the flags travel as the kernel's first scalar arguments: built with
 // -amdgpu-kernarg-preload-count the hardware delivers them in SGPRs at wave launch, so a workgroup knows its problem
 // without a memory round trip and the one scalar load left (the problem's fields) is issued at once.
+// What a workgroup needs before its first weight request, 32 bytes per problem at the head of the argument block: one
+// scalar load instead of one per field.
+struct GemvEarly {
+    const uint8_t* w;
+    const float* x;
+    int N, K;
+    uint32_t w_bytes;
+    uint32_t pad;
+};
 struct GemvProblems {
+    GemvEarly e[kMaxGroup];
     GemvProblem p[kMaxGroup];
 };
-template <int TYPE, int ACT, bool TL, int EAGER>
+// SIMPLE: no problem of the launch has expert indirection, a paired store or a routed sum (the streaming build then takes
+// its first fields from the early records and has those three switched off at compile time)
+template <int TYPE, int ACT, bool TL, int EAGER, bool SIMPLE>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) gemv_kernel(int b0, int b1, int b2, int b3, int b4, int b5, int b6, int b7, int b8, int count,
                                                         int strict, const GemvProblems G, uint64_t* tl)
 {
@@ -1222,11 +1234,11 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4
     if (6 < count && bx >= b6) { i = 6; lo = b6; hi = b7; }
     if (7 < count && bx >= b7) { i = 7; lo = b7; hi = b8; }
     const int wg = bx - lo, nwg = hi - lo;
-    // Eager build: the problem's fields arrive with one round trip.  Read lazily, where the code first needs them, they
-    // cost one dependent scalar load after the other (seven before the first weight request, about 1 us), which a launch of
-    // a few microseconds feels (MXFP4 5760 x 2880: 6.3 -> 6.0 us).  The streaming build keeps the lazy reads: with them
-    // the wavefronts of a long launch start a little apart and it measured faster that way (123 MB grouped launch 24.0
-    // against 25.1 us, Q8_0 4096 x 4096 8.2 against 8.9 us on one box).
+    // Read where the code first needs them, the problem's fields cost one dependent scalar load after the other (seven
+    // before the first weight request, about 1 us).  Eager build: the whole struct in one round trip, pinned in SGPRs.
+    // Streaming build: the early record in one load and the rest where it is used.  (Pinning the whole struct as the eager
+    // build does starts the streaming build 1 us earlier too, by the per-wavefront timeline, but its loop then runs 10 %
+    // slower - 123 MB grouped launch 25.1 against 24.4 us - where the early record gives 23.4.)
     GemvProblem Pv;
     if constexpr (EAGER > 0) {
         Pv = G.p[i];
@@ -1240,7 +1252,16 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4
         Pv.w = reinterpret_cast<const uint8_t*>(w), Pv.x = reinterpret_cast<const float*>(x), Pv.y = reinterpret_cast<float*>(y);
         Pv.add = reinterpret_cast<const float*>(add), Pv.norm_w = reinterpret_cast<const float*>(nw), Pv.expert_id = reinterpret_cast<const int*>(eid);
     }
-    const GemvProblem& P = EAGER > 0 ? Pv : G.p[i];
+    if constexpr (EAGER == 0 && SIMPLE) {
+        const GemvEarly E = G.e[i];
+        Pv.w = E.w, Pv.x = E.x, Pv.N = E.N, Pv.K = E.K, Pv.w_bytes = (int64_t)E.w_bytes;
+        Pv.y = G.p[i].y, Pv.add = G.p[i].add, Pv.norm_w = G.p[i].norm_w, Pv.eps = G.p[i].eps, Pv.limit = 0.f, Pv.act = ACT;
+        Pv.expert_id = nullptr, Pv.expert_stride = 0, Pv.n_experts = 0, Pv.pair_rows = 0, Pv.pair_kind = 0;
+        Pv.slot_ids = nullptr, Pv.slot_w = nullptr, Pv.slot_bias = nullptr;
+    }
+    // (problems with expert indirection, paired or routed stores keep the lazy reads: an early record carrying those fields
+    // too measured 0.3 - 0.5 us slower on the two launches of a GPT-OSS token)
+    const GemvProblem& P = (EAGER > 0 || SIMPLE) ? Pv : G.p[i];
     if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
@@ -1248,6 +1269,39 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4
     else if (TYPE == kTypeQ4_0 || TYPE == kTypeQ4_1 || TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1 || TYPE == kTypeIQ4_NL)
         gemv_body<FmtLegacy<TYPE>, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else gemv_body<FmtQ80, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
+}
+
+// A launch of ONE problem without expert indirection: everything the kernel needs before its first weight request -
+// weight, activations, result, sizes, the residual and the norm weight, and one word with the mode (bits 0..1), the kind
+// of paired store (bits 2..3) and its row count (bits 4..) - are the first scalar arguments, which the hardware delivers
+// in SGPRs at wave launch (14 dwords).  No scalar load stands between entry and that request; read one after the other
+// from the argument block, as the grouped kernel must (its problem depends on the workgroup), the fields cost 1 - 1.8 us
+// per launch (Q4_K 14336 x 4096 10.2 -> 8.4 us, 4096 x 4096 6.0 -> 4.8, MXFP4 5760 x 2880 6.4 -> 5.2, a decode layer
+// 52.8 -> 49.2 us).  eps and limit are read where the code reaches them.
+// (PAIR as a compile-time switch: with the row count of the paired store as a run-time value the plain launches carry its
+// code and measured 0.1 - 0.25 us slower.)
+constexpr int kOnePairShift = 4;
+template <int TYPE, int ACT, bool TL, int EAGER, bool PAIR>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) gemv_one_kernel(
+    const uint8_t* w, const float* x, float* y, int N, int K, int w_bytes, int flags, const float* add, const float* norm_w,
+    float eps, float limit, uint64_t* tl)
+{
+    extern __shared__ uint32_t lds[];
+    GemvProblem Pv;
+    Pv.w = w, Pv.x = x, Pv.y = y, Pv.N = N, Pv.K = K, Pv.w_bytes = (int64_t)(uint32_t)w_bytes, Pv.add = add, Pv.norm_w = norm_w;
+    Pv.act = ACT;
+    Pv.eps = eps, Pv.limit = limit;
+    Pv.expert_id = nullptr, Pv.expert_stride = 0, Pv.n_experts = 0;
+    Pv.pair_rows = PAIR ? (int)((uint32_t)flags >> kOnePairShift) : 0, Pv.pair_kind = PAIR ? (flags >> 2) & 3 : 0;
+    Pv.slot_ids = nullptr, Pv.slot_w = nullptr, Pv.slot_bias = nullptr;
+    const int strict = flags & 3, wg = (int)blockIdx.x, nwg = (int)gridDim.x;
+    if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
+    else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
+    else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
+    else if (TYPE == kTypeQ5_K) gemv_body<FmtQ5K, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
+    else if (TYPE == kTypeQ4_0 || TYPE == kTypeQ4_1 || TYPE == kTypeQ5_0 || TYPE == kTypeQ5_1 || TYPE == kTypeIQ4_NL)
+        gemv_body<FmtLegacy<TYPE>, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
+    else gemv_body<FmtQ80, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
 }
 
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
@@ -1278,14 +1332,41 @@ int64_t g_timeline_waves = 0;
 template <int TYPE, int ACT, bool TL, int EAGER>
 bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    auto kern = gemv_kernel<TYPE, ACT, TL, EAGER>;
-    if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+    if (g.count == 1 && !g.p[0].expert_id && !g.p[0].slot_ids &&
+        g.p[0].pair_rows < (1 << (31 - kOnePairShift)) && g.p[0].pair_kind >= 0 && g.p[0].pair_kind < 4) {
+        const GemvProblem& p = g.p[0];
+        const int flags = (g.strict & 3) | (p.pair_kind << 2) | (int)((uint32_t)p.pair_rows << kOnePairShift);
+        auto launch_one = [&](auto one) {
+            if (!raise_lds_limit(reinterpret_cast<const void*>(one), lds)) return false;
+            hipLaunchKernelGGL(one, dim3(grid), dim3(kThreads), lds, stream, p.w, p.x, p.y, p.N, p.K, (int)(uint32_t)p.w_bytes, flags, p.add,
+                               p.norm_w, p.eps, p.limit, TL ? g_timeline : nullptr);
+            return hip_ok(hipGetLastError(), "gemv launch");
+        };
+        // (the paired store exists for plain and RMSNorm staging without timeline or eager build)
+        if constexpr (!TL && EAGER == 0 && ACT != kActSiluMul) {
+            if (p.pair_rows) return launch_one(gemv_one_kernel<TYPE, ACT, TL, EAGER, true>);
+        }
+        if (!p.pair_rows) return launch_one(gemv_one_kernel<TYPE, ACT, TL, EAGER, false>);
+    }
     GemvProblems gp;
     std::memcpy(gp.p, g.p, sizeof(gp.p));
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g.wg_begin[0], g.wg_begin[1], g.wg_begin[2], g.wg_begin[3],
-                       g.wg_begin[4], g.wg_begin[5], g.wg_begin[6], g.wg_begin[7], g.wg_begin[8], g.count, g.strict, gp,
-                       TL ? g_timeline : nullptr);
-    return hip_ok(hipGetLastError(), "gemv launch");
+    bool simple = EAGER == 0;
+    for (int i = 0; i < kMaxGroup; ++i) {
+        const GemvProblem& p = g.p[i];
+        gp.e[i] = GemvEarly{p.w, p.x, p.N, p.K, (uint32_t)p.w_bytes, 0u};
+        if (i < g.count) simple = simple && !p.expert_id && !p.pair_rows && !p.slot_ids;
+    }
+    auto launch = [&](auto kern) {
+        if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, g.wg_begin[0], g.wg_begin[1], g.wg_begin[2], g.wg_begin[3],
+                           g.wg_begin[4], g.wg_begin[5], g.wg_begin[6], g.wg_begin[7], g.wg_begin[8], g.count, g.strict, gp,
+                           TL ? g_timeline : nullptr);
+        return hip_ok(hipGetLastError(), "gemv launch");
+    };
+    if constexpr (EAGER == 0) {
+        if (simple) return launch(gemv_kernel<TYPE, ACT, TL, EAGER, true>);
+    }
+    return launch(gemv_kernel<TYPE, ACT, TL, EAGER, false>);
 }
 
 // steps the eager build of a format holds in registers (0: the format has no eager build)
