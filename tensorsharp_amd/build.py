@@ -13,10 +13,12 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    # the leading scalar arguments of every kernel (up to 14 dwords) arrive preloaded in SGPRs at wave launch; the code
+    # objects keep a loading prologue for firmware without the feature
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
 ]
-# per-source additions.  gemv.hip: the first 11 dwords of kernel arguments (the workgroup -> problem table of
-# gemv_kernel) arrive preloaded in SGPRs; the code object keeps a loading prologue for firmware without the feature.
-EXTRA_FLAGS = {"gemv.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
+# per-source additions
+EXTRA_FLAGS = {}
 
 
 def build(verbose=False, jobs=8):

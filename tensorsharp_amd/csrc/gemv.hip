@@ -1077,6 +1077,8 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
 #pragma unroll
         for (int s = 0; s < EAGER; ++s) fetch(s < nsteps ? gw : ngroups, s, eager[s]);
     } else {
+        // (with expert indirection, requesting the activations first so that they travel while the id is on its way gained
+        // 0.15 us on a GPT-OSS token: not kept)
         fetch(fgroup, fstep, cur);
         advance(fgroup, fstep);
         if (deep) {
@@ -1203,22 +1205,30 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
 // The workgroup -> problem table and the flags travel as the kernel's first scalar arguments: built with
 // -amdgpu-kernarg-preload-count the hardware delivers them in SGPRs at wave launch, so a workgroup knows its problem
 // without a memory round trip and the one scalar load left (the problem's fields) is issued at once.
-// What a workgroup needs before its first weight request, 32 bytes per problem at the head of the argument block: one
-// scalar load instead of one per field.
+// What a workgroup needs before its first weight request, 32 bytes per problem (64 with expert indirection) at the head of
+// the argument block: one scalar load instead of one per field.
 struct GemvEarly {
     const uint8_t* w;
     const float* x;
     int N, K;
     uint32_t w_bytes;
-    uint32_t pad;
+    int pair_rows;
+    // problems whose weight is chosen by an expert id read on the device
+    const int* expert_id;
+    int64_t expert_stride;
+    int n_experts;
+    int pair_kind;
+    int64_t pad;
 };
+static_assert(sizeof(GemvEarly) == 64, "at most one 16-dword scalar load");
 struct GemvProblems {
     GemvEarly e[kMaxGroup];
     GemvProblem p[kMaxGroup];
 };
-// SIMPLE: no problem of the launch has expert indirection, a paired store or a routed sum (the streaming build then takes
-// its first fields from the early records and has those three switched off at compile time)
-template <int TYPE, int ACT, bool TL, int EAGER, bool SIMPLE>
+// EARLY 1: no problem of the launch has expert indirection, a paired store or a routed sum; 2: every problem has expert
+// indirection and none a routed sum (the streaming build then takes its first fields from the early records and has the
+// absent features switched off at compile time); 0: fields read where the code needs them
+template <int TYPE, int ACT, bool TL, int EAGER, int EARLY>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) gemv_kernel(int b0, int b1, int b2, int b3, int b4, int b5, int b6, int b7, int b8, int count,
                                                         int strict, const GemvProblems G, uint64_t* tl)
 {
@@ -1252,16 +1262,22 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4
         Pv.w = reinterpret_cast<const uint8_t*>(w), Pv.x = reinterpret_cast<const float*>(x), Pv.y = reinterpret_cast<float*>(y);
         Pv.add = reinterpret_cast<const float*>(add), Pv.norm_w = reinterpret_cast<const float*>(nw), Pv.expert_id = reinterpret_cast<const int*>(eid);
     }
-    if constexpr (EAGER == 0 && SIMPLE) {
+    if constexpr (EAGER == 0 && EARLY == 1) {
         const GemvEarly E = G.e[i];
         Pv.w = E.w, Pv.x = E.x, Pv.N = E.N, Pv.K = E.K, Pv.w_bytes = (int64_t)E.w_bytes;
         Pv.y = G.p[i].y, Pv.add = G.p[i].add, Pv.norm_w = G.p[i].norm_w, Pv.eps = G.p[i].eps, Pv.limit = 0.f, Pv.act = ACT;
         Pv.expert_id = nullptr, Pv.expert_stride = 0, Pv.n_experts = 0, Pv.pair_rows = 0, Pv.pair_kind = 0;
         Pv.slot_ids = nullptr, Pv.slot_w = nullptr, Pv.slot_bias = nullptr;
     }
-    // (problems with expert indirection, paired or routed stores keep the lazy reads: an early record carrying those fields
-    // too measured 0.3 - 0.5 us slower on the two launches of a GPT-OSS token)
-    const GemvProblem& P = (EAGER > 0 || SIMPLE) ? Pv : G.p[i];
+    if constexpr (EAGER == 0 && EARLY == 2) {
+        const GemvEarly E = G.e[i];
+        Pv.w = E.w, Pv.x = E.x, Pv.N = E.N, Pv.K = E.K, Pv.w_bytes = (int64_t)E.w_bytes, Pv.pair_rows = E.pair_rows;
+        Pv.expert_id = E.expert_id, Pv.expert_stride = E.expert_stride, Pv.n_experts = E.n_experts, Pv.pair_kind = E.pair_kind;
+        Pv.y = G.p[i].y, Pv.add = G.p[i].add, Pv.norm_w = G.p[i].norm_w, Pv.eps = G.p[i].eps, Pv.limit = G.p[i].limit, Pv.act = ACT;
+        Pv.slot_ids = nullptr, Pv.slot_w = nullptr, Pv.slot_bias = nullptr;
+    }
+    // (a launch that mixes the features keeps the lazy reads)
+    const GemvProblem& P = (EAGER > 0 || EARLY != 0) ? Pv : G.p[i];
     if (TYPE == kTypeQ4_K) gemv_body<FmtQ4K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
     else if (TYPE == kTypeQ6_K) gemv_body<FmtQ6K, ACT, TL, EAGER>(P, wg, nwg, strict, lds, tl, i);
@@ -1304,6 +1320,26 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4
     else gemv_body<FmtQ80, ACT, TL, EAGER>(Pv, wg, nwg, strict, lds, tl, 0);
 }
 
+// The routed sum of one token (MoE decode: down projections + weighted sum) as a launch of its own argument list: the
+// stack of expert matrices, the staged activation vectors, the slot tables and the geometry are the preloaded scalars; the
+// result pointer and the bias are read where the code reaches them.
+template <int TYPE>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) gemv_routed_kernel(
+    const uint8_t* w, const float* x, int N, int K, int w_bytes, int flags, const int* slot_ids, const float* slot_w, int expert_stride,
+    float* y, const float* slot_bias)
+{
+    extern __shared__ uint32_t lds[];
+    GemvProblem Pv;
+    Pv.w = w, Pv.x = x, Pv.y = y, Pv.N = N, Pv.K = K, Pv.w_bytes = (int64_t)(uint32_t)w_bytes, Pv.add = nullptr, Pv.norm_w = nullptr;
+    Pv.act = kActPlain, Pv.eps = 0.f, Pv.limit = 0.f;
+    Pv.expert_id = nullptr, Pv.expert_stride = (int64_t)(uint32_t)expert_stride, Pv.n_experts = (int)((uint32_t)flags >> 8);
+    Pv.pair_rows = 0, Pv.pair_kind = 0;
+    Pv.slot_ids = slot_ids, Pv.slot_w = slot_w, Pv.slot_bias = slot_bias;
+    const int strict = flags & 3, wg = (int)blockIdx.x, nwg = (int)gridDim.x;
+    if (TYPE == kTypeMXFP4) gemv_body<FmtMXFP4, kActPlain, false, 0>(Pv, wg, nwg, strict, lds, nullptr, 0);
+    else gemv_body<FmtQ80, kActPlain, false, 0>(Pv, wg, nwg, strict, lds, nullptr, 0);
+}
+
 int unit_elems(int type) { return type == kTypeQ4_K || type == kTypeQ5_K || type == kTypeQ6_K ? 64 : 32; }
 bool legacy_type(int type) { return type == kTypeQ4_0 || type == kTypeQ4_1 || type == kTypeQ5_0 || type == kTypeQ5_1 || type == kTypeIQ4_NL; }
 int unit_lds_bytes(int type) { return type == kTypeMXFP4 || legacy_type(type) ? 80 : type == kTypeQ6_K ? 176 : 144; }
@@ -1332,6 +1368,17 @@ int64_t g_timeline_waves = 0;
 template <int TYPE, int ACT, bool TL, int EAGER>
 bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
+    if constexpr ((TYPE == kTypeMXFP4 || TYPE == kTypeQ8_0) && ACT == kActPlain && !TL && EAGER == 0) {
+        const GemvProblem& p = g.p[0];
+        if (g.count == 1 && p.slot_ids && !p.expert_id && !p.pair_rows && !p.add && p.n_experts < (1 << 23) &&
+            p.expert_stride < ((int64_t)1 << 31)) {
+            auto kern = gemv_routed_kernel<TYPE>;
+            if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, stream, p.w, p.x, p.N, p.K, (int)(uint32_t)p.w_bytes,
+                               (g.strict & 3) | (p.n_experts << 8), p.slot_ids, p.slot_w, (int)p.expert_stride, p.y, p.slot_bias);
+            return hip_ok(hipGetLastError(), "gemv launch");
+        }
+    }
     if (g.count == 1 && !g.p[0].expert_id && !g.p[0].slot_ids &&
         g.p[0].pair_rows < (1 << (31 - kOnePairShift)) && g.p[0].pair_kind >= 0 && g.p[0].pair_kind < 4) {
         const GemvProblem& p = g.p[0];
@@ -1350,11 +1397,14 @@ bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream
     }
     GemvProblems gp;
     std::memcpy(gp.p, g.p, sizeof(gp.p));
-    bool simple = EAGER == 0;
+    bool simple = EAGER == 0, expert = EAGER == 0;
     for (int i = 0; i < kMaxGroup; ++i) {
         const GemvProblem& p = g.p[i];
-        gp.e[i] = GemvEarly{p.w, p.x, p.N, p.K, (uint32_t)p.w_bytes, 0u};
-        if (i < g.count) simple = simple && !p.expert_id && !p.pair_rows && !p.slot_ids;
+        gp.e[i] = GemvEarly{p.w, p.x, p.N, p.K, (uint32_t)p.w_bytes, p.pair_rows, p.expert_id, p.expert_stride, p.n_experts, p.pair_kind, 0};
+        if (i < g.count) {
+            simple = simple && !p.expert_id && !p.pair_rows && !p.slot_ids;
+            expert = expert && p.expert_id && !p.slot_ids;
+        }
     }
     auto launch = [&](auto kern) {
         if (!raise_lds_limit(reinterpret_cast<const void*>(kern), lds)) return false;
@@ -1364,9 +1414,13 @@ bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream
         return hip_ok(hipGetLastError(), "gemv launch");
     };
     if constexpr (EAGER == 0) {
-        if (simple) return launch(gemv_kernel<TYPE, ACT, TL, EAGER, true>);
+        if (simple) return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 1>);
     }
-    return launch(gemv_kernel<TYPE, ACT, TL, EAGER, false>);
+    // (expert indirection goes with plain staging: the MoE decode launches)
+    if constexpr (EAGER == 0 && ACT == kActPlain && !TL && (TYPE == kTypeMXFP4 || TYPE == kTypeQ8_0 || TYPE == kTypeQ4_K)) {
+        if (expert) return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 2>);
+    }
+    return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 0>);
 }
 
 // steps the eager build of a format holds in registers (0: the format has no eager build)

@@ -96,10 +96,13 @@ __device__ __forceinline__ float sum16(float v)
 // the split, kInFlight at a time (all their loads are issued before the first is used: the loop is latency bound), lane l of
 // a group holds the head dimensions l, l + 16, ... (PER of them).  Groups, then wavefronts, merge their softmax states.
 template <int PER, int G>
-__global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const AttnFront F, int group, int max_seq_len, int total,
-                                                                       int split_len, float scale, int splits,
-                                                                       float* __restrict__ partial, float* __restrict__ out_direct)
+__global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(float* k_cache, float* v_cache, const float* qkv, int group,
+                                                                       int max_seq_len, int total, int split_len, float scale, int splits,
+                                                                       int num_heads, float* __restrict__ partial, const AttnFront F,
+                                                                       float* __restrict__ out_direct)
 {
+    // (what the first loads need - the caches, the projections, the geometry - are leading scalar arguments: the hardware
+    // delivers the first 14 dwords in SGPRs at wave launch, the rest is read from the argument block)
     constexpr int HD = 16 * PER;
     __shared__ float sm[kAttnWaves][G], sl[kAttnWaves][G], sacc[kAttnWaves][G][HD];
     __shared__ float sq[G][HD], sk[HD], sv[HD], tmp[kAttnWaves][HD];
@@ -107,8 +110,8 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
     const int h0 = kvh * group + blockIdx.z * G;                     // first query head of this workgroup
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lg = lane & 15, grp = (wave << 2) | (lane >> 4);       // 16 groups per workgroup
-    const float* kb = F.k_cache + (int64_t)kvh * max_seq_len * HD;
-    const float* vb = F.v_cache + (int64_t)kvh * max_seq_len * HD;
+    const float* kb = k_cache + (int64_t)kvh * max_seq_len * HD;
+    const float* vb = v_cache + (int64_t)kvh * max_seq_len * HD;
     const int position = total - 1;
     const bool last = split == splits - 1;                           // the split that holds the new position
     // kInFlight rows of K and of V per group, all requested before the first is used; the first set is requested
@@ -137,7 +140,7 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
         constexpr int kPer = (HD + 63) / 64, kPairs = (HD / 2 + 63) / 64;
         constexpr int half = HD / 2;
         const int nprep = G + (last ? 1 : 0);
-        auto head_src = [&](int hh) { return F.qkv + (int64_t)(hh < G ? h0 + hh : F.num_heads + kvh) * HD; };
+        auto head_src = [&](int hh) { return qkv + (int64_t)(hh < G ? h0 + hh : num_heads + kvh) * HD; };
         // the wavefront's first head is requested before the angles are worked out
         float xv[kPer];
 #pragma unroll
@@ -194,7 +197,7 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             float* dst = is_q ? sq[hh] : sk;
-            float* cache = (!is_q && blockIdx.z == 0) ? F.k_cache + ((int64_t)kvh * max_seq_len + position) * HD : nullptr;
+            float* cache = (!is_q && blockIdx.z == 0) ? k_cache + ((int64_t)kvh * max_seq_len + position) * HD : nullptr;
 #pragma unroll
             for (int j = 0; j < kPairs; ++j) {
                 const int p = lane + 64 * j;
@@ -214,8 +217,8 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(const Attn
             __builtin_amdgcn_wave_barrier();
         }
         if (last) {
-            const float* src = F.qkv + (int64_t)(F.num_heads + F.num_kv_heads + kvh) * HD;
-            float* cache = blockIdx.z == 0 ? F.v_cache + ((int64_t)kvh * max_seq_len + position) * HD : nullptr;
+            const float* src = qkv + (int64_t)(num_heads + F.num_kv_heads + kvh) * HD;
+            float* cache = blockIdx.z == 0 ? v_cache + ((int64_t)kvh * max_seq_len + position) * HD : nullptr;
             for (int d = threadIdx.x; d < HD; d += kAttnWaves * 64) {
                 const float v = src[d];
                 sv[d] = v;
@@ -471,8 +474,8 @@ bool launch_attention_decode(const float* qkv, const float* q_norm_w, const floa
     while (g > 2 && num_kv_heads * splits * (group / g) < 128) g >>= 1;
     const dim3 grid(num_kv_heads, splits, group / g), block(kAttnWaves * 64);
 #define TSHIP_ATTN_LAUNCH(PER, GG)                                                                                              \
-    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, front, group, max_seq_len, total, split_len, scale, \
-                       splits, partial_ws, splits == 1 ? out : nullptr)
+    hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, front.k_cache, front.v_cache, front.qkv, group,     \
+                       max_seq_len, total, split_len, scale, splits, num_heads, partial_ws, front, splits == 1 ? out : nullptr)
 #define TSHIP_ATTN_G(PER)                                                    \
     switch (g) {                                                             \
     case 8: TSHIP_ATTN_LAUNCH(PER, 8); break;                                \
