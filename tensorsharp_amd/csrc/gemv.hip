@@ -1221,6 +1221,8 @@ struct GemvEarly {
     int64_t pad;
 };
 static_assert(sizeof(GemvEarly) == 64, "at most one 16-dword scalar load");
+// (The size of the argument block does not matter: plain launches with a 512-byte block of their own instead of these
+// 1.5 KB measured the same 23.2 us and the same gap between launches.)
 struct GemvProblems {
     GemvEarly e[kMaxGroup];
     GemvProblem p[kMaxGroup];
