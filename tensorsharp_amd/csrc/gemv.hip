@@ -913,7 +913,9 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const int nsteps = (upr + LPR - 1) / LPR;   // steps per row group
     // Plain: a group is RPG consecutive rows.  Paired (gate | up stacks of pair_rows rows each): a group is RPG / 2
     // consecutive gate rows in the lower half of the wavefront and the matching up rows in the upper half, so that gate j
-    // and up j finish in lanes 32 apart and meet at the store.
+    // and up j finish in lanes 32 apart and meet at the store.  (The other mapping - a group is RPG gate rows and then,
+    // in the same lanes, their RPG up rows, the gate sums kept meanwhile, so that a wavefront's requests stay within one
+    // stretch of rows - measured 0.3 us slower on a llama-3-8B decode layer and 1.0 us slower on a GPT-OSS token.)
     const int pair = P.pair_rows;                      // uniform
     constexpr int HALF = RPG / 2;
     const int gstep_plain = pair ? HALF : RPG;
