@@ -609,7 +609,7 @@ def main():
             "bound": "hbm", "achieved": chain["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(chain["GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
             "workload": "configs[1] shapes as one dependent decode layer at context 512 (TSHip_TransformerLayerDecodeDevice)",
-            "kernel": "six launches: tship::gemv_kernel<12, ...> x 4, tship::attn_decode_kernel, tship::attn_combine_kernel",
+            "kernel": "six launches: tship::gemv_one_kernel<12, ...> x 4, tship::attn_decode_kernel, tship::attn_combine_kernel",
             "avg_call_us": chain["us_per_layer_events"], "bytes_per_call": chain["bytes"]}
         # fused SwiGLU FFN at decode (configs[1] shapes: hidden 4096, intermediate 14336, Q4_K, one token):
         # RMSNorm -> gate_up GEMV -> SiLU*up -> down GEMV + residual, one ABI call (4 launches)

@@ -312,8 +312,15 @@ bool check_device_operands(const TSHipTensorView2D& m1, const void* w, int type)
 // rows (output columns) in slices below 2 GiB, activation rows in slices whose fp16 copy stays below 2 GiB.
 constexpr size_t kQ81SliceBytes = (size_t)32 << 20;
 
+// Results of fewer than this many columns, with more than three rows of activations, go through an exact fp32 copy of
+// the (small) weight instead of the matrix cores: the fp16 operands of the offset formats carry rounded scale products
+// (Q4_K: every result about 7.5e-4 of the results' magnitude off, one sigma), and the row norm that the 1e-3 bound is
+// taken against grows with the square root of the columns - on 32 columns a sweep of random cases reached 1.03e-3.
+constexpr int kNarrowColumns = 64;
+
 struct MatmulPlan {
     bool gemv;            // decode / tiny batch: one bandwidth-bound GEMV per activation row
+    bool narrow;          // few result columns: fp32 copy of the weight + the dense kernel
     int m_step;           // activation rows per launch
     int64_t n_step;       // weight rows per launch
     size_t conv_bytes;    // [row scales][fp16 activations] of one slice of rows (prefill), or the RMSNorm rows (decode)
@@ -343,6 +350,13 @@ MatmulPlan plan_matmul(int type, int M, int64_t K, int64_t N, bool norm, bool ac
         p.n_step = std::max<int64_t>(256, (int64_t)((size_t)(kMaxOperandBytes - 1) / rs) / 256 * 256);
     }
     p.gemv = M <= 3 && K <= gemv_max_k(type);
+    if (!p.gemv && N < kNarrowColumns) {
+        p.narrow = true;
+        p.m_step = M;
+        p.conv_bytes = norm ? al((size_t)M * (size_t)K * sizeof(float)) : 0;
+        p.chunk_bytes = al((size_t)N * (size_t)K * sizeof(float));
+        return p;
+    }
     if (p.gemv) {
         p.m_step = M;
         // RMSNorm is formed by the GEMV while it stages x (rows up to gemv_rms_max_k()), else by a kernel of its own
@@ -382,7 +396,7 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
     }
     const uint8_t* wb = static_cast<const uint8_t*>(w);
     float* out = static_cast<float*>(result.data);
-    if (is_dense_type(type) || type == kTypeQ8_1) {
+    if (is_dense_type(type) || type == kTypeQ8_1 || plan.narrow) {
         const float* xs = static_cast<const float*>(m1.data);
         int64_t ldx = m1.stride0;
         if (norm_w) {
@@ -390,9 +404,9 @@ bool run_matmul_device_ws(const TSHipTensorView2D& result, const TSHipTensorView
             xs = static_cast<const float*>(ws);
             ldx = K;
         }
-        if (type != kTypeQ8_1) return launch_dense_matmul(type, w, xs, ldx, out, result.stride0, M, (int)N, (int)K, accumulate, stream);
+        if (is_dense_type(type)) return launch_dense_matmul(type, w, xs, ldx, out, result.stride0, M, (int)N, (int)K, accumulate, stream);
         if (plan.total() > ws_bytes) {
-            set_last_error("matmul: the device workspace is too small for the fp32 copy of a Q8_1 weight slice.");
+            set_last_error("matmul: the device workspace is too small for the fp32 copy of a weight slice.");
             return false;
         }
         float* rows = reinterpret_cast<float*>(static_cast<char*>(ws) + plan.conv_bytes);

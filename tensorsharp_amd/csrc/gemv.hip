@@ -1393,8 +1393,8 @@ bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream
                                p.norm_w, p.eps, p.limit, TL ? g_timeline : nullptr);
             return hip_ok(hipGetLastError(), "gemv launch");
         };
-        // (the paired store exists for plain and RMSNorm staging without timeline or eager build)
-        if constexpr (!TL && EAGER == 0 && ACT != kActSiluMul) {
+        // (one problem with a paired store and no expert indirection: the gate | up launch of the fused FFN, RMSNorm staging)
+        if constexpr (!TL && EAGER == 0 && ACT == kActRmsNorm) {
             if (p.pair_rows) return launch_one(gemv_one_kernel<TYPE, ACT, TL, EAGER, true>);
         }
         if (!p.pair_rows) return launch_one(gemv_one_kernel<TYPE, ACT, TL, EAGER, false>);
@@ -1417,14 +1417,24 @@ bool launch_type_tl(const GemvGroup& g, int grid, size_t lds, hipStream_t stream
                            TL ? g_timeline : nullptr);
         return hip_ok(hipGetLastError(), "gemv launch");
     };
-    if constexpr (EAGER == 0) {
+    // (RMSNorm staging only ever comes as one problem per launch: it has the one-problem kernels above)
+    if constexpr (EAGER == 0 && ACT != kActRmsNorm) {
         if (simple) return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 1>);
     }
     // (expert indirection goes with plain staging: the MoE decode launches)
-    if constexpr (EAGER == 0 && ACT == kActPlain && !TL && (TYPE == kTypeMXFP4 || TYPE == kTypeQ8_0 || TYPE == kTypeQ4_K)) {
+    constexpr bool kExpertRecords = EAGER == 0 && ACT == kActPlain && !TL && (TYPE == kTypeMXFP4 || TYPE == kTypeQ8_0 || TYPE == kTypeQ4_K);
+    if constexpr (kExpertRecords) {
         if (expert) return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 2>);
     }
-    return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 0>);
+    // The build that reads every field where it needs it serves what is left: the eager builds (they take the whole
+    // problem in one load anyway) and expert indirection for the formats without early expert records.  Other
+    // combinations are not instantiated.
+    if constexpr (EAGER > 0 || (ACT == kActPlain && !TL && !kExpertRecords)) {
+        return launch(gemv_kernel<TYPE, ACT, TL, EAGER, 0>);
+    } else {
+        set_last_error("gemv: no kernel for this combination of problems (activation mode, paired store, expert indirection).");
+        return false;
+    }
 }
 
 // steps the eager build of a format holds in registers (0: the format has no eager build)
@@ -1438,7 +1448,10 @@ int eager_steps(int type)
 template <int TYPE, int ACT>
 bool launch_type(const GemvGroup& g, int grid, size_t lds, hipStream_t stream)
 {
-    const bool tl = ACT == kActPlain && g_timeline != nullptr && (int64_t)grid * kWaves <= g_timeline_waves;
+    // (the timeline build stamps launches of plain problems only)
+    bool plain = true;
+    for (int i = 0; i < g.count; ++i) plain = plain && !g.p[i].expert_id && !g.p[i].pair_rows && !g.p[i].slot_ids;
+    const bool tl = ACT == kActPlain && plain && g_timeline != nullptr && (int64_t)grid * kWaves <= g_timeline_waves;
     if constexpr (ACT == kActPlain && kEagerSteps<TYPE> > 0) {
         if (g.strict == 2)
             return tl ? launch_type_tl<TYPE, kActPlain, true, kEagerSteps<TYPE>>(g, grid, lds, stream)

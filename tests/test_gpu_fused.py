@@ -58,6 +58,28 @@ def test_rms_norm_matmul(hip, oracle, name, M, device):
     assert ok, (name, M, device, worst)
 
 
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "q5_k", "q6_k"])
+@pytest.mark.parametrize("M", [1, 3])
+def test_rms_norm_matmul_decode_every_other_gemv_format(hip, oracle, name, M):
+    # one launch per row with RMSNorm(x) * w formed while the activations are staged: each block format stages them in
+    # its own unpack order (random valid blocks; the three headline formats are covered above)
+    import torch
+    from oracle.oracle import MORE_TYPES
+    from tensorsharp_amd import QuantizedWeight, synth
+    t = MORE_TYPES[name]
+    rng = np.random.default_rng(17 + M)
+    N, K = 392, 1024
+    w = synth.random_weight(t, N, K, torch.device("cuda"), seed=31, sigma=0.03)
+    x = (rng.standard_normal((M, K)) * 3).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    ref = oracle.matmul_f64(t, w.cpu().numpy(), N, K, oracle.rms_norm_mul(x, nw, EPS))
+    res = torch.empty((M, N), device="cuda")
+    hip.FusedRmsNormMatMulQuant(res, torch.from_numpy(x).cuda(), torch.from_numpy(nw).cuda(), EPS, QuantizedWeight(w, t, K, N))
+    torch.cuda.synchronize()
+    ok, worst = bound_ok(res.cpu().numpy(), ref, ref)
+    assert ok, (name, M, worst)
+
+
 @pytest.mark.parametrize("name", ["q8_0", "q4_k", "mxfp4"])
 @pytest.mark.parametrize("M", [1, 2, 70, 300])
 @pytest.mark.parametrize("device", [False, True])

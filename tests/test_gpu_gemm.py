@@ -463,3 +463,24 @@ def test_config5_full_size(hip, oracle, tname):
     y4 = hip.LinearForward(x * 4.0, w)
     torch.cuda.synchronize()
     assert torch.equal(y4, y * 4.0)
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q8_0", "mxfp4", "q5_k", "q6_k", "q4_1"])
+@pytest.mark.parametrize("M,N,K", [(200, 32, 1024), (9, 63, 2048), (4, 1, 512)])
+def test_narrow_results_are_formed_from_exact_weights(hip, oracle, name, M, N, K):
+    """Fewer than 64 result columns with more than three rows: the row norm the 1e-3 bound is taken against is that of a
+    few numbers, and the rounded scale products of fp16 operands (Q4_K: every result 7.5e-4 of the results' magnitude off,
+    one sigma) would come within reach of it.  Such calls multiply by an exact fp32 copy of the small weight instead, and
+    agree with the fp64 reference to fp32 rounding."""
+    import torch
+    from oracle.oracle import MORE_TYPES, Q6_K
+    from tensorsharp_amd import QuantizedWeight, synth
+    t = T.get(name) or MORE_TYPES.get(name) or Q6_K
+    rng = np.random.default_rng(M + N + K)
+    w = synth.random_weight(t, N, K, torch.device("cuda"), seed=7, sigma=0.03)
+    x = (rng.standard_normal((M, K)) * 2).astype(np.float32)
+    ref = oracle.matmul_f64(t, w.cpu().numpy(), N, K, x)
+    y = hip.LinearForward(torch.from_numpy(x).cuda(), QuantizedWeight(w, t, K, N))
+    torch.cuda.synchronize()
+    err = inputs.row_l2_err(y.cpu().numpy(), ref)         # fp16 operands would leave 1e-4 ... 1e-3 here
+    assert err <= 1e-5, (name, M, N, K, err)

@@ -429,3 +429,44 @@ def test_timeline_build_same_results_and_ordered_stamps(hip, oracle, name, N, K)
     hip.LinearForward(x, qw)
     torch.cuda.synchronize()
     assert int(buf.abs().sum().item()) == 0
+
+
+@pytest.mark.parametrize("name,shapes", [("q4_k", [(4096, 4096), (1024, 4096)]), ("q4_k", [(9000, 1024), (300, 1024), (5000, 2048)]),
+                                         ("mxfp4", [(2880, 2880), (2880, 2880)]), ("mxfp4", [(20000, 512), (64, 512)]),
+                                         ("q8_0", [(1000, 2560), (3000, 512)]), ("q6_k", [(700, 1024), (900, 512)]),
+                                         ("q5_k", [(700, 1024), (900, 512)]), ("q4_0", [(900, 1024), (700, 512)]),
+                                         ("q4_1", [(900, 1024), (700, 512)]), ("q5_0", [(900, 1024), (700, 512)]),
+                                         ("q5_1", [(900, 1024), (700, 512)]), ("iq4_nl", [(900, 1024), (700, 512)])])
+def test_timeline_build_of_a_grouped_launch(hip, oracle, name, shapes):
+    """Several matrices in one launch with the timeline buffer set (the first and third case fit one row group per
+    wavefront and take the eager build): same bits as the normal build, and the stamps name every problem of the launch."""
+    import ctypes as C
+    import torch
+    from tensorsharp_amd import QuantizedWeight, hip_native as Nat, synth
+    from oracle.oracle import MORE_TYPES, Q6_K
+    t = {"q4_k": Q4_K, "mxfp4": MXFP4, "q8_0": Q8_0, "q6_k": Q6_K}.get(name) or MORE_TYPES[name]
+    dev = torch.device("cuda:0")
+    ws = [QuantizedWeight(synth.random_weight(t, n, k, dev, seed=91 + i), t, k, n) for i, (n, k) in enumerate(shapes)]
+    g = torch.Generator(device=dev).manual_seed(5)
+    xs = [torch.randn((1, k), device=dev, generator=g) for _, k in shapes]
+    want = [torch.empty((1, n), device=dev) for n, _ in shapes]
+    got = [torch.empty((1, n), device=dev) for n, _ in shapes]
+    hip.AddmmQuantGroupDevice(hip.PrepareGroup(want, xs, ws))
+    torch.cuda.synchronize()
+    waves = 8 * 4 * 256 + 64
+    buf = torch.zeros((waves, 8), dtype=torch.int64, device=dev)
+    Nat.check_result(Nat.lib().TSHip_SetGemvTimeline(C.c_void_p(buf.data_ptr()), waves * 64), "timeline")
+    try:
+        hip.AddmmQuantGroupDevice(hip.PrepareGroup(got, xs, ws))
+        torch.cuda.synchronize()
+    finally:
+        Nat.check_result(Nat.lib().TSHip_SetGemvTimeline(None, 0), "timeline")
+    for a, b in zip(got, want):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    a = buf.cpu().numpy()
+    ran = a[a[:, 4] != 0]
+    assert ran.shape[0] >= 8 * len(shapes) and ran.shape[0] % 8 == 0, ran.shape
+    assert np.all(ran[:, 0] <= ran[:, 2]) and np.all(ran[:, 2] <= ran[:, 4])
+    problems = set(int(v) for v in (ran[:, 5] >> 8) & 0xff)
+    assert problems == set(range(len(shapes))), problems
+

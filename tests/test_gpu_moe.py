@@ -64,6 +64,30 @@ def test_expert_stage_small_dims(hip, oracle, name, T, k):
     assert inputs.row_l2_err(got2, ref2) <= 1e-3
 
 
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "q5_k", "q6_k"])
+@pytest.mark.parametrize("T", [1, 2])
+def test_decode_stage_every_other_gemv_format(hip, oracle, name, T):
+    """One or two tokens of experts in the block formats that have a GEMV kernel but no early expert records: the gate_up
+    launch (expert ids read on the device, paired store) and the down launches read their problem fields where they need
+    them.  Random valid blocks; reference = the oracle's expert stage over the bit-exact dequantized weights."""
+    import torch
+    from oracle.oracle import MORE_TYPES
+    from tensorsharp_amd import synth
+    t = MORE_TYPES[name]
+    rng = np.random.default_rng(77 + T)
+    E, H, F, k = 6, 512, 768, 4
+    cpu = torch.device("cpu")
+    gu = synth.random_weight(t, E * 2 * F, H, cpu, seed=21, sigma=0.05).numpy()
+    dn = synth.random_weight(t, E * H, F, cpu, seed=22, sigma=0.05).numpy()
+    gb = (rng.standard_normal((E, 2 * F)) * 0.1).astype(np.float32)
+    db = (rng.standard_normal((E, H)) * 0.1).astype(np.float32)
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    ids, wts = oracle.moe_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    ref = oracle.moe_forward(t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    got = run_gpu(hip, t, gu, gb, dn, db, E, H, F, hidden, ids, wts)
+    assert inputs.row_l2_err(got, ref) <= 1e-3, (name, T, inputs.row_l2_err(got, ref))
+
+
 @pytest.mark.parametrize("name", ["mxfp4", "q4_k"])
 def test_expert_tiles_of_128_rows(hip, oracle, name):
     # more than 160 rows per expert on average: the grouped GEMM runs 128-row tiles instead of 32-row ones (MXFP4: with a

@@ -56,7 +56,7 @@ def test_rejects_sizes_beyond_the_static_scratch(hip):
     import torch
     from tensorsharp_amd import hip_native
     # 20000 rows x 4096: 164 MB of converted activations > 64 MiB
-    M, N, K = 20000, 32, 4096
+    M, N, K = 20000, 256, 4096
     w = torch.zeros(N * (K // 256) * 144, dtype=torch.uint8, device="cuda")
     x = torch.zeros((M, K), dtype=torch.float32, device="cuda")
     y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
