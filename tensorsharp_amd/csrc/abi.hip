@@ -2632,7 +2632,8 @@ bool validate_layer(const LayerShape& L, int64_t qkv_ne0, int64_t qkv_ne1, int64
 // one token through one layer (ggml_ops_transformer.cpp:379-470); every pointer in device memory
 bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm, const void* qkv, const float* q_norm,
                       const float* k_norm, const void* o, const float* ffn_norm, const void* gu, const void* down, float* k_cache,
-                      float* v_cache, int position, float eps, float rope_base, float rope_freq_scale, int rope_mode, hipStream_t stream)
+                      float* v_cache, int position, float eps, float rope_base, float rope_freq_scale, int rope_mode, hipStream_t stream,
+                      const float* next_attn_norm = nullptr)
 {
     const int q_dim = L.num_heads * L.head_dim, k_dim = L.num_kv_heads * L.head_dim, qkv_n = q_dim + 2 * k_dim;
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
@@ -2652,7 +2653,7 @@ bool run_layer_decode(float* hidden, const LayerShape& L, const float* attn_norm
     const TSHipTensorView2D attn_view{attn, 1, q_dim, q_dim, 1, (int64_t)q_dim * 4};
     if (!run_matmul_device_ws(qkv_view, h_view, qkv, L.qkv_type, L.hidden, qkv_n, stream, mm_ws, b_mm, attn_norm, eps, false)) return false;
     if (!launch_attention_decode(qkv_out, q_norm, k_norm, eps, rope_base, rope_freq_scale, rope_mode, k_cache, v_cache, L.num_heads,
-                                 L.num_kv_heads, L.head_dim, L.max_seq_len, position, part, attn, stream))
+                                 L.num_kv_heads, L.head_dim, L.max_seq_len, position, part, attn, stream, ffn_norm, next_attn_norm, L.hidden))
         return false;
     // hidden += W_o attn
     if (!run_matmul_device_ws(h_view, attn_view, o, L.o_type, q_dim, L.hidden, stream, mm_ws, b_mm, nullptr, 0.f, true)) return false;
@@ -2773,7 +2774,7 @@ int TSHip_TransformerModelDecodeDevice(float* hidden, int hidden_size, int num_l
             }
             if (!run_layer_decode(hidden, L, attn_norm[l], qkv[l], q_norm ? q_norm[l] : nullptr, k_norm ? k_norm[l] : nullptr, o[l],
                                   ffn_norm[l], gu[l], down[l], k_cache[l], v_cache[l], position, eps, rope_base, rope_freq_scale,
-                                  rope_mode, t_stream))
+                                  rope_mode, t_stream, l + 1 < num_layers ? static_cast<const float*>(attn_norm[l + 1]) : nullptr))
                 return 0;
         }
         clear_last_error();
@@ -2837,10 +2838,13 @@ int TSHip_TransformerModelDecode(void* hidden, int hidden_size, int num_layers, 
                 return 0;
         }
         return decode_with_host_hidden(static_cast<float*>(hidden), hidden_size, [&](float* h, hipStream_t stream) {
-            for (const HostLayer& x : d)
+            for (size_t l = 0; l < d.size(); ++l) {
+                const HostLayer& x = d[l];
                 if (!run_layer_decode(h, L, x.attn_norm, x.qkv, x.q_norm, x.k_norm, x.o, x.ffn_norm, x.gu, x.down, x.k_cache, x.v_cache,
-                                      position, eps, rope_base, rope_freq_scale, rope_mode, stream))
+                                      position, eps, rope_base, rope_freq_scale, rope_mode, stream,
+                                      l + 1 < d.size() ? d[l + 1].attn_norm : nullptr))
                     return false;
+            }
             return true;
         });
     });

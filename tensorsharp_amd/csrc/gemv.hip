@@ -999,7 +999,8 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const __amdgpu_buffer_rsrc_t x2rs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(act == kActRmsNorm ? P.norm_w : P.x + K), 0, K * 4, 0x00020000);
     float4 x2[kStageChunk][F::kStageF4];
-    auto stage_issue = [&](int base) {
+    // what == 1: the activations, 2: the second operand, 3: both
+    auto stage_issue = [&](int base, int what = 3) {
 #pragma unroll
         for (int c = 0; c < kStageChunk; ++c) {
             const int it = base + c * kThreads + (int)threadIdx.x;
@@ -1008,9 +1009,11 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
 #pragma unroll
             for (int q = 0; q < F::kStageF4; ++q) {
                 // items past the end fall outside the resource and read as zeros
-                const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
-                xv[c][q] = float4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
-                if (act != kActPlain) {
+                if (what & 1) {
+                    const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
+                    xv[c][q] = float4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+                }
+                if (act != kActPlain && (what & 2)) {
                     const uint4_t u = __builtin_amdgcn_raw_buffer_load_b128(x2rs, (int)(it < items ? off[q] : kDeadOffset), 0, 0);
                     x2[c][q] = float4{__uint_as_float(u.x), __uint_as_float(u.y), __uint_as_float(u.z), __uint_as_float(u.w)};
                 }
@@ -1081,13 +1084,21 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     } else {
         // (with expert indirection, requesting the activations first so that they travel while the id is on its way gained
         // 0.15 us on a GPT-OSS token: not kept)
+        // The norm weight of the RMSNorm mode is asked for before anything else.  Unlike the activations, which the launch
+        // before this one has just written, it comes from HBM, and asked for behind the first weight step it queues up
+        // behind the 37 MB that the launch's wavefronts request at the same moment: 1.25 us per launch, measured by leaving
+        // the load out.
+        if (act == kActRmsNorm) {
+            stage_issue(0, 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         fetch(fgroup, fstep, cur);
         advance(fgroup, fstep);
         if (deep) {
             fetch(fgroup, fstep, nxt);
             advance(fgroup, fstep);
         }
-        stage_issue(0);
+        stage_issue(0, act == kActRmsNorm ? 1 : 3);
     }
     if (TL && EAGER == 0) {
         // the first chunk of activations is in registers (the weight step requested before them has arrived too: memory

@@ -99,7 +99,8 @@ template <int PER, int G>
 __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(float* k_cache, float* v_cache, const float* qkv, int group,
                                                                        int max_seq_len, int total, int split_len, float scale, int splits,
                                                                        int num_heads, float* __restrict__ partial, const AttnFront F,
-                                                                       float* __restrict__ out_direct)
+                                                                       float* __restrict__ out_direct, const float* pre0, const float* pre1,
+                                                                       int pre_floats)
 {
     // (what the first loads need - the caches, the projections, the geometry - are leading scalar arguments: the hardware
     // delivers the first 14 dwords in SGPRs at wave launch, the rest is read from the argument block)
@@ -107,6 +108,23 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(float* k_c
     __shared__ float sm[kAttnWaves][G], sl[kAttnWaves][G], sacc[kAttnWaves][G][HD];
     __shared__ float sq[G][HD], sk[HD], sv[HD], tmp[kAttnWaves][HD];
     const int kvh = blockIdx.x, split = blockIdx.y;
+    if (split == splits) {
+        // One more row of workgroups than there are splits: they only read the vectors that the launches after this one
+        // ask for first (the norm weights of the FFN and of the next layer) and leave.  Read from HBM by this kernel's
+        // spare workgroups, the vectors wait in the memory-side cache (and, consecutive workgroups being dealt to
+        // consecutive XCDs, in every L2) instead of queueing up behind a launch's first weight requests: 1.25 us per
+        // RMSNorm launch, measured by leaving the vector out.
+        if (blockIdx.z == 0) {
+            for (int i = (int)threadIdx.x * 4; i < pre_floats; i += kAttnWaves * 64 * 4) {
+                typedef float f4_t __attribute__((ext_vector_type(4)));
+                f4_t a, b;                                     // never used: the loads are for the caches
+                if (pre0) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(a) : "v"(pre0 + i) : "memory");
+                if (pre1) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(b) : "v"(pre1 + i) : "memory");
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        return;
+    }
     const int h0 = kvh * group + blockIdx.z * G;                     // first query head of this workgroup
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lg = lane & 15, grp = (wave << 2) | (lane >> 4);       // 16 groups per workgroup
@@ -437,7 +455,8 @@ size_t attention_decode_ws_bytes(int num_heads, int total)
 
 bool launch_attention_decode(const float* qkv, const float* q_norm_w, const float* k_norm_w, float eps, float rope_base,
                              float rope_freq_scale, int rope_mode, float* k_cache, float* v_cache, int num_heads, int num_kv_heads,
-                             int head_dim, int max_seq_len, int position, float* partial_ws, float* out, hipStream_t stream)
+                             int head_dim, int max_seq_len, int position, float* partial_ws, float* out, hipStream_t stream,
+                             const float* prefetch0, const float* prefetch1, int prefetch_floats)
 {
     const int total = position + 1;
     if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || total <= 0 || total > max_seq_len) {
@@ -472,10 +491,14 @@ bool launch_attention_decode(const float* qkv, const float* q_norm_w, const floa
     // the launch with too few workgroups to hide its latency
     int g = group % 8 == 0 ? 8 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
     while (g > 2 && num_kv_heads * splits * (group / g) < 128) g >>= 1;
-    const dim3 grid(num_kv_heads, splits, group / g), block(kAttnWaves * 64);
+    // (vectors to prefetch: whole float4s at 16-byte aligned addresses, else none)
+    const bool pre = (prefetch0 || prefetch1) && prefetch_floats > 0 && prefetch_floats % 4 == 0 && splits < 65535 &&
+                     ((reinterpret_cast<uintptr_t>(prefetch0) | reinterpret_cast<uintptr_t>(prefetch1)) & 15) == 0;
+    const dim3 grid(num_kv_heads, splits + (pre ? 1 : 0), group / g), block(kAttnWaves * 64);
 #define TSHIP_ATTN_LAUNCH(PER, GG)                                                                                              \
     hipLaunchKernelGGL((attn_decode_kernel<PER, GG>), grid, block, 0, stream, front.k_cache, front.v_cache, front.qkv, group,     \
-                       max_seq_len, total, split_len, scale, splits, num_heads, partial_ws, front, splits == 1 ? out : nullptr)
+                       max_seq_len, total, split_len, scale, splits, num_heads, partial_ws, front, splits == 1 ? out : nullptr,           \
+                       pre ? prefetch0 : nullptr, pre ? prefetch1 : nullptr, pre ? prefetch_floats : 0)
 #define TSHIP_ATTN_G(PER)                                                    \
     switch (g) {                                                             \
     case 8: TSHIP_ATTN_LAUNCH(PER, 8); break;                                \

@@ -241,7 +241,10 @@ inline bool is_matmul_type(int type) { return is_quant_type(type) || is_dense_ty
 size_t attention_decode_ws_bytes(int num_heads, int total);
 bool launch_attention_decode(const float* qkv, const float* q_norm_w, const float* k_norm_w, float eps, float rope_base,
                              float rope_freq_scale, int rope_mode, float* k_cache, float* v_cache, int num_heads, int num_kv_heads,
-                             int head_dim, int max_seq_len, int position, float* partial_ws, float* out, hipStream_t stream);
+                             int head_dim, int max_seq_len, int position, float* partial_ws, float* out, hipStream_t stream,
+                             const float* prefetch0 = nullptr, const float* prefetch1 = nullptr, int prefetch_floats = 0);
+// prefetch0 / prefetch1: optional vectors of prefetch_floats floats that later launches ask for first (norm weights); spare
+// workgroups of the attention launch read them so that they wait in the caches
 
 // ---- MoE (GPT-OSS expert stage) -------------------------------------------------------------
 // ids / weights: [T x k] device; top-k by repeated argmax (first maximum wins), softmax over the k logits.
