@@ -171,19 +171,25 @@ __global__ void __launch_bounds__(kAttnWaves * 64) attn_decode_kernel(float* k_c
             // the reference builds theta by repeated multiplication; the same float products in the same order.  One
             // uniform chain of half - 1 products, every lane keeping the value of its own pair (a loop of lane-dependent
             // length costs several times as many instructions per product).
+            // theta_i = theta_(i-1) * theta_scale, i = lane + 64 j: every step each lane takes its lower neighbour's value
+            // times theta_scale (lane 0: its own value times one), so that after 63 steps lane i has been through exactly
+            // the products 1 .. i of the chain - one instruction per step instead of a multiply, a compare and a select.
+            const float factor = lane == 0 ? 1.0f : F.theta_scale;
             float chain = (float)position;
 #pragma unroll
-            for (int j = 0; j < kPairs; ++j) cs[j] = chain;       // pair 0
-            for (int i = 1; i < half; ++i) {
-                chain *= F.theta_scale;
-#pragma unroll
-                for (int j = 0; j < kPairs; ++j) cs[j] = (lane + 64 * j == i) ? chain : cs[j];
+            for (int j = 0; j < kPairs; ++j) {
+                if (j > 0) chain = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(chain), 63)) * F.theta_scale;
+                const int steps = min(half - 64 * j, 64) - 1;
+                for (int i = 0; i < steps; ++i) {
+                    const int below = __builtin_amdgcn_update_dpp(__float_as_int(chain), __float_as_int(chain), 0x138, 0xf, 0xf, false);   // wave_shr:1
+                    chain = __int_as_float(below) * factor;
+                }
+                cs[j] = chain;
             }
 #pragma unroll
             for (int j = 0; j < kPairs; ++j) {
                 const float ang = F.freq_scale * cs[j];
-                cs[j] = cosf(ang);
-                sn[j] = sinf(ang);
+                sincosf(ang, &sn[j], &cs[j]);
             }
         }
         for (int hh = wave; hh < nprep; hh += kAttnWaves) {          // uniform per wavefront
