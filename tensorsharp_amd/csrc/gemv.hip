@@ -928,63 +928,9 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const uint32_t row_bytes = (uint32_t)F::row_bytes(K);
     const int wave_stride = nwg * kWaves;
     const int gw = __builtin_amdgcn_readfirstlane(wg * kWaves + (int)(threadIdx.x >> 6));
-    // an expert id from the device is not trusted: one outside the table gets an empty resource (every load reads
-    // zero, so the result row is the `add` term alone) instead of an address computed from it
-    const int eid = P.expert_id ? __builtin_amdgcn_readfirstlane(P.expert_id[0]) : 0;
-    const bool bad_expert = P.expert_id && (eid < 0 || eid >= P.n_experts);
-    const uintptr_t w_begin = reinterpret_cast<uintptr_t>(P.w) + (P.expert_id && !bad_expert ? (uintptr_t)((int64_t)eid * P.expert_stride) : 0);
-    // one range-checked resource for the whole tensor (host guarantees w_bytes < 2 GiB); the extent is
-    // rounded up to whole dwords, which stay inside the last 4-byte word the tensor touches
-    const uintptr_t base = w_begin & ~(uintptr_t)3;
-    const uint32_t base_delta = (uint32_t)(w_begin & 3);
-    const uint32_t extent = bad_expert ? 0u : ((uint32_t)P.w_bytes + base_delta + 3u) & ~3u;
-    const __amdgpu_buffer_rsrc_t rs =
-        __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, (int)extent, 0x00020000);
-    typename F::Lane L = F::lane_setup(lane_row, l16, row_bytes);
-    uint32_t lds_lane = (uint32_t)l16 * F::kLdsDwords;
-    // routed sum: the lane's sub-row is a slot; its expert's matrix starts slot_id * expert_stride into the stack and
-    // its activations are vector `slot` of the staged ones
-    int slot_id = 0;
-    bool slot_ok = true;
-    // the four slot ids and weights come through the scalar cache in one round trip each (a per-lane load would stand in
-    // front of every weight request, and memory answers a wavefront in order)
-    typedef int int4v_t __attribute__((ext_vector_type(4)));
-    typedef float float4v_t __attribute__((ext_vector_type(4)));
-    int4v_t slot_id4 = {0, 0, 0, 0};
-    float4v_t slot_w4 = {0.f, 0.f, 0.f, 0.f};
-    if (routed) {
-        if constexpr (RPG == 4) {
-            asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx4 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
-                         : "=&s"(slot_id4), "=&s"(slot_w4)
-                         : "s"(P.slot_ids), "s"(P.slot_w)
-                         : "memory");
-        }
-        slot_id = sub == 0 ? slot_id4.x : sub == 1 ? slot_id4.y : sub == 2 ? slot_id4.z : slot_id4.w;
-        slot_ok = slot_id >= 0 && slot_id < P.n_experts;
-        L.voff += slot_ok ? (uint32_t)slot_id * (uint32_t)P.expert_stride : 0u;
-        lds_lane += (uint32_t)sub * (uint32_t)(upr * F::kLdsDwords);
-    }
-
-    // issue the loads of step (group, step); no waiting, no branches
-    auto fetch = [&](int group, int step, Step<F>& st) {
-        const bool group_ok = group < ngroups;                         // uniform
-        const int row0 = group_ok ? group * gstep : 0;
-        const uint32_t start = base_delta + (uint32_t)row0 * row_bytes + (uint32_t)step * F::kSlotBytes;
-        const uint32_t soff = start & ~3u;                             // scalar part of the address
-        const bool live = group_ok && (row0 + osub < N) && (l16 + step * LPR < upr) && slot_ok;
-        st.step = step;
-        st.group = group;
-        st.aux = F::load(rs, L, soff, start & 3u, step, live, st.w);
-        // routed sum: the slot's bias for this row rides with the group's first step
-        st.extra = (routed && step == 0 && P.slot_bias && live && l16 == 0) ? P.slot_bias[(int64_t)slot_id * N + row0] : 0.f;
-    };
-    auto advance = [&](int& group, int& step) {
-        if (++step == nsteps) {
-            step = 0;
-            group += wave_stride;
-        }
-    };
-
+    // The expert id is requested here and looked at after the activations have been requested: between the two lies a
+    // memory round trip (a probe with a constant id: 2.2 us of a GPT-OSS token), which the activations' own then overlaps.
+    const int eid_raw = P.expert_id ? P.expert_id[0] : 0;
     // x is requested first (it mostly hits L2 and memory answers a wavefront in order), then the
     // first weight steps, and only then is x converted into LDS - with the weights already in flight.
     const int kx = routed ? K * RPG : K;          // staged activations: one vector, or one per slot back to back
@@ -1063,6 +1009,65 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         }
     };
 
+    stage_issue(0);
+    __builtin_amdgcn_sched_barrier(0);       // the operands' loads stay ahead of everything that waits for the expert id
+    // an expert id from the device is not trusted: one outside the table gets an empty resource (every load reads
+    // zero, so the result row is the `add` term alone) instead of an address computed from it
+    const int eid = P.expert_id ? __builtin_amdgcn_readfirstlane(eid_raw) : 0;
+    const bool bad_expert = P.expert_id && (eid < 0 || eid >= P.n_experts);
+    const uintptr_t w_begin = reinterpret_cast<uintptr_t>(P.w) + (P.expert_id && !bad_expert ? (uintptr_t)((int64_t)eid * P.expert_stride) : 0);
+    // one range-checked resource for the whole tensor (host guarantees w_bytes < 2 GiB); the extent is
+    // rounded up to whole dwords, which stay inside the last 4-byte word the tensor touches
+    const uintptr_t base = w_begin & ~(uintptr_t)3;
+    const uint32_t base_delta = (uint32_t)(w_begin & 3);
+    const uint32_t extent = bad_expert ? 0u : ((uint32_t)P.w_bytes + base_delta + 3u) & ~3u;
+    const __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, (int)extent, 0x00020000);
+    typename F::Lane L = F::lane_setup(lane_row, l16, row_bytes);
+    uint32_t lds_lane = (uint32_t)l16 * F::kLdsDwords;
+    // routed sum: the lane's sub-row is a slot; its expert's matrix starts slot_id * expert_stride into the stack and
+    // its activations are vector `slot` of the staged ones
+    int slot_id = 0;
+    bool slot_ok = true;
+    // the four slot ids and weights come through the scalar cache in one round trip each (a per-lane load would stand in
+    // front of every weight request, and memory answers a wavefront in order)
+    typedef int int4v_t __attribute__((ext_vector_type(4)));
+    typedef float float4v_t __attribute__((ext_vector_type(4)));
+    int4v_t slot_id4 = {0, 0, 0, 0};
+    float4v_t slot_w4 = {0.f, 0.f, 0.f, 0.f};
+    if (routed) {
+        if constexpr (RPG == 4) {
+            asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx4 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&s"(slot_id4), "=&s"(slot_w4)
+                         : "s"(P.slot_ids), "s"(P.slot_w)
+                         : "memory");
+        }
+        slot_id = sub == 0 ? slot_id4.x : sub == 1 ? slot_id4.y : sub == 2 ? slot_id4.z : slot_id4.w;
+        slot_ok = slot_id >= 0 && slot_id < P.n_experts;
+        L.voff += slot_ok ? (uint32_t)slot_id * (uint32_t)P.expert_stride : 0u;
+        lds_lane += (uint32_t)sub * (uint32_t)(upr * F::kLdsDwords);
+    }
+
+    // issue the loads of step (group, step); no waiting, no branches
+    auto fetch = [&](int group, int step, Step<F>& st) {
+        const bool group_ok = group < ngroups;                         // uniform
+        const int row0 = group_ok ? group * gstep : 0;
+        const uint32_t start = base_delta + (uint32_t)row0 * row_bytes + (uint32_t)step * F::kSlotBytes;
+        const uint32_t soff = start & ~3u;                             // scalar part of the address
+        const bool live = group_ok && (row0 + osub < N) && (l16 + step * LPR < upr) && slot_ok;
+        st.step = step;
+        st.group = group;
+        st.aux = F::load(rs, L, soff, start & 3u, step, live, st.w);
+        // routed sum: the slot's bias for this row rides with the group's first step
+        st.extra = (routed && step == 0 && P.slot_bias && live && l16 == 0) ? P.slot_bias[(int64_t)slot_id * N + row0] : 0.f;
+    };
+    auto advance = [&](int& group, int& step) {
+        if (++step == nsteps) {
+            step = 0;
+            group += wave_stride;
+        }
+    };
+
     // The first step of a wavefront is requested before x is staged, so weight latency overlaps the prologue; in the
     // loop the next step is requested before the current one is consumed.
     Step<F> cur, nxt;
@@ -1074,8 +1079,6 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
     const bool strict = mode == 1, deep = ACT == kActSiluMul && !strict;
     Step<F> eager[EAGER > 0 ? EAGER : 1];
     if constexpr (EAGER > 0) {
-        stage_issue(0);
-        __builtin_amdgcn_sched_barrier(0);       // the activations' loads stay ahead of the weights'
 #pragma unroll
         for (int s = 0; s < EAGER; ++s) fetch(s < nsteps ? gw : ngroups, s, eager[s]);
     } else {
@@ -1085,8 +1088,7 @@ __device__ __forceinline__ void gemv_body(const GemvProblem& P, int wg, int nwg,
         // before: a probe that left the norm weight out gained 1.25 us per launch.  Measured on one box, weights first /
         // operands first: Q4_K 4096 x 14336 9.44 / 8.42 us, Q8_0 9728 x 2560 8.85 / 8.70, Q8_0 4096 x 4096 7.60 / 7.26, the
         // 123 MB grouped launch 23.31 / 23.24, a decode layer 47.7 / 46.2 (of which the norm weights 0.7).
-        stage_issue(0);
-        __builtin_amdgcn_sched_barrier(0);
+        // (They are requested above, ahead of the expert id's use as well.)
         fetch(fgroup, fstep, cur);
         advance(fgroup, fstep);
         if (deep) {
